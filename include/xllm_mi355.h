@@ -1,0 +1,211 @@
+/*
+ * xllm_mi355.h -- C ABI of the MI355X (gfx950) paged-KV decode path.
+ *
+ * Two operations and their helpers:
+ *   1. reshape_and_cache: scatter new K/V token rows into block-table-addressed
+ *      cache pages, optionally quantising to fp8 e4m3fn with per-KV-head scales.
+ *   2. paged decode attention: GQA (block-table and CSR addressing) and the MLA
+ *      latent-KV variant, split over long contexts with a log-sum-exp merge.
+ *
+ * All pointers are DEVICE pointers unless a comment says "host".  Every entry
+ * point only enqueues work on `stream` (a hipStream_t passed as void*); none of
+ * them synchronises, allocates or frees device memory, or reads device memory
+ * from the host, so they are legal inside a HIP graph capture.
+ *
+ * Return value of every int function: 0 = ok; negative = argument error
+ * (XLLM_MI355_E*); positive = a hipError_t raised by a launch.
+ * The reference aborts the process on a failed CHECK; the C++ shim above this
+ * ABI turns a non-zero return into the same abort.
+ *
+ * Tensor layouts follow the reference (paths relative to the xLLM source tree):
+ *   key/value          [T, Hkv, D]      last two dims contiguous, token stride free
+ *                                       (xllm/core/kernels/param.h:126-161)
+ *   k_cache/v_cache    [P, bs, Hkv, D]  contiguous
+ *                                       (xllm/core/framework/kv_cache/kv_cache_shape.cpp:303-311)
+ *   MLA latent cache   [P, bs, 1, d_latent + d_rope], no V cache
+ *                                       (kv_cache_shape.cpp:433-441)
+ *   slot_mapping       [T] int32, slot = page * bs + offset, negative = skip
+ *                                       (xllm/core/kernels/cuda/reshape_paged_cache.cu:36-41)
+ *   block_table        [B, >= ceil(L/bs)] int32 rows with a row stride; entries
+ *                      past ceil(L/bs) are never read (padding may be 0 or -1)
+ *   seq_lens           [B] int32, context length including the new token
+ *   LSE                natural log, fp32, [B, Hq]
+ *                                       (tests/core/layers/mlu/dcp_attention_merge_test.cpp:127-143)
+ */
+#ifndef XLLM_MI355_H_
+#define XLLM_MI355_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types. */
+enum {
+  XLLM_MI355_BF16 = 0,
+  XLLM_MI355_FP16 = 1,
+  XLLM_MI355_FP32 = 2,
+  XLLM_MI355_FP8_E4M3 = 3 /* OCP e4m3fn, the format of torch.float8_e4m3fn */
+};
+
+/* Argument errors. */
+enum {
+  XLLM_MI355_OK = 0,
+  XLLM_MI355_EINVAL = -1,      /* null pointer, non-positive size, bad stride   */
+  XLLM_MI355_EDTYPE = -2,      /* dtype combination not implemented             */
+  XLLM_MI355_ESHAPE = -3,      /* head_dim / group / block size not implemented */
+  XLLM_MI355_EWORKSPACE = -4,  /* workspace missing or too small                */
+  XLLM_MI355_EALIGN = -5       /* pointer or stride not 16-byte aligned         */
+};
+
+/* Human-readable text for a return code of this library (host pointer, static). */
+const char* xllm_mi355_error_string(int code);
+
+/* Library version, "major.minor.patch" (host pointer, static). */
+const char* xllm_mi355_version(void);
+
+/*
+ * reshape_and_cache.
+ * Replaces xllm::kernel::reshape_paged_cache (xllm/core/kernels/ops_api.h:31,
+ * ops_api.cpp:248-278) and its CUDA kernel (kernels/cuda/reshape_paged_cache.cu:23-99).
+ * With cache_dtype == XLLM_MI355_FP8_E4M3 it also covers the quantising store
+ * selected where the cache carries scales (xllm/core/layers/mlu/attention.cpp:109-117),
+ * using the reference's fp8 convention (kernels/cuda/fp8_quant.cu:92-103,
+ * fp8_quant_utils.cuh:111-130):
+ *     q = e4m3fn_rne(fmaxf(-448, fminf(float(x) * (1.0f / scale[h]), 448)))
+ * `value` and `v_cache` may both be null (MLA latent store, the counterpart of
+ * xllm/core/layers/dcu/deepseek_v2_attention.cpp:221-229).
+ * Slots < 0 are skipped as in the reference; slots >= num_blocks * block_size
+ * are skipped too (the reference leaves them undefined).
+ * k_scale / v_scale: [Hkv] fp32, required iff cache_dtype is fp8.
+ * Token strides are in elements.
+ */
+int xllm_mi355_reshape_and_cache(const void* key, const void* value,
+                                 void* k_cache, void* v_cache,
+                                 const int32_t* slot_mapping,
+                                 const float* k_scale, const float* v_scale,
+                                 int64_t n_tokens, int64_t n_kv_heads, int64_t head_dim,
+                                 int64_t block_size, int64_t num_blocks,
+                                 int64_t k_token_stride, int64_t v_token_stride,
+                                 int in_dtype, int cache_dtype, void* stream);
+
+/*
+ * Per-KV-head fp8 scales: scale[h] = max(absmax(x[:, h, :]) / 448, 1e-12).
+ * Replaces the dynamic branch of xllm::kernel::cuda::fp8_scaled_quantize
+ * (xllm/core/kernels/cuda/fp8_scaled_quantize.cpp:38-42) at per-head granularity.
+ * scales: [Hkv] fp32, fully overwritten.
+ */
+int xllm_mi355_kv_head_scales(const void* x, float* scales,
+                              int64_t n_tokens, int64_t n_kv_heads, int64_t head_dim,
+                              int64_t token_stride, int in_dtype, void* stream);
+
+/*
+ * Bytes of split-K workspace the decode entry points need for this problem.
+ * max_seq_len is an upper bound on every seq_lens[b] (AttentionMetadata::max_seq_len,
+ * xllm/core/layers/common/attention_metadata.h:99-156).  Counterpart of the
+ * FlashInfer float workspace (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41).
+ */
+size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads,
+                                               int64_t v_head_dim, int64_t max_seq_len);
+
+/*
+ * Paged decode attention, GQA, block-table addressing.
+ * Replaces xllm::kernel::npu::batch_decode (xllm/core/kernels/npu/npu_ops_api.h:46,
+ * npu/attention.cpp:26-78,141-167) and the block-table subset of
+ * xllm::kernel::mlu::batch_decode (kernels/mlu/mlu_ops_api.h:127):
+ *     out[b, h, :] = softmax(sm_scale * q[b, h, :] . K_b[:, h / group, :]^T) . V_b[:, h / group, :]
+ * q/out: [B, Hq, D] with token strides in elements; lse: [B, Hq] fp32 natural log or null.
+ * k_scale / v_scale: [Hkv] fp32, required iff cache_dtype is fp8 (dequantised value
+ * = float(code) * scale[h]).  q_dtype also is the dtype of `out`.
+ * max_seq_len <= 0 means "table_stride * block_size".
+ * A sequence with seq_lens[b] <= 0 gets out = 0 and lse = -inf.
+ */
+int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache,
+                                void* out, float* lse,
+                                const int32_t* block_table, int64_t table_stride,
+                                const int32_t* seq_lens,
+                                const float* k_scale, const float* v_scale,
+                                int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
+                                int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                int64_t q_token_stride, int64_t out_token_stride,
+                                int64_t max_seq_len, float sm_scale,
+                                void* workspace, size_t workspace_bytes,
+                                int q_dtype, int cache_dtype, void* stream);
+
+/*
+ * Same, CSR addressing.  Replaces xllm::kernel::cuda::batch_decode
+ * (xllm/core/kernels/cuda/cuda_ops_api.h:128-144, cuda/batch_decode.cpp:26-86) without
+ * its FlashInfer plan/uri/workspace triple, and the decode branch of
+ * TorchAttentionImpl::forward (xllm/core/layers/dcu/torch_attention.cpp:285-347):
+ * pages of sequence b are paged_kv_indices[indptr[b] .. indptr[b+1]), the last of
+ * them holds paged_kv_last_page_len[b] tokens.
+ */
+int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const void* v_cache,
+                                    void* out, float* lse,
+                                    const int32_t* paged_kv_indptr,
+                                    const int32_t* paged_kv_indices,
+                                    const int32_t* paged_kv_last_page_len,
+                                    const float* k_scale, const float* v_scale,
+                                    int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
+                                    int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                    int64_t q_token_stride, int64_t out_token_stride,
+                                    int64_t max_seq_len, float sm_scale,
+                                    void* workspace, size_t workspace_bytes,
+                                    int q_dtype, int cache_dtype, void* stream);
+
+/*
+ * Paged decode attention, MLA latent-KV variant.
+ * Replaces xllm::kernel::dcu::flash_mla::dense_decode
+ * (xllm/core/kernels/dcu/flash_mla_adapter.h:40-53, flash_mla_adapter.cpp:104-153):
+ *     out[b, h, :] = softmax(sm_scale * [q_nope | q_pe][b, h, :] . C_b^T) . C_b[:, :d_latent]
+ * with C_b the latent rows of sequence b, [L_b, d_latent + d_rope].
+ * q_nope: [B, H, d_latent], q_pe: [B, H, d_rope], out: [B, H, d_latent], all
+ * contiguous bf16; k_cache: [P, bs, 1, d_latent + d_rope] bf16.
+ */
+int xllm_mi355_paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache,
+                                void* out, float* lse,
+                                const int32_t* block_table, int64_t table_stride,
+                                const int32_t* seq_lens,
+                                int64_t batch, int64_t n_heads,
+                                int64_t d_latent, int64_t d_rope,
+                                int64_t block_size, int64_t num_blocks,
+                                int64_t max_seq_len, float sm_scale,
+                                void* workspace, size_t workspace_bytes,
+                                int dtype, void* stream);
+
+/*
+ * Log-sum-exp merge of S partial attention results.
+ * Replaces xllm::layer::merge_dcp_attention_shards
+ * (xllm/core/layers/mlu/dcp_attention_merge.cpp:26-65):
+ *     w_s = exp(lse_s - max_s lse_s);  out = sum_s w_s o_s / sum_s w_s;
+ *     lse = max + log(sum_s w_s);  shards with lse = -inf are ignored;
+ *     all shards empty -> out = 0, lse = -inf.
+ * partial_out: [S, B, H, Dv] of `dtype`; partial_lse: [S, B, H] fp32 natural log;
+ * out: [B, H, Dv] of `dtype`; lse: [B, H] fp32 or null.
+ */
+int xllm_mi355_lse_merge(const void* partial_out, const float* partial_lse,
+                         void* out, float* lse,
+                         int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim,
+                         int dtype, void* stream);
+
+/*
+ * CSR -> padded block table.  Replaces build_block_table_from_paged_kv
+ * (xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip:44-149):
+ * block_table[b, j] = indices[indptr[b] + j] for j < pages(b), -1 elsewhere;
+ * seq_lens[b] = (pages(b) - 1) * block_size + last_page_len[b] (0 if no pages).
+ * seq_lens may be null.
+ */
+int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr,
+                                 const int32_t* paged_kv_indices,
+                                 const int32_t* paged_kv_last_page_len,
+                                 int32_t* block_table, int64_t table_stride,
+                                 int32_t* seq_lens,
+                                 int64_t batch, int64_t block_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* XLLM_MI355_H_ */

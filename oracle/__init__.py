@@ -1,0 +1,238 @@
+"""ctypes bindings of the two CPU oracles.  TEST INFRASTRUCTURE: only tests, the smoke
+run and the benchmark's CPU-baseline leg may import this package.
+
+All functions take contiguous torch CPU tensors and return new CPU tensors.
+"""
+import ctypes
+import os
+
+import torch
+
+from . import build as _build
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+BF16, FP16, FP32, FP8_E4M3 = 0, 1, 2, 3
+_DT = {torch.bfloat16: BF16, torch.float16: FP16, torch.float32: FP32,
+       torch.float8_e4m3fn: FP8_E4M3, torch.uint8: FP8_E4M3}
+
+_c = None
+_aten = None
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_i32 = ctypes.c_int
+_f32 = ctypes.c_float
+_f64 = ctypes.c_double
+
+
+def dtype_code(t):
+    return _DT[t.dtype]
+
+
+def c_lib():
+    """The plain-C oracle, built on first use if missing."""
+    global _c
+    if _c is None:
+        path = _build.C_LIB
+        if not os.path.exists(path):
+            _build.build_c()
+        lib = ctypes.CDLL(path)
+        lib.oracle_bf16_to_f32.restype = _f32
+        lib.oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
+        lib.oracle_f32_to_bf16.restype = ctypes.c_uint16
+        lib.oracle_f32_to_bf16.argtypes = [_f32]
+        lib.oracle_fp16_to_f32.restype = _f32
+        lib.oracle_fp16_to_f32.argtypes = [ctypes.c_uint16]
+        lib.oracle_f32_to_fp16.restype = ctypes.c_uint16
+        lib.oracle_f32_to_fp16.argtypes = [_f32]
+        lib.oracle_e4m3fn_to_f32.restype = _f32
+        lib.oracle_e4m3fn_to_f32.argtypes = [ctypes.c_uint8]
+        lib.oracle_f32_to_e4m3fn.restype = ctypes.c_uint8
+        lib.oracle_f32_to_e4m3fn.argtypes = [_f32]
+        lib.oracle_fp8_quantize.restype = ctypes.c_uint8
+        lib.oracle_fp8_quantize.argtypes = [_f32, _f32]
+        lib.oracle_reshape_and_cache.restype = _i32
+        lib.oracle_reshape_and_cache.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64,
+                                                 _i64, _i64, _i64, _i32, _i32]
+        lib.oracle_kv_head_scales.restype = None
+        lib.oracle_kv_head_scales.argtypes = [_p, _p, _i64, _i64, _i64, _i64, _i32]
+        lib.oracle_paged_decode_f64.restype = _i32
+        lib.oracle_paged_decode_f64.argtypes = [_p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64,
+                                                _i64, _i64, _i64, _i64, _f64, _i32, _i32, _i32]
+        lib.oracle_lse_merge.restype = None
+        lib.oracle_lse_merge.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64]
+        lib.oracle_build_block_table.restype = None
+        lib.oracle_build_block_table.argtypes = [_p, _p, _p, _p, _i64, _p, _i64, _i64]
+        _c = lib
+    return _c
+
+
+def aten_lib():
+    """The ATen-op-order oracle, built on first use if missing."""
+    global _aten
+    if _aten is None:
+        path = _build.ATEN_LIB
+        if not os.path.exists(path):
+            _build.build_aten()
+        lib = ctypes.CDLL(path)
+        lib.aten_oracle_num_threads.restype = _i32
+        lib.aten_oracle_set_num_threads.argtypes = [_i32]
+        lib.aten_paged_decode.restype = _i32
+        lib.aten_paged_decode.argtypes = [_p, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64, _i64,
+                                          _i64, _i64, _i64, _f32, _i32, _i32]
+        lib.aten_paged_decode_csr.restype = _i32
+        lib.aten_paged_decode_csr.argtypes = [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64,
+                                              _i64, _i32]
+        lib.aten_paged_decode_lse.restype = _i32
+        lib.aten_paged_decode_lse.argtypes = [_p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64,
+                                              _i64, _i64, _f32, _i32, _i32]
+        lib.aten_lse_merge.restype = _i32
+        lib.aten_lse_merge.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32]
+        lib.aten_fp8_quantize.restype = _i32
+        lib.aten_fp8_quantize.argtypes = [_p, _p, _p, _i64, _i64, _i64, _i32]
+        _aten = lib
+    return _aten
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.device.type == "cpu" and t.is_contiguous(), "oracle wants contiguous CPU tensors"
+    return t.data_ptr()
+
+
+# ------------------------------------------------------------------------------ op 1
+
+def reshape_and_cache(key, value, k_cache, v_cache, slot_mapping, k_scale=None, v_scale=None):
+    """In place on k_cache / v_cache (CPU).  key/value [T,Hkv,D] may be strided in dim 0."""
+    T, Hkv, D = key.shape
+    P, bs = k_cache.shape[0], k_cache.shape[1]
+    assert key.stride(2) == 1 and key.stride(1) == D
+    assert slot_mapping.dtype == torch.int32
+    if value is not None:
+        assert value.stride(2) == 1 and value.stride(1) == D
+    rc = c_lib().oracle_reshape_and_cache(
+        key.data_ptr(), None if value is None else value.data_ptr(), _ptr(k_cache), _ptr(v_cache),
+        _ptr(slot_mapping), _ptr(k_scale), _ptr(v_scale), T, Hkv, D, bs, P,
+        key.stride(0), 0 if value is None else value.stride(0), dtype_code(key), dtype_code(k_cache))
+    if rc != 0:
+        raise ValueError("oracle_reshape_and_cache: unsupported dtype pair")
+
+
+def kv_head_scales(x):
+    T, Hkv, D = x.shape
+    out = torch.empty(Hkv, dtype=torch.float32)
+    assert x.stride(2) == 1 and x.stride(1) == D
+    c_lib().oracle_kv_head_scales(x.data_ptr(), _ptr(out), T, Hkv, D, x.stride(0), dtype_code(x))
+    return out
+
+
+def fp8_encode(x_f32):
+    """Plain cast fp32 -> e4m3fn codes (uint8), element by element."""
+    lib = c_lib()
+    flat = x_f32.reshape(-1).tolist()
+    return torch.tensor([lib.oracle_f32_to_e4m3fn(v) for v in flat], dtype=torch.uint8).reshape(x_f32.shape)
+
+
+def fp8_decode_table():
+    lib = c_lib()
+    return torch.tensor([lib.oracle_e4m3fn_to_f32(c) for c in range(256)], dtype=torch.float32)
+
+
+# ------------------------------------------------------------------------------ op 2
+
+def paged_decode_f64(q, k_cache, v_cache, block_table, seq_lens, sm_scale, k_scale=None,
+                     v_scale=None, dv=None, round_dequant=True):
+    """Exact-arithmetic attention.  Returns (out fp32 [B,Hq,dv], lse fp32 [B,Hq])."""
+    B, Hq, Dqk = q.shape
+    bs, Hkv = k_cache.shape[1], k_cache.shape[2]
+    if dv is None:
+        dv = Dqk if v_cache is None else v_cache.shape[3]
+    out = torch.empty(B, Hq, dv, dtype=torch.float32)
+    lse = torch.empty(B, Hq, dtype=torch.float32)
+    rc = c_lib().oracle_paged_decode_f64(
+        _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(lse), _ptr(block_table),
+        block_table.stride(0), _ptr(seq_lens), _ptr(k_scale), _ptr(v_scale), B, Hq, Hkv, Dqk, dv, bs,
+        float(sm_scale), dtype_code(q), dtype_code(k_cache), int(round_dequant))
+    if rc != 0:
+        raise ValueError("oracle_paged_decode_f64 failed")
+    return out, lse
+
+
+def aten_paged_decode(q, k_cache, v_cache, block_table, seq_lens, sm_scale, k_scale=None,
+                      v_scale=None, dv=None):
+    """The reference's libtorch block-table decode.  Returns out [B,Hq,dv] in q.dtype."""
+    B, Hq, Dqk = q.shape
+    P, bs, Hkv = k_cache.shape[0], k_cache.shape[1], k_cache.shape[2]
+    if dv is None:
+        dv = Dqk if v_cache is None else v_cache.shape[3]
+    out = torch.empty(B, Hq, dv, dtype=q.dtype)
+    rc = aten_lib().aten_paged_decode(
+        _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_table), block_table.stride(0),
+        _ptr(seq_lens), _ptr(k_scale), _ptr(v_scale), B, Hq, Hkv, Dqk, dv, bs, P, float(sm_scale),
+        dtype_code(q), dtype_code(k_cache))
+    if rc != 0:
+        raise ValueError("aten_paged_decode: seq_len must be positive")
+    return out
+
+
+def aten_paged_decode_csr(q, k_cache, v_cache, indptr, indices, last_page_len):
+    B, Hq, D = q.shape
+    P, bs, Hkv = k_cache.shape[0], k_cache.shape[1], k_cache.shape[2]
+    out = torch.empty_like(q)
+    rc = aten_lib().aten_paged_decode_csr(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(indptr),
+                                          _ptr(indices), _ptr(last_page_len), B, Hq, Hkv, D, bs, P,
+                                          dtype_code(q))
+    if rc != 0:
+        raise ValueError("aten_paged_decode_csr: empty sequence")
+    return out
+
+
+def aten_paged_decode_lse(q, k_cache, block_table, seq_lens, sm_scale, k_scale=None):
+    B, Hq, Dqk = q.shape
+    P, bs, Hkv = k_cache.shape[0], k_cache.shape[1], k_cache.shape[2]
+    lse = torch.empty(B, Hq, dtype=torch.float32)
+    rc = aten_lib().aten_paged_decode_lse(_ptr(q), _ptr(k_cache), _ptr(lse), _ptr(block_table),
+                                          block_table.stride(0), _ptr(seq_lens), _ptr(k_scale), B, Hq,
+                                          Hkv, Dqk, bs, P, float(sm_scale), dtype_code(q),
+                                          dtype_code(k_cache))
+    if rc != 0:
+        raise ValueError("aten_paged_decode_lse failed")
+    return lse
+
+
+# ------------------------------------------------------------------------------ merge
+
+def lse_merge(partial_out_f32, partial_lse):
+    """C oracle.  partial_out [S,B,H,Dv] fp32, partial_lse [S,B,H] fp32."""
+    S, B, H, Dv = partial_out_f32.shape
+    out = torch.empty(B, H, Dv, dtype=torch.float32)
+    lse = torch.empty(B, H, dtype=torch.float32)
+    c_lib().oracle_lse_merge(_ptr(partial_out_f32), _ptr(partial_lse), _ptr(out), _ptr(lse), S, B, H, Dv)
+    return out, lse
+
+
+def aten_lse_merge(partial_out, partial_lse):
+    S, B, H, Dv = partial_out.shape
+    out = torch.empty(B, H, Dv, dtype=partial_out.dtype)
+    lse = torch.empty(B, H, dtype=torch.float32)
+    aten_lib().aten_lse_merge(_ptr(partial_out), _ptr(partial_lse), _ptr(out), _ptr(lse), S, B, H, Dv,
+                              dtype_code(partial_out))
+    return out, lse
+
+
+def aten_fp8_quantize(x, scale):
+    T, Hkv, D = x.shape
+    out = torch.empty(T, Hkv, D, dtype=torch.uint8)
+    aten_lib().aten_fp8_quantize(_ptr(x), _ptr(out), _ptr(scale), T, Hkv, D, dtype_code(x))
+    return out
+
+
+def build_block_table(indptr, indices, last_page_len, table_stride, block_size):
+    B = indptr.numel() - 1
+    table = torch.empty(B, table_stride, dtype=torch.int32)
+    seq_lens = torch.empty(B, dtype=torch.int32)
+    c_lib().oracle_build_block_table(_ptr(indptr), _ptr(indices), _ptr(last_page_len), _ptr(table),
+                                     table_stride, _ptr(seq_lens), B, block_size)
+    return table, seq_lens

@@ -1,0 +1,228 @@
+"""GPU parity of the GQA paged decode against the reference's libtorch CPU path (ATen oracle)."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close_to_reference, fill_caches_cpu, fill_caches_gpu
+from xllm_amd import ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode_gpu(inp, k_cache, v_cache, device, k_scale=None, v_scale=None, return_lse=True, table=None):
+    cfg, lay = inp.cfg, inp.layout
+    q = inp.q.to(device)
+    out = torch.empty_like(q)
+    table = (lay.block_table if table is None else table).to(device)
+    out, lse = ops.batch_decode(q, k_cache, out, table, lay.seq_lens.to(device), v_cache=v_cache,
+                                k_cache_quant_scale=k_scale, v_cache_quant_scale=v_scale,
+                                scale=cfg.scale, return_lse=return_lse,
+                                max_seq_len=int(lay.seq_lens.max()))
+    torch.cuda.synchronize()
+    return out, lse
+
+
+def _check_config(cfg, seed, device, dtype=torch.bfloat16):
+    inp = workloads.make_inputs(cfg, seed, dtype=dtype)
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    kc, vc = fill_caches_cpu(inp)
+    assert torch.equal(kg.cpu(), kc) and torch.equal(vg.cpu(), vc), "cache bytes must be bit-exact"
+    out, lse = _decode_gpu(inp, kg, vg, device)
+    lay = inp.layout
+    ref = oracle.aten_paged_decode(inp.q, kc, vc, lay.block_table, lay.seq_lens, cfg.scale)
+    mx, mean = assert_close_to_reference(out, ref, cfg.name)
+    ref_lse = oracle.aten_paged_decode_lse(inp.q, kc, lay.block_table, lay.seq_lens, cfg.scale)
+    assert torch.allclose(lse.cpu().view_as(ref_lse), ref_lse, rtol=1e-3, atol=1e-3)
+    return mx, mean
+
+
+def test_config1_tiny_write_then_attend(device):
+    _check_config(workloads.CONFIGS["tiny"], 1234, device)
+
+
+def test_config2_llama3_shape_reduced_batch(device):
+    cfg = workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=8)
+    _check_config(cfg, 2024, device)
+
+
+def test_config3_block128_group8_split_k(device):
+    cfg = workloads.scaled(workloads.CONFIGS["long_b256"], batch=6)
+    _check_config(cfg, 77, device)
+
+
+def test_fp16_and_other_head_dims(device):
+    for D, Hq, Hkv, dt in ((64, 8, 2, torch.float16), (256, 6, 1, torch.bfloat16), (128, 28, 4, torch.float16),
+                           (128, 4, 4, torch.bfloat16), (128, 16, 8, torch.bfloat16), (64, 40, 2, torch.bfloat16)):
+        cfg = workloads.DecodeConfig(f"d{D}_h{Hq}_{Hkv}", 5, Hq, Hkv, D, 32, 1, 700)
+        _check_config(cfg, 100 + D + Hq, device, dtype=dt)
+
+
+def test_reference_npu_case_130_tokens_block128(device):
+    # Qwen35_27B_TP4_KvCacheCrosses128TokenBoundary (tests/core/kernels/npu/npu_xllm_ops_test.cpp:305-394):
+    # seq 130, block 128, 3 blocks, Hq 6 / Hkv 1 / D 256, scale 1/16, table [[2, 0]], tolerance 5e-2
+    g = torch.Generator().manual_seed(20260730)
+    key = torch.randn(130, 1, 256, generator=g).to(torch.bfloat16)
+    value = torch.randn(130, 1, 256, generator=g).to(torch.bfloat16)
+    query = (0.25 * torch.randn(1, 6, 256, generator=g)).to(torch.bfloat16)
+    slots = torch.cat([torch.arange(256, 384), torch.arange(0, 2)]).to(torch.int32)
+    kg = torch.zeros(3, 128, 1, 256, dtype=torch.bfloat16, device=device)
+    vg = torch.zeros_like(kg)
+    ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=key.to(device), value=value.to(device),
+                                                        k_cache=kg, v_cache=vg, slot_mapping=slots.to(device)))
+    table = torch.tensor([[2, 0]], dtype=torch.int32, device=device)
+    lens = torch.tensor([130], dtype=torch.int32, device=device)
+    out = torch.empty(1, 6, 256, dtype=torch.bfloat16, device=device)
+    ops.batch_decode(query.to(device), kg, out, table, lens, v_cache=vg, scale=1.0 / 16.0)
+    # decode_attention_reference of the same test file (:109-125): fp32 matmul / softmax
+    qf, kf, vf = query.float()[0], key.float()[:, 0], value.float()[:, 0]
+    expected = torch.softmax(qf @ kf.T / 16.0, -1) @ vf
+    assert torch.allclose(out.cpu().float()[0], expected, rtol=5e-2, atol=5e-2)
+    assert (out.cpu().float()[0] - expected).abs().max() < 2e-2
+
+
+def test_invariants_single_token_equal_rows_and_page_permutation(device):
+    cfg = workloads.DecodeConfig("inv", 3, 8, 2, 128, 16, 200, 300)
+    inp = workloads.make_inputs(cfg, 5)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    # (1) L = 1: the output is V[0] of the mapped KV head, bit for bit
+    one = torch.ones_like(lay.seq_lens)
+    q = inp.q.to(device)
+    out = torch.empty_like(q)
+    ops.batch_decode(q, kg, out, lay.block_table.to(device), one.to(device), v_cache=vg, scale=cfg.scale)
+    for b in range(cfg.batch):
+        v0 = vg[lay.block_table[b, 0].item(), 0]                         # [Hkv, D]
+        assert torch.equal(out[b], v0.repeat_interleave(cfg.n_q_heads // cfg.n_kv_heads, 0))
+    # (2) moving every page to another physical page, table permuted accordingly: identical bits
+    out_a, _ = _decode_gpu(inp, kg, vg, device)
+    perm = torch.randperm(lay.num_blocks, generator=torch.Generator().manual_seed(9))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(lay.num_blocks)
+    kg2, vg2 = kg[perm.to(device)], vg[perm.to(device)]                  # new page j holds old page perm[j]
+    table2 = inv[lay.block_table.long().clamp(0, lay.num_blocks - 1)].to(torch.int32)
+    out_b, _ = _decode_gpu(inp, kg2.contiguous(), vg2.contiguous(), device, table=table2)
+    assert torch.equal(out_a, out_b)
+    # (3) all V rows equal -> out == that row; all K rows equal -> out == mean(V) (uniform softmax)
+    vconst = torch.randn(cfg.n_kv_heads, cfg.head_dim, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    vg3 = vconst.to(device).expand_as(vg).contiguous()
+    out_c, _ = _decode_gpu(inp, kg, vg3, device)
+    expect = vconst.repeat_interleave(cfg.n_q_heads // cfg.n_kv_heads, 0).float()
+    assert (out_c.cpu().float() - expect).abs().max() <= 2 ** -7 * expect.abs().max()
+
+
+def test_table_padding_is_never_read_and_strided_views(device):
+    cfg = workloads.DecodeConfig("pad", 4, 8, 4, 128, 16, 30, 400)
+    inp = workloads.make_inputs(cfg, 31)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    out_a, _ = _decode_gpu(inp, kg, vg, device)
+    # poison every unused column with huge / negative page ids
+    t = lay.block_table.clone()
+    for b in range(cfg.batch):
+        n = (int(lay.seq_lens[b]) + cfg.block_size - 1) // cfg.block_size
+        t[b, n:] = torch.tensor([-1, 2 ** 30, -2 ** 31][: t.shape[1] - n] + [7] * max(0, t.shape[1] - n - 3))
+    out_b, _ = _decode_gpu(inp, kg, vg, device, table=t)
+    assert torch.equal(out_a, out_b)
+    # a wide persistent table buffer (row stride > width) and a strided query, as under graph capture
+    wide = torch.full((cfg.batch, 1024), -1, dtype=torch.int32, device=device)
+    wide[:, : t.shape[1]] = lay.block_table.to(device)
+    qkv = torch.zeros(cfg.batch, 3 * cfg.n_q_heads * cfg.head_dim, dtype=torch.bfloat16, device=device)
+    qview = qkv[:, : cfg.n_q_heads * cfg.head_dim].view(cfg.batch, cfg.n_q_heads, cfg.head_dim)
+    qview.copy_(inp.q.to(device))
+    out_c = torch.empty(cfg.batch, cfg.n_q_heads, cfg.head_dim, dtype=torch.bfloat16, device=device)
+    ops.batch_decode(qview, kg, out_c, wide[:, : t.shape[1]], lay.seq_lens.to(device), v_cache=vg,
+                     scale=cfg.scale, max_seq_len=int(lay.seq_lens.max()))
+    assert torch.equal(out_a, out_c)
+
+
+def test_csr_form_matches_block_table_form_and_csr_oracle(device):
+    cfg = workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=5, len_lo=17, len_hi=900)
+    inp = workloads.make_inputs(cfg, 8)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    out_a, _ = _decode_gpu(inp, kg, vg, device)
+    q = inp.q.to(device)
+    out_b = torch.empty_like(q)
+    ops.batch_decode_csr(q, kg, vg, lay.indptr.to(device), lay.indices.to(device),
+                         lay.last_page_len.to(device), cfg.scale, out_b, max_seq_len=int(lay.seq_lens.max()))
+    assert torch.equal(out_a, out_b)
+    ref = oracle.aten_paged_decode_csr(inp.q, kg.cpu(), vg.cpu(), lay.indptr, lay.indices, lay.last_page_len)
+    assert_close_to_reference(out_b, ref, "csr")
+    # CSR -> table builder against the C oracle
+    tg, lg = ops.build_block_table_from_paged_kv(lay.indptr.to(device), lay.indices.to(device),
+                                                 lay.last_page_len.to(device), lay.block_table.shape[1],
+                                                 cfg.block_size)
+    tc, lc = oracle.build_block_table(lay.indptr, lay.indices, lay.last_page_len, lay.block_table.shape[1],
+                                      cfg.block_size)
+    assert torch.equal(tg.cpu(), tc) and torch.equal(lg.cpu(), lc) and torch.equal(lc, lay.seq_lens)
+
+
+def test_fp8_kv_cache_decode(device):
+    cfg = workloads.scaled(workloads.CONFIGS["fp8_kv"], batch=4, len_lo=300, len_hi=3000)
+    inp = workloads.make_inputs(cfg, 4242)
+    lay = inp.layout
+    kg, vg, ks, vs = fill_caches_gpu(inp, device, cache_dtype=torch.float8_e4m3fn)
+    kc, vc = fill_caches_cpu(inp, torch.float8_e4m3fn, ks.cpu(), vs.cpu())
+    assert torch.equal(kg.view(torch.uint8).cpu(), kc) and torch.equal(vg.view(torch.uint8).cpu(), vc)
+    out, lse = _decode_gpu(inp, kg, vg, device, ks, vs)
+    ref = oracle.aten_paged_decode(inp.q, kc.view(torch.float8_e4m3fn), vc.view(torch.float8_e4m3fn),
+                                   lay.block_table, lay.seq_lens, cfg.scale, ks.cpu(), vs.cpu())
+    assert_close_to_reference(out, ref, "fp8")
+
+
+def test_empty_sequence_and_argument_errors(device):
+    cfg = workloads.DecodeConfig("e", 3, 8, 2, 128, 16, 10, 50)
+    inp = workloads.make_inputs(cfg, 2)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    lens = lay.seq_lens.clone()
+    lens[1] = 0
+    q = inp.q.to(device)
+    out = torch.full_like(q, 7.0)
+    out, lse = ops.batch_decode(q, kg, out, lay.block_table.to(device), lens.to(device), v_cache=vg,
+                                scale=cfg.scale, return_lse=True)
+    assert (out[1] == 0).all() and torch.isneginf(lse[1]).all()
+    with pytest.raises(Exception):
+        ops.batch_decode(q[:, :, :100], kg, out, lay.block_table.to(device), lens.to(device), v_cache=vg)
+    with pytest.raises(Exception):
+        ops.batch_decode(q.cpu(), kg, out, lay.block_table.to(device), lens.to(device), v_cache=vg)
+
+
+def test_full_size_config2_split_invariance_and_sampled_parity(device):
+    """BASELINE config 2 at full size: (a) sequences sampled from the batch agree with the oracle,
+    (b) LSE-merging the decode of two context halves equals the unsplit decode."""
+    cfg = workloads.CONFIGS["llama3_8b"]
+    inp = workloads.make_inputs(cfg, 2, device=device)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    out, lse = _decode_gpu(inp, kg, vg, device)
+    sample = [0, 17, 41, 63]
+    kc, vc = kg.cpu(), vg.cpu()
+    ref = oracle.aten_paged_decode(inp.q.cpu()[sample].contiguous(), kc, vc,
+                                   lay.block_table[sample].contiguous(), lay.seq_lens[sample].contiguous(),
+                                   cfg.scale)
+    assert_close_to_reference(out[sample], ref, "cfg2 sample")
+    # halves: first ceil(n/2) pages, and the rest as its own table
+    bs = cfg.block_size
+    n_pages = (lay.seq_lens + bs - 1) // bs
+    h = (n_pages + 1) // 2
+    len_a = torch.minimum(lay.seq_lens, h * bs)
+    len_b = lay.seq_lens - len_a
+    table_b = torch.zeros_like(lay.block_table)
+    for b in range(cfg.batch):
+        nb = int(n_pages[b] - h[b])
+        table_b[b, :nb] = lay.block_table[b, int(h[b]) : int(h[b]) + nb]
+    q = inp.q
+    parts_o, parts_l = [], []
+    for table, lens in ((lay.block_table, len_a), (table_b, len_b)):
+        o = torch.empty_like(q)
+        o, l = ops.batch_decode(q, kg, o, table.to(device), lens.to(device), v_cache=vg, scale=cfg.scale,
+                                return_lse=True, max_seq_len=int(lens.max()))
+        parts_o.append(o.view(cfg.batch, 1, cfg.n_q_heads, cfg.head_dim))
+        parts_l.append(l.view(cfg.batch, cfg.n_q_heads, 1))
+    merged, mlse = ops.merge_dcp_attention_shards(torch.stack(parts_o), torch.stack(parts_l))
+    diff = (merged.view_as(out).float() - out.float()).abs()
+    assert diff.max() <= 1e-2 and diff.mean() <= 1e-3
+    assert torch.allclose(mlse.view_as(lse), lse, rtol=1e-3, atol=1e-3)

@@ -1,0 +1,176 @@
+"""GPU parity of reshape_and_cache against the C oracle: cache bytes must be identical."""
+import pytest
+import torch
+
+import oracle
+from xllm_amd import ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+# The five shape cases of ReshapePagedCacheTest.MatchesReference
+# (tests/core/kernels/dcu/reshape_paged_cache_test.cpp:135-158): tokens, blocks, bs, heads, dim, dtype
+REFERENCE_CASES = [
+    (4, 1, 16, 1, 64, torch.float32),
+    (32, 8, 16, 4, 128, torch.float16),
+    (64, 4, 64, 8, 128, torch.bfloat16),
+    (256, 16, 64, 8, 128, torch.float16),
+    (1, 4, 16, 4, 128, torch.float32),
+]
+
+
+def _run_both(key, value, slots, shape, cache_dtype, device, k_scale=None, v_scale=None):
+    store = torch.uint8 if cache_dtype == torch.float8_e4m3fn else cache_dtype
+    kc = torch.zeros(shape, dtype=store)
+    vc = None if value is None else torch.zeros(shape, dtype=store)
+    oracle.reshape_and_cache(key, value, kc, vc, slots, k_scale, v_scale)
+    kg = torch.zeros(shape, dtype=store, device=device)
+    vg = None if value is None else torch.zeros(shape, dtype=store, device=device)
+    p = ops.ReshapePagedCacheParams(
+        key=key.to(device), value=None if value is None else value.to(device), k_cache=kg, v_cache=vg,
+        slot_mapping=slots.to(device),
+        k_cache_scale=None if k_scale is None else k_scale.to(device),
+        v_cache_scale=None if v_scale is None else v_scale.to(device))
+    (ops.quant_to_paged_cache if k_scale is not None else ops.reshape_paged_cache)(p)
+    torch.cuda.synchronize()
+    return (kc, vc), (kg.cpu(), None if vg is None else vg.cpu())
+
+
+def _equal_bytes(a, b):
+    return torch.equal(a.contiguous().view(torch.uint8), b.contiguous().view(torch.uint8))
+
+
+@pytest.mark.parametrize("case", REFERENCE_CASES)
+def test_reference_shape_cases_bit_exact(device, case):
+    T, P, bs, H, D, dt = case
+    g = torch.Generator().manual_seed(2026)
+    key = torch.randn(T, H, D, generator=g).to(dt)
+    value = torch.randn(T, H, D, generator=g).to(dt)
+    slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+    (kc, vc), (kg, vg) = _run_both(key, value, slots, (P, bs, H, D), dt, device)
+    assert _equal_bytes(kc, kg) and _equal_bytes(vc, vg)
+    assert kc.float().abs().sum() > 0
+
+
+def test_crosses_block_boundary_like_reference(device):
+    # Qwen35_27B_TP4_KvCacheCrosses128TokenBoundary (tests/core/kernels/npu/npu_xllm_ops_test.cpp:305-364):
+    # 130 tokens, block 128, 3 physical blocks, slots [256..383] ++ [0, 1]
+    g = torch.Generator().manual_seed(20260730)
+    key = torch.randn(130, 1, 256, generator=g).to(torch.bfloat16)
+    value = torch.randn(130, 1, 256, generator=g).to(torch.bfloat16)
+    slots = torch.cat([torch.arange(256, 384), torch.arange(0, 2)]).to(torch.int32)
+    (kc, vc), (kg, vg) = _run_both(key, value, slots, (3, 128, 1, 256), torch.bfloat16, device)
+    expected = torch.zeros(3, 128, 1, 256, dtype=torch.bfloat16)
+    expected[2] = key[:128]
+    expected[0, :2] = key[128:]
+    assert torch.equal(kg, expected)
+    assert torch.equal(kg, kc) and torch.equal(vg, vc)
+
+
+def test_negative_and_out_of_range_slots_skipped_and_rest_untouched(device):
+    g = torch.Generator().manual_seed(7)
+    T, P, bs, H, D = 16, 4, 16, 2, 128
+    key = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    value = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+    slots[3] = -1
+    slots[5] = -7
+    slots[9] = P * bs + 5
+    kg = torch.full((P, bs, H, D), 3.0, dtype=torch.bfloat16, device=device)
+    vg = torch.full((P, bs, H, D), -2.0, dtype=torch.bfloat16, device=device)
+    ops.reshape_paged_cache(ops.ReshapePagedCacheParams(
+        key=key.to(device), value=value.to(device), k_cache=kg, v_cache=vg, slot_mapping=slots.to(device)))
+    kc = torch.full((P, bs, H, D), 3.0, dtype=torch.bfloat16)
+    vc = torch.full((P, bs, H, D), -2.0, dtype=torch.bfloat16)
+    oracle.reshape_and_cache(key, value, kc, vc, slots)
+    assert torch.equal(kg.cpu(), kc) and torch.equal(vg.cpu(), vc)
+    written = set(int(s) for s in slots if 0 <= s < P * bs)
+    flat = kg.cpu().view(P * bs, -1)
+    for s in range(P * bs):
+        if s not in written:
+            assert (flat[s] == 3.0).all()
+
+
+def test_independent_token_strides_and_unaligned_rows(device):
+    g = torch.Generator().manual_seed(11)
+    T, P, bs, H, D = 9, 3, 8, 2, 128
+    # K and V are slices of one fused qkv buffer: different offsets, a common long stride
+    qkv = torch.randn(T, 6 * H * D, generator=g).to(torch.bfloat16)
+    key = qkv[:, 2 * H * D : 3 * H * D].view(T, H, D)
+    value = qkv[:, 5 * H * D :].view(T, H, D)
+    slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+    dev_qkv = qkv.to(device)
+    kg = torch.zeros(P, bs, H, D, dtype=torch.bfloat16, device=device)
+    vg = torch.zeros_like(kg)
+    ops.reshape_paged_cache(ops.ReshapePagedCacheParams(
+        key=dev_qkv[:, 2 * H * D : 3 * H * D].view(T, H, D), value=dev_qkv[:, 5 * H * D :].view(T, H, D),
+        k_cache=kg, v_cache=vg, slot_mapping=slots.to(device)))
+    kc = torch.zeros(P, bs, H, D, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    oracle.reshape_and_cache(key, value, kc, vc, slots)
+    assert torch.equal(kg.cpu(), kc) and torch.equal(vg.cpu(), vc)
+    # head_dim 20 (40-byte rows): the element-wise kernel
+    key2 = torch.randn(5, 3, 20, generator=g).to(torch.float16)
+    val2 = torch.randn(5, 3, 20, generator=g).to(torch.float16)
+    s2 = torch.tensor([4, 0, 7, 2, 5], dtype=torch.int32)
+    (kc2, vc2), (kg2, vg2) = _run_both(key2, val2, s2, (2, 4, 3, 20), torch.float16, device)
+    assert torch.equal(kc2, kg2) and torch.equal(vc2, vg2)
+
+
+def test_mla_latent_store_without_value(device):
+    # k_cache.view({-1, 576}).index_copy_(0, slots, latent) of layers/dcu/deepseek_v2_attention.cpp:221-229
+    g = torch.Generator().manual_seed(5)
+    T, P, bs = 64, 8, 64
+    latent = (0.5 * torch.randn(T, 1, 576, generator=g)).to(torch.bfloat16)
+    slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+    (kc, _), (kg, _) = _run_both(latent, None, slots, (P, bs, 1, 576), torch.bfloat16, device)
+    expected = torch.zeros(P * bs, 576, dtype=torch.bfloat16)
+    expected.index_copy_(0, slots.to(torch.int64), latent.view(T, 576))
+    assert torch.equal(kg.view(P * bs, 576), expected) and torch.equal(kg, kc)
+
+
+def test_fp8_exhaustive_bf16_patterns_bit_exact(device):
+    # every bf16 bit pattern through the quantising store, several scales, vs the C oracle
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.bfloat16).view(512, 1, 128)
+    slots = torch.arange(512, dtype=torch.int32)
+    for scale in (1.0, 0.00390625, 0.013671875, 3.0e-3, 1.7, 1e-12, 37.5):
+        ks = torch.tensor([scale], dtype=torch.float32)
+        vs = torch.tensor([scale * 0.75], dtype=torch.float32)
+        (kc, vc), (kg, vg) = _run_both(x, x, slots, (32, 16, 1, 128), torch.float8_e4m3fn, device, ks, vs)
+        assert torch.equal(kc, kg), f"K codes differ at scale {scale}"
+        assert torch.equal(vc, vg), f"V codes differ at scale {scale}"
+
+
+def test_fp8_per_head_scales_fp16_fp32_inputs(device):
+    g = torch.Generator().manual_seed(99)
+    for dt in (torch.float16, torch.float32, torch.bfloat16):
+        T, P, bs, H, D = 40, 4, 16, 8, 128
+        key = (torch.randn(T, H, D, generator=g) * torch.linspace(0.1, 30, H).view(1, H, 1)).to(dt)
+        value = torch.randn(T, H, D, generator=g).to(dt)
+        slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+        ks = oracle.kv_head_scales(key)
+        vs = oracle.kv_head_scales(value)
+        gk = ops.kv_head_scales(key.to(device)).cpu()
+        gv = ops.kv_head_scales(value.to(device)).cpu()
+        assert torch.equal(gk, ks) and torch.equal(gv, vs), "per-head scales must match bit for bit"
+        (kc, vc), (kg, vg) = _run_both(key, value, slots, (P, bs, H, D), torch.float8_e4m3fn, device, ks, vs)
+        assert torch.equal(kc, kg) and torch.equal(vc, vg)
+        # properties the reference's fp8 tests check (tests/core/kernels/cuda/fp8_quant_test.cpp:70-82,321-348)
+        deq = kg.view(torch.float8_e4m3fn).float()
+        assert torch.isfinite(deq).all() and deq.abs().max() <= 448
+
+
+def test_prefill_sized_scatter_is_a_permutation(device):
+    # full-size property: scattering to a permutation of all slots and gathering back is the identity
+    g = torch.Generator(device=device).manual_seed(3)
+    P, bs, H, D = 2048, 16, 8, 128
+    T = P * bs
+    key = torch.randn(T, H, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    value = torch.randn(T, H, D, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    slots = torch.randperm(T, generator=g, device=device).to(torch.int32)
+    kg = torch.zeros(P, bs, H, D, dtype=torch.bfloat16, device=device)
+    vg = torch.zeros_like(kg)
+    ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=key, value=value, k_cache=kg, v_cache=vg,
+                                                        slot_mapping=slots))
+    assert torch.equal(kg.view(T, H, D)[slots.long()], key)
+    assert torch.equal(vg.view(T, H, D)[slots.long()], value)

@@ -1,0 +1,165 @@
+"""Pins the two attention oracles and the LSE merge without the GPU.
+
+aten_oracle.cpp restates the reference's libtorch decode op for op; paged_kv_oracle.c is exact
+fp64 softmax attention.  They are checked against each other, against closed forms and against
+the known answers the reference's own tests hold."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import fill_caches_cpu
+from xllm_amd import workloads
+
+
+def _setup(cfg, seed, dtype=torch.bfloat16):
+    inp = workloads.make_inputs(cfg, seed, dtype=dtype)
+    kc, vc = fill_caches_cpu(inp)
+    return inp, kc, vc
+
+
+def _dense_reference(inp, b):
+    """Textbook attention from the token streams, no paging at all (fp64)."""
+    cfg, lay = inp.cfg, inp.layout
+    lo, hi = int(lay.ctx_offsets[b]), int(lay.ctx_offsets[b + 1])
+    k = torch.cat([inp.k_ctx[lo:hi], inp.k_new[b : b + 1]]).double()
+    v = k[..., : cfg.dv] if cfg.mla else torch.cat([inp.v_ctx[lo:hi], inp.v_new[b : b + 1]]).double()
+    g = cfg.n_q_heads // cfg.n_kv_heads
+    q = inp.q[b].double()
+    outs, lses = [], []
+    for h in range(cfg.n_q_heads):
+        s = (k[:, h // g] @ q[h]) * cfg.scale
+        p = torch.softmax(s, 0)
+        outs.append(p @ v[:, h // g])
+        lses.append(torch.logsumexp(s, 0))
+    return torch.stack(outs), torch.stack(lses)
+
+
+@pytest.mark.parametrize("name,batch", [("tiny", 4), ("llama3_8b", 2), ("long_b256", 2), ("mla_dsv3", 1)])
+def test_f64_oracle_equals_dense_attention_and_aten_oracle_is_within_bf16_rounding(name, batch):
+    cfg = workloads.scaled(workloads.CONFIGS[name], batch=batch, len_hi=min(workloads.CONFIGS[name].len_hi, 3000))
+    inp, kc, vc = _setup(cfg, 11)
+    lay = inp.layout
+    out64, lse64 = oracle.paged_decode_f64(inp.q, kc, vc, lay.block_table, lay.seq_lens, cfg.scale, dv=cfg.dv)
+    for b in range(cfg.batch):
+        o, l = _dense_reference(inp, b)
+        assert torch.allclose(out64[b].double(), o, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(lse64[b].double(), l, rtol=1e-6, atol=1e-5)
+    aten = oracle.aten_paged_decode(inp.q, kc, vc, lay.block_table, lay.seq_lens, cfg.scale, dv=cfg.dv)
+    diff = (aten.float() - out64).abs()
+    assert diff.max() < 2e-3 and diff.mean() < 2e-4, (diff.max(), diff.mean())
+    lse = oracle.aten_paged_decode_lse(inp.q, kc, lay.block_table, lay.seq_lens, cfg.scale)
+    assert torch.allclose(lse, lse64, rtol=1e-4, atol=1e-4)
+
+
+def test_invariants_of_both_oracles():
+    cfg = workloads.DecodeConfig("inv", 3, 8, 2, 64, 16, 40, 90)
+    inp, kc, vc = _setup(cfg, 3)
+    lay = inp.layout
+    g = cfg.n_q_heads // cfg.n_kv_heads
+    # L = 1 -> V[0] of the mapped head (checks the head mapping h -> h / group too)
+    one = torch.ones_like(lay.seq_lens)
+    for fn in (lambda: oracle.aten_paged_decode(inp.q, kc, vc, lay.block_table, one, cfg.scale).float(),
+               lambda: oracle.paged_decode_f64(inp.q, kc, vc, lay.block_table, one, cfg.scale)[0]):
+        out = fn()
+        for b in range(cfg.batch):
+            v0 = vc[lay.block_table[b, 0].item(), 0].float()
+            assert torch.equal(out[b], v0.repeat_interleave(g, 0))
+    # equal K rows -> mean of V; equal V rows -> V
+    kc_eq = kc.clone()
+    kc_eq[:] = kc[0, 0]
+    out, _ = oracle.paged_decode_f64(inp.q, kc_eq, vc, lay.block_table, lay.seq_lens, cfg.scale)
+    for b in range(cfg.batch):
+        L = int(lay.seq_lens[b])
+        lo, hi = int(lay.ctx_offsets[b]), int(lay.ctx_offsets[b + 1])
+        vmean = torch.cat([inp.v_ctx[lo:hi], inp.v_new[b : b + 1]]).double().mean(0)
+        assert torch.allclose(out[b].double(), vmean.repeat_interleave(g, 0), atol=1e-6)
+    # page permutation
+    perm = torch.randperm(lay.num_blocks, generator=torch.Generator().manual_seed(4))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(lay.num_blocks)
+    t2 = inv[lay.block_table.long()].to(torch.int32)
+    a = oracle.aten_paged_decode(inp.q, kc, vc, lay.block_table, lay.seq_lens, cfg.scale)
+    b_ = oracle.aten_paged_decode(inp.q, kc[perm].contiguous(), vc[perm].contiguous(), t2, lay.seq_lens, cfg.scale)
+    assert torch.equal(a, b_)
+
+
+def test_csr_oracle_equals_block_table_oracle_at_default_scale():
+    cfg = workloads.DecodeConfig("csr", 4, 8, 4, 128, 16, 5, 300)
+    inp, kc, vc = _setup(cfg, 9)
+    lay = inp.layout
+    a = oracle.aten_paged_decode(inp.q, kc, vc, lay.block_table, lay.seq_lens, 1.0 / math.sqrt(128))
+    b = oracle.aten_paged_decode_csr(inp.q, kc, vc, lay.indptr, lay.indices, lay.last_page_len)
+    assert (a.float() - b.float()).abs().max() <= 2 ** -8 * a.float().abs().max()
+    table, lens = oracle.build_block_table(lay.indptr, lay.indices, lay.last_page_len, 40, 16)
+    assert torch.equal(lens, lay.seq_lens)
+    w = lay.block_table.shape[1]
+    for bb in range(cfg.batch):
+        n = int(lay.indptr[bb + 1] - lay.indptr[bb])
+        assert torch.equal(table[bb, :n], lay.block_table[bb, :n]) and (table[bb, n:] == -1).all()
+
+
+def test_mla_lse_closed_form_like_reference_test():
+    # MluMlaDecodeLseTest.ReturnsFloat32NaturalLogNormalizer
+    # (tests/core/layers/mlu/dcp_attention_merge_test.cpp:77-144): H=2, D=576, Dv=512, L=2
+    g = torch.Generator().manual_seed(0)
+    q = torch.rand(1, 2, 576, generator=g).to(torch.bfloat16)
+    cache = torch.rand(1, 16, 1, 576, generator=g).to(torch.bfloat16)
+    table = torch.zeros(1, 1, dtype=torch.int32)
+    lens = torch.tensor([2], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(576.0)
+    expected = torch.logsumexp((q[0].float() @ cache[0, :2, 0].float().T) * scale, -1)
+    _, lse64 = oracle.paged_decode_f64(q, cache, None, table, lens, scale, dv=512)
+    lse = oracle.aten_paged_decode_lse(q, cache, table, lens, scale)
+    assert lse.dtype == torch.float32 and tuple(lse.shape) == (1, 2)
+    assert torch.allclose(lse[0], expected, rtol=1e-3, atol=1e-3)
+    assert torch.allclose(lse64[0], expected, rtol=1e-3, atol=1e-3)
+    out = oracle.aten_paged_decode(q, cache, None, table, lens, scale, dv=512)
+    p = torch.softmax((q[0].float() @ cache[0, :2, 0].float().T) * scale, -1)
+    assert torch.allclose(out[0].float(), p @ cache[0, :2, 0, :512].float(), atol=1e-2)
+
+
+MERGE_FNS = [
+    lambda o, l: oracle.lse_merge(o, l),
+    lambda o, l: tuple(t.float() for t in oracle.aten_lse_merge(o, l)),
+]
+
+
+@pytest.mark.parametrize("merge", MERGE_FNS)
+def test_merge_known_answers_of_the_reference(merge):
+    # DcpAttentionMergeTest (tests/core/layers/mlu/dcp_attention_merge_test.cpp:34-75)
+    o = torch.tensor([2.0, 4.0, 6.0, 8.0]).reshape(2, 1, 1, 2)
+    l = torch.tensor([math.log(2.0), math.log(6.0)]).reshape(2, 1, 1)
+    out, lse = merge(o, l)
+    assert torch.allclose(out, torch.tensor([5.0, 7.0]).reshape(1, 1, 2))
+    assert torch.allclose(lse, torch.tensor([math.log(8.0)]).reshape(1, 1))
+    o = torch.tensor([0.0, 0.0, 3.0, 9.0]).reshape(2, 1, 1, 2)
+    l = torch.tensor([-math.inf, math.log(4.0)]).reshape(2, 1, 1)
+    out, lse = merge(o, l)
+    assert torch.equal(out, torch.tensor([3.0, 9.0]).reshape(1, 1, 2))
+    assert torch.allclose(lse, torch.tensor([math.log(4.0)]).reshape(1, 1))
+    o = torch.ones(2, 1, 2, 3)
+    l = torch.full((2, 1, 2), -math.inf)
+    out, lse = merge(o, l)
+    assert torch.equal(out, torch.zeros(1, 2, 3)) and torch.isneginf(lse).all()
+
+
+def test_merge_of_context_shards_equals_unsplit_decode():
+    # ArtificialShardMergeMatchesFullCacheDecode (same file :146-224), tolerances 1e-2 / 1e-3
+    cfg = workloads.DecodeConfig("m", 2, 4, 1, 576, 16, 40, 64, mla=True, v_dim=512, sigma=0.5,
+                                 sm_scale=1 / math.sqrt(576.0))
+    inp, kc, _ = _setup(cfg, 21)
+    lay = inp.layout
+    full, full_lse = oracle.paged_decode_f64(inp.q, kc, None, lay.block_table, lay.seq_lens, cfg.scale, dv=512)
+    # shard A: first 2 pages (32 tokens); shard B: the rest through a shifted table
+    la = torch.full_like(lay.seq_lens, 32)
+    lb = lay.seq_lens - 32
+    tb = torch.zeros_like(lay.block_table)
+    tb[:, :-2] = lay.block_table[:, 2:]
+    oa, lsa = oracle.paged_decode_f64(inp.q, kc, None, lay.block_table, la, cfg.scale, dv=512)
+    ob, lsb = oracle.paged_decode_f64(inp.q, kc, None, tb, lb, cfg.scale, dv=512)
+    for merge in MERGE_FNS:
+        out, lse = merge(torch.stack([oa, ob]), torch.stack([lsa, lsb]))
+        assert torch.allclose(out, full, rtol=1e-2, atol=1e-2) and torch.allclose(lse, full_lse, rtol=1e-3, atol=1e-3)
+        assert (out - full).abs().max() < 1e-5

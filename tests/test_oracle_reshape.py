@@ -1,0 +1,59 @@
+"""Pins the C oracle's reshape_and_cache: it is a permutation copy, so it is checked against
+torch indexing on the reference tests' own shape cases."""
+import pytest
+import torch
+
+import oracle
+
+CASES = [  # tests/core/kernels/dcu/reshape_paged_cache_test.cpp:135-158
+    (4, 1, 16, 1, 64, torch.float32),
+    (32, 8, 16, 4, 128, torch.float16),
+    (64, 4, 64, 8, 128, torch.bfloat16),
+    (256, 16, 64, 8, 128, torch.float16),
+    (1, 4, 16, 4, 128, torch.float32),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_matches_index_assignment(case):
+    T, P, bs, H, D, dt = case
+    g = torch.Generator().manual_seed(2026)
+    key = torch.randn(T, H, D, generator=g).to(dt)
+    value = torch.randn(T, H, D, generator=g).to(dt)
+    slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+    kc = torch.zeros(P, bs, H, D, dtype=dt)
+    vc = torch.zeros_like(kc)
+    oracle.reshape_and_cache(key, value, kc, vc, slots)
+    ek = torch.zeros(P * bs, H, D, dtype=dt)
+    ev = torch.zeros_like(ek)
+    ek[slots.long()] = key
+    ev[slots.long()] = value
+    assert torch.equal(kc.view(P * bs, H, D), ek) and torch.equal(vc.view(P * bs, H, D), ev)
+
+
+def test_npu_case_and_negative_slots_and_strides():
+    g = torch.Generator().manual_seed(20260730)
+    key = torch.randn(130, 1, 256, generator=g).to(torch.bfloat16)
+    value = torch.randn(130, 1, 256, generator=g).to(torch.bfloat16)
+    slots = torch.cat([torch.arange(256, 384), torch.arange(0, 2)]).to(torch.int32)
+    kc = torch.zeros(3, 128, 1, 256, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    oracle.reshape_and_cache(key, value, kc, vc, slots)
+    expected = torch.zeros_like(kc)
+    expected[2] = key[:128]
+    expected[0, :2] = key[128:]
+    assert torch.equal(kc, expected)
+    # negative slot skipped, independent strides
+    big = torch.randn(6, 4 * 2 * 32, generator=g).to(torch.float16)
+    k = big[:, 64:128].view(6, 2, 32)
+    v = big[:, 192:].view(6, 2, 32)
+    s = torch.tensor([3, -1, 0, 7, -5, 2], dtype=torch.int32)
+    kc = torch.full((2, 4, 2, 32), 9.0, dtype=torch.float16)
+    vc = torch.full((2, 4, 2, 32), 9.0, dtype=torch.float16)
+    oracle.reshape_and_cache(k, v, kc, vc, s)
+    flat_k, flat_v = kc.view(8, 2, 32), vc.view(8, 2, 32)
+    for t, slot in enumerate(s.tolist()):
+        if slot >= 0:
+            assert torch.equal(flat_k[slot], k[t]) and torch.equal(flat_v[slot], v[t])
+    for slot in (1, 4, 5, 6):
+        assert (flat_k[slot] == 9).all() and (flat_v[slot] == 9).all()

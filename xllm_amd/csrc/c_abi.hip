@@ -1,0 +1,119 @@
+// extern "C" surface of libxllm_mi355.so: plain pointers and sizes in, enqueue only.
+#include "launch.h"
+
+using namespace xllm_mi355;
+
+extern "C" {
+
+const char* xllm_mi355_version(void) { return "0.1.0"; }
+
+const char* xllm_mi355_error_string(int code) {
+  switch (code) {
+    case XLLM_MI355_OK: return "ok";
+    case XLLM_MI355_EINVAL: return "invalid argument (null pointer, non-positive size or bad stride)";
+    case XLLM_MI355_EDTYPE: return "dtype combination not implemented";
+    case XLLM_MI355_ESHAPE: return "head dim, group size or block size not implemented";
+    case XLLM_MI355_EWORKSPACE: return "split-K workspace missing, misaligned or too small";
+    case XLLM_MI355_EALIGN: return "pointer or stride not 16-byte aligned";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+  return "unknown error";
+}
+
+int xllm_mi355_reshape_and_cache(const void* key, const void* value, void* k_cache, void* v_cache,
+                                 const int32_t* slot_mapping, const float* k_scale,
+                                 const float* v_scale, int64_t n_tokens, int64_t n_kv_heads,
+                                 int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                 int64_t k_token_stride, int64_t v_token_stride, int in_dtype,
+                                 int cache_dtype, void* stream) {
+  return reshape_and_cache(key, value, k_cache, v_cache, slot_mapping, k_scale, v_scale, n_tokens,
+                           n_kv_heads, head_dim, block_size, num_blocks, k_token_stride,
+                           v_token_stride, in_dtype, cache_dtype, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_kv_head_scales(const void* x, float* scales, int64_t n_tokens, int64_t n_kv_heads,
+                              int64_t head_dim, int64_t token_stride, int in_dtype, void* stream) {
+  return kv_head_scales(x, scales, n_tokens, n_kv_heads, head_dim, token_stride, in_dtype,
+                        static_cast<hipStream_t>(stream));
+}
+
+size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t v_head_dim,
+                                               int64_t max_seq_len) {
+  if (batch <= 0 || n_q_heads <= 0 || v_head_dim <= 0) return 0;
+  // The fewest head blocks any layout of n_q_heads can have gives the most splits.
+  const int64_t head_blocks = (n_q_heads + 127) / 128;
+  const SplitPlan plan = plan_splits(batch, head_blocks, max_seq_len);
+  return split_workspace_bytes(batch, n_q_heads, v_head_dim, plan.max_splits);
+}
+
+int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                float* lse, const int32_t* block_table, int64_t table_stride,
+                                const int32_t* seq_lens, const float* k_scale, const float* v_scale,
+                                int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim,
+                                int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
+                                int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
+                                void* workspace, size_t workspace_bytes, int q_dtype, int cache_dtype,
+                                void* stream) {
+  PageAddressing addr;
+  addr.block_table = block_table;
+  addr.table_stride = table_stride;
+  addr.seq_lens = seq_lens;
+  return paged_decode_gqa(q, k_cache, v_cache, out, lse, addr, k_scale, v_scale, batch, n_q_heads,
+                          n_kv_heads, head_dim, block_size, num_blocks, q_token_stride,
+                          out_token_stride, max_seq_len, sm_scale, workspace, workspace_bytes, q_dtype,
+                          cache_dtype, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                    float* lse, const int32_t* paged_kv_indptr,
+                                    const int32_t* paged_kv_indices,
+                                    const int32_t* paged_kv_last_page_len, const float* k_scale,
+                                    const float* v_scale, int64_t batch, int64_t n_q_heads,
+                                    int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
+                                    int64_t num_blocks, int64_t q_token_stride,
+                                    int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
+                                    void* workspace, size_t workspace_bytes, int q_dtype,
+                                    int cache_dtype, void* stream) {
+  if (paged_kv_indptr == nullptr) return XLLM_MI355_EINVAL;
+  PageAddressing addr;
+  addr.indptr = paged_kv_indptr;
+  addr.indices = paged_kv_indices;
+  addr.last_page_len = paged_kv_last_page_len;
+  return paged_decode_gqa(q, k_cache, v_cache, out, lse, addr, k_scale, v_scale, batch, n_q_heads,
+                          n_kv_heads, head_dim, block_size, num_blocks, q_token_stride,
+                          out_token_stride, max_seq_len, sm_scale, workspace, workspace_bytes, q_dtype,
+                          cache_dtype, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out,
+                                float* lse, const int32_t* block_table, int64_t table_stride,
+                                const int32_t* seq_lens, int64_t batch, int64_t n_heads,
+                                int64_t d_latent, int64_t d_rope, int64_t block_size,
+                                int64_t num_blocks, int64_t max_seq_len, float sm_scale,
+                                void* workspace, size_t workspace_bytes, int dtype, void* stream) {
+  PageAddressing addr;
+  addr.block_table = block_table;
+  addr.table_stride = table_stride;
+  addr.seq_lens = seq_lens;
+  return paged_decode_mla(q_nope, q_pe, k_cache, out, lse, addr, batch, n_heads, d_latent, d_rope,
+                          block_size, num_blocks, max_seq_len, sm_scale, workspace, workspace_bytes,
+                          dtype, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,
+                         int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim,
+                         int dtype, void* stream) {
+  return lse_merge(partial_out, partial_lse, out, lse, n_shards, batch, n_heads, v_head_dim, dtype,
+                   static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr, const int32_t* paged_kv_indices,
+                                 const int32_t* paged_kv_last_page_len, int32_t* block_table,
+                                 int64_t table_stride, int32_t* seq_lens, int64_t batch,
+                                 int64_t block_size, void* stream) {
+  return build_block_table(paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len, block_table,
+                           table_stride, seq_lens, batch, block_size, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

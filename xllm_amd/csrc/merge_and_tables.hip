@@ -1,0 +1,106 @@
+// Small data-movement kernels either side of the decode kernels:
+//   lse_merge          -- log-sum-exp merge of S partial attention results
+//                         (xllm/core/layers/mlu/dcp_attention_merge.cpp:26-65)
+//   build_block_table  -- CSR page lists -> padded [B, stride] table, -1 fill
+//                         (xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip:44-149)
+#include "common.cuh"
+#include "launch.h"
+
+namespace xllm_mi355 {
+
+namespace {
+
+// One workgroup per (batch, head).  natural-log LSE in and out, fp32 arithmetic in the
+// order of the reference: max over shards, weights exp(lse - max) with non-finite
+// shards weighted 0, weighted sum, division by the weight sum.
+template <int DT>
+__global__ __launch_bounds__(128) void lse_merge_kernel(const char* partial_out,
+                                                        const float* partial_lse, char* out,
+                                                        float* lse, int n_shards, int64_t bh, int dv) {
+  constexpr int ES = DT == XLLM_MI355_FP32 ? 4 : 2;
+  const int64_t i = blockIdx.x;
+  float mx = -INFINITY;
+  for (int s = 0; s < n_shards; ++s) mx = fmaxf(mx, partial_lse[s * bh + i]);
+  const float safe_max = isfinite(mx) ? mx : 0.0f;
+  float wsum = 0.0f;
+  for (int s = 0; s < n_shards; ++s) {
+    const float v = partial_lse[s * bh + i];
+    wsum += isfinite(v) ? expf(v - safe_max) : 0.0f;
+  }
+  for (int d = threadIdx.x; d < dv; d += 128) {
+    float o = 0.0f;
+    for (int s = 0; s < n_shards; ++s) {
+      const float v = partial_lse[s * bh + i];
+      const float w = isfinite(v) ? expf(v - safe_max) : 0.0f;
+      const char* p = partial_out + ((s * bh + i) * dv + d) * ES;
+      float x;
+      if constexpr (DT == XLLM_MI355_FP32) x = *reinterpret_cast<const float*>(p);
+      else if constexpr (DT == XLLM_MI355_BF16) x = BF16::to_f32(*reinterpret_cast<const uint16_t*>(p));
+      else x = FP16::to_f32(*reinterpret_cast<const uint16_t*>(p));
+      o += x * w;
+    }
+    const float val = wsum > 0.0f ? o / wsum : 0.0f;
+    char* q = out + (i * dv + d) * ES;
+    if constexpr (DT == XLLM_MI355_FP32) *reinterpret_cast<float*>(q) = val;
+    else if constexpr (DT == XLLM_MI355_BF16) *reinterpret_cast<uint16_t*>(q) = BF16::from_f32(val);
+    else *reinterpret_cast<uint16_t*>(q) = FP16::from_f32(val);
+  }
+  if (lse != nullptr && threadIdx.x == 0) lse[i] = wsum > 0.0f ? safe_max + logf(wsum) : -INFINITY;
+}
+
+__global__ __launch_bounds__(256) void build_block_table_kernel(const int32_t* indptr,
+                                                                const int32_t* indices,
+                                                                const int32_t* last_page_len,
+                                                                int32_t* table, int64_t stride,
+                                                                int32_t* seq_lens, int block_size) {
+  const int b = blockIdx.x;
+  const int p0 = indptr[b];
+  const int n = indptr[b + 1] - p0;
+  for (int64_t j = threadIdx.x; j < stride; j += 256)
+    table[b * stride + j] = j < n ? indices[p0 + j] : -1;
+  if (seq_lens != nullptr && threadIdx.x == 0)
+    seq_lens[b] = n > 0 ? (n - 1) * block_size + last_page_len[b] : 0;
+}
+
+}  // namespace
+
+int lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,
+              int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim, int dtype,
+              hipStream_t stream) {
+  if (batch == 0 || n_heads == 0) return XLLM_MI355_OK;
+  if (partial_out == nullptr || partial_lse == nullptr || out == nullptr) return XLLM_MI355_EINVAL;
+  if (n_shards <= 0 || batch < 0 || n_heads < 0 || v_head_dim <= 0) return XLLM_MI355_EINVAL;
+  const int64_t bh = batch * n_heads;
+  if (bh > 0x7fffffffLL || n_shards > 0x7fffffffLL) return XLLM_MI355_ESHAPE;
+  dim3 grid(static_cast<unsigned>(bh));
+  const char* po = static_cast<const char*>(partial_out);
+  char* o = static_cast<char*>(out);
+  const int s = static_cast<int>(n_shards), dv = static_cast<int>(v_head_dim);
+  switch (dtype) {
+    case XLLM_MI355_BF16:
+      lse_merge_kernel<XLLM_MI355_BF16><<<grid, 128, 0, stream>>>(po, partial_lse, o, lse, s, bh, dv);
+      break;
+    case XLLM_MI355_FP16:
+      lse_merge_kernel<XLLM_MI355_FP16><<<grid, 128, 0, stream>>>(po, partial_lse, o, lse, s, bh, dv);
+      break;
+    case XLLM_MI355_FP32:
+      lse_merge_kernel<XLLM_MI355_FP32><<<grid, 128, 0, stream>>>(po, partial_lse, o, lse, s, bh, dv);
+      break;
+    default: return XLLM_MI355_EDTYPE;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+int build_block_table(const int32_t* indptr, const int32_t* indices, const int32_t* last_page_len,
+                      int32_t* block_table, int64_t table_stride, int32_t* seq_lens, int64_t batch,
+                      int64_t block_size, hipStream_t stream) {
+  if (batch == 0) return XLLM_MI355_OK;
+  if (indptr == nullptr || indices == nullptr || block_table == nullptr) return XLLM_MI355_EINVAL;
+  if (seq_lens != nullptr && last_page_len == nullptr) return XLLM_MI355_EINVAL;
+  if (batch < 0 || batch > 0x7fffffffLL || table_stride <= 0 || block_size <= 0) return XLLM_MI355_EINVAL;
+  build_block_table_kernel<<<dim3(static_cast<unsigned>(batch)), 256, 0, stream>>>(
+      indptr, indices, last_page_len, block_table, table_stride, seq_lens, static_cast<int>(block_size));
+  return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace xllm_mi355

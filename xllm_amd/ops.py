@@ -1,0 +1,332 @@
+"""Host-side mirror of the reference's kernel op interface for the paged-KV decode path,
+over the C ABI.  torch is used for device memory and the current stream only.
+
+Reference interface mirrored here (paths relative to the xLLM source tree):
+  ReshapePagedCacheParams / reshape_paged_cache   xllm/core/kernels/param.h:126-161, ops_api.h:31
+  quant_to_paged_cache                            xllm/core/kernels/ops_api.cpp:296-310
+  batch_decode (block table + seq_lens)           xllm/core/kernels/npu/npu_ops_api.h:46,
+                                                  xllm/core/kernels/mlu/mlu_ops_api.h:127
+  batch_decode (CSR)                              xllm/core/kernels/cuda/cuda_ops_api.h:128-144
+  flash_mla::DenseDecodeParams / dense_decode     xllm/core/kernels/dcu/flash_mla_adapter.h:40-53
+  merge_dcp_attention_shards                      xllm/core/layers/mlu/dcp_attention_merge.h:28-34
+  build_block_table_from_paged_kv                 xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip
+
+Errors: the reference CHECK-aborts; here every violated precondition raises.
+"""
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import capi
+
+_DT = {torch.bfloat16: capi.BF16, torch.float16: capi.FP16, torch.float32: capi.FP32,
+       torch.float8_e4m3fn: capi.FP8_E4M3, torch.uint8: capi.FP8_E4M3}
+
+
+def _dtype_code(t):
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}") from None
+
+
+def _stream(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _require_cuda(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("this path runs on the GPU only: every tensor must be a device tensor")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError("all tensors must live on the same device")
+    return dev
+
+
+# ------------------------------------------------------------------------------------------
+# workspace: one per device, grown on demand, same lifetime as the reference's
+# FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41)
+
+_workspaces = {}
+
+
+def decode_workspace(device, nbytes):
+    ws = _workspaces.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[device] = ws
+    return ws
+
+
+# ------------------------------------------------------------------------------------------
+# op 1
+
+@dataclass
+class ReshapePagedCacheParams:
+    """Field for field the reference struct (xllm/core/kernels/param.h:126-161).  For the fp8
+    cache of this build k_cache_scale / v_cache_scale are per-KV-head [Hkv] fp32."""
+    key: torch.Tensor
+    k_cache: torch.Tensor
+    slot_mapping: torch.Tensor
+    value: Optional[torch.Tensor] = None
+    v_cache: Optional[torch.Tensor] = None
+    direction: bool = False
+    k_cache_scale: Optional[torch.Tensor] = None
+    v_cache_scale: Optional[torch.Tensor] = None
+
+
+def _reshape(params, quantized):
+    key, value = params.key, params.value
+    k_cache, v_cache = params.k_cache, params.v_cache
+    slots = params.slot_mapping
+    dev = _require_cuda(key, value, k_cache, v_cache, slots, params.k_cache_scale, params.v_cache_scale)
+    if params.direction:
+        raise NotImplementedError("CACHE2CONTEXT is MLU-only in the reference and not part of this path")
+    if key.dim() != 3 or k_cache.dim() != 4:
+        raise ValueError("key must be [T, Hkv, D] and k_cache [P, bs, Hkv, D]")
+    if (value is None) != (v_cache is None):
+        raise ValueError("value and v_cache must be given together")
+    T, Hkv, D = key.shape
+    if not (key.stride(-1) == 1 and key.stride(-2) == D):
+        raise ValueError("key: last two dims must be contiguous")
+    if value is not None and not (value.stride(-1) == 1 and value.stride(-2) == D and value.shape == key.shape):
+        raise ValueError("value: last two dims must be contiguous and the shape must match key")
+    if not k_cache.is_contiguous() or (v_cache is not None and not v_cache.is_contiguous()):
+        raise ValueError("caches must be contiguous")
+    if tuple(k_cache.shape[2:]) != (Hkv, D):
+        raise ValueError("k_cache heads / head_dim do not match key")
+    if slots.dtype != torch.int32 or not slots.is_contiguous() or slots.numel() != T:
+        raise ValueError("slot_mapping must be contiguous int32 [T]")
+    if quantized:
+        if params.k_cache_scale is None:
+            raise ValueError("k_cache_scale is required for quant_to_paged_cache")
+        for s in (params.k_cache_scale, params.v_cache_scale):
+            if s is not None and (s.dtype != torch.float32 or s.numel() != Hkv or not s.is_contiguous()):
+                raise ValueError("cache scales must be contiguous fp32 [Hkv]")
+    elif k_cache.dtype != key.dtype:
+        raise ValueError("key and k_cache must have the same dtype (use quant_to_paged_cache for fp8)")
+    P, bs = k_cache.shape[0], k_cache.shape[1]
+    rc = capi.lib().xllm_mi355_reshape_and_cache(
+        key.data_ptr(), _ptr(value), k_cache.data_ptr(), _ptr(v_cache), slots.data_ptr(),
+        _ptr(params.k_cache_scale) if quantized else None,
+        _ptr(params.v_cache_scale) if quantized else None,
+        T, Hkv, D, bs, P, key.stride(0), 0 if value is None else value.stride(0),
+        _dtype_code(key), _dtype_code(k_cache), _stream(dev))
+    capi.check(rc, "xllm_mi355_reshape_and_cache")
+
+
+def reshape_paged_cache(params: ReshapePagedCacheParams):
+    """xllm::kernel::reshape_paged_cache (ops_api.cpp:248-278): scales are ignored, dtypes equal."""
+    _reshape(params, quantized=False)
+
+
+def quant_to_paged_cache(params: ReshapePagedCacheParams):
+    """xllm::kernel::quant_to_paged_cache (ops_api.cpp:296-310), fp8 e4m3fn with per-head scales."""
+    _reshape(params, quantized=True)
+
+
+def kv_head_scales(x):
+    """scale[h] = max(absmax(x[:, h, :]) / 448, 1e-12) (fp8_scaled_quantize.cpp:38-42, per KV head)."""
+    dev = _require_cuda(x)
+    T, Hkv, D = x.shape
+    if not (x.stride(-1) == 1 and x.stride(-2) == D):
+        raise ValueError("x: last two dims must be contiguous")
+    out = torch.empty(Hkv, dtype=torch.float32, device=dev)
+    rc = capi.lib().xllm_mi355_kv_head_scales(x.data_ptr(), out.data_ptr(), T, Hkv, D, x.stride(0),
+                                              _dtype_code(x), _stream(dev))
+    capi.check(rc, "xllm_mi355_kv_head_scales")
+    return out
+
+
+# ------------------------------------------------------------------------------------------
+# op 2
+
+def _decode_common(query, k_cache, output):
+    if query.dim() != 3:
+        raise ValueError("query must be [B, Hq, D]")
+    if not (query.stride(-1) == 1 and query.stride(-2) == query.shape[-1]):
+        raise ValueError("query: last two dims must be contiguous")
+    if not (output.stride(-1) == 1 and output.stride(-2) == output.shape[-1]):
+        raise ValueError("output: last two dims must be contiguous")
+    if not k_cache.is_contiguous() or k_cache.dim() != 4:
+        raise ValueError("k_cache must be contiguous [P, bs, Hkv, D]")
+
+
+def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, output_lse=None,
+                 k_cache_quant_scale=None, v_cache_quant_scale=None, scale=None, return_lse=False,
+                 max_seq_len=0):
+    """Block-table paged decode.  Argument order and meaning follow mlu::batch_decode
+    (mlu_ops_api.h:127) restricted to what npu::batch_decode (npu_ops_api.h:46) also has.
+    query/output [B, Hq, D]; caches [P, bs, Hkv, D]; block_table [B, W] int32; seq_lens [B] int32.
+    Returns (output, lse or None) with lse [B, Hq, 1] fp32 natural log."""
+    if v_cache is None:
+        raise ValueError("GQA decode needs v_cache; the latent-KV variant is dense_decode")
+    dev = _require_cuda(query, k_cache, v_cache, output, block_table, seq_lens, output_lse,
+                        k_cache_quant_scale, v_cache_quant_scale)
+    _decode_common(query, k_cache, output)
+    B, Hq, D = query.shape
+    P, bs, Hkv, _ = k_cache.shape
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise ValueError("block_table must be int32 [B, W] with unit column stride")
+    if seq_lens.dtype != torch.int32 or seq_lens.numel() != B or not seq_lens.is_contiguous():
+        raise ValueError("seq_lens must be contiguous int32 [B]")
+    if block_table.shape[0] != B:
+        raise ValueError("block_table rows must equal the batch")
+    if scale is None:
+        scale = D ** -0.5
+    lse = None
+    if return_lse or output_lse is not None:
+        lse = output_lse if output_lse is not None else torch.empty(B, Hq, 1, dtype=torch.float32, device=dev)
+        if lse.dtype != torch.float32 or lse.numel() != B * Hq or not lse.is_contiguous():
+            raise ValueError("output_lse must be contiguous fp32 [B, Hq, 1]")
+    if max_seq_len <= 0:
+        max_seq_len = block_table.shape[1] * bs
+    lib = capi.lib()
+    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len)
+    ws = decode_workspace(dev, nbytes)
+    rc = lib.xllm_mi355_paged_decode_gqa(
+        query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(lse),
+        block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(),
+        _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D, bs, P,
+        query.stride(0), output.stride(0), max_seq_len, float(scale), ws.data_ptr(), ws.numel(),
+        _dtype_code(query), _dtype_code(k_cache), _stream(dev))
+    capi.check(rc, "xllm_mi355_paged_decode_gqa")
+    return output, lse
+
+
+def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
+                     paged_kv_last_page_len, sm_scale, output, output_lse=None, max_seq_len=0,
+                     k_cache_quant_scale=None, v_cache_quant_scale=None):
+    """CSR paged decode: cuda::batch_decode (cuda_ops_api.h:128-144) without the FlashInfer
+    uri / plan_info / workspace arguments.  max_seq_len bounds the longest context; 0 means
+    "all pages of the call could belong to one sequence"."""
+    dev = _require_cuda(query, k_cache, v_cache, output, paged_kv_indptr, paged_kv_indices,
+                        paged_kv_last_page_len, output_lse)
+    _decode_common(query, k_cache, output)
+    B, Hq, D = query.shape
+    P, bs, Hkv, _ = k_cache.shape
+    for t, n in ((paged_kv_indptr, B + 1), (paged_kv_last_page_len, B)):
+        if t.dtype != torch.int32 or t.numel() != n or not t.is_contiguous():
+            raise ValueError("CSR arrays must be contiguous int32 of the documented sizes")
+    if paged_kv_indices.dtype != torch.int32 or not paged_kv_indices.is_contiguous():
+        raise ValueError("paged_kv_indices must be contiguous int32")
+    if max_seq_len <= 0:
+        max_seq_len = max(1, paged_kv_indices.numel()) * bs
+    lib = capi.lib()
+    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len)
+    ws = decode_workspace(dev, nbytes)
+    rc = lib.xllm_mi355_paged_decode_gqa_csr(
+        query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(output_lse),
+        paged_kv_indptr.data_ptr(), paged_kv_indices.data_ptr(), paged_kv_last_page_len.data_ptr(),
+        _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D, bs, P,
+        query.stride(0), output.stride(0), max_seq_len, float(sm_scale), ws.data_ptr(), ws.numel(),
+        _dtype_code(query), _dtype_code(k_cache), _stream(dev))
+    capi.check(rc, "xllm_mi355_paged_decode_gqa_csr")
+    return output
+
+
+@dataclass
+class DenseDecodeParams:
+    """flash_mla::DenseDecodeParams (xllm/core/kernels/dcu/flash_mla_adapter.h:40-53)."""
+    q_nope: torch.Tensor       # [B, S_q, H, kv_lora_rank]
+    q_pe: torch.Tensor         # [B, S_q, H, rope]
+    k_cache: torch.Tensor      # [P, bs, 1, kv_lora_rank + rope]
+    seqlens_k: torch.Tensor    # [B] int32
+    block_table: torch.Tensor  # [B, W] int32
+    head_size_v: int = 0
+    softmax_scale: float = -1.0
+    is_causal: bool = False
+
+
+def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0):
+    """flash_mla::dense_decode (flash_mla_adapter.cpp:104-153): returns [B, S_q, H, head_size_v]
+    (and lse [B, H, 1] when asked).  The same argument checks; S_q must be 1 on this path."""
+    p = params
+    dev = _require_cuda(p.q_nope, p.q_pe, p.k_cache, p.seqlens_k, p.block_table)
+    if p.q_nope.dim() != 4 or p.q_pe.dim() != 4:
+        raise ValueError("flash_mla: q_nope / q_pe must be 4D [B,S_q,H_q,D]")
+    if p.k_cache.dim() != 4 or p.k_cache.shape[2] != 1:
+        raise ValueError("flash_mla: k_cache must be 4D [blocks,page,1,D] with a single KV head")
+    B, Sq, H, d_latent = p.q_nope.shape
+    d_rope = p.q_pe.shape[3]
+    if p.q_pe.shape[:3] != p.q_nope.shape[:3]:
+        raise ValueError("flash_mla: q_nope/q_pe batch, seq and head count must match")
+    if p.k_cache.shape[3] != d_latent + d_rope:
+        raise ValueError("flash_mla: k_cache last dim must equal q_nope.dim + q_pe.dim")
+    if p.head_size_v <= 0:
+        raise ValueError("flash_mla: head_size_v must be positive")
+    if p.softmax_scale <= 0:
+        raise ValueError("flash_mla: softmax_scale must be set by the MLA attention layer")
+    if Sq != 1:
+        raise NotImplementedError("decode path: one query token per sequence")
+    if p.head_size_v != d_latent:
+        raise NotImplementedError("V is the latent part of the cache: head_size_v must equal kv_lora_rank")
+    seqlens = p.seqlens_k if p.seqlens_k.dtype == torch.int32 else p.seqlens_k.to(torch.int32)
+    table = p.block_table if p.block_table.dtype == torch.int32 else p.block_table.to(torch.int32)
+    q_nope = p.q_nope.contiguous()
+    q_pe = p.q_pe.contiguous()
+    P, bs = p.k_cache.shape[0], p.k_cache.shape[1]
+    out = torch.empty(B, Sq, H, p.head_size_v, dtype=q_nope.dtype, device=dev)
+    lse = torch.empty(B, H, 1, dtype=torch.float32, device=dev) if return_lse else None
+    if max_seq_len <= 0:
+        max_seq_len = table.shape[1] * bs
+    lib = capi.lib()
+    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, H, d_latent, max_seq_len)
+    ws = decode_workspace(dev, nbytes)
+    rc = lib.xllm_mi355_paged_decode_mla(
+        q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), _ptr(lse),
+        table.data_ptr(), table.stride(0), seqlens.data_ptr(), B, H, d_latent, d_rope, bs, P,
+        max_seq_len, float(p.softmax_scale), ws.data_ptr(), ws.numel(), _dtype_code(q_nope),
+        _stream(dev))
+    capi.check(rc, "xllm_mi355_paged_decode_mla")
+    return (out, lse) if return_lse else out
+
+
+# ------------------------------------------------------------------------------------------
+# merge and table helpers
+
+def merge_dcp_attention_shards(partial_outputs, partial_lse):
+    """merge_dcp_attention_shards (dcp_attention_merge.cpp:26-65).
+    partial_outputs [S, B, Q=1, H, Dv]; partial_lse [S, B, H, Q=1] -> (output [B,1,H,Dv], lse [B,H,1])."""
+    dev = _require_cuda(partial_outputs, partial_lse)
+    if partial_outputs.dim() != 5:
+        raise ValueError("partial outputs must have shape [dcp, batch, query, heads, value]")
+    if partial_lse.dim() != 4:
+        raise ValueError("partial LSE must have shape [dcp, batch, heads, query]")
+    S, B, Q, H, Dv = partial_outputs.shape
+    if tuple(partial_lse.shape) != (S, B, H, Q):
+        raise ValueError("partial outputs and LSE disagree on [dcp, batch, heads, query]")
+    if Q != 1:
+        raise NotImplementedError("decode path: one query token per sequence")
+    po = partial_outputs.contiguous()
+    pl = partial_lse.to(torch.float32).contiguous()
+    out = torch.empty(B, Q, H, Dv, dtype=po.dtype, device=dev)
+    lse = torch.empty(B, H, Q, dtype=torch.float32, device=dev)
+    rc = capi.lib().xllm_mi355_lse_merge(po.data_ptr(), pl.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                                         S, B, H, Dv, _dtype_code(po), _stream(dev))
+    capi.check(rc, "xllm_mi355_lse_merge")
+    return out, lse
+
+
+def build_block_table_from_paged_kv(paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len,
+                                    table_width, block_size):
+    """CSR -> (block_table [B, table_width] int32 with -1 padding, seq_lens [B] int32)."""
+    dev = _require_cuda(paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len)
+    B = paged_kv_indptr.numel() - 1
+    table = torch.empty(B, table_width, dtype=torch.int32, device=dev)
+    seq_lens = torch.empty(B, dtype=torch.int32, device=dev)
+    rc = capi.lib().xllm_mi355_build_block_table(
+        paged_kv_indptr.data_ptr(), paged_kv_indices.data_ptr(), paged_kv_last_page_len.data_ptr(),
+        table.data_ptr(), table_width, seq_lens.data_ptr(), B, block_size, _stream(dev))
+    capi.check(rc, "xllm_mi355_build_block_table")
+    return table, seq_lens
