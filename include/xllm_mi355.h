@@ -204,6 +204,18 @@ int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr,
                                  int32_t* seq_lens,
                                  int64_t batch, int64_t block_size, void* stream);
 
+/*
+ * Opt-in timing of the dominant decode kernel.  No counterpart in the reference, which
+ * relies on external profilers (xllm/core/platform/cuda_profiler.cpp,
+ * xllm/core/platform/torch_profiler.cpp).  After xllm_mi355_profile_enable(n) the next n
+ * calls of a decode entry point record a HIP event pair around their main kernel on the
+ * caller's stream; xllm_mi355_profile_collect waits for them, writes the elapsed
+ * milliseconds of each (host pointer) and returns how many, or a value < -1000 on a HIP
+ * error.  Process-wide, single caller thread, not usable under graph capture.
+ */
+int xllm_mi355_profile_enable(int capacity);
+int xllm_mi355_profile_collect(float* ms_out, int max_n);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,6 +35,8 @@ SIGNATURES = {
                                            _i64, _i64, _i64, _f32, _p, _sz, _i32, _p]),
     "xllm_mi355_lse_merge": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "xllm_mi355_build_block_table": (_i32, [_p, _p, _p, _p, _i64, _p, _i64, _i64, _p]),
+    "xllm_mi355_profile_enable": (_i32, [_i32]),
+    "xllm_mi355_profile_collect": (_i32, [_p, _i32]),
 }
 
 _lib = None

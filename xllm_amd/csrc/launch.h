@@ -63,4 +63,9 @@ int build_block_table(const int32_t* indptr, const int32_t* indices, const int32
                       int32_t* block_table, int64_t table_stride, int32_t* seq_lens, int64_t batch,
                       int64_t block_size, hipStream_t stream);
 
+// Opt-in timing of the dominant kernel (profile.hip).  profile_begin returns true when a
+// start event was recorded; the caller then must call profile_end after its launch.
+bool profile_begin(hipStream_t stream);
+void profile_end(hipStream_t stream);
+
 }  // namespace xllm_mi355

@@ -554,12 +554,14 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
   }
 
   int rc;
+  const bool timed = profile_begin(stream);
   if (q_dtype == XLLM_MI355_BF16)
     rc = fp8 ? dispatch_dim<BF16, true>(a, batch, static_cast<int>(head_dim), g_block, stream)
              : dispatch_dim<BF16, false>(a, batch, static_cast<int>(head_dim), g_block, stream);
   else
     rc = fp8 ? dispatch_dim<FP16, true>(a, batch, static_cast<int>(head_dim), g_block, stream)
              : dispatch_dim<FP16, false>(a, batch, static_cast<int>(head_dim), g_block, stream);
+  if (timed) profile_end(stream);
   if (rc != 0 || plan.max_splits <= 1) return rc;
   return merge_splits(a.ws_out, a.ws_lse, out, lse, addr, batch, n_q_heads, head_dim, block_size,
                       out_token_stride, plan.chunk_tokens, plan.max_splits, q_dtype, stream);
