@@ -1,0 +1,122 @@
+"""GPU parity of the MLA latent-KV paged decode against the reference's libtorch CPU path."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close_to_reference, fill_caches_cpu, fill_caches_gpu
+from xllm_amd import ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode_gpu(inp, k_cache, device, return_lse=True, table=None, seq_lens=None):
+    cfg, lay = inp.cfg, inp.layout
+    q = inp.q.to(device)
+    B, H = cfg.batch, cfg.n_q_heads
+    lens = lay.seq_lens if seq_lens is None else seq_lens
+    p = ops.DenseDecodeParams(
+        q_nope=q[:, :, : cfg.v_dim].contiguous().view(B, 1, H, cfg.v_dim),
+        q_pe=q[:, :, cfg.v_dim :].contiguous().view(B, 1, H, cfg.head_dim - cfg.v_dim),
+        k_cache=k_cache, seqlens_k=lens.to(device),
+        block_table=(lay.block_table if table is None else table).to(device),
+        head_size_v=cfg.v_dim, softmax_scale=cfg.scale)
+    res = ops.dense_decode(p, return_lse=return_lse, max_seq_len=int(lens.max()))
+    torch.cuda.synchronize()
+    if return_lse:
+        return res[0].view(B, H, cfg.v_dim), res[1].view(B, H)
+    return res.view(B, H, cfg.v_dim), None
+
+
+def _mla_cfg(name, batch, heads, lo, hi, bs=64):
+    return workloads.DecodeConfig(name, batch, heads, 1, 576, bs, lo, hi, mla=True, v_dim=512, sigma=0.5,
+                                  sm_scale=1.0 / math.sqrt(192.0))
+
+
+def _check(cfg, seed, device):
+    inp = workloads.make_inputs(cfg, seed)
+    lay = inp.layout
+    kg, _, _, _ = fill_caches_gpu(inp, device)
+    kc, _ = fill_caches_cpu(inp)
+    assert torch.equal(kg.cpu(), kc), "latent cache bytes must be bit-exact"
+    out, lse = _decode_gpu(inp, kg, device)
+    ref = oracle.aten_paged_decode(inp.q, kc, None, lay.block_table, lay.seq_lens, cfg.scale, dv=cfg.v_dim)
+    assert_close_to_reference(out, ref, cfg.name)
+    ref_lse = oracle.aten_paged_decode_lse(inp.q, kc, lay.block_table, lay.seq_lens, cfg.scale)
+    assert torch.allclose(lse.cpu(), ref_lse, rtol=1e-3, atol=1e-3)
+    return inp, kg, out, lse
+
+
+def test_config5_shape_reduced_batch_and_context(device):
+    _check(_mla_cfg("mla128", 3, 128, 100, 1500), 5, device)
+
+
+def test_head_counts_of_tp_shards_and_reference_test_shape(device):
+    # 128 heads / tp; H = 2 is the shape of MluMlaDecodeLseTest (dcp_attention_merge_test.cpp:77-144)
+    for heads in (2, 16, 32, 64, 80):
+        _check(_mla_cfg(f"mla{heads}", 2, heads, 1, 400), 40 + heads, device)
+
+
+def test_reference_lse_closed_form_two_tokens(device):
+    # ReturnsFloat32NaturalLogNormalizer: H=2, D=576, Dv=512, L=2, page of 16 rows, scale 1/sqrt(576)
+    g = torch.Generator().manual_seed(0)
+    q = torch.rand(1, 2, 576, generator=g).to(torch.bfloat16)
+    cache = torch.rand(1, 16, 1, 576, generator=g).to(torch.bfloat16)
+    scale = 1.0 / math.sqrt(576.0)
+    p = ops.DenseDecodeParams(
+        q_nope=q[:, :, :512].contiguous().view(1, 1, 2, 512).to(device),
+        q_pe=q[:, :, 512:].contiguous().view(1, 1, 2, 64).to(device), k_cache=cache.to(device),
+        seqlens_k=torch.tensor([2], dtype=torch.int32, device=device),
+        block_table=torch.zeros(1, 1, dtype=torch.int32, device=device), head_size_v=512, softmax_scale=scale)
+    out, lse = ops.dense_decode(p, return_lse=True)
+    assert lse.dtype == torch.float32 and tuple(lse.shape) == (1, 2, 1)
+    scores = (q[0].float() @ cache[0, :2, 0].float().T) * scale
+    assert torch.allclose(lse.cpu().view(2), torch.logsumexp(scores, -1), rtol=1e-3, atol=1e-3)
+    expect = torch.softmax(scores, -1) @ cache[0, :2, 0, :512].float()
+    assert torch.allclose(out.cpu().float().view(2, 512), expect, atol=1e-2)
+
+
+def test_block_sizes_other_than_64_and_long_context_splits(device):
+    _check(_mla_cfg("bs16", 2, 16, 50, 700, bs=16), 3, device)
+    _check(_mla_cfg("bs128", 2, 32, 50, 900, bs=128), 4, device)
+    _check(_mla_cfg("long", 1, 128, 6000, 9000), 6, device)
+
+
+def test_shard_merge_equals_full_decode(device):
+    # ArtificialShardMergeMatchesFullCacheDecode (dcp_attention_merge_test.cpp:146-224): rtol/atol 1e-2, 1e-3
+    cfg = _mla_cfg("merge", 4, 128, 256, 2000)
+    inp, kg, full, full_lse = _check(cfg, 9, device)
+    lay = inp.layout
+    bs = cfg.block_size
+    n_pages = (lay.seq_lens + bs - 1) // bs
+    h = (n_pages + 1) // 2
+    len_a = torch.minimum(lay.seq_lens, h * bs)
+    len_b = lay.seq_lens - len_a
+    table_b = torch.zeros_like(lay.block_table)
+    for b in range(cfg.batch):
+        nb = int(n_pages[b] - h[b])
+        table_b[b, :nb] = lay.block_table[b, int(h[b]) : int(h[b]) + nb]
+    oa, la = _decode_gpu(inp, kg, device, seq_lens=len_a)
+    ob, lb = _decode_gpu(inp, kg, device, table=table_b, seq_lens=len_b)
+    B, H = cfg.batch, cfg.n_q_heads
+    merged, mlse = ops.merge_dcp_attention_shards(
+        torch.stack([oa.view(B, 1, H, 512), ob.view(B, 1, H, 512)]),
+        torch.stack([la.view(B, H, 1), lb.view(B, H, 1)]))
+    assert torch.allclose(merged.view_as(full).float(), full.float(), rtol=1e-2, atol=1e-2)
+    assert torch.allclose(mlse.view_as(full_lse), full_lse, rtol=1e-3, atol=1e-3)
+
+
+def test_full_size_config5_sampled_parity(device):
+    cfg = workloads.CONFIGS["mla_dsv3"]
+    inp = workloads.make_inputs(cfg, 2, device=device)
+    lay = inp.layout
+    kg, _, _, _ = fill_caches_gpu(inp, device)
+    out, lse = _decode_gpu(inp, kg, device)
+    sample = [int(lay.seq_lens.argmin()), int(lay.seq_lens.argmax())]
+    kc = kg.cpu()
+    ref = oracle.aten_paged_decode(inp.q.cpu()[sample].contiguous(), kc, None,
+                                   lay.block_table[sample].contiguous(), lay.seq_lens[sample].contiguous(),
+                                   cfg.scale, dv=512)
+    assert_close_to_reference(out[sample], ref, "cfg5 sample")
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()

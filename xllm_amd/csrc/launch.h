@@ -34,6 +34,7 @@ struct SplitPlan {
   int max_splits;    // ceil(max_seq_len / chunk_tokens)
 };
 SplitPlan plan_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len);
+SplitPlan plan_mla_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len);
 size_t split_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t v_head_dim, int max_splits);
 
 int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out, float* lse,

@@ -20,6 +20,8 @@
 // Arithmetic follows the block-table oracle of the reference,
 // xllm/core/kernels/npu/attention.cpp:26-78 (head h reads KV head h / group, explicit
 // scale, non-causal softmax over the first L tokens of the listed pages).
+#include <cstdlib>
+
 #include "common.cuh"
 #include "launch.h"
 
@@ -424,9 +426,14 @@ int group_block(int group) {
 }  // namespace
 
 SplitPlan plan_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len) {
-  // Enough workgroups to fill 256 CUs several times over, splits never shorter than 256
-  // tokens nor longer than 8192 (the slot list of a split lives in LDS).
-  constexpr int64_t kTargetWorkgroups = 8192;
+  // Enough workgroups to fill the 256 CUs a few times over (each workgroup pays a fixed
+  // prologue and merge, so fewer and longer splits win once the chip is full); splits are
+  // never shorter than 256 tokens nor longer than 8192 (their slot list lives in LDS).
+  static const int64_t kTargetWorkgroups = [] {
+    const char* e = getenv("XLLM_MI355_TARGET_WGS");  // tuning knob
+    const long v = e ? atol(e) : 0;
+    return static_cast<int64_t>(v > 0 ? v : 1024);
+  }();
   constexpr int64_t kMinChunk = 256, kMaxChunk = 8192;
   if (max_seq_len < 1) max_seq_len = 1;
   const int64_t units = batch * n_head_blocks > 0 ? batch * n_head_blocks : 1;
@@ -437,6 +444,29 @@ SplitPlan plan_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len)
   int64_t chunk = (max_seq_len + splits - 1) / splits;
   chunk = (chunk + kMinChunk - 1) / kMinChunk * kMinChunk;
   if (chunk > kMaxChunk) chunk = kMaxChunk;
+  SplitPlan p;
+  p.chunk_tokens = static_cast<int>(chunk);
+  p.max_splits = static_cast<int>((max_seq_len + chunk - 1) / chunk);
+  return p;
+}
+
+SplitPlan plan_mla_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len) {
+  // One MLA workgroup owns a CU (its two LDS tiles fill it) and every split costs a
+  // [heads, 512] fp32 partial, so: about two workgroups per CU, splits of at least 512 tokens.
+  static const int64_t kTarget = [] {
+    const char* e = getenv("XLLM_MI355_MLA_TARGET_WGS");  // tuning knob
+    const long v = e ? atol(e) : 0;
+    return static_cast<int64_t>(v > 0 ? v : 512);
+  }();
+  constexpr int64_t kMinChunk = 512, kTileTokens = 64;
+  if (max_seq_len < 1) max_seq_len = 1;
+  const int64_t units = batch * n_head_blocks > 0 ? batch * n_head_blocks : 1;
+  int64_t splits = (kTarget + units - 1) / units;
+  const int64_t max_by_len = (max_seq_len + kMinChunk - 1) / kMinChunk;
+  if (splits > max_by_len) splits = max_by_len;
+  if (splits < 1) splits = 1;
+  int64_t chunk = (max_seq_len + splits - 1) / splits;
+  chunk = (chunk + kTileTokens - 1) / kTileTokens * kTileTokens;
   SplitPlan p;
   p.chunk_tokens = static_cast<int>(chunk);
   p.max_splits = static_cast<int>((max_seq_len + chunk - 1) / chunk);
