@@ -41,16 +41,9 @@ int xllm_mi355_kv_head_scales(const void* x, float* scales, int64_t n_tokens, in
 size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t v_head_dim,
                                                int64_t max_seq_len) {
   if (batch <= 0 || n_q_heads <= 0 || v_head_dim <= 0) return 0;
-  if (max_seq_len <= 0) return 0;
-  SplitPlan plan;
-  if (v_head_dim == 512) {
-    // the latent-KV kernel: 64 heads per workgroup
-    plan = plan_mla_splits(batch, (n_q_heads + 63) / 64, max_seq_len);
-  } else {
-    // The fewest head blocks any GQA layout of n_q_heads can have gives the most splits.
-    plan = plan_splits(batch, (n_q_heads + 127) / 128, max_seq_len);
-  }
-  return split_workspace_bytes(batch, n_q_heads, v_head_dim, plan.max_splits);
+  // 512 is the latent width of the MLA kernel; every other width is a GQA head dim
+  if (v_head_dim == 512) return mla_workspace_bytes(batch, n_q_heads, max_seq_len);
+  return gqa_workspace_bytes(batch, n_q_heads, v_head_dim);
 }
 
 int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out,

@@ -28,14 +28,10 @@ struct PageAddressing {
   const int32_t* last_page_len = nullptr;
 };
 
-// Split plan shared by the decode kernels and the workspace query.
-struct SplitPlan {
-  int chunk_tokens;  // tokens of one split (multiple of 256)
-  int max_splits;    // ceil(max_seq_len / chunk_tokens)
-};
-SplitPlan plan_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len);
-SplitPlan plan_mla_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len);
-size_t split_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t v_head_dim, int max_splits);
+// Workspace bytes of the GQA decode (item prefix + two partial slots per persistent workgroup).
+size_t gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim);
+// Workspace bytes of the MLA decode for an upper bound of the context length.
+size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len);
 
 int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out, float* lse,
                      const PageAddressing& addr, const float* k_scale, const float* v_scale,
@@ -49,12 +45,6 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
                      int64_t d_rope, int64_t block_size, int64_t num_blocks, int64_t max_seq_len,
                      float sm_scale, void* workspace, size_t workspace_bytes, int dtype,
                      hipStream_t stream);
-
-// Merge of split partials written by the decode kernels (log2-domain LSE, fp32 partials).
-int merge_splits(const float* ws_out, const float* ws_lse, void* out, float* lse,
-                 const PageAddressing& addr, int64_t batch, int64_t n_heads, int64_t v_head_dim,
-                 int64_t block_size, int64_t out_token_stride, int chunk_tokens, int max_splits,
-                 int out_dtype, hipStream_t stream);
 
 int lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,
               int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim, int dtype,

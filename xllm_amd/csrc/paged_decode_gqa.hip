@@ -1,26 +1,38 @@
 // Paged decode attention, GQA, for gfx950.
 //
-// Work decomposition: one 256-thread workgroup per (sequence, KV-head block, split),
-// a split being `chunk_tokens` consecutive context tokens.  Inside the workgroup each
-// of the 4 wavefronts walks its own interleaved share of the split's pages:
+// Scheduling.  The context of every (sequence, KV-head block) is cut into items of 64
+// tokens; the items of the whole batch form one flat list ordered (sequence, head block,
+// item).  A fixed grid of persistent 256-thread workgroups (as many as fit on the chip at
+// once) splits that list into equal contiguous ranges, so every workgroup streams the same
+// number of KV bytes whatever the mix of context lengths, and a workgroup keeps its online
+// softmax state in registers for as long as it stays inside one (sequence, head block).
+// A run of items that covers a whole context writes the output directly; a run that
+// covers part of one (only the first and the last run of a workgroup can) writes a
+// normalised fp32 partial + log2-domain LSE, and a small merge kernel folds those.
+// The item counts are prefix-summed inside every workgroup (no extra launch, no host read).
+//
+// Inner loop, per wavefront (the 4 wavefronts of a workgroup take steps round-robin):
 //   * a token's [D] row of one KV head is read by LPT adjacent lanes with one 16-byte
 //     load each (64/LPT tokens per load instruction), K and V alike, so every load
-//     instruction covers whole contiguous rows of the [P, bs, Hkv, D] pages;
-//   * q.k is v_dot2 on packed 16-bit pairs into fp32, reduced over the LPT lanes by
-//     DPP row operations; all G query heads of the KV head reuse the same K registers;
-//   * each row of LPT lanes keeps its own running (max, sum, acc) -- no cross-row
-//     traffic inside the loop; rows and wavefronts are merged once through LDS;
-//   * fp8 pages are converted to the 16-bit pair type in registers (exact), the
-//     per-head scales are folded into the score scale (K) and the output (V).
-// The page walk reads slot ids (page * bs + row) staged in LDS once per split, so the
+//     instruction covers whole contiguous rows of the [P, bs, Hkv, D] pages; two register
+//     tiles alternate so the next step's loads fly while the current step is reduced;
+//   * q.k is v_dot2 on packed 16-bit pairs into fp32, reduced over the LPT lanes by DPP
+//     row operations; all G query heads of the KV head reuse the same K registers;
+//   * p.v is v_dot2 as well: V words of two consecutive token rows are byte-permuted into
+//     (token, token+1) pairs and dotted with the packed pair of probabilities;
+//   * each row of LPT lanes keeps its own running (max, sum, acc); the accumulator is
+//     rescaled only on steps where some maximum moved; rows and wavefronts are merged
+//     through LDS once per run;
+//   * fp8 pages are converted to 16-bit pairs in registers (exact), the per-head scales are
+//     folded into the score scale (K) and the output (V).
+// The page walk reads slot ids (page * bs + row) staged in LDS per 2048 tokens, so the
 // loop has no division and never touches table columns past ceil(L / bs).
-// Splits write normalised fp32 partials + log2-domain LSE to the workspace and a small
-// merge kernel combines them; a sequence with one split writes its output directly.
 //
 // Arithmetic follows the block-table oracle of the reference,
 // xllm/core/kernels/npu/attention.cpp:26-78 (head h reads KV head h / group, explicit
 // scale, non-causal softmax over the first L tokens of the listed pages).
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.cuh"
 #include "launch.h"
@@ -31,6 +43,9 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
+constexpr int kItem = 64;      // tokens per schedulable item
+constexpr int kSub = 2048;     // tokens whose slot ids are staged in LDS at a time
+constexpr int kMaxBatch = 8192;  // sequences per launch (their item prefix lives in LDS)
 
 struct GqaArgs {
   const char* q;
@@ -45,21 +60,23 @@ struct GqaArgs {
   const int32_t* last_page_len;
   const float* k_scale;
   const float* v_scale;
-  float* ws_out;
-  float* ws_lse;
+  int* ws_prefix;  // [batch + 1] item prefix, written by workgroup 0 for the merge kernel
+  float* ws_out;   // [2 * n_workgroups][G][D]
+  float* ws_lse;   // [2 * n_workgroups][G]
   int64_t table_stride;
   int64_t q_stride_bytes;
   int64_t out_stride_bytes;
   int64_t row_bytes;  // Hkv * D * sizeof(cache element)
+  int batch;
   int n_q_heads;
   int n_kv_heads;
   int group;
+  int g_block;        // query heads per head block (the kernel's G)
   int block_size;
-  int bs_shift;  // log2(block_size) or -1
+  int bs_shift;       // log2(block_size) or -1
   int num_blocks;
-  int chunk_tokens;
-  int max_splits;
-  float scale_log2;  // sm_scale * log2(e)
+  int n_workgroups;   // grid size of the decode kernel
+  float scale_log2;   // sm_scale * log2(e)
 };
 
 __device__ __forceinline__ void sequence_of(const GqaArgs& a, int b, const int32_t*& pages, int& L) {
@@ -74,9 +91,49 @@ __device__ __forceinline__ void sequence_of(const GqaArgs& a, int b, const int32
   }
 }
 
+__device__ __forceinline__ int items_of(int L) { return L > 0 ? (L + kItem - 1) / kItem : 0; }
+
+// First flat item of workgroup w when `total` items are dealt to `n` workgroups.
+__device__ __forceinline__ int64_t range_start(int64_t w, int64_t total, int64_t n) { return w * total / n; }
+
+// The workgroup whose range holds flat item `id`.
+__device__ __forceinline__ int workgroup_of(int64_t id, int64_t total, int64_t n) {
+  int64_t w = id * n / total;
+  while (w + 1 < n && range_start(w + 1, total, n) <= id) ++w;
+  return static_cast<int>(w);
+}
+
+// Exclusive prefix sum of the per-sequence item counts into prefix[0..batch] (LDS).
+// Every thread sums a contiguous slice, then adds the totals of the slices before it.
+__device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* tmp) {
+  const int tid = threadIdx.x;
+  const int per = (a.batch + kThreads - 1) / kThreads;
+  const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
+  int local = 0;
+  for (int b = lo; b < hi; ++b) {
+    const int32_t* pages;
+    int L;
+    sequence_of(a, b, pages, L);
+    local += items_of(L);
+  }
+  tmp[tid] = local;
+  __syncthreads();
+  int excl = 0;
+  for (int j = 0; j < tid; ++j) excl += tmp[j];
+  for (int b = lo; b < hi; ++b) {
+    const int32_t* pages;
+    int L;
+    sequence_of(a, b, pages, L);
+    prefix[b] = excl;
+    excl += items_of(L);
+  }
+  if (lo < hi && hi == a.batch) prefix[a.batch] = excl;  // the last non-empty slice holds the total
+  __syncthreads();
+}
+
 // QT: BF16 or FP16 (query, output and non-fp8 cache element).  FP8: cache holds e4m3fn.
 // D: head dim.  LPT: lanes per token row.  G: query heads per workgroup.  U: token rows
-// per lane and step.
+// per lane and step (even).
 template <typename QT, bool FP8, int D, int LPT, int G, int U>
 __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
   constexpr int TPP = kWave / LPT;       // token rows per load instruction
@@ -86,331 +143,425 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
   constexpr int STEP = U * TPP;          // tokens per wavefront step
   constexpr int NP = kWaves * TPP;       // partial softmax states per workgroup
   constexpr int PSTRIDE = D + 2;         // acc[D], max, sum
+  constexpr int CES = FP8 ? 1 : 2;
   static_assert(NLD >= 1 && NLD * EPL * LPT == D, "lane mapping must tile the head dim");
+  static_assert(U % 2 == 0 && kItem % STEP == 0 && kSub % kItem == 0, "step must tile an item");
 
   extern __shared__ __align__(16) char smem[];
-  int* slots = reinterpret_cast<int*>(smem);
-  float* part = reinterpret_cast<float*>(smem + static_cast<size_t>(a.chunk_tokens) * 4);
+  int* slots = reinterpret_cast<int*>(smem);                       // [kSub]
+  float* part = reinterpret_cast<float*>(smem + kSub * 4);         // [NP][PSTRIDE]
+  int* tmp = reinterpret_cast<int*>(smem + kSub * 4 + NP * PSTRIDE * 4);  // [kThreads]
+  int* prefix = tmp + kThreads;                                    // [batch + 1]
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
   const int c = lane % LPT;  // 16-byte column of the row
   const int r = lane / LPT;  // token row within a load
-  const int split = blockIdx.x;
-  const int b = blockIdx.z;
   const int hb_per_kv = (a.group + G - 1) / G;
-  const int kvh = blockIdx.y / hb_per_kv;
-  const int h0 = kvh * a.group + (blockIdx.y % hb_per_kv) * G;
-  const int nh = min(G, (kvh + 1) * a.group - h0);
+  const int n_hb = a.n_kv_heads * hb_per_kv;
 
-  const int32_t* pages;
-  int L;
-  sequence_of(a, b, pages, L);
-  if (L <= 0) {
-    if (split == 0) {
-      for (int i = tid; i < nh * D; i += kThreads) {
-        const int h = i / D, d = i % D;
-        reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes)[(h0 + h) * D + d] = 0;
-      }
-      if (a.lse != nullptr && tid < nh) a.lse[b * a.n_q_heads + h0 + tid] = -INFINITY;
-    }
-    return;
+  item_prefix(a, prefix, tmp);
+  const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
+  if (blockIdx.x == 0) {
+    for (int i = tid; i <= a.batch; i += kThreads) a.ws_prefix[i] = prefix[i];
   }
-  const int n_splits = (L + a.chunk_tokens - 1) / a.chunk_tokens;
-  if (split >= n_splits) return;
-  const int t0 = split * a.chunk_tokens;
-  const int t1 = min(L, t0 + a.chunk_tokens);
-  const int n_steps = (t1 - t0 + STEP - 1) / STEP;
-
-  // slot id of every token of the split (tail entries repeat the last valid token)
-  for (int i = tid; i < n_steps * STEP; i += kThreads) {
-    const int tok = min(t0 + i, L - 1);
-    int pg, off;
-    if (a.bs_shift >= 0) {
-      pg = tok >> a.bs_shift;
-      off = tok & (a.block_size - 1);
-    } else {
-      pg = tok / a.block_size;
-      off = tok - pg * a.block_size;
-    }
-    int page = pages[pg];
-    page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
-    slots[i] = page * a.block_size + off;
-  }
-
-  // query registers: for each head the 16-bit pairs matching this lane's cache columns
-  u32 qreg[G][NLD][EPL / 2];
-#pragma unroll
-  for (int h = 0; h < G; ++h) {
-#pragma unroll
-    for (int j = 0; j < NLD; ++j) {
-      if (h < nh) {
-        const char* qp = a.q + b * a.q_stride_bytes +
-                         (static_cast<int64_t>(h0 + h) * D + (j * LPT + c) * EPL) * 2;
-#pragma unroll
-        for (int e = 0; e < EPL / 8; ++e) {
-          const u32x4 x = ldg16(qp + e * 16);
-          qreg[h][j][e * 4 + 0] = x[0];
-          qreg[h][j][e * 4 + 1] = x[1];
-          qreg[h][j][e * 4 + 2] = x[2];
-          qreg[h][j][e * 4 + 3] = x[3];
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < EPL / 2; ++e) qreg[h][j][e] = 0u;
-      }
-    }
-  }
-
-  float score_scale = a.scale_log2;
-  if constexpr (FP8) score_scale *= a.k_scale[kvh];
-
-  float m[G], l[G], acc[G][NLD * EPL];
-#pragma unroll
-  for (int h = 0; h < G; ++h) {
-    m[h] = kNegBig;
-    l[h] = 0.0f;
-#pragma unroll
-    for (int e = 0; e < NLD * EPL; ++e) acc[h][e] = 0.0f;
-  }
-
-  constexpr int CES = FP8 ? 1 : 2;
-  const int64_t lane_off = static_cast<int64_t>(kvh) * D * CES + c * 16;
-  const char* kbase = a.k_cache + lane_off;
-  const char* vbase = a.v_cache + lane_off;
+  if (total == 0) return;
+  const int64_t n_wg = gridDim.x;
+  int64_t cur = range_start(blockIdx.x, total, n_wg);
+  const int64_t end = range_start(blockIdx.x + 1, total, n_wg);
+  bool first_run = true;
 
   struct Tile {
     u32x4 k[U][NLD];
     u32x4 v[U][NLD];
   };
 
-  __syncthreads();  // slots ready
-
-  auto load_tile = [&](Tile& t, int step) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int slot = slots[step * STEP + u * TPP + r];
-      const int64_t off = static_cast<int64_t>(slot) * a.row_bytes;
-#pragma unroll
-      for (int j = 0; j < NLD; ++j) {
-        t.k[u][j] = ldg16(kbase + off + j * (LPT * 16));
-        t.v[u][j] = ldg16(vbase + off + j * (LPT * 16));
-      }
+  while (cur < end) {
+    // ---- locate the run: sequence b (binary search in the prefix), head block, first item
+    int lo = 0, hi = a.batch;  // prefix[lo] * n_hb <= cur < prefix[hi] * n_hb
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (static_cast<int64_t>(prefix[mid]) * n_hb <= cur) lo = mid; else hi = mid;
     }
-  };
+    const int b = lo;
+    const int n_items = prefix[b + 1] - prefix[b];
+    const int64_t rem = cur - static_cast<int64_t>(prefix[b]) * n_hb;
+    const int hbk = static_cast<int>(rem / n_items);
+    const int item0 = static_cast<int>(rem - static_cast<int64_t>(hbk) * n_items);
+    const int run_items = static_cast<int>(min<int64_t>(n_items - item0, end - cur));
+    const bool complete = item0 == 0 && run_items == n_items;
+    cur += run_items;
 
-  auto compute_tile = [&](const Tile& t, int step) {
-    float s[U][G];
+    const int32_t* pages;
+    int L;
+    sequence_of(a, b, pages, L);
+    const int kvh = hbk / hb_per_kv;
+    const int h0 = kvh * a.group + (hbk % hb_per_kv) * G;
+    const int nh = min(G, (kvh + 1) * a.group - h0);
+    const int run_t0 = item0 * kItem;
+    const int run_t1 = min(L, (item0 + run_items) * kItem);
+
+    // query registers: for each head the 16-bit pairs matching this lane's cache columns
+    u32 qreg[G][NLD][EPL / 2];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      u32 kp[NLD][EPL / 2];
+    for (int h = 0; h < G; ++h) {
 #pragma unroll
       for (int j = 0; j < NLD; ++j) {
+        if (h < nh) {
+          const char* qp = a.q + b * a.q_stride_bytes +
+                           (static_cast<int64_t>(h0 + h) * D + (j * LPT + c) * EPL) * 2;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          if constexpr (FP8) {
-            kp[j][2 * w] = QT::template from_fp8x2<false>(t.k[u][j][w]);
-            kp[j][2 * w + 1] = QT::template from_fp8x2<true>(t.k[u][j][w]);
-          } else {
-            kp[j][w] = t.k[u][j][w];
+          for (int e = 0; e < EPL / 8; ++e) {
+            const u32x4 x = ldg16(qp + e * 16);
+            qreg[h][j][e * 4 + 0] = x[0];
+            qreg[h][j][e * 4 + 1] = x[1];
+            qreg[h][j][e * 4 + 2] = x[2];
+            qreg[h][j][e * 4 + 3] = x[3];
           }
+        } else {
+#pragma unroll
+          for (int e = 0; e < EPL / 2; ++e) qreg[h][j][e] = 0u;
         }
       }
-      const bool valid = t0 + step * STEP + u * TPP + r < t1;
+    }
+    float score_scale = a.scale_log2;
+    if constexpr (FP8) score_scale *= a.k_scale[kvh];
+
+    float m[G], l[G], acc[G][NLD * EPL];
 #pragma unroll
-      for (int h = 0; h < G; ++h) {
-        float d = 0.0f;
+    for (int h = 0; h < G; ++h) {
+      m[h] = kNegBig;
+      l[h] = 0.0f;
+#pragma unroll
+      for (int e = 0; e < NLD * EPL; ++e) acc[h][e] = 0.0f;
+    }
+    const int64_t lane_off = static_cast<int64_t>(kvh) * D * CES + c * 16;
+    const char* kbase = a.k_cache + lane_off;
+    const char* vbase = a.v_cache + lane_off;
+
+    for (int t0 = run_t0; t0 < run_t1; t0 += kSub) {
+      const int t1 = min(run_t1, t0 + kSub);
+      const int n_steps = (t1 - t0 + STEP - 1) / STEP;
+      const bool ragged = (t1 - t0) % STEP != 0;  // only the last step of a context can be
+
+      __syncthreads();  // the previous slot list (and the merge buffer) are no longer read
+      for (int i = tid; i < n_steps * STEP; i += kThreads) {
+        const int tok = min(t0 + i, L - 1);  // tail entries repeat the last valid token
+        int pg, off;
+        if (a.bs_shift >= 0) {
+          pg = tok >> a.bs_shift;
+          off = tok & (a.block_size - 1);
+        } else {
+          pg = tok / a.block_size;
+          off = tok - pg * a.block_size;
+        }
+        int page = pages[pg];
+        page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
+        slots[i] = page * a.block_size + off;
+      }
+      __syncthreads();
+
+      auto load_tile = [&](Tile& t, int step) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int slot = slots[step * STEP + u * TPP + r];
+          const int64_t off = static_cast<int64_t>(slot) * a.row_bytes;
+#pragma unroll
+          for (int j = 0; j < NLD; ++j) {
+            t.k[u][j] = ldg16(kbase + off + j * (LPT * 16));
+            t.v[u][j] = ldg16(vbase + off + j * (LPT * 16));
+          }
+        }
+      };
+
+      auto compute_tile = [&](const Tile& t, int step, auto masked) {
+        constexpr bool MASKED = decltype(masked)::value;
+        // ---- scores: raw q.k per (token row u, head h), summed over the LPT lanes
+        float s[U][G];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          u32 kp[NLD][EPL / 2];
+#pragma unroll
+          for (int j = 0; j < NLD; ++j) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              if constexpr (FP8) {
+                kp[j][2 * w] = QT::template from_fp8x2<false>(t.k[u][j][w]);
+                kp[j][2 * w + 1] = QT::template from_fp8x2<true>(t.k[u][j][w]);
+              } else {
+                kp[j][w] = t.k[u][j][w];
+              }
+            }
+          }
+#pragma unroll
+          for (int h = 0; h < G; ++h) {
+            float d = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NLD; ++j)
+#pragma unroll
+              for (int e = 0; e < EPL / 2; ++e) d = QT::dot2(kp[j][e], qreg[h][j][e], d);
+            s[u][h] = group_sum<LPT>(d);
+          }
+          if constexpr (MASKED) {
+            if (t0 + step * STEP + u * TPP + r >= t1) {
+#pragma unroll
+              for (int h = 0; h < G; ++h) s[u][h] = -INFINITY;
+            }
+          }
+        }
+        // ---- online softmax of this lane row's U tokens, in the log2 domain:
+        // p = exp2(s * c - m) with m the running maximum of s * c (c > 0)
+        bool moved = false;
+        float alpha[G];
+        u32 pp[U / 2][G];
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+          float mx = s[0][h];
+#pragma unroll
+          for (int u = 1; u < U; ++u) mx = fmaxf(mx, s[u][h]);
+          const float m_new = fmaxf(m[h], mx * score_scale);
+          alpha[h] = fast_exp2(m[h] - m_new);
+          moved |= m_new != m[h];
+          m[h] = m_new;
+          float sum = 0.0f;
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            s[u][h] = fast_exp2(__builtin_fmaf(s[u][h], score_scale, -m_new));
+            sum += s[u][h];
+          }
+          l[h] = __builtin_fmaf(l[h], alpha[h], sum);
+#pragma unroll
+          for (int up = 0; up < U / 2; ++up) pp[up][h] = QT::pack(s[2 * up][h], s[2 * up + 1][h]);
+        }
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {  // rare once the maxima have settled
+#pragma unroll
+          for (int h = 0; h < G; ++h)
+#pragma unroll
+            for (int e = 0; e < NLD * EPL; ++e) acc[h][e] *= alpha[h];
+        }
+        // ---- acc += p . v on (token, token + 1) pairs
+#pragma unroll
+        for (int up = 0; up < U / 2; ++up) {
+#pragma unroll
+          for (int j = 0; j < NLD; ++j) {
+            u32 v0[EPL / 2], v1[EPL / 2];  // pairs of consecutive dims of rows 2up and 2up+1
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+              if constexpr (FP8) {
+                v0[2 * w] = QT::template from_fp8x2<false>(t.v[2 * up][j][w]);
+                v0[2 * w + 1] = QT::template from_fp8x2<true>(t.v[2 * up][j][w]);
+                v1[2 * w] = QT::template from_fp8x2<false>(t.v[2 * up + 1][j][w]);
+                v1[2 * w + 1] = QT::template from_fp8x2<true>(t.v[2 * up + 1][j][w]);
+              } else {
+                v0[w] = t.v[2 * up][j][w];
+                v1[w] = t.v[2 * up + 1][j][w];
+              }
+            }
+#pragma unroll
+            for (int w = 0; w < EPL / 2; ++w) {
+              const u32 even = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);  // dim 2w of both rows
+              const u32 odd = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u);   // dim 2w+1
+#pragma unroll
+              for (int h = 0; h < G; ++h) {
+                acc[h][j * EPL + 2 * w] = QT::dot2(even, pp[up][h], acc[h][j * EPL + 2 * w]);
+                acc[h][j * EPL + 2 * w + 1] = QT::dot2(odd, pp[up][h], acc[h][j * EPL + 2 * w + 1]);
+              }
+            }
+          }
+        }
+      };
+
+      auto compute = [&](const Tile& t, int step) {
+        if (ragged && step == n_steps - 1) compute_tile(t, step, std::true_type{});
+        else compute_tile(t, step, std::false_type{});
+      };
+
+      // steps are dealt round-robin to the wavefronts; two register tiles alternate so that
+      // the loads of the next step are in flight while the current one is reduced
+      Tile ta, tb;
+      int step = wave;
+      if (step < n_steps) load_tile(ta, step);
+      while (step < n_steps) {
+        const int next = step + kWaves;
+        if (next < n_steps) load_tile(tb, next);
+        compute(ta, step);
+        if (next >= n_steps) break;
+        const int next2 = next + kWaves;
+        if (next2 < n_steps) load_tile(ta, next2);
+        compute(tb, next);
+        step = next2;
+      }
+    }
+
+    // ---- end of the run: one head at a time every lane row publishes its state and the
+    // workgroup folds the NP states into the output or into a partial
+    float out_scale = 1.0f;
+    if constexpr (FP8) out_scale = a.v_scale[kvh];
+    const int pi = wave * TPP + r;
+    const int64_t pslot = static_cast<int64_t>(blockIdx.x) * 2 + (first_run ? 0 : 1);
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      __syncthreads();  // the slot list / the previous head's states have been consumed
+      {
+        float* p = part + pi * PSTRIDE;
 #pragma unroll
         for (int j = 0; j < NLD; ++j)
 #pragma unroll
-          for (int e = 0; e < EPL / 2; ++e) d = QT::dot2(kp[j][e], qreg[h][j][e], d);
-        d = group_sum<LPT>(d);
-        s[u][h] = valid ? d * score_scale : -INFINITY;
+          for (int e = 0; e < EPL; ++e) p[(j * LPT + c) * EPL + e] = acc[h][j * EPL + e];
+        if (c == 0) {
+          p[D] = m[h];
+          p[D + 1] = l[h];
+        }
       }
-    }
-    // online softmax of this lane row's U tokens
+      __syncthreads();
+      if (h < nh) {
+        for (int d = tid; d < D; d += kThreads) {
+          float mx = kNegBig;
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      float mx = s[0][h];
+          for (int p = 0; p < NP; ++p) mx = fmaxf(mx, part[p * PSTRIDE + D]);
+          float lsum = 0.0f, o = 0.0f;
 #pragma unroll
-      for (int u = 1; u < U; ++u) mx = fmaxf(mx, s[u][h]);
-      const float m_new = fmaxf(m[h], mx);
-      const float alpha = fast_exp2(m[h] - m_new);
-      m[h] = m_new;
-      float sum = 0.0f;
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        s[u][h] = fast_exp2(s[u][h] - m_new);
-        sum += s[u][h];
-      }
-      l[h] = l[h] * alpha + sum;
-#pragma unroll
-      for (int e = 0; e < NLD * EPL; ++e) acc[h][e] *= alpha;
-    }
-    // acc += p . v
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int j = 0; j < NLD; ++j) {
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const u32 x = t.v[u][j][w];
-          if constexpr (FP8) {
-            const f32x2 f01 = fp8x2_to_f32<false>(x);
-            const f32x2 f23 = fp8x2_to_f32<true>(x);
-#pragma unroll
-            for (int h = 0; h < G; ++h) {
-              acc[h][j * EPL + 4 * w + 0] += s[u][h] * f01[0];
-              acc[h][j * EPL + 4 * w + 1] += s[u][h] * f01[1];
-              acc[h][j * EPL + 4 * w + 2] += s[u][h] * f23[0];
-              acc[h][j * EPL + 4 * w + 3] += s[u][h] * f23[1];
-            }
+          for (int p = 0; p < NP; ++p) {
+            const float* pp = part + p * PSTRIDE;
+            const float w = fast_exp2(pp[D] - mx);
+            lsum += w * pp[D + 1];
+            o += w * pp[d];
+          }
+          const float val = o / lsum * out_scale;
+          const int hq = h0 + h;
+          if (complete) {
+            reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes)[hq * D + d] = QT::from_f32(val);
+            if (a.lse != nullptr && d == 0) a.lse[b * a.n_q_heads + hq] = (mx + fast_log2(lsum)) * kLn2;
           } else {
-            const float v0 = QT::lo(x);
-            const float v1 = QT::hi(x);
-#pragma unroll
-            for (int h = 0; h < G; ++h) {
-              acc[h][j * EPL + 2 * w + 0] += s[u][h] * v0;
-              acc[h][j * EPL + 2 * w + 1] += s[u][h] * v1;
-            }
+            a.ws_out[(pslot * G + h) * D + d] = val;
+            if (d == 0) a.ws_lse[pslot * G + h] = mx + fast_log2(lsum);
           }
         }
       }
     }
-  };
-
-  // steps are dealt round-robin to the wavefronts; two register tiles alternate so that
-  // the loads of the next step are in flight while the current one is reduced
-  Tile ta, tb;
-  int step = wave;
-  if (step < n_steps) load_tile(ta, step);
-  while (step < n_steps) {
-    const int next = step + kWaves;
-    if (next < n_steps) load_tile(tb, next);
-    compute_tile(ta, step);
-    if (next >= n_steps) break;
-    const int next2 = next + kWaves;
-    if (next2 < n_steps) load_tile(ta, next2);
-    compute_tile(tb, next);
-    step = next2;
-  }
-
-  // one head at a time: every lane row publishes its state, the workgroup folds the NP states
-  float out_scale = 1.0f;
-  if constexpr (FP8) out_scale = a.v_scale[kvh];
-  const int pi = wave * TPP + r;
-#pragma unroll
-  for (int h = 0; h < G; ++h) {
-    if (h > 0) __syncthreads();  // the previous head's states have been consumed
-    {
-      float* p = part + pi * PSTRIDE;
-#pragma unroll
-      for (int j = 0; j < NLD; ++j)
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) p[(j * LPT + c) * EPL + e] = acc[h][j * EPL + e];
-      if (c == 0) {
-        p[D] = m[h];
-        p[D + 1] = l[h];
-      }
-    }
-    __syncthreads();
-    if (h < nh) {
-      for (int d = tid; d < D; d += kThreads) {
-        float mx = kNegBig;
-#pragma unroll
-        for (int p = 0; p < NP; ++p) mx = fmaxf(mx, part[p * PSTRIDE + D]);
-        float lsum = 0.0f, o = 0.0f;
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-          const float* pp = part + p * PSTRIDE;
-          const float w = fast_exp2(pp[D] - mx);
-          lsum += w * pp[D + 1];
-          o += w * pp[d];
-        }
-        const float val = o / lsum * out_scale;
-        const int hq = h0 + h;
-        if (n_splits == 1) {
-          reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes)[hq * D + d] = QT::from_f32(val);
-          if (a.lse != nullptr && d == 0) a.lse[b * a.n_q_heads + hq] = (mx + fast_log2(lsum)) * kLn2;
-        } else {
-          const int64_t wi = (static_cast<int64_t>(b) * a.n_q_heads + hq) * a.max_splits + split;
-          a.ws_out[wi * D + d] = val;
-          if (d == 0) a.ws_lse[wi] = mx + fast_log2(lsum);
-        }
-      }
-    }
+    first_run = false;
   }
 }
 
-// Merge of split partials: one workgroup per (sequence, query head).
+// Merge of the partials of contexts that span several workgroups; also writes the output
+// of empty sequences.  One workgroup per (query head, sequence).
 template <typename QT>
-__global__ __launch_bounds__(128) void merge_splits_kernel(const float* ws_out, const float* ws_lse,
-                                                           char* out, float* lse, GqaArgs a, int dv) {
+__global__ __launch_bounds__(128) void merge_partials_kernel(GqaArgs a, int dv) {
   const int hq = blockIdx.x;
   const int b = blockIdx.y;
+  const int G = a.g_block;
   const int32_t* pages;
   int L;
   sequence_of(a, b, pages, L);
-  const int n_splits = (L + a.chunk_tokens - 1) / a.chunk_tokens;
-  if (n_splits <= 1) return;  // written directly by the decode kernel
-  const int64_t w0 = (static_cast<int64_t>(b) * a.n_q_heads + hq) * a.max_splits;
+  uint16_t* out = reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes) + hq * dv;
+  if (L <= 0) {
+    for (int d = threadIdx.x; d < dv; d += 128) out[d] = 0;
+    if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * a.n_q_heads + hq] = -INFINITY;
+    return;
+  }
+  const int hb_per_kv = (a.group + G - 1) / G;
+  const int n_hb = a.n_kv_heads * hb_per_kv;
+  const int kvh = hq / a.group;
+  const int hbk = kvh * hb_per_kv + (hq - kvh * a.group) / G;
+  const int h = (hq - kvh * a.group) % G;
+  const int64_t total = static_cast<int64_t>(a.ws_prefix[a.batch]) * n_hb;
+  const int n_items = a.ws_prefix[b + 1] - a.ws_prefix[b];
+  const int64_t first = static_cast<int64_t>(a.ws_prefix[b]) * n_hb + static_cast<int64_t>(hbk) * n_items;
+  const int64_t last = first + n_items - 1;
+  const int64_t n_wg = a.n_workgroups;
+  const int w_first = workgroup_of(first, total, n_wg);
+  const int w_last = workgroup_of(last, total, n_wg);
+  if (w_first == w_last) return;  // one workgroup saw the whole context and wrote the output
+  // the first workgroup holds this context as its last run (slot 1) unless its range starts
+  // exactly here; every later one holds it as its first run (slot 0)
+  const int slot_first = range_start(w_first, total, n_wg) < first ? 1 : 0;
+  auto pslot = [&](int w) { return static_cast<int64_t>(w) * 2 + (w == w_first ? slot_first : 0); };
+  // with fewer items than workgroups some ranges in between are empty and own no partial
+  auto has_items = [&](int w) { return range_start(w, total, n_wg) < range_start(w + 1, total, n_wg); };
   float mx = kNegBig;
-  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, ws_lse[w0 + s]);
+  for (int w = w_first; w <= w_last; ++w)
+    if (has_items(w)) mx = fmaxf(mx, a.ws_lse[pslot(w) * G + h]);
   float wsum = 0.0f;
-  for (int s = 0; s < n_splits; ++s) wsum += fast_exp2(ws_lse[w0 + s] - mx);
+  for (int w = w_first; w <= w_last; ++w)
+    if (has_items(w)) wsum += fast_exp2(a.ws_lse[pslot(w) * G + h] - mx);
   const float inv = 1.0f / wsum;
   for (int d = threadIdx.x; d < dv; d += 128) {
     float o = 0.0f;
-    for (int s = 0; s < n_splits; ++s)
-      o += fast_exp2(ws_lse[w0 + s] - mx) * ws_out[(w0 + s) * dv + d];
-    reinterpret_cast<uint16_t*>(out + b * a.out_stride_bytes)[hq * dv + d] = QT::from_f32(o * inv);
+    for (int w = w_first; w <= w_last; ++w) {
+      if (!has_items(w)) continue;
+      const int64_t ps = pslot(w) * G + h;
+      o += fast_exp2(a.ws_lse[ps] - mx) * a.ws_out[ps * dv + d];
+    }
+    out[d] = QT::from_f32(o * inv);
   }
-  if (lse != nullptr && threadIdx.x == 0) lse[b * a.n_q_heads + hq] = (mx + fast_log2(wsum)) * kLn2;
+  if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * a.n_q_heads + hq] = (mx + fast_log2(wsum)) * kLn2;
+}
+
+int device_cu_count() {
+  static const int n = [] {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 256;
+    return p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
+  }();
+  return n;
 }
 
 template <typename QT, bool FP8, int D, int LPT, int G, int U>
-int launch_gqa(const GqaArgs& a, int64_t batch, int n_head_blocks, hipStream_t stream) {
+int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
   constexpr int NP = kWaves * (kWave / LPT);
-  const size_t smem = static_cast<size_t>(a.chunk_tokens) * 4 + static_cast<size_t>(NP) * (D + 2) * 4;
   auto kern = gqa_decode_kernel<QT, FP8, D, LPT, G, U>;
-  if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
-    if (e != hipSuccess) return static_cast<int>(e);
-  }
-  dim3 grid(static_cast<unsigned>(a.max_splits), static_cast<unsigned>(n_head_blocks),
-            static_cast<unsigned>(batch));
-  kern<<<grid, kThreads, smem, stream>>>(a);
+  const size_t smem = kSub * 4 + static_cast<size_t>(NP) * (D + 2) * 4 + kThreads * 4 +
+                      (static_cast<size_t>(a.batch) + 1) * 4;
+  static const int per_cu = [&] {
+    const char* e = getenv("XLLM_MI355_GQA_WGS_PER_CU");  // tuning knob
+    if (e != nullptr && atoi(e) > 0) return atoi(e);
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(kern), kThreads,
+                                                     kSub * 4 + NP * (D + 2) * 4 + kThreads * 4 + 1028) != hipSuccess || n < 1)
+      n = 2;
+    return n;
+  }();
+  a.n_workgroups = device_cu_count() * per_cu;
+  const size_t prefix_bytes = ((static_cast<size_t>(a.batch) + 1) * 4 + 255) / 256 * 256;
+  const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * G * (D + 1);
+  *need = prefix_bytes + part_floats * 4;
+  if (plan_only) return XLLM_MI355_OK;
+  if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
+  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_prefix) + prefix_bytes);
+  a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * G * D;
+  const bool timed = profile_begin(stream);
+  kern<<<dim3(static_cast<unsigned>(a.n_workgroups)), kThreads, smem, stream>>>(a);
+  if (timed) profile_end(stream);
   return static_cast<int>(hipGetLastError());
 }
 
 template <typename QT, bool FP8, int D, int LPT, int U>
-int dispatch_group(const GqaArgs& a, int64_t batch, int g_block, hipStream_t stream) {
-  const int hb = a.n_kv_heads * ((a.group + g_block - 1) / g_block);
-  switch (g_block) {
-    case 1: return launch_gqa<QT, FP8, D, LPT, 1, U>(a, batch, hb, stream);
-    case 2: return launch_gqa<QT, FP8, D, LPT, 2, U>(a, batch, hb, stream);
-    case 4: return launch_gqa<QT, FP8, D, LPT, 4, U>(a, batch, hb, stream);
-    default: return launch_gqa<QT, FP8, D, LPT, 8, U>(a, batch, hb, stream);
+int dispatch_group(GqaArgs& a, size_t wsb, hipStream_t s, bool plan_only, size_t* need) {
+  switch (a.g_block) {
+    case 1: return launch_gqa<QT, FP8, D, LPT, 1, U>(a, wsb, s, plan_only, need);
+    case 2: return launch_gqa<QT, FP8, D, LPT, 2, U>(a, wsb, s, plan_only, need);
+    case 4: return launch_gqa<QT, FP8, D, LPT, 4, U>(a, wsb, s, plan_only, need);
+    default: return launch_gqa<QT, FP8, D, LPT, 8, U>(a, wsb, s, plan_only, need);
   }
 }
 
 template <typename QT, bool FP8>
-int dispatch_dim(const GqaArgs& a, int64_t batch, int head_dim, int g_block, hipStream_t stream) {
-  // lanes per token row: 16-byte loads, one per lane (two for bf16 D=256)
+int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_only, size_t* need) {
+  // lanes per token row: one 16-byte load per lane and row
   if constexpr (FP8) {
     switch (head_dim) {
-      case 64: return dispatch_group<QT, true, 64, 4, 1>(a, batch, g_block, stream);
-      case 128: return dispatch_group<QT, true, 128, 8, 2>(a, batch, g_block, stream);
-      case 256: return dispatch_group<QT, true, 256, 16, 4>(a, batch, g_block, stream);
+      case 64: return dispatch_group<QT, true, 64, 4, 2>(a, wsb, s, plan_only, need);
+      case 128: return dispatch_group<QT, true, 128, 8, 2>(a, wsb, s, plan_only, need);
+      case 256: return dispatch_group<QT, true, 256, 16, 4>(a, wsb, s, plan_only, need);
       default: return XLLM_MI355_ESHAPE;
     }
   } else {
     switch (head_dim) {
-      case 64: return dispatch_group<QT, false, 64, 8, 2>(a, batch, g_block, stream);
-      case 128: return dispatch_group<QT, false, 128, 16, 4>(a, batch, g_block, stream);
-      case 256: return dispatch_group<QT, false, 256, 32, 4>(a, batch, g_block, stream);
+      case 64: return dispatch_group<QT, false, 64, 8, 2>(a, wsb, s, plan_only, need);
+      case 128: return dispatch_group<QT, false, 128, 16, 4>(a, wsb, s, plan_only, need);
+      case 256: return dispatch_group<QT, false, 256, 32, 4>(a, wsb, s, plan_only, need);
       default: return XLLM_MI355_ESHAPE;
     }
   }
@@ -425,83 +576,12 @@ int group_block(int group) {
 
 }  // namespace
 
-SplitPlan plan_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len) {
-  // Enough workgroups to fill the 256 CUs a few times over (each workgroup pays a fixed
-  // prologue and merge, so fewer and longer splits win once the chip is full); splits are
-  // never shorter than 256 tokens nor longer than 8192 (their slot list lives in LDS).
-  static const int64_t kTargetWorkgroups = [] {
-    const char* e = getenv("XLLM_MI355_TARGET_WGS");  // tuning knob
-    const long v = e ? atol(e) : 0;
-    return static_cast<int64_t>(v > 0 ? v : 1024);
-  }();
-  constexpr int64_t kMinChunk = 256, kMaxChunk = 8192;
-  if (max_seq_len < 1) max_seq_len = 1;
-  const int64_t units = batch * n_head_blocks > 0 ? batch * n_head_blocks : 1;
-  int64_t splits = (kTargetWorkgroups + units - 1) / units;
-  const int64_t max_by_len = (max_seq_len + kMinChunk - 1) / kMinChunk;
-  if (splits > max_by_len) splits = max_by_len;
-  if (splits < 1) splits = 1;
-  int64_t chunk = (max_seq_len + splits - 1) / splits;
-  chunk = (chunk + kMinChunk - 1) / kMinChunk * kMinChunk;
-  if (chunk > kMaxChunk) chunk = kMaxChunk;
-  SplitPlan p;
-  p.chunk_tokens = static_cast<int>(chunk);
-  p.max_splits = static_cast<int>((max_seq_len + chunk - 1) / chunk);
-  return p;
-}
-
-SplitPlan plan_mla_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len) {
-  // One MLA workgroup owns a CU (its two LDS tiles fill it) and every split costs a
-  // [heads, 512] fp32 partial, so: about two workgroups per CU, splits of at least 512 tokens.
-  static const int64_t kTarget = [] {
-    const char* e = getenv("XLLM_MI355_MLA_TARGET_WGS");  // tuning knob
-    const long v = e ? atol(e) : 0;
-    return static_cast<int64_t>(v > 0 ? v : 512);
-  }();
-  constexpr int64_t kMinChunk = 512, kTileTokens = 64;
-  if (max_seq_len < 1) max_seq_len = 1;
-  const int64_t units = batch * n_head_blocks > 0 ? batch * n_head_blocks : 1;
-  int64_t splits = (kTarget + units - 1) / units;
-  const int64_t max_by_len = (max_seq_len + kMinChunk - 1) / kMinChunk;
-  if (splits > max_by_len) splits = max_by_len;
-  if (splits < 1) splits = 1;
-  int64_t chunk = (max_seq_len + splits - 1) / splits;
-  chunk = (chunk + kTileTokens - 1) / kTileTokens * kTileTokens;
-  SplitPlan p;
-  p.chunk_tokens = static_cast<int>(chunk);
-  p.max_splits = static_cast<int>((max_seq_len + chunk - 1) / chunk);
-  return p;
-}
-
-size_t split_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t v_head_dim, int max_splits) {
-  if (max_splits <= 1) return 0;
-  return static_cast<size_t>(batch) * n_q_heads * max_splits * (v_head_dim + 1) * sizeof(float);
-}
-
-int merge_splits(const float* ws_out, const float* ws_lse, void* out, float* lse,
-                 const PageAddressing& addr, int64_t batch, int64_t n_heads, int64_t v_head_dim,
-                 int64_t block_size, int64_t out_token_stride, int chunk_tokens, int max_splits,
-                 int out_dtype, hipStream_t stream) {
-  GqaArgs a = {};
-  a.block_table = addr.block_table;
-  a.seq_lens = addr.seq_lens;
-  a.indptr = addr.indptr;
-  a.indices = addr.indices;
-  a.last_page_len = addr.last_page_len;
-  a.table_stride = addr.table_stride;
-  a.out_stride_bytes = out_token_stride * 2;
-  a.n_q_heads = static_cast<int>(n_heads);
-  a.block_size = static_cast<int>(block_size);
-  a.chunk_tokens = chunk_tokens;
-  a.max_splits = max_splits;
-  dim3 grid(static_cast<unsigned>(n_heads), static_cast<unsigned>(batch));
-  if (out_dtype == XLLM_MI355_BF16)
-    merge_splits_kernel<BF16><<<grid, 128, 0, stream>>>(ws_out, ws_lse, static_cast<char*>(out), lse, a,
-                                                        static_cast<int>(v_head_dim));
-  else
-    merge_splits_kernel<FP16><<<grid, 128, 0, stream>>>(ws_out, ws_lse, static_cast<char*>(out), lse, a,
-                                                        static_cast<int>(v_head_dim));
-  return static_cast<int>(hipGetLastError());
+size_t gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim) {
+  // Upper bound over every kernel variant: at most 8 workgroups per CU, 8 heads per block.
+  (void)n_q_heads;
+  const size_t b = static_cast<size_t>(batch < kMaxBatch ? batch : kMaxBatch);
+  const size_t prefix_bytes = ((b + 1) * 4 + 255) / 256 * 256;
+  return prefix_bytes + static_cast<size_t>(device_cu_count()) * 8 * 2 * 8 * (head_dim + 1) * 4;
 }
 
 int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out, float* lse,
@@ -510,14 +590,15 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
                      int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
                      int64_t out_token_stride, int64_t max_seq_len, float sm_scale, void* workspace,
                      size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream) {
+  (void)max_seq_len;  // the schedule is computed on the device from the actual lengths
   if (batch == 0) return XLLM_MI355_OK;
   if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr) return XLLM_MI355_EINVAL;
   const bool csr = addr.indptr != nullptr;
   if (csr ? (addr.indices == nullptr || addr.last_page_len == nullptr)
           : (addr.block_table == nullptr || addr.seq_lens == nullptr || addr.table_stride <= 0))
     return XLLM_MI355_EINVAL;
-  if (batch < 0 || batch > 65535 || n_q_heads <= 0 || n_kv_heads <= 0 || block_size <= 0 ||
-      num_blocks <= 0 || n_q_heads % n_kv_heads != 0 || n_q_heads > 65535)
+  if (batch < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || block_size <= 0 || num_blocks <= 0 ||
+      n_q_heads % n_kv_heads != 0 || n_q_heads > 65535 || !(sm_scale > 0.0f))
     return XLLM_MI355_EINVAL;
   if (num_blocks * block_size > 0x7fffffffLL) return XLLM_MI355_ESHAPE;
   if (q_dtype != XLLM_MI355_BF16 && q_dtype != XLLM_MI355_FP16) return XLLM_MI355_EDTYPE;
@@ -530,71 +611,61 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
   auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (q_token_stride * 2) % 16 != 0)
     return XLLM_MI355_EALIGN;
-  if (max_seq_len <= 0) {
-    if (csr) return XLLM_MI355_EINVAL;  // CSR carries no host-visible bound
-    max_seq_len = addr.table_stride * block_size;
-  }
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return XLLM_MI355_EWORKSPACE;
 
   const int group = static_cast<int>(n_q_heads / n_kv_heads);
-  const int g_block = group_block(group);
-  const int hb = static_cast<int>(n_kv_heads) * ((group + g_block - 1) / g_block);
-  if (hb > 65535) return XLLM_MI355_ESHAPE;
-  SplitPlan plan = plan_splits(batch, hb, max_seq_len);
-  // fewer, longer splits if the caller's workspace is small
-  while (plan.max_splits > 1 &&
-         split_workspace_bytes(batch, n_q_heads, head_dim, plan.max_splits) > workspace_bytes) {
-    if (plan.chunk_tokens >= 8192) return XLLM_MI355_EWORKSPACE;
-    plan.chunk_tokens *= 2;
-    if (plan.chunk_tokens > 8192) plan.chunk_tokens = 8192;
-    plan.max_splits = static_cast<int>((max_seq_len + plan.chunk_tokens - 1) / plan.chunk_tokens);
-  }
-  if (plan.max_splits > 1 && (workspace == nullptr || !aligned16(workspace))) return XLLM_MI355_EWORKSPACE;
+  // Batches beyond the LDS prefix capacity are decoded in slices; each slice is an
+  // independent launch pair on the same stream and workspace.
+  for (int64_t b0 = 0; b0 < batch; b0 += kMaxBatch) {
+    const int64_t nb = batch - b0 < kMaxBatch ? batch - b0 : kMaxBatch;
+    GqaArgs a = {};
+    a.q = static_cast<const char*>(q) + b0 * q_token_stride * 2;
+    a.k_cache = static_cast<const char*>(k_cache);
+    a.v_cache = static_cast<const char*>(v_cache);
+    a.out = static_cast<char*>(out) + b0 * out_token_stride * 2;
+    a.lse = lse == nullptr ? nullptr : lse + b0 * n_q_heads;
+    a.block_table = csr ? nullptr : addr.block_table + b0 * addr.table_stride;
+    a.seq_lens = csr ? nullptr : addr.seq_lens + b0;
+    a.indptr = csr ? addr.indptr + b0 : nullptr;
+    a.indices = addr.indices;
+    a.last_page_len = csr ? addr.last_page_len + b0 : nullptr;
+    a.k_scale = k_scale;
+    a.v_scale = v_scale;
+    a.ws_prefix = static_cast<int*>(workspace);
+    a.table_stride = addr.table_stride;
+    a.q_stride_bytes = q_token_stride * 2;
+    a.out_stride_bytes = out_token_stride * 2;
+    a.row_bytes = n_kv_heads * head_dim * (fp8 ? 1 : 2);
+    a.batch = static_cast<int>(nb);
+    a.n_q_heads = static_cast<int>(n_q_heads);
+    a.n_kv_heads = static_cast<int>(n_kv_heads);
+    a.group = group;
+    a.g_block = group_block(group);
+    a.block_size = static_cast<int>(block_size);
+    a.bs_shift = -1;
+    for (int s = 0; s < 31; ++s)
+      if ((1LL << s) == block_size) a.bs_shift = s;
+    a.num_blocks = static_cast<int>(num_blocks);
+    a.scale_log2 = sm_scale * kLog2e;
 
-  GqaArgs a = {};
-  a.q = static_cast<const char*>(q);
-  a.k_cache = static_cast<const char*>(k_cache);
-  a.v_cache = static_cast<const char*>(v_cache);
-  a.out = static_cast<char*>(out);
-  a.lse = lse;
-  a.block_table = addr.block_table;
-  a.seq_lens = addr.seq_lens;
-  a.indptr = addr.indptr;
-  a.indices = addr.indices;
-  a.last_page_len = addr.last_page_len;
-  a.k_scale = k_scale;
-  a.v_scale = v_scale;
-  a.table_stride = addr.table_stride;
-  a.q_stride_bytes = q_token_stride * 2;
-  a.out_stride_bytes = out_token_stride * 2;
-  a.row_bytes = n_kv_heads * head_dim * (fp8 ? 1 : 2);
-  a.n_q_heads = static_cast<int>(n_q_heads);
-  a.n_kv_heads = static_cast<int>(n_kv_heads);
-  a.group = group;
-  a.block_size = static_cast<int>(block_size);
-  a.bs_shift = -1;
-  for (int s = 0; s < 31; ++s)
-    if ((1LL << s) == block_size) a.bs_shift = s;
-  a.num_blocks = static_cast<int>(num_blocks);
-  a.chunk_tokens = plan.chunk_tokens;
-  a.max_splits = plan.max_splits;
-  a.scale_log2 = sm_scale * kLog2e;
-  if (plan.max_splits > 1) {
-    a.ws_out = static_cast<float*>(workspace);
-    a.ws_lse = a.ws_out + static_cast<size_t>(batch) * n_q_heads * plan.max_splits * head_dim;
+    size_t need = 0;
+    int rc;
+    if (q_dtype == XLLM_MI355_BF16)
+      rc = fp8 ? dispatch_dim<BF16, true>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need)
+               : dispatch_dim<BF16, false>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need);
+    else
+      rc = fp8 ? dispatch_dim<FP16, true>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need)
+               : dispatch_dim<FP16, false>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need);
+    if (rc != 0) return rc;
+    dim3 grid(static_cast<unsigned>(n_q_heads), static_cast<unsigned>(nb));
+    if (q_dtype == XLLM_MI355_BF16)
+      merge_partials_kernel<BF16><<<grid, 128, 0, stream>>>(a, static_cast<int>(head_dim));
+    else
+      merge_partials_kernel<FP16><<<grid, 128, 0, stream>>>(a, static_cast<int>(head_dim));
+    rc = static_cast<int>(hipGetLastError());
+    if (rc != 0) return rc;
   }
-
-  int rc;
-  const bool timed = profile_begin(stream);
-  if (q_dtype == XLLM_MI355_BF16)
-    rc = fp8 ? dispatch_dim<BF16, true>(a, batch, static_cast<int>(head_dim), g_block, stream)
-             : dispatch_dim<BF16, false>(a, batch, static_cast<int>(head_dim), g_block, stream);
-  else
-    rc = fp8 ? dispatch_dim<FP16, true>(a, batch, static_cast<int>(head_dim), g_block, stream)
-             : dispatch_dim<FP16, false>(a, batch, static_cast<int>(head_dim), g_block, stream);
-  if (timed) profile_end(stream);
-  if (rc != 0 || plan.max_splits <= 1) return rc;
-  return merge_splits(a.ws_out, a.ws_lse, out, lse, addr, batch, n_q_heads, head_dim, block_size,
-                      out_token_stride, plan.chunk_tokens, plan.max_splits, q_dtype, stream);
+  return XLLM_MI355_OK;
 }
 
 }  // namespace xllm_mi355

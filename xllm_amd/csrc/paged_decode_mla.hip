@@ -19,6 +19,8 @@
 //
 // Semantics: xllm/core/kernels/dcu/flash_mla_adapter.h:40-53 (shapes, single KV head),
 // tests/core/layers/mlu/dcp_attention_merge_test.cpp:77-144 (V = K[..., :512], natural-log LSE).
+#include <cstdlib>
+
 #include "common.cuh"
 #include "launch.h"
 
@@ -63,6 +65,63 @@ struct MlaArgs {
   int max_splits;
   float scale_log2;
 };
+
+struct SplitPlan {
+  int chunk_tokens;  // tokens of one split (multiple of the tile)
+  int max_splits;    // ceil(max_seq_len / chunk_tokens)
+};
+
+SplitPlan plan_mla_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len) {
+  // One MLA workgroup owns a CU (its two LDS tiles fill it) and every split costs a
+  // [heads, 512] fp32 partial, so: about two workgroups per CU, splits of at least 512 tokens.
+  static const int64_t kTarget = [] {
+    const char* e = getenv("XLLM_MI355_MLA_TARGET_WGS");  // tuning knob
+    const long v = e ? atol(e) : 0;
+    return static_cast<int64_t>(v > 0 ? v : 512);
+  }();
+  constexpr int64_t kMinChunk = 512;
+  if (max_seq_len < 1) max_seq_len = 1;
+  const int64_t units = batch * n_head_blocks > 0 ? batch * n_head_blocks : 1;
+  int64_t splits = (kTarget + units - 1) / units;
+  const int64_t max_by_len = (max_seq_len + kMinChunk - 1) / kMinChunk;
+  if (splits > max_by_len) splits = max_by_len;
+  if (splits < 1) splits = 1;
+  int64_t chunk = (max_seq_len + splits - 1) / splits;
+  chunk = (chunk + kTile - 1) / kTile * kTile;
+  SplitPlan p;
+  p.chunk_tokens = static_cast<int>(chunk);
+  p.max_splits = static_cast<int>((max_seq_len + chunk - 1) / chunk);
+  return p;
+}
+
+size_t split_workspace_bytes(int64_t batch, int64_t n_heads, int max_splits) {
+  if (max_splits <= 1) return 0;
+  return static_cast<size_t>(batch) * n_heads * max_splits * (kDL + 1) * sizeof(float);
+}
+
+// Merge of split partials: one workgroup per (head, sequence).
+__global__ __launch_bounds__(128) void mla_merge_kernel(const float* ws_out, const float* ws_lse,
+                                                        char* out, float* lse, const int32_t* seq_lens,
+                                                        int n_heads, int chunk_tokens, int max_splits) {
+  const int h = blockIdx.x;
+  const int b = blockIdx.y;
+  const int L = seq_lens[b];
+  const int n_splits = (L + chunk_tokens - 1) / chunk_tokens;
+  if (n_splits <= 1) return;  // written directly by the decode kernel
+  const int64_t w0 = (static_cast<int64_t>(b) * n_heads + h) * max_splits;
+  float mx = kNegBig;
+  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, ws_lse[w0 + s]);
+  float wsum = 0.0f;
+  for (int s = 0; s < n_splits; ++s) wsum += fast_exp2(ws_lse[w0 + s] - mx);
+  const float inv = 1.0f / wsum;
+  uint16_t* o = reinterpret_cast<uint16_t*>(out) + (static_cast<int64_t>(b) * n_heads + h) * kDL;
+  for (int d = threadIdx.x; d < kDL; d += 128) {
+    float acc = 0.0f;
+    for (int s = 0; s < n_splits; ++s) acc += fast_exp2(ws_lse[w0 + s] - mx) * ws_out[(w0 + s) * kDL + d];
+    o[d] = BF16::from_f32(acc * inv);
+  }
+  if (lse != nullptr && threadIdx.x == 0) lse[b * n_heads + h] = (mx + fast_log2(wsum)) * kLn2;
+}
 
 __device__ __forceinline__ float xlane_max(float x) {  // over lanes l, l^16, l^32, l^48
   auto r = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
@@ -278,7 +337,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   if (q_nope == nullptr || q_pe == nullptr || k_cache == nullptr || out == nullptr ||
       addr.block_table == nullptr || addr.seq_lens == nullptr || addr.table_stride <= 0)
     return XLLM_MI355_EINVAL;
-  if (batch < 0 || batch > 65535 || n_heads <= 0 || n_heads > 65535 * kHeadsPerWg || block_size <= 0 ||
+  if (batch < 0 || batch > 65535 || n_heads <= 0 || n_heads > 65535 || block_size <= 0 ||
       num_blocks <= 0)
     return XLLM_MI355_EINVAL;
   if (d_latent != kDL || d_rope != kDR) return XLLM_MI355_ESHAPE;
@@ -292,7 +351,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   const int head_blocks = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
   SplitPlan plan = plan_mla_splits(batch, head_blocks, max_seq_len);
   while (plan.max_splits > 1 &&
-         split_workspace_bytes(batch, n_heads, kDL, plan.max_splits) > workspace_bytes) {
+         split_workspace_bytes(batch, n_heads, plan.max_splits) > workspace_bytes) {
     if (plan.chunk_tokens >= (1 << 20)) return XLLM_MI355_EWORKSPACE;
     plan.chunk_tokens *= 2;
     plan.max_splits = static_cast<int>((max_seq_len + plan.chunk_tokens - 1) / plan.chunk_tokens);
@@ -337,8 +396,16 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   if (timed) profile_end(stream);
   int rc = static_cast<int>(hipGetLastError());
   if (rc != 0 || plan.max_splits <= 1) return rc;
-  return merge_splits(a.ws_out, a.ws_lse, out, lse, addr, batch, n_heads, kDL, block_size,
-                      n_heads * kDL, plan.chunk_tokens, plan.max_splits, dtype, stream);
+  mla_merge_kernel<<<dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(batch)), 128, 0, stream>>>(
+      a.ws_out, a.ws_lse, static_cast<char*>(out), lse, addr.seq_lens, static_cast<int>(n_heads),
+      plan.chunk_tokens, plan.max_splits);
+  return static_cast<int>(hipGetLastError());
+}
+
+size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) {
+  if (max_seq_len <= 0) return 0;
+  const SplitPlan plan = plan_mla_splits(batch, (n_heads + kHeadsPerWg - 1) / kHeadsPerWg, max_seq_len);
+  return split_workspace_bytes(batch, n_heads, plan.max_splits);
 }
 
 }  // namespace xllm_mi355
