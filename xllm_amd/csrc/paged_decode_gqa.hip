@@ -377,20 +377,31 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
         else compute_tile(t, step, std::false_type{});
       };
 
-      // steps are dealt round-robin to the wavefronts; two register tiles alternate so that
-      // the loads of the next step are in flight while the current one is reduced
-      Tile ta, tb;
+      // Steps are dealt round-robin to the wavefronts; three register tiles rotate so that the
+      // loads of the next two steps are in flight while the current one is reduced.  Every
+      // iteration issues its prefetch unconditionally (past the end it re-reads the last
+      // step), so the number of loads in flight at each use is a compile-time constant and
+      // the compiler can wait for exactly the tile it needs instead of draining the queue.
       int step = wave;
-      if (step < n_steps) load_tile(ta, step);
-      while (step < n_steps) {
-        const int next = step + kWaves;
-        if (next < n_steps) load_tile(tb, next);
-        compute(ta, step);
-        if (next >= n_steps) break;
-        const int next2 = next + kWaves;
-        if (next2 < n_steps) load_tile(ta, next2);
-        compute(tb, next);
-        step = next2;
+      if (step < n_steps) {
+        const int last = n_steps - 1;
+        Tile ta, tb, tc;
+        load_tile(ta, step);
+        load_tile(tb, min(step + kWaves, last));
+        while (true) {
+          load_tile(tc, min(step + 2 * kWaves, last));
+          compute(ta, step);
+          step += kWaves;
+          if (step >= n_steps) break;
+          load_tile(ta, min(step + 2 * kWaves, last));
+          compute(tb, step);
+          step += kWaves;
+          if (step >= n_steps) break;
+          load_tile(tb, min(step + 2 * kWaves, last));
+          compute(tc, step);
+          step += kWaves;
+          if (step >= n_steps) break;
+        }
       }
     }
 
