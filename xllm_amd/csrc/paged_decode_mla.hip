@@ -1,21 +1,33 @@
 // Paged decode attention, MLA latent-KV variant, for gfx950.
 //
 // All query heads share ONE latent KV head of 576 dims (512 latent + 64 rope); V is the
-// first 512 dims of the same rows.  With 16..128 heads per sequence the two products are
-// dense contractions, so they run on MFMA (v_mfma_f32_16x16x32_bf16):
-//   S^T[tok, head]  = K[tok, 576] . Q^T[576, head]       A = K tile from LDS (16-byte rows)
+// first 512 dims of the same rows.  With up to 128 heads per sequence the two products are
+// dense contractions, so they run on MFMA (v_mfma_f32_32x32x16_bf16):
+//   S^T[tok, head]  = K[tok, 576] . Q^T[576, head]       A = K rows from the LDS tile
 //                                                        B = Q^T, resident in registers
-//   O^T[dim, head] += V^T[dim, tok] . P^T[tok, head]     A = V^T read from the SAME LDS tile
+//   O^T[dim, head] += V^T[dim, tok] . P^T[tok, head]     A = V^T, read from the SAME LDS tile
 //                                                            with the transposing LDS load
-//                                                        B = P^T, taken straight from the
-//                                                            S^T accumulator registers
-// so each 64-token page is staged in LDS once (rows padded to 1168 bytes, which spreads
-// 16 consecutive rows over all banks for the 16-byte operand reads) and serves both
-// products; softmax state lives in the lanes that own a head column, and the rescale of
-// the 128 output accumulators is skipped while the running maximum does not move.
-// One 256-thread workgroup covers 64 heads (16 per wavefront) of one (sequence, split);
-// tiles are double-buffered in LDS with the next tile's global loads in flight during
-// the MFMAs.  Splits write normalised fp32 partials that merge_splits folds.
+//                                                        B = P^T, taken from the S^T
+//                                                            accumulator registers
+// so every 64-token tile is staged in LDS once (rows padded to 1168 bytes: 16 consecutive
+// rows then cover all banks for the 16-byte operand reads) and serves both products.
+//
+// Tiles travel from global memory straight into LDS (global_load_lds_dwordx4), double
+// buffered, with the next tile in flight during the whole current tile.
+//
+// Workgroup = 256 threads = 64 heads: wavefront (hb, t) owns heads 32hb..32hb+31; for
+// Q.K it takes token block t (32 tokens) over all 576 dims, for P.V it takes dims
+// 256t..256t+255 over all 64 tokens.  The two wavefronts of a head block swap their
+// bf16 P^T block and its row maxima through LDS once per tile.  Two barriers per tile:
+// (A) tile landed / previous P.V done, (B) exchange visible.  The accumulators are
+// rescaled only on tiles where a running maximum moved.
+//
+// Scheduling: the 64-token tiles of the whole batch form one flat list; a fixed grid of
+// persistent workgroups, one per CU, grouped in teams of ceil(H/64) that share a tile
+// range (team members get block ids 8 apart, i.e. the same XCD, so the second reader of a
+// tile hits that XCD's L2), splits the list into equal contiguous ranges.  A run that
+// covers a whole context writes the output, a partial run writes a normalised fp32 partial
+// + log2-domain LSE and a small merge kernel folds those.
 //
 // Semantics: xllm/core/kernels/dcu/flash_mla_adapter.h:40-53 (shapes, single KV head),
 // tests/core/layers/mlu/dcp_attention_merge_test.cpp:77-144 (V = K[..., :512], natural-log LSE).
@@ -31,20 +43,23 @@ namespace {
 constexpr int kDL = 512;            // latent dims (= V dims)
 constexpr int kDR = 64;             // rope dims
 constexpr int kDK = kDL + kDR;      // QK dims
-constexpr int kTile = 64;           // tokens per LDS tile
+constexpr int kTile = 64;           // tokens per LDS tile (= one schedulable item)
 constexpr int kRowBytes = kDK * 2;  // 1152
 constexpr int kLdsRow = kRowBytes + 16;
 constexpr int kTileBytes = kTile * kLdsRow;  // 74752
 constexpr int kMlaThreads = 256;
-constexpr int kMlaWaves = kMlaThreads / kWave;
-constexpr int kHeadsPerWg = 16 * kMlaWaves;  // 64
-constexpr int kChunksPerRow = kRowBytes / 16;                                 // 72
-constexpr int kLoadsPerThread = kTile * kChunksPerRow / kMlaThreads;          // 18
-constexpr int kKSteps = kDK / 32;   // 18
-constexpr int kMBlocks = kDL / 16;  // 32
+constexpr int kHeadsPerWg = 64;
+constexpr int kKSteps = kDK / 16;   // 36 k-steps of the 32x32x16 MFMA
+constexpr int kMaxBatchMla = 1024;  // sequences per launch (their tile prefix lives in LDS)
+// LDS map: two tiles | P^T exchange [4 waves][8 regs][64 lanes] | row-max exchange [4][32] | prefix
+constexpr int kXchPOff = 2 * kTileBytes;
+constexpr int kXchMOff = kXchPOff + 4 * 8 * 64 * 4;
+constexpr int kPrefixOff = kXchMOff + 4 * 32 * 4;
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 struct MlaArgs {
   const char* q_nope;
@@ -54,147 +69,139 @@ struct MlaArgs {
   float* lse;
   const int32_t* block_table;
   const int32_t* seq_lens;
-  float* ws_out;
-  float* ws_lse;
+  int* ws_prefix;  // [batch + 1]
+  float* ws_out;   // [2 * n_teams][H][512]
+  float* ws_lse;   // [2 * n_teams][H]
   int64_t table_stride;
+  int batch;
   int n_heads;
+  int n_hb;        // head blocks of 64 = workgroups per team
+  int n_teams;
   int block_size;
   int bs_shift;
   int num_blocks;
-  int chunk_tokens;
-  int max_splits;
   float scale_log2;
 };
 
-struct SplitPlan {
-  int chunk_tokens;  // tokens of one split (multiple of the tile)
-  int max_splits;    // ceil(max_seq_len / chunk_tokens)
-};
-
-SplitPlan plan_mla_splits(int64_t batch, int64_t n_head_blocks, int64_t max_seq_len) {
-  // One MLA workgroup owns a CU (its two LDS tiles fill it) and every split costs a
-  // [heads, 512] fp32 partial, so: about two workgroups per CU, splits of at least 512 tokens.
-  static const int64_t kTarget = [] {
-    const char* e = getenv("XLLM_MI355_MLA_TARGET_WGS");  // tuning knob
-    const long v = e ? atol(e) : 0;
-    return static_cast<int64_t>(v > 0 ? v : 512);
-  }();
-  constexpr int64_t kMinChunk = 512;
-  if (max_seq_len < 1) max_seq_len = 1;
-  const int64_t units = batch * n_head_blocks > 0 ? batch * n_head_blocks : 1;
-  int64_t splits = (kTarget + units - 1) / units;
-  const int64_t max_by_len = (max_seq_len + kMinChunk - 1) / kMinChunk;
-  if (splits > max_by_len) splits = max_by_len;
-  if (splits < 1) splits = 1;
-  int64_t chunk = (max_seq_len + splits - 1) / splits;
-  chunk = (chunk + kTile - 1) / kTile * kTile;
-  SplitPlan p;
-  p.chunk_tokens = static_cast<int>(chunk);
-  p.max_splits = static_cast<int>((max_seq_len + chunk - 1) / chunk);
-  return p;
+__device__ __forceinline__ int tiles_of(int L) { return L > 0 ? (L + kTile - 1) / kTile : 0; }
+__device__ __forceinline__ int64_t team_start(int64_t t, int64_t total, int64_t n) { return t * total / n; }
+__device__ __forceinline__ int team_of(int64_t id, int64_t total, int64_t n) {
+  int64_t t = id * n / total;
+  while (t + 1 < n && team_start(t + 1, total, n) <= id) ++t;
+  return static_cast<int>(t);
 }
 
-size_t split_workspace_bytes(int64_t batch, int64_t n_heads, int max_splits) {
-  if (max_splits <= 1) return 0;
-  return static_cast<size_t>(batch) * n_heads * max_splits * (kDL + 1) * sizeof(float);
-}
-
-// Merge of split partials: one workgroup per (head, sequence).
-__global__ __launch_bounds__(128) void mla_merge_kernel(const float* ws_out, const float* ws_lse,
-                                                        char* out, float* lse, const int32_t* seq_lens,
-                                                        int n_heads, int chunk_tokens, int max_splits) {
-  const int h = blockIdx.x;
-  const int b = blockIdx.y;
-  const int L = seq_lens[b];
-  const int n_splits = (L + chunk_tokens - 1) / chunk_tokens;
-  if (n_splits <= 1) return;  // written directly by the decode kernel
-  const int64_t w0 = (static_cast<int64_t>(b) * n_heads + h) * max_splits;
-  float mx = kNegBig;
-  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, ws_lse[w0 + s]);
-  float wsum = 0.0f;
-  for (int s = 0; s < n_splits; ++s) wsum += fast_exp2(ws_lse[w0 + s] - mx);
-  const float inv = 1.0f / wsum;
-  uint16_t* o = reinterpret_cast<uint16_t*>(out) + (static_cast<int64_t>(b) * n_heads + h) * kDL;
-  for (int d = threadIdx.x; d < kDL; d += 128) {
-    float acc = 0.0f;
-    for (int s = 0; s < n_splits; ++s) acc += fast_exp2(ws_lse[w0 + s] - mx) * ws_out[(w0 + s) * kDL + d];
-    o[d] = BF16::from_f32(acc * inv);
-  }
-  if (lse != nullptr && threadIdx.x == 0) lse[b * n_heads + h] = (mx + fast_log2(wsum)) * kLn2;
-}
-
-__device__ __forceinline__ float xlane_max(float x) {  // over lanes l, l^16, l^32, l^48
-  auto r = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
-  x = fmaxf(as_f32(r[0]), as_f32(r[1]));
+__device__ __forceinline__ float half_swap_max(float x) {  // over lanes l and l ^ 32
   auto t = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
   return fmaxf(as_f32(t[0]), as_f32(t[1]));
 }
-
-__device__ __forceinline__ float xlane_sum(float x) {
-  auto r = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
-  x = as_f32(r[0]) + as_f32(r[1]);
+__device__ __forceinline__ float half_swap_sum(float x) {
   auto t = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
   return as_f32(t[0]) + as_f32(t[1]);
 }
 
+// 16 bytes per active lane from global memory straight into LDS at lds_addr + lane * 16
+// (lds_addr is wave-uniform; it travels in M0).
+__device__ __forceinline__ void dma16(const void* gptr, u32 lds_addr) {
+  const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
-  extern __shared__ __align__(16) char smem[];  // two tiles of [64][1168] bytes
+  extern __shared__ __align__(16) char smem[];
+  u32* xch_p = reinterpret_cast<u32*>(smem + kXchPOff);
+  float* xch_m = reinterpret_cast<float*>(smem + kXchMOff);
+  int* prefix = reinterpret_cast<int*>(smem + kPrefixOff);
+  int* tmp = reinterpret_cast<int*>(smem + kXchPOff);  // prologue only
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = tid >> 6;
-  const int c16 = lane & 15;  // MFMA row / column index owned by the lane
-  const int g = lane >> 4;    // MFMA k-group of the lane
-  const int split = blockIdx.x;
-  const int b = blockIdx.z;
-  const int head_base = blockIdx.y * kHeadsPerWg;
-  const int head = head_base + wave * 16 + c16;
-  const bool head_ok = head < a.n_heads;
-  const bool wave_ok = head_base + wave * 16 < a.n_heads;
+  const int hb32 = wave >> 1;   // 32-head block of the wavefront
+  const int tblk = wave & 1;    // its token block for Q.K and its dim half for P.V
+  const int c32 = lane & 31;    // MFMA row / column index owned by the lane
+  const int g = lane >> 5;      // MFMA k-group of the lane
   const int H = a.n_heads;
 
-  const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
-  const int L = a.seq_lens[b];
-  if (L <= 0) {
-    if (split == 0 && head_ok) {
-      u32x2* o = reinterpret_cast<u32x2*>(a.out + (static_cast<int64_t>(b) * H + head) * kDL * 2);
-      for (int i = g; i < kDL / 4; i += 4) o[i] = u32x2{0u, 0u};
-      if (a.lse != nullptr && g == 0) a.lse[b * H + head] = -INFINITY;
-    }
-    return;
-  }
-  const int n_splits = (L + a.chunk_tokens - 1) / a.chunk_tokens;
-  if (split >= n_splits) return;
-  const int t0 = split * a.chunk_tokens;
-  const int t1 = min(L, t0 + a.chunk_tokens);
-  const int n_tiles = (t1 - t0 + kTile - 1) / kTile;
+  // block id -> (team, head block): members of a team are 8 ids apart (same XCD)
+  const int xcd = blockIdx.x & 7;
+  const int y = blockIdx.x >> 3;
+  const int hb64 = y % a.n_hb;
+  const int team = (y / a.n_hb) * 8 + xcd;
+  const int head = hb64 * kHeadsPerWg + hb32 * 32 + c32;
+  const bool head_ok = head < H;
+  const bool wave_ok = hb64 * kHeadsPerWg + hb32 * 32 < H;
 
-  // Q^T operand: lane (head c16, k-group g) keeps dims ks*32 + g*8 .. +8 of every k-step
-  bf16x8 q[kKSteps];
+  // ---- tile prefix over the batch (every workgroup computes it; no extra launch)
   {
-    const char* qn = a.q_nope + (static_cast<int64_t>(b) * H + head) * kDL * 2;
-    const char* qp = a.q_pe + (static_cast<int64_t>(b) * H + head) * kDR * 2;
-#pragma unroll
-    for (int ks = 0; ks < kKSteps; ++ks) {
-      u32x4 x = {0u, 0u, 0u, 0u};
-      if (head_ok) x = ks < kDL / 32 ? ldg16(qn + (ks * 32 + g * 8) * 2) : ldg16(qp + ((ks - kDL / 32) * 32 + g * 8) * 2);
-      q[ks] = __builtin_bit_cast(bf16x8, x);
+    const int per = (a.batch + kMlaThreads - 1) / kMlaThreads;
+    const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
+    int local = 0;
+    for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
+    tmp[tid] = local;
+    __syncthreads();
+    int excl = 0;
+    for (int j = 0; j < tid; ++j) excl += tmp[j];
+    for (int b = lo; b < hi; ++b) {
+      prefix[b] = excl;
+      excl += tiles_of(a.seq_lens[b]);
     }
+    if (lo < hi && hi == a.batch) prefix[a.batch] = excl;
+    __syncthreads();
   }
+  const int64_t total = prefix[a.batch];
+  if (blockIdx.x == 0)
+    for (int i = tid; i <= a.batch; i += kMlaThreads) a.ws_prefix[i] = prefix[i];
+  if (total == 0) return;
+  int64_t cur = team_start(team, total, a.n_teams);
+  const int64_t end = team_start(team + 1, total, a.n_teams);
+  bool first_run = true;
 
-  f32x4 o[kMBlocks];
-#pragma unroll
-  for (int i = 0; i < kMBlocks; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = kNegBig, l = 0.0f;
+  const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
 
-  u32x4 stage[kLoadsPerThread];
-  auto load_tile = [&](int tile) {
+  while (cur < end) {
+    int lo = 0, hi = a.batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (prefix[mid] <= cur) lo = mid; else hi = mid;
+    }
+    const int b = lo;
+    const int n_tiles_seq = prefix[b + 1] - prefix[b];
+    const int tile0 = static_cast<int>(cur - prefix[b]);
+    const int run_tiles = static_cast<int>(min<int64_t>(n_tiles_seq - tile0, end - cur));
+    const bool complete = tile0 == 0 && run_tiles == n_tiles_seq;
+    cur += run_tiles;
+    const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
+    const int L = a.seq_lens[b];
+
+    // Q^T operand: lane (head c32, k-group g) keeps dims ks*16 + g*8 .. +8 of every k-step
+    bf16x8 q[kKSteps];
+    {
+      const char* qn = a.q_nope + (static_cast<int64_t>(b) * H + head) * kDL * 2;
+      const char* qp = a.q_pe + (static_cast<int64_t>(b) * H + head) * kDR * 2;
 #pragma unroll
-    for (int i = 0; i < kLoadsPerThread; ++i) {
-      const int c = i * kMlaThreads + tid;
-      const int row = c / kChunksPerRow;
-      const int col = c - row * kChunksPerRow;
-      const int tok = min(t0 + tile * kTile + row, L - 1);
+      for (int ks = 0; ks < kKSteps; ++ks) {
+        u32x4 x = {0u, 0u, 0u, 0u};
+        if (head_ok)
+          x = ks < kDL / 16 ? ldg16(qn + (ks * 16 + g * 8) * 2) : ldg16(qp + ((ks - kDL / 16) * 16 + g * 8) * 2);
+        q[ks] = __builtin_bit_cast(bf16x8, x);
+      }
+    }
+    f32x16 o[8];  // O^T blocks: dims tblk*256 + mb*32 + (8*(r/4) + 4g + r%4), head c32
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[i][r] = 0.0f;
+    float m = kNegBig, l = 0.0f;
+
+    // Tile rows go from global memory straight into LDS (no staging registers): one
+    // 64-lane load moves the 1024 latent bytes of a row, a second one with 8 lanes the 128
+    // rope bytes.  Each wavefront moves 16 rows; lane i < 16 first looks up the slot of row i.
+    // The loads are issued from inline assembly so that the compiler's own wait insertion
+    // does not see them: they are awaited explicitly (dma_wait) one tile later.
+    auto issue_tile = [&](int tile, int buf) {
+      const int tok = min((tile0 + tile) * kTile + wave * 16 + (lane & 15), L - 1);
       int pg, off;
       if (a.bs_shift >= 0) {
         pg = tok >> a.bs_shift;
@@ -204,141 +211,255 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         off = tok - pg * a.block_size;
       }
       int page = pages[pg];
-      page = max(0, min(page, a.num_blocks - 1));
-      const int64_t slot = static_cast<int64_t>(page) * a.block_size + off;
-      stage[i] = ldg16(a.k_cache + slot * kRowBytes + col * 16);
-    }
-  };
-  auto store_tile = [&](int buf) {
+      page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
+      const int slot = page * a.block_size + off;
+      const u32 lds_tile = lds_base + buf * kTileBytes + wave * 16 * kLdsRow;
 #pragma unroll
-    for (int i = 0; i < kLoadsPerThread; ++i) {
-      const int c = i * kMlaThreads + tid;
-      const int row = c / kChunksPerRow;
-      const int col = c - row * kChunksPerRow;
-      *reinterpret_cast<u32x4*>(smem + buf * kTileBytes + row * kLdsRow + col * 16) = stage[i];
-    }
-  };
+      for (int i = 0; i < 16; ++i) {
+        const int64_t s_i = __builtin_amdgcn_readlane(slot, i);
+        const char* row = a.k_cache + s_i * kRowBytes + lane * 16;
+        dma16(row, lds_tile + i * kLdsRow);
+        if (lane < kDR * 2 / 16) dma16(row + kDL * 2, lds_tile + i * kLdsRow + kDL * 2);
+      }
+    };
 
-  auto compute = [&](int buf, int tile) {
-    const char* kb = smem + buf * kTileBytes;
-    // ---- S^T = K . Q^T : 4 token blocks of 16, 18 k-steps
-    f32x4 s[4];
-#pragma unroll
-    for (int tb = 0; tb < 4; ++tb) s[tb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // make the compiler wait for the Q loads here, not after the first tile prefetch
 #pragma unroll
     for (int ks = 0; ks < kKSteps; ++ks) {
-#pragma unroll
-      for (int tb = 0; tb < 4; ++tb) {
-        const u32x4 x = *reinterpret_cast<const u32x4*>(kb + (tb * 16 + c16) * kLdsRow + (ks * 32 + g * 8) * 2);
-        s[tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x), q[ks], s[tb], 0, 0, 0);
-      }
+      u32x4 x = __builtin_bit_cast(u32x4, q[ks]);
+      asm volatile("" : "+v"(x));
+      q[ks] = __builtin_bit_cast(bf16x8, x);
     }
-    // ---- online softmax; the lane owns head c16 and tokens tb*16 + g*4 + i
-    const int tok_base = t0 + tile * kTile + g * 4;
-    float mx = kNegBig;
-#pragma unroll
-    for (int tb = 0; tb < 4; ++tb)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float v = tok_base + tb * 16 + i < t1 ? s[tb][i] * a.scale_log2 : -INFINITY;
-        s[tb][i] = v;
-        mx = fmaxf(mx, v);
-      }
-    mx = xlane_max(mx);
-    const float m_new = fmaxf(m, mx);
-    const float alpha = fast_exp2(m - m_new);
-    m = m_new;
-    float sum = 0.0f;
-#pragma unroll
-    for (int tb = 0; tb < 4; ++tb)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        s[tb][i] = fast_exp2(s[tb][i] - m_new);
-        sum += s[tb][i];
-      }
-    l = l * alpha + sum;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-      for (int i = 0; i < kMBlocks; ++i) o[i] *= alpha;
-    }
-    // P^T operands: k-step kk uses token blocks 2kk and 2kk+1, k-slot g*8+i <-> token block
-    // (2kk + i/4), row g*4 + i%4 -- the V^T operand below is gathered in the same order
-    bf16x8 pb[2];
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      u32x4 x;
-      x[0] = BF16::pack(s[2 * kk][0], s[2 * kk][1]);
-      x[1] = BF16::pack(s[2 * kk][2], s[2 * kk][3]);
-      x[2] = BF16::pack(s[2 * kk + 1][0], s[2 * kk + 1][1]);
-      x[3] = BF16::pack(s[2 * kk + 1][2], s[2 * kk + 1][3]);
-      pb[kk] = __builtin_bit_cast(bf16x8, x);
-    }
-    // ---- O^T += V^T . P^T : the transposing LDS load hands lane c16 the 4 tokens g*4..+4
-    // of dim column mb*16 + c16; each lane supplies the address of 4 dims of one token row
-    const char* vb = kb + (g * 4 + (c16 >> 2)) * kLdsRow + (c16 & 3) * 8;
-#pragma unroll
-    for (int mb = 0; mb < kMBlocks; ++mb) {
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s16x4*)(vb + (2 * kk) * 16 * kLdsRow + mb * 32));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s16x4*)(vb + (2 * kk + 1) * 16 * kLdsRow + mb * 32));
-        typedef __attribute__((ext_vector_type(8))) short s16x8;
-        const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        o[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb[kk], o[mb], 0, 0, 0);
-      }
-    }
-  };
+    __syncthreads();  // the previous run no longer reads the tiles or the exchange buffers
+    issue_tile(0, 0);
 
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    const int buf = tile & 1;
-    const bool more = tile + 1 < n_tiles;
-    if (more) load_tile(tile + 1);
-    if (wave_ok) compute(buf, tile);
-    if (more) store_tile(buf ^ 1);
+    for (int tile = 0; tile < run_tiles; ++tile) {
+      const int buf = tile & 1;
+      const char* kb = smem + buf * kTileBytes;
+      dma_wait();
+      __syncthreads();  // (A) this tile has landed in LDS; every wavefront is past the previous P.V
+      if (tile + 1 < run_tiles) issue_tile(tile + 1, buf ^ 1);  // in flight during the whole tile
+
+      float p_own[16];
+      float m_own = kNegBig;
+      if (wave_ok) {
+        // ---- S^T block of this wavefront: tokens tblk*32 + (8*(r/4) + 4g + r%4), head c32
+        f32x16 s, s2;  // two accumulation chains over alternate k-steps
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = s2[r] = 0.0f;
+        const char* ka = kb + (tblk * 32 + c32) * kLdsRow + g * 16;
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ks += 2) {
+          const u32x4 x0 = *reinterpret_cast<const u32x4*>(ka + ks * 32);
+          const u32x4 x1 = *reinterpret_cast<const u32x4*>(ka + ks * 32 + 32);
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x0), q[ks], s, 0, 0, 0);
+          s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x1), q[ks + 1], s2, 0, 0, 0);
+        }
+        s += s2;
+        const int tok_base = (tile0 + tile) * kTile + tblk * 32 + g * 4;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float v = tok_base + 8 * (r >> 2) + (r & 3) < L ? s[r] * a.scale_log2 : -INFINITY;
+          p_own[r] = v;
+          m_own = fmaxf(m_own, v);
+        }
+        m_own = half_swap_max(m_own);  // row maximum of this token block
+        u32 pk[8];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) p_own[r] = fast_exp2(p_own[r] - m_own);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pk[i] = BF16::pack(p_own[2 * i], p_own[2 * i + 1]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xch_p[(wave * 8 + i) * 64 + lane] = pk[i];
+        if (g == 0) xch_m[wave * 32 + c32] = m_own;
+      }
+      __syncthreads();  // (B) P^T blocks and maxima of this tile are visible
+      float m_other = kNegBig;
+      u32 theirs_raw[8];
+      if (wave_ok) {
+        m_other = xch_m[(wave ^ 1) * 32 + c32];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) theirs_raw[i] = xch_p[((wave ^ 1) * 8 + i) * 64 + lane];
+      }
+
+      if (wave_ok) {
+        const float m_new = fmaxf(m, fmaxf(m_own, m_other));
+        const float alpha = fast_exp2(m - m_new);
+        const float f_own = fast_exp2(m_own - m_new);
+        const float f_other = fast_exp2(m_other - m_new);
+        m = m_new;
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          p_own[r] *= f_own;
+          sum += p_own[r];
+        }
+        l = l * alpha + sum;  // this wavefront's share of the normaliser (its own token block)
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) o[i] *= alpha;
+        }
+        // B operands per k-step: k-slot g*8 + j <-> rows 16*kk + 4g + j (j < 4), + 8 more (j >= 4)
+        // of the own token block (pb_own) and of the partner's (pb_other)
+        bf16x8 pb_own[2], pb_other[2];
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          u32x4 mine, theirs;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            mine[i] = BF16::pack(p_own[8 * kk + 2 * i], p_own[8 * kk + 2 * i + 1]);
+            const u32 t = theirs_raw[4 * kk + i];
+            theirs[i] = BF16::pack(BF16::lo(t) * f_other, BF16::hi(t) * f_other);
+          }
+          pb_own[kk] = __builtin_bit_cast(bf16x8, mine);
+          pb_other[kk] = __builtin_bit_cast(bf16x8, theirs);
+        }
+        // ---- O^T += V^T . P^T over the 64 tokens, dims tblk*256 .. +256.  The transposing
+        // LDS load works on groups of 16 lanes: lane p of a group supplies the address of 4
+        // dims of token row p/4 and receives the 4 tokens of dim column p.
+        const int p16 = lane & 15;
+        const char* vb = kb + (g * 4 + (p16 >> 2)) * kLdsRow +
+                         (tblk * 256 + ((lane >> 4) & 1) * 16 + (p16 & 3) * 4) * 2;
+        const char* vb_own = vb + tblk * 32 * kLdsRow;
+        const char* vb_other = vb + (tblk ^ 1) * 32 * kLdsRow;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) {  // own token block: k-steps 0, 1; the partner's: 2, 3
+            const char* rows = (ks < 2 ? vb_own : vb_other) + (16 * (ks & 1)) * kLdsRow + mb * 64;
+            const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows));
+            const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows + 8 * kLdsRow));
+            const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+            o[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8, v), ks < 2 ? pb_own[ks & 1] : pb_other[ks & 1], o[mb], 0, 0, 0);
+          }
+        }
+      }
+    }
+
+    // ---- end of the run: the two wavefronts of a head block add their normaliser shares
     __syncthreads();
-  }
-
-  if (!head_ok) return;
-  l = xlane_sum(l);
-  const float inv = 1.0f / l;
-  if (n_splits == 1) {
-    char* op = a.out + (static_cast<int64_t>(b) * H + head) * kDL * 2;
+    const float l_wave = half_swap_sum(l);
+    if (wave_ok && g == 0) xch_m[wave * 32 + c32] = l_wave;
+    __syncthreads();
+    if (head_ok) {
+      const float lsum = xch_m[wave * 32 + c32] + xch_m[(wave ^ 1) * 32 + c32];
+      const float inv = 1.0f / lsum;
+      if (complete) {
+        char* op = a.out + ((static_cast<int64_t>(b) * H + head) * kDL + tblk * 256) * 2;
 #pragma unroll
-    for (int mb = 0; mb < kMBlocks; ++mb) {
-      u32x2 w;
-      w[0] = BF16::pack(o[mb][0] * inv, o[mb][1] * inv);
-      w[1] = BF16::pack(o[mb][2] * inv, o[mb][3] * inv);
-      *reinterpret_cast<u32x2*>(op + (mb * 16 + g * 4) * 2) = w;
+        for (int mb = 0; mb < 8; ++mb)
+#pragma unroll
+          for (int qd = 0; qd < 4; ++qd) {
+            u32x2 w;
+            w[0] = BF16::pack(o[mb][4 * qd] * inv, o[mb][4 * qd + 1] * inv);
+            w[1] = BF16::pack(o[mb][4 * qd + 2] * inv, o[mb][4 * qd + 3] * inv);
+            *reinterpret_cast<u32x2*>(op + (mb * 32 + 8 * qd + 4 * g) * 2) = w;
+          }
+        if (a.lse != nullptr && g == 0 && tblk == 0) a.lse[b * H + head] = (m + fast_log2(lsum)) * kLn2;
+      } else {
+        const int64_t ps = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H + head;
+        float* wp = a.ws_out + ps * kDL + tblk * 256;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb)
+#pragma unroll
+          for (int qd = 0; qd < 4; ++qd) {
+            f32x4 w = {o[mb][4 * qd] * inv, o[mb][4 * qd + 1] * inv, o[mb][4 * qd + 2] * inv,
+                       o[mb][4 * qd + 3] * inv};
+            *reinterpret_cast<f32x4*>(wp + mb * 32 + 8 * qd + 4 * g) = w;
+          }
+        if (g == 0 && tblk == 0) a.ws_lse[ps] = m + fast_log2(lsum);
+      }
     }
-    if (a.lse != nullptr && g == 0) a.lse[b * H + head] = (m + fast_log2(l)) * kLn2;
-  } else {
-    const int64_t wi = (static_cast<int64_t>(b) * H + head) * a.max_splits + split;
-    float* wp = a.ws_out + wi * kDL;
-#pragma unroll
-    for (int mb = 0; mb < kMBlocks; ++mb)
-      *reinterpret_cast<f32x4*>(wp + mb * 16 + g * 4) = o[mb] * inv;
-    if (g == 0) a.ws_lse[wi] = m + fast_log2(l);
+    first_run = false;
   }
 }
 
+// Merge of the partials of contexts that span several teams; also writes the output of
+// empty sequences.  One workgroup per (head, sequence).
+__global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
+  const int h = blockIdx.x;
+  const int b = blockIdx.y;
+  const int H = a.n_heads;
+  const int L = a.seq_lens[b];
+  uint16_t* out = reinterpret_cast<uint16_t*>(a.out) + (static_cast<int64_t>(b) * H + h) * kDL;
+  if (L <= 0) {
+    for (int d = threadIdx.x; d < kDL; d += 128) out[d] = 0;
+    if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = -INFINITY;
+    return;
+  }
+  const int64_t total = a.ws_prefix[a.batch];
+  const int64_t first = a.ws_prefix[b];
+  const int64_t last = a.ws_prefix[b + 1] - 1;
+  const int64_t n = a.n_teams;
+  const int t_first = team_of(first, total, n);
+  const int t_last = team_of(last, total, n);
+  if (t_first == t_last) return;  // one team saw the whole context and wrote the output
+  const int slot_first = team_start(t_first, total, n) < first ? 1 : 0;
+  auto pslot = [&](int t) { return (static_cast<int64_t>(t) * 2 + (t == t_first ? slot_first : 0)) * H + h; };
+  auto has_items = [&](int t) { return team_start(t, total, n) < team_start(t + 1, total, n); };
+  float mx = kNegBig;
+  for (int t = t_first; t <= t_last; ++t)
+    if (has_items(t)) mx = fmaxf(mx, a.ws_lse[pslot(t)]);
+  float wsum = 0.0f;
+  for (int t = t_first; t <= t_last; ++t)
+    if (has_items(t)) wsum += fast_exp2(a.ws_lse[pslot(t)] - mx);
+  const float inv = 1.0f / wsum;
+  for (int d = threadIdx.x; d < kDL; d += 128) {
+    float acc = 0.0f;
+    for (int t = t_first; t <= t_last; ++t) {
+      if (!has_items(t)) continue;
+      const int64_t ps = pslot(t);
+      acc += fast_exp2(a.ws_lse[ps] - mx) * a.ws_out[ps * kDL + d];
+    }
+    out[d] = BF16::from_f32(acc * inv);
+  }
+  if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = (mx + fast_log2(wsum)) * kLn2;
+}
+
+int mla_cu_count() {
+  static const int n = [] {
+    int dev = 0;
+    hipDeviceProp_t p;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 256;
+    return p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
+  }();
+  return n;
+}
+
+// Teams: as many as there are CUs for the team size, a multiple of 8 (one per XCD slot).
+int mla_teams(int n_hb) {
+  static const int wgs = [] {
+    const char* e = getenv("XLLM_MI355_MLA_WGS");  // tuning knob: workgroups in flight
+    const int v = e ? atoi(e) : 0;
+    return v > 0 ? v : mla_cu_count();
+  }();
+  int teams = wgs / n_hb / 8 * 8;
+  return teams < 8 ? 8 : teams;
+}
+
 }  // namespace
+
+size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) {
+  (void)max_seq_len;
+  const size_t b = static_cast<size_t>(batch < kMaxBatchMla ? batch : kMaxBatchMla);
+  const size_t prefix_bytes = ((b + 1) * 4 + 255) / 256 * 256;
+  const int n_hb = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
+  return prefix_bytes + static_cast<size_t>(mla_teams(n_hb)) * 2 * n_heads * (kDL + 1) * 4;
+}
 
 int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out, float* lse,
                      const PageAddressing& addr, int64_t batch, int64_t n_heads, int64_t d_latent,
                      int64_t d_rope, int64_t block_size, int64_t num_blocks, int64_t max_seq_len,
                      float sm_scale, void* workspace, size_t workspace_bytes, int dtype,
                      hipStream_t stream) {
+  (void)max_seq_len;  // the schedule is computed on the device from the actual lengths
   if (batch == 0) return XLLM_MI355_OK;
   if (q_nope == nullptr || q_pe == nullptr || k_cache == nullptr || out == nullptr ||
       addr.block_table == nullptr || addr.seq_lens == nullptr || addr.table_stride <= 0)
     return XLLM_MI355_EINVAL;
-  if (batch < 0 || batch > 65535 || n_heads <= 0 || n_heads > 65535 || block_size <= 0 ||
-      num_blocks <= 0)
+  if (batch < 0 || n_heads <= 0 || n_heads > 65535 || block_size <= 0 || num_blocks <= 0 ||
+      !(sm_scale > 0.0f))
     return XLLM_MI355_EINVAL;
   if (d_latent != kDL || d_rope != kDR) return XLLM_MI355_ESHAPE;
   if (dtype != XLLM_MI355_BF16) return XLLM_MI355_EDTYPE;
@@ -346,66 +467,55 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   if (!aligned16(q_nope) || !aligned16(q_pe) || !aligned16(k_cache) || !aligned16(out))
     return XLLM_MI355_EALIGN;
-  if (max_seq_len <= 0) max_seq_len = addr.table_stride * block_size;
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
+      workspace_bytes < mla_workspace_bytes(batch, n_heads, 0))
+    return XLLM_MI355_EWORKSPACE;
 
-  const int head_blocks = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
-  SplitPlan plan = plan_mla_splits(batch, head_blocks, max_seq_len);
-  while (plan.max_splits > 1 &&
-         split_workspace_bytes(batch, n_heads, plan.max_splits) > workspace_bytes) {
-    if (plan.chunk_tokens >= (1 << 20)) return XLLM_MI355_EWORKSPACE;
-    plan.chunk_tokens *= 2;
-    plan.max_splits = static_cast<int>((max_seq_len + plan.chunk_tokens - 1) / plan.chunk_tokens);
-  }
-  if (plan.max_splits > 1 && (workspace == nullptr || !aligned16(workspace))) return XLLM_MI355_EWORKSPACE;
-
-  MlaArgs a = {};
-  a.q_nope = static_cast<const char*>(q_nope);
-  a.q_pe = static_cast<const char*>(q_pe);
-  a.k_cache = static_cast<const char*>(k_cache);
-  a.out = static_cast<char*>(out);
-  a.lse = lse;
-  a.block_table = addr.block_table;
-  a.seq_lens = addr.seq_lens;
-  a.table_stride = addr.table_stride;
-  a.n_heads = static_cast<int>(n_heads);
-  a.block_size = static_cast<int>(block_size);
-  a.bs_shift = -1;
-  for (int s = 0; s < 31; ++s)
-    if ((1LL << s) == block_size) a.bs_shift = s;
-  a.num_blocks = static_cast<int>(num_blocks);
-  a.chunk_tokens = plan.chunk_tokens;
-  a.max_splits = plan.max_splits;
-  a.scale_log2 = sm_scale * kLog2e;
-  if (plan.max_splits > 1) {
-    a.ws_out = static_cast<float*>(workspace);
-    a.ws_lse = a.ws_out + static_cast<size_t>(batch) * n_heads * plan.max_splits * kDL;
-  }
-
-  const size_t smem = 2 * static_cast<size_t>(kTileBytes);
+  const int n_hb = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
   static bool attr_set = false;
+  const size_t smem = kPrefixOff + (kMaxBatchMla + 1) * 4;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (e != hipSuccess) return static_cast<int>(e);
     attr_set = true;
   }
-  dim3 grid(static_cast<unsigned>(plan.max_splits), static_cast<unsigned>(head_blocks),
-            static_cast<unsigned>(batch));
-  const bool timed = profile_begin(stream);
-  mla_decode_kernel<<<grid, kMlaThreads, smem, stream>>>(a);
-  if (timed) profile_end(stream);
-  int rc = static_cast<int>(hipGetLastError());
-  if (rc != 0 || plan.max_splits <= 1) return rc;
-  mla_merge_kernel<<<dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(batch)), 128, 0, stream>>>(
-      a.ws_out, a.ws_lse, static_cast<char*>(out), lse, addr.seq_lens, static_cast<int>(n_heads),
-      plan.chunk_tokens, plan.max_splits);
-  return static_cast<int>(hipGetLastError());
-}
+  for (int64_t b0 = 0; b0 < batch; b0 += kMaxBatchMla) {
+    const int64_t nb = batch - b0 < kMaxBatchMla ? batch - b0 : kMaxBatchMla;
+    MlaArgs a = {};
+    a.q_nope = static_cast<const char*>(q_nope) + b0 * n_heads * kDL * 2;
+    a.q_pe = static_cast<const char*>(q_pe) + b0 * n_heads * kDR * 2;
+    a.k_cache = static_cast<const char*>(k_cache);
+    a.out = static_cast<char*>(out) + b0 * n_heads * kDL * 2;
+    a.lse = lse == nullptr ? nullptr : lse + b0 * n_heads;
+    a.block_table = addr.block_table + b0 * addr.table_stride;
+    a.seq_lens = addr.seq_lens + b0;
+    a.table_stride = addr.table_stride;
+    a.batch = static_cast<int>(nb);
+    a.n_heads = static_cast<int>(n_heads);
+    a.n_hb = n_hb;
+    a.n_teams = mla_teams(n_hb);
+    a.block_size = static_cast<int>(block_size);
+    a.bs_shift = -1;
+    for (int s = 0; s < 31; ++s)
+      if ((1LL << s) == block_size) a.bs_shift = s;
+    a.num_blocks = static_cast<int>(num_blocks);
+    a.scale_log2 = sm_scale * kLog2e;
+    const size_t prefix_bytes = ((static_cast<size_t>(nb) + 1) * 4 + 255) / 256 * 256;
+    a.ws_prefix = static_cast<int*>(workspace);
+    a.ws_out = reinterpret_cast<float*>(static_cast<char*>(workspace) + prefix_bytes);
+    a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * n_heads * kDL;
 
-size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) {
-  if (max_seq_len <= 0) return 0;
-  const SplitPlan plan = plan_mla_splits(batch, (n_heads + kHeadsPerWg - 1) / kHeadsPerWg, max_seq_len);
-  return split_workspace_bytes(batch, n_heads, plan.max_splits);
+    const bool timed = profile_begin(stream);
+    mla_decode_kernel<<<dim3(static_cast<unsigned>(a.n_teams * n_hb)), kMlaThreads, smem, stream>>>(a);
+    if (timed) profile_end(stream);
+    int rc = static_cast<int>(hipGetLastError());
+    if (rc != 0) return rc;
+    mla_merge_kernel<<<dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb)), 128, 0, stream>>>(a);
+    rc = static_cast<int>(hipGetLastError());
+    if (rc != 0) return rc;
+  }
+  return XLLM_MI355_OK;
 }
 
 }  // namespace xllm_mi355
