@@ -244,18 +244,27 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       float m_own = kNegBig;
       if (wave_ok) {
         // ---- S^T block of this wavefront: tokens tblk*32 + (8*(r/4) + 4g + r%4), head c32
-        f32x16 s, s2;  // two accumulation chains over alternate k-steps
+        f32x16 s;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = s2[r] = 0.0f;
+        for (int r = 0; r < 16; ++r) s[r] = 0.0f;
         const char* ka = kb + (tblk * 32 + c32) * kLdsRow + g * 16;
+        __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the Q.K reads only
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ks += 2) {
           const u32x4 x0 = *reinterpret_cast<const u32x4*>(ka + ks * 32);
           const u32x4 x1 = *reinterpret_cast<const u32x4*>(ka + ks * 32 + 32);
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x0), q[ks], s, 0, 0, 0);
-          s2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x1), q[ks + 1], s2, 0, 0, 0);
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x1), q[ks + 1], s, 0, 0, 0);
         }
-        s += s2;
+        // pipeline the LDS operand reads four MFMAs ahead of their use
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < kKSteps - 4; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_barrier(0);
         const int tok_base = (tile0 + tile) * kTile + tblk * 32 + g * 4;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -322,10 +331,11 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
                          (tblk * 256 + ((lane >> 4) & 1) * 16 + (p16 & 3) * 4) * 2;
         const char* vb_own = vb + tblk * 32 * kLdsRow;
         const char* vb_other = vb + (tblk ^ 1) * 32 * kLdsRow;
+        __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the P.V reads only
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
+        for (int ks = 0; ks < 4; ++ks) {  // own token block: k-steps 0, 1; the partner's: 2, 3
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks) {  // own token block: k-steps 0, 1; the partner's: 2, 3
+          for (int mb = 0; mb < 8; ++mb) {  // 8 independent accumulators per k-step
             const char* rows = (ks < 2 ? vb_own : vb_other) + (16 * (ks & 1)) * kLdsRow + mb * 64;
             const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows));
             const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows + 8 * kLdsRow));
@@ -334,6 +344,15 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
                 __builtin_bit_cast(bf16x8, v), ks < 2 ? pb_own[ks & 1] : pb_other[ks & 1], o[mb], 0, 0, 0);
           }
         }
+        // pipeline the transposing reads (two per MFMA) four MFMAs ahead of their use
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+        for (int i = 0; i < 28; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
