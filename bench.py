@@ -31,6 +31,8 @@ def parse_args():
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="run only the plain stream_read / stream_copy kernels over 1 GiB (counter calibration)")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="measured HBM bytes per launch by workload (written from rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -95,6 +97,40 @@ def cpu_baseline(inp, k_cache, v_cache, k_scale, v_scale, n_sample, budget_s=6.0
     }
 
 
+def stream_rate(lib, capi, torch, dev, nbytes, copy=False, reps=10):
+    """GB/s of the library's plain read (or copy) kernel over nbytes: what this GPU sustains for a
+    working set of that size, measured with the same event hook as the decode kernel."""
+    import ctypes
+    nbytes = max(16, nbytes // 16 * 16)
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty(nbytes, dtype=torch.uint8, device=dev) if copy else None
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def run():
+        if copy:
+            return lib.xllm_mi355_stream_copy(dst.data_ptr(), src.data_ptr(), nbytes, stream)
+        return lib.xllm_mi355_stream_read(src.data_ptr(), nbytes, None, stream)
+
+    for _ in range(3):
+        capi.check(run(), "stream kernel")
+    torch.cuda.synchronize()
+    capi.check(lib.xllm_mi355_profile_enable(reps), "profile_enable")
+    for _ in range(reps):
+        run()
+    ms = (ctypes.c_float * reps)()
+    n = lib.xllm_mi355_profile_collect(ms, reps)
+    avg = sum(ms[i] for i in range(n)) / max(n, 1)
+    return (2 if copy else 1) * nbytes / (avg * 1e-3) / 1e9, avg
+
+
+def calibrate(lib, capi, torch, dev):
+    nbytes = 1 << 30
+    read_gbs, read_ms = stream_rate(lib, capi, torch, dev, nbytes)
+    copy_gbs, copy_ms = stream_rate(lib, capi, torch, dev, nbytes, copy=True)
+    return {"bytes": nbytes, "stream_read_gbs": read_gbs, "stream_read_ms": read_ms,
+            "stream_copy_gbs_read_plus_write": copy_gbs, "stream_copy_ms": copy_ms}
+
+
 def main():
     args = parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -112,6 +148,9 @@ def main():
         sys.exit(1)
     lib = capi.lib()  # raises if the HIP library has not been built
     dev = torch.device("cuda:0")
+    if args.calibrate:
+        print(json.dumps(calibrate(lib, capi, torch, dev)))
+        return
     cfg = workloads.CONFIGS[args.workload]
     fp8 = cfg.cache_dtype == "fp8"
 
@@ -223,6 +262,9 @@ def main():
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                     "kernel": "gqa_decode_kernel", "kernel_ms": kernel_ms, "algorithmic_bytes": nbytes}
+
+    # the same number of bytes through the plain read kernel: the rate this GPU sustains at this size
+    roofline["stream_read_gbs_same_bytes"], _ = stream_rate(lib, capi, torch, dev, nbytes)
 
     result = {
         "metric": "paged-decode tokens/s + achieved HBM GB/s (% of 8 TB/s) on 1 MI355X",

@@ -216,6 +216,16 @@ int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr,
 int xllm_mi355_profile_enable(int capacity);
 int xllm_mi355_profile_collect(float* ms_out, int max_n);
 
+/*
+ * Plain streaming kernels of known size, the yardstick for the decode kernels.  No
+ * counterpart in the reference (its own micro-benchmarks time block copies with device
+ * events, tests/core/kernels/dcu/block_copy_test.cpp:195-215).  stream_read reads `bytes`
+ * once (sink: 4 writable bytes or null); stream_copy reads and writes them once.  Pointers
+ * 16-byte aligned, bytes a multiple of 16.  Both take part in the timing hook above.
+ */
+int xllm_mi355_stream_read(const void* src, size_t bytes, void* sink, void* stream);
+int xllm_mi355_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,72 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/xllm_mi355.h declares."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from xllm_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "xllm_mi355.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(xllm_mi355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_table_agree():
+    declared = _declared_functions()
+    assert declared, "no declarations found in the header"
+    assert sorted(capi.SIGNATURES) == declared
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    if not os.path.exists(capi.LIB_PATH):
+        pytest.fail(f"{capi.LIB_PATH} is missing: run `python -m xllm_amd.build`")
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    for name in _declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+
+
+def test_host_only_entry_points_without_a_gpu():
+    lib = capi.lib()
+    assert re.fullmatch(rb"\d+\.\d+\.\d+", lib.xllm_mi355_version())
+    assert lib.xllm_mi355_error_string(0) == b"ok"
+    for code in (-1, -2, -3, -4, -5):
+        assert len(lib.xllm_mi355_error_string(code)) > 4
+    # argument validation happens before any HIP call
+    assert lib.xllm_mi355_reshape_and_cache(None, None, None, None, None, None, None, 4, 8, 128, 16, 10,
+                                            1024, 1024, capi.BF16, capi.BF16, None) == -1
+    assert lib.xllm_mi355_paged_decode_gqa(None, None, None, None, None, None, 0, None, None, None, 4, 32,
+                                           8, 128, 16, 10, 4096, 4096, 100, 0.1, None, 0, capi.BF16,
+                                           capi.BF16, None) == -1
+    assert lib.xllm_mi355_paged_decode_mla(None, None, None, None, None, None, 0, None, 4, 128, 512, 64, 64,
+                                           10, 100, 0.1, None, 0, capi.BF16, None) == -1
+    assert lib.xllm_mi355_lse_merge(None, None, None, None, 2, 1, 1, 8, capi.FP32, None) == -1
+    assert lib.xllm_mi355_reshape_and_cache(None, None, None, None, None, None, None, 0, 8, 128, 16, 10,
+                                            1024, 1024, capi.BF16, capi.BF16, None) == 0  # no tokens: no-op
+    # workspace sizes are positive and grow with the head dim
+    a = lib.xllm_mi355_paged_decode_workspace_bytes(64, 32, 128, 4096)
+    b = lib.xllm_mi355_paged_decode_workspace_bytes(64, 32, 256, 4096)
+    c = lib.xllm_mi355_paged_decode_workspace_bytes(64, 128, 512, 16384)
+    assert 0 < a < b and c > 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(capi.XllmMi355Error):
+        capi.lib()
+
+
+def test_python_ops_refuse_cpu_tensors():
+    import torch
+    from xllm_amd import ops
+    k = torch.zeros(2, 1, 64, dtype=torch.bfloat16)
+    cache = torch.zeros(1, 16, 1, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=k, value=k, k_cache=cache, v_cache=cache,
+                                                            slot_mapping=torch.zeros(2, dtype=torch.int32)))

@@ -1,0 +1,87 @@
+"""The C++ host side (torch::Tensor interface registered as torch.ops.xllm_ops.*) gives the same
+bytes as the direct C-ABI calls and follows the reference's schema."""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close_to_reference, fill_caches_cpu
+from xllm_amd import ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def xops(device):
+    from xllm_amd import torch_ops
+    return torch_ops.load()
+
+
+def test_reshape_and_decode_through_the_dispatcher(device, xops):
+    cfg = workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=6, len_lo=40, len_hi=1500)
+    inp = workloads.make_inputs(cfg, 17)
+    lay = inp.layout
+    shape = (lay.num_blocks, cfg.block_size, cfg.n_kv_heads, cfg.head_dim)
+    kg = torch.zeros(shape, dtype=torch.bfloat16, device=device)
+    vg = torch.zeros_like(kg)
+    for k, v, slots in ((inp.k_ctx, inp.v_ctx, lay.ctx_slots), (inp.k_new, inp.v_new, lay.new_slots)):
+        ret = xops.reshape_paged_cache(slots.to(device), k.to(device), v.to(device), kg, vg)
+        assert ret.data_ptr() == kg.data_ptr()          # the reference's op returns key_cache
+    kc, vc = fill_caches_cpu(inp)
+    assert torch.equal(kg.cpu(), kc) and torch.equal(vg.cpu(), vc)
+    q = inp.q.to(device)
+    out = torch.empty_like(q)
+    out, lse = xops.batch_decode(q, kg, vg, out, lay.block_table.to(device), lay.seq_lens.to(device), None, None,
+                                 int(lay.seq_lens.max()), cfg.scale)
+    ref = oracle.aten_paged_decode(inp.q, kc, vc, lay.block_table, lay.seq_lens, cfg.scale)
+    assert_close_to_reference(out, ref, "dispatcher batch_decode")
+    direct = torch.empty_like(q)
+    ops.batch_decode(q, kg, direct, lay.block_table.to(device), lay.seq_lens.to(device), v_cache=vg,
+                     scale=cfg.scale, max_seq_len=int(lay.seq_lens.max()))
+    assert torch.equal(out, direct)
+    assert tuple(lse.shape) == (cfg.batch, cfg.n_q_heads, 1) and lse.dtype == torch.float32
+
+
+def test_fp8_mla_and_merge_through_the_dispatcher(device, xops):
+    g = torch.Generator().manual_seed(3)
+    T, P, bs, H, D = 48, 4, 16, 2, 128
+    key = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    val = torch.randn(T, H, D, generator=g).to(torch.bfloat16)
+    slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+    ks, vs = oracle.kv_head_scales(key), oracle.kv_head_scales(val)
+    kg = torch.zeros(P, bs, H, D, dtype=torch.float8_e4m3fn, device=device)
+    vg = torch.zeros_like(kg)
+    xops.quant_to_paged_cache(slots.to(device), key.to(device), val.to(device), kg, vg, ks.to(device), vs.to(device))
+    kc = torch.zeros(P, bs, H, D, dtype=torch.uint8)
+    vc = torch.zeros_like(kc)
+    oracle.reshape_and_cache(key, val, kc, vc, slots, ks, vs)
+    assert torch.equal(kg.view(torch.uint8).cpu(), kc) and torch.equal(vg.view(torch.uint8).cpu(), vc)
+
+    cfg = workloads.DecodeConfig("mla", 2, 16, 1, 576, 64, 30, 300, mla=True, v_dim=512, sigma=0.5,
+                                 sm_scale=1 / math.sqrt(192.0))
+    inp = workloads.make_inputs(cfg, 5)
+    lay = inp.layout
+    cache = torch.zeros(lay.num_blocks, 64, 1, 576, dtype=torch.bfloat16, device=device)
+    for k, slots in ((inp.k_ctx, lay.ctx_slots), (inp.k_new, lay.new_slots)):
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=k.to(device), k_cache=cache,
+                                                            slot_mapping=slots.to(device)))
+    q = inp.q.to(device)
+    out, lse = xops.mla_dense_decode(q[:, :, :512].contiguous().view(2, 1, 16, 512),
+                                     q[:, :, 512:].contiguous().view(2, 1, 16, 64), cache,
+                                     lay.seq_lens.to(device), lay.block_table.to(device), 512, cfg.scale)
+    ref = oracle.aten_paged_decode(inp.q, cache.cpu(), None, lay.block_table, lay.seq_lens, cfg.scale, dv=512)
+    assert_close_to_reference(out.view(2, 16, 512), ref, "dispatcher mla")
+    # DcpAttentionMergeTest.WeightsPartialOutputsByNaturalLogLse on the device
+    po = torch.tensor([2.0, 4.0, 6.0, 8.0], device=device).reshape(2, 1, 1, 1, 2)
+    pl = torch.tensor([math.log(2.0), math.log(6.0)], device=device).reshape(2, 1, 1, 1)
+    mo, ml = xops.merge_dcp_attention_shards(po, pl)
+    assert torch.allclose(mo.cpu(), torch.tensor([5.0, 7.0]).reshape(1, 1, 1, 2))
+    assert torch.allclose(ml.cpu(), torch.tensor([math.log(8.0)]).reshape(1, 1, 1))
+    po = torch.tensor([0.0, 0.0, 3.0, 9.0], device=device).reshape(2, 1, 1, 1, 2)
+    pl = torch.tensor([-math.inf, math.log(4.0)], device=device).reshape(2, 1, 1, 1)
+    mo, ml = xops.merge_dcp_attention_shards(po, pl)
+    assert torch.equal(mo.cpu(), torch.tensor([3.0, 9.0]).reshape(1, 1, 1, 2))
+    mo, ml = xops.merge_dcp_attention_shards(torch.ones(2, 1, 1, 2, 3, device=device),
+                                             torch.full((2, 1, 2, 1), -math.inf, device=device))
+    assert torch.equal(mo.cpu(), torch.zeros(1, 1, 2, 3)) and torch.isneginf(ml).all()

@@ -37,6 +37,8 @@ SIGNATURES = {
     "xllm_mi355_build_block_table": (_i32, [_p, _p, _p, _p, _i64, _p, _i64, _i64, _p]),
     "xllm_mi355_profile_enable": (_i32, [_i32]),
     "xllm_mi355_profile_collect": (_i32, [_p, _i32]),
+    "xllm_mi355_stream_read": (_i32, [_p, _sz, _p, _p]),
+    "xllm_mi355_stream_copy": (_i32, [_p, _p, _sz, _p]),
 }
 
 _lib = None

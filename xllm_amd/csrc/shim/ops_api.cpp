@@ -1,0 +1,302 @@
+// See ops_api.h.  Host code only: it unpacks torch::Tensor arguments, checks what the
+// reference checks, fetches the current HIP stream from PyTorch and calls the C ABI.
+#include "ops_api.h"
+
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <mutex>
+#include <unordered_map>
+
+#include "../../../include/xllm_mi355.h"
+
+namespace {
+
+int dtype_code(const torch::Tensor& t) {
+  switch (t.scalar_type()) {
+    case torch::kBFloat16: return XLLM_MI355_BF16;
+    case torch::kFloat16: return XLLM_MI355_FP16;
+    case torch::kFloat32: return XLLM_MI355_FP32;
+    case torch::kFloat8_e4m3fn:
+    case torch::kUInt8: return XLLM_MI355_FP8_E4M3;
+    default: TORCH_CHECK(false, "unsupported dtype ", t.scalar_type()); return -1;
+  }
+}
+
+void* current_stream(const torch::Tensor& t) {
+  return c10::hip::getCurrentHIPStream(t.device().index()).stream();
+}
+
+void check_rc(int rc, const char* what) {
+  TORCH_CHECK(rc == 0, what, " failed with code ", rc, ": ", xllm_mi355_error_string(rc));
+}
+
+const void* ptr_or_null(const std::optional<torch::Tensor>& t) {
+  return t.has_value() && t->defined() ? t->data_ptr() : nullptr;
+}
+
+void reshape_impl(xllm::kernel::ReshapePagedCacheParams& p, bool quantized) {
+  TORCH_CHECK(!p.direction, "CACHE2CONTEXT is not part of the decode path");
+  const torch::Tensor& key = p.key;
+  TORCH_CHECK(key.is_cuda() && key.dim() == 3, "key must be a device tensor [T, Hkv, D]");
+  TORCH_CHECK(key.stride(-1) == 1 && key.stride(-2) == key.size(-1), "key: last two dims must be contiguous");
+  const bool has_v = p.value.has_value() && p.value->defined();
+  TORCH_CHECK(has_v == (p.v_cache.has_value() && p.v_cache->defined()), "value and v_cache go together");
+  if (has_v) {
+    TORCH_CHECK(p.value->stride(-1) == 1 && p.value->stride(-2) == p.value->size(-1) &&
+                    p.value->sizes() == key.sizes(),
+                "value: last two dims must be contiguous and the shape must match key");
+  }
+  TORCH_CHECK(p.k_cache.dim() == 4 && p.k_cache.is_contiguous(), "k_cache must be contiguous [P, bs, Hkv, D]");
+  TORCH_CHECK(p.slot_mapping.scalar_type() == torch::kInt32 && p.slot_mapping.is_contiguous() &&
+                  p.slot_mapping.numel() == key.size(0),
+              "slot_mapping must be contiguous int32 [T]");
+  if (quantized) {
+    TORCH_CHECK(p.k_cache_scale.has_value(), "k_cache_scale is required for quant_to_paged_cache");
+  } else {
+    TORCH_CHECK(p.k_cache.scalar_type() == key.scalar_type(), "key and k_cache must have the same dtype");
+  }
+  const int rc = xllm_mi355_reshape_and_cache(
+      key.data_ptr(), has_v ? p.value->data_ptr() : nullptr, p.k_cache.data_ptr(),
+      has_v ? p.v_cache->data_ptr() : nullptr, p.slot_mapping.data_ptr<int32_t>(),
+      quantized ? static_cast<const float*>(ptr_or_null(p.k_cache_scale)) : nullptr,
+      quantized ? static_cast<const float*>(ptr_or_null(p.v_cache_scale)) : nullptr, key.size(0), key.size(1),
+      key.size(2), p.k_cache.size(1), p.k_cache.size(0), key.stride(0), has_v ? p.value->stride(0) : 0,
+      dtype_code(key), dtype_code(p.k_cache), current_stream(key));
+  check_rc(rc, "xllm_mi355_reshape_and_cache");
+}
+
+}  // namespace
+
+namespace xllm::kernel {
+
+void reshape_paged_cache(ReshapePagedCacheParams& params) { reshape_impl(params, false); }
+void quant_to_paged_cache(ReshapePagedCacheParams& params) { reshape_impl(params, true); }
+
+namespace mi355 {
+
+torch::Tensor decode_workspace(const torch::Device& device, size_t nbytes) {
+  static std::mutex mu;
+  static std::unordered_map<int, torch::Tensor> ws;
+  std::lock_guard<std::mutex> lock(mu);
+  torch::Tensor& t = ws[device.index()];
+  if (!t.defined() || static_cast<size_t>(t.numel()) < nbytes)
+    t = torch::empty({static_cast<int64_t>(std::max<size_t>(nbytes, 1 << 20))},
+                     torch::TensorOptions().dtype(torch::kUInt8).device(device));
+  return t;
+}
+
+void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torch::Tensor& output,
+                  const torch::Tensor& block_table, const torch::Tensor& seq_lens,
+                  const std::optional<torch::Tensor>& v_cache, std::optional<torch::Tensor>& output_lse,
+                  const std::optional<torch::Tensor>& k_cache_quant_scale,
+                  const std::optional<torch::Tensor>& v_cache_quant_scale, int64_t max_seq_len,
+                  float scale, bool return_lse) {
+  TORCH_CHECK(v_cache.has_value() && v_cache->defined(), "GQA decode needs v_cache");
+  TORCH_CHECK(query.is_cuda() && query.dim() == 3, "query must be a device tensor [B, Hq, D]");
+  TORCH_CHECK(query.stride(-1) == 1 && query.stride(-2) == query.size(-1), "query: last two dims contiguous");
+  TORCH_CHECK(output.stride(-1) == 1 && output.stride(-2) == output.size(-1), "output: last two dims contiguous");
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && v_cache->is_contiguous(), "caches contiguous");
+  TORCH_CHECK(block_table.scalar_type() == torch::kInt32 && block_table.dim() == 2 && block_table.stride(1) == 1 &&
+                  block_table.size(0) == query.size(0),
+              "block_table must be int32 [B, W]");
+  TORCH_CHECK(seq_lens.scalar_type() == torch::kInt32 && seq_lens.is_contiguous() && seq_lens.numel() == query.size(0),
+              "seq_lens must be contiguous int32 [B]");
+  const int64_t B = query.size(0), Hq = query.size(1), D = query.size(2);
+  if (return_lse && !(output_lse.has_value() && output_lse->defined()))
+    output_lse = torch::empty({B, Hq, 1}, query.options().dtype(torch::kFloat32));
+  float* lse = nullptr;
+  if (output_lse.has_value() && output_lse->defined()) {
+    TORCH_CHECK(output_lse->scalar_type() == torch::kFloat32 && output_lse->is_contiguous() &&
+                    output_lse->numel() == B * Hq,
+                "output_lse must be contiguous fp32 [B, Hq, 1]");
+    lse = output_lse->data_ptr<float>();
+  }
+  if (max_seq_len <= 0) max_seq_len = block_table.size(1) * k_cache.size(1);
+  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len);
+  torch::Tensor ws = decode_workspace(query.device(), nbytes);
+  const int rc = xllm_mi355_paged_decode_gqa(
+      query.data_ptr(), k_cache.data_ptr(), v_cache->data_ptr(), output.data_ptr(), lse,
+      block_table.data_ptr<int32_t>(), block_table.stride(0), seq_lens.data_ptr<int32_t>(),
+      static_cast<const float*>(ptr_or_null(k_cache_quant_scale)),
+      static_cast<const float*>(ptr_or_null(v_cache_quant_scale)), B, Hq, k_cache.size(2), D, k_cache.size(1),
+      k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, scale, ws.data_ptr(),
+      static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
+  check_rc(rc, "xllm_mi355_paged_decode_gqa");
+}
+
+void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache,
+                      torch::Tensor paged_kv_indptr, torch::Tensor paged_kv_indices,
+                      torch::Tensor paged_kv_last_page_len, double sm_scale, torch::Tensor output,
+                      std::optional<torch::Tensor>& output_lse, int64_t max_seq_len) {
+  TORCH_CHECK(query.is_cuda() && query.dim() == 3, "query must be a device tensor [B, Hq, D]");
+  const int64_t B = query.size(0), Hq = query.size(1), D = query.size(2);
+  for (const torch::Tensor* t : {&paged_kv_indptr, &paged_kv_indices, &paged_kv_last_page_len})
+    TORCH_CHECK(t->scalar_type() == torch::kInt32 && t->is_contiguous(), "CSR arrays must be contiguous int32");
+  TORCH_CHECK(paged_kv_indptr.numel() == B + 1 && paged_kv_last_page_len.numel() == B, "CSR sizes");
+  float* lse = output_lse.has_value() && output_lse->defined() ? output_lse->data_ptr<float>() : nullptr;
+  if (max_seq_len <= 0) max_seq_len = std::max<int64_t>(1, paged_kv_indices.numel()) * k_cache.size(1);
+  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len);
+  torch::Tensor ws = decode_workspace(query.device(), nbytes);
+  const int rc = xllm_mi355_paged_decode_gqa_csr(
+      query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), lse,
+      paged_kv_indptr.data_ptr<int32_t>(), paged_kv_indices.data_ptr<int32_t>(),
+      paged_kv_last_page_len.data_ptr<int32_t>(), nullptr, nullptr, B, Hq, k_cache.size(2), D, k_cache.size(1),
+      k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, static_cast<float>(sm_scale),
+      ws.data_ptr(), static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache),
+      current_stream(query));
+  check_rc(rc, "xllm_mi355_paged_decode_gqa_csr");
+}
+
+namespace flash_mla {
+
+torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {
+  // the checks of check_dense_decode_inputs, xllm/core/kernels/dcu/flash_mla_adapter.cpp:55-100
+  TORCH_CHECK(p.q_nope.defined() && p.q_pe.defined() && p.k_cache.defined() && p.seqlens_k.defined() &&
+                  p.block_table.defined(),
+              "flash_mla: all tensors must be defined");
+  TORCH_CHECK(p.q_nope.dim() == 4 && p.q_pe.dim() == 4, "flash_mla: q_nope / q_pe must be 4D [B,S_q,H_q,D]");
+  TORCH_CHECK(p.k_cache.dim() == 4 && p.k_cache.size(2) == 1,
+              "flash_mla: k_cache must be 4D [blocks,page,1,D] with a single KV head");
+  TORCH_CHECK(p.k_cache.size(3) == p.q_nope.size(3) + p.q_pe.size(3),
+              "flash_mla: k_cache last dim must equal q_nope.dim + q_pe.dim");
+  TORCH_CHECK(p.head_size_v > 0, "flash_mla: head_size_v must be positive");
+  TORCH_CHECK(p.softmax_scale > 0.0F, "flash_mla: softmax_scale must be set by the MLA attention layer");
+  TORCH_CHECK(p.q_nope.size(1) == 1, "decode path: one query token per sequence");
+  TORCH_CHECK(p.head_size_v == p.q_nope.size(3), "V is the latent part of the cache");
+  torch::Tensor seqlens = p.seqlens_k.scalar_type() == torch::kInt32 ? p.seqlens_k : p.seqlens_k.to(torch::kInt32);
+  torch::Tensor table = p.block_table.scalar_type() == torch::kInt32 ? p.block_table : p.block_table.to(torch::kInt32);
+  torch::Tensor q_nope = p.q_nope.contiguous(), q_pe = p.q_pe.contiguous();
+  const int64_t B = q_nope.size(0), H = q_nope.size(2);
+  torch::Tensor out = torch::empty({B, 1, H, p.head_size_v}, q_nope.options());
+  float* lse = nullptr;
+  if (lse_out != nullptr) {
+    *lse_out = torch::empty({B, H, 1}, q_nope.options().dtype(torch::kFloat32));
+    lse = lse_out->data_ptr<float>();
+  }
+  const int64_t max_seq_len = table.size(1) * p.k_cache.size(1);
+  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, H, p.head_size_v, max_seq_len);
+  torch::Tensor ws = decode_workspace(q_nope.device(), nbytes);
+  const int rc = xllm_mi355_paged_decode_mla(
+      q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), lse, table.data_ptr<int32_t>(),
+      table.stride(0), seqlens.data_ptr<int32_t>(), B, H, q_nope.size(3), q_pe.size(3), p.k_cache.size(1),
+      p.k_cache.size(0), max_seq_len, p.softmax_scale, ws.data_ptr(), static_cast<size_t>(ws.numel()),
+      dtype_code(q_nope), current_stream(q_nope));
+  check_rc(rc, "xllm_mi355_paged_decode_mla");
+  return out;
+}
+
+}  // namespace flash_mla
+}  // namespace mi355
+}  // namespace xllm::kernel
+
+namespace xllm::layer {
+
+DcpAttentionResult merge_dcp_attention_shards(const torch::Tensor& partial_outputs,
+                                              const torch::Tensor& partial_lse) {
+  TORCH_CHECK(partial_outputs.dim() == 5, "partial outputs must have shape [dcp, batch, query, heads, value]");
+  TORCH_CHECK(partial_lse.dim() == 4, "partial LSE must have shape [dcp, batch, heads, query]");
+  const int64_t S = partial_outputs.size(0), B = partial_outputs.size(1), Q = partial_outputs.size(2),
+                H = partial_outputs.size(3), Dv = partial_outputs.size(4);
+  TORCH_CHECK(partial_lse.size(0) == S && partial_lse.size(1) == B && partial_lse.size(3) == Q &&
+                  partial_lse.size(2) == H,
+              "partial outputs and LSE disagree");
+  TORCH_CHECK(Q == 1, "decode path: one query token per sequence");
+  torch::Tensor po = partial_outputs.contiguous();
+  torch::Tensor pl = partial_lse.to(torch::kFloat32).contiguous();
+  torch::Tensor out = torch::empty({B, Q, H, Dv}, po.options());
+  torch::Tensor lse = torch::empty({B, H, Q}, pl.options());
+  const int rc = xllm_mi355_lse_merge(po.data_ptr(), pl.data_ptr<float>(), out.data_ptr(), lse.data_ptr<float>(), S, B,
+                                      H, Dv, dtype_code(po), current_stream(po));
+  check_rc(rc, "xllm_mi355_lse_merge");
+  return {out, lse};
+}
+
+}  // namespace xllm::layer
+
+// torch dispatcher registration: the schema of xllm_ops::reshape_paged_cache is the reference's
+// (xllm/core/kernels/cuda/cuda_ops_library.cpp:286-287); the decode ops are this build's.
+namespace {
+
+torch::Tensor op_reshape_paged_cache(torch::Tensor slot_mapping, torch::Tensor keys, torch::Tensor values,
+                                     torch::Tensor key_cache, torch::Tensor value_cache) {
+  xllm::kernel::ReshapePagedCacheParams p;
+  p.key = keys;
+  p.value = values;
+  p.k_cache = key_cache;
+  p.v_cache = value_cache;
+  p.slot_mapping = slot_mapping;
+  xllm::kernel::reshape_paged_cache(p);
+  return key_cache;
+}
+
+torch::Tensor op_quant_to_paged_cache(torch::Tensor slot_mapping, torch::Tensor keys, torch::Tensor values,
+                                      torch::Tensor key_cache, torch::Tensor value_cache,
+                                      torch::Tensor k_scale, torch::Tensor v_scale) {
+  xllm::kernel::ReshapePagedCacheParams p;
+  p.key = keys;
+  p.value = values;
+  p.k_cache = key_cache;
+  p.v_cache = value_cache;
+  p.slot_mapping = slot_mapping;
+  p.k_cache_scale = k_scale;
+  p.v_cache_scale = v_scale;
+  xllm::kernel::quant_to_paged_cache(p);
+  return key_cache;
+}
+
+std::tuple<torch::Tensor, torch::Tensor> op_batch_decode(torch::Tensor query, torch::Tensor k_cache,
+                                                         torch::Tensor v_cache, torch::Tensor output,
+                                                         torch::Tensor block_table, torch::Tensor seq_lens,
+                                                         std::optional<torch::Tensor> k_scale,
+                                                         std::optional<torch::Tensor> v_scale, int64_t max_seq_len,
+                                                         double scale) {
+  std::optional<torch::Tensor> lse;
+  xllm::kernel::mi355::batch_decode(query, k_cache, output, block_table, seq_lens, v_cache, lse, k_scale, v_scale,
+                                    max_seq_len, static_cast<float>(scale), /*return_lse=*/true);
+  return {output, lse.value()};
+}
+
+std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nope, torch::Tensor q_pe,
+                                                             torch::Tensor k_cache, torch::Tensor seqlens_k,
+                                                             torch::Tensor block_table, int64_t head_size_v,
+                                                             double softmax_scale) {
+  xllm::kernel::mi355::flash_mla::DenseDecodeParams p;
+  p.q_nope = q_nope;
+  p.q_pe = q_pe;
+  p.k_cache = k_cache;
+  p.seqlens_k = seqlens_k;
+  p.block_table = block_table;
+  p.head_size_v = head_size_v;
+  p.softmax_scale = static_cast<float>(softmax_scale);
+  torch::Tensor lse;
+  torch::Tensor out = xllm::kernel::mi355::flash_mla::dense_decode(p, &lse);
+  return {out, lse};
+}
+
+std::tuple<torch::Tensor, torch::Tensor> op_merge(torch::Tensor partial_outputs, torch::Tensor partial_lse) {
+  auto r = xllm::layer::merge_dcp_attention_shards(partial_outputs, partial_lse);
+  return {r.output, r.lse};
+}
+
+}  // namespace
+
+TORCH_LIBRARY(xllm_ops, m) {
+  m.def("reshape_paged_cache(Tensor slot_mapping, Tensor keys, Tensor values, Tensor(a!) key_cache, "
+        "Tensor(b!) value_cache) -> Tensor");
+  m.def("quant_to_paged_cache(Tensor slot_mapping, Tensor keys, Tensor values, Tensor(a!) key_cache, "
+        "Tensor(b!) value_cache, Tensor k_scale, Tensor v_scale) -> Tensor");
+  m.def("batch_decode(Tensor query, Tensor k_cache, Tensor v_cache, Tensor(a!) output, Tensor block_table, "
+        "Tensor seq_lens, Tensor? k_scale, Tensor? v_scale, int max_seq_len, float scale) -> (Tensor, Tensor)");
+  m.def("mla_dense_decode(Tensor q_nope, Tensor q_pe, Tensor k_cache, Tensor seqlens_k, Tensor block_table, "
+        "int head_size_v, float softmax_scale) -> (Tensor, Tensor)");
+  m.def("merge_dcp_attention_shards(Tensor partial_outputs, Tensor partial_lse) -> (Tensor, Tensor)");
+}
+
+TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
+  m.impl("reshape_paged_cache", &op_reshape_paged_cache);
+  m.impl("quant_to_paged_cache", &op_quant_to_paged_cache);
+  m.impl("batch_decode", &op_batch_decode);
+  m.impl("mla_dense_decode", &op_mla_dense_decode);
+  m.impl("merge_dcp_attention_shards", &op_merge);
+}

@@ -1,0 +1,84 @@
+// C++ host side of the MI355X paged-KV decode path: the reference's kernel op interface
+// (torch::Tensor structs and free functions) over the C ABI of include/xllm_mi355.h.
+//
+// Names, argument order and meaning follow the reference (paths relative to the xLLM tree):
+//   xllm::kernel::ReshapePagedCacheParams, reshape_paged_cache, quant_to_paged_cache
+//       xllm/core/kernels/param.h:126-161, ops_api.h:31, ops_api.cpp:248-310
+//   xllm::kernel::mi355::batch_decode (block table)   xllm/core/kernels/mlu/mlu_ops_api.h:127,
+//                                                     xllm/core/kernels/npu/npu_ops_api.h:46
+//   xllm::kernel::mi355::batch_decode_csr             xllm/core/kernels/cuda/cuda_ops_api.h:128-144
+//   xllm::kernel::mi355::flash_mla::dense_decode      xllm/core/kernels/dcu/flash_mla_adapter.h:40-53
+//   xllm::layer::merge_dcp_attention_shards           xllm/core/layers/mlu/dcp_attention_merge.h:28-34
+// A violated precondition throws c10::Error (TORCH_CHECK) where the reference CHECK-aborts.
+#pragma once
+
+#include <torch/torch.h>
+
+#include <optional>
+#include <tuple>
+
+namespace xllm::kernel {
+
+struct ReshapePagedCacheParams {
+  torch::Tensor key;                       // [T, Hkv, D], last two dims contiguous
+  std::optional<torch::Tensor> value;      // same shape; given iff v_cache is
+  torch::Tensor k_cache;                   // [P, bs, Hkv, D] contiguous
+  std::optional<torch::Tensor> v_cache;
+  torch::Tensor slot_mapping;              // [T] int32
+  bool direction = false;                  // CACHE2CONTEXT is not part of this path
+  std::optional<torch::Tensor> k_cache_scale;  // [Hkv] fp32 for the fp8 cache
+  std::optional<torch::Tensor> v_cache_scale;
+};
+
+void reshape_paged_cache(ReshapePagedCacheParams& params);
+void quant_to_paged_cache(ReshapePagedCacheParams& params);
+
+namespace mi355 {
+
+// Per-device split workspace, grown on demand; same lifetime as the reference's
+// FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41).
+torch::Tensor decode_workspace(const torch::Device& device, size_t nbytes);
+
+void batch_decode(const torch::Tensor& query,        // [B, Hq, D]
+                  const torch::Tensor& k_cache,      // [P, bs, Hkv, D]
+                  torch::Tensor& output,             // [B, Hq, D]
+                  const torch::Tensor& block_table,  // [B, W] int32
+                  const torch::Tensor& seq_lens,     // [B] int32
+                  const std::optional<torch::Tensor>& v_cache,
+                  std::optional<torch::Tensor>& output_lse,  // [B, Hq, 1] fp32, natural log
+                  const std::optional<torch::Tensor>& k_cache_quant_scale,
+                  const std::optional<torch::Tensor>& v_cache_quant_scale,
+                  int64_t max_seq_len, float scale, bool return_lse);
+
+void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache,
+                      torch::Tensor paged_kv_indptr, torch::Tensor paged_kv_indices,
+                      torch::Tensor paged_kv_last_page_len, double sm_scale, torch::Tensor output,
+                      std::optional<torch::Tensor>& output_lse, int64_t max_seq_len);
+
+namespace flash_mla {
+struct DenseDecodeParams {
+  torch::Tensor q_nope;       // [B, S_q, H, kv_lora_rank]
+  torch::Tensor q_pe;         // [B, S_q, H, rope]
+  torch::Tensor k_cache;      // [P, bs, 1, kv_lora_rank + rope]
+  torch::Tensor seqlens_k;    // [B] int32
+  torch::Tensor block_table;  // [B, W] int32
+  int64_t head_size_v = 0;
+  float softmax_scale = -1.0F;
+  bool is_causal = false;
+};
+// Returns [B, S_q, H, head_size_v]; lse (if not null) receives [B, H, 1] fp32.
+torch::Tensor dense_decode(DenseDecodeParams& params, torch::Tensor* lse = nullptr);
+}  // namespace flash_mla
+
+}  // namespace mi355
+}  // namespace xllm::kernel
+
+namespace xllm::layer {
+struct DcpAttentionResult {
+  torch::Tensor output;
+  torch::Tensor lse;
+};
+// partial_outputs [S, B, Q=1, H, Dv], partial_lse [S, B, H, Q=1] (natural log).
+DcpAttentionResult merge_dcp_attention_shards(const torch::Tensor& partial_outputs,
+                                              const torch::Tensor& partial_lse);
+}  // namespace xllm::layer

@@ -1,0 +1,29 @@
+"""Loads the C++ host side (libxllm_mi355_torch.so): the reference's torch::Tensor op interface
+over the C ABI, registered with the torch dispatcher as torch.ops.xllm_ops.*.
+
+  torch.ops.xllm_ops.reshape_paged_cache(slot_mapping, keys, values, key_cache, value_cache)
+      -- the reference's schema (xllm/core/kernels/cuda/cuda_ops_library.cpp:286-287)
+  torch.ops.xllm_ops.quant_to_paged_cache(..., k_scale, v_scale)
+  torch.ops.xllm_ops.batch_decode(query, k_cache, v_cache, output, block_table, seq_lens,
+                                  k_scale, v_scale, max_seq_len, scale) -> (output, lse)
+  torch.ops.xllm_ops.mla_dense_decode(q_nope, q_pe, k_cache, seqlens_k, block_table,
+                                      head_size_v, softmax_scale) -> (out, lse)
+  torch.ops.xllm_ops.merge_dcp_attention_shards(partial_outputs, partial_lse) -> (out, lse)
+"""
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SHIM_PATH = os.path.join(_HERE, "libxllm_mi355_torch.so")
+_loaded = False
+
+
+def load():
+    global _loaded
+    if not _loaded:
+        if not os.path.exists(SHIM_PATH):
+            raise RuntimeError(f"{SHIM_PATH} is missing: build it with `python -m xllm_amd.build`")
+        torch.ops.load_library(SHIM_PATH)
+        _loaded = True
+    return torch.ops.xllm_ops
