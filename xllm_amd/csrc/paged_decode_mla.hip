@@ -50,6 +50,7 @@ constexpr int kTileBytes = kTile * kLdsRow;  // 74752
 constexpr int kMlaThreads = 256;
 constexpr int kHeadsPerWg = 64;
 constexpr int kKSteps = kDK / 16;   // 36 k-steps of the 32x32x16 MFMA
+constexpr float kSlack = 8.0f;    // log2 head room of the running maximum
 constexpr int kMaxBatchMla = 1024;  // sequences per launch (their tile prefix lives in LDS)
 // LDS map: two tiles | P^T exchange [4 waves][8 regs][64 lanes] | row-max exchange [4][32] | prefix
 constexpr int kXchPOff = 2 * kTileBytes;
@@ -105,6 +106,11 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 __device__ __forceinline__ void dma16(const void* gptr, u32 lds_addr) {
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
+}
+// Same with a wave-uniform 64-bit row base in SGPRs plus a 32-bit per-lane byte offset.
+__device__ __forceinline__ void dma16_row(uint64_t row_base, u32 lane_off, u32 lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
+               : "memory");
 }
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
@@ -213,13 +219,15 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       int page = pages[pg];
       page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
       const int slot = page * a.block_size + off;
-      const u32 lds_tile = lds_base + buf * kTileBytes + wave * 16 * kLdsRow;
+      const u32 lds_tile =
+          __builtin_amdgcn_readfirstlane(lds_base + buf * kTileBytes + wave * 16 * kLdsRow);
+      const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
+      const u32 lane_off = lane * 16;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int64_t s_i = __builtin_amdgcn_readlane(slot, i);
-        const char* row = a.k_cache + s_i * kRowBytes + lane * 16;
-        dma16(row, lds_tile + i * kLdsRow);
-        if (lane < kDR * 2 / 16) dma16(row + kDL * 2, lds_tile + i * kLdsRow + kDL * 2);
+        const uint64_t row = cache + static_cast<uint64_t>(static_cast<u32>(__builtin_amdgcn_readlane(slot, i))) * kRowBytes;
+        dma16_row(row, lane_off, lds_tile + i * kLdsRow);
+        if (lane < kDR * 2 / 16) dma16_row(row + kDL * 2, lane_off, lds_tile + i * kLdsRow + kDL * 2);
       }
     };
 
@@ -240,8 +248,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       __syncthreads();  // (A) this tile has landed in LDS; every wavefront is past the previous P.V
       if (tile + 1 < run_tiles) issue_tile(tile + 1, buf ^ 1);  // in flight during the whole tile
 
-      float p_own[16];
-      float m_own = kNegBig;
+      u32 pk_own[8];
+      float m_own = kNegBig, sum_own = 0.0f;
       if (wave_ok) {
         // ---- S^T block of this wavefront: tokens tblk*32 + (8*(r/4) + 4g + r%4), head c32
         f32x16 s;
@@ -266,20 +274,23 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         __builtin_amdgcn_sched_barrier(0);
         const int tok_base = (tile0 + tile) * kTile + tblk * 32 + g * 4;
+        if ((tile0 + tile + 1) * kTile > L) {  // only the last tile of a context is ragged
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (tok_base + 8 * (r >> 2) + (r & 3) >= L) s[r] = -INFINITY;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) m_own = fmaxf(m_own, s[r]);
+        m_own = half_swap_max(m_own) * a.scale_log2;  // row maximum of this token block (scale > 0)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float v = tok_base + 8 * (r >> 2) + (r & 3) < L ? s[r] * a.scale_log2 : -INFINITY;
-          p_own[r] = v;
-          m_own = fmaxf(m_own, v);
+          s[r] = fast_exp2(__builtin_fmaf(s[r], a.scale_log2, -m_own));
+          sum_own += s[r];
         }
-        m_own = half_swap_max(m_own);  // row maximum of this token block
-        u32 pk[8];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) p_own[r] = fast_exp2(p_own[r] - m_own);
+        for (int i = 0; i < 8; ++i) pk_own[i] = BF16::pack(s[2 * i], s[2 * i + 1]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) pk[i] = BF16::pack(p_own[2 * i], p_own[2 * i + 1]);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) xch_p[(wave * 8 + i) * 64 + lane] = pk[i];
+        for (int i = 0; i < 8; ++i) xch_p[(wave * 8 + i) * 64 + lane] = pk_own[i];
         if (g == 0) xch_m[wave * 32 + c32] = m_own;
       }
       __syncthreads();  // (B) P^T blocks and maxima of this tile are visible
@@ -292,18 +303,16 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       }
 
       if (wave_ok) {
-        const float m_new = fmaxf(m, fmaxf(m_own, m_other));
+        // The reference maximum m only follows the tile maxima when they exceed it by more than
+        // kSlack (log2 units): probabilities then stay below 2^kSlack, well inside bf16 / fp32
+        // range, and the 128 accumulators are rescaled a handful of times per context.
+        const float m_tile = fmaxf(m_own, m_other);
+        const float m_new = m_tile > m + kSlack ? m_tile : m;
         const float alpha = fast_exp2(m - m_new);
         const float f_own = fast_exp2(m_own - m_new);
         const float f_other = fast_exp2(m_other - m_new);
         m = m_new;
-        float sum = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          p_own[r] *= f_own;
-          sum += p_own[r];
-        }
-        l = l * alpha + sum;  // this wavefront's share of the normaliser (its own token block)
+        l = l * alpha + sum_own * f_own;  // this wavefront's share of the normaliser
         if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
           for (int i = 0; i < 8; ++i) o[i] *= alpha;
@@ -316,7 +325,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
           u32x4 mine, theirs;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            mine[i] = BF16::pack(p_own[8 * kk + 2 * i], p_own[8 * kk + 2 * i + 1]);
+            const u32 w = pk_own[4 * kk + i];
+            mine[i] = BF16::pack(BF16::lo(w) * f_own, BF16::hi(w) * f_own);
             const u32 t = theirs_raw[4 * kk + i];
             theirs[i] = BF16::pack(BF16::lo(t) * f_other, BF16::hi(t) * f_other);
           }
