@@ -206,7 +206,9 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     // rope bytes.  Each wavefront moves 16 rows; lane i < 16 first looks up the slot of row i.
     // The loads are issued from inline assembly so that the compiler's own wait insertion
     // does not see them: they are awaited explicitly (dma_wait) one tile later.
-    auto issue_tile = [&](int tile, int buf) {
+    // slot (page * bs + row) of row wave*16 + (lane & 15) of a tile; looked up one tile before
+    // the tile is issued, so the table load's latency never sits in front of the tile loads
+    auto lookup_page = [&](int tile, int& row_off) {
       const int tok = min((tile0 + tile) * kTile + wave * 16 + (lane & 15), L - 1);
       int pg, off;
       if (a.bs_shift >= 0) {
@@ -216,7 +218,11 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         pg = tok / a.block_size;
         off = tok - pg * a.block_size;
       }
-      int page = pages[pg];
+      row_off = off;
+      return pages[pg];  // raw: nothing may depend on the loaded value before the tile is issued
+    };
+    auto issue_tile = [&](int page, int off, int buf) {
+      asm volatile("" : "+v"(page));  // the wait for the table load belongs here, one tile later
       page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
       const int slot = page * a.block_size + off;
       const u32 lds_tile =
@@ -239,14 +245,20 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
       q[ks] = __builtin_bit_cast(bf16x8, x);
     }
     __syncthreads();  // the previous run no longer reads the tiles or the exchange buffers
-    issue_tile(0, 0);
+    int off_next = 0;
+    int page_next = lookup_page(0, off_next);
+    issue_tile(page_next, off_next, 0);
+    page_next = lookup_page(1, off_next);
 
     for (int tile = 0; tile < run_tiles; ++tile) {
       const int buf = tile & 1;
       const char* kb = smem + buf * kTileBytes;
       dma_wait();
       __syncthreads();  // (A) this tile has landed in LDS; every wavefront is past the previous P.V
-      if (tile + 1 < run_tiles) issue_tile(tile + 1, buf ^ 1);  // in flight during the whole tile
+      if (tile + 1 < run_tiles) {
+        issue_tile(page_next, off_next, buf ^ 1);  // in flight during the whole tile
+        page_next = lookup_page(tile + 2, off_next);
+      }
 
       u32 pk_own[8];
       float m_own = kNegBig, sum_own = 0.0f;
