@@ -159,9 +159,8 @@ def test_csr_form_matches_block_table_form_and_csr_oracle(device):
     assert torch.equal(tg.cpu(), tc) and torch.equal(lg.cpu(), lc) and torch.equal(lc, lay.seq_lens)
 
 
-def test_fp8_kv_cache_decode(device):
-    cfg = workloads.scaled(workloads.CONFIGS["fp8_kv"], batch=4, len_lo=300, len_hi=3000)
-    inp = workloads.make_inputs(cfg, 4242)
+def _check_fp8(cfg, seed, device):
+    inp = workloads.make_inputs(cfg, seed)
     lay = inp.layout
     kg, vg, ks, vs = fill_caches_gpu(inp, device, cache_dtype=torch.float8_e4m3fn)
     kc, vc = fill_caches_cpu(inp, torch.float8_e4m3fn, ks.cpu(), vs.cpu())
@@ -169,7 +168,30 @@ def test_fp8_kv_cache_decode(device):
     out, lse = _decode_gpu(inp, kg, vg, device, ks, vs)
     ref = oracle.aten_paged_decode(inp.q, kc.view(torch.float8_e4m3fn), vc.view(torch.float8_e4m3fn),
                                    lay.block_table, lay.seq_lens, cfg.scale, ks.cpu(), vs.cpu())
-    assert_close_to_reference(out, ref, "fp8")
+    assert_close_to_reference(out, ref, "fp8 " + cfg.name)
+
+
+def test_fp8_kv_cache_decode(device):
+    cfg = workloads.scaled(workloads.CONFIGS["fp8_kv"], batch=4, len_lo=300, len_hi=3000)
+    _check_fp8(cfg, 4242, device)
+
+
+def test_whole_contexts_in_one_workgroup_every_group_size(device):
+    # Few short sequences: every context is a single item, so one workgroup sees it whole and
+    # writes the caller's output itself (no partials, no merge), with most wavefronts idle.
+    # Then contexts of a few items each, enough of them that workgroups own several whole ones.
+    for Hq, Hkv in ((4, 4), (8, 4), (12, 4), (16, 4), (20, 4), (28, 4), (32, 4)):
+        for batch, hi in ((5, 64), (160, 400)):
+            cfg = workloads.DecodeConfig(f"whole_h{Hq}_{Hkv}_b{batch}", batch, Hq, Hkv, 128, 32, 1, hi)
+            _check_config(cfg, 300 + Hq + batch, device)
+    for Hq, Hkv in ((8, 4), (28, 4), (32, 4)):
+        cfg = workloads.DecodeConfig(f"whole_fp8_h{Hq}_{Hkv}", 5, Hq, Hkv, 128, 32, 1, 64, cache_dtype="fp8")
+        _check_fp8(cfg, 400 + Hq, device)
+        cfg = workloads.DecodeConfig(f"whole_fp8_h{Hq}_{Hkv}_b96", 96, Hq, Hkv, 128, 32, 1, 500, cache_dtype="fp8")
+        _check_fp8(cfg, 500 + Hq, device)
+    for D, Hq, Hkv in ((64, 16, 2), (256, 8, 1)):
+        cfg = workloads.DecodeConfig(f"whole_d{D}", 5, Hq, Hkv, D, 16, 1, 64)
+        _check_config(cfg, 600 + D, device)
 
 
 def test_empty_sequence_and_argument_errors(device):

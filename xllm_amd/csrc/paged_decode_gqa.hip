@@ -45,7 +45,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kItem = 64;      // tokens per schedulable item
 constexpr int kSub = 2048;     // tokens whose slot ids are staged in LDS at a time
-constexpr int kMaxBatch = 8192;  // sequences per launch (their item prefix lives in LDS)
+constexpr int kMaxBatch = 2048;  // sequences per launch (their item prefix lives in LDS)
 
 struct GqaArgs {
   const char* q;
@@ -129,6 +129,40 @@ __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* 
   }
   if (lo < hi && hi == a.batch) prefix[a.batch] = excl;  // the last non-empty slice holds the total
   __syncthreads();
+}
+
+// End-of-run fold: NP per-lane-row states (D accumulators, maximum, sum; stride D + 2 floats) of
+// one head lie in LDS; thread tid produces dimension tid of the head's normalised output and
+// the head's LSE.  A whole context goes to the caller's output, a piece of one to the partial
+// slot pidx.  Every thread computes (threads past D repeat a dimension) and the stores hang off
+// flat, un-nested conditions: a divergent branch nested at the tail of another one has been
+// seen to leave the register allocator's copies for the code after it under the narrowed
+// execution mask.
+template <typename QT, int D, int NP>
+__device__ __forceinline__ void fold_states(const GqaArgs& a, const float* part, int tid, bool head_on,
+                                            bool complete, int b, int hq, int64_t pidx, float out_scale) {
+  static_assert(D <= kThreads, "one thread per output dimension");
+  constexpr int PSTRIDE = D + 2;
+  const int d = tid & (D - 1);
+  float mx = kNegBig;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) mx = fmaxf(mx, part[p * PSTRIDE + D]);
+  float lsum = 0.0f, o = 0.0f;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const float* pp = part + p * PSTRIDE;
+    const float w = fast_exp2(pp[D] - mx);
+    lsum += w * pp[D + 1];
+    o += w * pp[d];
+  }
+  const float val = o / lsum * out_scale;
+  const float lse2 = mx + fast_log2(lsum);
+  const bool wr = head_on && tid < D;
+  const bool wl = head_on && tid == 0;
+  if (wr && complete) reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes)[hq * D + d] = QT::from_f32(val);
+  if (wr && !complete) a.ws_out[pidx * D + d] = val;
+  if (wl && complete && a.lse != nullptr) a.lse[b * a.n_q_heads + hq] = lse2 * kLn2;
+  if (wl && !complete) a.ws_lse[pidx] = lse2;
 }
 
 // QT: BF16 or FP16 (query, output and non-fp8 cache element).  FP8: cache holds e4m3fn.
@@ -426,30 +460,7 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
         }
       }
       __syncthreads();
-      if (h < nh) {
-        for (int d = tid; d < D; d += kThreads) {
-          float mx = kNegBig;
-#pragma unroll
-          for (int p = 0; p < NP; ++p) mx = fmaxf(mx, part[p * PSTRIDE + D]);
-          float lsum = 0.0f, o = 0.0f;
-#pragma unroll
-          for (int p = 0; p < NP; ++p) {
-            const float* pp = part + p * PSTRIDE;
-            const float w = fast_exp2(pp[D] - mx);
-            lsum += w * pp[D + 1];
-            o += w * pp[d];
-          }
-          const float val = o / lsum * out_scale;
-          const int hq = h0 + h;
-          if (complete) {
-            reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes)[hq * D + d] = QT::from_f32(val);
-            if (a.lse != nullptr && d == 0) a.lse[b * a.n_q_heads + hq] = (mx + fast_log2(lsum)) * kLn2;
-          } else {
-            a.ws_out[(pslot * G + h) * D + d] = val;
-            if (d == 0) a.ws_lse[pslot * G + h] = mx + fast_log2(lsum);
-          }
-        }
-      }
+      fold_states<QT, D, NP>(a, part, tid, h < nh, complete, b, h0 + h, pslot * G + h, out_scale);
     }
     first_run = false;
   }
@@ -554,7 +565,7 @@ int dispatch_group(GqaArgs& a, size_t wsb, hipStream_t s, bool plan_only, size_t
     case 1: return launch_gqa<QT, FP8, D, LPT, 1, U>(a, wsb, s, plan_only, need);
     case 2: return launch_gqa<QT, FP8, D, LPT, 2, U>(a, wsb, s, plan_only, need);
     case 4: return launch_gqa<QT, FP8, D, LPT, 4, U>(a, wsb, s, plan_only, need);
-    default: return launch_gqa<QT, FP8, D, LPT, 8, U>(a, wsb, s, plan_only, need);
+    default: return launch_gqa<QT, FP8, D, LPT, 8, (U > 2 ? U / 2 : U)>(a, wsb, s, plan_only, need);
   }
 }
 
