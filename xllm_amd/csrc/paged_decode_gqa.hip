@@ -466,6 +466,366 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Matrix-core variant for D = 128 with 16-bit pages.
+//
+// Every WAVEFRONT is an independent worker: it owns a contiguous range of the flat item list,
+// keeps its own softmax state, and never meets the other wavefronts of its workgroup after the
+// common item prefix sum, so there is no barrier anywhere in the streaming loop.
+//
+// Data path.  A stage is 16 tokens of one KV head: K rows (16 x 256 bytes) and V rows, 8 KB.
+// Stages travel from global memory straight into the wavefront's private LDS ring
+// (global_load_lds_dwordx4, 16 adjacent lanes per row so every instruction reads whole
+// contiguous rows), NS stages deep, NS - 1 in flight while one is consumed.  Within a row the
+// 16-byte chunks are XOR-swizzled (K by the row number, V by twice its low two bits) so that both
+// operand reads below touch every LDS bank once.
+//   S^T[tok, head] = K[tok, 128] . Q^T[128, head]   v_mfma_f32_16x16x32: A = K rows read from LDS
+//                                                   (16 bytes per lane), B = Q^T resident in registers
+//   O^T[dim, head] += V^T[dim, tok] . P^T[tok, head] v_mfma_f32_16x16x16: A = V^T through the
+//                                                   transposing LDS read, B = P^T taken from the
+//                                                   S^T accumulator registers as they are
+// Up to 16 query heads of the KV head ride in the MFMA columns (heads past the group are zero
+// columns), so a lane owns one head: its running maximum and sum are plain per-lane scalars.
+// The maximum only moves when a score exceeds it by more than kSlack (log2 units).
+//
+// Nothing in the loop waits on a register load from global memory: such a wait would also wait
+// for every younger stage in flight.  Page ids come through the same LDS path one item ahead,
+// sequence lengths through the scalar cache; only the Q rows at the start of a run are loaded
+// to registers.
+constexpr float kSlack = 8.0f;
+constexpr int kStageTokens = 16;
+constexpr int kStageBytes = 2 * kStageTokens * 256;  // K rows then V rows
+constexpr int kMfmaHeads = 16;                        // head columns of one MFMA
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+
+template <typename QT>
+struct Mfma;
+template <>
+struct Mfma<BF16> {
+  static __device__ __forceinline__ f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 k16(s16x4 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<FP16> {
+  static __device__ __forceinline__ f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 k16(s16x4 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+  }
+};
+
+// 16 (4) bytes per lane from global memory straight into LDS at lds_addr + lane * 16 (4);
+// lds_addr is wave-uniform and travels in M0.
+__device__ __forceinline__ void dma16(const void* gptr, u32 lds_addr) {
+  const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void dma4(const void* gptr, u32 lds_addr) {
+  const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gptr) : "memory");
+}
+// Wait until at most 8 * stages of the wavefront's vector memory operations are outstanding.
+__device__ __forceinline__ void wait_younger_stages(int stages) {
+  if (stages <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else if (stages == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (stages == 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+}
+// One dword through the scalar cache (wave-uniform address); does not touch the vector memory counter.
+__device__ __forceinline__ int sload32(const int32_t* p) {
+  const uint64_t x = reinterpret_cast<uint64_t>(p);
+  // (the builtin returns a signed int: each half goes through u32 so the low one is not sign-extended)
+  const u32 lo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(x)));
+  const u32 hi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(x >> 32)));
+  const uint64_t u = (static_cast<uint64_t>(hi) << 32) | lo;
+  int v;
+  asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(u) : "memory");
+  return v;
+}
+__device__ __forceinline__ void sequence_of_scalar(const GqaArgs& a, int b, const int32_t*& pages, int& L) {
+  if (a.indptr != nullptr) {
+    const int p0 = sload32(a.indptr + b);
+    const int np = sload32(a.indptr + b + 1) - p0;
+    pages = a.indices + p0;
+    L = np > 0 ? (np - 1) * a.block_size + sload32(a.last_page_len + b) : 0;
+  } else {
+    pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
+    L = sload32(a.seq_lens + b);
+  }
+}
+__device__ __forceinline__ float quad_rows_max(float x) {  // over lanes l, l ^ 16, l ^ 32, l ^ 48
+  auto t = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
+  x = fmaxf(as_f32(t[0]), as_f32(t[1]));
+  auto u = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
+  return fmaxf(as_f32(u[0]), as_f32(u[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float x) {
+  auto t = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
+  x = as_f32(t[0]) + as_f32(t[1]);
+  auto u = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
+  return as_f32(u[0]) + as_f32(u[1]);
+}
+
+// Position of an item in the flat list (sequence, head block, item), advanced one item at a time.
+struct ItemCursor {
+  int b, hbk, it, n_items;
+  int L;
+  const int32_t* pages;
+};
+
+template <int NS>
+struct MfmaLayout {
+  // LDS: ring [waves][NS][stage] | page ids [waves][2][64] | scan scratch [kThreads] | item prefix [batch + 1]
+  static constexpr int kRingBytes = kWaves * NS * kStageBytes;
+  static constexpr int kPageOff = kRingBytes;
+  static constexpr int kTmpOff = kPageOff + kWaves * 2 * kWave * 4;
+  static constexpr int kPrefixOff = kTmpOff + kThreads * 4;
+};
+
+template <typename QT, int NS>
+__global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
+  static_assert(NS >= 2 && NS <= 5, "page ids are fetched exactly one item (four stages) ahead");
+  using Lay = MfmaLayout<NS>;
+  constexpr int D = 128, RB = 256, G = kMfmaHeads;
+  constexpr int kStagesPerItem = kItem / kStageTokens;
+
+  extern __shared__ __align__(16) char smem[];
+  int* tmp = reinterpret_cast<int*>(smem + Lay::kTmpOff);
+  int* prefix = reinterpret_cast<int*>(smem + Lay::kPrefixOff);
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15;   // MFMA column (head) / row (token, dim); 16-byte chunk of a row in the loads
+  const int g = lane >> 4;     // MFMA k-group; token row of a load instruction
+  const int hb_per_kv = (a.group + G - 1) / G;
+  const int n_hb = a.n_kv_heads * hb_per_kv;
+
+  item_prefix(a, prefix, tmp);
+  const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
+  if (blockIdx.x == 0) {
+    for (int i = tid; i <= a.batch; i += kThreads) a.ws_prefix[i] = prefix[i];
+  }
+  if (total == 0) return;
+  // ---- from here on the wavefronts are independent: no workgroup barrier below this line
+  const int64_t n_workers = static_cast<int64_t>(gridDim.x) * kWaves;
+  const int64_t worker = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
+  const int64_t cur = range_start(worker, total, n_workers);
+  const int64_t end = range_start(worker + 1, total, n_workers);
+  if (cur >= end) return;
+  const int n_stages = static_cast<int>(end - cur) * kStagesPerItem;
+
+  const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
+  const u32 ring_lds = __builtin_amdgcn_readfirstlane(lds_base + wave * NS * kStageBytes);
+  const char* ring = smem + wave * NS * kStageBytes;
+  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + wave * 2 * kWave * 4);
+  const int* pagebuf = reinterpret_cast<const int*>(smem + Lay::kPageOff + wave * 2 * kWave * 4);
+
+  auto locate = [&](int64_t f, ItemCursor& cu) {
+    int lo = 0, hi = a.batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (static_cast<int64_t>(prefix[mid]) * n_hb <= f) lo = mid; else hi = mid;
+    }
+    cu.b = __builtin_amdgcn_readfirstlane(lo);
+    cu.n_items = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
+    const int64_t rem = f - static_cast<int64_t>(prefix[cu.b]) * n_hb;
+    cu.hbk = __builtin_amdgcn_readfirstlane(static_cast<int>(rem / cu.n_items));
+    cu.it = __builtin_amdgcn_readfirstlane(static_cast<int>(rem - static_cast<int64_t>(cu.hbk) * cu.n_items));
+    sequence_of_scalar(a, cu.b, cu.pages, cu.L);
+  };
+  auto advance = [&](ItemCursor& cu) {  // to the next item of the flat list
+    if (++cu.it < cu.n_items) return;
+    cu.it = 0;
+    if (++cu.hbk < n_hb) return;
+    cu.hbk = 0;
+    do {
+      ++cu.b;
+      cu.n_items = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
+    } while (cu.n_items == 0);  // the caller never advances past the last item of the batch
+    sequence_of_scalar(a, cu.b, cu.pages, cu.L);
+  };
+  // page ids of the item's 64 tokens (tail lanes repeat the last valid token) -> LDS, one per lane
+  auto issue_pages = [&](const ItemCursor& cu, int par) {
+    const int tok = min(cu.it * kItem + lane, cu.L - 1);
+    dma4(cu.pages + (tok >> a.bs_shift), page_lds + par * kWave * 4);
+  };
+
+  // ---- producer state: the item whose stages are being issued
+  ItemCursor pc;
+  locate(cur, pc);
+  ItemCursor pn = pc;       // the item after it (its page ids are in flight)
+  int p_par = 0;            // page-id buffer of the producer's item
+  int p_stage = 0;          // next stage to issue
+  int p_slot = 0;           // lane t: slot (page * bs + row) of token t of the producer's item
+  int64_t p_kv_off = 0;     // byte offset of the KV head within a token row
+  issue_pages(pc, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  auto begin_item = [&]() {  // the page ids of pc have landed in buffer p_par
+    const int tok = min(pc.it * kItem + lane, pc.L - 1);
+    int page = pagebuf[p_par * kWave + lane];
+    page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
+    p_slot = page * a.block_size + (tok & (a.block_size - 1));
+    p_kv_off = static_cast<int64_t>(pc.hbk / hb_per_kv) * RB;
+    if (p_stage + kStagesPerItem < n_stages) {
+      pn = pc;
+      advance(pn);
+      issue_pages(pn, p_par ^ 1);
+    }
+  };
+  auto issue_stage = [&]() {
+    const int j = p_stage % kStagesPerItem;
+    if (j == 0) {
+      if (p_stage != 0) {
+        pc = pn;
+        p_par ^= 1;
+      }
+      begin_item();
+    }
+    const u32 dst = ring_lds + (p_stage % NS) * kStageBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 4 * i + g;  // token row of this lane within the stage
+      const int slot = __builtin_amdgcn_ds_bpermute((j * kStageTokens + row) * 4, p_slot);
+      const int64_t goff = static_cast<int64_t>(slot) * a.row_bytes + p_kv_off;
+      dma16(a.k_cache + goff + ((c16 ^ row) * 16), dst + i * 1024);
+      dma16(a.v_cache + goff + ((c16 ^ ((row & 3) << 1)) * 16), dst + kStageTokens * RB + i * 1024);
+    }
+    ++p_stage;
+  };
+
+  for (int s = 0; s < NS - 1 && s < n_stages; ++s) issue_stage();
+
+  // ---- consumer state
+  ItemCursor cc;
+  locate(cur, cc);
+  bool first_run = true;
+  bool run_open = false;
+  bool complete = false;
+  int h0 = 0, nh = 0;
+  u32x4 q[4];
+  f32x4 o[8];
+  float m = kNegBig, l = 0.0f;
+  // per-lane constants of the operand reads
+  const int k_read = c16 * RB;                                   // + ((chunk ^ c16) * 16)
+  const int v_read = kStageTokens * RB + (4 * g + (c16 >> 2)) * RB + ((c16 & 3) >> 1) * 16 + (c16 & 1) * 8;
+  const int v_y = (c16 >> 2) << 5;                                // swizzle term of the lane's row
+
+  for (int s = 0; s < n_stages; ++s) {
+    wait_younger_stages(min(NS - 2, n_stages - 1 - s));
+    if (s + NS - 1 < n_stages) issue_stage();
+
+    const int j = s % kStagesPerItem;
+    if (j == 0) {
+      if (s != 0) advance(cc);
+      if (!run_open) {  // first item of a run: (sequence, head block) changes
+        const int kvh = cc.hbk / hb_per_kv;
+        h0 = kvh * a.group + (cc.hbk % hb_per_kv) * G;
+        nh = min(G, (kvh + 1) * a.group - h0);
+        const int items_left = static_cast<int>(min<int64_t>(cc.n_items - cc.it, (n_stages - s) / kStagesPerItem));
+        complete = cc.it == 0 && items_left == cc.n_items;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          u32x4 x = {0u, 0u, 0u, 0u};
+          if (c16 < nh)
+            x = ldg16(a.q + cc.b * a.q_stride_bytes + (static_cast<int64_t>(h0 + c16) * D + kk * 32 + g * 8) * 2);
+          q[kk] = x;
+        }
+        // The wait for these loads (it also drains the stages in flight) must stay on this path:
+        // left to the first use after the join it would run on every stage.
+        asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]));
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) o[mb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        m = kNegBig;
+        l = 0.0f;
+        run_open = true;
+      }
+    }
+
+    // ---- scores of the stage's 16 tokens: lane (head c16, tokens 4g .. 4g+3)
+    const char* st = ring + (s % NS) * kStageBytes;
+    f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const u32x4 kr = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ c16) * 16));
+      sc = Mfma<QT>::k32(kr, q[kk], sc);
+    }
+    const int tok0 = cc.it * kItem + j * kStageTokens + 4 * g;
+    float sv[4];
+    bool over = false;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      sv[r] = tok0 + r < cc.L ? sc[r] * a.scale_log2 : -INFINITY;
+      over |= sv[r] > m + kSlack;
+    }
+    if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+      const float mx = quad_rows_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+      if (mx > m + kSlack) {
+        const float alpha = fast_exp2(m - mx);
+        m = mx;
+        l *= alpha;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) o[mb] *= alpha;
+      }
+    }
+    float p[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      p[r] = fast_exp2(sv[r] - m);
+      l += p[r];
+    }
+    const u32x2 pb = {QT::pack(p[0], p[1]), QT::pack(p[2], p[3])};
+    // ---- O^T += V^T . P^T: lane c16 of a 16-lane group supplies the address of 4 dims of token
+    // row 4g + c16/4 and receives the 4 tokens of dim column 16 mb + c16
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) {
+      const s16x4 vt = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (lds_s16x4*)(st + v_read + (v_y ^ (mb << 5))));
+      o[mb] = Mfma<QT>::k16(vt, pb, o[mb]);
+    }
+
+    // ---- end of a run: last item of the context or of the worker's range
+    if (j == kStagesPerItem - 1 && (cc.it == cc.n_items - 1 || s == n_stages - 1)) {
+      const float lsum = quad_rows_sum(l);
+      const float inv = 1.0f / lsum;
+      const float lse2 = m + fast_log2(lsum);
+      const bool head_on = c16 < nh;
+      const int hq = h0 + c16;
+      const int64_t pidx = (worker * 2 + (first_run ? 0 : 1)) * G + c16;
+      if (head_on && complete) {
+        char* op = a.out + cc.b * a.out_stride_bytes + (static_cast<int64_t>(hq) * D + 4 * g) * 2;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+          const u32x2 w = {QT::pack(o[mb][0] * inv, o[mb][1] * inv), QT::pack(o[mb][2] * inv, o[mb][3] * inv)};
+          *reinterpret_cast<u32x2*>(op + mb * 32) = w;
+        }
+      }
+      if (head_on && !complete) {
+        float* wp = a.ws_out + pidx * D + 4 * g;
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+          const f32x4 w = {o[mb][0] * inv, o[mb][1] * inv, o[mb][2] * inv, o[mb][3] * inv};
+          *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
+        }
+      }
+      if (head_on && g == 0 && complete && a.lse != nullptr) a.lse[cc.b * a.n_q_heads + hq] = lse2 * kLn2;
+      if (head_on && g == 0 && !complete) a.ws_lse[pidx] = lse2;
+      first_run = false;
+      run_open = false;
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // Merge of the partials of contexts that span several workgroups; also writes the output
 // of empty sequences.  One workgroup per (query head, sequence).
 template <typename QT>
@@ -559,6 +919,46 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
   return static_cast<int>(hipGetLastError());
 }
 
+constexpr int kMfmaStages = 4;
+
+template <typename QT>
+int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
+  using Lay = MfmaLayout<kMfmaStages>;
+  constexpr int D = 128;
+  auto kern = gqa_mfma_kernel<QT, kMfmaStages>;
+  static const bool configured = [&] {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              Lay::kPrefixOff + (kMaxBatch + 1) * 4);
+    return true;
+  }();
+  (void)configured;
+  a.g_block = kMfmaHeads;
+  const int n_wg = device_cu_count();  // the ring fills a CU's LDS: one workgroup each
+  a.n_workgroups = n_wg * kWaves;      // independent workers = wavefronts
+  const size_t prefix_bytes = ((static_cast<size_t>(a.batch) + 1) * 4 + 255) / 256 * 256;
+  const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * (D + 1);
+  *need = prefix_bytes + part_floats * 4;
+  if (plan_only) return XLLM_MI355_OK;
+  if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
+  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_prefix) + prefix_bytes);
+  a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
+  const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 1) * 4;
+  const bool timed = profile_begin(stream);
+  kern<<<dim3(static_cast<unsigned>(n_wg)), kThreads, smem, stream>>>(a);
+  if (timed) profile_end(stream);
+  return static_cast<int>(hipGetLastError());
+}
+
+// Which kernel serves head_dim 128 with 16-bit pages and a power-of-two block size: the
+// matrix-core one ("mfma", default) or the dot-product one ("rows").
+bool use_mfma_kernel() {
+  static const bool v = [] {
+    const char* e = getenv("XLLM_MI355_GQA_KERNEL");  // tuning knob
+    return !(e != nullptr && e[0] == 'r');
+  }();
+  return v;
+}
+
 template <typename QT, bool FP8, int D, int LPT, int U>
 int dispatch_group(GqaArgs& a, size_t wsb, hipStream_t s, bool plan_only, size_t* need) {
   switch (a.g_block) {
@@ -580,6 +980,7 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
       default: return XLLM_MI355_ESHAPE;
     }
   } else {
+    if (head_dim == 128 && a.bs_shift >= 0 && use_mfma_kernel()) return launch_gqa_mfma<QT>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, false, 64, 8, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, false, 128, 16, 4>(a, wsb, s, plan_only, need);
