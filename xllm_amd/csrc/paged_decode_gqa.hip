@@ -91,7 +91,8 @@ __device__ __forceinline__ void sequence_of(const GqaArgs& a, int b, const int32
   }
 }
 
-__device__ __forceinline__ int items_of(int L) { return L > 0 ? (L + kItem - 1) / kItem : 0; }
+template <int ITEM>
+__device__ __forceinline__ int items_of(int L) { return L > 0 ? (L + ITEM - 1) / ITEM : 0; }
 
 // First flat item of workgroup w when `total` items are dealt to `n` workgroups.
 __device__ __forceinline__ int64_t range_start(int64_t w, int64_t total, int64_t n) { return w * total / n; }
@@ -105,6 +106,7 @@ __device__ __forceinline__ int workgroup_of(int64_t id, int64_t total, int64_t n
 
 // Exclusive prefix sum of the per-sequence item counts into prefix[0..batch] (LDS).
 // Every thread sums a contiguous slice, then adds the totals of the slices before it.
+template <int ITEM>
 __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* tmp) {
   const int tid = threadIdx.x;
   const int per = (a.batch + kThreads - 1) / kThreads;
@@ -114,7 +116,7 @@ __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* 
     const int32_t* pages;
     int L;
     sequence_of(a, b, pages, L);
-    local += items_of(L);
+    local += items_of<ITEM>(L);
   }
   tmp[tid] = local;
   __syncthreads();
@@ -125,7 +127,7 @@ __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* 
     int L;
     sequence_of(a, b, pages, L);
     prefix[b] = excl;
-    excl += items_of(L);
+    excl += items_of<ITEM>(L);
   }
   if (lo < hi && hi == a.batch) prefix[a.batch] = excl;  // the last non-empty slice holds the total
   __syncthreads();
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
   const int hb_per_kv = (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
 
-  item_prefix(a, prefix, tmp);
+  item_prefix<kItem>(a, prefix, tmp);
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
   if (blockIdx.x == 0) {
     for (int i = tid; i <= a.batch; i += kThreads) a.ws_prefix[i] = prefix[i];
@@ -490,8 +492,7 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
 //
 // Nothing in the loop waits on a register load from global memory: such a wait would also wait
 // for every younger stage in flight.  Page ids come through the same LDS path one item ahead,
-// sequence lengths through the scalar cache; only the Q rows at the start of a run are loaded
-// to registers.
+// the Q rows of a run just before its first stage, sequence lengths through the scalar cache.
 constexpr float kSlack = 8.0f;
 constexpr int kStageTokens = 16;
 constexpr int kStageBytes = 2 * kStageTokens * 256;  // K rows then V rows
@@ -532,6 +533,14 @@ __device__ __forceinline__ void dma16(const void* gptr, u32 lds_addr) {
 __device__ __forceinline__ void dma4(const void* gptr, u32 lds_addr) {
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gptr) : "memory");
+}
+// Same as dma16 with a wave-uniform 64-bit base in SGPRs plus a 32-bit per-lane byte offset.
+__device__ __forceinline__ void dma16_row(uint64_t base, u32 lane_off, u32 lds_addr) {
+  const u32 m0 = __builtin_amdgcn_readfirstlane(lds_addr);
+  const u32 lo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(base)));
+  const u32 hi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(base >> 32)));
+  const uint64_t sb = (static_cast<uint64_t>(hi) << 32) | lo;
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(lane_off), "s"(sb) : "memory");
 }
 // Wait until at most 8 * stages of the wavefront's vector memory operations are outstanding.
 __device__ __forceinline__ void wait_younger_stages(int stages) {
@@ -575,28 +584,29 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
   return as_f32(u[0]) + as_f32(u[1]);
 }
 
-// Position of an item in the flat list (sequence, head block, item), advanced one item at a time.
-struct ItemCursor {
-  int b, hbk, it, n_items;
+// Position of a stage in the flat list (sequence, head block, stage of 16 tokens).
+struct CtxCursor {
+  int b, hbk, st, n_st;
   int L;
   const int32_t* pages;
 };
 
 template <int NS>
 struct MfmaLayout {
-  // LDS: ring [waves][NS][stage] | page ids [waves][2][64] | scan scratch [kThreads] | item prefix [batch + 1]
+  // LDS: ring [waves][NS][stage] | Q rows [waves][16][256 B] | page-table chunks [waves][3][64] |
+  //      scan scratch [kThreads] | stage prefix [batch + 1]
   static constexpr int kRingBytes = kWaves * NS * kStageBytes;
-  static constexpr int kPageOff = kRingBytes;
-  static constexpr int kTmpOff = kPageOff + kWaves * 2 * kWave * 4;
+  static constexpr int kQOff = kRingBytes;
+  static constexpr int kPageOff = kQOff + kWaves * kMfmaHeads * 256;
+  static constexpr int kTmpOff = kPageOff + kWaves * 3 * kWave * 4;
   static constexpr int kPrefixOff = kTmpOff + kThreads * 4;
 };
 
 template <typename QT, int NS>
 __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
-  static_assert(NS >= 2 && NS <= 5, "page ids are fetched exactly one item (four stages) ahead");
+  static_assert(NS >= 2 && NS <= 4, "wait_younger_stages covers up to three stages in flight");
   using Lay = MfmaLayout<NS>;
-  constexpr int D = 128, RB = 256, G = kMfmaHeads;
-  constexpr int kStagesPerItem = kItem / kStageTokens;
+  constexpr int D = 128, RB = 256, G = kMfmaHeads, T = kStageTokens;
 
   extern __shared__ __align__(16) char smem[];
   int* tmp = reinterpret_cast<int*>(smem + Lay::kTmpOff);
@@ -609,7 +619,7 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   const int hb_per_kv = (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
 
-  item_prefix(a, prefix, tmp);
+  item_prefix<T>(a, prefix, tmp);
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
   if (blockIdx.x == 0) {
     for (int i = tid; i <= a.batch; i += kThreads) a.ws_prefix[i] = prefix[i];
@@ -621,134 +631,214 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   const int64_t cur = range_start(worker, total, n_workers);
   const int64_t end = range_start(worker + 1, total, n_workers);
   if (cur >= end) return;
-  const int n_stages = static_cast<int>(end - cur) * kStagesPerItem;
+  const int n_stages = static_cast<int>(end - cur);
 
   const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
   const u32 ring_lds = __builtin_amdgcn_readfirstlane(lds_base + wave * NS * kStageBytes);
   const char* ring = smem + wave * NS * kStageBytes;
-  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + wave * 2 * kWave * 4);
-  const int* pagebuf = reinterpret_cast<const int*>(smem + Lay::kPageOff + wave * 2 * kWave * 4);
+  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + wave * 3 * kWave * 4);
+  const char* pagebuf = smem + Lay::kPageOff + wave * 3 * kWave * 4;
+  const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + wave * G * RB);
+  const char* qbuf = smem + Lay::kQOff + wave * G * RB;
 
-  auto locate = [&](int64_t f, ItemCursor& cu) {
+  auto locate = [&](int64_t f, CtxCursor& cu) {
     int lo = 0, hi = a.batch;
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
       if (static_cast<int64_t>(prefix[mid]) * n_hb <= f) lo = mid; else hi = mid;
     }
     cu.b = __builtin_amdgcn_readfirstlane(lo);
-    cu.n_items = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
+    cu.n_st = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
     const int64_t rem = f - static_cast<int64_t>(prefix[cu.b]) * n_hb;
-    cu.hbk = __builtin_amdgcn_readfirstlane(static_cast<int>(rem / cu.n_items));
-    cu.it = __builtin_amdgcn_readfirstlane(static_cast<int>(rem - static_cast<int64_t>(cu.hbk) * cu.n_items));
+    cu.hbk = __builtin_amdgcn_readfirstlane(static_cast<int>(rem / cu.n_st));
+    cu.st = __builtin_amdgcn_readfirstlane(static_cast<int>(rem - static_cast<int64_t>(cu.hbk) * cu.n_st));
     sequence_of_scalar(a, cu.b, cu.pages, cu.L);
   };
-  auto advance = [&](ItemCursor& cu) {  // to the next item of the flat list
-    if (++cu.it < cu.n_items) return;
-    cu.it = 0;
+  auto next_context = [&](CtxCursor& cu) {  // the caller never steps past the last context of the batch
+    cu.st = 0;
     if (++cu.hbk < n_hb) return;
     cu.hbk = 0;
     do {
       ++cu.b;
-      cu.n_items = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
-    } while (cu.n_items == 0);  // the caller never advances past the last item of the batch
+      cu.n_st = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
+    } while (cu.n_st == 0);
     sequence_of_scalar(a, cu.b, cu.pages, cu.L);
   };
-  // page ids of the item's 64 tokens (tail lanes repeat the last valid token) -> LDS, one per lane
-  auto issue_pages = [&](const ItemCursor& cu, int par) {
-    const int tok = min(cu.it * kItem + lane, cu.L - 1);
-    dma4(cu.pages + (tok >> a.bs_shift), page_lds + par * kWave * 4);
+  // 64 entries of the context's page table, from page 64 ck on (the tail repeats the last page),
+  // into the chunk buffer at byte offset off
+  auto issue_chunk = [&](const CtxCursor& cu, int ck, u32 off) {
+    const int n_pages = (cu.L + a.block_size - 1) >> a.bs_shift;
+    dma4(cu.pages + min(ck * kWave + lane, n_pages - 1), page_lds + off);
   };
 
-  // ---- producer state: the item whose stages are being issued
-  ItemCursor pc;
+  // ---- producer: issues stage p of the worker's range; pc is the context of that stage
+  CtxCursor pc;
   locate(cur, pc);
-  ItemCursor pn = pc;       // the item after it (its page ids are in flight)
-  int p_par = 0;            // page-id buffer of the producer's item
-  int p_stage = 0;          // next stage to issue
-  int p_slot = 0;           // lane t: slot (page * bs + row) of token t of the producer's item
-  int64_t p_kv_off = 0;     // byte offset of the KV head within a token row
-  issue_pages(pc, 0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  CtxCursor pn = pc;                         // the context after pc (valid while has_c)
+  int p = 0;
+  u32 off_a = 0, off_b = kWave * 4, off_c = 2 * kWave * 4;  // chunk buffers: current, next of pc, first of pn
+  int ck_a = 0;
+  int t_b = 0, t_c = 0;                      // value of p when the buffer's load was issued
+  bool has_b = false, has_c = false;
+  int p_ctx_first = 0, p_prev_len = 0;
+  // byte offset of the lane's 16 bytes from the first row of a stage: row 4i + g, chunk swizzled
+  u32 lane_k[4], lane_v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * i + g;
+    lane_k[i] = static_cast<u32>(row * a.row_bytes) + ((c16 ^ row) * 16);
+    lane_v[i] = static_cast<u32>(row * a.row_bytes) + ((c16 ^ (g << 1)) * 16);
+  }
 
-  auto begin_item = [&]() {  // the page ids of pc have landed in buffer p_par
-    const int tok = min(pc.it * kItem + lane, pc.L - 1);
-    int page = pagebuf[p_par * kWave + lane];
-    page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
-    p_slot = page * a.block_size + (tok & (a.block_size - 1));
-    p_kv_off = static_cast<int64_t>(pc.hbk / hb_per_kv) * RB;
-    if (p_stage + kStagesPerItem < n_stages) {
+  // A chunk or Q load issued while p was t has landed once the consumer has waited for stage t,
+  // which it has done when p >= t + NS - 1; otherwise everything in flight is awaited (short
+  // contexts only).
+  auto ensure_landed = [&](bool issued, int t) {
+    if (!(issued && t + NS - 1 <= p)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+  auto begin_context = [&](bool first) {
+    if (first) {
+      ck_a = ((pc.st * T) >> a.bs_shift) >> 6;
+      issue_chunk(pc, ck_a, off_a);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+      const u32 t = off_a;
+      off_a = off_c;
+      off_c = t;
+      ck_a = 0;
+      ensure_landed(has_c, t_c);
+    }
+    has_b = has_c = false;
+    p_ctx_first = p;
+    if (pc.n_st - pc.st < n_stages - p) {  // the range goes on into another context
       pn = pc;
-      advance(pn);
-      issue_pages(pn, p_par ^ 1);
+      next_context(pn);
+      issue_chunk(pn, 0, off_c);
+      t_c = p;
+      has_c = true;
+    }
+    const int n_pages = (pc.L + a.block_size - 1) >> a.bs_shift;
+    if ((ck_a + 1) * kWave < n_pages) {
+      issue_chunk(pc, ck_a + 1, off_b);
+      t_b = p;
+      has_b = true;
+    }
+    if (first || p_prev_len >= NS) {
+      // Q rows of the context's heads travel ahead of its first stage, swizzled like K rows (rows
+      // past the group repeat the last head; the consumer zeroes them).  The single buffer is
+      // free: the consumer copied the previous context's rows to registers when it began that
+      // context, at least NS stages ago.  After a shorter context the consumer loads Q itself.
+      const int kvh = pc.hbk / hb_per_kv;
+      const int h0p = kvh * a.group + (pc.hbk % hb_per_kv) * G;
+      const int nhp = min(G, (kvh + 1) * a.group - h0p);
+      const char* qb = a.q + pc.b * a.q_stride_bytes;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = 4 * i + g;
+        dma16(qb + (static_cast<int64_t>(h0p + min(row, nhp - 1)) * D) * 2 + ((c16 ^ row) * 16), q_lds + i * 1024);
+      }
     }
   };
   auto issue_stage = [&]() {
-    const int j = p_stage % kStagesPerItem;
-    if (j == 0) {
-      if (p_stage != 0) {
-        pc = pn;
-        p_par ^= 1;
+    if (p == 0) {
+      begin_context(true);
+    } else if (pc.st == pc.n_st) {
+      p_prev_len = p - p_ctx_first;
+      pc = pn;
+      begin_context(false);
+    }
+    const int tok0 = pc.st * T;
+    const int pi = tok0 >> a.bs_shift;  // block_size >= 16: one page holds the whole stage
+    if ((pi >> 6) != ck_a) {
+      const u32 t = off_a;
+      off_a = off_b;
+      off_b = t;
+      ck_a = pi >> 6;
+      ensure_landed(has_b, t_b);
+      has_b = false;
+      const int n_pages = (pc.L + a.block_size - 1) >> a.bs_shift;
+      if ((ck_a + 1) * kWave < n_pages) {
+        issue_chunk(pc, ck_a + 1, off_b);
+        t_b = p;
+        has_b = true;
       }
-      begin_item();
     }
-    const u32 dst = ring_lds + (p_stage % NS) * kStageBytes;
+    int page = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(pagebuf + off_a + (pi & 63) * 4));
+    page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
+    const int slot0 = page * a.block_size + (tok0 & (a.block_size - 1));
+    const uint64_t row0 = static_cast<uint64_t>(slot0) * static_cast<uint64_t>(a.row_bytes) +
+                          static_cast<uint64_t>(pc.hbk / hb_per_kv) * RB;
+    const uint64_t kb = reinterpret_cast<uint64_t>(a.k_cache) + row0;
+    const uint64_t vb = reinterpret_cast<uint64_t>(a.v_cache) + row0;
+    const u32 dst = ring_lds + (p % NS) * kStageBytes;
+    const int lim = pc.L - tok0 - 1;  // last valid row of the stage
+    if (lim >= T - 1) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = 4 * i + g;  // token row of this lane within the stage
-      const int slot = __builtin_amdgcn_ds_bpermute((j * kStageTokens + row) * 4, p_slot);
-      const int64_t goff = static_cast<int64_t>(slot) * a.row_bytes + p_kv_off;
-      dma16(a.k_cache + goff + ((c16 ^ row) * 16), dst + i * 1024);
-      dma16(a.v_cache + goff + ((c16 ^ ((row & 3) << 1)) * 16), dst + kStageTokens * RB + i * 1024);
+      for (int i = 0; i < 4; ++i) {
+        dma16_row(kb, lane_k[i], dst + i * 1024);
+        dma16_row(vb, lane_v[i], dst + T * RB + i * 1024);
+      }
+    } else {  // ragged end of a context: rows past it repeat the last valid row
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = 4 * i + g;
+        const u32 ro = static_cast<u32>(min(row, lim) * a.row_bytes);
+        dma16_row(kb, ro + ((c16 ^ row) * 16), dst + i * 1024);
+        dma16_row(vb, ro + ((c16 ^ (g << 1)) * 16), dst + T * RB + i * 1024);
+      }
     }
-    ++p_stage;
+    ++p;
+    ++pc.st;
   };
 
   for (int s = 0; s < NS - 1 && s < n_stages; ++s) issue_stage();
 
-  // ---- consumer state
-  ItemCursor cc;
+  // ---- consumer
+  CtxCursor cc;
   locate(cur, cc);
   bool first_run = true;
-  bool run_open = false;
   bool complete = false;
   int h0 = 0, nh = 0;
+  int c_ctx_first = 0, c_prev_len = 0;
   u32x4 q[4];
   f32x4 o[8];
   float m = kNegBig, l = 0.0f;
   // per-lane constants of the operand reads
   const int k_read = c16 * RB;                                   // + ((chunk ^ c16) * 16)
-  const int v_read = kStageTokens * RB + (4 * g + (c16 >> 2)) * RB + ((c16 & 3) >> 1) * 16 + (c16 & 1) * 8;
+  const int v_read = T * RB + (4 * g + (c16 >> 2)) * RB + ((c16 & 3) >> 1) * 16 + (c16 & 1) * 8;
   const int v_y = (c16 >> 2) << 5;                                // swizzle term of the lane's row
 
   for (int s = 0; s < n_stages; ++s) {
     wait_younger_stages(min(NS - 2, n_stages - 1 - s));
     if (s + NS - 1 < n_stages) issue_stage();
 
-    const int j = s % kStagesPerItem;
-    if (j == 0) {
-      if (s != 0) advance(cc);
-      if (!run_open) {  // first item of a run: (sequence, head block) changes
-        const int kvh = cc.hbk / hb_per_kv;
-        h0 = kvh * a.group + (cc.hbk % hb_per_kv) * G;
-        nh = min(G, (kvh + 1) * a.group - h0);
-        const int items_left = static_cast<int>(min<int64_t>(cc.n_items - cc.it, (n_stages - s) / kStagesPerItem));
-        complete = cc.it == 0 && items_left == cc.n_items;
+    if (s == 0 || cc.st == 0) {  // first stage of a run: the (sequence, head block) changes
+      const int kvh = cc.hbk / hb_per_kv;
+      h0 = kvh * a.group + (cc.hbk % hb_per_kv) * G;
+      nh = min(G, (kvh + 1) * a.group - h0);
+      complete = cc.st == 0 && cc.n_st <= n_stages - s;
+      if (s == 0 || c_prev_len >= NS) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          u32x4 x = {0u, 0u, 0u, 0u};
-          if (c16 < nh)
-            x = ldg16(a.q + cc.b * a.q_stride_bytes + (static_cast<int64_t>(h0 + c16) * D + kk * 32 + g * 8) * 2);
-          q[kk] = x;
-        }
+        for (int kk = 0; kk < 4; ++kk)  // the rows landed before this stage's tiles did
+          q[kk] = *reinterpret_cast<const u32x4*>(qbuf + k_read + (((kk * 4 + g) ^ c16) * 16));
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+          q[kk] = ldg16(a.q + cc.b * a.q_stride_bytes +
+                        (static_cast<int64_t>(h0 + min(c16, nh - 1)) * D + kk * 32 + g * 8) * 2);
         // The wait for these loads (it also drains the stages in flight) must stay on this path:
         // left to the first use after the join it would run on every stage.
         asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]));
-#pragma unroll
-        for (int mb = 0; mb < 8; ++mb) o[mb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        m = kNegBig;
-        l = 0.0f;
-        run_open = true;
       }
+      if (c16 >= nh) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) q[kk] = u32x4{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int mb = 0; mb < 8; ++mb) o[mb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      m = kNegBig;
+      l = 0.0f;
+      c_ctx_first = s;
     }
 
     // ---- scores of the stage's 16 tokens: lane (head c16, tokens 4g .. 4g+3)
@@ -759,7 +849,7 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       const u32x4 kr = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ c16) * 16));
       sc = Mfma<QT>::k32(kr, q[kk], sc);
     }
-    const int tok0 = cc.it * kItem + j * kStageTokens + 4 * g;
+    const int tok0 = cc.st * T + 4 * g;
     float sv[4];
     bool over = false;
 #pragma unroll
@@ -777,13 +867,13 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
         for (int mb = 0; mb < 8; ++mb) o[mb] *= alpha;
       }
     }
-    float p[4];
+    float pr[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      p[r] = fast_exp2(sv[r] - m);
-      l += p[r];
+      pr[r] = fast_exp2(sv[r] - m);
+      l += pr[r];
     }
-    const u32x2 pb = {QT::pack(p[0], p[1]), QT::pack(p[2], p[3])};
+    const u32x2 pb = {QT::pack(pr[0], pr[1]), QT::pack(pr[2], pr[3])};
     // ---- O^T += V^T . P^T: lane c16 of a 16-lane group supplies the address of 4 dims of token
     // row 4g + c16/4 and receives the 4 tokens of dim column 16 mb + c16
 #pragma unroll
@@ -793,8 +883,9 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       o[mb] = Mfma<QT>::k16(vt, pb, o[mb]);
     }
 
-    // ---- end of a run: last item of the context or of the worker's range
-    if (j == kStagesPerItem - 1 && (cc.it == cc.n_items - 1 || s == n_stages - 1)) {
+    // ---- end of a run: last stage of the context or of the worker's range
+    const bool ctx_end = cc.st == cc.n_st - 1;
+    if (ctx_end || s == n_stages - 1) {
       const float lsum = quad_rows_sum(l);
       const float inv = 1.0f / lsum;
       const float lse2 = m + fast_log2(lsum);
@@ -820,26 +911,34 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       if (head_on && g == 0 && complete && a.lse != nullptr) a.lse[cc.b * a.n_q_heads + hq] = lse2 * kLn2;
       if (head_on && g == 0 && !complete) a.ws_lse[pidx] = lse2;
       first_run = false;
-      run_open = false;
+    }
+    ++cc.st;
+    if (ctx_end && s + 1 < n_stages) {
+      c_prev_len = s + 1 - c_ctx_first;
+      next_context(cc);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-// Merge of the partials of contexts that span several workgroups; also writes the output
-// of empty sequences.  One workgroup per (query head, sequence).
+// Merge of the partials of contexts that span several workers (workgroups of the dot-product
+// kernel, wavefronts of the matrix-core kernel); also writes the output of empty sequences.
+// One workgroup per (query head, sequence), thread t owns dims t and t + 128.  The kernel is a
+// chain of dependent round trips to memory, so it keeps them to two: the item prefix, then the
+// LSEs and accumulators of four consecutive workers at a time, all loads of a group issued
+// together.
 template <typename QT>
 __global__ __launch_bounds__(128) void merge_partials_kernel(GqaArgs a, int dv) {
   const int hq = blockIdx.x;
   const int b = blockIdx.y;
+  const int tid = threadIdx.x;
   const int G = a.g_block;
-  const int32_t* pages;
-  int L;
-  sequence_of(a, b, pages, L);
+  const int p0 = a.ws_prefix[b], p1 = a.ws_prefix[b + 1], pt = a.ws_prefix[a.batch];
   uint16_t* out = reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes) + hq * dv;
-  if (L <= 0) {
-    for (int d = threadIdx.x; d < dv; d += 128) out[d] = 0;
-    if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * a.n_q_heads + hq] = -INFINITY;
+  const int n_items = p1 - p0;
+  if (n_items <= 0) {  // empty sequence
+    for (int d = tid; d < dv; d += 128) out[d] = 0;
+    if (a.lse != nullptr && tid == 0) a.lse[b * a.n_q_heads + hq] = -INFINITY;
     return;
   }
   const int hb_per_kv = (a.group + G - 1) / G;
@@ -847,37 +946,59 @@ __global__ __launch_bounds__(128) void merge_partials_kernel(GqaArgs a, int dv) 
   const int kvh = hq / a.group;
   const int hbk = kvh * hb_per_kv + (hq - kvh * a.group) / G;
   const int h = (hq - kvh * a.group) % G;
-  const int64_t total = static_cast<int64_t>(a.ws_prefix[a.batch]) * n_hb;
-  const int n_items = a.ws_prefix[b + 1] - a.ws_prefix[b];
-  const int64_t first = static_cast<int64_t>(a.ws_prefix[b]) * n_hb + static_cast<int64_t>(hbk) * n_items;
+  const int64_t total = static_cast<int64_t>(pt) * n_hb;
+  const int64_t first = static_cast<int64_t>(p0) * n_hb + static_cast<int64_t>(hbk) * n_items;
   const int64_t last = first + n_items - 1;
-  const int64_t n_wg = a.n_workgroups;
-  const int w_first = workgroup_of(first, total, n_wg);
-  const int w_last = workgroup_of(last, total, n_wg);
-  if (w_first == w_last) return;  // one workgroup saw the whole context and wrote the output
-  // the first workgroup holds this context as its last run (slot 1) unless its range starts
+  const int64_t n = a.n_workgroups;
+  const int w_first = workgroup_of(first, total, n);
+  const int w_last = workgroup_of(last, total, n);
+  if (w_first == w_last) return;  // one worker saw the whole context and wrote the output
+  // range_start(w) = w * q + floor(w * r / n) with total = q * n + r: stepped from w to w + 1
+  // without a division
+  const int64_t q = total / n, r = total - q * n;
+  int64_t rs = range_start(w_first, total, n);
+  int64_t acc = (static_cast<int64_t>(w_first) * r) % n;
+  // the first worker holds this context as its last run (slot 1) unless its range starts
   // exactly here; every later one holds it as its first run (slot 0)
-  const int slot_first = range_start(w_first, total, n_wg) < first ? 1 : 0;
-  auto pslot = [&](int w) { return static_cast<int64_t>(w) * 2 + (w == w_first ? slot_first : 0); };
-  // with fewer items than workgroups some ranges in between are empty and own no partial
-  auto has_items = [&](int w) { return range_start(w, total, n_wg) < range_start(w + 1, total, n_wg); };
-  float mx = kNegBig;
-  for (int w = w_first; w <= w_last; ++w)
-    if (has_items(w)) mx = fmaxf(mx, a.ws_lse[pslot(w) * G + h]);
-  float wsum = 0.0f;
-  for (int w = w_first; w <= w_last; ++w)
-    if (has_items(w)) wsum += fast_exp2(a.ws_lse[pslot(w) * G + h] - mx);
-  const float inv = 1.0f / wsum;
-  for (int d = threadIdx.x; d < dv; d += 128) {
-    float o = 0.0f;
-    for (int w = w_first; w <= w_last; ++w) {
-      if (!has_items(w)) continue;
-      const int64_t ps = pslot(w) * G + h;
-      o += fast_exp2(a.ws_lse[ps] - mx) * a.ws_out[ps * dv + d];
+  const int slot_first = rs < first ? 1 : 0;
+  const int d0 = tid, d1 = tid + 128;
+  const bool on0 = d0 < dv, on1 = d1 < dv;
+  float M = kNegBig, W = 0.0f, O0 = 0.0f, O1 = 0.0f;
+  for (int wb = w_first; wb <= w_last; wb += 4) {
+    float lse[4], x0[4], x1[4];
+    bool on[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int w = wb + k;
+      acc += r;
+      const int64_t step = q + (acc >= n ? 1 : 0);
+      acc -= acc >= n ? n : 0;
+      // with fewer items than workers some ranges in between are empty and own no partial
+      on[k] = w <= w_last && step > 0;
+      rs += step;
+      const int64_t ps = (static_cast<int64_t>(w) * 2 + (w == w_first ? slot_first : 0)) * G + h;
+      lse[k] = on[k] ? a.ws_lse[ps] : kNegBig;
+      x0[k] = on[k] && on0 ? a.ws_out[ps * dv + d0] : 0.0f;
+      x1[k] = on[k] && on1 ? a.ws_out[ps * dv + d1] : 0.0f;
     }
-    out[d] = QT::from_f32(o * inv);
+    const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
+    const float keep = fast_exp2(M - m_new);
+    W *= keep;
+    O0 *= keep;
+    O1 *= keep;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
+      W += e;
+      O0 += e * x0[k];
+      O1 += e * x1[k];
+    }
+    M = m_new;
   }
-  if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * a.n_q_heads + hq] = (mx + fast_log2(wsum)) * kLn2;
+  const float inv = 1.0f / W;
+  if (on0) out[d0] = QT::from_f32(O0 * inv);
+  if (on1) out[d1] = QT::from_f32(O1 * inv);
+  if (a.lse != nullptr && tid == 0) a.lse[b * a.n_q_heads + hq] = (M + fast_log2(W)) * kLn2;
 }
 
 int device_cu_count() {
@@ -980,7 +1101,9 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
       default: return XLLM_MI355_ESHAPE;
     }
   } else {
-    if (head_dim == 128 && a.bs_shift >= 0 && use_mfma_kernel()) return launch_gqa_mfma<QT>(a, wsb, s, plan_only, need);
+    // (its epilogue stores 8 output bytes at a time)
+    const bool out_aligned = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
+    if (head_dim == 128 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel()) return launch_gqa_mfma<QT>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, false, 64, 8, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, false, 128, 16, 4>(a, wsb, s, plan_only, need);
