@@ -923,29 +923,47 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
 
 // Merge of the partials of contexts that span several workers (workgroups of the dot-product
 // kernel, wavefronts of the matrix-core kernel); also writes the output of empty sequences.
-// One workgroup per (query head, sequence), thread t owns dims t and t + 128.  The kernel is a
-// chain of dependent round trips to memory, so it keeps them to two: the item prefix, then the
-// LSEs and accumulators of four consecutive workers at a time, all loads of a group issued
-// together.
+// One workgroup per (head block, sequence); a thread owns four consecutive dims of one head, so
+// a partial's rows (contiguous over the heads of the block) are read with 16-byte loads.  The
+// kernel is a chain of dependent round trips to memory, so it keeps them to two: the item
+// prefix, then the LSEs and accumulators of four consecutive workers at a time, all loads of a
+// group issued together.
 template <typename QT>
-__global__ __launch_bounds__(128) void merge_partials_kernel(GqaArgs a, int dv) {
-  const int hq = blockIdx.x;
+__global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int dv) {
+  const int hbk = blockIdx.x;
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
   const int G = a.g_block;
   const int p0 = a.ws_prefix[b], p1 = a.ws_prefix[b + 1], pt = a.ws_prefix[a.batch];
-  uint16_t* out = reinterpret_cast<uint16_t*>(a.out + b * a.out_stride_bytes) + hq * dv;
-  const int n_items = p1 - p0;
-  if (n_items <= 0) {  // empty sequence
-    for (int d = tid; d < dv; d += 128) out[d] = 0;
-    if (a.lse != nullptr && tid == 0) a.lse[b * a.n_q_heads + hq] = -INFINITY;
-    return;
-  }
   const int hb_per_kv = (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
-  const int kvh = hq / a.group;
-  const int hbk = kvh * hb_per_kv + (hq - kvh * a.group) / G;
-  const int h = (hq - kvh * a.group) % G;
+  const int kvh = hbk / hb_per_kv;
+  const int h0 = kvh * a.group + (hbk - kvh * hb_per_kv) * G;
+  const int nh = min(G, (kvh + 1) * a.group - h0);
+  const int dv4 = dv >> 2;         // 16-byte groups per head row
+  const int n_vec = nh * dv4;      // per partial
+  char* out_row = a.out + b * a.out_stride_bytes;
+  const bool wide = ((reinterpret_cast<uintptr_t>(a.out) | static_cast<uintptr_t>(a.out_stride_bytes)) & 7) == 0;
+  auto store4 = [&](int h, int d, float x0, float x1, float x2, float x3) {
+    uint16_t* o = reinterpret_cast<uint16_t*>(out_row) + static_cast<int64_t>(h0 + h) * dv + d;
+    if (wide) {
+      const u32x2 w = {QT::pack(x0, x1), QT::pack(x2, x3)};
+      *reinterpret_cast<u32x2*>(o) = w;
+    } else {
+      o[0] = QT::from_f32(x0);
+      o[1] = QT::from_f32(x1);
+      o[2] = QT::from_f32(x2);
+      o[3] = QT::from_f32(x3);
+    }
+  };
+  const int n_items = p1 - p0;
+  if (n_items <= 0) {  // empty sequence
+    for (int v = tid; v < n_vec; v += kThreads) {
+      store4(v / dv4, (v % dv4) * 4, 0.0f, 0.0f, 0.0f, 0.0f);
+      if (a.lse != nullptr && v % dv4 == 0) a.lse[b * a.n_q_heads + h0 + v / dv4] = -INFINITY;
+    }
+    return;
+  }
   const int64_t total = static_cast<int64_t>(pt) * n_hb;
   const int64_t first = static_cast<int64_t>(p0) * n_hb + static_cast<int64_t>(hbk) * n_items;
   const int64_t last = first + n_items - 1;
@@ -956,49 +974,47 @@ __global__ __launch_bounds__(128) void merge_partials_kernel(GqaArgs a, int dv) 
   // range_start(w) = w * q + floor(w * r / n) with total = q * n + r: stepped from w to w + 1
   // without a division
   const int64_t q = total / n, r = total - q * n;
-  int64_t rs = range_start(w_first, total, n);
-  int64_t acc = (static_cast<int64_t>(w_first) * r) % n;
+  const int64_t acc0 = (static_cast<int64_t>(w_first) * r) % n;
   // the first worker holds this context as its last run (slot 1) unless its range starts
   // exactly here; every later one holds it as its first run (slot 0)
-  const int slot_first = rs < first ? 1 : 0;
-  const int d0 = tid, d1 = tid + 128;
-  const bool on0 = d0 < dv, on1 = d1 < dv;
-  float M = kNegBig, W = 0.0f, O0 = 0.0f, O1 = 0.0f;
-  for (int wb = w_first; wb <= w_last; wb += 4) {
-    float lse[4], x0[4], x1[4];
-    bool on[4];
+  const int slot_first = range_start(w_first, total, n) < first ? 1 : 0;
+  for (int v = tid; v < n_vec; v += kThreads) {
+    const int h = v / dv4, d = (v - h * dv4) * 4;
+    int64_t acc = acc0;
+    float M = kNegBig, W = 0.0f;
+    f32x4 O = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int wb = w_first; wb <= w_last; wb += 4) {
+      float lse[4];
+      f32x4 x[4];
+      bool on[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int w = wb + k;
-      acc += r;
-      const int64_t step = q + (acc >= n ? 1 : 0);
-      acc -= acc >= n ? n : 0;
-      // with fewer items than workers some ranges in between are empty and own no partial
-      on[k] = w <= w_last && step > 0;
-      rs += step;
-      const int64_t ps = (static_cast<int64_t>(w) * 2 + (w == w_first ? slot_first : 0)) * G + h;
-      lse[k] = on[k] ? a.ws_lse[ps] : kNegBig;
-      x0[k] = on[k] && on0 ? a.ws_out[ps * dv + d0] : 0.0f;
-      x1[k] = on[k] && on1 ? a.ws_out[ps * dv + d1] : 0.0f;
-    }
-    const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
-    const float keep = fast_exp2(M - m_new);
-    W *= keep;
-    O0 *= keep;
-    O1 *= keep;
+      for (int k = 0; k < 4; ++k) {
+        const int w = wb + k;
+        acc += r;
+        const int64_t step = q + (acc >= n ? 1 : 0);
+        acc -= acc >= n ? n : 0;
+        // with fewer items than workers some ranges in between are empty and own no partial
+        on[k] = w <= w_last && step > 0;
+        const int64_t ps = (static_cast<int64_t>(w) * 2 + (w == w_first ? slot_first : 0)) * G + h;
+        lse[k] = on[k] ? a.ws_lse[ps] : kNegBig;
+        x[k] = on[k] ? *reinterpret_cast<const f32x4*>(a.ws_out + ps * dv + d) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+      const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
+      const float keep = fast_exp2(M - m_new);
+      W *= keep;
+      O *= keep;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
-      W += e;
-      O0 += e * x0[k];
-      O1 += e * x1[k];
+      for (int k = 0; k < 4; ++k) {
+        const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
+        W += e;
+        O += e * x[k];
+      }
+      M = m_new;
     }
-    M = m_new;
+    const float inv = 1.0f / W;
+    store4(h, d, O[0] * inv, O[1] * inv, O[2] * inv, O[3] * inv);
+    if (a.lse != nullptr && d == 0) a.lse[b * a.n_q_heads + h0 + h] = (M + fast_log2(W)) * kLn2;
   }
-  const float inv = 1.0f / W;
-  if (on0) out[d0] = QT::from_f32(O0 * inv);
-  if (on1) out[d1] = QT::from_f32(O1 * inv);
-  if (a.lse != nullptr && tid == 0) a.lse[b * a.n_q_heads + hq] = (M + fast_log2(W)) * kLn2;
 }
 
 int device_cu_count() {
@@ -1203,11 +1219,12 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
       rc = fp8 ? dispatch_dim<FP16, true>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need)
                : dispatch_dim<FP16, false>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need);
     if (rc != 0) return rc;
-    dim3 grid(static_cast<unsigned>(n_q_heads), static_cast<unsigned>(nb));
+    const int hb_per_kv = (group + a.g_block - 1) / a.g_block;
+    dim3 grid(static_cast<unsigned>(n_kv_heads * hb_per_kv), static_cast<unsigned>(nb));
     if (q_dtype == XLLM_MI355_BF16)
-      merge_partials_kernel<BF16><<<grid, 128, 0, stream>>>(a, static_cast<int>(head_dim));
+      merge_partials_kernel<BF16><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
     else
-      merge_partials_kernel<FP16><<<grid, 128, 0, stream>>>(a, static_cast<int>(head_dim));
+      merge_partials_kernel<FP16><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
     rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
   }

@@ -419,43 +419,65 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 // Merge of the partials of contexts that span several teams; also writes the output of
 // empty sequences.  One workgroup per (head, sequence).
 __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
+  // One workgroup per (head, sequence); thread t owns dims 4t .. 4t+3, read from the fp32 partials
+  // with 16-byte loads.  Two dependent round trips to memory: the tile prefix, then the LSEs and
+  // accumulators of four consecutive teams at a time, all loads of a group issued together.
   const int h = blockIdx.x;
   const int b = blockIdx.y;
   const int H = a.n_heads;
-  const int L = a.seq_lens[b];
-  uint16_t* out = reinterpret_cast<uint16_t*>(a.out) + (static_cast<int64_t>(b) * H + h) * kDL;
-  if (L <= 0) {
-    for (int d = threadIdx.x; d < kDL; d += 128) out[d] = 0;
+  const int d = threadIdx.x * 4;
+  const int64_t first = a.ws_prefix[b];
+  const int64_t last = static_cast<int64_t>(a.ws_prefix[b + 1]) - 1;
+  const int64_t total = a.ws_prefix[a.batch];
+  uint16_t* out = reinterpret_cast<uint16_t*>(a.out) + (static_cast<int64_t>(b) * H + h) * kDL + d;
+  if (last < first) {  // empty sequence
+    *reinterpret_cast<u32x2*>(out) = u32x2{0u, 0u};
     if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = -INFINITY;
     return;
   }
-  const int64_t total = a.ws_prefix[a.batch];
-  const int64_t first = a.ws_prefix[b];
-  const int64_t last = a.ws_prefix[b + 1] - 1;
   const int64_t n = a.n_teams;
   const int t_first = team_of(first, total, n);
   const int t_last = team_of(last, total, n);
   if (t_first == t_last) return;  // one team saw the whole context and wrote the output
+  // team_start(t) = t * q + floor(t * r / n) with total = q * n + r: stepped without a division
+  const int64_t q = total / n, r = total - q * n;
+  int64_t acc = (static_cast<int64_t>(t_first) * r) % n;
+  // the first team holds this context as its last run (slot 1) unless its range starts exactly
+  // here; every later one holds it as its first run (slot 0)
   const int slot_first = team_start(t_first, total, n) < first ? 1 : 0;
-  auto pslot = [&](int t) { return (static_cast<int64_t>(t) * 2 + (t == t_first ? slot_first : 0)) * H + h; };
-  auto has_items = [&](int t) { return team_start(t, total, n) < team_start(t + 1, total, n); };
-  float mx = kNegBig;
-  for (int t = t_first; t <= t_last; ++t)
-    if (has_items(t)) mx = fmaxf(mx, a.ws_lse[pslot(t)]);
-  float wsum = 0.0f;
-  for (int t = t_first; t <= t_last; ++t)
-    if (has_items(t)) wsum += fast_exp2(a.ws_lse[pslot(t)] - mx);
-  const float inv = 1.0f / wsum;
-  for (int d = threadIdx.x; d < kDL; d += 128) {
-    float acc = 0.0f;
-    for (int t = t_first; t <= t_last; ++t) {
-      if (!has_items(t)) continue;
-      const int64_t ps = pslot(t);
-      acc += fast_exp2(a.ws_lse[ps] - mx) * a.ws_out[ps * kDL + d];
+  float M = kNegBig, W = 0.0f;
+  f32x4 O = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int tb = t_first; tb <= t_last; tb += 4) {
+    float lse[4];
+    f32x4 x[4];
+    bool on[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = tb + k;
+      acc += r;
+      const int64_t step = q + (acc >= n ? 1 : 0);
+      acc -= acc >= n ? n : 0;
+      // with fewer tiles than teams some ranges in between are empty and own no partial
+      on[k] = t <= t_last && step > 0;
+      const int64_t ps = (static_cast<int64_t>(t) * 2 + (t == t_first ? slot_first : 0)) * H + h;
+      lse[k] = on[k] ? a.ws_lse[ps] : kNegBig;
+      x[k] = on[k] ? *reinterpret_cast<const f32x4*>(a.ws_out + ps * kDL + d) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    out[d] = BF16::from_f32(acc * inv);
+    const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
+    const float keep = fast_exp2(M - m_new);
+    W *= keep;
+    O *= keep;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
+      W += e;
+      O += e * x[k];
+    }
+    M = m_new;
   }
-  if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = (mx + fast_log2(wsum)) * kLn2;
+  const float inv = 1.0f / W;
+  *reinterpret_cast<u32x2*>(out) = u32x2{BF16::pack(O[0] * inv, O[1] * inv), BF16::pack(O[2] * inv, O[3] * inv)};
+  if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = (M + fast_log2(W)) * kLn2;
 }
 
 int mla_cu_count() {

@@ -108,34 +108,73 @@ __global__ __launch_bounds__(256) void reshape_elem_kernel(ReshapeArgs a) {
   }
 }
 
-// scale[h] = max(absmax / 448, 1e-12).  One workgroup per KV head; |x| is compared as
-// an integer after clearing the sign, which orders finite floats and is exact.
+// Per-KV-head dynamic scale max(|x|) / 448 (floor 1e-12), the quantity the reference's
+// fp8_scaled_quantize derives when no scale is given (kernels/cuda/fp8_scaled_quantize.cpp:38-42).
+// scales[] is first cleared, then every workgroup folds a chunk of tokens of one head and
+// publishes its candidate with an integer atomic maximum on the float's bits (all candidates are
+// positive, so the bit patterns order like the values); dividing before or after the maximum gives
+// the same float.
+constexpr int kScaleChunk = 512;  // tokens per workgroup
+
+__global__ void clear_scales_kernel(float* scales, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) scales[i] = 0.0f;
+}
+
 template <int IN>
 __global__ __launch_bounds__(256) void kv_head_scales_kernel(const char* x, float* scales,
                                                              int64_t n_tokens, int head_dim,
-                                                             int64_t stride_bytes) {
+                                                             int64_t stride_bytes, int vec_ok) {
   constexpr int ES = IN == 2 ? 4 : 2;
-  const int h = blockIdx.x;
+  const int h = blockIdx.y;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kScaleChunk;
+  const int64_t t1 = min(n_tokens, t0 + kScaleChunk);
+  const char* base = x + static_cast<int64_t>(h) * head_dim * ES;
   float amax = 0.0f;
-  const int64_t n = n_tokens * head_dim;
-  for (int64_t i = threadIdx.x; i < n; i += 256) {
-    const int64_t t = i / head_dim;
-    const int d = static_cast<int>(i - t * head_dim);
-    const char* p = x + t * stride_bytes + (static_cast<int64_t>(h) * head_dim + d) * ES;
-    float v;
-    if constexpr (IN == 2) v = *reinterpret_cast<const float*>(p);
-    else if constexpr (IN == 0) v = BF16::to_f32(*reinterpret_cast<const uint16_t*>(p));
-    else v = FP16::to_f32(*reinterpret_cast<const uint16_t*>(p));
-    amax = fmaxf(amax, fabsf(v));
+  auto fold = [&](u32 w) {
+    if constexpr (IN == 2) {
+      amax = fmaxf(amax, fabsf(as_f32(w)));
+    } else if constexpr (IN == 0) {
+      amax = fmaxf(amax, fmaxf(fabsf(BF16::lo(w)), fabsf(BF16::hi(w))));
+    } else {
+      amax = fmaxf(amax, fmaxf(fabsf(FP16::lo(w)), fabsf(FP16::hi(w))));
+    }
+  };
+  const int vpr = head_dim * ES / 16;  // 16-byte vectors per head row
+  if (vec_ok && vpr <= 256) {
+    const int v = threadIdx.x % vpr, tr = threadIdx.x / vpr, tpp = 256 / vpr;
+    if (tr < tpp) {
+      for (int64_t t = t0 + tr; t < t1; t += tpp) {
+        const u32x4 w = ldg16(base + t * stride_bytes + v * 16);
+        fold(w[0]);
+        fold(w[1]);
+        fold(w[2]);
+        fold(w[3]);
+      }
+    }
+  } else {
+    for (int64_t t = t0; t < t1; ++t) {
+      for (int d = threadIdx.x; d < head_dim; d += 256) {
+        const char* p = base + t * stride_bytes + static_cast<int64_t>(d) * ES;
+        float val;
+        if constexpr (IN == 2) val = *reinterpret_cast<const float*>(p);
+        else if constexpr (IN == 0) val = BF16::to_f32(*reinterpret_cast<const uint16_t*>(p));
+        else val = FP16::to_f32(*reinterpret_cast<const uint16_t*>(p));
+        amax = fmaxf(amax, fabsf(val));
+      }
+    }
   }
   __shared__ float red[256];
   red[threadIdx.x] = amax;
   __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if (threadIdx.x < s) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+  for (int st = 128; st > 0; st >>= 1) {
+    if (threadIdx.x < st) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + st]);
     __syncthreads();
   }
-  if (threadIdx.x == 0) scales[h] = fmaxf(red[0] / 448.0f, 1e-12f);
+  if (threadIdx.x == 0) {
+    const float cand = fmaxf(red[0] / 448.0f, 1e-12f);
+    atomicMax(reinterpret_cast<unsigned int*>(scales + h), __float_as_uint(cand));
+  }
 }
 
 template <int IN>
@@ -213,16 +252,21 @@ int kv_head_scales(const void* x, float* scales, int64_t n_tokens, int64_t n_kv_
   if (token_stride < n_kv_heads * head_dim || n_kv_heads > 65535 || head_dim > (1 << 20))
     return XLLM_MI355_EINVAL;
   const char* p = static_cast<const char*>(x);
-  dim3 grid(static_cast<unsigned>(n_kv_heads));
+  const int es = in_dtype == XLLM_MI355_FP32 ? 4 : 2;
+  const int vec_ok = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (token_stride * es) % 16 == 0 &&
+                     (head_dim * es) % 16 == 0;
+  clear_scales_kernel<<<dim3(static_cast<unsigned>((n_kv_heads + 255) / 256)), 256, 0, stream>>>(
+      scales, static_cast<int>(n_kv_heads));
+  dim3 grid(static_cast<unsigned>((n_tokens + kScaleChunk - 1) / kScaleChunk), static_cast<unsigned>(n_kv_heads));
   switch (in_dtype) {
     case XLLM_MI355_BF16:
-      kv_head_scales_kernel<0><<<grid, 256, 0, stream>>>(p, scales, n_tokens, (int)head_dim, token_stride * 2);
+      kv_head_scales_kernel<0><<<grid, 256, 0, stream>>>(p, scales, n_tokens, (int)head_dim, token_stride * 2, vec_ok);
       break;
     case XLLM_MI355_FP16:
-      kv_head_scales_kernel<1><<<grid, 256, 0, stream>>>(p, scales, n_tokens, (int)head_dim, token_stride * 2);
+      kv_head_scales_kernel<1><<<grid, 256, 0, stream>>>(p, scales, n_tokens, (int)head_dim, token_stride * 2, vec_ok);
       break;
     case XLLM_MI355_FP32:
-      kv_head_scales_kernel<2><<<grid, 256, 0, stream>>>(p, scales, n_tokens, (int)head_dim, token_stride * 4);
+      kv_head_scales_kernel<2><<<grid, 256, 0, stream>>>(p, scales, n_tokens, (int)head_dim, token_stride * 4, vec_ok);
       break;
     default: return XLLM_MI355_EDTYPE;
   }
