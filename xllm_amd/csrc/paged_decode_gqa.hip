@@ -494,12 +494,13 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
 // for every younger stage in flight.  Page ids come through the same LDS path one item ahead,
 // the Q rows of a run just before its first stage, sequence lengths through the scalar cache.
 constexpr float kSlack = 8.0f;
-constexpr int kStageTokens = 16;
-constexpr int kStageBytes = 2 * kStageTokens * 256;  // K rows then V rows
+constexpr int kStageBytes = 8192;  // K rows then V rows: 16 tokens of 16-bit pages, 32 of fp8 pages
 constexpr int kMfmaHeads = 16;                        // head columns of one MFMA
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
 typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 
@@ -602,11 +603,15 @@ struct MfmaLayout {
   static constexpr int kPrefixOff = kTmpOff + kThreads * 4;
 };
 
-template <typename QT, int NS>
+template <typename QT, bool FP8, int NS>
 __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   static_assert(NS >= 2 && NS <= 4, "wait_younger_stages covers up to three stages in flight");
   using Lay = MfmaLayout<NS>;
-  constexpr int D = 128, RB = 256, G = kMfmaHeads, T = kStageTokens;
+  constexpr int D = 128, G = kMfmaHeads;
+  constexpr int RB = FP8 ? 128 : 256;      // bytes of one token row of one KV head
+  constexpr int T = kStageBytes / 2 / RB;  // tokens per stage
+  constexpr int LPR = RB / 16;             // lanes (16-byte chunks) per row in a load instruction
+  constexpr int RPI = kWave / LPR;         // rows per load instruction
 
   extern __shared__ __align__(16) char smem[];
   int* tmp = reinterpret_cast<int*>(smem + Lay::kTmpOff);
@@ -616,6 +621,12 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15;   // MFMA column (head) / row (token, dim); 16-byte chunk of a row in the loads
   const int g = lane >> 4;     // MFMA k-group; token row of a load instruction
+  const int dc = lane % LPR;   // chunk and row of the lane in a load instruction of a K / V tile
+  const int dr = lane / LPR;
+  // chunk swizzles within a row: K by the row number; V by twice its low two bits (16-bit pages,
+  // whose transposing read takes 4 rows x 32 bytes per 16 lanes) or by its low three bits (fp8)
+  auto swz_k = [](int row) { return row & (LPR - 1); };
+  auto swz_v = [](int row) { return FP8 ? (row & 7) : ((row & 3) << 1); };
   const int hb_per_kv = (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
 
@@ -638,8 +649,8 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   const char* ring = smem + wave * NS * kStageBytes;
   const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + wave * 3 * kWave * 4);
   const char* pagebuf = smem + Lay::kPageOff + wave * 3 * kWave * 4;
-  const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + wave * G * RB);
-  const char* qbuf = smem + Lay::kQOff + wave * G * RB;
+  const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + wave * G * 256);
+  const char* qbuf = smem + Lay::kQOff + wave * G * 256;
 
   auto locate = [&](int64_t f, CtxCursor& cu) {
     int lo = 0, hi = a.batch;
@@ -685,9 +696,9 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   u32 lane_k[4], lane_v[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int row = 4 * i + g;
-    lane_k[i] = static_cast<u32>(row * a.row_bytes) + ((c16 ^ row) * 16);
-    lane_v[i] = static_cast<u32>(row * a.row_bytes) + ((c16 ^ (g << 1)) * 16);
+    const int row = RPI * i + dr;  // its sub-block of 16 tokens has its own base address
+    lane_k[i] = static_cast<u32>((row & 15) * a.row_bytes) + ((dc ^ swz_k(row)) * 16);
+    lane_v[i] = static_cast<u32>((row & 15) * a.row_bytes) + ((dc ^ swz_v(row)) * 16);
   }
 
   // A chunk or Q load issued while p was t has landed once the consumer has waited for stage t,
@@ -748,43 +759,56 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       begin_context(false);
     }
     const int tok0 = pc.st * T;
-    const int pi = tok0 >> a.bs_shift;  // block_size >= 16: one page holds the whole stage
-    if ((pi >> 6) != ck_a) {
-      const u32 t = off_a;
-      off_a = off_b;
-      off_b = t;
-      ck_a = pi >> 6;
-      ensure_landed(has_b, t_b);
-      has_b = false;
-      const int n_pages = (pc.L + a.block_size - 1) >> a.bs_shift;
-      if ((ck_a + 1) * kWave < n_pages) {
-        issue_chunk(pc, ck_a + 1, off_b);
-        t_b = p;
-        has_b = true;
+    const int lim = pc.L - tok0 - 1;  // last valid row of the stage
+    // block_size >= 16: a sub-block of 16 tokens lies in one page
+    constexpr int NSUB = T / 16;
+    uint64_t kb[NSUB], vb[NSUB];
+#pragma unroll
+    for (int sub = 0; sub < NSUB; ++sub) {
+      if (sub == 0 || sub * 16 <= lim) {
+        const int tok = tok0 + sub * 16;
+        const int pi = tok >> a.bs_shift;
+        if ((pi >> 6) != ck_a) {
+          const u32 t = off_a;
+          off_a = off_b;
+          off_b = t;
+          ck_a = pi >> 6;
+          ensure_landed(has_b, t_b);
+          has_b = false;
+          const int n_pages = (pc.L + a.block_size - 1) >> a.bs_shift;
+          if ((ck_a + 1) * kWave < n_pages) {
+            issue_chunk(pc, ck_a + 1, off_b);
+            t_b = p;
+            has_b = true;
+          }
+        }
+        int page = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(pagebuf + off_a + (pi & 63) * 4));
+        page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
+        const int slot0 = page * a.block_size + (tok & (a.block_size - 1));
+        const uint64_t row0 = static_cast<uint64_t>(slot0) * static_cast<uint64_t>(a.row_bytes) +
+                              static_cast<uint64_t>(pc.hbk / hb_per_kv) * RB;
+        kb[sub] = reinterpret_cast<uint64_t>(a.k_cache) + row0;
+        vb[sub] = reinterpret_cast<uint64_t>(a.v_cache) + row0;
+      } else {  // past the end of the context: its rows repeat the last valid one
+        kb[sub] = kb[sub - 1];
+        vb[sub] = vb[sub - 1];
       }
     }
-    int page = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(pagebuf + off_a + (pi & 63) * 4));
-    page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
-    const int slot0 = page * a.block_size + (tok0 & (a.block_size - 1));
-    const uint64_t row0 = static_cast<uint64_t>(slot0) * static_cast<uint64_t>(a.row_bytes) +
-                          static_cast<uint64_t>(pc.hbk / hb_per_kv) * RB;
-    const uint64_t kb = reinterpret_cast<uint64_t>(a.k_cache) + row0;
-    const uint64_t vb = reinterpret_cast<uint64_t>(a.v_cache) + row0;
     const u32 dst = ring_lds + (p % NS) * kStageBytes;
-    const int lim = pc.L - tok0 - 1;  // last valid row of the stage
     if (lim >= T - 1) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        dma16_row(kb, lane_k[i], dst + i * 1024);
-        dma16_row(vb, lane_v[i], dst + T * RB + i * 1024);
+        dma16_row(kb[(RPI * i) >> 4], lane_k[i], dst + i * 1024);
+        dma16_row(vb[(RPI * i) >> 4], lane_v[i], dst + T * RB + i * 1024);
       }
     } else {  // ragged end of a context: rows past it repeat the last valid row
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int row = 4 * i + g;
-        const u32 ro = static_cast<u32>(min(row, lim) * a.row_bytes);
-        dma16_row(kb, ro + ((c16 ^ row) * 16), dst + i * 1024);
-        dma16_row(vb, ro + ((c16 ^ (g << 1)) * 16), dst + T * RB + i * 1024);
+        const int row = RPI * i + dr;
+        const int sub = min(RPI * i, lim) >> 4;  // sub-block of the rows this instruction reads
+        const u32 ro = static_cast<u32>((min(row, lim) & 15) * a.row_bytes);
+        dma16_row(NSUB > 1 && sub > 0 ? kb[NSUB - 1] : kb[0], ro + ((dc ^ swz_k(row)) * 16), dst + i * 1024);
+        dma16_row(NSUB > 1 && sub > 0 ? vb[NSUB - 1] : vb[0], ro + ((dc ^ swz_v(row)) * 16), dst + T * RB + i * 1024);
       }
     }
     ++p;
@@ -804,9 +828,19 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   f32x4 o[8];
   float m = kNegBig, l = 0.0f;
   // per-lane constants of the operand reads
-  const int k_read = c16 * RB;                                   // + ((chunk ^ c16) * 16)
+  const int q_read = c16 * 256;  // Q rows (16-bit): + ((chunk ^ c16) * 16)
+  // 16-bit pages.  K: row c16, + ((chunk ^ c16) * 16).  V: lane c16 of a 16-lane group addresses 4 dims
+  // (8 bytes) of token row 4g + c16/4; + (v_y ^ (mb << 5)) selects dims 16 mb ..
+  const int k_read = c16 * RB;
   const int v_read = T * RB + (4 * g + (c16 >> 2)) * RB + ((c16 & 3) >> 1) * 16 + (c16 & 1) * 8;
-  const int v_y = (c16 >> 2) << 5;                                // swizzle term of the lane's row
+  const int v_y = (c16 >> 2) << 5;
+  // fp8 pages.  K: rows c16 and 16 + c16, 8 bytes of chunk kk*2 + g/2.  V: lane c16 of a 16-lane group
+  // addresses 8 dims (8 bytes) of the token in k-slot c16/2 of the group: tokens 4g .. 4g+3, then
+  // 16 + 4g .. 16 + 4g+3 -- the order in which the two score blocks leave the P^T registers
+  const int v8_row = ((c16 >> 1) < 4 ? 0 : 12) + 4 * g + (c16 >> 1);
+  const int v8_read = T * RB + v8_row * RB + (c16 & 1) * 8;
+  const int v8_y = (v8_row & 7) << 4;
+  float score_scale = a.scale_log2, out_scale = 1.0f;
 
   for (int s = 0; s < n_stages; ++s) {
     wait_younger_stages(min(NS - 2, n_stages - 1 - s));
@@ -820,7 +854,7 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       if (s == 0 || c_prev_len >= NS) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)  // the rows landed before this stage's tiles did
-          q[kk] = *reinterpret_cast<const u32x4*>(qbuf + k_read + (((kk * 4 + g) ^ c16) * 16));
+          q[kk] = *reinterpret_cast<const u32x4*>(qbuf + q_read + (((kk * 4 + g) ^ c16) * 16));
       } else {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
@@ -839,55 +873,115 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       m = kNegBig;
       l = 0.0f;
       c_ctx_first = s;
-    }
-
-    // ---- scores of the stage's 16 tokens: lane (head c16, tokens 4g .. 4g+3)
-    const char* st = ring + (s % NS) * kStageBytes;
-    f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const u32x4 kr = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ c16) * 16));
-      sc = Mfma<QT>::k32(kr, q[kk], sc);
-    }
-    const int tok0 = cc.st * T + 4 * g;
-    float sv[4];
-    bool over = false;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      sv[r] = tok0 + r < cc.L ? sc[r] * a.scale_log2 : -INFINITY;
-      over |= sv[r] > m + kSlack;
-    }
-    if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
-      const float mx = quad_rows_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
-      if (mx > m + kSlack) {
-        const float alpha = fast_exp2(m - mx);
-        m = mx;
-        l *= alpha;
-#pragma unroll
-        for (int mb = 0; mb < 8; ++mb) o[mb] *= alpha;
+      if constexpr (FP8) {  // per-KV-head scales, through the scalar cache like the lengths
+        score_scale = a.scale_log2 * as_f32(sload32(reinterpret_cast<const int32_t*>(a.k_scale) + kvh));
+        out_scale = as_f32(sload32(reinterpret_cast<const int32_t*>(a.v_scale) + kvh));
       }
     }
-    float pr[4];
+
+    const char* st = ring + (s % NS) * kStageBytes;
+    if constexpr (!FP8) {
+      // ---- scores of the stage's 16 tokens: lane (head c16, tokens 4g .. 4g+3)
+      f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      pr[r] = fast_exp2(sv[r] - m);
-      l += pr[r];
-    }
-    const u32x2 pb = {QT::pack(pr[0], pr[1]), QT::pack(pr[2], pr[3])};
-    // ---- O^T += V^T . P^T: lane c16 of a 16-lane group supplies the address of 4 dims of token
-    // row 4g + c16/4 and receives the 4 tokens of dim column 16 mb + c16
+      for (int kk = 0; kk < 4; ++kk) {
+        const u32x4 kr = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ c16) * 16));
+        sc = Mfma<QT>::k32(kr, q[kk], sc);
+      }
+      const int tok0 = cc.st * T + 4 * g;
+      float sv[4];
+      bool over = false;
 #pragma unroll
-    for (int mb = 0; mb < 8; ++mb) {
-      const s16x4 vt = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (lds_s16x4*)(st + v_read + (v_y ^ (mb << 5))));
-      o[mb] = Mfma<QT>::k16(vt, pb, o[mb]);
+      for (int r = 0; r < 4; ++r) {
+        sv[r] = tok0 + r < cc.L ? sc[r] * score_scale : -INFINITY;
+        over |= sv[r] > m + kSlack;
+      }
+      if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+        const float mx = quad_rows_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+        if (mx > m + kSlack) {
+          const float alpha = fast_exp2(m - mx);
+          m = mx;
+          l *= alpha;
+#pragma unroll
+          for (int mb = 0; mb < 8; ++mb) o[mb] *= alpha;
+        }
+      }
+      float pr[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pr[r] = fast_exp2(sv[r] - m);
+        l += pr[r];
+      }
+      const u32x2 pb = {QT::pack(pr[0], pr[1]), QT::pack(pr[2], pr[3])};
+      // ---- O^T += V^T . P^T: lane c16 of a 16-lane group supplies the address of 4 dims of token
+      // row 4g + c16/4 and receives the 4 tokens of dim column 16 mb + c16
+#pragma unroll
+      for (int mb = 0; mb < 8; ++mb) {
+        const s16x4 vt = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_s16x4*)(st + v_read + (v_y ^ (mb << 5))));
+        o[mb] = Mfma<QT>::k16(vt, pb, o[mb]);
+      }
+    } else {
+      // ---- scores of the stage's 32 tokens, two blocks of 16: lane (head c16, tokens 16 tb + 4g ..)
+      float sv[8];
+      bool over = false;
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb) {
+        f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+        const int tok = tb * 16 + c16;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const u32x2 k8 = *reinterpret_cast<const u32x2*>(
+              st + tok * RB + (((kk * 2 + (g >> 1)) ^ (tok & 7)) * 16) + (g & 1) * 8);
+          const u32x4 kr = {QT::template from_fp8x2<false>(k8[0]), QT::template from_fp8x2<true>(k8[0]),
+                            QT::template from_fp8x2<false>(k8[1]), QT::template from_fp8x2<true>(k8[1])};
+          sc = Mfma<QT>::k32(kr, q[kk], sc);
+        }
+        const int tok0 = cc.st * T + tb * 16 + 4 * g;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          sv[tb * 4 + r] = tok0 + r < cc.L ? sc[r] * score_scale : -INFINITY;
+          over |= sv[tb * 4 + r] > m + kSlack;
+        }
+      }
+      if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+        float mx = sv[0];
+#pragma unroll
+        for (int r = 1; r < 8; ++r) mx = fmaxf(mx, sv[r]);
+        mx = quad_rows_max(mx);
+        if (mx > m + kSlack) {
+          const float alpha = fast_exp2(m - mx);
+          m = mx;
+          l *= alpha;
+#pragma unroll
+          for (int mb = 0; mb < 8; ++mb) o[mb] *= alpha;
+        }
+      }
+      float pr[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        pr[r] = fast_exp2(sv[r] - m);
+        l += pr[r];
+      }
+      const u32x4 pb = {QT::pack(pr[0], pr[1]), QT::pack(pr[2], pr[3]), QT::pack(pr[4], pr[5]), QT::pack(pr[6], pr[7])};
+      // ---- O^T += V^T . P^T over the 32 tokens: the 8-bit transposing read hands lane c16 the
+      // eight tokens of its group's k-slots for dim column 16 mb + c16
+#pragma unroll
+      for (int mb = 0; mb < 8; ++mb) {
+        const i32x2 v8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(st + v8_read + (v8_y ^ (mb << 4))));
+        const u32x4 vt = {QT::template from_fp8x2<false>(static_cast<u32>(v8[0])),
+                          QT::template from_fp8x2<true>(static_cast<u32>(v8[0])),
+                          QT::template from_fp8x2<false>(static_cast<u32>(v8[1])),
+                          QT::template from_fp8x2<true>(static_cast<u32>(v8[1]))};
+        o[mb] = Mfma<QT>::k32(vt, pb, o[mb]);
+      }
     }
 
     // ---- end of a run: last stage of the context or of the worker's range
     const bool ctx_end = cc.st == cc.n_st - 1;
     if (ctx_end || s == n_stages - 1) {
       const float lsum = quad_rows_sum(l);
-      const float inv = 1.0f / lsum;
+      const float inv = out_scale / lsum;
       const float lse2 = m + fast_log2(lsum);
       const bool head_on = c16 < nh;
       const int hq = h0 + c16;
@@ -1058,11 +1152,11 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
 
 constexpr int kMfmaStages = 4;
 
-template <typename QT>
+template <typename QT, bool FP8>
 int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
   using Lay = MfmaLayout<kMfmaStages>;
   constexpr int D = 128;
-  auto kern = gqa_mfma_kernel<QT, kMfmaStages>;
+  auto kern = gqa_mfma_kernel<QT, FP8, kMfmaStages>;
   static const bool configured = [&] {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                               Lay::kPrefixOff + (kMaxBatch + 1) * 4);
@@ -1110,6 +1204,9 @@ template <typename QT, bool FP8>
 int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_only, size_t* need) {
   // lanes per token row: one 16-byte load per lane and row
   if constexpr (FP8) {
+    const bool out_aligned8 = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
+    if (head_dim == 128 && a.bs_shift >= 4 && out_aligned8 && use_mfma_kernel())
+      return launch_gqa_mfma<QT, true>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, true, 64, 4, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, true, 128, 8, 2>(a, wsb, s, plan_only, need);
@@ -1119,7 +1216,8 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
   } else {
     // (its epilogue stores 8 output bytes at a time)
     const bool out_aligned = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
-    if (head_dim == 128 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel()) return launch_gqa_mfma<QT>(a, wsb, s, plan_only, need);
+    if (head_dim == 128 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
+      return launch_gqa_mfma<QT, false>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, false, 64, 8, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, false, 128, 16, 4>(a, wsb, s, plan_only, need);
