@@ -1,21 +1,25 @@
 // Paged decode attention, GQA, for gfx950.
 //
-// Scheduling.  The context of every (sequence, KV-head block) is cut into items of 64
-// tokens; the items of the whole batch form one flat list ordered (sequence, head block,
-// item).  A fixed grid of persistent 256-thread workgroups (as many as fit on the chip at
-// once) splits that list into equal contiguous ranges, so every workgroup streams the same
-// number of KV bytes whatever the mix of context lengths, and a workgroup keeps its online
-// softmax state in registers for as long as it stays inside one (sequence, head block).
-// A run of items that covers a whole context writes the output directly; a run that
-// covers part of one (only the first and the last run of a workgroup can) writes a
-// normalised fp32 partial + log2-domain LSE, and a small merge kernel folds those.
+// Scheduling (both kernels of this file).  The context of every (sequence, KV-head block) is cut
+// into items; the items of the whole batch form one flat list ordered (sequence, head block,
+// item).  A fixed set of persistent workers splits that list into equal contiguous ranges, so
+// every worker streams the same number of KV bytes whatever the mix of context lengths, and a
+// worker keeps its online softmax state in registers for as long as it stays inside one
+// (sequence, head block).  A run of items that covers a whole context writes the output
+// directly; a run that covers part of one (only the first and the last run of a worker can)
+// writes a normalised fp32 partial + log2-domain LSE, and a small merge kernel folds those.
 // The item counts are prefix-summed inside every workgroup (no extra launch, no host read).
 //
-// Inner loop, per wavefront (the 4 wavefronts of a workgroup take steps round-robin):
+// gqa_mfma_kernel (head_dim 128, block size a power of two >= 16): worker = wavefront, item = 16
+// tokens (32 for fp8 pages); rows travel global memory -> LDS directly into a private ring per
+// wavefront and both products run on the matrix cores.  Its own comment below has the details.
+//
+// gqa_decode_kernel (every other shape): worker = workgroup, item = 64 tokens, the 4 wavefronts
+// of a workgroup take steps round-robin:
 //   * a token's [D] row of one KV head is read by LPT adjacent lanes with one 16-byte
 //     load each (64/LPT tokens per load instruction), K and V alike, so every load
-//     instruction covers whole contiguous rows of the [P, bs, Hkv, D] pages; two register
-//     tiles alternate so the next step's loads fly while the current step is reduced;
+//     instruction covers whole contiguous rows of the [P, bs, Hkv, D] pages; three register
+//     tiles rotate so the next steps' loads fly while the current step is reduced;
 //   * q.k is v_dot2 on packed 16-bit pairs into fp32, reduced over the LPT lanes by DPP
 //     row operations; all G query heads of the KV head reuse the same K registers;
 //   * p.v is v_dot2 as well: V words of two consecutive token rows are byte-permuted into
@@ -24,9 +28,9 @@
 //     rescaled only on steps where some maximum moved; rows and wavefronts are merged
 //     through LDS once per run;
 //   * fp8 pages are converted to 16-bit pairs in registers (exact), the per-head scales are
-//     folded into the score scale (K) and the output (V).
-// The page walk reads slot ids (page * bs + row) staged in LDS per 2048 tokens, so the
-// loop has no division and never touches table columns past ceil(L / bs).
+//     folded into the score scale (K) and the output (V);
+//   * the page walk reads slot ids (page * bs + row) staged in LDS per 2048 tokens, so the
+//     loop has no division and never touches table columns past ceil(L / bs).
 //
 // Arithmetic follows the block-table oracle of the reference,
 // xllm/core/kernels/npu/attention.cpp:26-78 (head h reads KV head h / group, explicit
@@ -475,24 +479,30 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
 // keeps its own softmax state, and never meets the other wavefronts of its workgroup after the
 // common item prefix sum, so there is no barrier anywhere in the streaming loop.
 //
-// Data path.  A stage is 16 tokens of one KV head: K rows (16 x 256 bytes) and V rows, 8 KB.
+// Data path.  A stage is 16 tokens of one KV head (32 for fp8 pages): K rows, then V rows, 8 KB.
 // Stages travel from global memory straight into the wavefront's private LDS ring
-// (global_load_lds_dwordx4, 16 adjacent lanes per row so every instruction reads whole
+// (global_load_lds_dwordx4, 16 adjacent lanes per 256-byte row so every instruction reads whole
 // contiguous rows), NS stages deep, NS - 1 in flight while one is consumed.  Within a row the
-// 16-byte chunks are XOR-swizzled (K by the row number, V by twice its low two bits) so that both
-// operand reads below touch every LDS bank once.
+// 16-byte chunks are XOR-swizzled so that both operand reads below touch every LDS bank once.
 //   S^T[tok, head] = K[tok, 128] . Q^T[128, head]   v_mfma_f32_16x16x32: A = K rows read from LDS
 //                                                   (16 bytes per lane), B = Q^T resident in registers
 //   O^T[dim, head] += V^T[dim, tok] . P^T[tok, head] v_mfma_f32_16x16x16: A = V^T through the
 //                                                   transposing LDS read, B = P^T taken from the
 //                                                   S^T accumulator registers as they are
+// fp8 pages are converted to 16-bit after the LDS read (exact); their V^T comes through the 8-bit
+// transposing read (within 16 lanes, result lane i element j = input lane 2j + i/8, element
+// i%8) and P.V runs on the 16x16x32 MFMA over both score blocks of the stage.
 // Up to 16 query heads of the KV head ride in the MFMA columns (heads past the group are zero
 // columns), so a lane owns one head: its running maximum and sum are plain per-lane scalars.
 // The maximum only moves when a score exceeds it by more than kSlack (log2 units).
 //
 // Nothing in the loop waits on a register load from global memory: such a wait would also wait
-// for every younger stage in flight.  Page ids come through the same LDS path one item ahead,
-// the Q rows of a run just before its first stage, sequence lengths through the scalar cache.
+// for every younger stage in flight (the counter is in order).  Page-table entries (64 at a
+// time: the current chunk, the next one, and the first one of the next context), the Q rows of
+// the next context and the stages all take the LDS path and are covered by one explicit wait per
+// stage; sequence lengths and fp8 scales come through the scalar cache.  Loads that write
+// registers are never issued from inline assembly: the register allocator does not know they
+// are pending and may hand their destination to something else.
 constexpr float kSlack = 8.0f;
 constexpr int kStageBytes = 8192;  // K rows then V rows: 16 tokens of 16-bit pages, 32 of fp8 pages
 constexpr int kMfmaHeads = 16;                        // head columns of one MFMA
