@@ -539,11 +539,11 @@ struct Mfma<FP16> {
 // lds_addr is wave-uniform and travels in M0.
 __device__ __forceinline__ void dma16(const void* gptr, u32 lds_addr) {
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
 }
 __device__ __forceinline__ void dma4(const void* gptr, u32 lds_addr) {
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gptr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gptr) : "memory");
 }
 // Same as dma16 with a wave-uniform 64-bit base in SGPRs plus a 32-bit per-lane byte offset.
 __device__ __forceinline__ void dma16_row(uint64_t base, u32 lane_off, u32 lds_addr) {
@@ -551,7 +551,7 @@ __device__ __forceinline__ void dma16_row(uint64_t base, u32 lane_off, u32 lds_a
   const u32 lo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(base)));
   const u32 hi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(base >> 32)));
   const uint64_t sb = (static_cast<uint64_t>(hi) << 32) | lo;
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(lane_off), "s"(sb) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(lane_off), "s"(sb) : "memory");
 }
 // Wait until at most 8 * stages of the wavefront's vector memory operations are outstanding.
 __device__ __forceinline__ void wait_younger_stages(int stages) {

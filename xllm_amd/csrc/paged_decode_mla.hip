@@ -105,11 +105,11 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 // (lds_addr is wave-uniform; it travels in M0).
 __device__ __forceinline__ void dma16(const void* gptr, u32 lds_addr) {
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
 }
 // Same with a wave-uniform 64-bit row base in SGPRs plus a 32-bit per-lane byte offset.
 __device__ __forceinline__ void dma16_row(uint64_t row_base, u32 lane_off, u32 lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
                : "memory");
 }
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -416,6 +416,364 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Variant with 16 heads per wavefront, no per-tile exchange and a four-deep ring of 32-token
+// sub-tiles.
+//
+// Workgroup = 512 threads = 8 wavefronts = 64 heads: wavefront (hb, th) owns heads 16hb..16hb+15
+// and the token half th (16 tokens) of every 32-token sub-tile, for BOTH products:
+//   S^T[tok, head] = K[tok, 576] . Q^T[576, head]    v_mfma_f32_16x16x32_bf16, A = K rows of its tokens
+//                                                    from the LDS sub-tile, B = Q^T in 72 VGPRs
+//   O^T[dim, head] += V^T[dim, tok] . P^T[tok, head]  v_mfma_f32_16x16x16_bf16 over its 16 tokens and all
+//                                                    512 dims, A = V^T through the transposing LDS read,
+//                                                    B = P^T taken from the S^T accumulator registers
+// so a lane owns one head, its softmax state is a pair of per-lane scalars, and the two wavefronts of
+// a head block only meet at the end of a run, where their (max, sum, O) states are folded through
+// LDS.  One barrier per sub-tile (sub-tile landed / oldest ring slot released).  With at most 256
+// registers per wavefront two wavefronts share a SIMD, so one's softmax overlaps the other's MFMAs.
+//
+// Three sub-tiles are in flight while one is consumed: with a single tile of prefetch the loop ran
+// at the latency of a tile fetch.  As in the GQA matrix-core kernel nothing in the loop waits on a
+// register load (the in-order counter would drain the ring): page-table entries come through the
+// LDS path in chunks of 64, fetched by wavefront 0 at least 32 sub-tiles ahead.
+//
+// Rows are 1184 bytes apart in LDS and the 16-byte chunks of a row are XOR-ed with bit 2 of the row
+// number: the 16-byte operand reads (8 consecutive rows per cycle) and the transposing reads
+// (4 rows x 32 bytes per cycle) then both touch every LDS bank once.
+constexpr int kRow16 = kRowBytes + 32;
+constexpr int kSubTok = 32;                      // tokens per sub-tile
+constexpr int kRing16 = 4;                       // ring slots
+constexpr int kSubBytes = kSubTok * kRow16;      // 37888
+constexpr int kThreads16 = 512;
+constexpr int kPage16Off = kRing16 * kSubBytes;  // LDS: ring | page-table chunks [2][64] | prefix
+constexpr int kPrefix16Off = kPage16Off + 2 * kWave * 4;
+constexpr int kKSteps32 = kDK / 32;              // 18 k-steps of the 16x16x32 MFMA
+constexpr int kAhead = 4;                        // LDS operand reads in flight ahead of the MFMAs
+
+__device__ __forceinline__ float quad_rows_max(float x) {  // over lanes l, l ^ 16, l ^ 32, l ^ 48
+  auto t = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
+  x = fmaxf(as_f32(t[0]), as_f32(t[1]));
+  auto u = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
+  return fmaxf(as_f32(u[0]), as_f32(u[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float x) {
+  auto t = __builtin_amdgcn_permlane16_swap(as_u32(x), as_u32(x), false, false);
+  x = as_f32(t[0]) + as_f32(t[1]);
+  auto u = __builtin_amdgcn_permlane32_swap(as_u32(x), as_u32(x), false, false);
+  return as_f32(u[0]) + as_f32(u[1]);
+}
+// 4 bytes per lane from global memory straight into LDS at lds_addr + lane * 4
+__device__ __forceinline__ void dma4(const void* gptr, u32 lds_addr) {
+  const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gptr) : "memory");
+}
+// Four adjacent cache rows (1152 bytes apart) of one page into four LDS rows (kRow16 apart): per
+// row the 1024 latent bytes with all lanes, then the 128 rope bytes with the lanes of `rope`.
+// The instruction offset is added to the global AND to the LDS address (LDS address = M0 +
+// offset + lane * 16), so M0 only carries the difference of the two row strides.
+__device__ __forceinline__ void dma_rows4(uint64_t base, u32 lane_off, u32 lds_addr, bool rope) {
+  constexpr int kPad = kRow16 - kRowBytes;  // 32
+#define XLLM_DMA(lds, gbase, m0_add, goff)                                                               \
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4" ::"s"(lds), \
+               "v"(lane_off), "s"(gbase), "n"(m0_add), "n"(goff)                                         \
+               : "memory", "scc")
+  // instruction offsets reach 4095: rows 2 and 3 go through a second base
+  const uint64_t base2 = base + 2 * kRowBytes;
+  const u32 lds2 = lds_addr + 2 * kRow16;
+  XLLM_DMA(lds_addr, base, 0, 0);
+  XLLM_DMA(lds_addr, base, kPad, kRowBytes);
+  XLLM_DMA(lds2, base2, 0, 0);
+  XLLM_DMA(lds2, base2, kPad, kRowBytes);
+  if (rope) {
+    XLLM_DMA(lds_addr, base, 0, kDL * 2);
+    XLLM_DMA(lds_addr, base, kPad, kRowBytes + kDL * 2);
+    XLLM_DMA(lds2, base2, 0, kDL * 2);
+    XLLM_DMA(lds2, base2, kPad, kRowBytes + kDL * 2);
+  }
+#undef XLLM_DMA
+}
+// Wait until at most 8 * subs of the wavefront's vector memory operations are outstanding
+// (a wavefront issues 8 loads per sub-tile).
+__device__ __forceinline__ void wait_younger_subs(int subs) {
+  if (subs <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else if (subs == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+}
+
+__global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
+  extern __shared__ __align__(16) char smem[];
+  int* prefix = reinterpret_cast<int*>(smem + kPrefix16Off);
+  const int* pagebuf = reinterpret_cast<const int*>(smem + kPage16Off);
+  int* tmp = reinterpret_cast<int*>(smem);  // prologue only
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hb16 = wave >> 1;   // 16-head block of the wavefront
+  const int th = wave & 1;      // its token half of every sub-tile
+  const int c16 = lane & 15;    // MFMA row / column index owned by the lane
+  const int g = lane >> 4;      // MFMA k-group of the lane
+  const int H = a.n_heads;
+
+  // block id -> (team, head block): members of a team are 8 ids apart (same XCD)
+  const int xcd = blockIdx.x & 7;
+  const int y = blockIdx.x >> 3;
+  const int hb64 = y % a.n_hb;
+  const int team = (y / a.n_hb) * 8 + xcd;
+  const int head = hb64 * kHeadsPerWg + hb16 * 16 + c16;
+  const bool head_ok = head < H;
+  const bool wave_ok = hb64 * kHeadsPerWg + hb16 * 16 < H;
+
+  // ---- tile prefix over the batch (every workgroup computes it; no extra launch)
+  {
+    const int per = (a.batch + kThreads16 - 1) / kThreads16;
+    const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
+    int local = 0;
+    for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
+    tmp[tid] = local;
+    __syncthreads();
+    int excl = 0;
+    for (int j = 0; j < tid; ++j) excl += tmp[j];
+    for (int b = lo; b < hi; ++b) {
+      prefix[b] = excl;
+      excl += tiles_of(a.seq_lens[b]);
+    }
+    if (lo < hi && hi == a.batch) prefix[a.batch] = excl;
+    __syncthreads();
+  }
+  const int64_t total = prefix[a.batch];
+  if (blockIdx.x == 0)
+    for (int i = tid; i <= a.batch; i += kThreads16) a.ws_prefix[i] = prefix[i];
+  if (total == 0) return;
+  int64_t cur = team_start(team, total, a.n_teams);
+  const int64_t end = team_start(team + 1, total, a.n_teams);
+  bool first_run = true;
+
+  const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
+  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + kPage16Off);
+  // per-lane constants of the operand reads (byte offsets inside a sub-tile)
+  //   K: row th*16 + c16, 16-byte chunk kk*4 + g XOR-ed with bit 2 of the row: + kk * 64
+  const int k_row0 = (th * 16 + c16) * kRow16 + ((g ^ ((c16 >> 2) & 1)) * 16);
+  //   V: lane c16 of a 16-lane group addresses 4 dims (8 bytes) of token row th*16 + 4g + c16/4,
+  //      chunk 2 mb + (c16 & 3) / 2 XOR-ed with bit 2 of the row (= g & 1): + mb * 32
+  const int v_row0 = (th * 16 + 4 * g + (c16 >> 2)) * kRow16 + ((((c16 & 3) >> 1) ^ (g & 1)) * 16) + (c16 & 1) * 8;
+  // tile loads: this wavefront moves rows wave*4 .. +3 of a sub-tile; bit 2 of those rows is wave & 1
+  const u32 lane_off = (lane ^ (wave & 1)) * 16;
+
+  while (cur < end) {
+    int lo = 0, hi = a.batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (prefix[mid] <= cur) lo = mid; else hi = mid;
+    }
+    const int b = __builtin_amdgcn_readfirstlane(lo);
+    const int n_tiles_seq = prefix[b + 1] - prefix[b];
+    const int tile0 = static_cast<int>(cur - prefix[b]);
+    const int run_tiles = static_cast<int>(min<int64_t>(n_tiles_seq - tile0, end - cur));
+    const bool complete = tile0 == 0 && run_tiles == n_tiles_seq;
+    cur += run_tiles;
+    const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
+    const int L = __builtin_amdgcn_readfirstlane(a.seq_lens[b]);
+    const int t_begin = tile0 * kTile;
+    const int t_end = min(L, (tile0 + run_tiles) * kTile);
+    const int n_sub = (t_end - t_begin + kSubTok - 1) / kSubTok;
+    const int n_pages = (L + a.block_size - 1) >> a.bs_shift;
+
+    // Q^T operand: lane (head c16, k-group g) keeps dims kk*32 + g*8 .. +8 of every k-step
+    u32x4 q[kKSteps32];
+    {
+      const char* qn = a.q_nope + (static_cast<int64_t>(b) * H + head) * kDL * 2;
+      const char* qp = a.q_pe + (static_cast<int64_t>(b) * H + head) * kDR * 2;
+#pragma unroll
+      for (int kk = 0; kk < kKSteps32; ++kk) {
+        u32x4 x = {0u, 0u, 0u, 0u};
+        if (head_ok)
+          x = kk < kDL / 32 ? ldg16(qn + (kk * 32 + g * 8) * 2) : ldg16(qp + ((kk - kDL / 32) * 32 + g * 8) * 2);
+        q[kk] = x;
+      }
+    }
+    f32x4 o[32];  // O^T blocks: dims mb*16 + 4g + r, head c16
+#pragma unroll
+    for (int i = 0; i < 32; ++i) o[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = kNegBig, l = 0.0f;
+
+    // 64 entries of the page table from page 64 ck on (the tail repeats the last page) -> chunk buffer ck & 1
+    auto issue_chunk = [&](int ck) {
+      dma4(pages + min(ck * kWave + lane, n_pages - 1), page_lds + (ck & 1) * kWave * 4);
+    };
+    int ck_cur = (t_begin >> a.bs_shift) >> 6;  // chunk of the sub-tile being issued
+    // Rows go from global memory straight into LDS: one 64-lane load moves the 1024 latent bytes
+    // of a row, a second one with 8 lanes the 128 rope bytes; 8 loads per wavefront and sub-tile.
+    auto issue_sub = [&](int sub) {
+      const int tok0 = t_begin + sub * kSubTok + wave * 4;  // block_size >= 16: the 4 rows share a page
+      const u32 dst = __builtin_amdgcn_readfirstlane(lds_base + (sub & (kRing16 - 1)) * kSubBytes + wave * 4 * kRow16);
+      const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
+      const int ck = (min(tok0, L - 1) >> a.bs_shift) >> 6;
+      if (ck != ck_cur) {  // first sub-tile of a chunk: wavefront 0 fetches the one after it
+        ck_cur = ck;
+        if (wave == 0 && (ck + 1) * kWave < n_pages) issue_chunk(ck + 1);
+      }
+      if (tok0 + 3 < L) {
+        int page = __builtin_amdgcn_readfirstlane(pagebuf[(ck & 1) * kWave + ((tok0 >> a.bs_shift) & 63)]);
+        page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
+        const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tok0 & (a.block_size - 1))) * kRowBytes;
+        const u32 lo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row)));
+        const u32 hi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row >> 32)));
+        const uint64_t sb = (static_cast<uint64_t>(hi) << 32) | lo;
+        // the 4 rows are adjacent in the page: one base, the row offset in the instruction
+        dma_rows4(sb, lane_off, dst, lane < kDR * 2 / 16);
+      } else {  // ragged end of the context: rows past it repeat the last valid row
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tok = min(tok0 + i, L - 1);
+          int page = __builtin_amdgcn_readfirstlane(pagebuf[(((tok >> a.bs_shift) >> 6) & 1) * kWave + ((tok >> a.bs_shift) & 63)]);
+          page = max(0, min(page, a.num_blocks - 1));
+          const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tok & (a.block_size - 1))) * kRowBytes;
+          dma16_row(row, lane_off, dst + i * kRow16);
+          if (lane < kDR * 2 / 16) dma16_row(row + kDL * 2, lane_off, dst + i * kRow16 + kDL * 2);
+        }
+      }
+    };
+
+    // make the compiler wait for the Q loads here, not inside the loop
+#pragma unroll
+    for (int kk = 0; kk < kKSteps32; ++kk) asm volatile("" : "+v"(q[kk]));
+    __syncthreads();  // the previous run no longer reads the ring, the chunks or the fold buffers
+    if (wave == 0) {
+      issue_chunk(ck_cur);
+      if ((ck_cur + 1) * kWave < n_pages) issue_chunk(ck_cur + 1);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    for (int sub = 0; sub < kRing16 - 1 && sub < n_sub; ++sub) issue_sub(sub);
+
+    for (int sub = 0; sub < n_sub; ++sub) {
+      wait_younger_subs(min(kRing16 - 2, n_sub - 1 - sub));
+      __syncthreads();  // this sub-tile has landed in LDS; every wavefront is past the previous one
+      // Wavefronts 0-3 issue their rows of sub-tile sub + 3 (into the slot released just now)
+      // before they compute, wavefronts 4-7 (the second wavefront of each SIMD) after: the phases
+      // of the two groups then interleave instead of all eight hitting LDS at the same time.
+      if (wave < 4 && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
+      const char* kb = smem + (sub & (kRing16 - 1)) * kSubBytes;
+      if (wave_ok) {
+        // ---- S^T of the wavefront's 16 tokens: lane (head c16, tokens 4g + r); two accumulator chains
+        f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+        const char* ka = kb + k_row0;
+        __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the Q.K reads only
+#pragma unroll
+        for (int kk = 0; kk < kKSteps32; kk += 2) {
+          const u32x4 x0 = *reinterpret_cast<const u32x4*>(ka + kk * 64);
+          const u32x4 x1 = *reinterpret_cast<const u32x4*>(ka + kk * 64 + 64);
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x0), __builtin_bit_cast(bf16x8, q[kk]), s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x1), __builtin_bit_cast(bf16x8, q[kk + 1]), s1, 0, 0, 0);
+        }
+        // pipeline the LDS operand reads kAhead MFMAs ahead of their use
+        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+        for (int i = 0; i < kKSteps32 - kAhead; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        float sv[4];
+        const int tok_base = t_begin + sub * kSubTok + th * 16 + 4 * g;
+        bool over = false;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          sv[r] = tok_base + r < L ? (s0[r] + s1[r]) * a.scale_log2 : -INFINITY;
+          over |= sv[r] > m + kSlack;
+        }
+        if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+          const float mx = quad_rows_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+          if (mx > m + kSlack) {
+            const float alpha = fast_exp2(m - mx);
+            m = mx;
+            l *= alpha;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) o[i] *= alpha;
+          }
+        }
+        float p[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          p[r] = fast_exp2(sv[r] - m);
+          l += p[r];
+        }
+        const u32x2 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3])};
+        const s16x4 pb = __builtin_bit_cast(s16x4, pbw);
+        // ---- O^T += V^T . P^T over the 16 tokens and all 512 dims.  The transposing LDS load works on
+        // groups of 16 lanes: lane p of a group supplies the address of 4 dims of token row p/4 and
+        // receives the 4 tokens of dim column p.
+        const char* va = kb + v_row0;
+        __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the P.V reads only
+#pragma unroll
+        for (int mb = 0; mb < 32; ++mb) {
+          const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
+          o[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb, o[mb], 0, 0, 0);
+        }
+        // pipeline the transposing reads kAhead MFMAs ahead of their use
+        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+        for (int i = 0; i < 32 - kAhead; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (wave >= 4 && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
+    }
+
+    // ---- end of the run: the two token halves of a head block are folded through LDS (the ring
+    // is free now); the th = 0 wavefront writes the result
+    const float l_half = quad_rows_sum(l);
+    __syncthreads();  // every wavefront is past its last sub-tile
+    float* fold = reinterpret_cast<float*>(smem) + hb16 * (32 * 4 * kWave + 2 * 16);
+    if (wave_ok && th == 1) {
+#pragma unroll
+      for (int mb = 0; mb < 32; ++mb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) fold[(mb * 4 + r) * kWave + lane] = o[mb][r];
+      if (g == 0) {
+        fold[32 * 4 * kWave + c16] = m;
+        fold[32 * 4 * kWave + 16 + c16] = l_half;
+      }
+    }
+    __syncthreads();
+    if (wave_ok && th == 0) {
+      const float m1 = fold[32 * 4 * kWave + c16], l1 = fold[32 * 4 * kWave + 16 + c16];
+      const float m_all = fmaxf(m, m1);
+      const float f0 = fast_exp2(m - m_all), f1 = fast_exp2(m1 - m_all);
+      const float lsum = l_half * f0 + l1 * f1;
+      const float inv = 1.0f / lsum;
+      const float w0 = f0 * inv, w1 = f1 * inv;
+#pragma unroll
+      for (int mb = 0; mb < 32; ++mb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[mb][r] = o[mb][r] * w0 + fold[(mb * 4 + r) * kWave + lane] * w1;
+      const float lse2 = m_all + fast_log2(lsum);
+      const int64_t ps = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H + head;
+      if (head_ok && complete) {
+        char* op = a.out + ((static_cast<int64_t>(b) * H + head) * kDL + 4 * g) * 2;
+#pragma unroll
+        for (int mb = 0; mb < 32; ++mb) {
+          const u32x2 w = {BF16::pack(o[mb][0], o[mb][1]), BF16::pack(o[mb][2], o[mb][3])};
+          *reinterpret_cast<u32x2*>(op + mb * 32) = w;
+        }
+      }
+      if (head_ok && !complete) {
+        float* wp = a.ws_out + ps * kDL + 4 * g;
+#pragma unroll
+        for (int mb = 0; mb < 32; ++mb) *reinterpret_cast<f32x4*>(wp + mb * 16) = o[mb];
+      }
+      if (head_ok && g == 0 && complete && a.lse != nullptr) a.lse[b * H + head] = lse2 * kLn2;
+      if (head_ok && g == 0 && !complete) a.ws_lse[ps] = lse2;
+    }
+    first_run = false;
+  }
+}
+
 // Merge of the partials of contexts that span several teams; also writes the output of
 // empty sequences.  One workgroup per (head, sequence).
 __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
@@ -535,11 +893,22 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     return XLLM_MI355_EWORKSPACE;
 
   const int n_hb = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
+  static const bool pairs_env = [] {  // tuning knob: "pairs" selects the 32-heads-per-wavefront kernel
+    const char* e = getenv("XLLM_MI355_MLA_KERNEL");
+    return e != nullptr && e[0] == 'p';
+  }();
+  // the 16-heads-per-wavefront kernel looks pages up per group of 16 tokens
+  const bool pairs = pairs_env || block_size < 16 || (block_size & (block_size - 1)) != 0;
   static bool attr_set = false;
-  const size_t smem = kPrefixOff + (kMaxBatchMla + 1) * 4;
+  const size_t smem = pairs ? kPrefixOff + (kMaxBatchMla + 1) * 4 : kPrefix16Off + (kMaxBatchMla + 1) * 4;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       static_cast<int>(kPrefixOff + (kMaxBatchMla + 1) * 4));
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode16_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(kPrefix16Off + (kMaxBatchMla + 1) * 4));
     if (e != hipSuccess) return static_cast<int>(e);
     attr_set = true;
   }
@@ -570,7 +939,10 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * n_heads * kDL;
 
     const bool timed = profile_begin(stream);
-    mla_decode_kernel<<<dim3(static_cast<unsigned>(a.n_teams * n_hb)), kMlaThreads, smem, stream>>>(a);
+    if (pairs)
+      mla_decode_kernel<<<dim3(static_cast<unsigned>(a.n_teams * n_hb)), kMlaThreads, smem, stream>>>(a);
+    else
+      mla_decode16_kernel<<<dim3(static_cast<unsigned>(a.n_teams * n_hb)), kThreads16, smem, stream>>>(a);
     if (timed) profile_end(stream);
     int rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
