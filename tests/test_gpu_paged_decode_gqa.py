@@ -194,6 +194,24 @@ def test_whole_contexts_in_one_workgroup_every_group_size(device):
         _check_config(cfg, 600 + D, device)
 
 
+def test_block_sizes_and_page_table_chunks_of_both_kernels(device):
+    # head_dim 128: block sizes >= 16 that are powers of two take the matrix-core kernel (which walks
+    # the page table in chunks of 64 pages), the others the dot-product kernel
+    for bs in (1, 8, 16, 24, 32, 64, 256):
+        cfg = workloads.DecodeConfig(f"bs{bs}", 3, 8, 2, 128, bs, 30, 900)
+        _check_config(cfg, 700 + bs, device)
+    # contexts that end just before, at and after chunk (1024 tokens at block 16) and stage boundaries
+    for i, L in enumerate((1023, 1024, 1025, 1040, 2047, 2048, 2049, 5000)):
+        cfg = workloads.DecodeConfig(f"chunks{L}", 1, 4, 1, 128, 16, L, L)
+        _check_config(cfg, 800 + i, device)
+    for i, L in enumerate((2047, 2048, 2049, 2080)):
+        cfg = workloads.DecodeConfig(f"chunks_fp8_{L}", 1, 4, 1, 128, 16, L, L, cache_dtype="fp8")
+        _check_fp8(cfg, 850 + i, device)
+    # more than 16 query heads per KV head: two head blocks per KV head
+    cfg = workloads.DecodeConfig("group24", 2, 48, 2, 128, 16, 100, 600)
+    _check_config(cfg, 900, device)
+
+
 def test_empty_sequence_and_argument_errors(device):
     cfg = workloads.DecodeConfig("e", 3, 8, 2, 128, 16, 10, 50)
     inp = workloads.make_inputs(cfg, 2)

@@ -83,6 +83,18 @@ def test_block_sizes_other_than_64_and_long_context_splits(device):
     _check(_mla_cfg("long", 1, 128, 6000, 9000), 6, device)
 
 
+def test_small_and_odd_block_sizes_and_page_table_chunks(device):
+    # block sizes below 16 or not a power of two take the kernel with the per-tile exchange
+    _check(_mla_cfg("bs8", 2, 32, 40, 500, bs=8), 11, device)
+    _check(_mla_cfg("bs24", 2, 16, 40, 500, bs=24), 12, device)
+    # block 16: the page table is walked in chunks of 64 pages = 1024 tokens; contexts that end
+    # just before, at and after chunk and sub-tile boundaries
+    for i, L in enumerate((1023, 1024, 1025, 1056, 2047, 2049, 3100)):
+        _check(_mla_cfg(f"chunks{L}", 1, 16, L, L, bs=16), 20 + i, device)
+    # many short sequences: workgroups own several whole contexts
+    _check(_mla_cfg("short", 96, 16, 1, 200, bs=16), 13, device)
+
+
 def test_shard_merge_equals_full_decode(device):
     # ArtificialShardMergeMatchesFullCacheDecode (dcp_attention_merge_test.cpp:146-224): rtol/atol 1e-2, 1e-3
     cfg = _mla_cfg("merge", 4, 128, 256, 2000)
