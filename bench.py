@@ -253,7 +253,7 @@ def main():
         achieved = flops / (kernel_ms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
                     "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic,
-                    "kernel": "mla_decode_kernel", "kernel_ms": kernel_ms, "algorithmic_flops": flops,
+                    "kernel": "mla_decode16_kernel", "kernel_ms": kernel_ms, "algorithmic_flops": flops,
                     "algorithmic_bytes": nbytes,
                     "hbm_gbs": nbytes / (kernel_ms * 1e-3) / 1e9}
     else:
@@ -261,7 +261,7 @@ def main():
         achieved = nbytes / (kernel_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                    "kernel": "gqa_decode_kernel" if fp8 or cfg.head_dim != 128 else "gqa_mfma_kernel",
+                    "kernel": "gqa_mfma_kernel" if cfg.head_dim == 128 else "gqa_decode_kernel",
                     "kernel_ms": kernel_ms, "algorithmic_bytes": nbytes}
 
     # the same number of bytes through the plain read kernel: the rate this GPU sustains at this size
