@@ -417,20 +417,21 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Variant with 16 heads per wavefront, no per-tile exchange and a four-deep ring of 32-token
-// sub-tiles.
+// Main kernel: 16 heads per wavefront, nothing exchanged between wavefronts, and a four-deep ring
+// of 32-token sub-tiles.
 //
-// Workgroup = 512 threads = 8 wavefronts = 64 heads: wavefront (hb, th) owns heads 16hb..16hb+15
-// and the token half th (16 tokens) of every 32-token sub-tile, for BOTH products:
-//   S^T[tok, head] = K[tok, 576] . Q^T[576, head]    v_mfma_f32_16x16x32_bf16, A = K rows of its tokens
-//                                                    from the LDS sub-tile, B = Q^T in 72 VGPRs
-//   O^T[dim, head] += V^T[dim, tok] . P^T[tok, head]  v_mfma_f32_16x16x16_bf16 over its 16 tokens and all
-//                                                    512 dims, A = V^T through the transposing LDS read,
-//                                                    B = P^T taken from the S^T accumulator registers
-// so a lane owns one head, its softmax state is a pair of per-lane scalars, and the two wavefronts of
-// a head block only meet at the end of a run, where their (max, sum, O) states are folded through
-// LDS.  One barrier per sub-tile (sub-tile landed / oldest ring slot released).  With at most 256
-// registers per wavefront two wavefronts share a SIMD, so one's softmax overlaps the other's MFMAs.
+// Workgroup = 512 threads = 8 wavefronts = 128 heads: wavefront w owns heads 16w..16w+15 for all
+// 32 tokens of every sub-tile and all 512 output dims, with v_mfma_f32_16x16x32_bf16 for BOTH
+// products:
+//   S^T[tok, head] = K[tok, 576] . Q^T[576, head]    2 token blocks x 18 k-steps, A = K rows from the
+//                                                    LDS sub-tile, B = Q^T in 72 VGPRs
+//   O^T[dim, head] += V^T[dim, tok] . P^T[tok, head]  32 dim blocks over the 32 tokens, A = V^T through the
+//                                                    transposing LDS read, B = P^T taken from the S^T
+//                                                    accumulator registers
+// so a lane owns one head, its softmax state is a pair of per-lane scalars and a wavefront writes
+// its own heads at the end of a run.  One barrier per sub-tile (sub-tile landed / oldest ring
+// slot released).  With at most 256 registers per wavefront two wavefronts share a SIMD, so
+// one's softmax overlaps the other's MFMAs.
 //
 // Three sub-tiles are in flight while one is consumed: with a single tile of prefetch the loop ran
 // at the latency of a tile fetch.  As in the GQA matrix-core kernel nothing in the loop waits on a
@@ -445,6 +446,7 @@ constexpr int kSubTok = 32;                      // tokens per sub-tile
 constexpr int kRing16 = 4;                       // ring slots
 constexpr int kSubBytes = kSubTok * kRow16;      // 37888
 constexpr int kThreads16 = 512;
+constexpr int kHeadsPerWg16 = 128;
 constexpr int kPage16Off = kRing16 * kSubBytes;  // LDS: ring | page-table chunks [2][64] | prefix
 constexpr int kPrefix16Off = kPage16Off + 2 * kWave * 4;
 constexpr int kKSteps32 = kDK / 32;              // 18 k-steps of the 16x16x32 MFMA
@@ -509,8 +511,6 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int hb16 = wave >> 1;   // 16-head block of the wavefront
-  const int th = wave & 1;      // its token half of every sub-tile
   const int c16 = lane & 15;    // MFMA row / column index owned by the lane
   const int g = lane >> 4;      // MFMA k-group of the lane
   const int H = a.n_heads;
@@ -518,11 +518,11 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
   // block id -> (team, head block): members of a team are 8 ids apart (same XCD)
   const int xcd = blockIdx.x & 7;
   const int y = blockIdx.x >> 3;
-  const int hb64 = y % a.n_hb;
+  const int hb128 = y % a.n_hb;
   const int team = (y / a.n_hb) * 8 + xcd;
-  const int head = hb64 * kHeadsPerWg + hb16 * 16 + c16;
+  const int head = hb128 * kHeadsPerWg16 + wave * 16 + c16;
   const bool head_ok = head < H;
-  const bool wave_ok = hb64 * kHeadsPerWg + hb16 * 16 < H;
+  const bool wave_ok = hb128 * kHeadsPerWg16 + wave * 16 < H;
 
   // ---- tile prefix over the batch (every workgroup computes it; no extra launch)
   {
@@ -552,11 +552,11 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
   const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
   const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + kPage16Off);
   // per-lane constants of the operand reads (byte offsets inside a sub-tile)
-  //   K: row th*16 + c16, 16-byte chunk kk*4 + g XOR-ed with bit 2 of the row: + kk * 64
-  const int k_row0 = (th * 16 + c16) * kRow16 + ((g ^ ((c16 >> 2) & 1)) * 16);
-  //   V: lane c16 of a 16-lane group addresses 4 dims (8 bytes) of token row th*16 + 4g + c16/4,
+  //   K: row c16 (+ 16 for the second token block), 16-byte chunk kk*4 + g XOR-ed with bit 2 of the row: + kk * 64
+  const int k_row0 = c16 * kRow16 + ((g ^ ((c16 >> 2) & 1)) * 16);
+  //   V: lane c16 of a 16-lane group addresses 4 dims (8 bytes) of token row 4g + c16/4 (+ 16),
   //      chunk 2 mb + (c16 & 3) / 2 XOR-ed with bit 2 of the row (= g & 1): + mb * 32
-  const int v_row0 = (th * 16 + 4 * g + (c16 >> 2)) * kRow16 + ((((c16 & 3) >> 1) ^ (g & 1)) * 16) + (c16 & 1) * 8;
+  const int v_row0 = (4 * g + (c16 >> 2)) * kRow16 + ((((c16 & 3) >> 1) ^ (g & 1)) * 16) + (c16 & 1) * 8;
   // tile loads: this wavefront moves rows wave*4 .. +3 of a sub-tile; bit 2 of those rows is wave & 1
   const u32 lane_off = (lane ^ (wave & 1)) * 16;
 
@@ -638,7 +638,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
     // make the compiler wait for the Q loads here, not inside the loop
 #pragma unroll
     for (int kk = 0; kk < kKSteps32; ++kk) asm volatile("" : "+v"(q[kk]));
-    __syncthreads();  // the previous run no longer reads the ring, the chunks or the fold buffers
+    __syncthreads();  // the previous run no longer reads the ring or the chunks
     if (wave == 0) {
       issue_chunk(ck_cur);
       if ((ck_cur + 1) * kWave < n_pages) issue_chunk(ck_cur + 1);
@@ -656,36 +656,41 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
       if (wave < 4 && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
       const char* kb = smem + (sub & (kRing16 - 1)) * kSubBytes;
       if (wave_ok) {
-        // ---- S^T of the wavefront's 16 tokens: lane (head c16, tokens 4g + r); two accumulator chains
+        // ---- S^T of the sub-tile, two blocks of 16 tokens: lane (head c16, tokens 16 tb + 4g + r)
         f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
         const char* ka = kb + k_row0;
         __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the Q.K reads only
 #pragma unroll
-        for (int kk = 0; kk < kKSteps32; kk += 2) {
+        for (int kk = 0; kk < kKSteps32; ++kk) {
           const u32x4 x0 = *reinterpret_cast<const u32x4*>(ka + kk * 64);
-          const u32x4 x1 = *reinterpret_cast<const u32x4*>(ka + kk * 64 + 64);
+          const u32x4 x1 = *reinterpret_cast<const u32x4*>(ka + 16 * kRow16 + kk * 64);
           s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x0), __builtin_bit_cast(bf16x8, q[kk]), s0, 0, 0, 0);
-          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x1), __builtin_bit_cast(bf16x8, q[kk + 1]), s1, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x1), __builtin_bit_cast(bf16x8, q[kk]), s1, 0, 0, 0);
         }
         // pipeline the LDS operand reads kAhead MFMAs ahead of their use
         __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
-        for (int i = 0; i < kKSteps32 - kAhead; ++i) {
+        for (int i = 0; i < 2 * kKSteps32 - kAhead; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
-        float sv[4];
-        const int tok_base = t_begin + sub * kSubTok + th * 16 + 4 * g;
+        float sv[8];
+        const int tok_base = t_begin + sub * kSubTok + 4 * g;
         bool over = false;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          sv[r] = tok_base + r < L ? (s0[r] + s1[r]) * a.scale_log2 : -INFINITY;
-          over |= sv[r] > m + kSlack;
+          sv[r] = tok_base + r < L ? s0[r] * a.scale_log2 : -INFINITY;
+          sv[4 + r] = tok_base + 16 + r < L ? s1[r] * a.scale_log2 : -INFINITY;
         }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) over |= sv[r] > m + kSlack;
         if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
-          const float mx = quad_rows_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+          float mx = sv[0];
+#pragma unroll
+          for (int r = 1; r < 8; ++r) mx = fmaxf(mx, sv[r]);
+          mx = quad_rows_max(mx);
           if (mx > m + kSlack) {
             const float alpha = fast_exp2(m - mx);
             m = mx;
@@ -694,30 +699,33 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
             for (int i = 0; i < 32; ++i) o[i] *= alpha;
           }
         }
-        float p[4];
+        float p[8];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int r = 0; r < 8; ++r) {
           p[r] = fast_exp2(sv[r] - m);
           l += p[r];
         }
-        const u32x2 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3])};
-        const s16x4 pb = __builtin_bit_cast(s16x4, pbw);
-        // ---- O^T += V^T . P^T over the 16 tokens and all 512 dims.  The transposing LDS load works on
+        // k-slot g*8 + j of the P.V MFMA <-> token 4g + j of block 0 (j < 4), of block 1 (j >= 4)
+        const u32x4 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3]), BF16::pack(p[4], p[5]), BF16::pack(p[6], p[7])};
+        const bf16x8 pb = __builtin_bit_cast(bf16x8, pbw);
+        // ---- O^T += V^T . P^T over the 32 tokens and all 512 dims.  The transposing LDS load works on
         // groups of 16 lanes: lane p of a group supplies the address of 4 dims of token row p/4 and
         // receives the 4 tokens of dim column p.
         const char* va = kb + v_row0;
         __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the P.V reads only
 #pragma unroll
         for (int mb = 0; mb < 32; ++mb) {
-          const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
-          o[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v, pb, o[mb], 0, 0, 0);
+          const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
+          const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + 16 * kRow16 + mb * 32));
+          const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+          o[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, o[mb], 0, 0, 0);
         }
-        // pipeline the transposing reads kAhead MFMAs ahead of their use
-        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+        // pipeline the transposing reads (two per MFMA) kAhead MFMAs ahead of their use
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
 #pragma unroll
         for (int i = 0; i < 32 - kAhead; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -725,51 +733,29 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
       if (wave >= 4 && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
     }
 
-    // ---- end of the run: the two token halves of a head block are folded through LDS (the ring
-    // is free now); the th = 0 wavefront writes the result
-    const float l_half = quad_rows_sum(l);
-    __syncthreads();  // every wavefront is past its last sub-tile
-    float* fold = reinterpret_cast<float*>(smem) + hb16 * (32 * 4 * kWave + 2 * 16);
-    if (wave_ok && th == 1) {
+    // ---- end of the run: every wavefront writes its own heads
+    const float lsum = quad_rows_sum(l);
+    const float inv = 1.0f / lsum;
+    const float lse2 = m + fast_log2(lsum);
+    const int64_t ps = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H + head;
+    if (head_ok && complete) {
+      char* op = a.out + ((static_cast<int64_t>(b) * H + head) * kDL + 4 * g) * 2;
 #pragma unroll
-      for (int mb = 0; mb < 32; ++mb)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) fold[(mb * 4 + r) * kWave + lane] = o[mb][r];
-      if (g == 0) {
-        fold[32 * 4 * kWave + c16] = m;
-        fold[32 * 4 * kWave + 16 + c16] = l_half;
+      for (int mb = 0; mb < 32; ++mb) {
+        const u32x2 w = {BF16::pack(o[mb][0] * inv, o[mb][1] * inv), BF16::pack(o[mb][2] * inv, o[mb][3] * inv)};
+        *reinterpret_cast<u32x2*>(op + mb * 32) = w;
       }
     }
-    __syncthreads();
-    if (wave_ok && th == 0) {
-      const float m1 = fold[32 * 4 * kWave + c16], l1 = fold[32 * 4 * kWave + 16 + c16];
-      const float m_all = fmaxf(m, m1);
-      const float f0 = fast_exp2(m - m_all), f1 = fast_exp2(m1 - m_all);
-      const float lsum = l_half * f0 + l1 * f1;
-      const float inv = 1.0f / lsum;
-      const float w0 = f0 * inv, w1 = f1 * inv;
+    if (head_ok && !complete) {
+      float* wp = a.ws_out + ps * kDL + 4 * g;
 #pragma unroll
-      for (int mb = 0; mb < 32; ++mb)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[mb][r] = o[mb][r] * w0 + fold[(mb * 4 + r) * kWave + lane] * w1;
-      const float lse2 = m_all + fast_log2(lsum);
-      const int64_t ps = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H + head;
-      if (head_ok && complete) {
-        char* op = a.out + ((static_cast<int64_t>(b) * H + head) * kDL + 4 * g) * 2;
-#pragma unroll
-        for (int mb = 0; mb < 32; ++mb) {
-          const u32x2 w = {BF16::pack(o[mb][0], o[mb][1]), BF16::pack(o[mb][2], o[mb][3])};
-          *reinterpret_cast<u32x2*>(op + mb * 32) = w;
-        }
+      for (int mb = 0; mb < 32; ++mb) {
+        const f32x4 w = {o[mb][0] * inv, o[mb][1] * inv, o[mb][2] * inv, o[mb][3] * inv};
+        *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
       }
-      if (head_ok && !complete) {
-        float* wp = a.ws_out + ps * kDL + 4 * g;
-#pragma unroll
-        for (int mb = 0; mb < 32; ++mb) *reinterpret_cast<f32x4*>(wp + mb * 16) = o[mb];
-      }
-      if (head_ok && g == 0 && complete && a.lse != nullptr) a.lse[b * H + head] = lse2 * kLn2;
-      if (head_ok && g == 0 && !complete) a.ws_lse[ps] = lse2;
     }
+    if (head_ok && g == 0 && complete && a.lse != nullptr) a.lse[b * H + head] = lse2 * kLn2;
+    if (head_ok && g == 0 && !complete) a.ws_lse[ps] = lse2;
     first_run = false;
   }
 }
@@ -865,7 +851,8 @@ size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) 
   (void)max_seq_len;
   const size_t b = static_cast<size_t>(batch < kMaxBatchMla ? batch : kMaxBatchMla);
   const size_t prefix_bytes = ((b + 1) * 4 + 255) / 256 * 256;
-  const int n_hb = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
+  // the kernel with 128 heads per workgroup has the fewer workgroups per team, hence the more teams
+  const int n_hb = static_cast<int>((n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
   return prefix_bytes + static_cast<size_t>(mla_teams(n_hb)) * 2 * n_heads * (kDL + 1) * 4;
 }
 
@@ -892,13 +879,14 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       workspace_bytes < mla_workspace_bytes(batch, n_heads, 0))
     return XLLM_MI355_EWORKSPACE;
 
-  const int n_hb = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
-  static const bool pairs_env = [] {  // tuning knob: "pairs" selects the 32-heads-per-wavefront kernel
+  static const bool pairs_env = [] {  // tuning knob: "pairs" selects the kernel with the per-tile exchange
     const char* e = getenv("XLLM_MI355_MLA_KERNEL");
     return e != nullptr && e[0] == 'p';
   }();
-  // the 16-heads-per-wavefront kernel looks pages up per group of 16 tokens
+  // the main kernel looks pages up per group of 4 tokens inside chunks of 64 pages
   const bool pairs = pairs_env || block_size < 16 || (block_size & (block_size - 1)) != 0;
+  const int n_hb = static_cast<int>(pairs ? (n_heads + kHeadsPerWg - 1) / kHeadsPerWg
+                                          : (n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
   static bool attr_set = false;
   const size_t smem = pairs ? kPrefixOff + (kMaxBatchMla + 1) * 4 : kPrefix16Off + (kMaxBatchMla + 1) * 4;
   if (!attr_set) {
