@@ -95,6 +95,44 @@ def test_small_and_odd_block_sizes_and_page_table_chunks(device):
     _check(_mla_cfg("short", 96, 16, 1, 200, bs=16), 13, device)
 
 
+def test_scores_that_rise_along_the_context(device):
+    # the rope dims of K carry a ramp and those of Q a constant, so the scores rise by about 120 log2 units from
+    # the first token to the last: every running maximum is overtaken many times and whatever was accumulated
+    # before has to be rescaled (or restarted) again and again; V = K[..., :512] is unaffected
+    for heads, lo, hi, bs in ((128, 1500, 2500, 64), (16, 700, 900, 16)):
+        cfg = _mla_cfg(f"ramp{heads}", 3, heads, lo, hi, bs=bs)
+        inp = workloads.make_inputs(cfg, 31)
+        lay = inp.layout
+        inp.q[:, :, 512:] = 2.0
+        for b in range(cfg.batch):
+            o0, o1 = int(lay.ctx_offsets[b]), int(lay.ctx_offsets[b + 1])
+            n = o1 - o0
+            ramp = (torch.arange(n, dtype=torch.float32) * (9.0 / max(n, 1))).to(torch.bfloat16)
+            inp.k_ctx[o0:o1, 0, 512:] = ramp[:, None]
+        inp.k_new[:, 0, 512:] = 9.0
+        kg, _, _, _ = fill_caches_gpu(inp, device)
+        kc, _ = fill_caches_cpu(inp)
+        out, lse = _decode_gpu(inp, kg, device)
+        ref = oracle.aten_paged_decode(inp.q, kc, None, lay.block_table, lay.seq_lens, cfg.scale, dv=cfg.v_dim)
+        assert_close_to_reference(out, ref, cfg.name)
+        ref_lse = oracle.aten_paged_decode_lse(inp.q, kc, lay.block_table, lay.seq_lens, cfg.scale)
+        assert torch.allclose(lse.cpu(), ref_lse, rtol=1e-3, atol=1e-3)
+
+
+def test_producer_consumer_kernel(device, monkeypatch):
+    # the kernel with the two products on different wavefronts, selected by the tuning knob
+    monkeypatch.setenv("XLLM_MI355_MLA_KERNEL", "split")
+    _check(_mla_cfg("split128", 3, 128, 100, 1500), 5, device)
+    for heads in (2, 16, 80):
+        _check(_mla_cfg(f"split{heads}", 2, heads, 1, 400), 60 + heads, device)
+    _check(_mla_cfg("split_bs16", 2, 16, 50, 700, bs=16), 3, device)
+    for i, L in enumerate((1023, 1025, 2049, 3100)):  # page-table chunk boundaries (block 16: 1024 tokens per chunk)
+        _check(_mla_cfg(f"split_chunks{L}", 1, 16, L, L, bs=16), 70 + i, device)
+    _check(_mla_cfg("split_short", 96, 16, 1, 200, bs=16), 13, device)
+    _check(_mla_cfg("split_long", 1, 128, 6000, 9000), 6, device)
+    test_scores_that_rise_along_the_context(device)
+
+
 def test_shard_merge_equals_full_decode(device):
     # ArtificialShardMergeMatchesFullCacheDecode (dcp_attention_merge_test.cpp:146-224): rtol/atol 1e-2, 1e-3
     cfg = _mla_cfg("merge", 4, 128, 256, 2000)
