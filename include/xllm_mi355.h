@@ -156,6 +156,33 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                                     int q_dtype, int cache_dtype, void* stream);
 
 /*
+ * Short query chunks through the decode kernels: chunked prefill and speculative-decoding
+ * verification with a few query tokens per sequence.  Replaces the decode branch of
+ * FlashAttentionImpl::paged_forward (xllm/core/layers/dcu/flash_attention.cpp:447-545: packed q
+ * [total_tokens, Hq, D] with q_cu_seq_lens, hg_prefix_decode_varlen_fwd for chunks of up to 16 tokens):
+ *     token j of the q_len = cu[b+1] - cu[b] tokens of sequence b attends to the first
+ *     kv_seq_lens[b] - q_len + j + 1 tokens of its context when causal != 0 (the chunk is the
+ *     tail of the context, AttentionMetadata::is_causal), to all kv_seq_lens[b] otherwise.
+ * q/out: [n_tokens, Hq, D]; cu_seqlens_q: [B + 1] int32 starting at 0; block_table: [B, table_stride].
+ * Every query token is decoded as an entry of its own against its sequence's pages, so the pages of a
+ * sequence are read once per query token (mostly from L2): meant for the reference's limit of 16
+ * tokens per chunk, correct for any.  Workspace: xllm_mi355_paged_decode_varlen_workspace_bytes.
+ */
+size_t xllm_mi355_paged_decode_varlen_workspace_bytes(int64_t n_tokens, int64_t n_q_heads,
+                                                      int64_t head_dim);
+int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_cache,
+                                       void* out,
+                                       const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
+                                       const int32_t* block_table, int64_t table_stride,
+                                       const float* k_scale, const float* v_scale,
+                                       int64_t batch, int64_t n_tokens, int64_t n_q_heads,
+                                       int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
+                                       int64_t num_blocks, int64_t q_token_stride,
+                                       int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
+                                       int causal, void* workspace, size_t workspace_bytes,
+                                       int q_dtype, int cache_dtype, void* stream);
+
+/*
  * Paged decode attention, MLA latent-KV variant.
  * Replaces xllm::kernel::dcu::flash_mla::dense_decode
  * (xllm/core/kernels/dcu/flash_mla_adapter.h:40-53, flash_mla_adapter.cpp:104-153):

@@ -177,6 +177,32 @@ def aten_paged_decode(q, k_cache, v_cache, block_table, seq_lens, sm_scale, k_sc
     return out
 
 
+def aten_paged_forward(q, k_cache, v_cache, block_table, kv_seq_lens, q_cu_seq_lens, sm_scale, causal=True):
+    """Short query chunks against paged KV (layers/dcu/flash_attention.cpp:447-545, decode branch): packed
+    q [T,Hq,D]; token j of the q_len tokens of sequence b attends to the first kv_len - q_len + j + 1
+    tokens (causal: the chunk is the tail of the context, the bottom-right alignment that the call site's
+    window arguments select) or to all kv_len.  Restated with the libtorch decode above, one query token
+    at a time; tokens that attend to nothing give zeros.  The fast path itself is a closed library:
+    parity with it is unpinned, the semantics are pinned against dense masked attention in the tests."""
+    T = q.shape[0]
+    B = kv_seq_lens.numel()
+    lens = torch.zeros(T, dtype=torch.int32)
+    rows = torch.zeros(T, dtype=torch.int64)
+    for b in range(B):
+        q0, q1 = int(q_cu_seq_lens[b]), int(q_cu_seq_lens[b + 1])
+        kv = int(kv_seq_lens[b])
+        for t in range(q0, q1):
+            L = kv - (q1 - q0) + (t - q0) + 1 if causal else kv
+            lens[t] = max(0, min(L, kv))
+            rows[t] = b
+    out = torch.zeros_like(q)
+    live = (lens > 0).nonzero().flatten()
+    if live.numel() > 0:
+        out[live] = aten_paged_decode(q[live].contiguous(), k_cache, v_cache, block_table[rows[live]].contiguous(),
+                                      lens[live].contiguous(), sm_scale)
+    return out
+
+
 def aten_paged_decode_csr(q, k_cache, v_cache, indptr, indices, last_page_len):
     B, Hq, D = q.shape
     P, bs, Hkv = k_cache.shape[0], k_cache.shape[1], k_cache.shape[2]

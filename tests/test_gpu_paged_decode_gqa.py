@@ -266,3 +266,39 @@ def test_full_size_config2_split_invariance_and_sampled_parity(device):
     diff = (merged.view_as(out).float() - out.float()).abs()
     assert diff.max() <= 1e-2 and diff.mean() <= 1e-3
     assert torch.allclose(mlse.view_as(lse), lse, rtol=1e-3, atol=1e-3)
+
+
+def test_short_query_chunks_through_the_decode_kernels(device):
+    # chunked prefill / speculative-decoding verification (layers/dcu/flash_attention.cpp:447-545): up to 16 query
+    # tokens per sequence, the chunk being the tail of its context; both decode kernels, causal and not
+    for name, Hq, Hkv, D, bs, lo, hi, batch in (("mfma", 32, 8, 128, 16, 1, 900, 7), ("rows", 8, 2, 64, 32, 1, 500, 5),
+                                                ("long", 16, 2, 128, 128, 2000, 5000, 2)):
+        cfg = workloads.DecodeConfig(f"chunks_{name}", batch, Hq, Hkv, D, bs, lo, hi)
+        inp = workloads.make_inputs(cfg, 50 + batch)
+        lay = inp.layout
+        g = torch.Generator().manual_seed(99)
+        q_lens = [int(torch.randint(1, min(16, int(L)) + 1, (1,), generator=g)) for L in lay.seq_lens]
+        cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+        q = (torch.randn(int(cu[-1]), Hq, D, generator=g) * cfg.sigma).to(torch.bfloat16)
+        kg, vg, _, _ = fill_caches_gpu(inp, device)
+        kc, vc = fill_caches_cpu(inp)
+        for causal in (True, False):
+            out = ops.paged_forward(q.to(device), torch.empty_like(q, device=device), kg, vg,
+                                    lay.block_table.to(device), lay.seq_lens.to(device), cu.to(device),
+                                    scale=cfg.scale, is_causal=causal)
+            torch.cuda.synchronize()
+            ref = oracle.aten_paged_forward(q, kc, vc, lay.block_table, lay.seq_lens, cu, cfg.scale, causal=causal)
+            assert_close_to_reference(out, ref, f"{cfg.name} causal={causal}")
+    # one token per sequence is plain decode, bit for bit
+    cfg = workloads.DecodeConfig("chunks_one", 6, 32, 8, 128, 16, 1, 700)
+    inp = workloads.make_inputs(cfg, 8)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    ones = torch.arange(cfg.batch + 1, dtype=torch.int32, device=device)
+    q = inp.q.to(device)
+    a = ops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device), ones,
+                          scale=cfg.scale)
+    b, _ = ops.batch_decode(q, kg, torch.empty_like(q), lay.block_table.to(device), lay.seq_lens.to(device),
+                            v_cache=vg, scale=cfg.scale)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)

@@ -163,3 +163,42 @@ def test_merge_of_context_shards_equals_unsplit_decode():
         out, lse = merge(torch.stack([oa, ob]), torch.stack([lsa, lsb]))
         assert torch.allclose(out, full, rtol=1e-2, atol=1e-2) and torch.allclose(lse, full_lse, rtol=1e-3, atol=1e-3)
         assert (out - full).abs().max() < 1e-5
+
+
+def _chunk_inputs(cfg, seed, max_q=16):
+    """A decode workload whose last q_len tokens of every context form the query chunk."""
+    inp = workloads.make_inputs(cfg, seed)
+    lay = inp.layout
+    g = torch.Generator().manual_seed(seed + 7)
+    q_lens = [int(torch.randint(1, min(max_q, int(L)) + 1, (1,), generator=g)) for L in lay.seq_lens]
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    q = (torch.randn(int(cu[-1]), cfg.n_q_heads, cfg.head_dim, generator=g) * cfg.sigma).to(torch.bfloat16)
+    return inp, q, cu, q_lens
+
+
+def test_query_chunks_equal_dense_attention_with_the_causal_mask_at_the_bottom_right():
+    cfg = workloads.DecodeConfig("chunks", 4, 8, 2, 64, 16, 5, 120)
+    inp, q, cu, q_lens = _chunk_inputs(cfg, 21)
+    kc, vc = fill_caches_cpu(inp)
+    lay = inp.layout
+    g = cfg.n_q_heads // cfg.n_kv_heads
+    for causal in (True, False):
+        out = oracle.aten_paged_forward(q, kc, vc, lay.block_table, lay.seq_lens, cu, cfg.scale, causal=causal)
+        for b in range(cfg.batch):
+            lo, hi = int(lay.ctx_offsets[b]), int(lay.ctx_offsets[b + 1])
+            k = torch.cat([inp.k_ctx[lo:hi], inp.k_new[b : b + 1]]).double()   # [L, Hkv, D]
+            v = torch.cat([inp.v_ctx[lo:hi], inp.v_new[b : b + 1]]).double()
+            L, n = k.shape[0], q_lens[b]
+            qb = q[int(cu[b]) : int(cu[b + 1])].double()                      # [n, Hq, D]
+            s = torch.einsum("nhd,lhd->hnl", qb, k.repeat_interleave(g, 1)) * cfg.scale
+            if causal:  # query j sees keys 0 .. L - n + j
+                mask = torch.arange(L)[None, :] > (L - n + torch.arange(n))[:, None]
+                s = s.masked_fill(mask[None], float("-inf"))
+            ref = torch.einsum("hnl,lhd->nhd", torch.softmax(s, -1), v.repeat_interleave(g, 1))
+            got = out[int(cu[b]) : int(cu[b + 1])].double()
+            assert (got - ref).abs().max() < 3e-3, (causal, b)
+    # a chunk of one token is plain decode
+    ones = torch.arange(cfg.batch + 1, dtype=torch.int32)
+    q1 = inp.q.contiguous()
+    assert torch.equal(oracle.aten_paged_forward(q1, kc, vc, lay.block_table, lay.seq_lens, ones, cfg.scale),
+                       oracle.aten_paged_decode(q1, kc, vc, lay.block_table, lay.seq_lens, cfg.scale))

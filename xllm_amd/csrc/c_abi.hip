@@ -85,6 +85,27 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                           cache_dtype, static_cast<hipStream_t>(stream));
 }
 
+size_t xllm_mi355_paged_decode_varlen_workspace_bytes(int64_t n_tokens, int64_t n_q_heads, int64_t head_dim) {
+  if (n_tokens <= 0 || n_q_heads <= 0 || head_dim <= 0) return 0;
+  return varlen_extra_bytes(n_tokens) + gqa_workspace_bytes(n_tokens, n_q_heads, head_dim);
+}
+
+int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
+                                       const int32_t* block_table, int64_t table_stride,
+                                       const float* k_scale, const float* v_scale, int64_t batch,
+                                       int64_t n_tokens, int64_t n_q_heads, int64_t n_kv_heads,
+                                       int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                       int64_t q_token_stride, int64_t out_token_stride,
+                                       int64_t max_seq_len, float sm_scale, int causal, void* workspace,
+                                       size_t workspace_bytes, int q_dtype, int cache_dtype, void* stream) {
+  return paged_decode_gqa_varlen(q, k_cache, v_cache, out, cu_seqlens_q, kv_seq_lens, block_table,
+                                 table_stride, k_scale, v_scale, batch, n_tokens, n_q_heads, n_kv_heads,
+                                 head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
+                                 max_seq_len, sm_scale, causal, workspace, workspace_bytes, q_dtype,
+                                 cache_dtype, static_cast<hipStream_t>(stream));
+}
+
 int xllm_mi355_paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out,
                                 float* lse, const int32_t* block_table, int64_t table_stride,
                                 const int32_t* seq_lens, int64_t batch, int64_t n_heads,

@@ -5,6 +5,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/xllm_mi355.h"
 
 namespace xllm_mi355 {
@@ -23,6 +25,7 @@ struct PageAddressing {
   const int32_t* block_table = nullptr;  // [B, table_stride]
   int64_t table_stride = 0;
   const int32_t* seq_lens = nullptr;     // [B]
+  const int32_t* table_rows = nullptr;   // [B] block-table row of each entry, or null for row b (block-table form only)
   const int32_t* indptr = nullptr;       // CSR when non-null: [B+1]
   const int32_t* indices = nullptr;
   const int32_t* last_page_len = nullptr;
@@ -46,6 +49,19 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
                      float sm_scale, void* workspace, size_t workspace_bytes, int dtype,
                      hipStream_t stream);
 
+// Several query tokens per sequence (packed q, cu_seqlens_q) through the decode kernels: token j of a
+// sequence with q_len tokens attends to the first kv_len - q_len + j + 1 tokens (causal) or to all kv_len.
+// The first varlen_extra_bytes(n_tokens) of the workspace hold the per-token lengths and table rows.
+size_t varlen_extra_bytes(int64_t n_tokens);
+int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_cache, void* out,
+                            const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
+                            const int32_t* block_table, int64_t table_stride, const float* k_scale,
+                            const float* v_scale, int64_t batch, int64_t n_tokens, int64_t n_q_heads,
+                            int64_t n_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                            int64_t q_token_stride, int64_t out_token_stride, int64_t max_seq_len,
+                            float sm_scale, int causal, void* workspace, size_t workspace_bytes,
+                            int q_dtype, int cache_dtype, hipStream_t stream);
+
 int lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,
               int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim, int dtype,
               hipStream_t stream);
@@ -53,6 +69,17 @@ int lse_merge(const void* partial_out, const float* partial_lse, void* out, floa
 int build_block_table(const int32_t* indptr, const int32_t* indices, const int32_t* last_page_len,
                       int32_t* block_table, int64_t table_stride, int32_t* seq_lens, int64_t batch,
                       int64_t block_size, hipStream_t stream);
+
+// Kernel attributes (dynamic LDS size) are set per device.  Returns true the first time it is called with
+// `seen` on the current device (devices 0..63; beyond that always true: setting them again is harmless).
+inline bool first_use_on_current_device(std::atomic<uint64_t>& seen) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) return true;
+  const uint64_t bit = 1ull << dev;
+  if ((seen.load(std::memory_order_acquire) & bit) != 0) return false;
+  seen.fetch_or(bit, std::memory_order_acq_rel);
+  return true;
+}
 
 // Opt-in timing of the dominant kernel (profile.hip).  profile_begin returns true when a
 // start event was recorded; the caller then must call profile_end after its launch.

@@ -3,6 +3,9 @@
 //                         (xllm/core/layers/mlu/dcp_attention_merge.cpp:26-65)
 //   build_block_table  -- CSR page lists -> padded [B, stride] table, -1 fill
 //                         (xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip:44-149)
+//   expand_varlen      -- per query token of a packed batch: attended length and block-table row, so that
+//                         short query chunks run through the decode kernels
+//                         (xllm/core/layers/dcu/flash_attention.cpp:447-545, the hg_prefix_decode_varlen_fwd branch)
 #include "common.cuh"
 #include "launch.h"
 
@@ -62,7 +65,70 @@ __global__ __launch_bounds__(256) void build_block_table_kernel(const int32_t* i
     seq_lens[b] = n > 0 ? (n - 1) * block_size + last_page_len[b] : 0;
 }
 
+// One thread per query token.  Token t belongs to the sequence b with cu[b] <= t < cu[b + 1]; with q_len
+// tokens in that sequence, token j of them attends to kv_len - q_len + j + 1 tokens when causal (the chunk
+// is the tail of the context), to kv_len otherwise.  Tokens outside cu[0] .. cu[B] get length 0.
+__global__ __launch_bounds__(256) void expand_varlen_kernel(const int32_t* cu_seqlens_q,
+                                                            const int32_t* kv_seq_lens,
+                                                            int32_t* tok_lens, int32_t* tok_rows,
+                                                            int n_tokens, int batch, int causal) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= n_tokens) return;
+  int lo = 0, hi = batch;  // largest b in [0, batch) with cu[b] <= t (cu[0] is 0 for well-formed input)
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu_seqlens_q[mid] <= t) lo = mid; else hi = mid;
+  }
+  const int b = lo;
+  const int q0 = cu_seqlens_q[b], q1 = cu_seqlens_q[b + 1];
+  int L = 0;
+  if (t >= q0 && t < q1) {
+    const int kv = kv_seq_lens[b];
+    L = causal != 0 ? kv - (q1 - q0) + (t - q0) + 1 : kv;
+    L = L < 0 ? 0 : (L > kv ? kv : L);
+  }
+  tok_lens[t] = L;
+  tok_rows[t] = b;
+}
+
 }  // namespace
+
+size_t varlen_extra_bytes(int64_t n_tokens) {
+  return n_tokens <= 0 ? 0 : (static_cast<size_t>(n_tokens) * 2 * 4 + 255) / 256 * 256;
+}
+
+int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_cache, void* out,
+                            const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
+                            const int32_t* block_table, int64_t table_stride, const float* k_scale,
+                            const float* v_scale, int64_t batch, int64_t n_tokens, int64_t n_q_heads,
+                            int64_t n_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                            int64_t q_token_stride, int64_t out_token_stride, int64_t max_seq_len,
+                            float sm_scale, int causal, void* workspace, size_t workspace_bytes,
+                            int q_dtype, int cache_dtype, hipStream_t stream) {
+  if (batch == 0 || n_tokens == 0) return XLLM_MI355_OK;
+  if (cu_seqlens_q == nullptr || kv_seq_lens == nullptr || block_table == nullptr || table_stride <= 0)
+    return XLLM_MI355_EINVAL;
+  if (batch < 0 || n_tokens < 0 || batch > 0x7fffffffLL || n_tokens > 0x7fffffffLL) return XLLM_MI355_EINVAL;
+  const size_t extra = varlen_extra_bytes(n_tokens);
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 || workspace_bytes < extra)
+    return XLLM_MI355_EWORKSPACE;
+  int32_t* tok_lens = static_cast<int32_t*>(workspace);
+  int32_t* tok_rows = tok_lens + n_tokens;
+  const unsigned grid = static_cast<unsigned>((n_tokens + 255) / 256);
+  expand_varlen_kernel<<<dim3(grid), 256, 0, stream>>>(cu_seqlens_q, kv_seq_lens, tok_lens, tok_rows,
+                                                       static_cast<int>(n_tokens), static_cast<int>(batch), causal);
+  const int rc = static_cast<int>(hipGetLastError());
+  if (rc != 0) return rc;
+  PageAddressing addr;
+  addr.block_table = block_table;
+  addr.table_stride = table_stride;
+  addr.seq_lens = tok_lens;
+  addr.table_rows = tok_rows;
+  return paged_decode_gqa(q, k_cache, v_cache, out, nullptr, addr, k_scale, v_scale, n_tokens, n_q_heads,
+                          n_kv_heads, head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
+                          max_seq_len, sm_scale, static_cast<char*>(workspace) + extra, workspace_bytes - extra,
+                          q_dtype, cache_dtype, stream);
+}
 
 int lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,
               int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim, int dtype,

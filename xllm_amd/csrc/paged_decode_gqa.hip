@@ -58,6 +58,7 @@ struct GqaArgs {
   char* out;
   float* lse;
   const int32_t* block_table;
+  const int32_t* table_rows;  // block-table row of each batch entry, or null for row b (several query tokens of a sequence)
   const int32_t* seq_lens;
   const int32_t* indptr;
   const int32_t* indices;
@@ -90,7 +91,7 @@ __device__ __forceinline__ void sequence_of(const GqaArgs& a, int b, const int32
     pages = a.indices + p0;
     L = np > 0 ? (np - 1) * a.block_size + a.last_page_len[b] : 0;
   } else {
-    pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
+    pages = a.block_table + static_cast<int64_t>(a.table_rows != nullptr ? a.table_rows[b] : b) * a.table_stride;
     L = a.seq_lens[b];
   }
 }
@@ -578,7 +579,7 @@ __device__ __forceinline__ void sequence_of_scalar(const GqaArgs& a, int b, cons
     pages = a.indices + p0;
     L = np > 0 ? (np - 1) * a.block_size + sload32(a.last_page_len + b) : 0;
   } else {
-    pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
+    pages = a.block_table + static_cast<int64_t>(a.table_rows != nullptr ? sload32(a.table_rows + b) : b) * a.table_stride;
     L = sload32(a.seq_lens + b);
   }
 }
@@ -1167,12 +1168,13 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   using Lay = MfmaLayout<kMfmaStages>;
   constexpr int D = 128;
   auto kern = gqa_mfma_kernel<QT, FP8, kMfmaStages>;
-  static const bool configured = [&] {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              Lay::kPrefixOff + (kMaxBatch + 1) * 4);
-    return true;
-  }();
-  (void)configured;
+  static std::atomic<uint64_t> configured{0};
+  if (first_use_on_current_device(configured)) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             Lay::kPrefixOff + (kMaxBatch + 1) * 4);
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
   a.g_block = kMfmaHeads;
   const int n_wg = device_cu_count();  // the ring fills a CU's LDS: one workgroup each
   a.n_workgroups = n_wg * kWaves;      // independent workers = wavefronts
@@ -1294,7 +1296,8 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     a.v_cache = static_cast<const char*>(v_cache);
     a.out = static_cast<char*>(out) + b0 * out_token_stride * 2;
     a.lse = lse == nullptr ? nullptr : lse + b0 * n_q_heads;
-    a.block_table = csr ? nullptr : addr.block_table + b0 * addr.table_stride;
+    a.block_table = csr ? nullptr : (addr.table_rows != nullptr ? addr.block_table : addr.block_table + b0 * addr.table_stride);
+    a.table_rows = csr || addr.table_rows == nullptr ? nullptr : addr.table_rows + b0;
     a.seq_lens = csr ? nullptr : addr.seq_lens + b0;
     a.indptr = csr ? addr.indptr + b0 : nullptr;
     a.indices = addr.indices;

@@ -1455,9 +1455,9 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   const int n_hb = static_cast<int>(pairs ? (n_heads + kHeadsPerWg - 1) / kHeadsPerWg
                                           : (n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
   const int n_hb_p = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
-  static bool attr_set = false;
+  static std::atomic<uint64_t> configured{0};
   const size_t smem = pairs ? kPrefixOff + (kMaxBatchMla + 1) * 4 : kPrefix16Off + (kMaxBatchMla + 1) * 4;
-  if (!attr_set) {
+  if (first_use_on_current_device(configured)) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        static_cast<int>(kPrefixOff + (kMaxBatchMla + 1) * 4));
@@ -1469,7 +1469,6 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode32w_kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
     if (e != hipSuccess) return static_cast<int>(e);
-    attr_set = true;
   }
   for (int64_t b0 = 0; b0 < batch; b0 += kMaxBatchMla) {
     const int64_t nb = batch - b0 < kMaxBatchMla ? batch - b0 : kMaxBatchMla;

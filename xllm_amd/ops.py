@@ -235,6 +235,43 @@ def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
     return output
 
 
+def paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_cu_seq_lens, scale=None,
+                  is_causal=True, max_seq_len=0, k_cache_quant_scale=None, v_cache_quant_scale=None):
+    """Short query chunks (chunked prefill, speculative-decoding verification) against paged KV:
+    the decode branch of FlashAttentionImpl::paged_forward (layers/dcu/flash_attention.cpp:447-545).
+    query/output packed [T, Hq, D]; q_cu_seq_lens [B + 1] int32 from 0 to T; kv_seq_lens [B] int32 are
+    the context lengths INCLUDING the chunk; with is_causal token j of a chunk of q_len tokens attends
+    to the first kv_len - q_len + j + 1 tokens.  Returns output."""
+    dev = _require_cuda(query, k_cache, v_cache, output, block_table, kv_seq_lens, q_cu_seq_lens,
+                        k_cache_quant_scale, v_cache_quant_scale)
+    _decode_common(query, k_cache, output)
+    T, Hq, D = query.shape
+    P, bs, Hkv, _ = k_cache.shape
+    B = kv_seq_lens.numel()
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise ValueError("block_table must be int32 [B, W] with unit column stride")
+    if block_table.shape[0] != B:
+        raise ValueError("block_table rows must equal the batch")
+    for t, n in ((kv_seq_lens, B), (q_cu_seq_lens, B + 1)):
+        if t.dtype != torch.int32 or t.numel() != n or not t.is_contiguous():
+            raise ValueError("kv_seq_lens [B] and q_cu_seq_lens [B + 1] must be contiguous int32")
+    if scale is None:
+        scale = D ** -0.5
+    if max_seq_len <= 0:
+        max_seq_len = block_table.shape[1] * bs
+    lib = capi.lib()
+    nbytes = lib.xllm_mi355_paged_decode_varlen_workspace_bytes(T, Hq, D)
+    ws = decode_workspace(dev, nbytes)
+    rc = lib.xllm_mi355_paged_decode_gqa_varlen(
+        query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
+        q_cu_seq_lens.data_ptr(), kv_seq_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+        _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, T, Hq, Hkv, D, bs, P,
+        query.stride(0), output.stride(0), max_seq_len, float(scale), 1 if is_causal else 0,
+        ws.data_ptr(), ws.numel(), _dtype_code(query), _dtype_code(k_cache), _stream(dev))
+    capi.check(rc, "xllm_mi355_paged_decode_gqa_varlen")
+    return output
+
+
 @dataclass
 class DenseDecodeParams:
     """flash_mla::DenseDecodeParams (xllm/core/kernels/dcu/flash_mla_adapter.h:40-53)."""
