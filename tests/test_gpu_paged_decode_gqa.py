@@ -302,3 +302,73 @@ def test_short_query_chunks_through_the_decode_kernels(device):
                             v_cache=vg, scale=cfg.scale)
     torch.cuda.synchronize()
     assert torch.equal(a, b)
+
+
+def test_step_captured_in_a_graph_follows_new_metadata(device):
+    # The reference's graph executor replays one captured decode step while it rewrites the metadata in
+    # persistent buffers (runtime/dcu_graph_executor_impl.h:114-170).  Capture cache write + decode once, then
+    # replay with other lengths, slots and query rows; eager work and synchronisations sit between the replays
+    # and every replay is checked against the eager result of the same inputs.
+    cfg = workloads.DecodeConfig("graph", 12, 32, 8, 128, 16, 50, 1500)
+    inputs = [workloads.make_inputs(cfg, 300 + i) for i in range(3)]
+    width = max(inp.layout.block_table.shape[1] for inp in inputs)
+    blocks = max(inp.layout.num_blocks for inp in inputs)
+    shape = (blocks, cfg.block_size, cfg.n_kv_heads, cfg.head_dim)
+    k_cache = torch.zeros(shape, dtype=torch.bfloat16, device=device)
+    v_cache = torch.zeros_like(k_cache)
+    # persistent buffers of the captured step
+    table = torch.zeros(cfg.batch, width, dtype=torch.int32, device=device)
+    lens = torch.zeros(cfg.batch, dtype=torch.int32, device=device)
+    slots = torch.zeros(cfg.batch, dtype=torch.int32, device=device)
+    q = torch.zeros(cfg.batch, cfg.n_q_heads, cfg.head_dim, dtype=torch.bfloat16, device=device)
+    k_new = torch.zeros(cfg.batch, cfg.n_kv_heads, cfg.head_dim, dtype=torch.bfloat16, device=device)
+    v_new = torch.zeros_like(k_new)
+    out = torch.zeros_like(q)
+
+    def load(inp):  # what the executor does before a replay: fill the caches' context, rewrite the metadata
+        lay = inp.layout
+        k_cache.zero_()
+        v_cache.zero_()
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(
+            key=inp.k_ctx.to(device), value=inp.v_ctx.to(device), k_cache=k_cache, v_cache=v_cache,
+            slot_mapping=lay.ctx_slots.to(device)))
+        table.zero_()
+        table[:, : lay.block_table.shape[1]] = lay.block_table.to(device)
+        lens.copy_(lay.seq_lens.to(device))
+        slots.copy_(lay.new_slots.to(device))
+        q.copy_(inp.q.to(device))
+        k_new.copy_(inp.k_new.to(device))
+        v_new.copy_(inp.v_new.to(device))
+
+    def step():
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=k_new, value=v_new, k_cache=k_cache, v_cache=v_cache,
+                                                            slot_mapping=slots))
+        ops.batch_decode(q, k_cache, out, table, lens, v_cache=v_cache, scale=cfg.scale,
+                         max_seq_len=width * cfg.block_size)
+
+    load(inputs[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture: workspace allocation, kernel attributes
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(6):
+        inp = inputs[rep % 3]
+        load(inp)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out.clone()
+        out.zero_()
+        load(inp)
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, out), f"replay {rep}"
+        kc, vc = fill_caches_cpu(inp)
+        lay = inp.layout
+        ref = oracle.aten_paged_decode(inp.q, kc[: blocks], vc[: blocks], lay.block_table, lay.seq_lens, cfg.scale)
+        assert_close_to_reference(replayed, ref, f"graph replay {rep}")

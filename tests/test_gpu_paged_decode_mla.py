@@ -170,3 +170,68 @@ def test_full_size_config5_sampled_parity(device):
                                    cfg.scale, dv=512)
     assert_close_to_reference(out[sample], ref, "cfg5 sample")
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+
+
+def test_step_captured_in_a_graph_follows_new_metadata(device):
+    # latent store + dense_decode captured once and replayed over rewritten persistent buffers
+    # (runtime/dcu_graph_executor_impl.h:114-170); eager work and synchronisations between the replays
+    cfg = _mla_cfg("graph", 6, 128, 100, 2500)
+    inputs = [workloads.make_inputs(cfg, 400 + i) for i in range(2)]
+    width = max(inp.layout.block_table.shape[1] for inp in inputs)
+    blocks = max(inp.layout.num_blocks for inp in inputs)
+    k_cache = torch.zeros(blocks, cfg.block_size, 1, 576, dtype=torch.bfloat16, device=device)
+    table = torch.zeros(cfg.batch, width, dtype=torch.int32, device=device)
+    lens = torch.zeros(cfg.batch, dtype=torch.int32, device=device)
+    slots = torch.zeros(cfg.batch, dtype=torch.int32, device=device)
+    q_nope = torch.zeros(cfg.batch, 1, cfg.n_q_heads, 512, dtype=torch.bfloat16, device=device)
+    q_pe = torch.zeros(cfg.batch, 1, cfg.n_q_heads, 64, dtype=torch.bfloat16, device=device)
+    k_new = torch.zeros(cfg.batch, 1, 576, dtype=torch.bfloat16, device=device)
+    result = {}
+
+    def load(inp):
+        lay = inp.layout
+        k_cache.zero_()
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=inp.k_ctx.to(device), value=None, k_cache=k_cache,
+                                                            v_cache=None, slot_mapping=lay.ctx_slots.to(device)))
+        table.zero_()
+        table[:, : lay.block_table.shape[1]] = lay.block_table.to(device)
+        lens.copy_(lay.seq_lens.to(device))
+        slots.copy_(lay.new_slots.to(device))
+        q = inp.q.to(device)
+        q_nope.copy_(q[:, :, :512].reshape(cfg.batch, 1, cfg.n_q_heads, 512))
+        q_pe.copy_(q[:, :, 512:].reshape(cfg.batch, 1, cfg.n_q_heads, 64))
+        k_new.copy_(inp.k_new.to(device))
+
+    def step():
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=k_new, value=None, k_cache=k_cache, v_cache=None,
+                                                            slot_mapping=slots))
+        p = ops.DenseDecodeParams(q_nope=q_nope, q_pe=q_pe, k_cache=k_cache, seqlens_k=lens, block_table=table,
+                                  head_size_v=512, softmax_scale=cfg.scale)
+        result["out"] = ops.dense_decode(p, max_seq_len=width * cfg.block_size)
+
+    load(inputs[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture: workspace allocation, kernel attributes
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    captured_out = result["out"]
+    for rep in range(4):
+        inp = inputs[rep % 2]
+        load(inp)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = captured_out.clone()
+        load(inp)
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, result["out"]), f"replay {rep}"
+        kc, _ = fill_caches_cpu(inp)
+        lay = inp.layout
+        ref = oracle.aten_paged_decode(inp.q, kc, None, lay.block_table, lay.seq_lens, cfg.scale, dv=512)
+        assert_close_to_reference(replayed.view(cfg.batch, cfg.n_q_heads, 512), ref, f"mla graph replay {rep}")
