@@ -156,6 +156,21 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                                     int q_dtype, int cache_dtype, void* stream);
 
 /*
+ * Rows of paged sequences gathered into one packed buffer, sequence after sequence.
+ * Replaces xllm::kernel::dcu::gather_mla_latent_cache
+ * (xllm/core/kernels/dcu/gather_mla_latent_cache.hip:32-75,124-190; declared in dcu_ops_api.h:74; called for
+ * prefill with context at layers/dcu/deepseek_v2_attention.cpp:324):
+ *     out[cu_seq_lens[b] + t, :] = cache[block_table[b, t / bs] * bs + t % bs, :]   for t < cu[b+1] - cu[b]
+ * cache: [P, bs, row_bytes] contiguous (for the latent cache row_bytes = (kv_lora_rank + rope) * 2);
+ * cu_seq_lens: [B + 1] int32 starting at 0; out: [total_rows, row_bytes].  Rows whose page id is negative
+ * (table padding) or not below num_blocks are left untouched.
+ */
+int xllm_mi355_gather_paged_rows(const void* cache, const int32_t* block_table, int64_t table_stride,
+                                 const int32_t* cu_seq_lens, void* out,
+                                 int64_t batch, int64_t total_rows, int64_t block_size,
+                                 int64_t num_blocks, int64_t row_bytes, void* stream);
+
+/*
  * Short query chunks through the decode kernels: chunked prefill and speculative-decoding
  * verification with a few query tokens per sequence.  Replaces the decode branch of
  * FlashAttentionImpl::paged_forward (xllm/core/layers/dcu/flash_attention.cpp:447-545: packed q

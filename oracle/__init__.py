@@ -64,6 +64,8 @@ def c_lib():
         lib.oracle_lse_merge.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64]
         lib.oracle_build_block_table.restype = None
         lib.oracle_build_block_table.argtypes = [_p, _p, _p, _p, _i64, _p, _i64, _i64]
+        lib.oracle_gather_paged_rows.restype = None
+        lib.oracle_gather_paged_rows.argtypes = [_p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64]
         _c = lib
     return _c
 
@@ -262,3 +264,12 @@ def build_block_table(indptr, indices, last_page_len, table_stride, block_size):
     c_lib().oracle_build_block_table(_ptr(indptr), _ptr(indices), _ptr(last_page_len), _ptr(table),
                                      table_stride, _ptr(seq_lens), B, block_size)
     return table, seq_lens
+
+
+def gather_paged_rows(cache, block_table, cu_seq_lens, total_rows, fill=0):
+    """cache [P, bs, 1, D] -> [total_rows, D]; untouched rows keep `fill`."""
+    P, bs, D = cache.shape[0], cache.shape[1], cache.shape[-1]
+    out = torch.full((total_rows, D), fill, dtype=cache.dtype)
+    c_lib().oracle_gather_paged_rows(_ptr(cache), _ptr(block_table), block_table.stride(0), _ptr(cu_seq_lens),
+                                     _ptr(out), block_table.shape[0], bs, P, D * cache.element_size())
+    return out

@@ -345,3 +345,23 @@ void oracle_build_block_table(const int32_t* indptr, const int32_t* indices,
     if (seq_lens) seq_lens[b] = n > 0 ? (int32_t)((n - 1) * block_size + last_page_len[b]) : 0;
   }
 }
+
+/*
+ * Rows of paged sequences -> packed buffer (kernels/dcu/gather_mla_latent_cache.hip:32-75): for every sequence b
+ * and token t < cu[b+1] - cu[b], out row cu[b] + t = cache row block_table[b, t / bs] * bs + t % bs; rows with a
+ * negative page id are skipped (the reference's `physical_block < 0` return), and so are ids beyond the cache.
+ */
+void oracle_gather_paged_rows(const uint8_t* cache, const int32_t* block_table, int64_t table_stride,
+                              const int32_t* cu_seq_lens, uint8_t* out, int64_t batch, int64_t block_size,
+                              int64_t num_blocks, int64_t row_bytes) {
+  for (int64_t b = 0; b < batch; ++b) {
+    const int64_t n = (int64_t)cu_seq_lens[b + 1] - cu_seq_lens[b];
+    for (int64_t t = 0; t < n; ++t) {
+      const int64_t page = block_table[b * table_stride + t / block_size];
+      if (page < 0 || page >= num_blocks) continue;
+      const uint8_t* from = cache + (page * block_size + t % block_size) * row_bytes;
+      uint8_t* to = out + ((int64_t)cu_seq_lens[b] + t) * row_bytes;
+      for (int64_t i = 0; i < row_bytes; ++i) to[i] = from[i];
+    }
+  }
+}

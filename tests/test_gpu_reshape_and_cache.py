@@ -174,3 +174,31 @@ def test_prefill_sized_scatter_is_a_permutation(device):
                                                         slot_mapping=slots))
     assert torch.equal(kg.view(T, H, D)[slots.long()], key)
     assert torch.equal(vg.view(T, H, D)[slots.long()], value)
+
+
+def test_gather_of_paged_latent_rows(device):
+    # dcu::gather_mla_latent_cache (kernels/dcu/gather_mla_latent_cache.hip): bit-exact against the oracle, with
+    # ragged lengths, padding ids in the table, and row lengths that take the 16-, 4- and 1-byte paths
+    from helpers import fill_caches_cpu
+    for dim, dtype, bs in ((576, torch.bfloat16, 64), (576, torch.bfloat16, 16), (130, torch.float16, 16),
+                           (33, torch.uint8, 32)):
+        cfg = workloads.DecodeConfig(f"gather{dim}", 7, 4, 1, 576, bs, 1, 900, mla=True, v_dim=512)
+        lay = workloads.make_layout(cfg, 17 + dim)
+        g = torch.Generator().manual_seed(dim)
+        kc = torch.randint(0, 250, (lay.num_blocks, bs, 1, dim), generator=g, dtype=torch.uint8)
+        kc = kc if dtype == torch.uint8 else kc.to(torch.float32).to(dtype)
+        cu = torch.zeros(cfg.batch + 1, dtype=torch.int32)
+        cu[1:] = lay.seq_lens.cumsum(0)
+        total = int(cu[-1])
+        table = lay.block_table.clone()
+        table[2, 0] = -1                      # a lost page: its rows stay as they were
+        table[3, 1:] = -1
+        ref = oracle.gather_paged_rows(kc, table, cu, total)
+        out = ops.gather_mla_latent_cache(kc.to(device), table.to(device), cu.to(device), total)
+        torch.cuda.synchronize()
+        touched = torch.ones(total, dtype=torch.bool)
+        for b in (2, 3):
+            for t in range(int(lay.seq_lens[b])):
+                if int(table[b, t // bs]) < 0:
+                    touched[int(cu[b]) + t] = False
+        assert torch.equal(out.cpu()[touched].view(torch.uint8), ref[touched].view(torch.uint8)), (dim, dtype)

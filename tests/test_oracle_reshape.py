@@ -57,3 +57,33 @@ def test_npu_case_and_negative_slots_and_strides():
             assert torch.equal(flat_k[slot], k[t]) and torch.equal(flat_v[slot], v[t])
     for slot in (1, 4, 5, 6):
         assert (flat_k[slot] == 9).all() and (flat_v[slot] == 9).all()
+
+
+def test_gather_of_paged_rows_is_the_inverse_of_the_scatter():
+    # gather_mla_latent_cache (kernels/dcu/gather_mla_latent_cache.hip:32-75): the rows a sequence scattered
+    # into its pages come back in token order, sequence after sequence; padding ids (-1) leave rows untouched
+    import oracle
+    from helpers import fill_caches_cpu
+    from xllm_amd import workloads
+    cfg = workloads.DecodeConfig("gather", 5, 16, 1, 576, 16, 1, 300, mla=True, v_dim=512)
+    inp = workloads.make_inputs(cfg, 4)
+    lay = inp.layout
+    kc, _ = fill_caches_cpu(inp)
+    cu = torch.zeros(cfg.batch + 1, dtype=torch.int32)
+    cu[1:] = lay.seq_lens.cumsum(0)
+    total = int(cu[-1])
+    out = oracle.gather_paged_rows(kc, lay.block_table, cu, total)
+    for b in range(cfg.batch):
+        lo, hi = int(lay.ctx_offsets[b]), int(lay.ctx_offsets[b + 1])
+        rows = torch.cat([inp.k_ctx[lo:hi, 0], inp.k_new[b]])
+        assert torch.equal(out[int(cu[b]) : int(cu[b + 1])], rows)
+    # brute force with torch indexing, and a table whose second sequence lost a page
+    table = lay.block_table.clone()
+    table[1, 0] = -1
+    got = oracle.gather_paged_rows(kc, table, cu, total, fill=7)
+    flat = kc.view(-1, 576)
+    for b in range(cfg.batch):
+        for t in range(int(lay.seq_lens[b])):
+            page = int(table[b, t // 16])
+            expect = flat[page * 16 + t % 16] if page >= 0 else torch.full((576,), 7, dtype=kc.dtype)
+            assert torch.equal(got[int(cu[b]) + t], expect)

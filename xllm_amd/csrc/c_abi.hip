@@ -85,6 +85,13 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                           cache_dtype, static_cast<hipStream_t>(stream));
 }
 
+int xllm_mi355_gather_paged_rows(const void* cache, const int32_t* block_table, int64_t table_stride,
+                                 const int32_t* cu_seq_lens, void* out, int64_t batch, int64_t total_rows,
+                                 int64_t block_size, int64_t num_blocks, int64_t row_bytes, void* stream) {
+  return gather_paged_rows(cache, block_table, table_stride, cu_seq_lens, out, batch, total_rows, block_size,
+                           num_blocks, row_bytes, static_cast<hipStream_t>(stream));
+}
+
 size_t xllm_mi355_paged_decode_varlen_workspace_bytes(int64_t n_tokens, int64_t n_q_heads, int64_t head_dim) {
   if (n_tokens <= 0 || n_q_heads <= 0 || head_dim <= 0) return 0;
   return varlen_extra_bytes(n_tokens) + gqa_workspace_bytes(n_tokens, n_q_heads, head_dim);

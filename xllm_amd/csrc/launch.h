@@ -70,6 +70,10 @@ int build_block_table(const int32_t* indptr, const int32_t* indices, const int32
                       int32_t* block_table, int64_t table_stride, int32_t* seq_lens, int64_t batch,
                       int64_t block_size, hipStream_t stream);
 
+int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t table_stride,
+                      const int32_t* cu_seq_lens, void* out, int64_t batch, int64_t total_rows,
+                      int64_t block_size, int64_t num_blocks, int64_t row_bytes, hipStream_t stream);
+
 // Kernel attributes (dynamic LDS size) are set per device.  Returns true the first time it is called with
 // `seen` on the current device (devices 0..63; beyond that always true: setting them again is harmless).
 inline bool first_use_on_current_device(std::atomic<uint64_t>& seen) {

@@ -3,6 +3,9 @@
 //                         (xllm/core/layers/mlu/dcp_attention_merge.cpp:26-65)
 //   build_block_table  -- CSR page lists -> padded [B, stride] table, -1 fill
 //                         (xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip:44-149)
+//   gather_paged_rows  -- rows of paged sequences -> one packed [total_rows, row_bytes] buffer, sequence after
+//                         sequence (xllm/core/kernels/dcu/gather_mla_latent_cache.hip:32-75: the latent rows
+//                         of the context for prefill with context)
 //   expand_varlen      -- per query token of a packed batch: attended length and block-table row, so that
 //                         short query chunks run through the decode kernels
 //                         (xllm/core/layers/dcu/flash_attention.cpp:447-545, the hg_prefix_decode_varlen_fwd branch)
@@ -91,7 +94,77 @@ __global__ __launch_bounds__(256) void expand_varlen_kernel(const int32_t* cu_se
   tok_rows[t] = b;
 }
 
+// One workgroup per 32 output rows.  The first 32 threads find the sequence of their row (cu[b] <= row <
+// cu[b + 1]) and its source row in the paged cache; then the 256 threads copy the rows in pieces of VB bytes
+// (16 when the row length allows it), consecutive threads taking consecutive pieces of a row.  Rows whose
+// page id is negative or beyond the cache are left untouched, as in the reference kernel (which skips
+// negative ids; an id beyond the cache would be an out-of-bounds read there).
+template <int VB>
+__global__ __launch_bounds__(256) void gather_paged_rows_kernel(const char* cache, const int32_t* block_table,
+                                                                int64_t table_stride, const int32_t* cu_seq_lens,
+                                                                char* out, int batch, int64_t total_rows,
+                                                                int block_size, int num_blocks, int row_bytes) {
+  __shared__ int64_t src_row[32];
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * 32;
+  if (threadIdx.x < 32) {
+    const int64_t row = row0 + threadIdx.x;
+    int64_t src = -1;
+    if (row < total_rows) {
+      int lo = 0, hi = batch;  // largest b in [0, batch) with cu[b] <= row
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (cu_seq_lens[mid] <= row) lo = mid; else hi = mid;
+      }
+      const int64_t tok = row - cu_seq_lens[lo];
+      if (tok >= 0 && row < cu_seq_lens[lo + 1] && tok / block_size < table_stride) {
+        const int page = block_table[lo * table_stride + tok / block_size];
+        if (page >= 0 && page < num_blocks) src = static_cast<int64_t>(page) * block_size + tok % block_size;
+      }
+    }
+    src_row[threadIdx.x] = src;
+  }
+  __syncthreads();
+  const int pieces = row_bytes / VB;
+  for (int i = threadIdx.x; i < 32 * pieces; i += 256) {
+    const int r = i / pieces, c = i - r * pieces;
+    const int64_t src = src_row[r];
+    if (src < 0) continue;
+    const char* from = cache + src * row_bytes + static_cast<int64_t>(c) * VB;
+    char* to = out + (row0 + r) * row_bytes + static_cast<int64_t>(c) * VB;
+    if constexpr (VB == 16) *reinterpret_cast<u32x4*>(to) = *reinterpret_cast<const u32x4*>(from);
+    else if constexpr (VB == 4) *reinterpret_cast<uint32_t*>(to) = *reinterpret_cast<const uint32_t*>(from);
+    else *to = *from;
+  }
+}
+
 }  // namespace
+
+int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t table_stride,
+                      const int32_t* cu_seq_lens, void* out, int64_t batch, int64_t total_rows,
+                      int64_t block_size, int64_t num_blocks, int64_t row_bytes, hipStream_t stream) {
+  if (batch == 0 || total_rows == 0) return XLLM_MI355_OK;
+  if (cache == nullptr || block_table == nullptr || cu_seq_lens == nullptr || out == nullptr) return XLLM_MI355_EINVAL;
+  if (batch < 0 || total_rows < 0 || batch > 0x7fffffffLL || table_stride <= 0 || block_size <= 0 ||
+      block_size > 0x7fffffffLL || num_blocks <= 0 || num_blocks > 0x7fffffffLL || row_bytes <= 0 ||
+      row_bytes > 0x7fffffffLL / 32)
+    return XLLM_MI355_EINVAL;
+  const int64_t n_groups = (total_rows + 31) / 32;
+  if (n_groups > 0x7fffffffLL) return XLLM_MI355_ESHAPE;
+  const dim3 grid(static_cast<unsigned>(n_groups));
+  const char* c = static_cast<const char*>(cache);
+  char* o = static_cast<char*>(out);
+  const bool a16 = ((reinterpret_cast<uintptr_t>(cache) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  const bool a4 = ((reinterpret_cast<uintptr_t>(cache) | reinterpret_cast<uintptr_t>(out)) & 3) == 0;
+  const int b = static_cast<int>(batch), bs = static_cast<int>(block_size), nb = static_cast<int>(num_blocks),
+            rb = static_cast<int>(row_bytes);
+  if (row_bytes % 16 == 0 && a16)
+    gather_paged_rows_kernel<16><<<grid, 256, 0, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
+  else if (row_bytes % 4 == 0 && a4)
+    gather_paged_rows_kernel<4><<<grid, 256, 0, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
+  else
+    gather_paged_rows_kernel<1><<<grid, 256, 0, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
+  return static_cast<int>(hipGetLastError());
+}
 
 size_t varlen_extra_bytes(int64_t n_tokens) {
   return n_tokens <= 0 ? 0 : (static_cast<size_t>(n_tokens) * 2 * 4 + 255) / 256 * 256;

@@ -10,6 +10,8 @@ Reference interface mirrored here (paths relative to the xLLM source tree):
   flash_mla::DenseDecodeParams / dense_decode     xllm/core/kernels/dcu/flash_mla_adapter.h:40-53
   merge_dcp_attention_shards                      xllm/core/layers/mlu/dcp_attention_merge.h:28-34
   build_block_table_from_paged_kv                 xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip
+  gather_mla_latent_cache                         xllm/core/kernels/dcu/dcu_ops_api.h:74
+  FlashAttentionImpl::paged_forward (q chunks)    xllm/core/layers/dcu/flash_attention.cpp:447-545
 
 Errors: the reference CHECK-aborts; here every violated precondition raises.
 """
@@ -367,3 +369,28 @@ def build_block_table_from_paged_kv(paged_kv_indptr, paged_kv_indices, paged_kv_
         table.data_ptr(), table_width, seq_lens.data_ptr(), B, block_size, _stream(dev))
     capi.check(rc, "xllm_mi355_build_block_table")
     return table, seq_lens
+
+
+def gather_mla_latent_cache(k_cache, block_table, kv_cu_seq_lens, total_kv_len, max_seq_len=0):
+    """dcu::gather_mla_latent_cache (kernels/dcu/dcu_ops_api.h:74, gather_mla_latent_cache.hip:124-190):
+    k_cache [P, bs, 1, D] contiguous, block_table [B, W] int32, kv_cu_seq_lens [B + 1] int32 ->
+    [total_kv_len, D] with the rows of sequence b at kv_cu_seq_lens[b] ...  max_seq_len only sizes the
+    reference's launch grid and is ignored."""
+    del max_seq_len
+    dev = _require_cuda(k_cache, block_table, kv_cu_seq_lens)
+    if k_cache.dim() != 4 or k_cache.shape[2] != 1 or not k_cache.is_contiguous():
+        raise ValueError("k_cache must be contiguous [blocks, block_size, 1, dim]")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise ValueError("block_table must be int32 [B, W] with unit column stride")
+    B = block_table.shape[0]
+    if kv_cu_seq_lens.dtype != torch.int32 or kv_cu_seq_lens.numel() != B + 1 or not kv_cu_seq_lens.is_contiguous():
+        raise ValueError("kv_cu_seq_lens must be contiguous int32 [B + 1]")
+    if total_kv_len <= 0:
+        raise ValueError("total_kv_len must be positive")
+    P, bs, _, D = k_cache.shape
+    out = torch.empty(total_kv_len, D, dtype=k_cache.dtype, device=dev)
+    rc = capi.lib().xllm_mi355_gather_paged_rows(
+        k_cache.data_ptr(), block_table.data_ptr(), block_table.stride(0), kv_cu_seq_lens.data_ptr(),
+        out.data_ptr(), B, total_kv_len, bs, P, D * k_cache.element_size(), _stream(dev))
+    capi.check(rc, "xllm_mi355_gather_paged_rows")
+    return out
