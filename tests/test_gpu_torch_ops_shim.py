@@ -85,3 +85,31 @@ def test_fp8_mla_and_merge_through_the_dispatcher(device, xops):
     mo, ml = xops.merge_dcp_attention_shards(torch.ones(2, 1, 1, 2, 3, device=device),
                                              torch.full((2, 1, 2, 1), -math.inf, device=device))
     assert torch.equal(mo.cpu(), torch.zeros(1, 1, 2, 3)) and torch.isneginf(ml).all()
+
+
+def test_query_chunks_and_latent_gather_through_the_dispatcher(device, xops):
+    cfg = workloads.DecodeConfig("shim_chunks", 5, 32, 8, 128, 16, 10, 600)
+    inp = workloads.make_inputs(cfg, 23)
+    lay = inp.layout
+    from helpers import fill_caches_gpu
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    g = torch.Generator().manual_seed(5)
+    q_lens = [int(torch.randint(1, min(16, int(L)) + 1, (1,), generator=g)) for L in lay.seq_lens]
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    q = (torch.randn(int(cu[-1]), cfg.n_q_heads, cfg.head_dim, generator=g) * cfg.sigma).to(torch.bfloat16).to(device)
+    out = xops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device),
+                             cu.to(device), cfg.scale, True, 0)
+    direct = ops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device),
+                               cu.to(device), scale=cfg.scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out, direct)
+    # latent gather with the reference's argument list
+    mla = workloads.DecodeConfig("shim_gather", 4, 16, 1, 576, 64, 1, 500, mla=True, v_dim=512)
+    inp = workloads.make_inputs(mla, 9)
+    lay = inp.layout
+    kc, _ = fill_caches_cpu(inp)
+    kv_cu = torch.zeros(mla.batch + 1, dtype=torch.int32)
+    kv_cu[1:] = lay.seq_lens.cumsum(0)
+    got = xops.gather_mla_latent_cache(kc.to(device), lay.block_table.to(device), kv_cu.to(device), int(kv_cu[-1]),
+                                       int(lay.seq_lens.max()))
+    assert torch.equal(got.cpu(), oracle.gather_paged_rows(kc, lay.block_table, kv_cu, int(kv_cu[-1])))

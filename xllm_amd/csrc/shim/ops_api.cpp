@@ -148,6 +148,63 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
   check_rc(rc, "xllm_mi355_paged_decode_gqa_csr");
 }
 
+void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torch::Tensor& k_cache,
+                   const torch::Tensor& v_cache, const torch::Tensor& block_table,
+                   const torch::Tensor& kv_seq_lens, const torch::Tensor& q_cu_seq_lens, float scale,
+                   bool is_causal, int64_t max_seq_len) {
+  TORCH_CHECK(query.is_cuda() && query.dim() == 3 && query.stride(2) == 1 && query.stride(1) == query.size(2),
+              "query must be a device tensor [T, Hq, D] with contiguous heads");
+  TORCH_CHECK(output.dim() == 3 && output.sizes() == query.sizes() && output.stride(2) == 1 &&
+                  output.stride(1) == output.size(2),
+              "output must match query");
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.sizes() == k_cache.sizes() &&
+                  v_cache.is_contiguous(),
+              "caches must be contiguous [P, bs, Hkv, D]");
+  const int64_t T = query.size(0), Hq = query.size(1), D = query.size(2), B = kv_seq_lens.numel();
+  TORCH_CHECK(block_table.scalar_type() == torch::kInt32 && block_table.dim() == 2 && block_table.stride(1) == 1 &&
+                  block_table.size(0) == B,
+              "block_table must be int32 [B, W]");
+  TORCH_CHECK(kv_seq_lens.scalar_type() == torch::kInt32 && kv_seq_lens.is_contiguous() &&
+                  q_cu_seq_lens.scalar_type() == torch::kInt32 && q_cu_seq_lens.is_contiguous() &&
+                  q_cu_seq_lens.numel() == B + 1,
+              "kv_seq_lens [B] and q_cu_seq_lens [B + 1] must be contiguous int32");
+  if (max_seq_len <= 0) max_seq_len = block_table.size(1) * k_cache.size(1);
+  const size_t nbytes = xllm_mi355_paged_decode_varlen_workspace_bytes(T, Hq, D);
+  torch::Tensor ws = decode_workspace(query.device(), nbytes);
+  const int rc = xllm_mi355_paged_decode_gqa_varlen(
+      query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
+      q_cu_seq_lens.data_ptr<int32_t>(), kv_seq_lens.data_ptr<int32_t>(), block_table.data_ptr<int32_t>(),
+      block_table.stride(0), nullptr, nullptr, B, T, Hq, k_cache.size(2), D, k_cache.size(1), k_cache.size(0),
+      query.stride(0), output.stride(0), max_seq_len, scale, is_causal ? 1 : 0, ws.data_ptr(),
+      static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
+  check_rc(rc, "xllm_mi355_paged_decode_gqa_varlen");
+}
+
+torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch::Tensor& block_table,
+                                      const torch::Tensor& kv_cu_seq_lens, int64_t total_kv_len,
+                                      int64_t max_seq_len) {
+  // the checks of xllm/core/kernels/dcu/gather_mla_latent_cache.hip:124-150
+  TORCH_CHECK(k_cache.defined() && block_table.defined() && kv_cu_seq_lens.defined(),
+              "gather_mla_latent_cache requires k_cache, block_table and kv_cu_seq_lens");
+  TORCH_CHECK(k_cache.is_cuda() && block_table.is_cuda() && kv_cu_seq_lens.is_cuda(), "tensors must be on the device");
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.size(2) == 1, "k_cache must be [blocks, block_size, 1, dim]");
+  TORCH_CHECK(block_table.dim() == 2, "block_table must be [batch, max_blocks]");
+  TORCH_CHECK(kv_cu_seq_lens.dim() == 1 && kv_cu_seq_lens.size(0) == block_table.size(0) + 1,
+              "kv_cu_seq_lens must be [batch + 1]");
+  TORCH_CHECK(total_kv_len > 0 && max_seq_len > 0, "total_kv_len and max_seq_len must be positive");
+  TORCH_CHECK(k_cache.is_contiguous(), "k_cache must be contiguous");
+  torch::Tensor table = (block_table.scalar_type() == torch::kInt32 ? block_table : block_table.to(torch::kInt32)).contiguous();
+  torch::Tensor cu = (kv_cu_seq_lens.scalar_type() == torch::kInt32 ? kv_cu_seq_lens : kv_cu_seq_lens.to(torch::kInt32)).contiguous();
+  torch::Tensor out = torch::empty({total_kv_len, k_cache.size(3)}, k_cache.options());
+  const int rc = xllm_mi355_gather_paged_rows(k_cache.data_ptr(), table.data_ptr<int32_t>(), table.stride(0),
+                                              cu.data_ptr<int32_t>(), out.data_ptr(), table.size(0), total_kv_len,
+                                              k_cache.size(1), k_cache.size(0),
+                                              k_cache.size(3) * static_cast<int64_t>(k_cache.element_size()),
+                                              current_stream(k_cache));
+  check_rc(rc, "xllm_mi355_gather_paged_rows");
+  return out;
+}
+
 namespace flash_mla {
 
 torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {
@@ -274,6 +331,19 @@ std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nop
   return {out, lse};
 }
 
+torch::Tensor op_paged_forward(torch::Tensor query, torch::Tensor output, torch::Tensor k_cache, torch::Tensor v_cache,
+                               torch::Tensor block_table, torch::Tensor kv_seq_lens, torch::Tensor q_cu_seq_lens,
+                               double scale, bool is_causal, int64_t max_seq_len) {
+  xllm::kernel::mi355::paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_cu_seq_lens,
+                                     static_cast<float>(scale), is_causal, max_seq_len);
+  return output;
+}
+
+torch::Tensor op_gather_mla_latent_cache(torch::Tensor k_cache, torch::Tensor block_table,
+                                         torch::Tensor kv_cu_seq_lens, int64_t total_kv_len, int64_t max_seq_len) {
+  return xllm::kernel::mi355::gather_mla_latent_cache(k_cache, block_table, kv_cu_seq_lens, total_kv_len, max_seq_len);
+}
+
 std::tuple<torch::Tensor, torch::Tensor> op_merge(torch::Tensor partial_outputs, torch::Tensor partial_lse) {
   auto r = xllm::layer::merge_dcp_attention_shards(partial_outputs, partial_lse);
   return {r.output, r.lse};
@@ -291,6 +361,10 @@ TORCH_LIBRARY(xllm_ops, m) {
   m.def("mla_dense_decode(Tensor q_nope, Tensor q_pe, Tensor k_cache, Tensor seqlens_k, Tensor block_table, "
         "int head_size_v, float softmax_scale) -> (Tensor, Tensor)");
   m.def("merge_dcp_attention_shards(Tensor partial_outputs, Tensor partial_lse) -> (Tensor, Tensor)");
+  m.def("paged_forward(Tensor query, Tensor(a!) output, Tensor k_cache, Tensor v_cache, Tensor block_table, "
+        "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len) -> Tensor");
+  m.def("gather_mla_latent_cache(Tensor k_cache, Tensor block_table, Tensor kv_cu_seq_lens, int total_kv_len, "
+        "int max_seq_len) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
@@ -299,4 +373,6 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("batch_decode", &op_batch_decode);
   m.impl("mla_dense_decode", &op_mla_dense_decode);
   m.impl("merge_dcp_attention_shards", &op_merge);
+  m.impl("paged_forward", &op_paged_forward);
+  m.impl("gather_mla_latent_cache", &op_gather_mla_latent_cache);
 }

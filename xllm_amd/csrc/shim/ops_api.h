@@ -55,6 +55,19 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
                       torch::Tensor paged_kv_last_page_len, double sm_scale, torch::Tensor output,
                       std::optional<torch::Tensor>& output_lse, int64_t max_seq_len);
 
+// Short query chunks against paged KV: the decode branch of FlashAttentionImpl::paged_forward
+// (xllm/core/layers/dcu/flash_attention.cpp:447-545).  query / output packed [T, Hq, D]; kv_seq_lens [B] are the
+// context lengths including the chunk, q_cu_seq_lens [B + 1] the chunk boundaries.
+void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torch::Tensor& k_cache,
+                   const torch::Tensor& v_cache, const torch::Tensor& block_table,
+                   const torch::Tensor& kv_seq_lens, const torch::Tensor& q_cu_seq_lens, float scale,
+                   bool is_causal, int64_t max_seq_len);
+
+// xllm::kernel::dcu::gather_mla_latent_cache (xllm/core/kernels/dcu/dcu_ops_api.h:74), same arguments.
+torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch::Tensor& block_table,
+                                      const torch::Tensor& kv_cu_seq_lens, int64_t total_kv_len,
+                                      int64_t max_seq_len);
+
 namespace flash_mla {
 struct DenseDecodeParams {
   torch::Tensor q_nope;       // [B, S_q, H, kv_lora_rank]
