@@ -179,9 +179,13 @@ int xllm_mi355_gather_paged_rows(const void* cache, const int32_t* block_table, 
  *     kv_seq_lens[b] - q_len + j + 1 tokens of its context when causal != 0 (the chunk is the
  *     tail of the context, AttentionMetadata::is_causal), to all kv_seq_lens[b] otherwise.
  * q/out: [n_tokens, Hq, D]; cu_seqlens_q: [B + 1] int32 starting at 0; block_table: [B, table_stride].
- * Every query token is decoded as an entry of its own against its sequence's pages, so the pages of a
- * sequence are read once per query token (mostly from L2): meant for the reference's limit of 16
- * tokens per chunk, correct for any.  Workspace: xllm_mi355_paged_decode_varlen_workspace_bytes.
+ * max_q_len is the caller's bound on the chunk lengths (AttentionMetadata::max_query_len), 0 if unknown.
+ * With a bound (head dim 128, block size a power of two >= 16, Hq / Hkv <= 8 or the whole chunk in 16 columns)
+ * the (token, head) pairs of a chunk share the 16 columns of the matrix-core kernel: the pages of a sequence
+ * are read once per 16 / (Hq / Hkv) query tokens, and a chunk longer than the bound is cut to it.  Otherwise
+ * every query token is decoded as an entry of its own against its sequence's pages (read once per token,
+ * partly from L2), which is correct for any length.
+ * Workspace: xllm_mi355_paged_decode_varlen_workspace_bytes(max(n_tokens, batch), ...).
  */
 size_t xllm_mi355_paged_decode_varlen_workspace_bytes(int64_t n_tokens, int64_t n_q_heads,
                                                       int64_t head_dim);
@@ -190,7 +194,8 @@ int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const
                                        const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
                                        const int32_t* block_table, int64_t table_stride,
                                        const float* k_scale, const float* v_scale,
-                                       int64_t batch, int64_t n_tokens, int64_t n_q_heads,
+                                       int64_t batch, int64_t n_tokens, int64_t max_q_len,
+                                       int64_t n_q_heads,
                                        int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
                                        int64_t num_blocks, int64_t q_token_stride,
                                        int64_t out_token_stride, int64_t max_seq_len, float sm_scale,

@@ -289,6 +289,38 @@ def test_short_query_chunks_through_the_decode_kernels(device):
             torch.cuda.synchronize()
             ref = oracle.aten_paged_forward(q, kc, vc, lay.block_table, lay.seq_lens, cu, cfg.scale, causal=causal)
             assert_close_to_reference(out, ref, f"{cfg.name} causal={causal}")
+    # chunks whose (token, head) pairs fit the 16 columns of the matrix-core kernel share one pass over the pages:
+    # group 4 with up to 4 tokens, group 8 with up to 2, one KV head per query head with up to 16; fp16; a
+    # sequence without query tokens; bounds larger than the chunks
+    for name, Hq, Hkv, bs, lo, hi, batch, bound, dt in (("g4", 32, 8, 16, 1, 900, 9, 4, torch.bfloat16),
+                                                        ("g8", 64, 8, 128, 300, 3000, 4, 2, torch.bfloat16),
+                                                        ("g1", 4, 4, 32, 20, 400, 5, 16, torch.float16),
+                                                        ("g2", 8, 4, 16, 1, 2000, 6, 8, torch.bfloat16),
+                                                        # longer chunks take several column blocks per KV head
+                                                        ("g4_16", 32, 8, 16, 40, 1200, 5, 16, torch.bfloat16),
+                                                        ("g8_7", 64, 8, 64, 30, 800, 4, 7, torch.bfloat16)):
+        cfg = workloads.DecodeConfig(f"packed_{name}", batch, Hq, Hkv, 128, bs, lo, hi)
+        inp = workloads.make_inputs(cfg, 70 + batch, dtype=dt)
+        lay = inp.layout
+        g = torch.Generator().manual_seed(7 + batch)
+        q_lens = [int(torch.randint(1, min(bound, int(L)) + 1, (1,), generator=g)) for L in lay.seq_lens]
+        q_lens[1] = 0                                   # a sequence that takes no part in this step
+        cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+        q = (torch.randn(int(cu[-1]), Hq, 128, generator=g) * cfg.sigma).to(dt)
+        kg, vg, _, _ = fill_caches_gpu(inp, device)
+        kc, vc = fill_caches_cpu(inp)
+        for causal in (True, False):
+            out = ops.paged_forward(q.to(device), torch.empty_like(q, device=device), kg, vg,
+                                    lay.block_table.to(device), lay.seq_lens.to(device), cu.to(device),
+                                    scale=cfg.scale, is_causal=causal, max_query_len=bound)
+            torch.cuda.synchronize()
+            ref = oracle.aten_paged_forward(q, kc, vc, lay.block_table, lay.seq_lens, cu, cfg.scale, causal=causal)
+            assert_close_to_reference(out, ref, f"{cfg.name} causal={causal}")
+            spread = ops.paged_forward(q.to(device), torch.empty_like(q, device=device), kg, vg,
+                                       lay.block_table.to(device), lay.seq_lens.to(device), cu.to(device),
+                                       scale=cfg.scale, is_causal=causal)      # one entry per token
+            torch.cuda.synchronize()
+            assert (out.float() - spread.float()).abs().max() < 2e-2
     # one token per sequence is plain decode, bit for bit
     cfg = workloads.DecodeConfig("chunks_one", 6, 32, 8, 128, 16, 1, 700)
     inp = workloads.make_inputs(cfg, 8)

@@ -98,7 +98,7 @@ def test_query_chunks_and_latent_gather_through_the_dispatcher(device, xops):
     cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
     q = (torch.randn(int(cu[-1]), cfg.n_q_heads, cfg.head_dim, generator=g) * cfg.sigma).to(torch.bfloat16).to(device)
     out = xops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device),
-                             cu.to(device), cfg.scale, True, 0)
+                             cu.to(device), cfg.scale, True, 0, 0)
     direct = ops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device),
                                cu.to(device), scale=cfg.scale)
     torch.cuda.synchronize()

@@ -33,7 +33,7 @@ SIGNATURES = {
                                                _i32, _p]),
     "xllm_mi355_gather_paged_rows": (_i32, [_p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "xllm_mi355_paged_decode_varlen_workspace_bytes": (_sz, [_i64, _i64, _i64]),
-    "xllm_mi355_paged_decode_gqa_varlen": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64,
+    "xllm_mi355_paged_decode_gqa_varlen": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64,
                                                   _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _p,
                                                   _sz, _i32, _i32, _p]),
     "xllm_mi355_paged_decode_mla": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64,

@@ -101,13 +101,13 @@ int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const
                                        const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
                                        const int32_t* block_table, int64_t table_stride,
                                        const float* k_scale, const float* v_scale, int64_t batch,
-                                       int64_t n_tokens, int64_t n_q_heads, int64_t n_kv_heads,
+                                       int64_t n_tokens, int64_t max_q_len, int64_t n_q_heads, int64_t n_kv_heads,
                                        int64_t head_dim, int64_t block_size, int64_t num_blocks,
                                        int64_t q_token_stride, int64_t out_token_stride,
                                        int64_t max_seq_len, float sm_scale, int causal, void* workspace,
                                        size_t workspace_bytes, int q_dtype, int cache_dtype, void* stream) {
   return paged_decode_gqa_varlen(q, k_cache, v_cache, out, cu_seqlens_q, kv_seq_lens, block_table,
-                                 table_stride, k_scale, v_scale, batch, n_tokens, n_q_heads, n_kv_heads,
+                                 table_stride, k_scale, v_scale, batch, n_tokens, max_q_len, n_q_heads, n_kv_heads,
                                  head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
                                  max_seq_len, sm_scale, causal, workspace, workspace_bytes, q_dtype,
                                  cache_dtype, static_cast<hipStream_t>(stream));

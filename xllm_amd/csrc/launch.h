@@ -26,6 +26,12 @@ struct PageAddressing {
   int64_t table_stride = 0;
   const int32_t* seq_lens = nullptr;     // [B]
   const int32_t* table_rows = nullptr;   // [B] block-table row of each entry, or null for row b (block-table form only)
+  // packed query chunks (block-table form, head dim 128 on the matrix-core kernel only): entry b is a sequence
+  // with cu_q[b + 1] - cu_q[b] <= chunk_blocks * (16 / group) query tokens; q / out hold n_tokens rows
+  const int32_t* cu_q = nullptr;         // [B + 1]
+  int64_t n_tokens = 0;
+  int chunk_blocks = 0;
+  int causal = 0;
   const int32_t* indptr = nullptr;       // CSR when non-null: [B+1]
   const int32_t* indices = nullptr;
   const int32_t* last_page_len = nullptr;
@@ -56,11 +62,11 @@ size_t varlen_extra_bytes(int64_t n_tokens);
 int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_cache, void* out,
                             const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
                             const int32_t* block_table, int64_t table_stride, const float* k_scale,
-                            const float* v_scale, int64_t batch, int64_t n_tokens, int64_t n_q_heads,
-                            int64_t n_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
-                            int64_t q_token_stride, int64_t out_token_stride, int64_t max_seq_len,
-                            float sm_scale, int causal, void* workspace, size_t workspace_bytes,
-                            int q_dtype, int cache_dtype, hipStream_t stream);
+                            const float* v_scale, int64_t batch, int64_t n_tokens, int64_t max_q_len,
+                            int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
+                            int64_t num_blocks, int64_t q_token_stride, int64_t out_token_stride,
+                            int64_t max_seq_len, float sm_scale, int causal, void* workspace,
+                            size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream);
 
 int lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,
               int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim, int dtype,

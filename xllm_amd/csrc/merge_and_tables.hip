@@ -173,15 +173,41 @@ size_t varlen_extra_bytes(int64_t n_tokens) {
 int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_cache, void* out,
                             const int32_t* cu_seqlens_q, const int32_t* kv_seq_lens,
                             const int32_t* block_table, int64_t table_stride, const float* k_scale,
-                            const float* v_scale, int64_t batch, int64_t n_tokens, int64_t n_q_heads,
-                            int64_t n_kv_heads, int64_t head_dim, int64_t block_size, int64_t num_blocks,
-                            int64_t q_token_stride, int64_t out_token_stride, int64_t max_seq_len,
-                            float sm_scale, int causal, void* workspace, size_t workspace_bytes,
-                            int q_dtype, int cache_dtype, hipStream_t stream) {
+                            const float* v_scale, int64_t batch, int64_t n_tokens, int64_t max_q_len,
+                            int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
+                            int64_t num_blocks, int64_t q_token_stride, int64_t out_token_stride,
+                            int64_t max_seq_len, float sm_scale, int causal, void* workspace,
+                            size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream) {
   if (batch == 0 || n_tokens == 0) return XLLM_MI355_OK;
   if (cu_seqlens_q == nullptr || kv_seq_lens == nullptr || block_table == nullptr || table_stride <= 0)
     return XLLM_MI355_EINVAL;
-  if (batch < 0 || n_tokens < 0 || batch > 0x7fffffffLL || n_tokens > 0x7fffffffLL) return XLLM_MI355_EINVAL;
+  if (batch < 0 || n_tokens < 0 || batch > 0x7fffffffLL || n_tokens > 0x7fffffffLL || n_q_heads <= 0 ||
+      n_kv_heads <= 0 || n_q_heads % n_kv_heads != 0)
+    return XLLM_MI355_EINVAL;
+  // The (token, head) pairs of a chunk share the 16 columns of the matrix-core kernel, 16 / group tokens per
+  // pass over the pages; the kernel cuts a chunk longer than the caller's bound.
+  const int64_t group = n_q_heads / n_kv_heads;
+  bool pow2 = false;
+  for (int s = 4; s < 31; ++s) pow2 |= (1LL << s) == block_size;
+  const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 7) == 0 && ((out_token_stride * 2) & 7) == 0;
+  // tokens per column block, column blocks per KV head; with one token per block (group 16) and several
+  // blocks an entry per token is cheaper, its repeated page reads being served partly by L2
+  const int64_t per = group <= 16 ? 16 / group : 0;
+  const int64_t blocks = per > 0 && max_q_len > 0 ? (max_q_len + per - 1) / per : 0;
+  if (blocks >= 1 && blocks <= 16 && (per >= 2 || blocks == 1) && head_dim == 128 && pow2 && out_aligned) {
+    PageAddressing addr;
+    addr.chunk_blocks = static_cast<int>(blocks);
+    addr.block_table = block_table;
+    addr.table_stride = table_stride;
+    addr.seq_lens = kv_seq_lens;
+    addr.cu_q = cu_seqlens_q;
+    addr.n_tokens = n_tokens;
+    addr.causal = causal;
+    return paged_decode_gqa(q, k_cache, v_cache, out, nullptr, addr, k_scale, v_scale, batch, n_q_heads,
+                            n_kv_heads, head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
+                            max_seq_len, sm_scale, workspace, workspace_bytes, q_dtype, cache_dtype, stream);
+  }
+  // Otherwise every query token becomes a decode entry of its own.
   const size_t extra = varlen_extra_bytes(n_tokens);
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 || workspace_bytes < extra)
     return XLLM_MI355_EWORKSPACE;

@@ -59,6 +59,10 @@ struct GqaArgs {
   float* lse;
   const int32_t* block_table;
   const int32_t* table_rows;  // block-table row of each batch entry, or null for row b (several query tokens of a sequence)
+  const int32_t* cu_q;        // packed query chunks (matrix-core kernel only): [batch + 1] token offsets, or null
+  int n_tokens;               // rows of q / out in that case
+  int chunk_blocks;           // column blocks per KV head in that case: ceil(longest chunk * group / 16)
+  int causal;                 // query token j of a chunk of n attends to the first L - n + j + 1 tokens
   const int32_t* seq_lens;
   const int32_t* indptr;
   const int32_t* indices;
@@ -601,6 +605,10 @@ struct CtxCursor {
   int b, hbk, st, n_st;
   int L;
   const int32_t* pages;
+  // packed query chunks: the sequence's chunk (first query token, number of tokens), and the part of it that
+  // the column block hbk % chunk_blocks holds: its first token, its number of tokens, and the index of its
+  // first token inside the chunk
+  int Q0, QN, q0, qn, jb;
 };
 
 template <int NS>
@@ -614,7 +622,11 @@ struct MfmaLayout {
   static constexpr int kPrefixOff = kTmpOff + kThreads * 4;
 };
 
-template <typename QT, bool FP8, int NS>
+// VL (packed query chunks): a batch entry is a sequence with cu_q[b + 1] - cu_q[b] query tokens.  The 16 MFMA
+// columns hold (token j, head h) pairs, column j * group + h, all against the same pages: 16 / group tokens
+// per column block, chunk_blocks column blocks per KV head, so a chunk costs the page traffic of
+// ceil(tokens * group / 16) single tokens; column j is masked beyond its own length.
+template <typename QT, bool FP8, int NS, bool VL>
 __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   static_assert(NS >= 2 && NS <= 4, "wait_younger_stages covers up to three stages in flight");
   using Lay = MfmaLayout<NS>;
@@ -638,8 +650,31 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   // whose transposing read takes 4 rows x 32 bytes per 16 lanes) or by its low three bits (fp8)
   auto swz_k = [](int row) { return row & (LPR - 1); };
   auto swz_v = [](int row) { return FP8 ? (row & 7) : ((row & 3) << 1); };
-  const int hb_per_kv = (a.group + G - 1) / G;
+  const int hb_per_kv = VL ? a.chunk_blocks : (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
+  // packed query chunks: the part of the sequence's chunk that column block cu.hbk holds
+  auto chunk_part = [&](CtxCursor& cu) {
+    if constexpr (VL) {
+      const int per = G / a.group;
+      cu.jb = (cu.hbk % hb_per_kv) * per;
+      cu.qn = max(0, min(cu.QN - cu.jb, per));
+      cu.q0 = cu.Q0 + cu.jb;
+    }
+  };
+  // ... after loading the chunk of sequence cu.b, its size clamped to what the column blocks hold
+  auto chunk_of = [&](CtxCursor& cu) {
+    if constexpr (VL) {
+      cu.Q0 = sload32(a.cu_q + cu.b);
+      cu.QN = max(0, min(sload32(a.cu_q + cu.b + 1) - cu.Q0, hb_per_kv * (G / a.group)));
+      chunk_part(cu);
+    }
+  };
+  // byte offset of column c's row in q (VL: token q0 + c / group, clamped into the buffer; head kvh * group + c % group)
+  auto q_row_offset = [&](const CtxCursor& cu, int kvh, int c) -> int64_t {
+    const int j = c / a.group;
+    const int tok = max(0, min(cu.q0 + j, a.n_tokens - 1));
+    return tok * a.q_stride_bytes + (static_cast<int64_t>(kvh * a.group + (c - j * a.group)) * D) * 2;
+  };
 
   item_prefix<T>(a, prefix, tmp);
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
@@ -675,16 +710,21 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
     cu.hbk = __builtin_amdgcn_readfirstlane(static_cast<int>(rem / cu.n_st));
     cu.st = __builtin_amdgcn_readfirstlane(static_cast<int>(rem - static_cast<int64_t>(cu.hbk) * cu.n_st));
     sequence_of_scalar(a, cu.b, cu.pages, cu.L);
+    chunk_of(cu);
   };
   auto next_context = [&](CtxCursor& cu) {  // the caller never steps past the last context of the batch
     cu.st = 0;
-    if (++cu.hbk < n_hb) return;
+    if (++cu.hbk < n_hb) {
+      chunk_part(cu);
+      return;
+    }
     cu.hbk = 0;
     do {
       ++cu.b;
       cu.n_st = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
     } while (cu.n_st == 0);
     sequence_of_scalar(a, cu.b, cu.pages, cu.L);
+    chunk_of(cu);
   };
   // 64 entries of the context's page table, from page 64 ck on (the tail repeats the last page),
   // into the chunk buffer at byte offset off
@@ -751,13 +791,22 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       // free: the consumer copied the previous context's rows to registers when it began that
       // context, at least NS stages ago.  After a shorter context the consumer loads Q itself.
       const int kvh = pc.hbk / hb_per_kv;
-      const int h0p = kvh * a.group + (pc.hbk % hb_per_kv) * G;
-      const int nhp = min(G, (kvh + 1) * a.group - h0p);
-      const char* qb = a.q + pc.b * a.q_stride_bytes;
+      if constexpr (VL) {
+        const int nhp = pc.qn * a.group;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = 4 * i + g;
-        dma16(qb + (static_cast<int64_t>(h0p + min(row, nhp - 1)) * D) * 2 + ((c16 ^ row) * 16), q_lds + i * 1024);
+        for (int i = 0; i < 4; ++i) {
+          const int row = 4 * i + g;
+          dma16(a.q + q_row_offset(pc, kvh, max(0, min(row, nhp - 1))) + ((c16 ^ row) * 16), q_lds + i * 1024);
+        }
+      } else {
+        const int h0p = kvh * a.group + (pc.hbk % hb_per_kv) * G;
+        const int nhp = min(G, (kvh + 1) * a.group - h0p);
+        const char* qb = a.q + pc.b * a.q_stride_bytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = 4 * i + g;
+          dma16(qb + (static_cast<int64_t>(h0p + min(row, nhp - 1)) * D) * 2 + ((c16 ^ row) * 16), q_lds + i * 1024);
+        }
       }
     }
   };
@@ -834,6 +883,8 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
   bool first_run = true;
   bool complete = false;
   int h0 = 0, nh = 0;
+  int Lc = 0;                 // tokens the lane's column attends to (the context length unless VL and causal)
+  int64_t out_off = 0;        // VL: byte offset of the lane's output row
   int c_ctx_first = 0, c_prev_len = 0;
   u32x4 q[4];
   f32x4 o[8];
@@ -859,8 +910,18 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
 
     if (s == 0 || cc.st == 0) {  // first stage of a run: the (sequence, head block) changes
       const int kvh = cc.hbk / hb_per_kv;
-      h0 = kvh * a.group + (cc.hbk % hb_per_kv) * G;
-      nh = min(G, (kvh + 1) * a.group - h0);
+      if constexpr (VL) {
+        nh = cc.qn * a.group;
+        const int col = max(0, min(c16, nh - 1));
+        const int j = col / a.group;
+        Lc = a.causal != 0 ? cc.L - (cc.QN - 1 - (cc.jb + j)) : cc.L;
+        const int tok = max(0, min(cc.q0 + j, a.n_tokens - 1));
+        out_off = tok * a.out_stride_bytes + (static_cast<int64_t>(kvh * a.group + (col - j * a.group)) * D) * 2;
+      } else {
+        h0 = kvh * a.group + (cc.hbk % hb_per_kv) * G;
+        nh = min(G, (kvh + 1) * a.group - h0);
+        Lc = cc.L;
+      }
       complete = cc.st == 0 && cc.n_st <= n_stages - s;
       if (s == 0 || c_prev_len >= NS) {
 #pragma unroll
@@ -868,9 +929,13 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
           q[kk] = *reinterpret_cast<const u32x4*>(qbuf + q_read + (((kk * 4 + g) ^ c16) * 16));
       } else {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk)
-          q[kk] = ldg16(a.q + cc.b * a.q_stride_bytes +
-                        (static_cast<int64_t>(h0 + min(c16, nh - 1)) * D + kk * 32 + g * 8) * 2);
+        for (int kk = 0; kk < 4; ++kk) {
+          if constexpr (VL)
+            q[kk] = ldg16(a.q + q_row_offset(cc, kvh, max(0, min(c16, nh - 1))) + (kk * 32 + g * 8) * 2);
+          else
+            q[kk] = ldg16(a.q + cc.b * a.q_stride_bytes +
+                          (static_cast<int64_t>(h0 + min(c16, nh - 1)) * D + kk * 32 + g * 8) * 2);
+        }
         // The wait for these loads (it also drains the stages in flight) must stay on this path:
         // left to the first use after the join it would run on every stage.
         asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]));
@@ -904,7 +969,7 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
       bool over = false;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        sv[r] = tok0 + r < cc.L ? sc[r] * score_scale : -INFINITY;
+        sv[r] = tok0 + r < Lc ? sc[r] * score_scale : -INFINITY;
         over |= sv[r] > m + kSlack;
       }
       if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
@@ -951,7 +1016,7 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
         const int tok0 = cc.st * T + tb * 16 + 4 * g;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          sv[tb * 4 + r] = tok0 + r < cc.L ? sc[r] * score_scale : -INFINITY;
+          sv[tb * 4 + r] = tok0 + r < Lc ? sc[r] * score_scale : -INFINITY;
           over |= sv[tb * 4 + r] > m + kSlack;
         }
       }
@@ -992,13 +1057,15 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
     const bool ctx_end = cc.st == cc.n_st - 1;
     if (ctx_end || s == n_stages - 1) {
       const float lsum = quad_rows_sum(l);
-      const float inv = out_scale / lsum;
+      // (VL: a column that attends to nothing -- a chunk longer than its context -- gives zeros)
+      const float inv = VL && !(lsum > 0.0f) ? 0.0f : out_scale / lsum;
       const float lse2 = m + fast_log2(lsum);
       const bool head_on = c16 < nh;
       const int hq = h0 + c16;
       const int64_t pidx = (worker * 2 + (first_run ? 0 : 1)) * G + c16;
       if (head_on && complete) {
-        char* op = a.out + cc.b * a.out_stride_bytes + (static_cast<int64_t>(hq) * D + 4 * g) * 2;
+        char* op = VL ? a.out + out_off + 4 * g * 2
+                      : a.out + cc.b * a.out_stride_bytes + (static_cast<int64_t>(hq) * D + 4 * g) * 2;
 #pragma unroll
         for (int mb = 0; mb < 8; ++mb) {
           const u32x2 w = {QT::pack(o[mb][0] * inv, o[mb][1] * inv), QT::pack(o[mb][2] * inv, o[mb][3] * inv)};
@@ -1013,7 +1080,7 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
           *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
         }
       }
-      if (head_on && g == 0 && complete && a.lse != nullptr) a.lse[cc.b * a.n_q_heads + hq] = lse2 * kLn2;
+      if (!VL && head_on && g == 0 && complete && a.lse != nullptr) a.lse[cc.b * a.n_q_heads + hq] = lse2 * kLn2;
       if (head_on && g == 0 && !complete) a.ws_lse[pidx] = lse2;
       first_run = false;
     }
@@ -1033,24 +1100,39 @@ __global__ __launch_bounds__(kThreads) void gqa_mfma_kernel(GqaArgs a) {
 // kernel is a chain of dependent round trips to memory, so it keeps them to two: the item
 // prefix, then the LSEs and accumulators of four consecutive workers at a time, all loads of a
 // group issued together.
-template <typename QT>
+// VL: the columns of a partial are (query token, head) pairs of the sequence's chunk (see gqa_mfma_kernel).
+template <typename QT, bool VL>
 __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int dv) {
   const int hbk = blockIdx.x;
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
   const int G = a.g_block;
   const int p0 = a.ws_prefix[b], p1 = a.ws_prefix[b + 1], pt = a.ws_prefix[a.batch];
-  const int hb_per_kv = (a.group + G - 1) / G;
+  const int hb_per_kv = VL ? a.chunk_blocks : (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
   const int kvh = hbk / hb_per_kv;
   const int h0 = kvh * a.group + (hbk - kvh * hb_per_kv) * G;
-  const int nh = min(G, (kvh + 1) * a.group - h0);
+  int q0 = 0, qn = 0;
+  if constexpr (VL) {  // the part of the chunk in this column block, as in the decode kernel
+    const int per = G / a.group;
+    const int jb = (hbk - kvh * hb_per_kv) * per;
+    const int QN = max(0, min(a.cu_q[b + 1] - a.cu_q[b], hb_per_kv * per));
+    q0 = a.cu_q[b] + jb;
+    qn = max(0, min(QN - jb, per));
+  }
+  const int nh = VL ? qn * a.group : min(G, (kvh + 1) * a.group - h0);
   const int dv4 = dv >> 2;         // 16-byte groups per head row
   const int n_vec = nh * dv4;      // per partial
   char* out_row = a.out + b * a.out_stride_bytes;
   const bool wide = ((reinterpret_cast<uintptr_t>(a.out) | static_cast<uintptr_t>(a.out_stride_bytes)) & 7) == 0;
   auto store4 = [&](int h, int d, float x0, float x1, float x2, float x3) {
     uint16_t* o = reinterpret_cast<uint16_t*>(out_row) + static_cast<int64_t>(h0 + h) * dv + d;
+    if constexpr (VL) {
+      const int j = h / a.group;
+      const int tok = max(0, min(q0 + j, a.n_tokens - 1));
+      o = reinterpret_cast<uint16_t*>(a.out + tok * a.out_stride_bytes) +
+          static_cast<int64_t>(kvh * a.group + (h - j * a.group)) * dv + d;
+    }
     if (wide) {
       const u32x2 w = {QT::pack(x0, x1), QT::pack(x2, x3)};
       *reinterpret_cast<u32x2*>(o) = w;
@@ -1065,7 +1147,7 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
   if (n_items <= 0) {  // empty sequence
     for (int v = tid; v < n_vec; v += kThreads) {
       store4(v / dv4, (v % dv4) * 4, 0.0f, 0.0f, 0.0f, 0.0f);
-      if (a.lse != nullptr && v % dv4 == 0) a.lse[b * a.n_q_heads + h0 + v / dv4] = -INFINITY;
+      if (!VL && a.lse != nullptr && v % dv4 == 0) a.lse[b * a.n_q_heads + h0 + v / dv4] = -INFINITY;
     }
     return;
   }
@@ -1116,9 +1198,9 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
       }
       M = m_new;
     }
-    const float inv = 1.0f / W;
+    const float inv = VL && !(W > 0.0f) ? 0.0f : 1.0f / W;
     store4(h, d, O[0] * inv, O[1] * inv, O[2] * inv, O[3] * inv);
-    if (a.lse != nullptr && d == 0) a.lse[b * a.n_q_heads + h0 + h] = (M + fast_log2(W)) * kLn2;
+    if (!VL && a.lse != nullptr && d == 0) a.lse[b * a.n_q_heads + h0 + h] = (M + fast_log2(W)) * kLn2;
   }
 }
 
@@ -1163,11 +1245,11 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
 
 constexpr int kMfmaStages = 4;
 
-template <typename QT, bool FP8>
+template <typename QT, bool FP8, bool VL = false>
 int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
   using Lay = MfmaLayout<kMfmaStages>;
   constexpr int D = 128;
-  auto kern = gqa_mfma_kernel<QT, FP8, kMfmaStages>;
+  auto kern = gqa_mfma_kernel<QT, FP8, kMfmaStages, VL>;
   static std::atomic<uint64_t> configured{0};
   if (first_use_on_current_device(configured)) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1286,19 +1368,32 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return XLLM_MI355_EWORKSPACE;
 
   const int group = static_cast<int>(n_q_heads / n_kv_heads);
+  const bool packed = addr.cu_q != nullptr;  // several query tokens per sequence in the MFMA columns
+  if (packed) {
+    const bool out_aligned = (reinterpret_cast<uintptr_t>(out) & 7) == 0 && ((out_token_stride * 2) & 7) == 0;
+    bool pow2 = false;
+    for (int s = 4; s < 31; ++s) pow2 |= (1LL << s) == block_size;
+    if (csr || lse != nullptr || head_dim != 128 || !pow2 || !out_aligned || group > kMfmaHeads ||
+        addr.n_tokens <= 0 || addr.n_tokens > 0x7fffffffLL || addr.chunk_blocks <= 0 || addr.chunk_blocks > kMfmaHeads)
+      return XLLM_MI355_EINVAL;
+  }
   // Batches beyond the LDS prefix capacity are decoded in slices; each slice is an
   // independent launch pair on the same stream and workspace.
   for (int64_t b0 = 0; b0 < batch; b0 += kMaxBatch) {
     const int64_t nb = batch - b0 < kMaxBatch ? batch - b0 : kMaxBatch;
     GqaArgs a = {};
-    a.q = static_cast<const char*>(q) + b0 * q_token_stride * 2;
+    a.q = static_cast<const char*>(q) + (packed ? 0 : b0 * q_token_stride * 2);
     a.k_cache = static_cast<const char*>(k_cache);
     a.v_cache = static_cast<const char*>(v_cache);
-    a.out = static_cast<char*>(out) + b0 * out_token_stride * 2;
+    a.out = static_cast<char*>(out) + (packed ? 0 : b0 * out_token_stride * 2);
     a.lse = lse == nullptr ? nullptr : lse + b0 * n_q_heads;
     a.block_table = csr ? nullptr : (addr.table_rows != nullptr ? addr.block_table : addr.block_table + b0 * addr.table_stride);
     a.table_rows = csr || addr.table_rows == nullptr ? nullptr : addr.table_rows + b0;
     a.seq_lens = csr ? nullptr : addr.seq_lens + b0;
+    a.cu_q = packed ? addr.cu_q + b0 : nullptr;
+    a.n_tokens = static_cast<int>(addr.n_tokens);
+    a.chunk_blocks = addr.chunk_blocks;
+    a.causal = addr.causal;
     a.indptr = csr ? addr.indptr + b0 : nullptr;
     a.indices = addr.indices;
     a.last_page_len = csr ? addr.last_page_len + b0 : nullptr;
@@ -1323,6 +1418,23 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
 
     size_t need = 0;
     int rc;
+    if (packed) {
+      if (q_dtype == XLLM_MI355_BF16)
+        rc = fp8 ? launch_gqa_mfma<BF16, true, true>(a, workspace_bytes, stream, false, &need)
+                 : launch_gqa_mfma<BF16, false, true>(a, workspace_bytes, stream, false, &need);
+      else
+        rc = fp8 ? launch_gqa_mfma<FP16, true, true>(a, workspace_bytes, stream, false, &need)
+                 : launch_gqa_mfma<FP16, false, true>(a, workspace_bytes, stream, false, &need);
+      if (rc != 0) return rc;
+      dim3 grid(static_cast<unsigned>(n_kv_heads * addr.chunk_blocks), static_cast<unsigned>(nb));
+      if (q_dtype == XLLM_MI355_BF16)
+        merge_partials_kernel<BF16, true><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+      else
+        merge_partials_kernel<FP16, true><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+      rc = static_cast<int>(hipGetLastError());
+      if (rc != 0) return rc;
+      continue;
+    }
     if (q_dtype == XLLM_MI355_BF16)
       rc = fp8 ? dispatch_dim<BF16, true>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need)
                : dispatch_dim<BF16, false>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need);
@@ -1333,9 +1445,9 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     const int hb_per_kv = (group + a.g_block - 1) / a.g_block;
     dim3 grid(static_cast<unsigned>(n_kv_heads * hb_per_kv), static_cast<unsigned>(nb));
     if (q_dtype == XLLM_MI355_BF16)
-      merge_partials_kernel<BF16><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+      merge_partials_kernel<BF16, false><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
     else
-      merge_partials_kernel<FP16><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+      merge_partials_kernel<FP16, false><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
     rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
   }

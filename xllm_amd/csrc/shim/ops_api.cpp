@@ -151,7 +151,7 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
 void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torch::Tensor& k_cache,
                    const torch::Tensor& v_cache, const torch::Tensor& block_table,
                    const torch::Tensor& kv_seq_lens, const torch::Tensor& q_cu_seq_lens, float scale,
-                   bool is_causal, int64_t max_seq_len) {
+                   bool is_causal, int64_t max_seq_len, int64_t max_query_len) {
   TORCH_CHECK(query.is_cuda() && query.dim() == 3 && query.stride(2) == 1 && query.stride(1) == query.size(2),
               "query must be a device tensor [T, Hq, D] with contiguous heads");
   TORCH_CHECK(output.dim() == 3 && output.sizes() == query.sizes() && output.stride(2) == 1 &&
@@ -169,12 +169,12 @@ void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torc
                   q_cu_seq_lens.numel() == B + 1,
               "kv_seq_lens [B] and q_cu_seq_lens [B + 1] must be contiguous int32");
   if (max_seq_len <= 0) max_seq_len = block_table.size(1) * k_cache.size(1);
-  const size_t nbytes = xllm_mi355_paged_decode_varlen_workspace_bytes(T, Hq, D);
+  const size_t nbytes = xllm_mi355_paged_decode_varlen_workspace_bytes(std::max(T, B), Hq, D);
   torch::Tensor ws = decode_workspace(query.device(), nbytes);
   const int rc = xllm_mi355_paged_decode_gqa_varlen(
       query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
       q_cu_seq_lens.data_ptr<int32_t>(), kv_seq_lens.data_ptr<int32_t>(), block_table.data_ptr<int32_t>(),
-      block_table.stride(0), nullptr, nullptr, B, T, Hq, k_cache.size(2), D, k_cache.size(1), k_cache.size(0),
+      block_table.stride(0), nullptr, nullptr, B, T, max_query_len, Hq, k_cache.size(2), D, k_cache.size(1), k_cache.size(0),
       query.stride(0), output.stride(0), max_seq_len, scale, is_causal ? 1 : 0, ws.data_ptr(),
       static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
   check_rc(rc, "xllm_mi355_paged_decode_gqa_varlen");
@@ -333,9 +333,9 @@ std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nop
 
 torch::Tensor op_paged_forward(torch::Tensor query, torch::Tensor output, torch::Tensor k_cache, torch::Tensor v_cache,
                                torch::Tensor block_table, torch::Tensor kv_seq_lens, torch::Tensor q_cu_seq_lens,
-                               double scale, bool is_causal, int64_t max_seq_len) {
+                               double scale, bool is_causal, int64_t max_seq_len, int64_t max_query_len) {
   xllm::kernel::mi355::paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_cu_seq_lens,
-                                     static_cast<float>(scale), is_causal, max_seq_len);
+                                     static_cast<float>(scale), is_causal, max_seq_len, max_query_len);
   return output;
 }
 
@@ -362,7 +362,7 @@ TORCH_LIBRARY(xllm_ops, m) {
         "int head_size_v, float softmax_scale) -> (Tensor, Tensor)");
   m.def("merge_dcp_attention_shards(Tensor partial_outputs, Tensor partial_lse) -> (Tensor, Tensor)");
   m.def("paged_forward(Tensor query, Tensor(a!) output, Tensor k_cache, Tensor v_cache, Tensor block_table, "
-        "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len) -> Tensor");
+        "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len, int max_query_len) -> Tensor");
   m.def("gather_mla_latent_cache(Tensor k_cache, Tensor block_table, Tensor kv_cu_seq_lens, int total_kv_len, "
         "int max_seq_len) -> Tensor");
 }

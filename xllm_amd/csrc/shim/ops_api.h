@@ -57,11 +57,12 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
 
 // Short query chunks against paged KV: the decode branch of FlashAttentionImpl::paged_forward
 // (xllm/core/layers/dcu/flash_attention.cpp:447-545).  query / output packed [T, Hq, D]; kv_seq_lens [B] are the
-// context lengths including the chunk, q_cu_seq_lens [B + 1] the chunk boundaries.
+// context lengths including the chunk, q_cu_seq_lens [B + 1] the chunk boundaries, max_query_len the bound on
+// the chunk lengths (AttentionMetadata::max_query_len; 0 = unknown).
 void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torch::Tensor& k_cache,
                    const torch::Tensor& v_cache, const torch::Tensor& block_table,
                    const torch::Tensor& kv_seq_lens, const torch::Tensor& q_cu_seq_lens, float scale,
-                   bool is_causal, int64_t max_seq_len);
+                   bool is_causal, int64_t max_seq_len, int64_t max_query_len);
 
 // xllm::kernel::dcu::gather_mla_latent_cache (xllm/core/kernels/dcu/dcu_ops_api.h:74), same arguments.
 torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch::Tensor& block_table,

@@ -238,12 +238,14 @@ def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
 
 
 def paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_cu_seq_lens, scale=None,
-                  is_causal=True, max_seq_len=0, k_cache_quant_scale=None, v_cache_quant_scale=None):
+                  is_causal=True, max_seq_len=0, k_cache_quant_scale=None, v_cache_quant_scale=None,
+                  max_query_len=0):
     """Short query chunks (chunked prefill, speculative-decoding verification) against paged KV:
     the decode branch of FlashAttentionImpl::paged_forward (layers/dcu/flash_attention.cpp:447-545).
     query/output packed [T, Hq, D]; q_cu_seq_lens [B + 1] int32 from 0 to T; kv_seq_lens [B] int32 are
     the context lengths INCLUDING the chunk; with is_causal token j of a chunk of q_len tokens attends
-    to the first kv_len - q_len + j + 1 tokens.  Returns output."""
+    to the first kv_len - q_len + j + 1 tokens.  max_query_len (AttentionMetadata::max_query_len) bounds the
+    chunk lengths; 0 = unknown.  Returns output."""
     dev = _require_cuda(query, k_cache, v_cache, output, block_table, kv_seq_lens, q_cu_seq_lens,
                         k_cache_quant_scale, v_cache_quant_scale)
     _decode_common(query, k_cache, output)
@@ -262,12 +264,12 @@ def paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_c
     if max_seq_len <= 0:
         max_seq_len = block_table.shape[1] * bs
     lib = capi.lib()
-    nbytes = lib.xllm_mi355_paged_decode_varlen_workspace_bytes(T, Hq, D)
+    nbytes = lib.xllm_mi355_paged_decode_varlen_workspace_bytes(max(T, B), Hq, D)
     ws = decode_workspace(dev, nbytes)
     rc = lib.xllm_mi355_paged_decode_gqa_varlen(
         query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
         q_cu_seq_lens.data_ptr(), kv_seq_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
-        _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, T, Hq, Hkv, D, bs, P,
+        _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, T, int(max_query_len), Hq, Hkv, D, bs, P,
         query.stride(0), output.stride(0), max_seq_len, float(scale), 1 if is_causal else 0,
         ws.data_ptr(), ws.numel(), _dtype_code(query), _dtype_code(k_cache), _stream(dev))
     capi.check(rc, "xllm_mi355_paged_decode_gqa_varlen")
