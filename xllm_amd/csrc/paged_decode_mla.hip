@@ -105,14 +105,15 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 }
 
 // 16 bytes per active lane from global memory straight into LDS at lds_addr + lane * 16
-// (lds_addr is wave-uniform; it travels in M0).
+// (lds_addr is wave-uniform; it travels in M0).  Every tile load of this file is marked non-temporal:
+// a launch reads each latent row once, and streaming reads that bypass the caches move faster on this GPU.
 __device__ __forceinline__ void dma16(const void* gptr, u32 lds_addr) {
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(gptr) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(base), "v"(gptr) : "memory");
 }
 // Same with a wave-uniform 64-bit row base in SGPRs plus a 32-bit per-lane byte offset.
 __device__ __forceinline__ void dma16_row(uint64_t row_base, u32 lane_off, u32 lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(lane_off), "s"(row_base)
                : "memory");
 }
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -479,7 +480,7 @@ __device__ __forceinline__ void dma4(const void* gptr, u32 lds_addr) {
 __device__ __forceinline__ void dma_rows4(uint64_t base, u32 lane_off, u32 lds_addr, bool rope) {
   constexpr int kPad = kRow16 - kRowBytes;  // 32
 #define XLLM_DMA(lds, gbase, m0_add, goff)                                                               \
-  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4" ::"s"(lds), \
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4 nt" ::"s"(lds), \
                "v"(lane_off), "s"(gbase), "n"(m0_add), "n"(goff)                                         \
                : "memory", "scc")
   // instruction offsets reach 4095: rows 2 and 3 go through a second base
@@ -816,7 +817,7 @@ constexpr float kPSlack = 24.0f;                  // a reference follows scores 
 constexpr float kPRefInit = -1048576.0f;           // reference before any score was seen (integer valued)
 
 #define XLLM_DMA_ROWP(lds, gbase, lane_off, lds_off)                                                      \
-  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(lane_off), \
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds), "v"(lane_off), \
                "s"(gbase), "n"(lds_off)                                                                   \
                : "memory", "scc")
 
@@ -826,7 +827,7 @@ constexpr float kPRefInit = -1048576.0f;           // reference before any score
   do {                                                                                                     \
     uint64_t saved_;                                                                                       \
     asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, exec, %5\n\ts_add_u32 m0, %1, %4\n\ts_nop 0\n\t"  \
-                 "global_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"                                     \
+                 "global_load_lds_dwordx4 %2, %3 nt\n\ts_mov_b64 exec, %0"                                   \
                  : "=&s"(saved_)                                                                           \
                  : "s"(lds), "v"(lane_off), "s"(gbase), "n"(lds_off), "s"(mask)                            \
                  : "memory", "scc");                                                                       \
@@ -835,7 +836,7 @@ __device__ __forceinline__ void dma16_masked(const void* gptr, u32 lds_addr, uin
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
   uint64_t saved;
   asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, exec, %3\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-               "global_load_lds_dwordx4 %2, off\n\ts_mov_b64 exec, %0"
+               "global_load_lds_dwordx4 %2, off nt\n\ts_mov_b64 exec, %0"
                : "=&s"(saved)
                : "s"(base), "v"(gptr), "s"(mask)
                : "memory", "scc");
