@@ -269,14 +269,14 @@ def test_full_size_config2_split_invariance_and_sampled_parity(device):
 
 
 def test_shared_tail_of_the_item_list(device, monkeypatch):
-    # Batches long enough that the matrix-core kernel leaves the end of its item list to whoever is free
-    # (chunks taken from a counter in the workspace).  Every sequence against the oracle; against the same
-    # launch with everything dealt out in advance (XLLM_MI355_GQA_TAIL=0); launches in a row on one
-    # workspace; a captured launch replayed (its counter tag repeats) with eager launches in between.
+    # XLLM_MI355_GQA_TAIL=1: the matrix-core kernel leaves the end of a long item list to whoever is free
+    # (chunks taken from a counter in the workspace).  Sampled sequences against the oracle; against the same
+    # launch with everything dealt out in advance (the default); launches in a row on one workspace; a
+    # captured launch replayed (its counter tag repeats) with eager launches in between.
     def both(run):
-        monkeypatch.setenv("XLLM_MI355_GQA_TAIL", "0")
+        monkeypatch.delenv("XLLM_MI355_GQA_TAIL", raising=False)
         fixed = run()
-        monkeypatch.delenv("XLLM_MI355_GQA_TAIL")
+        monkeypatch.setenv("XLLM_MI355_GQA_TAIL", "1")
         shared = run()
         again = run()
         assert torch.equal(shared, again)

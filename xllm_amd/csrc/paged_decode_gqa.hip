@@ -150,7 +150,7 @@ __device__ __forceinline__ Pieces pieces_of(int64_t total, int64_t n, bool share
   if (!shared_tail) return p;
   // Chunks are at least kMinChunk items long (a worker fetches the operands of its next run while it
   // works on a run of at least that length) and the tail is about 22 % of the list.  Shorter lists are
-  // dealt out whole: there the partials of the chunks cost the merge kernel more than the launch gains.
+  // dealt out whole.
   const int64_t per = total / n;
   const int rounds = kTailRounds;
   if (static_cast<int64_t>(kMinChunk) * ((1 << rounds) - 1) * 100 > per * 45) return p;
@@ -590,6 +590,7 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((ext_vector_type(2))) int i32x2;
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
+typedef __attribute__((address_space(3))) volatile int lds_vint;  // a word of LDS that other wavefronts write
 typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 
@@ -680,6 +681,7 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
 // Position of a stage in the flat list (sequence, head block, stage of 16 tokens).
 struct CtxCursor {
   int b, hbk, st, n_st;
+  int kvh;  // KV head of the head block: hbk / (head blocks per KV head)
   int L;
   const int32_t* pages;
   // packed query chunks: the sequence's chunk (first query token, number of tokens), and the part of it that
@@ -687,6 +689,26 @@ struct CtxCursor {
   // first token inside the chunk
   int Q0, QN, q0, qn, jb;
 };
+// Field by field, and the chunk fields only where they are in use: a whole-struct copy with fields that
+// were never written goes through scratch memory, whose loads count on the same counter as the stages
+// in flight.
+template <bool VL>
+__device__ __forceinline__ void copy_cursor(CtxCursor& d, const CtxCursor& s) {
+  d.b = s.b;
+  d.hbk = s.hbk;
+  d.kvh = s.kvh;
+  d.st = s.st;
+  d.n_st = s.n_st;
+  d.L = s.L;
+  d.pages = s.pages;
+  if constexpr (VL) {
+    d.Q0 = s.Q0;
+    d.QN = s.QN;
+    d.q0 = s.q0;
+    d.qn = s.qn;
+    d.jb = s.jb;
+  }
+}
 
 constexpr int kPieceRing = 8;           // pieces a worker knows of and has not finished (at most 3)
 constexpr int kLookAhead = 8;           // stages before the end of a piece at which the next one is asked for
@@ -764,7 +786,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
 
   // mailboxes: mail[w] = 0 idle, 1 worker w asks for a chunk, chunk + 2 or kMailNone the answer;
   // mail[kWaves + w] != 0: worker w has finished
-  volatile int* mail = reinterpret_cast<volatile int*>(smem + Lay::kMailOff);
+  lds_vint* mail = (lds_vint*)(smem + Lay::kMailOff);
   if (tid < 2 * kWaves) mail[tid] = 0;
   item_prefix<T>(a, prefix, tmp);
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
@@ -797,7 +819,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     return;
   }
   // pieces the producer has opened, for the consumer that follows it: first item, items, piece number
-  volatile int* piece_ring = reinterpret_cast<volatile int*>(smem + Lay::kPieceOff + wave * kPieceRing * 16);
+  lds_vint* piece_ring = (lds_vint*)(smem + Lay::kPieceOff + wave * kPieceRing * 16);
 
   const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
   const u32 ring_lds = __builtin_amdgcn_readfirstlane(lds_base + wave * NS * kStageBytes);
@@ -818,16 +840,19 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     const int64_t rem = f - static_cast<int64_t>(prefix[cu.b]) * n_hb;
     cu.hbk = __builtin_amdgcn_readfirstlane(static_cast<int>(rem / cu.n_st));
     cu.st = __builtin_amdgcn_readfirstlane(static_cast<int>(rem - static_cast<int64_t>(cu.hbk) * cu.n_st));
+    cu.kvh = cu.hbk / hb_per_kv;
     sequence_of_scalar(a, cu.b, cu.pages, cu.L);
     chunk_of(cu);
   };
   auto next_context = [&](CtxCursor& cu) {  // the caller never steps past the last context of the batch
     cu.st = 0;
     if (++cu.hbk < n_hb) {
+      cu.kvh = cu.hbk / hb_per_kv;
       chunk_part(cu);
       return;
     }
     cu.hbk = 0;
+    cu.kvh = 0;
     do {
       ++cu.b;
       cu.n_st = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
@@ -868,7 +893,8 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // range, then chunks of the shared tail while there are any); pc is the context of stage p
   CtxCursor pc;
   locate(cur, pc);
-  CtxCursor pn = pc;                         // the context after pc (valid while has_c)
+  CtxCursor pn;                              // the context after pc (valid while has_c)
+  copy_cursor<VL>(pn, pc);
   int p = 0;
   int p_end = static_cast<int>(end - cur);   // first stage past the producer's piece
   int p_pieces = 0;                          // pieces opened after the first
@@ -905,7 +931,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     p_ctx_first = p;
     need_piece = !(pc.n_st - pc.st < p_end - p);
     if (!need_piece) {  // the piece goes on into another context
-      pn = pc;
+      copy_cursor<VL>(pn, pc);
       next_context(pn);
       issue_chunk(pn, 0, off_c);
       ck_c = 0;
@@ -923,7 +949,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       // past the group repeat the last head; the consumer zeroes them).  The single buffer is
       // free: the consumer copied the previous context's rows to registers when it began that
       // context, at least NS stages ago.  After a shorter context the consumer loads Q itself.
-      const int kvh = pc.hbk / hb_per_kv;
+      const int kvh = pc.kvh;
       if constexpr (VL) {
         const int nhp = pc.qn * a.group;
 #pragma unroll
@@ -969,7 +995,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     int64_t f, e;
     pieces.chunk_range(v - 2, f, e);
     nx_len = static_cast<int>(e - f);
-    volatile int* rec = piece_ring + ((p_pieces + 1) & (kPieceRing - 1)) * 4;
+    lds_vint* rec = piece_ring + ((p_pieces + 1) & (kPieceRing - 1)) * 4;
     rec[0] = static_cast<int>(f);
     rec[1] = static_cast<int>(f >> 32);
     rec[2] = nx_len;
@@ -986,19 +1012,19 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       begin_context(true);
     } else if (p == p_end) {  // into the next piece (known: see produce)
       p_prev_len = p - p_ctx_first;
-      pc = pn;
+      copy_cursor<VL>(pc, pn);
       ++p_pieces;
       p_end += nx_len;
       nx_state = 0;
       begin_context(false);
     } else if (pc.st == pc.n_st) {
       p_prev_len = p - p_ctx_first;
-      pc = pn;
+      copy_cursor<VL>(pc, pn);
       begin_context(false);
     }
     const int tok0 = pc.st * T;
     const int lim = pc.L - tok0 - 1;  // last valid row of the stage
-    // block_size >= 16: a sub-block of 16 tokens lies in one page
+    // block size >= 16: a sub-block of 16 tokens lies in one page
     constexpr int NSUB = T / 16;
     uint64_t kb[NSUB], vb[NSUB];
 #pragma unroll
@@ -1024,7 +1050,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
         const int slot0 = page * a.block_size + (tok & (a.block_size - 1));
         const uint64_t row0 = static_cast<uint64_t>(slot0) * static_cast<uint64_t>(a.row_bytes) +
-                              static_cast<uint64_t>(pc.hbk / hb_per_kv) * RB;
+                              static_cast<uint64_t>(pc.kvh) * RB;
         kb[sub] = reinterpret_cast<uint64_t>(a.k_cache) + row0;
         vb[sub] = reinterpret_cast<uint64_t>(a.v_cache) + row0;
       } else {  // past the end of the context: its rows repeat the last valid one
@@ -1088,7 +1114,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
 
     if (run_start) {  // first stage of a run: the (sequence, head block) or the piece changes
       run_start = false;
-      const int kvh = cc.hbk / hb_per_kv;
+      const int kvh = cc.kvh;
       if constexpr (VL) {
         nh = cc.qn * a.group;
         const int col = max(0, min(c16, nh - 1));
@@ -1270,7 +1296,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       // one, if there is one.
       if (c_pieces < p_pieces) {
         ++c_pieces;
-        volatile int* rec = piece_ring + (c_pieces & (kPieceRing - 1)) * 4;
+        lds_vint* rec = piece_ring + (c_pieces & (kPieceRing - 1)) * 4;
         const int64_t f = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(rec[1])) << 32) |
                           static_cast<u32>(__builtin_amdgcn_readfirstlane(rec[0]));
         c_end += __builtin_amdgcn_readfirstlane(rec[2]);
@@ -1472,8 +1498,11 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   const int n_wg = device_cu_count();  // the ring fills a CU's LDS: one workgroup each
   a.n_workgroups = n_wg * kWaves;      // independent workers = wavefronts
   // workspace: counter of the shared tail (256 bytes) | item prefix | partials, two slots per piece
-  const char* tail_knob = getenv("XLLM_MI355_GQA_TAIL");  // "0": every item dealt out in advance (A/B measurements)
-  const bool shared_tail = !(tail_knob != nullptr && tail_knob[0] == '0');
+  // "1": leave the end of long item lists to whoever is free.  Off by default: with non-temporal loads the
+  // launch gains at most 1-2 % from it and the merge kernel, which then folds several times as many
+  // partials, loses more than that.
+  const char* tail_knob = getenv("XLLM_MI355_GQA_TAIL");
+  const bool shared_tail = tail_knob != nullptr && tail_knob[0] == '1';
   static std::atomic<unsigned> launches{0};
   const size_t n_pieces = static_cast<size_t>(a.n_workgroups) * (1 + kTailRounds);
   const size_t prefix_bytes = ((static_cast<size_t>(a.batch) + 1) * 4 + 255) / 256 * 256;
