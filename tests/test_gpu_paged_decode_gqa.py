@@ -268,33 +268,28 @@ def test_full_size_config2_split_invariance_and_sampled_parity(device):
     assert torch.allclose(mlse.view_as(lse), lse, rtol=1e-3, atol=1e-3)
 
 
-def test_shared_tail_of_the_item_list(device, monkeypatch):
-    # XLLM_MI355_GQA_TAIL=1: the matrix-core kernel leaves the end of a long item list to whoever is free
-    # (chunks taken from a counter in the workspace).  Sampled sequences against the oracle; against the same
-    # launch with everything dealt out in advance (the default); launches in a row on one workspace; a
-    # captured launch replayed (its counter tag repeats) with eager launches in between.
-    def both(run):
-        monkeypatch.delenv("XLLM_MI355_GQA_TAIL", raising=False)
-        fixed = run()
-        monkeypatch.setenv("XLLM_MI355_GQA_TAIL", "1")
-        shared = run()
+def test_long_item_lists_of_the_matrix_core_kernel(device):
+    # Batches that give every pair of wavefronts of the matrix-core kernel 140 to 330 stages (the loading
+    # wavefront laps the ring of its pair dozens of times): sampled sequences against the oracle, launches in a
+    # row on one workspace bit-identical, a captured launch replayed with eager launches in between.
+    def twice(run):
+        first = run()
         again = run()
-        assert torch.equal(shared, again)
-        assert (shared.float() - fixed.float()).abs().max() < 2e-2
-        return shared
+        torch.cuda.synchronize()
+        assert torch.equal(first, again)
+        return first
 
-    # 16-bit pages: 140 and 330 stages of 16 tokens per wavefront (a shared tail needs about 134)
     for batch, lo, hi in ((64, 3000, 6000), (150, 3000, 6000)):
-        cfg = workloads.DecodeConfig(f"tail_b{batch}", batch, 32, 8, 128, 16, lo, hi)
+        cfg = workloads.DecodeConfig(f"long_b{batch}", batch, 32, 8, 128, 16, lo, hi)
         inp = workloads.make_inputs(cfg, 900 + batch, device=device)
         lay = inp.layout
         kg, vg, _, _ = fill_caches_gpu(inp, device)
-        out = both(lambda: _decode_gpu(inp, kg, vg, device)[0])
+        out = twice(lambda: _decode_gpu(inp, kg, vg, device)[0])
         sample = list(range(0, batch, 5)) + list(range(batch - 12, batch))
         ref = oracle.aten_paged_decode(inp.q.cpu()[sample].contiguous(), kg.cpu(), vg.cpu(),
                                        lay.block_table[sample].contiguous(), lay.seq_lens[sample].contiguous(), cfg.scale)
         assert_close_to_reference(out[sample], ref, cfg.name)
-        if batch == 64:  # replays of a captured launch, eager launches of other batches between them
+        if batch == 64:
             q, table, lens = inp.q.to(device), lay.block_table.to(device), lay.seq_lens.to(device)
             captured = torch.zeros_like(q)
             graph = torch.cuda.CUDAGraph()
@@ -307,17 +302,17 @@ def test_shared_tail_of_the_item_list(device, monkeypatch):
                 assert torch.equal(captured, out), f"replay {rep}"
                 assert torch.equal(_decode_gpu(inp, kg, vg, device)[0], out)
     # fp8 pages (stages of 32 tokens) and query chunks in the MFMA columns
-    cfg = workloads.DecodeConfig("tail_fp8", 192, 32, 8, 128, 16, 2000, 4000, cache_dtype="fp8")
+    cfg = workloads.DecodeConfig("long_fp8", 192, 32, 8, 128, 16, 2000, 4000, cache_dtype="fp8")
     inp = workloads.make_inputs(cfg, 77, device=device)
     lay = inp.layout
     kg, vg, ks, vs = fill_caches_gpu(inp, device, cache_dtype=torch.float8_e4m3fn)
-    out = both(lambda: _decode_gpu(inp, kg, vg, device, ks, vs)[0])
+    out = twice(lambda: _decode_gpu(inp, kg, vg, device, ks, vs)[0])
     sample = list(range(0, 192, 17)) + list(range(184, 192))
     ref = oracle.aten_paged_decode(inp.q.cpu()[sample].contiguous(), kg.cpu(), vg.cpu(), lay.block_table[sample].contiguous(),
                                    lay.seq_lens[sample].contiguous(), cfg.scale, ks.cpu(), vs.cpu())
     assert_close_to_reference(out[sample], ref, cfg.name)
 
-    cfg = workloads.DecodeConfig("tail_chunks", 64, 32, 8, 128, 16, 3000, 6000)
+    cfg = workloads.DecodeConfig("long_chunks", 64, 32, 8, 128, 16, 3000, 6000)
     inp = workloads.make_inputs(cfg, 78, device=device)
     lay = inp.layout
     kg, vg, _, _ = fill_caches_gpu(inp, device)
@@ -325,9 +320,8 @@ def test_shared_tail_of_the_item_list(device, monkeypatch):
     q_lens = torch.randint(1, 5, (cfg.batch,), generator=g)
     cu = torch.tensor([0] + list(q_lens.cumsum(0)), dtype=torch.int32)
     q = (torch.randn(int(cu[-1]), 32, 128, generator=g) * cfg.sigma).to(torch.bfloat16).to(device)
-    out = both(lambda: ops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device),
-                                         cu.to(device), scale=cfg.scale, is_causal=True, max_query_len=4))
-    torch.cuda.synchronize()
+    out = twice(lambda: ops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device),
+                                          cu.to(device), scale=cfg.scale, is_causal=True, max_query_len=4))
     ref = oracle.aten_paged_forward(q.cpu(), kg.cpu(), vg.cpu(), lay.block_table, lay.seq_lens, cu, cfg.scale, causal=True)
     assert_close_to_reference(out, ref, cfg.name)
 

@@ -84,10 +84,8 @@ struct GqaArgs {
   int block_size;
   int bs_shift;       // log2(block_size) or -1
   int num_blocks;
-  int n_workgroups;   // workers of the decode kernel (workgroups, or wavefronts of the matrix-core kernel)
+  int n_workgroups;   // workers of the decode kernel (workgroups; wavefront pairs of the matrix-core kernel)
   float scale_log2;   // sm_scale * log2(e)
-  unsigned long long* tickets;  // matrix-core kernel: counter of the shared tail of the item list, or null
-  unsigned launch_id;           // nonzero, differs from launch to launch (tag of the counter's contents)
 };
 
 __device__ __forceinline__ void sequence_of(const GqaArgs& a, int b, const int32_t*& pages, int& L) {
@@ -113,75 +111,6 @@ __device__ __forceinline__ int workgroup_of(int64_t id, int64_t total, int64_t n
   int64_t w = id * n / total;
   while (w + 1 < n && range_start(w + 1, total, n) <= id) ++w;
   return static_cast<int>(w);
-}
-
-// Split of the flat item list into pieces.  Pieces 0 .. n - 1 are the workers' own equal ranges of the
-// first `head` items.  When the list is long enough, its last fifth or so is not dealt out in advance: it
-// is cut into `rounds` rounds of n chunks each, the chunks of a round half as long as those of the round
-// before (unit << (rounds - 1 - round) items), and a worker that has finished a piece takes the next chunk
-// (piece n + t for chunk t) from a shared counter.  Workers read their items at different speeds -- by
-// 10-20 % on this GPU, by position on the die and by luck -- and a launch ends with its slowest worker;
-// the shared tail lets the fast ones take more.  Every piece owns two partial slots, as a worker does.
-constexpr int kTailRounds = 4;
-constexpr int kMinChunk = 4;
-struct Pieces {
-  int64_t head;   // items dealt out in advance
-  int rounds;     // 0: no shared tail
-  int unit;
-  int n;          // workers
-  __device__ __forceinline__ int n_chunks() const { return rounds * n; }
-  __device__ __forceinline__ int64_t round_start(int r) const {  // first item of round r (r = rounds: end of the list)
-    return head + static_cast<int64_t>(n) * unit * ((1 << rounds) - (1 << (rounds - r)));
-  }
-  __device__ __forceinline__ void chunk_range(int t, int64_t& first, int64_t& end) const {
-    const int r = t / n;
-    const int len = unit << (rounds - 1 - r);
-    first = round_start(r) + static_cast<int64_t>(t - r * n) * len;
-    end = first + len;
-  }
-  __device__ __forceinline__ int chunk_of(int64_t id) const {  // id >= head
-    int r = 0;
-    while (r + 1 < rounds && id >= round_start(r + 1)) ++r;
-    return r * n + static_cast<int>((id - round_start(r)) / (unit << (rounds - 1 - r)));
-  }
-};
-__device__ __forceinline__ Pieces pieces_of(int64_t total, int64_t n, bool shared_tail) {
-  Pieces p{total, 0, 0, static_cast<int>(n)};
-  if (!shared_tail) return p;
-  // Chunks are at least kMinChunk items long (a worker fetches the operands of its next run while it
-  // works on a run of at least that length) and the tail is about 22 % of the list.  Shorter lists are
-  // dealt out whole.
-  const int64_t per = total / n;
-  const int rounds = kTailRounds;
-  if (static_cast<int64_t>(kMinChunk) * ((1 << rounds) - 1) * 100 > per * 45) return p;
-  p.rounds = rounds;
-  p.unit = static_cast<int>(min<int64_t>(max<int64_t>(kMinChunk, per * 22 / 100 / ((1 << rounds) - 1)), 1 << 20));
-  p.head = total - static_cast<int64_t>(n) * p.unit * ((1 << p.rounds) - 1);
-  return p;
-}
-
-// Next chunk of the shared tail.  The counter word is (launch_id << 32 | chunks taken).  A word with
-// another tag is left over from an earlier launch or was never written, and counts as zero taken: whoever
-// meets one replaces it.  The merge kernel, which always follows, leaves (launch_id + 1) << 32, so launches
-// that follow one another find the word ready, and a replayed graph (same launch_id every time) starts from
-// a word it replaces.  Taking is one atomic add: a compare-and-swap per chunk would let one worker through
-// per round trip to the L2 when all of them come at once.  Called by one lane.
-__device__ __forceinline__ int take_chunk(unsigned long long* word, unsigned launch_id) {
-  const unsigned long long tag = static_cast<unsigned long long>(launch_id) << 32;
-  for (;;) {
-    unsigned long long seen = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((seen >> 32) == launch_id) return static_cast<int>(static_cast<unsigned>(seen));
-    // Not this launch's word.  Adds of other workers that met it too only move its low half, so it keeps
-    // its foreign tag until one compare-and-swap (each failure = someone else's add or swap) replaces it.
-    seen += 1ull;
-    while ((seen >> 32) != launch_id) {
-      unsigned long long expected = seen;
-      if (__hip_atomic_compare_exchange_strong(word, &expected, tag | 1ull, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT))
-        return 0;
-      seen = expected;
-    }
-  }
 }
 
 // Exclusive prefix sum of the per-sequence item counts into prefix[0..batch] (LDS).
@@ -710,24 +639,19 @@ __device__ __forceinline__ void copy_cursor(CtxCursor& d, const CtxCursor& s) {
   }
 }
 
-constexpr int kPieceRing = 8;           // pieces a worker knows of and has not finished (at most 3)
-constexpr int kLookAhead = 8;           // stages before the end of a piece at which the next one is asked for
-constexpr int kMailNone = 0x7fffffff;   // answer: the tail is used up
-constexpr int kMailSpins = 1 << 22;     // bound of every wait on a mailbox
-constexpr int kMfmaThreads = kThreads + kWave;  // the workers and the wavefront that takes chunks for them
+constexpr int kPairSpins = 1 << 22;          // bound of every wait of one wavefront of a pair on the other
+constexpr int kMfmaThreads = 2 * kThreads;   // kWaves loading wavefronts and kWaves computing wavefronts
 
 template <int NS>
 struct MfmaLayout {
   // LDS: ring [waves][NS][stage] | Q rows [waves][16][256 B] | page-table chunks [waves][3][64] |
-  //      scan scratch [kThreads] | mailboxes [2][waves] | piece records [waves][kPieceRing][4] |
-  //      stage prefix [batch + 1]
+  //      scan scratch [kThreads] | progress counters [waves][2] | stage prefix [batch + 1]
   static constexpr int kRingBytes = kWaves * NS * kStageBytes;
   static constexpr int kQOff = kRingBytes;
   static constexpr int kPageOff = kQOff + kWaves * kMfmaHeads * 256;
   static constexpr int kTmpOff = kPageOff + kWaves * 3 * kWave * 4;
-  static constexpr int kMailOff = kTmpOff + kThreads * 4;
-  static constexpr int kPieceOff = kMailOff + 2 * kWaves * 4;
-  static constexpr int kPrefixOff = kPieceOff + kWaves * kPieceRing * 16;
+  static constexpr int kSyncOff = kTmpOff + kThreads * 4;
+  static constexpr int kPrefixOff = kSyncOff + 2 * kWaves * 4;
 };
 
 // VL (packed query chunks): a batch entry is a sequence with cu_q[b + 1] - cu_q[b] query tokens.  The 16 MFMA
@@ -784,50 +708,34 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     return tok * a.q_stride_bytes + (static_cast<int64_t>(kvh * a.group + (c - j * a.group)) * D) * 2;
   };
 
-  // mailboxes: mail[w] = 0 idle, 1 worker w asks for a chunk, chunk + 2 or kMailNone the answer;
-  // mail[kWaves + w] != 0: worker w has finished
-  lds_vint* mail = (lds_vint*)(smem + Lay::kMailOff);
-  if (tid < 2 * kWaves) mail[tid] = 0;
+  // progress of pair w: sync[2 w] stages that have landed, sync[2 w + 1] stages whose slots are free again
+  lds_vint* sync = (lds_vint*)(smem + Lay::kSyncOff);
+  if (tid < 2 * kWaves) sync[tid] = 0;
   item_prefix<T>(a, prefix, tmp);
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
   if (blockIdx.x == 0) {
     for (int i = tid; i <= a.batch; i += kMfmaThreads) a.ws_prefix[i] = prefix[i];
   }
   if (total == 0) return;
-  // ---- from here on the wavefronts are independent: no workgroup barrier below this line
+  // ---- from here on the pairs are independent: no workgroup barrier below this line
+  const bool loader = wave < kWaves;   // wavefronts 0 .. kWaves - 1 load, wavefront kWaves + w computes what w loads
+  const int pair = wave & (kWaves - 1);
   const int64_t n_workers = static_cast<int64_t>(gridDim.x) * kWaves;
-  const Pieces pieces = pieces_of(total, n_workers, a.tickets != nullptr);
-  if (wave == kWaves) {
-    // The wavefront that takes chunks, one lane per worker.  A worker cannot wait for the answer of an
-    // atomic itself: the wait would also be one for all of its stages in flight.
-    if (pieces.rounds == 0 || lane >= kWaves) return;
-    for (int spin = 0; spin < kMailSpins; ++spin) {
-      if (mail[lane] == 1) {
-        const int t = take_chunk(a.tickets, a.launch_id);
-        mail[lane] = t < pieces.n_chunks() ? t + 2 : kMailNone;
-      }
-      if (mail[kWaves + lane] != 0) break;
-      __builtin_amdgcn_s_sleep(8);
-    }
-    return;
-  }
-  const int64_t worker = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
-  const int64_t cur = range_start(worker, pieces.head, n_workers);
-  const int64_t end = range_start(worker + 1, pieces.head, n_workers);
-  if (cur >= end) {  // (a list with a shared tail is long enough to give every worker a range)
-    mail[kWaves + wave] = 1;
-    return;
-  }
-  // pieces the producer has opened, for the consumer that follows it: first item, items, piece number
-  lds_vint* piece_ring = (lds_vint*)(smem + Lay::kPieceOff + wave * kPieceRing * 16);
+  const int64_t worker = static_cast<int64_t>(blockIdx.x) * kWaves + pair;
+  const int64_t cur = range_start(worker, total, n_workers);
+  const int64_t end = range_start(worker + 1, total, n_workers);
+  if (cur >= end) return;
+  const int n_stages = static_cast<int>(end - cur);
+  lds_vint* landed = sync + 2 * pair;
+  lds_vint* freed = landed + 1;
 
   const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
-  const u32 ring_lds = __builtin_amdgcn_readfirstlane(lds_base + wave * NS * kStageBytes);
-  const char* ring = smem + wave * NS * kStageBytes;
-  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + wave * 3 * kWave * 4);
-  const char* pagebuf = smem + Lay::kPageOff + wave * 3 * kWave * 4;
-  const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + wave * G * 256);
-  const char* qbuf = smem + Lay::kQOff + wave * G * 256;
+  const u32 ring_lds = __builtin_amdgcn_readfirstlane(lds_base + pair * NS * kStageBytes);
+  const char* ring = smem + pair * NS * kStageBytes;
+  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + pair * 3 * kWave * 4);
+  const char* pagebuf = smem + Lay::kPageOff + pair * 3 * kWave * 4;
+  const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + pair * G * 256);
+  const char* qbuf = smem + Lay::kQOff + pair * G * 256;
 
   auto locate = [&](int64_t f, CtxCursor& cu) {
     int lo = 0, hi = a.batch;
@@ -889,29 +797,22 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   const int v8_read = T * RB + v8_row * RB + (c16 & 1) * 8;
   const int v8_y = (v8_row & 7) << 4;
 
-  // ---- producer: issues stage p of the worker's stages, which run on from piece to piece (the worker's own
-  // range, then chunks of the shared tail while there are any); pc is the context of stage p
+  if (loader) {
+  // ---- the loading wavefront: issues stage p of the worker's range; pc is the context of that stage
   CtxCursor pc;
   locate(cur, pc);
   CtxCursor pn;                              // the context after pc (valid while has_c)
   copy_cursor<VL>(pn, pc);
   int p = 0;
-  int p_end = static_cast<int>(end - cur);   // first stage past the producer's piece
-  int p_pieces = 0;                          // pieces opened after the first
-  // the piece after this one: 0 not asked for, 1 asked, 2 known (pn, its first page-table chunk on the way), 3 none
-  int nx_state = pieces.rounds == 0 ? 3 : 0;
-  int nx_len = 0;
-  bool need_piece = false;                   // pc is the last context of the piece
-  bool p_final = false;                      // every stage of the worker has been issued
   u32 off_a = 0, off_b = kWave * 4, off_c = 2 * kWave * 4;  // chunk buffers: current, next of pc, first of pn
-  int ck_a = 0, ck_c = 0;
+  int ck_a = 0;
   int t_b = 0, t_c = 0;                      // value of p when the buffer's load was issued
   bool has_b = false, has_c = false;
   int p_ctx_first = 0, p_prev_len = 0;
 
-  // A chunk or Q load issued while p was t has landed once the consumer has waited for stage t,
-  // which it has done when p >= t + NS - 1; otherwise everything in flight is awaited (short
-  // contexts only).
+  // A chunk or Q load issued while p was t has landed once stage t has: this wavefront has waited for
+  // that before it issues stage t + NS - 1; otherwise everything in flight is awaited (short contexts
+  // only).
   auto ensure_landed = [&](bool issued, int t) {
     if (!(issued && t + NS - 1 <= p)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
@@ -924,17 +825,15 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       const u32 t = off_a;
       off_a = off_c;
       off_c = t;
-      ck_a = ck_c;
+      ck_a = 0;
       ensure_landed(has_c, t_c);
     }
     has_b = has_c = false;
     p_ctx_first = p;
-    need_piece = !(pc.n_st - pc.st < p_end - p);
-    if (!need_piece) {  // the piece goes on into another context
+    if (pc.n_st - pc.st < n_stages - p) {  // the range goes on into another context
       copy_cursor<VL>(pn, pc);
       next_context(pn);
       issue_chunk(pn, 0, off_c);
-      ck_c = 0;
       t_c = p;
       has_c = true;
     }
@@ -946,9 +845,10 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     }
     if (first || p_prev_len >= NS) {
       // Q rows of the context's heads travel ahead of its first stage, swizzled like K rows (rows
-      // past the group repeat the last head; the consumer zeroes them).  The single buffer is
-      // free: the consumer copied the previous context's rows to registers when it began that
-      // context, at least NS stages ago.  After a shorter context the consumer loads Q itself.
+      // past the group repeat the last head; the computing wavefront zeroes them).  The single buffer
+      // is free: that wavefront copied the previous context's rows to registers when it began that
+      // context, at least NS stages ago, and has released the slot of that stage since.  After a shorter
+      // context it loads Q itself.
       const int kvh = pc.kvh;
       if constexpr (VL) {
         const int nhp = pc.qn * a.group;
@@ -969,54 +869,9 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       }
     }
   };
-  // Asks for the next piece when the current one is about to end, and once the answer is there opens it:
-  // its place in the list, its first page-table chunk.  `await`: the answer is needed now.
-  auto look_ahead = [&](bool await) {
-    if (!need_piece || nx_state >= 2) return;
-    if (nx_state == 0) {
-      if (p_end - p > kLookAhead) return;
-      mail[wave] = 1;
-      nx_state = 1;
-    }
-    int v = mail[wave];
-    if (await) {
-      for (int spin = 0; v == 1 && spin < kMailSpins; ++spin) {
-        __builtin_amdgcn_s_sleep(2);
-        v = mail[wave];
-      }
-      if (v == 1) v = kMailNone;  // (never: the taking wavefront answers while this one lives)
-    }
-    v = __builtin_amdgcn_readfirstlane(v);
-    if (v == 1) return;
-    if (v == kMailNone) {
-      nx_state = 3;
-      return;
-    }
-    int64_t f, e;
-    pieces.chunk_range(v - 2, f, e);
-    nx_len = static_cast<int>(e - f);
-    lds_vint* rec = piece_ring + ((p_pieces + 1) & (kPieceRing - 1)) * 4;
-    rec[0] = static_cast<int>(f);
-    rec[1] = static_cast<int>(f >> 32);
-    rec[2] = nx_len;
-    rec[3] = v - 2;
-    locate(f, pn);
-    ck_c = ((pn.st * T) >> a.bs_shift) >> 6;
-    issue_chunk(pn, ck_c, off_c);
-    t_c = p;
-    has_c = true;
-    nx_state = 2;
-  };
   auto issue_stage = [&]() {
     if (p == 0) {
       begin_context(true);
-    } else if (p == p_end) {  // into the next piece (known: see produce)
-      p_prev_len = p - p_ctx_first;
-      copy_cursor<VL>(pc, pn);
-      ++p_pieces;
-      p_end += nx_len;
-      nx_state = 0;
-      begin_context(false);
     } else if (pc.st == pc.n_st) {
       p_prev_len = p - p_ctx_first;
       copy_cursor<VL>(pc, pn);
@@ -1079,23 +934,35 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     ++pc.st;
   };
 
-  auto produce = [&]() {
-    if (p_final) return;
-    look_ahead(p == p_end);
-    if (p == p_end && nx_state != 2) {
-      p_final = true;
-      return;
+  // Stage i goes out once stage i - (NS - 1) has landed -- said to the computing wavefront, which cannot
+  // wait for loads that another wavefront issued -- and the slot of stage i - NS has been given back.
+  // NS - 1 stages are in flight while the other wavefront computes on the oldest one.
+  int published = 0, released = 0;
+  for (int i = 0; i < n_stages; ++i) {
+    while (published < i - (NS - 2)) {
+      wait_younger_stages(i - 1 - published);
+      ++published;
+      *landed = published;
+    }
+    for (int spin = 0; i - released >= NS; ++spin) {
+      released = __builtin_amdgcn_readfirstlane(*freed);
+      if (i - released < NS) break;
+      if (spin > kPairSpins) return;  // (never: the computing wavefront gives every slot back)
+      __builtin_amdgcn_s_sleep(1);
     }
     issue_stage();
-  };
-  for (int s = 0; s < NS - 1; ++s) produce();
+  }
+  while (published < n_stages) {
+    wait_younger_stages(n_stages - 1 - published);
+    ++published;
+    *landed = published;
+  }
+  return;
+  }  // loader
 
-  // ---- consumer
+  // ---- the computing wavefront
   CtxCursor cc;
   locate(cur, cc);
-  int c_end = static_cast<int>(end - cur);  // first stage past the consumer's piece
-  int c_pieces = 0;
-  int64_t piece = worker;                   // its number: the worker's, or that of chunk t, n_workers + t
   bool run_start = true;
   bool first_run = true;
   bool complete = false;
@@ -1108,11 +975,17 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   float m = kNegBig, l = 0.0f;
   float score_scale = a.scale_log2, out_scale = 1.0f;
 
-  for (int s = 0; s < p; ++s) {  // (p moves ahead of s until the last piece has been issued)
-    wait_younger_stages(min(NS - 2, p - 1 - s));
-    produce();
+  int arrived = 0;
+  for (int s = 0; s < n_stages; ++s) {
+    for (int spin = 0; arrived <= s; ++spin) {
+      arrived = __builtin_amdgcn_readfirstlane(*landed);
+      if (arrived > s) break;
+      if (spin > kPairSpins) return;  // (never: the loading wavefront announces every stage)
+      __builtin_amdgcn_s_sleep(1);
+    }
+    asm volatile("" ::: "memory");  // no read of the stage moves above the poll
 
-    if (run_start) {  // first stage of a run: the (sequence, head block) or the piece changes
+    if (run_start) {  // first stage of a run: the (sequence, head block) changes
       run_start = false;
       const int kvh = cc.kvh;
       if constexpr (VL) {
@@ -1127,7 +1000,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         nh = min(G, (kvh + 1) * a.group - h0);
         Lc = cc.L;
       }
-      complete = cc.st == 0 && cc.n_st <= c_end - s;
+      complete = cc.st == 0 && cc.n_st <= n_stages - s;
       if (s == 0 || c_prev_len >= NS) {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)  // the rows landed before this stage's tiles did
@@ -1162,13 +1035,22 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
 
     const char* st = ring + (s % NS) * kStageBytes;
     if constexpr (!FP8) {
-      // ---- scores of the stage's 16 tokens: lane (head c16, tokens 4g .. 4g+3)
-      f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+      // ---- all operand reads of the stage first: the latency of the V^T reads passes behind the score
+      // MFMAs and the softmax (the scheduler would otherwise place them next to their use)
+      u32x4 kr[4];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const u32x4 kr = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ c16) * 16));
-        sc = Mfma<QT>::k32(kr, q[kk], sc);
-      }
+      for (int kk = 0; kk < 4; ++kk) kr[kk] = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ c16) * 16));
+      s16x4 vt[8];
+#pragma unroll
+      for (int mb = 0; mb < 8; ++mb)
+        vt[mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + v_read + (v_y ^ (mb << 5))));
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- scores of the stage's 16 tokens: lane (head c16, tokens 4g .. 4g+3); two chains of two MFMAs
+      f32x4 sc = Mfma<QT>::k32(kr[0], q[0], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+      f32x4 sc1 = Mfma<QT>::k32(kr[1], q[1], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
+      sc = Mfma<QT>::k32(kr[2], q[2], sc);
+      sc1 = Mfma<QT>::k32(kr[3], q[3], sc1);
+      sc += sc1;
       const int tok0 = cc.st * T + 4 * g;
       float sv[4];
       bool over = false;
@@ -1197,11 +1079,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       // ---- O^T += V^T . P^T: lane c16 of a 16-lane group supplies the address of 4 dims of token
       // row 4g + c16/4 and receives the 4 tokens of dim column 16 mb + c16
 #pragma unroll
-      for (int mb = 0; mb < 8; ++mb) {
-        const s16x4 vt = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (lds_s16x4*)(st + v_read + (v_y ^ (mb << 5))));
-        o[mb] = Mfma<QT>::k16(vt, pb, o[mb]);
-      }
+      for (int mb = 0; mb < 8; ++mb) o[mb] = Mfma<QT>::k16(vt[mb], pb, o[mb]);
     } else {
       // ---- scores of the stage's 32 tokens, two blocks of 16: lane (head c16, tokens 16 tb + 4g ..)
       float sv[8];
@@ -1260,15 +1138,14 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
 
     // ---- end of a run: last stage of the context or of the worker's range
     const bool ctx_end = cc.st == cc.n_st - 1;
-    const bool piece_end = s == c_end - 1;
-    if (ctx_end || piece_end) {
+    if (ctx_end || s == n_stages - 1) {
       const float lsum = quad_rows_sum(l);
       // (VL: a column that attends to nothing -- a chunk longer than its context -- gives zeros)
       const float inv = VL && !(lsum > 0.0f) ? 0.0f : out_scale / lsum;
       const float lse2 = m + fast_log2(lsum);
       const bool head_on = c16 < nh;
       const int hq = h0 + c16;
-      const int64_t pidx = (piece * 2 + (first_run ? 0 : 1)) * G + c16;
+      const int64_t pidx = (worker * 2 + (first_run ? 0 : 1)) * G + c16;
       if (head_on && complete) {
         char* op = VL ? a.out + out_off + 4 * g * 2
                       : a.out + cc.b * a.out_stride_bytes + (static_cast<int64_t>(hq) * D + 4 * g) * 2;
@@ -1290,29 +1167,17 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       if (head_on && g == 0 && !complete) a.ws_lse[pidx] = lse2;
       first_run = false;
     }
+    // The operand reads of the stage have returned (the MFMAs that take them have been issued) and LDS
+    // serves a wavefront's instructions in order: the slot may be written again.
+    asm volatile("" ::: "memory");  // no read of the stage moves below the store
+    *freed = s + 1;
     ++cc.st;
-    if (piece_end) {
-      // The producer went past the end of this piece at least NS - 1 stages ago: it has opened the next
-      // one, if there is one.
-      if (c_pieces < p_pieces) {
-        ++c_pieces;
-        lds_vint* rec = piece_ring + (c_pieces & (kPieceRing - 1)) * 4;
-        const int64_t f = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(rec[1])) << 32) |
-                          static_cast<u32>(__builtin_amdgcn_readfirstlane(rec[0]));
-        c_end += __builtin_amdgcn_readfirstlane(rec[2]);
-        piece = n_workers + __builtin_amdgcn_readfirstlane(rec[3]);
-        c_prev_len = s + 1 - c_ctx_first;
-        locate(f, cc);
-        first_run = true;
-        run_start = true;
-      }
-    } else if (ctx_end) {
+    if (ctx_end && s + 1 < n_stages) {
       c_prev_len = s + 1 - c_ctx_first;
       next_context(cc);
       run_start = true;
     }
   }
-  if (lane == 0) mail[kWaves + wave] = 1;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
@@ -1330,8 +1195,6 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
   const int b = blockIdx.y;
   const int tid = threadIdx.x;
   const int G = a.g_block;
-  if (a.tickets != nullptr && hbk == 0 && b == 0 && tid == 0)  // every chunk has been taken by now
-    *a.tickets = static_cast<unsigned long long>(a.launch_id + 1u) << 32;
   const int p0 = a.ws_prefix[b], p1 = a.ws_prefix[b + 1], pt = a.ws_prefix[a.batch];
   const int hb_per_kv = VL ? a.chunk_blocks : (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
@@ -1380,27 +1243,16 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
   const int64_t first = static_cast<int64_t>(p0) * n_hb + static_cast<int64_t>(hbk) * n_items;
   const int64_t last = first + n_items - 1;
   const int64_t n = a.n_workgroups;
-  const Pieces pieces = pieces_of(total, n, a.tickets != nullptr);
-  // pieces in list order: the workers' ranges of the first `head` items, then the chunks of the tail
-  auto piece_of = [&](int64_t id) {
-    return id < pieces.head ? workgroup_of(id, pieces.head, n) : static_cast<int>(n) + pieces.chunk_of(id);
-  };
-  auto piece_start = [&](int pc) {
-    if (pc < n) return range_start(pc, pieces.head, n);
-    int64_t f, e;
-    pieces.chunk_range(pc - static_cast<int>(n), f, e);
-    return f;
-  };
-  const int w_first = piece_of(first);
-  const int w_last = piece_of(last);
-  if (w_first == w_last) return;  // one piece held the whole context: its worker wrote the output
-  // range_start(w) = w * q + floor(w * r / n) with head = q * n + r: stepped from w to w + 1
+  const int w_first = workgroup_of(first, total, n);
+  const int w_last = workgroup_of(last, total, n);
+  if (w_first == w_last) return;  // one worker saw the whole context and wrote the output
+  // range_start(w) = w * q + floor(w * r / n) with total = q * n + r: stepped from w to w + 1
   // without a division
-  const int64_t q = pieces.head / n, r = pieces.head - q * n;
-  const int64_t acc0 = (static_cast<int64_t>(min<int64_t>(w_first, n)) * r) % n;
-  // the first piece holds this context as its last run (slot 1) unless it starts exactly here;
-  // every later one holds it as its first run (slot 0)
-  const int slot_first = piece_start(w_first) < first ? 1 : 0;
+  const int64_t q = total / n, r = total - q * n;
+  const int64_t acc0 = (static_cast<int64_t>(w_first) * r) % n;
+  // the first worker holds this context as its last run (slot 1) unless its range starts
+  // exactly here; every later one holds it as its first run (slot 0)
+  const int slot_first = range_start(w_first, total, n) < first ? 1 : 0;
   for (int v = tid; v < n_vec; v += kThreads) {
     const int h = v / dv4, d = (v - h * dv4) * 4;
     int64_t acc = acc0;
@@ -1417,8 +1269,7 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
         const int64_t step = q + (acc >= n ? 1 : 0);
         acc -= acc >= n ? n : 0;
         // with fewer items than workers some ranges in between are empty and own no partial
-        // (chunks of the tail never are)
-        on[k] = w <= w_last && (step > 0 || w >= n);
+        on[k] = w <= w_last && step > 0;
         const int64_t ps = (static_cast<int64_t>(w) * 2 + (w == w_first ? slot_first : 0)) * G + h;
         lse[k] = on[k] ? a.ws_lse[ps] : kNegBig;
         x[k] = on[k] ? *reinterpret_cast<const f32x4*>(a.ws_out + ps * dv + d) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -1497,24 +1348,13 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   a.g_block = kMfmaHeads;
   const int n_wg = device_cu_count();  // the ring fills a CU's LDS: one workgroup each
   a.n_workgroups = n_wg * kWaves;      // independent workers = wavefronts
-  // workspace: counter of the shared tail (256 bytes) | item prefix | partials, two slots per piece
-  // "1": leave the end of long item lists to whoever is free.  Off by default: with non-temporal loads the
-  // launch gains at most 1-2 % from it and the merge kernel, which then folds several times as many
-  // partials, loses more than that.
-  const char* tail_knob = getenv("XLLM_MI355_GQA_TAIL");
-  const bool shared_tail = tail_knob != nullptr && tail_knob[0] == '1';
-  static std::atomic<unsigned> launches{0};
-  const size_t n_pieces = static_cast<size_t>(a.n_workgroups) * (1 + kTailRounds);
   const size_t prefix_bytes = ((static_cast<size_t>(a.batch) + 1) * 4 + 255) / 256 * 256;
-  const size_t part_floats = n_pieces * 2 * kMfmaHeads * (D + 1);
-  *need = 256 + prefix_bytes + part_floats * 4;
+  const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * (D + 1);
+  *need = prefix_bytes + part_floats * 4;
   if (plan_only) return XLLM_MI355_OK;
   if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
-  a.tickets = shared_tail ? reinterpret_cast<unsigned long long*>(a.ws_prefix) : nullptr;
-  do a.launch_id = ++launches; while (a.launch_id == 0);
-  a.ws_prefix = reinterpret_cast<int*>(reinterpret_cast<char*>(a.ws_prefix) + 256);
   a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_prefix) + prefix_bytes);
-  a.ws_lse = a.ws_out + n_pieces * 2 * kMfmaHeads * D;
+  a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
   const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 1) * 4;
   const bool timed = profile_begin(stream);
   kern<<<dim3(static_cast<unsigned>(n_wg)), kMfmaThreads, smem, stream>>>(a);
@@ -1583,11 +1423,7 @@ size_t gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim) {
   (void)n_q_heads;
   const size_t b = static_cast<size_t>(batch < kMaxBatch ? batch : kMaxBatch);
   const size_t prefix_bytes = ((b + 1) * 4 + 255) / 256 * 256;
-  const size_t rows_kernel = prefix_bytes + static_cast<size_t>(device_cu_count()) * 8 * 2 * 8 * (head_dim + 1) * 4;
-  // matrix-core kernel: counter, prefix, two slots of 16 heads per piece (a worker's range + the tail's chunks)
-  const size_t mfma_kernel = 256 + prefix_bytes + static_cast<size_t>(device_cu_count()) * kWaves * (1 + kTailRounds) * 2 *
-                                                      kMfmaHeads * (head_dim + 1) * 4;
-  return head_dim == 128 && mfma_kernel > rows_kernel ? mfma_kernel : rows_kernel;
+  return prefix_bytes + static_cast<size_t>(device_cu_count()) * 8 * 2 * 8 * (head_dim + 1) * 4;
 }
 
 int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out, float* lse,
