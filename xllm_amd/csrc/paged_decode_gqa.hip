@@ -10,9 +10,10 @@
 // writes a normalised fp32 partial + log2-domain LSE, and a small merge kernel folds those.
 // The item counts are prefix-summed inside every workgroup (no extra launch, no host read).
 //
-// gqa_mfma_kernel (head_dim 128, block size a power of two >= 16): worker = wavefront, item = 16
-// tokens (32 for fp8 pages); rows travel global memory -> LDS directly into a private ring per
-// wavefront and both products run on the matrix cores.  Its own comment below has the details.
+// gqa_mfma_kernel (head_dim 128, block size a power of two >= 16): worker = a loading and a computing
+// wavefront, item = 16 tokens (32 for fp8 pages); rows travel global memory -> LDS directly into a
+// private ring per worker and both products run on the matrix cores.  Its own comment below has the
+// details.
 //
 // gqa_decode_kernel (every other shape): worker = workgroup, item = 64 tokens, the 4 wavefronts
 // of a workgroup take steps round-robin:
@@ -483,12 +484,18 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
 // ---------------------------------------------------------------------------------------------
 // Matrix-core variant for D = 128 with 16-bit pages.
 //
-// Every WAVEFRONT is an independent worker: it owns a contiguous range of the flat item list,
-// keeps its own softmax state, and never meets the other wavefronts of its workgroup after the
+// A worker is a PAIR of wavefronts that share a SIMD: wavefront w of the workgroup loads, wavefront
+// kWaves + w computes.  A wavefront cannot issue more than one load-to-LDS instruction per 90 ns or
+// so (0.75-0.85 us for the 8 of a stage) and does nothing else while it issues; in one wavefront the
+// 0.3-0.5 us of arithmetic per stage came on top of that, which is more than the memory system leaves
+// a wavefront per stage (1.15 us at 7.1 TB/s over 1024 workers).  The two meet in two LDS counters:
+// stages whose loads have completed (the computing wavefront cannot wait on loads it did not issue)
+// and stages whose ring slot has been given back.  A worker owns a contiguous range of the flat item
+// list, keeps its own softmax state, and never meets the other workers of its workgroup after the
 // common item prefix sum, so there is no barrier anywhere in the streaming loop.
 //
 // Data path.  A stage is 16 tokens of one KV head (32 for fp8 pages): K rows, then V rows, 8 KB.
-// Stages travel from global memory straight into the wavefront's private LDS ring
+// Stages travel from global memory straight into the worker's private LDS ring
 // (global_load_lds_dwordx4, 16 adjacent lanes per 256-byte row so every instruction reads whole
 // contiguous rows), NS stages deep, NS - 1 in flight while one is consumed.  Within a row the
 // 16-byte chunks are XOR-swizzled so that both operand reads below touch every LDS bank once.
@@ -504,8 +511,8 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
 // columns), so a lane owns one head: its running maximum and sum are plain per-lane scalars.
 // The maximum only moves when a score exceeds it by more than kSlack (log2 units).
 //
-// Nothing in the loop waits on a register load from global memory: such a wait would also wait
-// for every younger stage in flight (the counter is in order).  Page-table entries (64 at a
+// Nothing in the loading wavefront waits on a register load from global memory: such a wait would also
+// wait for every younger stage in flight (the counter is in order).  Page-table entries (64 at a
 // time: the current chunk, the next one, and the first one of the next context), the Q rows of
 // the next context and the stages all take the LDS path and are covered by one explicit wait per
 // stage; sequence lengths and fp8 scales come through the scalar cache.  Loads that write
