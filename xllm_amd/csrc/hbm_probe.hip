@@ -88,10 +88,8 @@ int xllm_mi355_stream_read(const void* src, size_t bytes, void* sink, void* stre
   }
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-  const bool timed = profile_begin(static_cast<hipStream_t>(stream));
-  stream_read_kernel<<<cus > 0 ? cus : 256, 256, kReadLds, static_cast<hipStream_t>(stream)>>>(
-      static_cast<const char*>(src), bytes, static_cast<u32*>(sink));
-  if (timed) profile_end(static_cast<hipStream_t>(stream));
+  launch_timed(stream_read_kernel, dim3(cus > 0 ? cus : 256), dim3(256), kReadLds, static_cast<hipStream_t>(stream),
+               static_cast<const char*>(src), bytes, static_cast<u32*>(sink));
   return static_cast<int>(hipGetLastError());
 }
 
@@ -100,10 +98,8 @@ int xllm_mi355_stream_copy(void* dst, const void* src, size_t bytes, void* strea
       bytes % 16 != 0)
     return XLLM_MI355_EALIGN;
   if (bytes == 0) return XLLM_MI355_OK;
-  const bool timed = profile_begin(static_cast<hipStream_t>(stream));
-  stream_copy_kernel<<<2048, 256, 0, static_cast<hipStream_t>(stream)>>>(
-      static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), bytes / 16);
-  if (timed) profile_end(static_cast<hipStream_t>(stream));
+  launch_timed(stream_copy_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream),
+               static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), bytes / 16);
   return static_cast<int>(hipGetLastError());
 }
 

@@ -1332,9 +1332,7 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
   if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
   a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_prefix) + prefix_bytes);
   a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * G * D;
-  const bool timed = profile_begin(stream);
-  kern<<<dim3(static_cast<unsigned>(a.n_workgroups)), kThreads, smem, stream>>>(a);
-  if (timed) profile_end(stream);
+  launch_timed(kern, dim3(static_cast<unsigned>(a.n_workgroups)), dim3(kThreads), smem, stream, a);
   return static_cast<int>(hipGetLastError());
 }
 
@@ -1363,9 +1361,7 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_prefix) + prefix_bytes);
   a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
   const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 1) * 4;
-  const bool timed = profile_begin(stream);
-  kern<<<dim3(static_cast<unsigned>(n_wg)), kMfmaThreads, smem, stream>>>(a);
-  if (timed) profile_end(stream);
+  launch_timed(kern, dim3(static_cast<unsigned>(n_wg)), dim3(kMfmaThreads), smem, stream, a);
   return static_cast<int>(hipGetLastError());
 }
 

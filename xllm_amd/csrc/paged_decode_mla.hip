@@ -1498,14 +1498,12 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.ws_out = reinterpret_cast<float*>(static_cast<char*>(workspace) + prefix_bytes);
     a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * n_heads * kDL;
 
-    const bool timed = profile_begin(stream);
     if (pairs)
-      mla_decode_kernel<<<dim3(static_cast<unsigned>(a.n_teams * n_hb)), kMlaThreads, smem, stream>>>(a);
+      launch_timed(mla_decode_kernel, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kMlaThreads), smem, stream, a);
     else if (use_p)
-      mla_decode32w_kernel<<<dim3(static_cast<unsigned>(a.n_teams * a.n_hb)), kWThreads, kPLdsBytes, stream>>>(a);
+      launch_timed(mla_decode32w_kernel, dim3(static_cast<unsigned>(a.n_teams * a.n_hb)), dim3(kWThreads), kPLdsBytes, stream, a);
     else
-      mla_decode16_kernel<<<dim3(static_cast<unsigned>(a.n_teams * n_hb)), kThreads16, smem, stream>>>(a);
-    if (timed) profile_end(stream);
+      launch_timed(mla_decode16_kernel, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kThreads16), smem, stream, a);
     int rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
     mla_merge_kernel<<<dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb)), 128, 0, stream>>>(a);

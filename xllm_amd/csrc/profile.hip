@@ -1,5 +1,5 @@
-// Opt-in kernel timing: while enabled, the decode entry points bracket their dominant
-// kernel with a pair of HIP events on the caller's stream, so a benchmark can read that
+// Opt-in kernel timing: while enabled, the decode entry points launch their dominant kernel with
+// a pair of HIP events attached to the dispatch (launch.h: launch_timed), so a benchmark can read that
 // kernel's duration without an external profiler.  Not for use under graph capture.
 #include <vector>
 
@@ -16,16 +16,15 @@ struct ProfileState {
 ProfileState g_profile;
 }  // namespace
 
-bool profile_begin(hipStream_t stream) {
+bool profile_events(hipEvent_t* start, hipEvent_t* stop) {
   ProfileState& p = g_profile;
   if (!p.enabled || p.used >= static_cast<int>(p.start.size())) return false;
-  return hipEventRecord(p.start[p.used], stream) == hipSuccess;
+  *start = p.start[p.used];
+  *stop = p.stop[p.used];
+  return true;
 }
 
-void profile_end(hipStream_t stream) {
-  ProfileState& p = g_profile;
-  if (hipEventRecord(p.stop[p.used], stream) == hipSuccess) ++p.used;
-}
+void profile_commit() { ++g_profile.used; }
 
 }  // namespace xllm_mi355
 
