@@ -252,6 +252,29 @@ int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr,
                                  int64_t batch, int64_t block_size, void* stream);
 
 /*
+ * Decode metadata into the persistent buffers of a captured step, with the padding a replay at a larger
+ * batch expects.  Replaces xllm::kernel::cuda::update_llm_decode_metadata and its parameter struct,
+ * field for field (xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56, .cu:27-71; caller
+ * xllm/core/runtime/cuda_graph_executor_impl.cpp:243-284).  All arrays int32; src_kv_seq_lens and
+ * src_paged_kv_indptr are cumulative, [actual_batch_size + 1].
+ *   tokens, positions, new_cache_slots : [0, actual_num_tokens) copied; up to padded_num_tokens 0, 0, -1
+ *   kv_seq_lens, paged_kv_indptr       : [0, actual_batch_size] copied; up to padded_num_tokens the last value
+ *   kv_seq_lens_delta                  : src_kv_seq_lens[i + 1] - src_kv_seq_lens[i]; up to padded_num_tokens 0
+ *   paged_kv_last_page_len             : copied; up to padded_num_tokens 1
+ *   paged_kv_indices                   : [0, actual_indices_size) copied
+ */
+int xllm_mi355_decode_metadata_update(const int32_t* src_tokens, const int32_t* src_positions,
+                                      const int32_t* src_new_cache_slots, const int32_t* src_kv_seq_lens,
+                                      const int32_t* src_paged_kv_indptr, const int32_t* src_paged_kv_indices,
+                                      const int32_t* src_paged_kv_last_page_len,
+                                      int32_t* dst_tokens, int32_t* dst_positions, int32_t* dst_new_cache_slots,
+                                      int32_t* dst_kv_seq_lens, int32_t* dst_kv_seq_lens_delta,
+                                      int32_t* dst_paged_kv_indptr, int32_t* dst_paged_kv_indices,
+                                      int32_t* dst_paged_kv_last_page_len,
+                                      int64_t actual_num_tokens, int64_t padded_num_tokens,
+                                      int64_t actual_batch_size, int64_t actual_indices_size, void* stream);
+
+/*
  * Opt-in timing of the dominant decode kernel.  No counterpart in the reference, which
  * relies on external profilers (xllm/core/platform/cuda_profiler.cpp,
  * xllm/core/platform/torch_profiler.cpp).  After xllm_mi355_profile_enable(n) the next n

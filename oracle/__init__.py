@@ -266,6 +266,40 @@ def build_block_table(indptr, indices, last_page_len, table_stride, block_size):
     return table, seq_lens
 
 
+def llm_decode_metadata_update(src, dst, actual_num_tokens, padded_num_tokens, actual_batch_size,
+                               actual_indices_size):
+    """Restatement of llm_decode_metadata_update_kernel, rule by rule and index by index
+    (xllm/core/kernels/cuda/llm_decode_metadata_update.cu:27-71).  `src` / `dst`: dicts of int32 tensors named as
+    in LlmDecodeMetadataUpdateParams without the prefix; dst is modified in place.  Pinned in
+    tests/test_oracle_reshape.py against the slice copies and fills of the executor's slow path
+    (xllm/core/runtime/cuda_graph_executor_impl.cpp:397-453), which the kernel replaces."""
+    n = max(actual_num_tokens, padded_num_tokens + 1, actual_batch_size + 1, actual_indices_size)
+    for i in range(n):
+        if i < actual_num_tokens:
+            dst["tokens"][i] = src["tokens"][i]
+            dst["positions"][i] = src["positions"][i]
+            dst["new_cache_slots"][i] = src["new_cache_slots"][i]
+        if actual_num_tokens <= i < padded_num_tokens:
+            dst["tokens"][i] = 0
+            dst["positions"][i] = 0
+            dst["new_cache_slots"][i] = -1
+        if i < actual_batch_size + 1:
+            dst["kv_seq_lens"][i] = src["kv_seq_lens"][i]
+            dst["paged_kv_indptr"][i] = src["paged_kv_indptr"][i]
+        if actual_batch_size + 1 <= i < padded_num_tokens + 1:
+            dst["kv_seq_lens"][i] = src["kv_seq_lens"][actual_batch_size]
+            dst["paged_kv_indptr"][i] = src["paged_kv_indptr"][actual_batch_size]
+        if i < actual_batch_size:
+            dst["kv_seq_lens_delta"][i] = src["kv_seq_lens"][i + 1] - src["kv_seq_lens"][i]
+            dst["paged_kv_last_page_len"][i] = src["paged_kv_last_page_len"][i]
+        if actual_batch_size <= i < padded_num_tokens:
+            dst["kv_seq_lens_delta"][i] = 0
+            dst["paged_kv_last_page_len"][i] = 1
+        if i < actual_indices_size:
+            dst["paged_kv_indices"][i] = src["paged_kv_indices"][i]
+    return dst
+
+
 def gather_paged_rows(cache, block_table, cu_seq_lens, total_rows, fill=0):
     """cache [P, bs, 1, D] -> [total_rows, D]; untouched rows keep `fill`."""
     P, bs, D = cache.shape[0], cache.shape[1], cache.shape[-1]

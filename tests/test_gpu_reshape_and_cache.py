@@ -202,3 +202,29 @@ def test_gather_of_paged_latent_rows(device):
                 if int(table[b, t // bs]) < 0:
                     touched[int(cu[b]) + t] = False
         assert torch.equal(out.cpu()[touched].view(torch.uint8), ref[touched].view(torch.uint8)), (dim, dtype)
+
+
+def test_decode_metadata_update_is_bit_exact(device):
+    # update_llm_decode_metadata (kernels/cuda/llm_decode_metadata_update.cu:27-104): integer copies and fills;
+    # every array equals the oracle's, the sentinel outside the padded range included
+    from test_oracle_reshape import _metadata_case
+    for seed, batch, padded, tokens in ((1, 7, 7, None), (2, 5, 16, None), (3, 1, 8, None), (4, 6, 32, 12),
+                                        (5, 40, 64, None), (6, 0, 4, 0), (7, 1500, 2048, None)):
+        src, want = _metadata_case(seed, batch, padded, tokens)
+        _, got = _metadata_case(seed, batch, padded, tokens)
+        n_tok, n_idx = src["tokens"].numel(), src["paged_kv_indices"].numel()
+        oracle.llm_decode_metadata_update(src, want, n_tok, padded, batch, n_idx)
+        s = {k: v.to(device) for k, v in src.items()}
+        d = {k: v.to(device) for k, v in got.items()}
+        ops.update_llm_decode_metadata(ops.LlmDecodeMetadataUpdateParams(
+            src_tokens=s["tokens"], src_positions=s["positions"], src_new_cache_slots=s["new_cache_slots"],
+            src_kv_seq_lens=s["kv_seq_lens"], src_paged_kv_indptr=s["paged_kv_indptr"],
+            src_paged_kv_indices=s["paged_kv_indices"], src_paged_kv_last_page_len=s["paged_kv_last_page_len"],
+            dst_tokens=d["tokens"], dst_positions=d["positions"], dst_new_cache_slots=d["new_cache_slots"],
+            dst_kv_seq_lens=d["kv_seq_lens"], dst_kv_seq_lens_delta=d["kv_seq_lens_delta"],
+            dst_paged_kv_indptr=d["paged_kv_indptr"], dst_paged_kv_indices=d["paged_kv_indices"],
+            dst_paged_kv_last_page_len=d["paged_kv_last_page_len"], actual_num_tokens=n_tok,
+            padded_num_tokens=padded, actual_batch_size=batch, actual_indices_size=n_idx))
+        torch.cuda.synchronize()
+        for k in want:
+            assert torch.equal(d[k].cpu(), want[k]), (seed, k)

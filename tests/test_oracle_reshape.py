@@ -87,3 +87,70 @@ def test_gather_of_paged_rows_is_the_inverse_of_the_scatter():
             page = int(table[b, t // 16])
             expect = flat[page * 16 + t % 16] if page >= 0 else torch.full((576,), 7, dtype=kc.dtype)
             assert torch.equal(got[int(cu[b]) + t], expect)
+
+
+def _metadata_case(seed, batch, padded, tokens=None):
+    """A decode step's metadata as the executor holds it (cumulative lengths, CSR pages) and persistent buffers
+    filled with a sentinel."""
+    g = torch.Generator().manual_seed(seed)
+    tokens = batch if tokens is None else tokens
+    lens = torch.randint(1, 300, (batch,), generator=g, dtype=torch.int32)
+    pages = (lens + 15) // 16
+    src = {
+        "tokens": torch.randint(0, 32000, (tokens,), generator=g, dtype=torch.int32),
+        "positions": torch.randint(0, 4096, (tokens,), generator=g, dtype=torch.int32),
+        "new_cache_slots": torch.randint(0, 1 << 20, (tokens,), generator=g, dtype=torch.int32),
+        "kv_seq_lens": torch.cat([torch.zeros(1, dtype=torch.int32), lens.cumsum(0).to(torch.int32)]),
+        "paged_kv_indptr": torch.cat([torch.zeros(1, dtype=torch.int32), pages.cumsum(0).to(torch.int32)]),
+        "paged_kv_indices": torch.randint(0, 5000, (int(pages.sum()),), generator=g, dtype=torch.int32),
+        "paged_kv_last_page_len": ((lens - 1) % 16 + 1).to(torch.int32),
+    }
+    width = max(padded, tokens, batch) + 3
+    dst = {k: torch.full((width + (1 if k in ("kv_seq_lens", "paged_kv_indptr") else 0),), -77, dtype=torch.int32)
+           for k in ("tokens", "positions", "new_cache_slots", "kv_seq_lens", "kv_seq_lens_delta", "paged_kv_indptr",
+                     "paged_kv_last_page_len")}
+    dst["paged_kv_indices"] = torch.full((int(pages.sum()) + 5,), -77, dtype=torch.int32)
+    return src, dst
+
+
+def _metadata_by_slices(src, dst, n_tok, n_pad, batch, n_idx):
+    """The executor's slow path that the kernel replaces: slice copies and fills
+    (xllm/core/runtime/cuda_graph_executor_impl.cpp:397-453 and the FlashInfer buffers after it)."""
+    for k in ("tokens", "positions", "new_cache_slots"):
+        dst[k][:n_tok] = src[k][:n_tok]
+    if n_pad > n_tok:
+        dst["tokens"][n_tok:n_pad] = 0
+        dst["positions"][n_tok:n_pad] = 0
+        dst["new_cache_slots"][n_tok:n_pad] = -1
+    for k in ("kv_seq_lens", "paged_kv_indptr"):
+        dst[k][: batch + 1] = src[k][: batch + 1]
+        if n_pad > batch:
+            dst[k][batch + 1 : n_pad + 1] = src[k][batch]
+    dst["kv_seq_lens_delta"][:batch] = src["kv_seq_lens"][1 : batch + 1] - src["kv_seq_lens"][:batch]
+    dst["paged_kv_last_page_len"][:batch] = src["paged_kv_last_page_len"][:batch]
+    if n_pad > batch:
+        dst["kv_seq_lens_delta"][batch:n_pad] = 0
+        dst["paged_kv_last_page_len"][batch:n_pad] = 1
+    dst["paged_kv_indices"][:n_idx] = src["paged_kv_indices"][:n_idx]
+    return dst
+
+
+def test_decode_metadata_update_rules_equal_the_slice_copies_they_replace():
+    # llm_decode_metadata_update.cu:27-71 states the update index by index; the executor path it replaces states it
+    # as slice copies and fills.  Equal on: no padding, padding, fewer sequences than tokens (speculative steps),
+    # an empty step, and nothing outside the padded range is touched (sentinel -77 survives).
+    import oracle
+    for seed, batch, padded, tokens in ((1, 7, 7, None), (2, 5, 16, None), (3, 1, 8, None), (4, 6, 32, 12),
+                                        (5, 40, 64, None), (6, 0, 4, 0)):
+        src, a = _metadata_case(seed, batch, padded, tokens)
+        _, b = _metadata_case(seed, batch, padded, tokens)
+        n_tok = src["tokens"].numel()
+        n_idx = src["paged_kv_indices"].numel()
+        oracle.llm_decode_metadata_update(src, a, n_tok, padded, batch, n_idx)
+        _metadata_by_slices(src, b, n_tok, padded, batch, n_idx)
+        for k in a:
+            assert torch.equal(a[k], b[k]), (seed, k)
+        assert int(a["tokens"][max(padded, n_tok)]) == -77 and int(a["kv_seq_lens"][max(padded, batch) + 1]) == -77
+        if padded > batch:
+            assert int(a["kv_seq_lens"][padded]) == int(src["kv_seq_lens"][batch])
+            assert int(a["paged_kv_last_page_len"][padded - 1]) == 1 and int(a["new_cache_slots"][padded - 1]) == -1

@@ -135,6 +135,22 @@ int xllm_mi355_lse_merge(const void* partial_out, const float* partial_lse, void
                    static_cast<hipStream_t>(stream));
 }
 
+int xllm_mi355_decode_metadata_update(const int32_t* src_tokens, const int32_t* src_positions,
+                                      const int32_t* src_new_cache_slots, const int32_t* src_kv_seq_lens,
+                                      const int32_t* src_paged_kv_indptr, const int32_t* src_paged_kv_indices,
+                                      const int32_t* src_paged_kv_last_page_len, int32_t* dst_tokens,
+                                      int32_t* dst_positions, int32_t* dst_new_cache_slots, int32_t* dst_kv_seq_lens,
+                                      int32_t* dst_kv_seq_lens_delta, int32_t* dst_paged_kv_indptr,
+                                      int32_t* dst_paged_kv_indices, int32_t* dst_paged_kv_last_page_len,
+                                      int64_t actual_num_tokens, int64_t padded_num_tokens, int64_t actual_batch_size,
+                                      int64_t actual_indices_size, void* stream) {
+  return decode_metadata_update(src_tokens, src_positions, src_new_cache_slots, src_kv_seq_lens, src_paged_kv_indptr,
+                                src_paged_kv_indices, src_paged_kv_last_page_len, dst_tokens, dst_positions,
+                                dst_new_cache_slots, dst_kv_seq_lens, dst_kv_seq_lens_delta, dst_paged_kv_indptr,
+                                dst_paged_kv_indices, dst_paged_kv_last_page_len, actual_num_tokens, padded_num_tokens,
+                                actual_batch_size, actual_indices_size, static_cast<hipStream_t>(stream));
+}
+
 int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr, const int32_t* paged_kv_indices,
                                  const int32_t* paged_kv_last_page_len, int32_t* block_table,
                                  int64_t table_stride, int32_t* seq_lens, int64_t batch,

@@ -81,6 +81,15 @@ int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t tab
                       const int32_t* cu_seq_lens, void* out, int64_t batch, int64_t total_rows,
                       int64_t block_size, int64_t num_blocks, int64_t row_bytes, hipStream_t stream);
 
+int decode_metadata_update(const int32_t* src_tokens, const int32_t* src_positions, const int32_t* src_new_cache_slots,
+                           const int32_t* src_kv_seq_lens, const int32_t* src_paged_kv_indptr,
+                           const int32_t* src_paged_kv_indices, const int32_t* src_paged_kv_last_page_len,
+                           int32_t* dst_tokens, int32_t* dst_positions, int32_t* dst_new_cache_slots,
+                           int32_t* dst_kv_seq_lens, int32_t* dst_kv_seq_lens_delta, int32_t* dst_paged_kv_indptr,
+                           int32_t* dst_paged_kv_indices, int32_t* dst_paged_kv_last_page_len,
+                           int64_t actual_num_tokens, int64_t padded_num_tokens, int64_t actual_batch_size,
+                           int64_t actual_indices_size, hipStream_t stream);
+
 // Kernel attributes (dynamic LDS size) are set per device.  Returns true the first time it is called with
 // `seen` on the current device (devices 0..63; beyond that always true: setting them again is harmless).
 inline bool first_use_on_current_device(std::atomic<uint64_t>& seen) {

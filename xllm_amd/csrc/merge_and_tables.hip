@@ -6,6 +6,8 @@
 //   gather_paged_rows  -- rows of paged sequences -> one packed [total_rows, row_bytes] buffer, sequence after
 //                         sequence (xllm/core/kernels/dcu/gather_mla_latent_cache.hip:32-75: the latent rows
 //                         of the context for prefill with context)
+//   decode_metadata_update -- a step's metadata into the persistent buffers of a captured step, padded
+//                         (xllm/core/kernels/cuda/llm_decode_metadata_update.cu:27-71)
 //   expand_varlen      -- per query token of a packed batch: attended length and block-table row, so that
 //                         short query chunks run through the decode kernels
 //                         (xllm/core/layers/dcu/flash_attention.cpp:447-545, the hg_prefix_decode_varlen_fwd branch)
@@ -66,6 +68,43 @@ __global__ __launch_bounds__(256) void build_block_table_kernel(const int32_t* i
     table[b * stride + j] = j < n ? indices[p0 + j] : -1;
   if (seq_lens != nullptr && threadIdx.x == 0)
     seq_lens[b] = n > 0 ? (n - 1) * block_size + last_page_len[b] : 0;
+}
+
+struct MetadataUpdate {
+  const int32_t *tokens, *positions, *slots, *kv_cu, *indptr, *indices, *last_page_len;
+  int32_t *d_tokens, *d_positions, *d_slots, *d_kv_cu, *d_kv_delta, *d_indptr, *d_indices, *d_last_page_len;
+  int64_t n_tokens, n_padded, batch, n_indices;
+};
+// One thread per index of the longest array.  Integer copies and fills, nothing else: the rules of the
+// reference kernel index by index.
+__global__ __launch_bounds__(256) void decode_metadata_update_kernel(MetadataUpdate u, int64_t n) {
+  const int64_t step = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += step) {
+    if (i < u.n_tokens) {
+      u.d_tokens[i] = u.tokens[i];
+      u.d_positions[i] = u.positions[i];
+      u.d_slots[i] = u.slots[i];
+    } else if (i < u.n_padded) {
+      u.d_tokens[i] = 0;
+      u.d_positions[i] = 0;
+      u.d_slots[i] = -1;
+    }
+    if (i < u.batch + 1) {
+      u.d_kv_cu[i] = u.kv_cu[i];
+      u.d_indptr[i] = u.indptr[i];
+    } else if (i < u.n_padded + 1) {
+      u.d_kv_cu[i] = u.kv_cu[u.batch];
+      u.d_indptr[i] = u.indptr[u.batch];
+    }
+    if (i < u.batch) {
+      u.d_kv_delta[i] = u.kv_cu[i + 1] - u.kv_cu[i];
+      u.d_last_page_len[i] = u.last_page_len[i];
+    } else if (i < u.n_padded) {
+      u.d_kv_delta[i] = 0;
+      u.d_last_page_len[i] = 1;
+    }
+    if (i < u.n_indices) u.d_indices[i] = u.indices[i];
+  }
 }
 
 // One thread per query token.  Token t belongs to the sequence b with cu[b] <= t < cu[b + 1]; with q_len
@@ -265,6 +304,43 @@ int build_block_table(const int32_t* indptr, const int32_t* indices, const int32
   if (batch < 0 || batch > 0x7fffffffLL || table_stride <= 0 || block_size <= 0) return XLLM_MI355_EINVAL;
   build_block_table_kernel<<<dim3(static_cast<unsigned>(batch)), 256, 0, stream>>>(
       indptr, indices, last_page_len, block_table, table_stride, seq_lens, static_cast<int>(block_size));
+  return static_cast<int>(hipGetLastError());
+}
+
+int decode_metadata_update(const int32_t* src_tokens, const int32_t* src_positions, const int32_t* src_new_cache_slots,
+                           const int32_t* src_kv_seq_lens, const int32_t* src_paged_kv_indptr,
+                           const int32_t* src_paged_kv_indices, const int32_t* src_paged_kv_last_page_len,
+                           int32_t* dst_tokens, int32_t* dst_positions, int32_t* dst_new_cache_slots,
+                           int32_t* dst_kv_seq_lens, int32_t* dst_kv_seq_lens_delta, int32_t* dst_paged_kv_indptr,
+                           int32_t* dst_paged_kv_indices, int32_t* dst_paged_kv_last_page_len,
+                           int64_t actual_num_tokens, int64_t padded_num_tokens, int64_t actual_batch_size,
+                           int64_t actual_indices_size, hipStream_t stream) {
+  if (actual_num_tokens < 0 || padded_num_tokens < 0 || actual_batch_size < 0 || actual_indices_size < 0)
+    return XLLM_MI355_EINVAL;
+  // the largest index any rule touches (llm_decode_metadata_update.cu:76-91)
+  int64_t n = actual_num_tokens;
+  if (padded_num_tokens + 1 > n) n = padded_num_tokens + 1;
+  if (actual_batch_size + 1 > n) n = actual_batch_size + 1;
+  if (actual_indices_size > n) n = actual_indices_size;
+  const bool tokens_on = actual_num_tokens > 0 || padded_num_tokens > 0;
+  if (tokens_on && (dst_tokens == nullptr || dst_positions == nullptr || dst_new_cache_slots == nullptr ||
+                    dst_kv_seq_lens_delta == nullptr || dst_paged_kv_last_page_len == nullptr))
+    return XLLM_MI355_EINVAL;
+  if (actual_num_tokens > 0 && (src_tokens == nullptr || src_positions == nullptr || src_new_cache_slots == nullptr))
+    return XLLM_MI355_EINVAL;
+  if (src_kv_seq_lens == nullptr || src_paged_kv_indptr == nullptr || dst_kv_seq_lens == nullptr ||
+      dst_paged_kv_indptr == nullptr)
+    return XLLM_MI355_EINVAL;
+  if (actual_batch_size > 0 && src_paged_kv_last_page_len == nullptr) return XLLM_MI355_EINVAL;
+  if (actual_indices_size > 0 && (src_paged_kv_indices == nullptr || dst_paged_kv_indices == nullptr))
+    return XLLM_MI355_EINVAL;
+  const MetadataUpdate u = {src_tokens, src_positions, src_new_cache_slots, src_kv_seq_lens, src_paged_kv_indptr,
+                            src_paged_kv_indices, src_paged_kv_last_page_len, dst_tokens, dst_positions,
+                            dst_new_cache_slots, dst_kv_seq_lens, dst_kv_seq_lens_delta, dst_paged_kv_indptr,
+                            dst_paged_kv_indices, dst_paged_kv_last_page_len, actual_num_tokens, padded_num_tokens,
+                            actual_batch_size, actual_indices_size};
+  const int64_t blocks = (n + 255) / 256;
+  decode_metadata_update_kernel<<<dim3(static_cast<unsigned>(blocks < 4096 ? blocks : 4096)), 256, 0, stream>>>(u, n);
   return static_cast<int>(hipGetLastError());
 }
 

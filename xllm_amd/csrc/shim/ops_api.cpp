@@ -205,6 +205,16 @@ torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch:
   return out;
 }
 
+void update_llm_decode_metadata(const LlmDecodeMetadataUpdateParams& p, void* stream) {
+  const int rc = xllm_mi355_decode_metadata_update(
+      p.src_tokens, p.src_positions, p.src_new_cache_slots, p.src_kv_seq_lens, p.src_paged_kv_indptr,
+      p.src_paged_kv_indices, p.src_paged_kv_last_page_len, p.dst_tokens, p.dst_positions, p.dst_new_cache_slots,
+      p.dst_kv_seq_lens, p.dst_kv_seq_lens_delta, p.dst_paged_kv_indptr, p.dst_paged_kv_indices,
+      p.dst_paged_kv_last_page_len, p.actual_num_tokens, p.padded_num_tokens, p.actual_batch_size,
+      p.actual_indices_size, stream);
+  check_rc(rc, "xllm_mi355_decode_metadata_update");
+}
+
 namespace flash_mla {
 
 torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {

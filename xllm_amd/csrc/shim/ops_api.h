@@ -69,6 +69,32 @@ torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch:
                                       const torch::Tensor& kv_cu_seq_lens, int64_t total_kv_len,
                                       int64_t max_seq_len);
 
+// xllm::kernel::cuda::LlmDecodeMetadataUpdateParams and update_llm_decode_metadata
+// (xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56), field for field; the stream is the
+// caller's, as there.
+struct LlmDecodeMetadataUpdateParams {
+  const int32_t* src_tokens;
+  const int32_t* src_positions;
+  const int32_t* src_new_cache_slots;
+  const int32_t* src_kv_seq_lens;
+  const int32_t* src_paged_kv_indptr;
+  const int32_t* src_paged_kv_indices;
+  const int32_t* src_paged_kv_last_page_len;
+  int32_t* dst_tokens;
+  int32_t* dst_positions;
+  int32_t* dst_new_cache_slots;
+  int32_t* dst_kv_seq_lens;
+  int32_t* dst_kv_seq_lens_delta;
+  int32_t* dst_paged_kv_indptr;
+  int32_t* dst_paged_kv_indices;
+  int32_t* dst_paged_kv_last_page_len;
+  int64_t actual_num_tokens;
+  int64_t padded_num_tokens;
+  int64_t actual_batch_size;
+  int64_t actual_indices_size;
+};
+void update_llm_decode_metadata(const LlmDecodeMetadataUpdateParams& params, void* stream);
+
 namespace flash_mla {
 struct DenseDecodeParams {
   torch::Tensor q_nope;       // [B, S_q, H, kv_lora_rank]

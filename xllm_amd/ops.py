@@ -10,6 +10,8 @@ Reference interface mirrored here (paths relative to the xLLM source tree):
   flash_mla::DenseDecodeParams / dense_decode     xllm/core/kernels/dcu/flash_mla_adapter.h:40-53
   merge_dcp_attention_shards                      xllm/core/layers/mlu/dcp_attention_merge.h:28-34
   build_block_table_from_paged_kv                 xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip
+  LlmDecodeMetadataUpdateParams, update_llm_decode_metadata
+                                                  xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56
   gather_mla_latent_cache                         xllm/core/kernels/dcu/dcu_ops_api.h:74
   FlashAttentionImpl::paged_forward (q chunks)    xllm/core/layers/dcu/flash_attention.cpp:447-545
 
@@ -371,6 +373,52 @@ def build_block_table_from_paged_kv(paged_kv_indptr, paged_kv_indices, paged_kv_
         table.data_ptr(), table_width, seq_lens.data_ptr(), B, block_size, _stream(dev))
     capi.check(rc, "xllm_mi355_build_block_table")
     return table, seq_lens
+
+
+@dataclass
+class LlmDecodeMetadataUpdateParams:
+    """Mirror of xllm::kernel::cuda::LlmDecodeMetadataUpdateParams
+    (xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-53): int32 device tensors and four sizes."""
+    src_tokens: torch.Tensor
+    src_positions: torch.Tensor
+    src_new_cache_slots: torch.Tensor
+    src_kv_seq_lens: torch.Tensor          # cumulative, [actual_batch_size + 1]
+    src_paged_kv_indptr: torch.Tensor
+    src_paged_kv_indices: torch.Tensor
+    src_paged_kv_last_page_len: torch.Tensor
+    dst_tokens: torch.Tensor
+    dst_positions: torch.Tensor
+    dst_new_cache_slots: torch.Tensor
+    dst_kv_seq_lens: torch.Tensor
+    dst_kv_seq_lens_delta: torch.Tensor
+    dst_paged_kv_indptr: torch.Tensor
+    dst_paged_kv_indices: torch.Tensor
+    dst_paged_kv_last_page_len: torch.Tensor
+    actual_num_tokens: int
+    padded_num_tokens: int
+    actual_batch_size: int
+    actual_indices_size: int
+
+
+_METADATA_FIELDS = ("src_tokens", "src_positions", "src_new_cache_slots", "src_kv_seq_lens", "src_paged_kv_indptr",
+                    "src_paged_kv_indices", "src_paged_kv_last_page_len", "dst_tokens", "dst_positions",
+                    "dst_new_cache_slots", "dst_kv_seq_lens", "dst_kv_seq_lens_delta", "dst_paged_kv_indptr",
+                    "dst_paged_kv_indices", "dst_paged_kv_last_page_len")
+
+
+def update_llm_decode_metadata(params: LlmDecodeMetadataUpdateParams):
+    """update_llm_decode_metadata (llm_decode_metadata_update.cu:74-104): one launch on the current stream that
+    copies a decode step's metadata into the persistent buffers of a captured step and pads them."""
+    tensors = [getattr(params, f) for f in _METADATA_FIELDS]
+    dev = _require_cuda(*[t for t in tensors if t is not None and t.numel() > 0])
+    for f, t in zip(_METADATA_FIELDS, tensors):
+        if t is not None and (t.dtype != torch.int32 or not t.is_contiguous()):
+            raise ValueError(f"{f} must be a contiguous int32 tensor")
+    rc = capi.lib().xllm_mi355_decode_metadata_update(
+        *[0 if t is None or t.numel() == 0 else t.data_ptr() for t in tensors],
+        params.actual_num_tokens, params.padded_num_tokens, params.actual_batch_size, params.actual_indices_size,
+        _stream(dev))
+    capi.check(rc, "xllm_mi355_decode_metadata_update")
 
 
 def gather_mla_latent_cache(k_cache, block_table, kv_cu_seq_lens, total_kv_len, max_seq_len=0):
