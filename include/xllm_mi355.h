@@ -252,6 +252,31 @@ int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr,
                                  int64_t batch, int64_t block_size, void* stream);
 
 /*
+ * Per-head RMS norm + rotary embedding of the q and k heads of a fused qkv buffer, in place; with a cache,
+ * also the cache write of the new k and v rows in the same launch.  Replaces
+ * xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/fused_qknorm_rope.cu:79-300, 388-470;
+ * caller xllm/core/layers/common/qwen2_attention.cpp:144-186) and, with k_cache / v_cache / slot_mapping, the
+ * reshape_paged_cache call that follows it (xllm/core/kernels/ops_api.h:31): the cache receives the bits
+ * stored in place for k and the untouched v (quantised per KV head when cache_dtype is fp8), what
+ * xllm_mi355_reshape_and_cache would write from the buffer afterwards.
+ *   qkv            [T, token_stride] 16-bit: n_heads_q, then n_heads_k, then n_heads_v heads of head_dim
+ *   q_weight, k_weight  [head_dim] of the qkv dtype, or both null (no norm)
+ *   cos_sin_cache  [max_position, rotary_dim]: cos of the rotary_dim / 2 frequencies, then sin
+ *   position_ids   [T] int64
+ *   interleave     nonzero: pairs (2i, 2i + 1); zero: pairs (i, i + rotary_dim / 2)
+ * head_dim 64, 128 or 256; rotary_dim a multiple of head_dim / 16.  k_cache null: no cache write.
+ */
+int xllm_mi355_rope_and_cache(void* qkv, const void* q_weight, const void* k_weight,
+                              const void* cos_sin_cache, const int64_t* position_ids,
+                              void* k_cache, void* v_cache, const int32_t* slot_mapping,
+                              const float* k_scale, const float* v_scale,
+                              int64_t n_tokens, int64_t token_stride,
+                              int64_t n_heads_q, int64_t n_heads_k, int64_t n_heads_v,
+                              int64_t head_dim, int64_t rotary_dim, float eps, int interleave,
+                              int64_t block_size, int64_t num_blocks,
+                              int dtype, int cos_sin_dtype, int cache_dtype, void* stream);
+
+/*
  * Decode metadata into the persistent buffers of a captured step, with the padding a replay at a larger
  * batch expects.  Replaces xllm::kernel::cuda::update_llm_decode_metadata and its parameter struct,
  * field for field (xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56, .cu:27-71; caller

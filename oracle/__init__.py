@@ -266,6 +266,35 @@ def build_block_table(indptr, indices, last_page_len, table_stride, block_size):
     return table, seq_lens
 
 
+def fused_qk_norm_rope(qkv, n_q, n_k, n_v, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleave,
+                       position_ids):
+    """Restatement of fused_qknorm_rope_kernel (xllm/core/kernels/cuda/fused_qknorm_rope.cu:79-300): fp32 between
+    one load and one store -- x * rsqrt(mean(x^2) + eps) * weight, then the rotation of the leading rotary_dim dims
+    by the cos | sin row of the token's position, rounded once.  Returns a new tensor.  Pinned in
+    tests/test_oracle_attention.py by rotations with known answers, norm preservation, and the torch reference of
+    the reference's own test (tests/core/kernels/dcu/fused_qknorm_rope_test.cpp:27-118) within its tolerance."""
+    T = qkv.shape[0]
+    rotary_dim = cos_sin_cache.shape[1]
+    half = rotary_dim // 2
+    out = qkv.clone()
+    x = qkv[:, : (n_q + n_k) * head_dim].float().view(T, n_q + n_k, head_dim)
+    if q_weight is not None:
+        w = torch.cat([q_weight.float().view(1, 1, -1).expand(1, n_q, -1), k_weight.float().view(1, 1, -1).expand(1, n_k, -1)], 1)
+        x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w
+    cs = cos_sin_cache.float()[position_ids.long()]
+    cos, sin = cs[:, None, :half], cs[:, None, half:]
+    rot = x[..., :rotary_dim]
+    if interleave:
+        e, o = rot[..., 0::2], rot[..., 1::2]
+        new = torch.stack([e * cos - o * sin, e * sin + o * cos], -1).flatten(-2)
+    else:
+        a, b = rot[..., :half], rot[..., half:]
+        new = torch.cat([a * cos - b * sin, b * cos + a * sin], -1)
+    y = torch.cat([new, x[..., rotary_dim:]], -1)
+    out[:, : (n_q + n_k) * head_dim] = y.reshape(T, -1).to(qkv.dtype)
+    return out
+
+
 def llm_decode_metadata_update(src, dst, actual_num_tokens, padded_num_tokens, actual_batch_size,
                                actual_indices_size):
     """Restatement of llm_decode_metadata_update_kernel, rule by rule and index by index

@@ -228,3 +228,50 @@ def test_decode_metadata_update_is_bit_exact(device):
         torch.cuda.synchronize()
         for k in want:
             assert torch.equal(d[k].cpu(), want[k]), (seed, k)
+
+
+def test_fused_qk_norm_rope_and_its_cache_write(device):
+    # fused_qk_norm_rope (kernels/cuda/fused_qknorm_rope.cu): q and k heads within the reference test's tolerance
+    # of the oracle (fp32 arithmetic, one rounding), v untouched; with a cache, the pages hold bit for bit what
+    # reshape_and_cache writes from the rotated buffer (16-bit and fp8 pages, skipped slots included).
+    g = torch.Generator().manual_seed(11)
+    cases = ((17, 8, 4, 4, 128, 128, torch.float16, torch.float32, False), (11, 6, 2, 2, 64, 64, torch.bfloat16, torch.float32, True),
+             (64, 32, 8, 8, 128, 128, torch.bfloat16, torch.bfloat16, False), (5, 4, 2, 2, 256, 128, torch.bfloat16, torch.float16, False),
+             (9, 4, 4, 4, 128, 64, torch.float16, torch.float32, True), (1, 16, 2, 2, 64, 32, torch.bfloat16, torch.float32, False))
+    for T, n_q, n_k, n_v, D, rd, dt, cdt, inter in cases:
+        qkv = (torch.randn(T, (n_q + n_k + n_v) * D, generator=g) * 0.3).to(dt)
+        qw, kw = (1 + 0.2 * torch.randn(D, generator=g)).to(dt), (1 + 0.2 * torch.randn(D, generator=g)).to(dt)
+        ang = torch.rand(300, rd // 2, generator=g) * 6.28
+        cs = torch.cat([ang.cos(), ang.sin()], 1).to(cdt)
+        pos = torch.randint(0, 300, (T,), generator=g)
+        want = oracle.fused_qk_norm_rope(qkv, n_q, n_k, n_v, D, 1e-6, qw, kw, cs, inter, pos)
+        got = ops.fused_qk_norm_rope(qkv.to(device), n_q, n_k, n_v, D, 1e-6, qw.to(device), kw.to(device),
+                                     cs.to(device), inter, pos.to(device))
+        torch.cuda.synchronize()
+        tol = 2e-3 if dt == torch.float16 else 1.6e-2    # one unit in the last place of the 16-bit type
+        assert torch.allclose(got.cpu().float(), want.float(), rtol=tol, atol=tol), (T, D, inter)
+        assert (got.cpu().float() - want.float()).abs().mean() < 2e-4
+        assert torch.equal(got.cpu()[:, (n_q + n_k) * D :], qkv[:, (n_q + n_k) * D :])
+        # the same launch with the cache write
+        bs, P = 16, 12
+        slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
+        slots[0] = -1
+        for cache_dt in (dt, torch.float8_e4m3fn):
+            kc = torch.zeros(P, bs, n_k, D, dtype=cache_dt, device=device)
+            vc = torch.zeros_like(kc)
+            ks = (0.5 + torch.rand(n_k, generator=g)).to(device) if cache_dt == torch.float8_e4m3fn else None
+            vs = (0.5 + torch.rand(n_k, generator=g)).to(device) if cache_dt == torch.float8_e4m3fn else None
+            buf = ops.fused_qk_norm_rope(qkv.to(device), n_q, n_k, n_v, D, 1e-6, qw.to(device), kw.to(device),
+                                         cs.to(device), inter, pos.to(device), k_cache=kc, v_cache=vc,
+                                         slot_mapping=slots.to(device), k_cache_scale=ks, v_cache_scale=vs)
+            torch.cuda.synchronize()
+            assert torch.equal(buf, got)
+            kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+            k_rows = buf[:, n_q * D : (n_q + n_k) * D].view(T, n_k, D)
+            v_rows = buf[:, (n_q + n_k) * D :].view(T, n_v, D)
+            params = ops.ReshapePagedCacheParams(key=k_rows, value=v_rows, k_cache=kc2, v_cache=vc2,
+                                                 slot_mapping=slots.to(device), k_cache_scale=ks, v_cache_scale=vs)
+            (ops.quant_to_paged_cache if ks is not None else ops.reshape_paged_cache)(params)
+            torch.cuda.synchronize()
+            assert torch.equal(kc.view(torch.uint8), kc2.view(torch.uint8))
+            assert torch.equal(vc.view(torch.uint8), vc2.view(torch.uint8))

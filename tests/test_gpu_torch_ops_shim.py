@@ -113,3 +113,31 @@ def test_query_chunks_and_latent_gather_through_the_dispatcher(device, xops):
     got = xops.gather_mla_latent_cache(kc.to(device), lay.block_table.to(device), kv_cu.to(device), int(kv_cu[-1]),
                                        int(lay.seq_lens.max()))
     assert torch.equal(got.cpu(), oracle.gather_paged_rows(kc, lay.block_table, kv_cu, int(kv_cu[-1])))
+
+
+def test_norm_rope_and_metadata_update_through_the_host_side(device, xops):
+    # fused_qk_norm_rope with the reference's arguments (kernels/cuda/cuda_ops_api.h:235-249) and its variant that
+    # also writes the cache: same bytes as the direct C-ABI calls
+    g = torch.Generator().manual_seed(3)
+    T, n_q, n_k, D = 9, 8, 2, 128
+    qkv = (torch.randn(T, (n_q + 2 * n_k) * D, generator=g) * 0.3).to(torch.bfloat16).to(device)
+    qw = (1 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).to(device)
+    kw = (1 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).to(device)
+    ang = torch.rand(64, D // 2, generator=g) * 6.28
+    cs = torch.cat([ang.cos(), ang.sin()], 1).to(device)
+    pos = torch.randint(0, 64, (T,), generator=g).to(device)
+    slots = torch.randperm(64, generator=g)[:T].to(torch.int32).to(device)
+    direct = ops.fused_qk_norm_rope(qkv.clone(), n_q, n_k, n_k, D, 1e-6, qw, kw, cs, False, pos)
+    via = qkv.clone()
+    ret = xops.fused_qk_norm_rope(via, n_q, n_k, n_k, D, 1e-6, qw, kw, cs, False, pos)
+    torch.cuda.synchronize()
+    assert torch.equal(via, direct) and ret.data_ptr() == via.data_ptr()   # the reference's op returns qkv
+    kc = torch.zeros(4, 16, n_k, D, dtype=torch.bfloat16, device=device)
+    vc = torch.zeros_like(kc)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(kc)
+    via2 = qkv.clone()
+    xops.fused_qk_norm_rope_and_cache(via2, n_q, n_k, n_k, D, 1e-6, qw, kw, cs, False, pos, slots, kc, vc, None, None)
+    ops.fused_qk_norm_rope(qkv.clone(), n_q, n_k, n_k, D, 1e-6, qw, kw, cs, False, pos, k_cache=kc2, v_cache=vc2,
+                           slot_mapping=slots)
+    torch.cuda.synchronize()
+    assert torch.equal(via2, direct) and torch.equal(kc, kc2) and torch.equal(vc, vc2) and bool(kc.abs().sum() > 0)

@@ -202,3 +202,73 @@ def test_query_chunks_equal_dense_attention_with_the_causal_mask_at_the_bottom_r
     q1 = inp.q.contiguous()
     assert torch.equal(oracle.aten_paged_forward(q1, kc, vc, lay.block_table, lay.seq_lens, ones, cfg.scale),
                        oracle.aten_paged_decode(q1, kc, vc, lay.block_table, lay.seq_lens, cfg.scale))
+
+
+def _reference_test_formula(qkv, n_q, n_k, D, eps, qw, kw, cos_sin, interleave, pos):
+    """The torch reference of the reference's own test (tests/core/kernels/dcu/fused_qknorm_rope_test.cpp:27-118):
+    it rounds to the qkv dtype between the norm and the rotation, which the kernel does not."""
+    T = qkv.shape[0]
+    rd = cos_sin.shape[1]
+    h = rd // 2
+    out = qkv.clone()
+    for lo, n, w in ((0, n_q, qw), (n_q * D, n_k, kw)):
+        x = qkv[:, lo : lo + n * D].view(T, n, D).float()
+        x = (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w.float().view(1, 1, D)).to(qkv.dtype).float()
+        sel = cos_sin.index_select(0, pos)
+        cos, sin = sel[:, :h].view(T, 1, h), sel[:, h:].view(T, 1, h)
+        rot, rest = x[..., :rd], x[..., rd:]
+        if interleave:
+            r = rot.reshape(T, n, h, 2)
+            ev, od = r[..., 0], r[..., 1]
+            rot = torch.stack([ev * cos - od * sin, ev * sin + od * cos], -1).view(T, n, rd)
+        else:
+            a, b = rot[..., :h], rot[..., h:]
+            rot = torch.cat([a * cos - b * sin, b * cos + a * sin], -1)
+        out[:, lo : lo + n * D] = torch.cat([rot, rest], -1).to(qkv.dtype).view(T, n * D)
+    return out
+
+
+def test_fused_qk_norm_rope_oracle_known_rotations_and_the_reference_tests_formula():
+    import oracle
+    g = torch.Generator().manual_seed(2026)
+    # (a) the two cases of the reference's test, against its torch formula, with its tolerance
+    for T, n_q, n_k, n_v, D, max_pos, dt, sig, inter in ((17, 8, 4, 4, 128, 512, torch.float16, 0.2, False),
+                                                         (11, 6, 2, 2, 64, 256, torch.bfloat16, 0.15, True)):
+        qkv = (torch.randn(T, (n_q + n_k + n_v) * D, generator=g) * sig).to(dt)
+        qw, kw = torch.randn(D, generator=g).to(dt), torch.randn(D, generator=g).to(dt)
+        cs = torch.randn(max_pos, D, generator=g)
+        pos = torch.randint(0, max_pos, (T,), generator=g)
+        got = oracle.fused_qk_norm_rope(qkv, n_q, n_k, n_v, D, 1e-6, qw, kw, cs, inter, pos)
+        want = _reference_test_formula(qkv, n_q, n_k, D, 1e-6, qw, kw, cs, inter, pos)
+        # (bf16 carries 8 bits: one rounding step between the two formulas is 2^-8 relative)
+        tol = 2e-3 if dt == torch.float16 else 1.6e-2
+        assert torch.allclose(got.float(), want.float(), rtol=tol, atol=tol)
+        assert torch.equal(got[:, (n_q + n_k) * D :], qkv[:, (n_q + n_k) * D :])   # v untouched
+    # (b) known answers.  No norm, a quarter turn (cos 0, sin 1): split form (a, b) -> (-b, a), interleaved
+    # (e, o) -> (-o, e), exactly; a zero turn returns the input; partial rotary_dim leaves the tail alone
+    T, n_q, n_k, D = 3, 2, 1, 64
+    x = torch.randn(T, (n_q + n_k) * D, generator=g).to(torch.bfloat16)
+    pos = torch.tensor([0, 1, 1])
+    for rd in (64, 32):
+        h = rd // 2
+        cs = torch.zeros(2, rd)
+        cs[0, :h] = 1.0          # position 0: zero turn
+        cs[1, h:] = 1.0          # position 1: quarter turn
+        v = x.view(T, n_q + n_k, D)
+        for inter in (False, True):
+            got = oracle.fused_qk_norm_rope(x, n_q, n_k, 0, D, 0.0, None, None, cs, inter, pos).view(T, n_q + n_k, D)
+            assert torch.equal(got[0], v[0])
+            assert torch.equal(got[1:, :, rd:], v[1:, :, rd:])
+            if inter:
+                assert torch.equal(got[1:, :, 0:rd:2], -v[1:, :, 1:rd:2]) and torch.equal(got[1:, :, 1:rd:2], v[1:, :, 0:rd:2])
+            else:
+                assert torch.equal(got[1:, :, :h], -v[1:, :, h:rd]) and torch.equal(got[1:, :, h:rd], v[1:, :, :h])
+    # (c) the norm: unit weights give unit mean square; a rotation by any angle keeps it
+    D = 128
+    x = (torch.randn(5, 3 * D, generator=g) * 3).to(torch.bfloat16)
+    ang = torch.rand(7, D // 2, generator=g) * 6.28
+    cs = torch.cat([ang.cos(), ang.sin()], 1)
+    ones = torch.ones(D, dtype=torch.bfloat16)
+    got = oracle.fused_qk_norm_rope(x, 2, 1, 0, D, 1e-6, ones, ones, cs, False, torch.tensor([0, 3, 6, 2, 2]))
+    ms = (got.float().view(5, 3, D) ** 2).mean(-1)
+    assert torch.allclose(ms, torch.ones_like(ms), atol=1e-2)

@@ -135,6 +135,19 @@ int xllm_mi355_lse_merge(const void* partial_out, const float* partial_lse, void
                    static_cast<hipStream_t>(stream));
 }
 
+int xllm_mi355_rope_and_cache(void* qkv, const void* q_weight, const void* k_weight, const void* cos_sin_cache,
+                              const int64_t* position_ids, void* k_cache, void* v_cache,
+                              const int32_t* slot_mapping, const float* k_scale, const float* v_scale,
+                              int64_t n_tokens, int64_t token_stride, int64_t n_heads_q, int64_t n_heads_k,
+                              int64_t n_heads_v, int64_t head_dim, int64_t rotary_dim, float eps, int interleave,
+                              int64_t block_size, int64_t num_blocks, int dtype, int cos_sin_dtype, int cache_dtype,
+                              void* stream) {
+  return rope_and_cache(qkv, q_weight, k_weight, cos_sin_cache, position_ids, k_cache, v_cache, slot_mapping, k_scale,
+                        v_scale, n_tokens, token_stride, n_heads_q, n_heads_k, n_heads_v, head_dim, rotary_dim, eps,
+                        interleave, block_size, num_blocks, dtype, cos_sin_dtype, cache_dtype,
+                        static_cast<hipStream_t>(stream));
+}
+
 int xllm_mi355_decode_metadata_update(const int32_t* src_tokens, const int32_t* src_positions,
                                       const int32_t* src_new_cache_slots, const int32_t* src_kv_seq_lens,
                                       const int32_t* src_paged_kv_indptr, const int32_t* src_paged_kv_indices,

@@ -81,6 +81,13 @@ int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t tab
                       const int32_t* cu_seq_lens, void* out, int64_t batch, int64_t total_rows,
                       int64_t block_size, int64_t num_blocks, int64_t row_bytes, hipStream_t stream);
 
+int rope_and_cache(void* qkv, const void* q_weight, const void* k_weight, const void* cos_sin_cache,
+                   const int64_t* position_ids, void* k_cache, void* v_cache, const int32_t* slot_mapping,
+                   const float* k_scale, const float* v_scale, int64_t n_tokens, int64_t token_stride,
+                   int64_t n_heads_q, int64_t n_heads_k, int64_t n_heads_v, int64_t head_dim, int64_t rotary_dim,
+                   float eps, int interleave, int64_t block_size, int64_t num_blocks, int dtype, int cos_sin_dtype,
+                   int cache_dtype, hipStream_t stream);
+
 int decode_metadata_update(const int32_t* src_tokens, const int32_t* src_positions, const int32_t* src_new_cache_slots,
                            const int32_t* src_kv_seq_lens, const int32_t* src_paged_kv_indptr,
                            const int32_t* src_paged_kv_indices, const int32_t* src_paged_kv_last_page_len,

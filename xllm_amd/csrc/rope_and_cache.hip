@@ -1,0 +1,251 @@
+// Per-head RMS norm + rotary embedding of the q and k heads of a fused qkv buffer, in place, and -- in the
+// same launch, when a paged cache is given -- the cache write of the new k and v rows.
+//
+// Replaces xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/fused_qknorm_rope.cu:79-300,
+// caller xllm/core/layers/common/qwen2_attention.cpp:144-186) and, with the cache arguments, the
+// reshape_paged_cache call that follows it (xllm/core/kernels/cuda/reshape_paged_cache.cu:23-63): at decode
+// both are launch bound, one launch does the work of two.
+//
+// Arithmetic of the reference kernel: everything in fp32 between one load and one store --
+//   y = x * rsqrt(mean(x^2) + eps) * weight          (weights of the qkv dtype, one set for q, one for k)
+//   rotary_dim leading dims rotated by the cos | sin row of the token's position, either
+//     interleaved  (y[2i], y[2i+1]) -> (y[2i] c_i - y[2i+1] s_i, y[2i] s_i + y[2i+1] c_i)
+//     or split     (y[i], y[i+h])   -> (y[i] c_i - y[i+h] s_i,  y[i+h] c_i + y[i] s_i),  h = rotary_dim / 2
+//   rounded once to the qkv dtype.
+// The cache receives the rounded k (the bits that were just stored in place) and the untouched v, quantised
+// with the per-head scales when the cache is fp8 -- exactly what reshape_and_cache would write from the
+// buffer afterwards.
+//
+// Mapping: 32 lanes per (token, head), two heads per wavefront; a lane owns head_dim / 32 consecutive
+// dims (2, 4 or 8: one 4-, 8- or 16-byte load).  Sum of squares by DPP within the 32 lanes; the partner of
+// the split form is (rotary_dim / 2) / (head_dim / 32) lanes away.
+#include "common.cuh"
+#include "launch.h"
+
+namespace xllm_mi355 {
+
+namespace {
+
+struct RopeArgs {
+  char* qkv;
+  const char* q_weight;
+  const char* k_weight;
+  const char* cos_sin;
+  const int64_t* positions;
+  char* k_cache;
+  char* v_cache;
+  const int32_t* slots;
+  const float* k_scale;
+  const float* v_scale;
+  int64_t token_stride_bytes;
+  int64_t n_units;   // tokens * heads handled per token
+  int64_t n_slots;   // P * block_size
+  float eps;
+  int n_q, n_k, n_v;
+  int rotary_dim;
+  int heads_per_token;  // n_q + n_k (+ n_v with a cache)
+  int norm;             // 0: no RMS norm (weights absent)
+};
+
+// cos / sin caches come in fp32 or in a 16-bit type
+template <int CT>
+__device__ __forceinline__ float cache_at(const char* p, int64_t i) {
+  if constexpr (CT == XLLM_MI355_FP32) return reinterpret_cast<const float*>(p)[i];
+  else if constexpr (CT == XLLM_MI355_BF16) return BF16::to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  else return FP16::to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+}
+
+__device__ __forceinline__ float lane_xor(float x, int mask, int lane) {
+  return as_f32(static_cast<u32>(__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, static_cast<int>(as_u32(x)))));
+}
+
+template <typename QT, int D, int CT, bool INTERLEAVE, bool FP8>
+__global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeArgs a) {
+  constexpr int E = D / 32;  // dims per lane
+  const int lane = threadIdx.x & 63;
+  const int sub = lane & 31;
+  const int64_t unit = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) >> 5;
+  const bool on = unit < a.n_units;  // (lanes past the end keep running: the exchanges below are wave wide)
+  const int64_t token = on ? unit / a.heads_per_token : 0;
+  const int head = on ? static_cast<int>(unit - token * a.heads_per_token) : 0;
+  const bool is_q = head < a.n_q;
+  const bool is_v = head >= a.n_q + a.n_k;
+  char* row = a.qkv + token * a.token_stride_bytes + (static_cast<int64_t>(head) * D + sub * E) * 2;
+
+  uint16_t raw[E];
+  if constexpr (E == 2) *reinterpret_cast<u32*>(raw) = *reinterpret_cast<const u32*>(row);
+  else if constexpr (E == 4) *reinterpret_cast<u32x2*>(raw) = *reinterpret_cast<const u32x2*>(row);
+  else *reinterpret_cast<u32x4*>(raw) = *reinterpret_cast<const u32x4*>(row);
+
+  float x[E];
+  float ss = 0.0f;
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    x[i] = QT::to_f32(raw[i]);
+    ss += x[i] * x[i];
+  }
+  ss = group_sum<32>(ss);
+  if (!is_v && a.norm != 0) {
+    const float r = __builtin_amdgcn_rsqf(ss / static_cast<float>(D) + a.eps);
+    const uint16_t* w = reinterpret_cast<const uint16_t*>(is_q ? a.q_weight : a.k_weight) + sub * E;
+#pragma unroll
+    for (int i = 0; i < E; ++i) x[i] *= r * QT::to_f32(w[i]);
+  }
+
+  // rotary embedding of the leading rotary_dim dims
+  const int64_t pos = on ? a.positions[token] : 0;
+  const int half = a.rotary_dim >> 1;
+  const int64_t cs = pos * a.rotary_dim;
+  const int rotary_lanes = a.rotary_dim / E;
+  if constexpr (INTERLEAVE) {
+    if (!is_v && sub < rotary_lanes) {
+#pragma unroll
+      for (int i = 0; i < E / 2; ++i) {
+        const int j = (sub * E) / 2 + i;
+        const float c = cache_at<CT>(a.cos_sin, cs + j), s = cache_at<CT>(a.cos_sin, cs + half + j);
+        const float e = x[2 * i], o = x[2 * i + 1];
+        x[2 * i] = e * c - o * s;
+        x[2 * i + 1] = e * s + o * c;
+      }
+    }
+  } else {
+    const int pair = half / E;  // lanes between a dim and its partner
+    float other[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) other[i] = lane_xor(x[i], pair, lane);
+    if (!is_v && sub < rotary_lanes) {
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const int d = sub * E + i;
+        const int j = d < half ? d : d - half;
+        const float c = cache_at<CT>(a.cos_sin, cs + j), s = cache_at<CT>(a.cos_sin, cs + half + j);
+        x[i] = x[i] * c + (d < half ? -other[i] : other[i]) * s;
+      }
+    }
+  }
+  if (!on) return;
+
+  if (!is_v) {
+#pragma unroll
+    for (int i = 0; i < E; ++i) raw[i] = QT::from_f32(x[i]);
+    if constexpr (E == 2) *reinterpret_cast<u32*>(row) = *reinterpret_cast<const u32*>(raw);
+    else if constexpr (E == 4) *reinterpret_cast<u32x2*>(row) = *reinterpret_cast<const u32x2*>(raw);
+    else *reinterpret_cast<u32x4*>(row) = *reinterpret_cast<const u32x4*>(raw);
+  }
+  if (a.k_cache == nullptr || is_q) return;
+
+  // cache write of the k head (the bits just stored) or the v head (as loaded)
+  const int64_t slot = a.slots[token];
+  if (slot < 0 || slot >= a.n_slots) return;
+  const int kvh = is_v ? head - a.n_q - a.n_k : head - a.n_q;
+  const int n_kv = is_v ? a.n_v : a.n_k;
+  const int64_t e0 = (slot * n_kv + kvh) * D + sub * E;
+  char* dst = (is_v ? a.v_cache : a.k_cache);
+  if constexpr (FP8) {
+    const float inv = 1.0f / (is_v ? a.v_scale : a.k_scale)[kvh];
+    uint8_t code[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) code[i] = static_cast<uint8_t>(fp8_quantize(QT::to_f32(raw[i]), inv));
+    if constexpr (E == 2) *reinterpret_cast<uint16_t*>(dst + e0) = *reinterpret_cast<const uint16_t*>(code);
+    else if constexpr (E == 4) *reinterpret_cast<u32*>(dst + e0) = *reinterpret_cast<const u32*>(code);
+    else *reinterpret_cast<u32x2*>(dst + e0) = *reinterpret_cast<const u32x2*>(code);
+  } else {
+    if constexpr (E == 2) *reinterpret_cast<u32*>(dst + e0 * 2) = *reinterpret_cast<const u32*>(raw);
+    else if constexpr (E == 4) *reinterpret_cast<u32x2*>(dst + e0 * 2) = *reinterpret_cast<const u32x2*>(raw);
+    else *reinterpret_cast<u32x4*>(dst + e0 * 2) = *reinterpret_cast<const u32x4*>(raw);
+  }
+}
+
+template <typename QT, int D, int CT>
+int launch_rope(const RopeArgs& a, bool interleave, bool fp8, hipStream_t stream) {
+  const int64_t threads = a.n_units * 32;
+  const dim3 grid(static_cast<unsigned>((threads + 255) / 256));
+  if (interleave) {
+    if (fp8) rope_and_cache_kernel<QT, D, CT, true, true><<<grid, 256, 0, stream>>>(a);
+    else rope_and_cache_kernel<QT, D, CT, true, false><<<grid, 256, 0, stream>>>(a);
+  } else {
+    if (fp8) rope_and_cache_kernel<QT, D, CT, false, true><<<grid, 256, 0, stream>>>(a);
+    else rope_and_cache_kernel<QT, D, CT, false, false><<<grid, 256, 0, stream>>>(a);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+template <typename QT, int D>
+int dispatch_cache_type(const RopeArgs& a, int cos_sin_dtype, bool interleave, bool fp8, hipStream_t stream) {
+  switch (cos_sin_dtype) {
+    case XLLM_MI355_FP32: return launch_rope<QT, D, XLLM_MI355_FP32>(a, interleave, fp8, stream);
+    case XLLM_MI355_BF16: return launch_rope<QT, D, XLLM_MI355_BF16>(a, interleave, fp8, stream);
+    case XLLM_MI355_FP16: return launch_rope<QT, D, XLLM_MI355_FP16>(a, interleave, fp8, stream);
+    default: return XLLM_MI355_EDTYPE;
+  }
+}
+
+template <typename QT>
+int dispatch_head_dim(const RopeArgs& a, int64_t head_dim, int cos_sin_dtype, bool interleave, bool fp8,
+                      hipStream_t stream) {
+  switch (head_dim) {
+    case 64: return dispatch_cache_type<QT, 64>(a, cos_sin_dtype, interleave, fp8, stream);
+    case 128: return dispatch_cache_type<QT, 128>(a, cos_sin_dtype, interleave, fp8, stream);
+    case 256: return dispatch_cache_type<QT, 256>(a, cos_sin_dtype, interleave, fp8, stream);
+    default: return XLLM_MI355_ESHAPE;
+  }
+}
+
+}  // namespace
+
+int rope_and_cache(void* qkv, const void* q_weight, const void* k_weight, const void* cos_sin_cache,
+                   const int64_t* position_ids, void* k_cache, void* v_cache, const int32_t* slot_mapping,
+                   const float* k_scale, const float* v_scale, int64_t n_tokens, int64_t token_stride,
+                   int64_t n_heads_q, int64_t n_heads_k, int64_t n_heads_v, int64_t head_dim, int64_t rotary_dim,
+                   float eps, int interleave, int64_t block_size, int64_t num_blocks, int dtype, int cos_sin_dtype,
+                   int cache_dtype, hipStream_t stream) {
+  if (n_tokens == 0) return XLLM_MI355_OK;
+  if (qkv == nullptr || cos_sin_cache == nullptr || position_ids == nullptr) return XLLM_MI355_EINVAL;
+  if ((q_weight == nullptr) != (k_weight == nullptr)) return XLLM_MI355_EINVAL;
+  if (n_tokens < 0 || n_heads_q <= 0 || n_heads_k <= 0 || n_heads_v < 0) return XLLM_MI355_EINVAL;
+  if (dtype != XLLM_MI355_BF16 && dtype != XLLM_MI355_FP16) return XLLM_MI355_EDTYPE;
+  const int64_t dims_per_lane = head_dim / 32;
+  // the reference's conditions (fused_qknorm_rope.cu:150-153, 420-440): an even number of dims per lane,
+  // the rotated lanes a power of two so that a dim's partner is a fixed number of lanes away
+  if (rotary_dim <= 0 || rotary_dim > head_dim || rotary_dim % (2 * dims_per_lane) != 0) return XLLM_MI355_ESHAPE;
+  const int64_t rotary_lanes = rotary_dim / (dims_per_lane > 0 ? dims_per_lane : 1);
+  if (interleave == 0 && (rotary_lanes & (rotary_lanes - 1)) != 0) return XLLM_MI355_ESHAPE;
+  if (token_stride < (n_heads_q + n_heads_k + n_heads_v) * head_dim) return XLLM_MI355_EINVAL;
+  if ((reinterpret_cast<uintptr_t>(qkv) & 15) != 0 || (token_stride * 2) % 16 != 0) return XLLM_MI355_EALIGN;
+  const bool with_cache = k_cache != nullptr;
+  const bool fp8 = with_cache && cache_dtype == XLLM_MI355_FP8_E4M3;
+  if (with_cache) {
+    if (v_cache == nullptr || slot_mapping == nullptr || n_heads_v != n_heads_k || block_size <= 0 || num_blocks <= 0)
+      return XLLM_MI355_EINVAL;
+    if (!fp8 && cache_dtype != dtype) return XLLM_MI355_EDTYPE;
+    if (fp8 && (k_scale == nullptr || v_scale == nullptr)) return XLLM_MI355_EINVAL;
+    if (((reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15) != 0) return XLLM_MI355_EALIGN;
+  }
+  RopeArgs a = {};
+  a.qkv = static_cast<char*>(qkv);
+  a.q_weight = static_cast<const char*>(q_weight);
+  a.k_weight = static_cast<const char*>(k_weight);
+  a.cos_sin = static_cast<const char*>(cos_sin_cache);
+  a.positions = position_ids;
+  a.k_cache = static_cast<char*>(k_cache);
+  a.v_cache = static_cast<char*>(v_cache);
+  a.slots = slot_mapping;
+  a.k_scale = k_scale;
+  a.v_scale = v_scale;
+  a.token_stride_bytes = token_stride * 2;
+  a.n_slots = with_cache ? num_blocks * block_size : 0;
+  a.eps = eps;
+  a.n_q = static_cast<int>(n_heads_q);
+  a.n_k = static_cast<int>(n_heads_k);
+  a.n_v = static_cast<int>(n_heads_v);
+  a.rotary_dim = static_cast<int>(rotary_dim);
+  a.heads_per_token = static_cast<int>(n_heads_q + n_heads_k + (with_cache ? n_heads_v : 0));
+  a.n_units = n_tokens * a.heads_per_token;
+  a.norm = q_weight != nullptr ? 1 : 0;
+  if (a.n_units * 32 / 256 > 0x7fffffffLL) return XLLM_MI355_ESHAPE;
+  return dtype == XLLM_MI355_BF16
+             ? dispatch_head_dim<BF16>(a, head_dim, cos_sin_dtype, interleave != 0, fp8, stream)
+             : dispatch_head_dim<FP16>(a, head_dim, cos_sin_dtype, interleave != 0, fp8, stream);
+}
+
+}  // namespace xllm_mi355

@@ -205,6 +205,73 @@ torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch:
   return out;
 }
 
+namespace {
+void rope_launch(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v, int64_t head_dim,
+                 double eps, const torch::Tensor& q_weight, const torch::Tensor& k_weight,
+                 const torch::Tensor& cos_sin_cache, bool interleaved, const torch::Tensor& position_ids,
+                 ReshapePagedCacheParams* cache) {
+  // the checks of xllm/core/kernels/cuda/fused_qknorm_rope.cu:402-447
+  TORCH_CHECK(qkv.is_cuda() && qkv.is_contiguous(), "qkv must be a contiguous device tensor");
+  TORCH_CHECK(position_ids.is_cuda() && position_ids.is_contiguous(), "position_ids must be a contiguous device tensor");
+  TORCH_CHECK(q_weight.is_cuda() && q_weight.is_contiguous() && k_weight.is_cuda() && k_weight.is_contiguous(),
+              "q_weight and k_weight must be contiguous device tensors");
+  TORCH_CHECK(cos_sin_cache.is_cuda() && cos_sin_cache.is_contiguous(), "cos_sin_cache must be a contiguous device tensor");
+  TORCH_CHECK(position_ids.scalar_type() == torch::kInt64, "position_ids must be int64");
+  TORCH_CHECK(qkv.dim() == 2 && position_ids.dim() == 1 && q_weight.dim() == 1 && k_weight.dim() == 1 &&
+                  cos_sin_cache.dim() == 2,
+              "qkv [T, (Hq + Hk + Hv) * D], position_ids [T], weights [D], cos_sin_cache [max_position, rotary_dim]");
+  TORCH_CHECK(q_weight.size(0) == head_dim && k_weight.size(0) == head_dim, "weights must be [head_dim]");
+  TORCH_CHECK(cos_sin_cache.size(1) % 2 == 0 && cos_sin_cache.size(1) <= head_dim, "rotary_dim must be even and <= head_dim");
+  TORCH_CHECK(qkv.scalar_type() == q_weight.scalar_type() && qkv.scalar_type() == k_weight.scalar_type(),
+              "qkv, q_weight and k_weight must have the same dtype");
+  TORCH_CHECK(position_ids.size(0) == qkv.size(0), "one position per token");
+  TORCH_CHECK(qkv.size(1) == (num_heads_q + num_heads_k + num_heads_v) * head_dim, "qkv width");
+  void* kc = nullptr;
+  void* vc = nullptr;
+  const int32_t* slots = nullptr;
+  const float* ks = nullptr;
+  const float* vs = nullptr;
+  int64_t bs = 0, blocks = 0;
+  int cache_dtype = dtype_code(qkv);
+  torch::Tensor slot32;
+  if (cache != nullptr) {
+    TORCH_CHECK(cache->v_cache.has_value(), "the fused cache write needs k_cache and v_cache");
+    TORCH_CHECK(cache->k_cache.is_contiguous() && cache->v_cache->is_contiguous(), "caches must be contiguous");
+    slot32 = (cache->slot_mapping.scalar_type() == torch::kInt32 ? cache->slot_mapping
+                                                                   : cache->slot_mapping.to(torch::kInt32)).contiguous();
+    kc = cache->k_cache.data_ptr();
+    vc = cache->v_cache->data_ptr();
+    slots = slot32.data_ptr<int32_t>();
+    bs = cache->k_cache.size(1);
+    blocks = cache->k_cache.size(0);
+    cache_dtype = dtype_code(cache->k_cache);
+    if (cache->k_cache_scale.has_value()) ks = cache->k_cache_scale->data_ptr<float>();
+    if (cache->v_cache_scale.has_value()) vs = cache->v_cache_scale->data_ptr<float>();
+  }
+  const int rc = xllm_mi355_rope_and_cache(
+      qkv.data_ptr(), q_weight.data_ptr(), k_weight.data_ptr(), cos_sin_cache.data_ptr(), position_ids.data_ptr<int64_t>(),
+      kc, vc, slots, ks, vs, qkv.size(0), qkv.stride(0), num_heads_q, num_heads_k, num_heads_v, head_dim,
+      cos_sin_cache.size(1), static_cast<float>(eps), interleaved ? 1 : 0, bs, blocks, dtype_code(qkv),
+      dtype_code(cos_sin_cache), cache_dtype, current_stream(qkv));
+  check_rc(rc, "xllm_mi355_rope_and_cache");
+}
+}  // namespace
+
+void fused_qk_norm_rope(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                        int64_t head_dim, double eps, const torch::Tensor& q_weight, const torch::Tensor& k_weight,
+                        const torch::Tensor& cos_sin_cache, bool interleaved, const torch::Tensor& position_ids) {
+  rope_launch(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleaved,
+              position_ids, nullptr);
+}
+
+void fused_qk_norm_rope_and_cache(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                                  int64_t head_dim, double eps, const torch::Tensor& q_weight,
+                                  const torch::Tensor& k_weight, const torch::Tensor& cos_sin_cache, bool interleaved,
+                                  const torch::Tensor& position_ids, ReshapePagedCacheParams& cache) {
+  rope_launch(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleaved,
+              position_ids, &cache);
+}
+
 void update_llm_decode_metadata(const LlmDecodeMetadataUpdateParams& p, void* stream) {
   const int rc = xllm_mi355_decode_metadata_update(
       p.src_tokens, p.src_positions, p.src_new_cache_slots, p.src_kv_seq_lens, p.src_paged_kv_indptr,
@@ -354,6 +421,31 @@ torch::Tensor op_gather_mla_latent_cache(torch::Tensor k_cache, torch::Tensor bl
   return xllm::kernel::mi355::gather_mla_latent_cache(k_cache, block_table, kv_cu_seq_lens, total_kv_len, max_seq_len);
 }
 
+// (the reference's op returns the mutated qkv, xllm/core/kernels/cuda/cuda_ops_library.cpp:121-149, 280-284)
+torch::Tensor op_fused_qk_norm_rope(torch::Tensor qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                           int64_t head_dim, double eps, torch::Tensor q_weight, torch::Tensor k_weight,
+                           torch::Tensor cos_sin_cache, bool interleaved, torch::Tensor position_ids) {
+  xllm::kernel::mi355::fused_qk_norm_rope(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight,
+                                          cos_sin_cache, interleaved, position_ids);
+  return qkv;
+}
+
+torch::Tensor op_fused_qk_norm_rope_and_cache(torch::Tensor qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                                     int64_t head_dim, double eps, torch::Tensor q_weight, torch::Tensor k_weight,
+                                     torch::Tensor cos_sin_cache, bool interleaved, torch::Tensor position_ids,
+                                     torch::Tensor slot_mapping, torch::Tensor key_cache, torch::Tensor value_cache,
+                                     std::optional<torch::Tensor> k_scale, std::optional<torch::Tensor> v_scale) {
+  xllm::kernel::ReshapePagedCacheParams p;
+  p.k_cache = key_cache;
+  p.v_cache = value_cache;
+  p.slot_mapping = slot_mapping;
+  p.k_cache_scale = k_scale;
+  p.v_cache_scale = v_scale;
+  xllm::kernel::mi355::fused_qk_norm_rope_and_cache(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight,
+                                                    k_weight, cos_sin_cache, interleaved, position_ids, p);
+  return qkv;
+}
+
 std::tuple<torch::Tensor, torch::Tensor> op_merge(torch::Tensor partial_outputs, torch::Tensor partial_lse) {
   auto r = xllm::layer::merge_dcp_attention_shards(partial_outputs, partial_lse);
   return {r.output, r.lse};
@@ -375,6 +467,11 @@ TORCH_LIBRARY(xllm_ops, m) {
         "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len, int max_query_len) -> Tensor");
   m.def("gather_mla_latent_cache(Tensor k_cache, Tensor block_table, Tensor kv_cu_seq_lens, int total_kv_len, "
         "int max_seq_len) -> Tensor");
+  m.def("fused_qk_norm_rope(Tensor(a!) qkv, int num_heads_q, int num_heads_k, int num_heads_v, int head_dim, "
+        "float eps, Tensor q_weight, Tensor k_weight, Tensor cos_sin_cache, bool interleaved, Tensor position_ids) -> Tensor");
+  m.def("fused_qk_norm_rope_and_cache(Tensor(a!) qkv, int num_heads_q, int num_heads_k, int num_heads_v, int head_dim, "
+        "float eps, Tensor q_weight, Tensor k_weight, Tensor cos_sin_cache, bool interleaved, Tensor position_ids, "
+        "Tensor slot_mapping, Tensor(b!) key_cache, Tensor(c!) value_cache, Tensor? k_scale, Tensor? v_scale) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
@@ -385,4 +482,6 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("merge_dcp_attention_shards", &op_merge);
   m.impl("paged_forward", &op_paged_forward);
   m.impl("gather_mla_latent_cache", &op_gather_mla_latent_cache);
+  m.impl("fused_qk_norm_rope", &op_fused_qk_norm_rope);
+  m.impl("fused_qk_norm_rope_and_cache", &op_fused_qk_norm_rope_and_cache);
 }

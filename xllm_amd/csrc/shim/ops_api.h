@@ -69,6 +69,18 @@ torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch:
                                       const torch::Tensor& kv_cu_seq_lens, int64_t total_kv_len,
                                       int64_t max_seq_len);
 
+// xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/cuda_ops_api.h:235-249), same arguments.
+void fused_qk_norm_rope(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                        int64_t head_dim, double eps, const torch::Tensor& q_weight, const torch::Tensor& k_weight,
+                        const torch::Tensor& cos_sin_cache, bool interleaved, const torch::Tensor& position_ids);
+// The same launch followed by nothing: it also stores the new k and v rows in the paged cache, which the
+// reference does with reshape_paged_cache / quant_to_paged_cache right after
+// (xllm/core/layers/common/qwen2_attention.cpp:149-186, xllm/core/layers/dcu/flash_attention.cpp:587-595).
+void fused_qk_norm_rope_and_cache(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
+                                  int64_t head_dim, double eps, const torch::Tensor& q_weight,
+                                  const torch::Tensor& k_weight, const torch::Tensor& cos_sin_cache, bool interleaved,
+                                  const torch::Tensor& position_ids, ReshapePagedCacheParams& cache);
+
 // xllm::kernel::cuda::LlmDecodeMetadataUpdateParams and update_llm_decode_metadata
 // (xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56), field for field; the stream is the
 // caller's, as there.

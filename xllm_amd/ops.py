@@ -10,6 +10,7 @@ Reference interface mirrored here (paths relative to the xLLM source tree):
   flash_mla::DenseDecodeParams / dense_decode     xllm/core/kernels/dcu/flash_mla_adapter.h:40-53
   merge_dcp_attention_shards                      xllm/core/layers/mlu/dcp_attention_merge.h:28-34
   build_block_table_from_paged_kv                 xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip
+  fused_qk_norm_rope                              xllm/core/kernels/cuda/fused_qknorm_rope.cu:388-470
   LlmDecodeMetadataUpdateParams, update_llm_decode_metadata
                                                   xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56
   gather_mla_latent_cache                         xllm/core/kernels/dcu/dcu_ops_api.h:74
@@ -373,6 +374,34 @@ def build_block_table_from_paged_kv(paged_kv_indptr, paged_kv_indices, paged_kv_
         table.data_ptr(), table_width, seq_lens.data_ptr(), B, block_size, _stream(dev))
     capi.check(rc, "xllm_mi355_build_block_table")
     return table, seq_lens
+
+
+def fused_qk_norm_rope(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight,
+                       cos_sin_cache, interleave, position_ids, k_cache=None, v_cache=None, slot_mapping=None,
+                       k_cache_scale=None, v_cache_scale=None):
+    """xllm::kernel::cuda::fused_qk_norm_rope with the reference's arguments in the reference's order
+    (kernels/cuda/fused_qknorm_rope.cu:388-470; caller layers/common/qwen2_attention.cpp:149-166): qkv
+    [T, (Hq + Hk + Hv) * D] is normalised and rotated in place.  With k_cache / v_cache / slot_mapping the same
+    launch also writes the new k and v rows into the paged cache (the reshape_paged_cache call that follows in the
+    reference); fp8 caches take the per-KV-head scales."""
+    dev = _require_cuda(qkv, cos_sin_cache, position_ids)
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise ValueError("qkv must be [tokens, (Hq + Hk + Hv) * head_dim] with contiguous rows")
+    if position_ids.dtype != torch.int64 or not position_ids.is_contiguous():
+        raise ValueError("position_ids must be a contiguous int64 tensor")
+    if cos_sin_cache.dim() != 2 or not cos_sin_cache.is_contiguous():
+        raise ValueError("cos_sin_cache must be [max_position, rotary_dim], contiguous")
+    with_cache = k_cache is not None
+    fp8 = with_cache and k_cache.dtype == torch.float8_e4m3fn
+    rc = capi.lib().xllm_mi355_rope_and_cache(
+        qkv.data_ptr(), _ptr(q_weight), _ptr(k_weight), cos_sin_cache.data_ptr(), position_ids.data_ptr(),
+        _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), _ptr(k_cache_scale), _ptr(v_cache_scale),
+        qkv.shape[0], qkv.stride(0), num_heads_q, num_heads_k, num_heads_v, head_dim, cos_sin_cache.shape[1],
+        float(eps), 1 if interleave else 0, k_cache.shape[1] if with_cache else 0,
+        k_cache.shape[0] if with_cache else 0, _dtype_code(qkv), _dtype_code(cos_sin_cache),
+        capi.FP8_E4M3 if fp8 else _dtype_code(qkv), _stream(dev))
+    capi.check(rc, "xllm_mi355_rope_and_cache")
+    return qkv
 
 
 @dataclass
