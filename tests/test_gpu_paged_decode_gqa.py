@@ -231,7 +231,7 @@ def test_empty_sequence_and_argument_errors(device):
 
 
 def test_full_size_config2_split_invariance_and_sampled_parity(device):
-    """BASELINE config 2 at full size: (a) sequences sampled from the batch agree with the oracle,
+    """The llama3_8b workload (batch 64, 32 / 8 heads, block 16, contexts of 512 to 4096 tokens) at full size: (a) sequences sampled from the batch agree with the oracle,
     (b) LSE-merging the decode of two context halves equals the unsplit decode."""
     cfg = workloads.CONFIGS["llama3_8b"]
     inp = workloads.make_inputs(cfg, 2, device=device)

@@ -132,17 +132,23 @@ __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* 
   }
   if (on) tmp[tid] = local;
   __syncthreads();
-  int excl = 0;
-  if (on)
+  if (lo < hi) {  // (threads without a slice have nothing to place: most of them at decode batch sizes)
+    int excl = 0;
     for (int j = 0; j < tid; ++j) excl += tmp[j];
-  for (int b = lo; b < hi; ++b) {
-    const int32_t* pages;
-    int L;
-    sequence_of(a, b, pages, L);
-    prefix[b] = excl;
-    excl += items_of<ITEM>(L);
+    if (per == 1) {  // the slice is one sequence: its count is still in `local`
+      prefix[lo] = excl;
+      excl += local;
+    } else {
+      for (int b = lo; b < hi; ++b) {
+        const int32_t* pages;
+        int L;
+        sequence_of(a, b, pages, L);
+        prefix[b] = excl;
+        excl += items_of<ITEM>(L);
+      }
+    }
+    if (hi == a.batch) prefix[a.batch] = excl;  // the last non-empty slice holds the total
   }
-  if (lo < hi && hi == a.batch) prefix[a.batch] = excl;  // the last non-empty slice holds the total
   __syncthreads();
 }
 

@@ -151,13 +151,20 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
     tmp[tid] = local;
     __syncthreads();
-    int excl = 0;
-    for (int j = 0; j < tid; ++j) excl += tmp[j];
-    for (int b = lo; b < hi; ++b) {
-      prefix[b] = excl;
-      excl += tiles_of(a.seq_lens[b]);
+    if (lo < hi) {  // (threads without a slice have nothing to place: most of them at decode batch sizes)
+      int excl = 0;
+      for (int j = 0; j < tid; ++j) excl += tmp[j];
+      if (per == 1) {  // the slice is one sequence: its count is still in `local`
+        prefix[lo] = excl;
+        excl += local;
+      } else {
+        for (int b = lo; b < hi; ++b) {
+          prefix[b] = excl;
+          excl += tiles_of(a.seq_lens[b]);
+        }
+      }
+      if (hi == a.batch) prefix[a.batch] = excl;
     }
-    if (lo < hi && hi == a.batch) prefix[a.batch] = excl;
     __syncthreads();
   }
   const int64_t total = prefix[a.batch];
@@ -536,13 +543,20 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
     for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
     tmp[tid] = local;
     __syncthreads();
-    int excl = 0;
-    for (int j = 0; j < tid; ++j) excl += tmp[j];
-    for (int b = lo; b < hi; ++b) {
-      prefix[b] = excl;
-      excl += tiles_of(a.seq_lens[b]);
+    if (lo < hi) {  // (threads without a slice have nothing to place: most of them at decode batch sizes)
+      int excl = 0;
+      for (int j = 0; j < tid; ++j) excl += tmp[j];
+      if (per == 1) {  // the slice is one sequence: its count is still in `local`
+        prefix[lo] = excl;
+        excl += local;
+      } else {
+        for (int b = lo; b < hi; ++b) {
+          prefix[b] = excl;
+          excl += tiles_of(a.seq_lens[b]);
+        }
+      }
+      if (hi == a.batch) prefix[a.batch] = excl;
     }
-    if (lo < hi && hi == a.batch) prefix[a.batch] = excl;
     __syncthreads();
   }
   const int64_t total = prefix[a.batch];
@@ -879,13 +893,20 @@ __global__ __launch_bounds__(kWThreads) void mla_decode32w_kernel(MlaArgs a) {
     for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
     tmp[tid] = local;
     __syncthreads();
-    int excl = 0;
-    for (int j = 0; j < tid; ++j) excl += tmp[j];
-    for (int b = lo; b < hi; ++b) {
-      prefix[b] = excl;
-      excl += tiles_of(a.seq_lens[b]);
+    if (lo < hi) {  // (threads without a slice have nothing to place: most of them at decode batch sizes)
+      int excl = 0;
+      for (int j = 0; j < tid; ++j) excl += tmp[j];
+      if (per == 1) {  // the slice is one sequence: its count is still in `local`
+        prefix[lo] = excl;
+        excl += local;
+      } else {
+        for (int b = lo; b < hi; ++b) {
+          prefix[b] = excl;
+          excl += tiles_of(a.seq_lens[b]);
+        }
+      }
+      if (hi == a.batch) prefix[a.batch] = excl;
     }
-    if (lo < hi && hi == a.batch) prefix[a.batch] = excl;
     __syncthreads();
   }
   const int64_t total = prefix[a.batch];
