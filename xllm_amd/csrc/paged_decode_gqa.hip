@@ -118,19 +118,21 @@ __device__ __forceinline__ int workgroup_of(int64_t id, int64_t total, int64_t n
 // Every thread sums a contiguous slice, then adds the totals of the slices before it.  Threads past
 // kThreads (the matrix-core kernel has a wavefront of them) only take part in the barriers.
 template <int ITEM>
-__device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* tmp) {
+__device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* tmp, int* lens = nullptr) {
   const int tid = threadIdx.x;
   const bool on = tid < kThreads;
   const int per = (a.batch + kThreads - 1) / kThreads;
   const int lo = on ? min(a.batch, tid * per) : a.batch, hi = min(a.batch, lo + per);
-  int local = 0;
+  int local = 0, last_len = 0;
   for (int b = lo; b < hi; ++b) {
     const int32_t* pages;
     int L;
     sequence_of(a, b, pages, L);
     local += items_of<ITEM>(L);
+    last_len = L;
   }
   if (on) tmp[tid] = local;
+  if (lens != nullptr && per == 1 && lo < hi) lens[lo] = last_len;  // (kept for the workers: saves them a load each)
   __syncthreads();
   if (lo < hi) {  // (threads without a slice have nothing to place: most of them at decode batch sizes)
     int excl = 0;
@@ -658,13 +660,15 @@ constexpr int kMfmaThreads = 2 * kThreads;   // kWaves loading wavefronts and kW
 template <int NS>
 struct MfmaLayout {
   // LDS: ring [waves][NS][stage] | Q rows [waves][16][256 B] | page-table chunks [waves][3][64] |
-  //      scan scratch [kThreads] | progress counters [waves][2] | stage prefix [batch + 1]
+  //      scan scratch [kThreads] | progress counters [waves][2] | context lengths [kThreads] |
+  //      stage prefix [batch + 1]
   static constexpr int kRingBytes = kWaves * NS * kStageBytes;
   static constexpr int kQOff = kRingBytes;
   static constexpr int kPageOff = kQOff + kWaves * kMfmaHeads * 256;
   static constexpr int kTmpOff = kPageOff + kWaves * 3 * kWave * 4;
   static constexpr int kSyncOff = kTmpOff + kThreads * 4;
-  static constexpr int kPrefixOff = kSyncOff + 2 * kWaves * 4;
+  static constexpr int kLensOff = kSyncOff + 2 * kWaves * 4;   // context lengths of up to kThreads sequences
+  static constexpr int kPrefixOff = kLensOff + kThreads * 4;
 };
 
 // VL (packed query chunks): a batch entry is a sequence with cu_q[b + 1] - cu_q[b] query tokens.  The 16 MFMA
@@ -724,11 +728,23 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // progress of pair w: sync[2 w] stages that have landed, sync[2 w + 1] stages whose slots are free again
   lds_vint* sync = (lds_vint*)(smem + Lay::kSyncOff);
   if (tid < 2 * kWaves) sync[tid] = 0;
-  item_prefix<T>(a, prefix, tmp);
+  // With a plain block table and at most kThreads sequences the context lengths stay in LDS: a worker
+  // then finds a sequence without a trip to memory (one of the four in a row before its first row moves).
+  int* lens = reinterpret_cast<int*>(smem + Lay::kLensOff);
+  const bool lens_in_lds = a.indptr == nullptr && a.table_rows == nullptr && a.batch <= kThreads;
+  item_prefix<T>(a, prefix, tmp, lens_in_lds ? lens : nullptr);
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hb;
   if (blockIdx.x == 0) {
     for (int i = tid; i <= a.batch; i += kMfmaThreads) a.ws_prefix[i] = prefix[i];
   }
+  auto sequence_at = [&](int b, const int32_t*& pages, int& L) {
+    if (lens_in_lds) {
+      pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
+      L = __builtin_amdgcn_readfirstlane(lens[b]);
+    } else {
+      sequence_of_scalar(a, b, pages, L);
+    }
+  };
   if (total == 0) return;
   // ---- from here on the pairs are independent: no workgroup barrier below this line
   const bool loader = wave < kWaves;   // wavefronts 0 .. kWaves - 1 load, wavefront kWaves + w computes what w loads
@@ -762,7 +778,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     cu.hbk = __builtin_amdgcn_readfirstlane(static_cast<int>(rem / cu.n_st));
     cu.st = __builtin_amdgcn_readfirstlane(static_cast<int>(rem - static_cast<int64_t>(cu.hbk) * cu.n_st));
     cu.kvh = cu.hbk / hb_per_kv;
-    sequence_of_scalar(a, cu.b, cu.pages, cu.L);
+    sequence_at(cu.b, cu.pages, cu.L);
     chunk_of(cu);
   };
   auto next_context = [&](CtxCursor& cu) {  // the caller never steps past the last context of the batch
@@ -778,7 +794,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       ++cu.b;
       cu.n_st = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
     } while (cu.n_st == 0);
-    sequence_of_scalar(a, cu.b, cu.pages, cu.L);
+    sequence_at(cu.b, cu.pages, cu.L);
     chunk_of(cu);
   };
   // 64 entries of the context's page table, from page 64 ck on (the tail repeats the last page),
