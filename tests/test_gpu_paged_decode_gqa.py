@@ -326,6 +326,15 @@ def test_long_item_lists_of_the_matrix_core_kernel(device):
     assert_close_to_reference(out, ref, cfg.name)
 
 
+def test_batches_larger_than_a_workgroup_and_than_a_launch(device):
+    # more sequences than threads in a workgroup (the item prefix then sums several sequences per thread and
+    # the workers read the lengths from memory), and more than one launch holds (2048): both kernels
+    for name, batch, Hq, Hkv, D, bs, hi in (("b700_mfma", 700, 8, 2, 128, 16, 200), ("b700_rows", 700, 8, 2, 64, 16, 120),
+                                            ("b2300_mfma", 2300, 4, 1, 128, 16, 70), ("b2300_rows", 2300, 4, 2, 256, 8, 40)):
+        cfg = workloads.DecodeConfig(name, batch, Hq, Hkv, D, bs, 1, hi)
+        _check_config(cfg, 40 + batch + D, device)
+
+
 def test_short_query_chunks_through_the_decode_kernels(device):
     # chunked prefill / speculative-decoding verification (layers/dcu/flash_attention.cpp:447-545): up to 16 query
     # tokens per sequence, the chunk being the tail of its context; both decode kernels, causal and not

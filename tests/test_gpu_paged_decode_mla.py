@@ -58,6 +58,16 @@ def test_head_counts_of_tp_shards_and_reference_test_shape(device):
         _check(_mla_cfg(f"mla{heads}", 2, heads, 1, 400), 40 + heads, device)
 
 
+def test_batches_larger_than_a_workgroup_and_than_a_launch(device, monkeypatch):
+    # more sequences than threads in a workgroup (several per thread in the tile prefix) and more than one launch
+    # holds (1024), in all three kernels
+    for knob in ("", "pairs", "split"):
+        monkeypatch.setenv("XLLM_MI355_MLA_KERNEL", knob)
+        _check(_mla_cfg(f"mla_b600_{knob}", 600, 16, 1, 150), 90, device)
+    monkeypatch.delenv("XLLM_MI355_MLA_KERNEL")
+    _check(_mla_cfg("mla_b1100", 1100, 8, 1, 80), 91, device)
+
+
 def test_reference_lse_closed_form_two_tokens(device):
     # ReturnsFloat32NaturalLogNormalizer: H=2, D=576, Dv=512, L=2, page of 16 rows, scale 1/sqrt(576)
     g = torch.Generator().manual_seed(0)
