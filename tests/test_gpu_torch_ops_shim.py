@@ -141,3 +141,21 @@ def test_norm_rope_and_metadata_update_through_the_host_side(device, xops):
                            slot_mapping=slots)
     torch.cuda.synchronize()
     assert torch.equal(via2, direct) and torch.equal(kc, kc2) and torch.equal(vc, vc2) and bool(kc.abs().sum() > 0)
+    # the graph executor's metadata update under the reference's op name and schema
+    # (kernels/cuda/cuda_ops_library.cpp:161-252, 288-295), against the oracle
+    from test_oracle_reshape import _metadata_case
+    src, want = _metadata_case(21, 9, 16)
+    _, got = _metadata_case(21, 9, 16)
+    n_tok, n_idx = src["tokens"].numel(), src["paged_kv_indices"].numel()
+    oracle.llm_decode_metadata_update(src, want, n_tok, 16, 9, n_idx)
+    sd = {k: v.to(device) for k, v in src.items()}
+    dd = {k: v.to(device) for k, v in got.items()}
+    ret = xops.update_decode_graph_metadata(sd["tokens"], sd["positions"], sd["new_cache_slots"], sd["kv_seq_lens"],
+                                            sd["paged_kv_indptr"], sd["paged_kv_indices"], sd["paged_kv_last_page_len"],
+                                            dd["tokens"], dd["positions"], dd["new_cache_slots"], dd["kv_seq_lens"],
+                                            dd["kv_seq_lens_delta"], dd["paged_kv_indptr"], dd["paged_kv_indices"],
+                                            dd["paged_kv_last_page_len"], 16)
+    torch.cuda.synchronize()
+    assert ret.data_ptr() == dd["tokens"].data_ptr()
+    for k in want:
+        assert torch.equal(dd[k].cpu(), want[k]), k

@@ -446,6 +446,48 @@ torch::Tensor op_fused_qk_norm_rope_and_cache(torch::Tensor qkv, int64_t num_hea
   return qkv;
 }
 
+// xllm_ops::update_decode_graph_metadata of the reference, argument for argument
+// (xllm/core/kernels/cuda/cuda_ops_library.cpp:161-252, schema :288-295): one token per sequence, the sizes
+// taken from the tensors, returns dst_tokens.
+torch::Tensor op_update_decode_graph_metadata(torch::Tensor tokens, torch::Tensor positions, torch::Tensor slot_mapping,
+                                              torch::Tensor kv_seq_lens, torch::Tensor paged_kv_indptr,
+                                              torch::Tensor paged_kv_indices, torch::Tensor paged_kv_last_page_len,
+                                              torch::Tensor dst_tokens, torch::Tensor dst_positions,
+                                              torch::Tensor dst_slot_mapping, torch::Tensor dst_kv_seq_lens,
+                                              torch::Tensor dst_kv_seq_lens_delta, torch::Tensor dst_paged_kv_indptr,
+                                              torch::Tensor dst_paged_kv_indices,
+                                              torch::Tensor dst_paged_kv_last_page_len, int64_t padded_num_tokens) {
+  for (const torch::Tensor* t : {&tokens, &positions, &slot_mapping, &kv_seq_lens, &paged_kv_indptr, &paged_kv_indices,
+                                 &paged_kv_last_page_len, &dst_tokens, &dst_positions, &dst_slot_mapping,
+                                 &dst_kv_seq_lens, &dst_kv_seq_lens_delta, &dst_paged_kv_indptr, &dst_paged_kv_indices,
+                                 &dst_paged_kv_last_page_len})
+    TORCH_CHECK(t->defined() && t->is_cuda() && t->scalar_type() == torch::kInt32 && t->is_contiguous(),
+                "update_decode_graph_metadata takes contiguous int32 device tensors");
+  const int64_t actual_num_tokens = tokens.numel();
+  const int64_t actual_batch_size = paged_kv_last_page_len.numel();
+  const int64_t actual_indices_size = paged_kv_indices.numel();
+  TORCH_CHECK(actual_num_tokens == actual_batch_size, "decode graph requires one token per sequence");
+  TORCH_CHECK(padded_num_tokens >= actual_num_tokens && positions.numel() >= actual_num_tokens &&
+                  slot_mapping.numel() >= actual_num_tokens && kv_seq_lens.numel() >= actual_batch_size + 1 &&
+                  paged_kv_indptr.numel() >= actual_batch_size + 1,
+              "source tensors shorter than the step");
+  TORCH_CHECK(dst_tokens.numel() >= padded_num_tokens && dst_positions.numel() >= padded_num_tokens &&
+                  dst_slot_mapping.numel() >= padded_num_tokens && dst_kv_seq_lens.numel() >= padded_num_tokens + 1 &&
+                  dst_kv_seq_lens_delta.numel() >= padded_num_tokens &&
+                  dst_paged_kv_indptr.numel() >= padded_num_tokens + 1 &&
+                  dst_paged_kv_indices.numel() >= actual_indices_size &&
+                  dst_paged_kv_last_page_len.numel() >= padded_num_tokens,
+              "persistent tensors shorter than the padded step");
+  auto ptr = [](const torch::Tensor& t) { return t.numel() > 0 ? t.data_ptr<int32_t>() : nullptr; };
+  xllm::kernel::mi355::LlmDecodeMetadataUpdateParams p{
+      ptr(tokens), ptr(positions), ptr(slot_mapping), ptr(kv_seq_lens), ptr(paged_kv_indptr), ptr(paged_kv_indices),
+      ptr(paged_kv_last_page_len), ptr(dst_tokens), ptr(dst_positions), ptr(dst_slot_mapping), ptr(dst_kv_seq_lens),
+      ptr(dst_kv_seq_lens_delta), ptr(dst_paged_kv_indptr), ptr(dst_paged_kv_indices), ptr(dst_paged_kv_last_page_len),
+      actual_num_tokens, padded_num_tokens, actual_batch_size, actual_indices_size};
+  xllm::kernel::mi355::update_llm_decode_metadata(p, current_stream(dst_tokens));
+  return dst_tokens;
+}
+
 std::tuple<torch::Tensor, torch::Tensor> op_merge(torch::Tensor partial_outputs, torch::Tensor partial_lse) {
   auto r = xllm::layer::merge_dcp_attention_shards(partial_outputs, partial_lse);
   return {r.output, r.lse};
@@ -467,6 +509,11 @@ TORCH_LIBRARY(xllm_ops, m) {
         "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len, int max_query_len) -> Tensor");
   m.def("gather_mla_latent_cache(Tensor k_cache, Tensor block_table, Tensor kv_cu_seq_lens, int total_kv_len, "
         "int max_seq_len) -> Tensor");
+  m.def("update_decode_graph_metadata(Tensor tokens, Tensor positions, Tensor slot_mapping, Tensor kv_seq_lens, "
+        "Tensor paged_kv_indptr, Tensor paged_kv_indices, Tensor paged_kv_last_page_len, Tensor(a!) dst_tokens, "
+        "Tensor(b!) dst_positions, Tensor(c!) dst_slot_mapping, Tensor(d!) dst_kv_seq_lens, "
+        "Tensor(e!) dst_kv_seq_lens_delta, Tensor(f!) dst_paged_kv_indptr, Tensor(g!) dst_paged_kv_indices, "
+        "Tensor(h!) dst_paged_kv_last_page_len, int padded_num_tokens) -> Tensor(a!)");
   m.def("fused_qk_norm_rope(Tensor(a!) qkv, int num_heads_q, int num_heads_k, int num_heads_v, int head_dim, "
         "float eps, Tensor q_weight, Tensor k_weight, Tensor cos_sin_cache, bool interleaved, Tensor position_ids) -> Tensor");
   m.def("fused_qk_norm_rope_and_cache(Tensor(a!) qkv, int num_heads_q, int num_heads_k, int num_heads_v, int head_dim, "
@@ -482,6 +529,7 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("merge_dcp_attention_shards", &op_merge);
   m.impl("paged_forward", &op_paged_forward);
   m.impl("gather_mla_latent_cache", &op_gather_mla_latent_cache);
+  m.impl("update_decode_graph_metadata", &op_update_decode_graph_metadata);
   m.impl("fused_qk_norm_rope", &op_fused_qk_norm_rope);
   m.impl("fused_qk_norm_rope_and_cache", &op_fused_qk_norm_rope_and_cache);
 }
