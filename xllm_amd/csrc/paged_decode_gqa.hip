@@ -767,10 +767,23 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   const char* qbuf = smem + Lay::kQOff + pair * G * 256;
 
   auto locate = [&](int64_t f, CtxCursor& cu) {
-    int lo = 0, hi = a.batch;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (static_cast<int64_t>(prefix[mid]) * n_hb <= f) lo = mid; else hi = mid;
+    int lo = 0;
+    if (a.batch <= 8 * kWave) {
+      // the prefix does not decrease, so the sequences that start at or before f are a leading run: count
+      // them, one comparison per lane and independent LDS reads, instead of a chain of dependent ones
+      int n_le = 0;
+      for (int b0 = 0; b0 < a.batch; b0 += kWave) {
+        const int b = b0 + lane;
+        const bool le = b < a.batch && static_cast<int64_t>(prefix[b]) * n_hb <= f;
+        n_le += __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+      }
+      lo = n_le - 1;
+    } else {
+      int hi = a.batch;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (static_cast<int64_t>(prefix[mid]) * n_hb <= f) lo = mid; else hi = mid;
+      }
     }
     cu.b = __builtin_amdgcn_readfirstlane(lo);
     cu.n_st = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
