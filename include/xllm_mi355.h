@@ -171,6 +171,24 @@ int xllm_mi355_gather_paged_rows(const void* cache, const int32_t* block_table, 
                                  int64_t num_blocks, int64_t row_bytes, void* stream);
 
 /*
+ * The per-head products either side of the MLA decode, on the matrix cores:
+ *     y[t, h, :] = x[t, h, :] . w[h, :, :]
+ * Replaces the two torch::bmm calls of the reference's absorbed MLA attention
+ * (xllm/core/layers/dcu/deepseek_v2_attention.cpp:428-430: q_nope [T, H, 128] with w_kc_ [H, 128, 512] into the
+ * q_nope operand of xllm_mi355_paged_decode_mla; :231-238: the decode output [T, H, 512] with w_vc_ [H, 512, 128]
+ * into the input of o_proj), with the weights in the layouts the reference prepares at load time (:479-485).
+ * x: [T, H, K] with free token and head strides (q_nope is a slice of q); w: [H, K, N] contiguous;
+ * y: [T, H, N] with free token and head strides; strides in elements.  fp32 accumulation, one rounding to
+ * dtype at the end.  dtype: XLLM_MI355_BF16.  K must be a multiple of 128, N of 64; pointers and strides
+ * multiples of 16 bytes.
+ */
+int xllm_mi355_mla_absorbed_bmm(const void* x, const void* w, void* y,
+                                int64_t n_tokens, int64_t n_heads, int64_t k, int64_t n,
+                                int64_t x_token_stride, int64_t x_head_stride,
+                                int64_t y_token_stride, int64_t y_head_stride,
+                                int dtype, void* stream);
+
+/*
  * Short query chunks through the decode kernels: chunked prefill and speculative-decoding
  * verification with a few query tokens per sequence.  Replaces the decode branch of
  * FlashAttentionImpl::paged_forward (xllm/core/layers/dcu/flash_attention.cpp:447-545: packed q

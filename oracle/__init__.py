@@ -336,3 +336,11 @@ def gather_paged_rows(cache, block_table, cu_seq_lens, total_rows, fill=0):
     c_lib().oracle_gather_paged_rows(_ptr(cache), _ptr(block_table), block_table.stride(0), _ptr(cu_seq_lens),
                                      _ptr(out), block_table.shape[0], bs, P, D * cache.element_size())
     return out
+
+
+def absorbed_bmm(x, w):
+    """x [T, H, K], w [H, K, N] -> [T, H, N] the way the reference writes it
+    (layers/dcu/deepseek_v2_attention.cpp:428-430, 231-238): bmm over the head-major views, here in fp32 with
+    one rounding to the input dtype at the end.  Also returns the unrounded fp32 result."""
+    exact = torch.bmm(x.float().transpose(0, 1), w.float()).transpose(0, 1).contiguous()
+    return exact.to(x.dtype), exact

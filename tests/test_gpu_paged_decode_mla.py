@@ -245,3 +245,57 @@ def test_step_captured_in_a_graph_follows_new_metadata(device):
         lay = inp.layout
         ref = oracle.aten_paged_decode(inp.q, kc, None, lay.block_table, lay.seq_lens, cfg.scale, dv=512)
         assert_close_to_reference(replayed.view(cfg.batch, cfg.n_q_heads, 512), ref, f"mla graph replay {rep}")
+
+
+def _bmm_case(T, H, K, N, seed, wide=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, K + wide, generator=g).bfloat16()
+    w = (torch.randn(H, K, N, generator=g) / math.sqrt(K)).bfloat16()
+    return x[..., :K], w
+
+
+@pytest.mark.parametrize("T,H,K,N,wide", [
+    (64, 128, 128, 512, 64),   # q_nope [B, H, 128] (a slice of q [B, H, 192]) with w_kc_ of DeepSeek-V3
+    (64, 128, 512, 128, 0),    # the decode output with w_vc_
+    (1, 16, 128, 512, 64),     # one token, a tensor-parallel shard of the heads
+    (67, 5, 256, 192, 0),      # token count that fills neither a wavefront nor a workgroup
+    (100, 4, 128, 128, 0),     # two token blocks per wavefront, the second one ragged
+    (200, 3, 128, 64, 8),      # four token blocks per wavefront
+    (700, 2, 256, 64, 0),      # several workgroups along the tokens
+])
+def test_absorbed_products_either_side_of_the_decode(device, T, H, K, N, wide):
+    # bmm(x.transpose(0, 1), w).transpose(0, 1) of layers/dcu/deepseek_v2_attention.cpp:428-430 and 231-238.
+    # Tolerance: fp32 accumulation and one rounding to bf16: half a bf16 unit in the last place of the exact
+    # value (2^-8 relative at most) plus 1e-4 for the order of the fp32 sums.
+    x, w = _bmm_case(T, H, K, N, seed=T + K)
+    ref, exact = oracle.absorbed_bmm(x, w)
+    xd = x.to(device) if wide == 0 else torch.cat([x, torch.zeros(T, H, wide, dtype=x.dtype)], dim=-1).to(device)[..., :K]
+    got = ops.absorbed_bmm(xd, w.to(device)).cpu()
+    assert got.shape == (T, H, N) and got.dtype == torch.bfloat16
+    err = (got.float() - exact).abs()
+    bound = exact.abs() * 2.0 ** -8 + 1e-4
+    assert (err <= bound).all(), f"max excess {(err - bound).max().item():.3e}"
+    assert (got != ref).float().mean().item() < 0.01  # the two roundings agree except at ties of the sum order
+    # into a slice of a wider output, as a caller that concatenates would
+    out = torch.full((T, H, N + 8), 7.0, dtype=torch.bfloat16, device=device)
+    ops.absorbed_bmm(xd, w.to(device), out=out[..., :N])
+    assert torch.equal(out[..., :N].cpu(), got) and (out[..., N:] == 7.0).all()
+
+
+def test_absorbed_product_selects_columns_bit_exactly_and_rejects_what_it_cannot_do(device):
+    g = torch.Generator().manual_seed(3)
+    T, H, K, N = 33, 6, 128, 64
+    x = torch.randn(T, H, K, generator=g).bfloat16()
+    perm = torch.stack([torch.randperm(K, generator=g)[:N] for _ in range(H)])
+    sel = torch.zeros(H, K, N)
+    for h in range(H):
+        sel[h, perm[h], torch.arange(N)] = 1.0
+    got = ops.absorbed_bmm(x.to(device), sel.bfloat16().to(device)).cpu()
+    assert torch.equal(got, torch.stack([x[:, h, perm[h]] for h in range(H)], dim=1))
+    assert ops.absorbed_bmm(x[:0].to(device), sel.bfloat16().to(device)).shape == (0, H, N)
+    with pytest.raises(ValueError):
+        ops.absorbed_bmm(x.to(device), sel[:, :64].bfloat16().to(device))        # K of x and w differ
+    with pytest.raises(RuntimeError):
+        ops.absorbed_bmm(x[..., :96].to(device), sel[:, :96].bfloat16().contiguous().to(device))  # K not a multiple of 128
+    with pytest.raises(RuntimeError):
+        ops.absorbed_bmm(x.half().to(device), sel.half().to(device))             # bf16 only

@@ -159,3 +159,25 @@ def test_norm_rope_and_metadata_update_through_the_host_side(device, xops):
     assert ret.data_ptr() == dd["tokens"].data_ptr()
     for k in want:
         assert torch.equal(dd[k].cpu(), want[k]), k
+
+
+def test_absorbed_products_through_the_host_side(device, xops):
+    # the two bmm calls of the absorbed MLA attention (layers/dcu/deepseek_v2_attention.cpp:428-430, 231-238)
+    # written the reference's way against the op that stands for them: same values as the direct C-ABI call, and
+    # the decode kernel between them takes the result as it comes
+    g = torch.Generator().manual_seed(21)
+    T, H = 5, 16
+    q = torch.randn(T, H, 192, generator=g).bfloat16().to(device)
+    w_kc = (torch.randn(H, 128, 512, generator=g) / math.sqrt(128)).bfloat16().to(device)
+    w_vc = (torch.randn(H, 512, 128, generator=g) / math.sqrt(512)).bfloat16().to(device)
+    q_nope = q[..., :128]
+    got = xops.mla_absorbed_bmm(q_nope, w_kc)
+    assert got.is_contiguous() and got.shape == (T, H, 512)
+    assert torch.equal(got, ops.absorbed_bmm(q_nope, w_kc))
+    _, exact = oracle.absorbed_bmm(q_nope.cpu(), w_kc.cpu())
+    assert ((got.cpu().float() - exact).abs() <= exact.abs() * 2.0 ** -8 + 1e-4).all()
+    back = xops.mla_absorbed_bmm(got, w_vc)
+    _, exact = oracle.absorbed_bmm(got.cpu(), w_vc.cpu())
+    assert ((back.cpu().float() - exact).abs() <= exact.abs() * 2.0 ** -8 + 1e-4).all()
+    with pytest.raises(RuntimeError):
+        xops.mla_absorbed_bmm(q_nope, w_vc)

@@ -272,3 +272,36 @@ def test_fused_qk_norm_rope_oracle_known_rotations_and_the_reference_tests_formu
     got = oracle.fused_qk_norm_rope(x, 2, 1, 0, D, 1e-6, ones, ones, cs, False, torch.tensor([0, 3, 6, 2, 2]))
     ms = (got.float().view(5, 3, D) ** 2).mean(-1)
     assert torch.allclose(ms, torch.ones_like(ms), atol=1e-2)
+
+
+def test_absorbed_bmm_oracle_against_loops_and_selections():
+    # The per-head products of the absorbed MLA attention (layers/dcu/deepseek_v2_attention.cpp:428-430, 231-238).
+    # Pins: explicit loops on a small case (a transposed operand or a swapped head/token index fails them),
+    # one-hot weights that select and permute columns (exact in bf16), and the reference's own expression on
+    # head-major views.
+    g = torch.Generator().manual_seed(5)
+    T, H, K, N = 3, 4, 6, 5
+    x = torch.randn(T, H, K, generator=g).bfloat16()
+    w = torch.randn(H, K, N, generator=g).bfloat16()
+    y, exact = oracle.absorbed_bmm(x, w)
+    loops = torch.zeros(T, H, N, dtype=torch.float64)
+    for t in range(T):
+        for h in range(H):
+            for n in range(N):
+                loops[t, h, n] = sum(float(x[t, h, k]) * float(w[h, k, n]) for k in range(K))
+    assert torch.allclose(exact.double(), loops, rtol=1e-6, atol=1e-6)
+    assert torch.equal(y, exact.bfloat16())
+    assert y.shape == (T, H, N) and y.dtype == torch.bfloat16
+    # head h picks column perm[h][n] of x: the result is a gather, bit for bit
+    perm = torch.stack([torch.randperm(K, generator=g)[:N] for _ in range(H)])
+    sel = torch.zeros(H, K, N)
+    for h in range(H):
+        sel[h, perm[h], torch.arange(N)] = 1.0
+    y_sel, _ = oracle.absorbed_bmm(x, sel.bfloat16())
+    want = torch.stack([x[:, h, perm[h]] for h in range(H)], dim=1)
+    assert torch.equal(y_sel, want)
+    # the reference's expression, on a slice of a wider tensor as q_nope is
+    q = torch.randn(T, H, K + 2, generator=g).bfloat16()
+    y_slice, _ = oracle.absorbed_bmm(q[..., :K], w)
+    ref = torch.bmm(q[..., :K].float().transpose(0, 1), w.float()).transpose(0, 1)
+    assert torch.equal(y_slice, ref.bfloat16())

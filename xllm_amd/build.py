@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libxllm_mi355.so")
-SOURCES = ["reshape_and_cache.hip", "rope_and_cache.hip", "paged_decode_gqa.hip", "paged_decode_mla.hip",
+SOURCES = ["reshape_and_cache.hip", "rope_and_cache.hip", "paged_decode_gqa.hip", "paged_decode_mla.hip", "absorbed_bmm.hip",
            "merge_and_tables.hip", "profile.hip", "hbm_probe.hip", "c_abi.hip"]
 HEADERS = ["common.cuh", "launch.h", os.path.join("..", "..", "include", "xllm_mi355.h")]
 # Packed-fp32 VALU forms stay off: every float op is a plain single-lane instruction.

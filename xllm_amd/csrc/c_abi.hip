@@ -92,6 +92,13 @@ int xllm_mi355_gather_paged_rows(const void* cache, const int32_t* block_table, 
                            num_blocks, row_bytes, static_cast<hipStream_t>(stream));
 }
 
+int xllm_mi355_mla_absorbed_bmm(const void* x, const void* w, void* y, int64_t n_tokens, int64_t n_heads,
+                                int64_t k, int64_t n, int64_t x_token_stride, int64_t x_head_stride,
+                                int64_t y_token_stride, int64_t y_head_stride, int dtype, void* stream) {
+  return absorbed_bmm(x, w, y, n_tokens, n_heads, k, n, x_token_stride, x_head_stride, y_token_stride,
+                      y_head_stride, dtype, static_cast<hipStream_t>(stream));
+}
+
 size_t xllm_mi355_paged_decode_varlen_workspace_bytes(int64_t n_tokens, int64_t n_q_heads, int64_t head_dim) {
   if (n_tokens <= 0 || n_q_heads <= 0 || head_dim <= 0) return 0;
   return varlen_extra_bytes(n_tokens) + gqa_workspace_bytes(n_tokens, n_q_heads, head_dim);

@@ -81,6 +81,11 @@ int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t tab
                       const int32_t* cu_seq_lens, void* out, int64_t batch, int64_t total_rows,
                       int64_t block_size, int64_t num_blocks, int64_t row_bytes, hipStream_t stream);
 
+// y[t, h, :] = x[t, h, :] . w[h, :, :]: the absorbed MLA products (strides in elements)
+int absorbed_bmm(const void* x, const void* w, void* y, int64_t n_tokens, int64_t n_heads, int64_t k, int64_t n,
+                 int64_t x_token_stride, int64_t x_head_stride, int64_t y_token_stride, int64_t y_head_stride,
+                 int dtype, hipStream_t stream);
+
 int rope_and_cache(void* qkv, const void* q_weight, const void* k_weight, const void* cos_sin_cache,
                    const int64_t* position_ids, void* k_cache, void* v_cache, const int32_t* slot_mapping,
                    const float* k_scale, const float* v_scale, int64_t n_tokens, int64_t token_stride,

@@ -180,6 +180,24 @@ void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torc
   check_rc(rc, "xllm_mi355_paged_decode_gqa_varlen");
 }
 
+torch::Tensor absorbed_bmm(const torch::Tensor& x, const torch::Tensor& w) {
+  // the conditions torch::bmm puts on its operands, on the head-major views of
+  // xllm/core/layers/dcu/deepseek_v2_attention.cpp:428-430, 231-238
+  TORCH_CHECK(x.defined() && w.defined(), "absorbed_bmm requires x and w");
+  TORCH_CHECK(x.is_cuda() && w.is_cuda(), "tensors must be on the device");
+  TORCH_CHECK(x.dim() == 3 && w.dim() == 3, "x must be [tokens, heads, k] and w [heads, k, n]");
+  TORCH_CHECK(x.size(1) == w.size(0) && x.size(2) == w.size(1), "x [tokens, heads, k] does not match w [heads, k, n]");
+  TORCH_CHECK(x.scalar_type() == w.scalar_type(), "x and w must have the same dtype");
+  const torch::Tensor xs = x.stride(2) == 1 ? x : x.contiguous();
+  const torch::Tensor ws = w.contiguous();
+  torch::Tensor out = torch::empty({x.size(0), x.size(1), w.size(2)}, x.options());
+  const int rc = xllm_mi355_mla_absorbed_bmm(xs.data_ptr(), ws.data_ptr(), out.data_ptr(), xs.size(0), xs.size(1),
+                                             xs.size(2), ws.size(2), xs.stride(0), xs.stride(1), out.stride(0),
+                                             out.stride(1), dtype_code(xs), current_stream(xs));
+  check_rc(rc, "xllm_mi355_mla_absorbed_bmm");
+  return out;
+}
+
 torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch::Tensor& block_table,
                                       const torch::Tensor& kv_cu_seq_lens, int64_t total_kv_len,
                                       int64_t max_seq_len) {
@@ -421,6 +439,8 @@ torch::Tensor op_gather_mla_latent_cache(torch::Tensor k_cache, torch::Tensor bl
   return xllm::kernel::mi355::gather_mla_latent_cache(k_cache, block_table, kv_cu_seq_lens, total_kv_len, max_seq_len);
 }
 
+torch::Tensor op_absorbed_bmm(torch::Tensor x, torch::Tensor w) { return xllm::kernel::mi355::absorbed_bmm(x, w); }
+
 // (the reference's op returns the mutated qkv, xllm/core/kernels/cuda/cuda_ops_library.cpp:121-149, 280-284)
 torch::Tensor op_fused_qk_norm_rope(torch::Tensor qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
                            int64_t head_dim, double eps, torch::Tensor q_weight, torch::Tensor k_weight,
@@ -509,6 +529,7 @@ TORCH_LIBRARY(xllm_ops, m) {
         "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len, int max_query_len) -> Tensor");
   m.def("gather_mla_latent_cache(Tensor k_cache, Tensor block_table, Tensor kv_cu_seq_lens, int total_kv_len, "
         "int max_seq_len) -> Tensor");
+  m.def("mla_absorbed_bmm(Tensor x, Tensor w) -> Tensor");
   m.def("update_decode_graph_metadata(Tensor tokens, Tensor positions, Tensor slot_mapping, Tensor kv_seq_lens, "
         "Tensor paged_kv_indptr, Tensor paged_kv_indices, Tensor paged_kv_last_page_len, Tensor(a!) dst_tokens, "
         "Tensor(b!) dst_positions, Tensor(c!) dst_slot_mapping, Tensor(d!) dst_kv_seq_lens, "
@@ -529,6 +550,7 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("merge_dcp_attention_shards", &op_merge);
   m.impl("paged_forward", &op_paged_forward);
   m.impl("gather_mla_latent_cache", &op_gather_mla_latent_cache);
+  m.impl("mla_absorbed_bmm", &op_absorbed_bmm);
   m.impl("update_decode_graph_metadata", &op_update_decode_graph_metadata);
   m.impl("fused_qk_norm_rope", &op_fused_qk_norm_rope);
   m.impl("fused_qk_norm_rope_and_cache", &op_fused_qk_norm_rope_and_cache);

@@ -69,6 +69,11 @@ torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch:
                                       const torch::Tensor& kv_cu_seq_lens, int64_t total_kv_len,
                                       int64_t max_seq_len);
 
+// The per-head products of the absorbed MLA attention: x [T, H, K], w [H, K, N] -> [T, H, N] contiguous.
+// Stands for torch::bmm(x.transpose(0, 1), w).transpose(0, 1) at xllm/core/layers/dcu/deepseek_v2_attention.cpp:428-430
+// (q_nope with w_kc_) and :231-238 (the decode output with w_vc_).  x may be a slice of a wider tensor.
+torch::Tensor absorbed_bmm(const torch::Tensor& x, const torch::Tensor& w);
+
 // xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/cuda_ops_api.h:235-249), same arguments.
 void fused_qk_norm_rope(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, int64_t num_heads_v,
                         int64_t head_dim, double eps, const torch::Tensor& q_weight, const torch::Tensor& k_weight,

@@ -14,6 +14,7 @@ Reference interface mirrored here (paths relative to the xLLM source tree):
   LlmDecodeMetadataUpdateParams, update_llm_decode_metadata
                                                   xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56
   gather_mla_latent_cache                         xllm/core/kernels/dcu/dcu_ops_api.h:74
+  absorbed MLA products (bmm with w_kc_ / w_vc_)  xllm/core/layers/dcu/deepseek_v2_attention.cpp:231-238,428-430
   FlashAttentionImpl::paged_forward (q chunks)    xllm/core/layers/dcu/flash_attention.cpp:447-545
 
 Errors: the reference CHECK-aborts; here every violated precondition raises.
@@ -472,4 +473,29 @@ def gather_mla_latent_cache(k_cache, block_table, kv_cu_seq_lens, total_kv_len, 
         k_cache.data_ptr(), block_table.data_ptr(), block_table.stride(0), kv_cu_seq_lens.data_ptr(),
         out.data_ptr(), B, total_kv_len, bs, P, D * k_cache.element_size(), _stream(dev))
     capi.check(rc, "xllm_mi355_gather_paged_rows")
+    return out
+
+
+def absorbed_bmm(x, w, out=None):
+    """The per-head product either side of the MLA decode kernel: x [T, H, K], w [H, K, N] -> [T, H, N], i.e.
+    torch.bmm(x.transpose(0, 1), w).transpose(0, 1) of layers/dcu/deepseek_v2_attention.cpp:428-430 (q_nope with
+    w_kc_) and :231-238 (the decode output with w_vc_).  x may be a slice of a wider tensor (unit stride in the
+    last dim); w contiguous.  fp32 accumulation, one rounding to bf16."""
+    dev = _require_cuda(x, w)
+    if x.dim() != 3 or w.dim() != 3 or x.shape[1] != w.shape[0] or x.shape[2] != w.shape[1]:
+        raise ValueError(f"shapes do not match: x {tuple(x.shape)} against w {tuple(w.shape)}")
+    if x.dtype != w.dtype:
+        raise TypeError("x and w must have the same dtype")
+    if x.stride(2) != 1 or not w.is_contiguous():
+        raise ValueError("x needs unit stride in its last dim and w must be contiguous")
+    T, H, K = x.shape
+    N = w.shape[2]
+    if out is None:
+        out = torch.empty(T, H, N, dtype=x.dtype, device=dev)
+    elif out.shape != (T, H, N) or out.dtype != x.dtype or out.stride(2) != 1 or out.device != x.device:
+        raise ValueError("out must be [T, H, N] of x's dtype and device with unit stride in its last dim")
+    rc = capi.lib().xllm_mi355_mla_absorbed_bmm(
+        x.data_ptr(), w.data_ptr(), out.data_ptr(), T, H, K, N, x.stride(0), x.stride(1), out.stride(0),
+        out.stride(1), _dtype_code(x), _stream(dev))
+    capi.check(rc, "xllm_mi355_mla_absorbed_bmm")
     return out
