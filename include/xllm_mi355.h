@@ -270,6 +270,19 @@ int xllm_mi355_build_block_table(const int32_t* paged_kv_indptr,
                                  int64_t batch, int64_t block_size, void* stream);
 
 /*
+ * Block-table hygiene for kernels that expect -1 in unused columns.  Replaces mask_block_table_padding
+ * (xllm/core/layers/dcu/flash_attention.cpp:194-218; the reference pads its tables with the valid page id 0,
+ * framework/batch/batch_input_builder.cpp:1233-1275):
+ *     out[b, j] = block_table[b, j] for j < ceil(kv_seq_lens[b] / block_size), -1 elsewhere
+ * for j < width.  Columns are masked by position only, never by page id.  out may be block_table itself.
+ * The decode kernels of this library do not need it: they never read a column beyond a sequence's pages.
+ */
+int xllm_mi355_mask_block_table_padding(const int32_t* block_table, int64_t table_stride,
+                                        const int32_t* kv_seq_lens,
+                                        int32_t* out, int64_t out_stride,
+                                        int64_t batch, int64_t width, int64_t block_size, void* stream);
+
+/*
  * Per-head RMS norm + rotary embedding of the q and k heads of a fused qkv buffer, in place; with a cache,
  * also the cache write of the new k and v rows in the same launch.  Replaces
  * xllm::kernel::cuda::fused_qk_norm_rope (xllm/core/kernels/cuda/fused_qknorm_rope.cu:79-300, 388-470;

@@ -31,12 +31,10 @@ def dtype_code(t):
 
 
 def c_lib():
-    """The plain-C oracle, built on first use if missing."""
+    """The plain-C oracle, built on first use if missing or older than its source."""
     global _c
     if _c is None:
-        path = _build.C_LIB
-        if not os.path.exists(path):
-            _build.build_c()
+        path = _build.build_c(force=False)
         lib = ctypes.CDLL(path)
         lib.oracle_bf16_to_f32.restype = _f32
         lib.oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
@@ -64,6 +62,8 @@ def c_lib():
         lib.oracle_lse_merge.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64]
         lib.oracle_build_block_table.restype = None
         lib.oracle_build_block_table.argtypes = [_p, _p, _p, _p, _i64, _p, _i64, _i64]
+        lib.oracle_mask_block_table_padding.restype = None
+        lib.oracle_mask_block_table_padding.argtypes = [_p, _i64, _p, _p, _i64, _i64, _i64]
         lib.oracle_gather_paged_rows.restype = None
         lib.oracle_gather_paged_rows.argtypes = [_p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64]
         _c = lib
@@ -71,12 +71,10 @@ def c_lib():
 
 
 def aten_lib():
-    """The ATen-op-order oracle, built on first use if missing."""
+    """The ATen-op-order oracle, built on first use if missing or older than its source."""
     global _aten
     if _aten is None:
-        path = _build.ATEN_LIB
-        if not os.path.exists(path):
-            _build.build_aten()
+        path = _build.build_aten(force=False)
         lib = ctypes.CDLL(path)
         lib.aten_oracle_num_threads.restype = _i32
         lib.aten_oracle_set_num_threads.argtypes = [_i32]
@@ -264,6 +262,15 @@ def build_block_table(indptr, indices, last_page_len, table_stride, block_size):
     c_lib().oracle_build_block_table(_ptr(indptr), _ptr(indices), _ptr(last_page_len), _ptr(table),
                                      table_stride, _ptr(seq_lens), B, block_size)
     return table, seq_lens
+
+
+def mask_block_table_padding(block_table, kv_seq_lens, block_size):
+    B, W = block_table.shape
+    out = torch.empty(B, W, dtype=torch.int32)
+    assert block_table.device.type == "cpu" and block_table.dtype == torch.int32 and block_table.stride(1) == 1
+    c_lib().oracle_mask_block_table_padding(ctypes.c_void_p(block_table.data_ptr()), block_table.stride(0),
+                                            _ptr(kv_seq_lens), _ptr(out), B, W, block_size)
+    return out
 
 
 def fused_qk_norm_rope(qkv, n_q, n_k, n_v, head_dim, eps, q_weight, k_weight, cos_sin_cache, interleave,

@@ -347,6 +347,20 @@ void oracle_build_block_table(const int32_t* indptr, const int32_t* indices,
 }
 
 /*
+ * mask_block_table_padding (layers/dcu/flash_attention.cpp:194-218): page_counts = (len + bs - 1) / bs;
+ * columns j >= page_counts[b] become -1, the others keep their value.
+ */
+void oracle_mask_block_table_padding(const int32_t* block_table, int64_t table_stride,
+                                     const int32_t* kv_seq_lens, int32_t* out, int64_t batch,
+                                     int64_t width, int64_t block_size) {
+  for (int64_t b = 0; b < batch; ++b) {
+    const int64_t pages = ((int64_t)kv_seq_lens[b] + block_size - 1) / block_size;
+    for (int64_t j = 0; j < width; ++j)
+      out[b * width + j] = j >= pages ? -1 : block_table[b * table_stride + j];
+  }
+}
+
+/*
  * Rows of paged sequences -> packed buffer (kernels/dcu/gather_mla_latent_cache.hip:32-75): for every sequence b
  * and token t < cu[b+1] - cu[b], out row cu[b] + t = cache row block_table[b, t / bs] * bs + t % bs; rows with a
  * negative page id are skipped (the reference's `physical_block < 0` return), and so are ids beyond the cache.

@@ -3,7 +3,7 @@ import pytest
 import torch
 
 import oracle
-from xllm_amd import ops, workloads
+from xllm_amd import capi, ops, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -275,3 +275,24 @@ def test_fused_qk_norm_rope_and_its_cache_write(device):
             torch.cuda.synchronize()
             assert torch.equal(kc.view(torch.uint8), kc2.view(torch.uint8))
             assert torch.equal(vc.view(torch.uint8), vc2.view(torch.uint8))
+
+
+def test_block_table_padding_mask_is_bit_exact(device):
+    # mask_block_table_padding (layers/dcu/flash_attention.cpp:194-218): bit-exact against the oracle on ragged
+    # lengths (empty, one token, page boundaries, the full width), a wide table, a strided table view, and in place
+    g = torch.Generator().manual_seed(12)
+    for bs, W, B in ((16, 9, 8), (64, 300, 40), (128, 1, 3)):
+        lens = torch.randint(0, W * bs + 1, (B,), generator=g, dtype=torch.int32)
+        lens[:3] = torch.tensor([0, 1, W * bs][:3], dtype=torch.int32)
+        wide = torch.randint(0, 1000, (B, W + 5), generator=g, dtype=torch.int32)
+        table = wide[:, :W]
+        ref = oracle.mask_block_table_padding(table, lens, bs)
+        got = ops.mask_block_table_padding(wide.to(device)[:, :W], lens.to(device), bs)
+        assert torch.equal(got.cpu(), ref)
+        own = table.contiguous().to(device)
+        rc = capi.lib().xllm_mi355_mask_block_table_padding(own.data_ptr(), W, lens.to(device).data_ptr(), own.data_ptr(),
+                                                            W, B, W, bs, torch.cuda.current_stream(device).cuda_stream)
+        assert rc == 0
+        assert torch.equal(own.cpu(), ref)
+    with pytest.raises(ValueError):
+        ops.mask_block_table_padding(table.to(device), lens[:-1].to(device), bs)

@@ -181,3 +181,14 @@ def test_absorbed_products_through_the_host_side(device, xops):
     assert ((back.cpu().float() - exact).abs() <= exact.abs() * 2.0 ** -8 + 1e-4).all()
     with pytest.raises(RuntimeError):
         xops.mla_absorbed_bmm(q_nope, w_vc)
+
+
+def test_block_table_padding_mask_through_the_host_side(device, xops):
+    # mask_block_table_padding with the reference's arguments (layers/dcu/flash_attention.cpp:194-218); int64
+    # lengths as torch::diff leaves them are accepted
+    g = torch.Generator().manual_seed(2)
+    table = torch.randint(0, 99, (6, 12), generator=g, dtype=torch.int32)
+    lens = torch.tensor([0, 5, 16, 17, 12 * 16, 100], dtype=torch.int64)
+    got = xops.mask_block_table_padding(table.to(device), lens.to(device), 16)
+    assert got.dtype == torch.int32
+    assert torch.equal(got.cpu(), oracle.mask_block_table_padding(table, lens.int(), 16))

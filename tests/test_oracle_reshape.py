@@ -154,3 +154,19 @@ def test_decode_metadata_update_rules_equal_the_slice_copies_they_replace():
         if padded > batch:
             assert int(a["kv_seq_lens"][padded]) == int(src["kv_seq_lens"][batch])
             assert int(a["paged_kv_last_page_len"][padded - 1]) == 1 and int(a["new_cache_slots"][padded - 1]) == -1
+
+
+def test_block_table_padding_mask_against_the_reference_expression():
+    # mask_block_table_padding (layers/dcu/flash_attention.cpp:194-218) written with the reference's own tensor
+    # expression: columns at or beyond ceil(len / bs) become -1 whatever they hold (page id 0 is a valid page and
+    # survives inside a sequence), the others are kept; empty sequences lose every column.
+    g = torch.Generator().manual_seed(4)
+    for bs, W in ((16, 9), (64, 5), (128, 1)):
+        lens = torch.tensor([0, 1, bs - 1, bs, bs + 1, W * bs, W * bs - 1, 3 * bs // 2], dtype=torch.int32).clamp(max=W * bs)
+        table = torch.randint(0, 50, (lens.numel(), W + 3), generator=g, dtype=torch.int32)[:, :W]  # row stride > width
+        table[:, 0] = 0                                            # a valid page 0 in the first column
+        got = oracle.mask_block_table_padding(table, lens, bs)
+        pages = ((lens.long() + bs - 1) // bs).view(-1, 1)
+        want = table.clone().masked_fill_(torch.arange(W).view(1, -1) >= pages, -1)
+        assert torch.equal(got, want)
+        assert (got[1:, 0] == 0).all() and (got[0] == -1).all()

@@ -41,6 +41,7 @@ SIGNATURES = {
     "xllm_mi355_lse_merge": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "xllm_mi355_build_block_table": (_i32, [_p, _p, _p, _p, _i64, _p, _i64, _i64, _p]),
     "xllm_mi355_decode_metadata_update": (_i32, [_p] * 15 + [_i64] * 4 + [_p]),
+    "xllm_mi355_mask_block_table_padding": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i64, _p]),
     "xllm_mi355_mla_absorbed_bmm": (_i32, [_p] * 3 + [_i64] * 8 + [_i32, _p]),
     "xllm_mi355_rope_and_cache": (_i32, [_p] * 10 + [_i64] * 7 + [_f32, _i32, _i64, _i64, _i32, _i32, _i32, _p]),
     "xllm_mi355_profile_enable": (_i32, [_i32]),

@@ -92,6 +92,13 @@ int xllm_mi355_gather_paged_rows(const void* cache, const int32_t* block_table, 
                            num_blocks, row_bytes, static_cast<hipStream_t>(stream));
 }
 
+int xllm_mi355_mask_block_table_padding(const int32_t* block_table, int64_t table_stride, const int32_t* kv_seq_lens,
+                                        int32_t* out, int64_t out_stride, int64_t batch, int64_t width,
+                                        int64_t block_size, void* stream) {
+  return mask_block_table_padding(block_table, table_stride, kv_seq_lens, out, out_stride, batch, width, block_size,
+                                  static_cast<hipStream_t>(stream));
+}
+
 int xllm_mi355_mla_absorbed_bmm(const void* x, const void* w, void* y, int64_t n_tokens, int64_t n_heads,
                                 int64_t k, int64_t n, int64_t x_token_stride, int64_t x_head_stride,
                                 int64_t y_token_stride, int64_t y_head_stride, int dtype, void* stream) {

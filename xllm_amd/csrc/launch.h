@@ -77,6 +77,10 @@ int build_block_table(const int32_t* indptr, const int32_t* indices, const int32
                       int32_t* block_table, int64_t table_stride, int32_t* seq_lens, int64_t batch,
                       int64_t block_size, hipStream_t stream);
 
+int mask_block_table_padding(const int32_t* block_table, int64_t table_stride, const int32_t* kv_seq_lens,
+                             int32_t* out, int64_t out_stride, int64_t batch, int64_t width, int64_t block_size,
+                             hipStream_t stream);
+
 int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t table_stride,
                       const int32_t* cu_seq_lens, void* out, int64_t batch, int64_t total_rows,
                       int64_t block_size, int64_t num_blocks, int64_t row_bytes, hipStream_t stream);

@@ -70,6 +70,17 @@ __global__ __launch_bounds__(256) void build_block_table_kernel(const int32_t* i
     seq_lens[b] = n > 0 ? (n - 1) * block_size + last_page_len[b] : 0;
 }
 
+// out[b, j] = table[b, j] for the columns a sequence of kv_seq_lens[b] tokens uses, -1 beyond them
+// (never by page id: page 0 is a valid page).  In place when out == table.
+__global__ __launch_bounds__(256) void mask_block_table_padding_kernel(const int32_t* table, int64_t stride,
+                                                                       const int32_t* kv_seq_lens, int32_t* out,
+                                                                       int64_t out_stride, int width, int block_size) {
+  const int b = blockIdx.x;
+  const int64_t len = kv_seq_lens[b];
+  const int64_t pages = len > 0 ? (len + block_size - 1) / block_size : 0;
+  for (int j = threadIdx.x; j < width; j += 256) out[b * out_stride + j] = j < pages ? table[b * stride + j] : -1;
+}
+
 struct MetadataUpdate {
   const int32_t *tokens, *positions, *slots, *kv_cu, *indptr, *indices, *last_page_len;
   int32_t *d_tokens, *d_positions, *d_slots, *d_kv_cu, *d_kv_delta, *d_indptr, *d_indices, *d_last_page_len;
@@ -292,6 +303,19 @@ int lse_merge(const void* partial_out, const float* partial_lse, void* out, floa
       break;
     default: return XLLM_MI355_EDTYPE;
   }
+  return static_cast<int>(hipGetLastError());
+}
+
+int mask_block_table_padding(const int32_t* block_table, int64_t table_stride, const int32_t* kv_seq_lens,
+                             int32_t* out, int64_t out_stride, int64_t batch, int64_t width, int64_t block_size,
+                             hipStream_t stream) {
+  if (batch == 0 || width == 0) return XLLM_MI355_OK;
+  if (block_table == nullptr || kv_seq_lens == nullptr || out == nullptr) return XLLM_MI355_EINVAL;
+  if (batch < 0 || batch > 0x7fffffffLL || width < 0 || width > 0x7fffffffLL || table_stride < width ||
+      out_stride < width || block_size <= 0 || block_size > 0x7fffffffLL)
+    return XLLM_MI355_EINVAL;
+  mask_block_table_padding_kernel<<<dim3(static_cast<unsigned>(batch)), 256, 0, stream>>>(
+      block_table, table_stride, kv_seq_lens, out, out_stride, static_cast<int>(width), static_cast<int>(block_size));
   return static_cast<int>(hipGetLastError());
 }
 

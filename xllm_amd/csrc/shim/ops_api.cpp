@@ -180,6 +180,26 @@ void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torc
   check_rc(rc, "xllm_mi355_paged_decode_gqa_varlen");
 }
 
+torch::Tensor mask_block_table_padding(const torch::Tensor& block_table, const torch::Tensor& kv_seq_lens,
+                                       int64_t page_block_size) {
+  // the checks of xllm/core/layers/dcu/flash_attention.cpp:200-202
+  TORCH_CHECK(block_table.defined(), "block_table must be defined");
+  TORCH_CHECK(kv_seq_lens.defined(), "kv_seq_lens must be defined");
+  TORCH_CHECK(page_block_size > 0, "page_block_size must be positive");
+  TORCH_CHECK(block_table.is_cuda() && kv_seq_lens.is_cuda(), "tensors must be on the device");
+  TORCH_CHECK(block_table.dim() == 2 && kv_seq_lens.numel() == block_table.size(0),
+              "block_table must be [batch, max_blocks] and kv_seq_lens [batch]");
+  torch::Tensor table = block_table.scalar_type() == torch::kInt32 ? block_table : block_table.to(torch::kInt32);
+  if (table.stride(1) != 1) table = table.contiguous();
+  torch::Tensor lens = (kv_seq_lens.scalar_type() == torch::kInt32 ? kv_seq_lens : kv_seq_lens.to(torch::kInt32)).contiguous();
+  torch::Tensor out = torch::empty({table.size(0), table.size(1)}, table.options());
+  const int rc = xllm_mi355_mask_block_table_padding(table.data_ptr<int32_t>(), table.stride(0), lens.data_ptr<int32_t>(),
+                                                     out.data_ptr<int32_t>(), out.stride(0), table.size(0),
+                                                     table.size(1), page_block_size, current_stream(table));
+  check_rc(rc, "xllm_mi355_mask_block_table_padding");
+  return out;
+}
+
 torch::Tensor absorbed_bmm(const torch::Tensor& x, const torch::Tensor& w) {
   // the conditions torch::bmm puts on its operands, on the head-major views of
   // xllm/core/layers/dcu/deepseek_v2_attention.cpp:428-430, 231-238
@@ -439,6 +459,9 @@ torch::Tensor op_gather_mla_latent_cache(torch::Tensor k_cache, torch::Tensor bl
   return xllm::kernel::mi355::gather_mla_latent_cache(k_cache, block_table, kv_cu_seq_lens, total_kv_len, max_seq_len);
 }
 
+torch::Tensor op_mask_block_table_padding(torch::Tensor block_table, torch::Tensor kv_seq_lens, int64_t page_block_size) {
+  return xllm::kernel::mi355::mask_block_table_padding(block_table, kv_seq_lens, page_block_size);
+}
 torch::Tensor op_absorbed_bmm(torch::Tensor x, torch::Tensor w) { return xllm::kernel::mi355::absorbed_bmm(x, w); }
 
 // (the reference's op returns the mutated qkv, xllm/core/kernels/cuda/cuda_ops_library.cpp:121-149, 280-284)
@@ -530,6 +553,7 @@ TORCH_LIBRARY(xllm_ops, m) {
   m.def("gather_mla_latent_cache(Tensor k_cache, Tensor block_table, Tensor kv_cu_seq_lens, int total_kv_len, "
         "int max_seq_len) -> Tensor");
   m.def("mla_absorbed_bmm(Tensor x, Tensor w) -> Tensor");
+  m.def("mask_block_table_padding(Tensor block_table, Tensor kv_seq_lens, int page_block_size) -> Tensor");
   m.def("update_decode_graph_metadata(Tensor tokens, Tensor positions, Tensor slot_mapping, Tensor kv_seq_lens, "
         "Tensor paged_kv_indptr, Tensor paged_kv_indices, Tensor paged_kv_last_page_len, Tensor(a!) dst_tokens, "
         "Tensor(b!) dst_positions, Tensor(c!) dst_slot_mapping, Tensor(d!) dst_kv_seq_lens, "
@@ -551,6 +575,7 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("paged_forward", &op_paged_forward);
   m.impl("gather_mla_latent_cache", &op_gather_mla_latent_cache);
   m.impl("mla_absorbed_bmm", &op_absorbed_bmm);
+  m.impl("mask_block_table_padding", &op_mask_block_table_padding);
   m.impl("update_decode_graph_metadata", &op_update_decode_graph_metadata);
   m.impl("fused_qk_norm_rope", &op_fused_qk_norm_rope);
   m.impl("fused_qk_norm_rope_and_cache", &op_fused_qk_norm_rope_and_cache);

@@ -69,6 +69,11 @@ torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch:
                                       const torch::Tensor& kv_cu_seq_lens, int64_t total_kv_len,
                                       int64_t max_seq_len);
 
+// mask_block_table_padding (xllm/core/layers/dcu/flash_attention.cpp:194-218), same arguments: a copy of
+// block_table with -1 in the columns beyond each sequence's pages.
+torch::Tensor mask_block_table_padding(const torch::Tensor& block_table, const torch::Tensor& kv_seq_lens,
+                                       int64_t page_block_size);
+
 // The per-head products of the absorbed MLA attention: x [T, H, K], w [H, K, N] -> [T, H, N] contiguous.
 // Stands for torch::bmm(x.transpose(0, 1), w).transpose(0, 1) at xllm/core/layers/dcu/deepseek_v2_attention.cpp:428-430
 // (q_nope with w_kc_) and :231-238 (the decode output with w_vc_).  x may be a slice of a wider tensor.

@@ -10,6 +10,7 @@ Reference interface mirrored here (paths relative to the xLLM source tree):
   flash_mla::DenseDecodeParams / dense_decode     xllm/core/kernels/dcu/flash_mla_adapter.h:40-53
   merge_dcp_attention_shards                      xllm/core/layers/mlu/dcp_attention_merge.h:28-34
   build_block_table_from_paged_kv                 xllm/core/kernels/dcu/build_block_table_from_paged_kv.hip
+  mask_block_table_padding                        xllm/core/layers/dcu/flash_attention.cpp:194-218
   fused_qk_norm_rope                              xllm/core/kernels/cuda/fused_qknorm_rope.cu:388-470
   LlmDecodeMetadataUpdateParams, update_llm_decode_metadata
                                                   xllm/core/kernels/cuda/llm_decode_metadata_update.h:33-56
@@ -375,6 +376,25 @@ def build_block_table_from_paged_kv(paged_kv_indptr, paged_kv_indices, paged_kv_
         table.data_ptr(), table_width, seq_lens.data_ptr(), B, block_size, _stream(dev))
     capi.check(rc, "xllm_mi355_build_block_table")
     return table, seq_lens
+
+
+def mask_block_table_padding(block_table, kv_seq_lens, page_block_size):
+    """layers/dcu/flash_attention.cpp:194-218: a copy of block_table [B, W] with -1 in the columns beyond each
+    sequence's ceil(kv_seq_lens / page_block_size) pages (by position, never by page id).  int32 result."""
+    dev = _require_cuda(block_table, kv_seq_lens)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise ValueError("block_table must be int32 [B, W] with unit column stride")
+    B, W = block_table.shape
+    if kv_seq_lens.dtype != torch.int32 or kv_seq_lens.numel() != B or not kv_seq_lens.is_contiguous():
+        raise ValueError("kv_seq_lens must be contiguous int32 [B]")
+    if page_block_size <= 0:
+        raise ValueError("page_block_size must be positive")
+    out = torch.empty(B, W, dtype=torch.int32, device=dev)
+    rc = capi.lib().xllm_mi355_mask_block_table_padding(
+        block_table.data_ptr(), block_table.stride(0), kv_seq_lens.data_ptr(), out.data_ptr(), out.stride(0),
+        B, W, page_block_size, _stream(dev))
+    capi.check(rc, "xllm_mi355_mask_block_table_padding")
+    return out
 
 
 def fused_qk_norm_rope(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps, q_weight, k_weight,
