@@ -237,7 +237,11 @@ def test_fused_qk_norm_rope_and_its_cache_write(device):
     g = torch.Generator().manual_seed(11)
     cases = ((17, 8, 4, 4, 128, 128, torch.float16, torch.float32, False), (11, 6, 2, 2, 64, 64, torch.bfloat16, torch.float32, True),
              (64, 32, 8, 8, 128, 128, torch.bfloat16, torch.bfloat16, False), (5, 4, 2, 2, 256, 128, torch.bfloat16, torch.float16, False),
-             (9, 4, 4, 4, 128, 64, torch.float16, torch.float32, True), (1, 16, 2, 2, 64, 32, torch.bfloat16, torch.float32, False))
+             (9, 4, 4, 4, 128, 64, torch.float16, torch.float32, True), (1, 16, 2, 2, 64, 32, torch.bfloat16, torch.float32, False),
+             # prefill sizes, where a lane group takes four (token, head) units: unit counts that are not multiples of
+             # four, head counts that let a group straddle two tokens
+             (4999, 11, 3, 3, 128, 128, torch.bfloat16, torch.float32, False),
+             (4501, 13, 2, 2, 64, 64, torch.float16, torch.float32, True))
     for T, n_q, n_k, n_v, D, rd, dt, cdt, inter in cases:
         qkv = (torch.randn(T, (n_q + n_k + n_v) * D, generator=g) * 0.3).to(dt)
         qw, kw = (1 + 0.2 * torch.randn(D, generator=g)).to(dt), (1 + 0.2 * torch.randn(D, generator=g)).to(dt)
@@ -253,7 +257,8 @@ def test_fused_qk_norm_rope_and_its_cache_write(device):
         assert (got.cpu().float() - want.float()).abs().mean() < 2e-4
         assert torch.equal(got.cpu()[:, (n_q + n_k) * D :], qkv[:, (n_q + n_k) * D :])
         # the same launch with the cache write
-        bs, P = 16, 12
+        bs = 16
+        P = max(12, T // bs + 2)
         slots = torch.randperm(P * bs, generator=g)[:T].to(torch.int32)
         slots[0] = -1
         for cache_dt in (dt, torch.float8_e4m3fn):

@@ -47,127 +47,193 @@ struct RopeArgs {
   int norm;             // 0: no RMS norm (weights absent)
 };
 
-// cos / sin caches come in fp32 or in a 16-bit type
-template <int CT>
-__device__ __forceinline__ float cache_at(const char* p, int64_t i) {
-  if constexpr (CT == XLLM_MI355_FP32) return reinterpret_cast<const float*>(p)[i];
-  else if constexpr (CT == XLLM_MI355_BF16) return BF16::to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
-  else return FP16::to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+// cos / sin caches come in fp32 or in a 16-bit type.  N consecutive entries from index i on, with one
+// vector load (two for 8 fp32 entries): i is a multiple of N and the rows of the cache start at multiples
+// of 2 N entries, so the load is aligned whenever the cache itself is 16-byte aligned.  Entry by entry
+// these loads were most of the kernel's memory instructions.
+template <int CT, int N>
+__device__ __forceinline__ void cache_vec(const char* p, int64_t i, float (&out)[N]) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8, "entries per lane");
+  if constexpr (CT == XLLM_MI355_FP32) {
+    const float* f = reinterpret_cast<const float*>(p) + i;
+    if constexpr (N == 1) {
+      out[0] = f[0];
+    } else if constexpr (N == 2) {
+      const f32x2 v = *reinterpret_cast<const f32x2*>(f);
+      out[0] = v[0];
+      out[1] = v[1];
+    } else {
+#pragma unroll
+      for (int k = 0; k < N / 4; ++k) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(f + 4 * k);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) out[4 * k + j] = v[j];
+      }
+    }
+  } else {
+    uint16_t h[N];
+    const uint16_t* q = reinterpret_cast<const uint16_t*>(p) + i;
+    if constexpr (N == 1) h[0] = q[0];
+    else if constexpr (N == 2) *reinterpret_cast<u32*>(h) = *reinterpret_cast<const u32*>(q);
+    else if constexpr (N == 4) *reinterpret_cast<u32x2*>(h) = *reinterpret_cast<const u32x2*>(q);
+    else *reinterpret_cast<u32x4*>(h) = *reinterpret_cast<const u32x4*>(q);
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = CT == XLLM_MI355_BF16 ? BF16::to_f32(h[j]) : FP16::to_f32(h[j]);
+  }
 }
 
 __device__ __forceinline__ float lane_xor(float x, int mask, int lane) {
   return as_f32(static_cast<u32>(__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, static_cast<int>(as_u32(x)))));
 }
 
-template <typename QT, int D, int CT, bool INTERLEAVE, bool FP8>
+// U = (token, head) units per 32-lane group.  With one unit a lane has 4 to 16 bytes in flight, which at
+// prefill sizes leaves the launch bound by memory latency; with four consecutive units (adjacent heads of a
+// token: adjacent rows) the loads of all four are issued before the first is used.
+template <typename QT, int D, int CT, bool INTERLEAVE, bool FP8, int U>
 __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeArgs a) {
   constexpr int E = D / 32;  // dims per lane
   const int lane = threadIdx.x & 63;
   const int sub = lane & 31;
-  const int64_t unit = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) >> 5;
-  const bool on = unit < a.n_units;  // (lanes past the end keep running: the exchanges below are wave wide)
-  const int64_t token = on ? unit / a.heads_per_token : 0;
-  const int head = on ? static_cast<int>(unit - token * a.heads_per_token) : 0;
-  const bool is_q = head < a.n_q;
-  const bool is_v = head >= a.n_q + a.n_k;
-  char* row = a.qkv + token * a.token_stride_bytes + (static_cast<int64_t>(head) * D + sub * E) * 2;
-
-  uint16_t raw[E];
-  if constexpr (E == 2) *reinterpret_cast<u32*>(raw) = *reinterpret_cast<const u32*>(row);
-  else if constexpr (E == 4) *reinterpret_cast<u32x2*>(raw) = *reinterpret_cast<const u32x2*>(row);
-  else *reinterpret_cast<u32x4*>(raw) = *reinterpret_cast<const u32x4*>(row);
-
-  float x[E];
-  float ss = 0.0f;
-#pragma unroll
-  for (int i = 0; i < E; ++i) {
-    x[i] = QT::to_f32(raw[i]);
-    ss += x[i] * x[i];
-  }
-  ss = group_sum<32>(ss);
-  if (!is_v && a.norm != 0) {
-    const float r = __builtin_amdgcn_rsqf(ss / static_cast<float>(D) + a.eps);
-    const uint16_t* w = reinterpret_cast<const uint16_t*>(is_q ? a.q_weight : a.k_weight) + sub * E;
-#pragma unroll
-    for (int i = 0; i < E; ++i) x[i] *= r * QT::to_f32(w[i]);
-  }
-
-  // rotary embedding of the leading rotary_dim dims
-  const int64_t pos = on ? a.positions[token] : 0;
+  const int64_t unit0 = ((static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) >> 5) * U;
   const int half = a.rotary_dim >> 1;
-  const int64_t cs = pos * a.rotary_dim;
   const int rotary_lanes = a.rotary_dim / E;
-  if constexpr (INTERLEAVE) {
-    if (!is_v && sub < rotary_lanes) {
+  const bool rotated = sub < rotary_lanes;
+
+  bool on[U], is_q[U], is_v[U];  // (lanes past the end keep running: the exchanges below are wave wide)
+  int64_t token[U];
+  int head[U];
+  char* row[U];
+  uint16_t raw[U][E];
 #pragma unroll
-      for (int i = 0; i < E / 2; ++i) {
-        const int j = (sub * E) / 2 + i;
-        const float c = cache_at<CT>(a.cos_sin, cs + j), s = cache_at<CT>(a.cos_sin, cs + half + j);
-        const float e = x[2 * i], o = x[2 * i + 1];
-        x[2 * i] = e * c - o * s;
-        x[2 * i + 1] = e * s + o * c;
+  for (int u = 0; u < U; ++u) {
+    const int64_t unit = unit0 + u;
+    on[u] = unit < a.n_units;
+    token[u] = on[u] ? unit / a.heads_per_token : 0;
+    head[u] = on[u] ? static_cast<int>(unit - token[u] * a.heads_per_token) : 0;
+    is_q[u] = head[u] < a.n_q;
+    is_v[u] = head[u] >= a.n_q + a.n_k;
+    row[u] = a.qkv + token[u] * a.token_stride_bytes + (static_cast<int64_t>(head[u]) * D + sub * E) * 2;
+    if constexpr (E == 2) *reinterpret_cast<u32*>(raw[u]) = *reinterpret_cast<const u32*>(row[u]);
+    else if constexpr (E == 4) *reinterpret_cast<u32x2*>(raw[u]) = *reinterpret_cast<const u32x2*>(row[u]);
+    else *reinterpret_cast<u32x4*>(raw[u]) = *reinterpret_cast<const u32x4*>(row[u]);
+  }
+  int64_t cs[U];
+  int64_t slot[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    cs[u] = (on[u] ? a.positions[token[u]] : 0) * a.rotary_dim;
+    slot[u] = a.k_cache != nullptr && on[u] && !is_q[u] ? a.slots[token[u]] : -1;
+  }
+  // cos | sin of the lane's dims: c[u][i], sn[u][i] belong to pair i of the interleaved form, to dim i of the split form
+  constexpr int NC = INTERLEAVE ? E / 2 : E;
+  float c[U][NC], sn[U][NC];
+  // the lane's dims lie on one side of the split form (rotary_dim / 2 is a multiple of E)
+  const int j0 = INTERLEAVE ? (sub * E) / 2 : (sub * E < half ? sub * E : sub * E - half);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (rotated && !is_v[u]) {
+      cache_vec<CT, NC>(a.cos_sin, cs[u] + j0, c[u]);
+      cache_vec<CT, NC>(a.cos_sin, cs[u] + half + j0, sn[u]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < NC; ++i) {
+        c[u][i] = 1.0f;
+        sn[u][i] = 0.0f;
       }
     }
-  } else {
-    const int pair = half / E;  // lanes between a dim and its partner
-    float other[E];
+  }
+
 #pragma unroll
-    for (int i = 0; i < E; ++i) other[i] = lane_xor(x[i], pair, lane);
-    if (!is_v && sub < rotary_lanes) {
+  for (int u = 0; u < U; ++u) {
+    float x[E];
+    float ss = 0.0f;
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const int d = sub * E + i;
-        const int j = d < half ? d : d - half;
-        const float c = cache_at<CT>(a.cos_sin, cs + j), s = cache_at<CT>(a.cos_sin, cs + half + j);
-        x[i] = x[i] * c + (d < half ? -other[i] : other[i]) * s;
+    for (int i = 0; i < E; ++i) {
+      x[i] = QT::to_f32(raw[u][i]);
+      ss += x[i] * x[i];
+    }
+    ss = group_sum<32>(ss);
+    if (!is_v[u] && a.norm != 0) {
+      const float r = __builtin_amdgcn_rsqf(ss / static_cast<float>(D) + a.eps);
+      const uint16_t* w = reinterpret_cast<const uint16_t*>(is_q[u] ? a.q_weight : a.k_weight) + sub * E;
+#pragma unroll
+      for (int i = 0; i < E; ++i) x[i] *= r * QT::to_f32(w[i]);
+    }
+    // rotary embedding of the leading rotary_dim dims
+    if constexpr (INTERLEAVE) {
+      if (!is_v[u] && rotated) {
+#pragma unroll
+        for (int i = 0; i < E / 2; ++i) {
+          const float e = x[2 * i], o = x[2 * i + 1];
+          x[2 * i] = e * c[u][i] - o * sn[u][i];
+          x[2 * i + 1] = e * sn[u][i] + o * c[u][i];
+        }
+      }
+    } else {
+      const int pair = half / E;  // lanes between a dim and its partner
+      float other[E];
+#pragma unroll
+      for (int i = 0; i < E; ++i) other[i] = lane_xor(x[i], pair, lane);
+      if (!is_v[u] && rotated) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const int d = sub * E + i;
+          x[i] = x[i] * c[u][i] + (d < half ? -other[i] : other[i]) * sn[u][i];
+        }
       }
     }
-  }
-  if (!on) return;
+    if (!on[u]) continue;
 
-  if (!is_v) {
+    if (!is_v[u]) {
 #pragma unroll
-    for (int i = 0; i < E; ++i) raw[i] = QT::from_f32(x[i]);
-    if constexpr (E == 2) *reinterpret_cast<u32*>(row) = *reinterpret_cast<const u32*>(raw);
-    else if constexpr (E == 4) *reinterpret_cast<u32x2*>(row) = *reinterpret_cast<const u32x2*>(raw);
-    else *reinterpret_cast<u32x4*>(row) = *reinterpret_cast<const u32x4*>(raw);
-  }
-  if (a.k_cache == nullptr || is_q) return;
+      for (int i = 0; i < E; ++i) raw[u][i] = QT::from_f32(x[i]);
+      if constexpr (E == 2) *reinterpret_cast<u32*>(row[u]) = *reinterpret_cast<const u32*>(raw[u]);
+      else if constexpr (E == 4) *reinterpret_cast<u32x2*>(row[u]) = *reinterpret_cast<const u32x2*>(raw[u]);
+      else *reinterpret_cast<u32x4*>(row[u]) = *reinterpret_cast<const u32x4*>(raw[u]);
+    }
+    if (a.k_cache == nullptr || is_q[u]) continue;
 
-  // cache write of the k head (the bits just stored) or the v head (as loaded)
-  const int64_t slot = a.slots[token];
-  if (slot < 0 || slot >= a.n_slots) return;
-  const int kvh = is_v ? head - a.n_q - a.n_k : head - a.n_q;
-  const int n_kv = is_v ? a.n_v : a.n_k;
-  const int64_t e0 = (slot * n_kv + kvh) * D + sub * E;
-  char* dst = (is_v ? a.v_cache : a.k_cache);
-  if constexpr (FP8) {
-    const float inv = 1.0f / (is_v ? a.v_scale : a.k_scale)[kvh];
-    uint8_t code[E];
+    // cache write of the k head (the bits just stored) or the v head (as loaded)
+    if (slot[u] < 0 || slot[u] >= a.n_slots) continue;
+    const int kvh = is_v[u] ? head[u] - a.n_q - a.n_k : head[u] - a.n_q;
+    const int n_kv = is_v[u] ? a.n_v : a.n_k;
+    const int64_t e0 = (slot[u] * n_kv + kvh) * D + sub * E;
+    char* dst = (is_v[u] ? a.v_cache : a.k_cache);
+    if constexpr (FP8) {
+      const float inv = 1.0f / (is_v[u] ? a.v_scale : a.k_scale)[kvh];
+      uint8_t code[E];
 #pragma unroll
-    for (int i = 0; i < E; ++i) code[i] = static_cast<uint8_t>(fp8_quantize(QT::to_f32(raw[i]), inv));
-    if constexpr (E == 2) *reinterpret_cast<uint16_t*>(dst + e0) = *reinterpret_cast<const uint16_t*>(code);
-    else if constexpr (E == 4) *reinterpret_cast<u32*>(dst + e0) = *reinterpret_cast<const u32*>(code);
-    else *reinterpret_cast<u32x2*>(dst + e0) = *reinterpret_cast<const u32x2*>(code);
+      for (int i = 0; i < E; ++i) code[i] = static_cast<uint8_t>(fp8_quantize(QT::to_f32(raw[u][i]), inv));
+      if constexpr (E == 2) *reinterpret_cast<uint16_t*>(dst + e0) = *reinterpret_cast<const uint16_t*>(code);
+      else if constexpr (E == 4) *reinterpret_cast<u32*>(dst + e0) = *reinterpret_cast<const u32*>(code);
+      else *reinterpret_cast<u32x2*>(dst + e0) = *reinterpret_cast<const u32x2*>(code);
+    } else {
+      if constexpr (E == 2) *reinterpret_cast<u32*>(dst + e0 * 2) = *reinterpret_cast<const u32*>(raw[u]);
+      else if constexpr (E == 4) *reinterpret_cast<u32x2*>(dst + e0 * 2) = *reinterpret_cast<const u32x2*>(raw[u]);
+      else *reinterpret_cast<u32x4*>(dst + e0 * 2) = *reinterpret_cast<const u32x4*>(raw[u]);
+    }
+  }
+}
+
+template <typename QT, int D, int CT, int U>
+int launch_rope_units(const RopeArgs& a, bool interleave, bool fp8, hipStream_t stream) {
+  const int64_t threads = (a.n_units + U - 1) / U * 32;
+  const dim3 grid(static_cast<unsigned>((threads + 255) / 256));
+  if (interleave) {
+    if (fp8) rope_and_cache_kernel<QT, D, CT, true, true, U><<<grid, 256, 0, stream>>>(a);
+    else rope_and_cache_kernel<QT, D, CT, true, false, U><<<grid, 256, 0, stream>>>(a);
   } else {
-    if constexpr (E == 2) *reinterpret_cast<u32*>(dst + e0 * 2) = *reinterpret_cast<const u32*>(raw);
-    else if constexpr (E == 4) *reinterpret_cast<u32x2*>(dst + e0 * 2) = *reinterpret_cast<const u32x2*>(raw);
-    else *reinterpret_cast<u32x4*>(dst + e0 * 2) = *reinterpret_cast<const u32x4*>(raw);
+    if (fp8) rope_and_cache_kernel<QT, D, CT, false, true, U><<<grid, 256, 0, stream>>>(a);
+    else rope_and_cache_kernel<QT, D, CT, false, false, U><<<grid, 256, 0, stream>>>(a);
   }
+  return static_cast<int>(hipGetLastError());
 }
 
 template <typename QT, int D, int CT>
 int launch_rope(const RopeArgs& a, bool interleave, bool fp8, hipStream_t stream) {
-  const int64_t threads = a.n_units * 32;
-  const dim3 grid(static_cast<unsigned>((threads + 255) / 256));
-  if (interleave) {
-    if (fp8) rope_and_cache_kernel<QT, D, CT, true, true><<<grid, 256, 0, stream>>>(a);
-    else rope_and_cache_kernel<QT, D, CT, true, false><<<grid, 256, 0, stream>>>(a);
-  } else {
-    if (fp8) rope_and_cache_kernel<QT, D, CT, false, true><<<grid, 256, 0, stream>>>(a);
-    else rope_and_cache_kernel<QT, D, CT, false, false><<<grid, 256, 0, stream>>>(a);
-  }
-  return static_cast<int>(hipGetLastError());
+  // one unit per group while that still gives every CU several workgroups (decode), four beyond
+  return a.n_units * 32 / 256 < 8192 ? launch_rope_units<QT, D, CT, 1>(a, interleave, fp8, stream)
+                                      : launch_rope_units<QT, D, CT, 4>(a, interleave, fp8, stream);
 }
 
 template <typename QT, int D>
@@ -211,7 +277,8 @@ int rope_and_cache(void* qkv, const void* q_weight, const void* k_weight, const 
   const int64_t rotary_lanes = rotary_dim / (dims_per_lane > 0 ? dims_per_lane : 1);
   if (interleave == 0 && (rotary_lanes & (rotary_lanes - 1)) != 0) return XLLM_MI355_ESHAPE;
   if (token_stride < (n_heads_q + n_heads_k + n_heads_v) * head_dim) return XLLM_MI355_EINVAL;
-  if ((reinterpret_cast<uintptr_t>(qkv) & 15) != 0 || (token_stride * 2) % 16 != 0) return XLLM_MI355_EALIGN;
+  if (((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(cos_sin_cache)) & 15) != 0 || (token_stride * 2) % 16 != 0)
+    return XLLM_MI355_EALIGN;
   const bool with_cache = k_cache != nullptr;
   const bool fp8 = with_cache && cache_dtype == XLLM_MI355_FP8_E4M3;
   if (with_cache) {
