@@ -449,13 +449,22 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 // register load (the in-order counter would drain the ring): page-table entries come through the
 // LDS path in chunks of 64, fetched by wavefront 0 at least 32 sub-tiles ahead.
 //
-// Rows are 1184 bytes apart in LDS and the 16-byte chunks of a row are XOR-ed with bit 2 of the row
-// number: the 16-byte operand reads (8 consecutive rows per cycle) and the transposing reads
-// (4 rows x 32 bytes per cycle) then both touch every LDS bank once.
-constexpr int kRow16 = kRowBytes + 32;
+// A sub-tile in LDS is two areas.  The latent parts of its rows are 1056 bytes apart and the 16-byte
+// chunks of a row are XOR-ed with bit 2 of the row number: the 16-byte operand reads (8 consecutive
+// rows per cycle) and the transposing reads (4 rows x 32 bytes per cycle) then both touch every LDS
+// bank once.  The rope parts sit behind them, 128 bytes per row, chunk XOR-ed with the low 3 bits of
+// the row number.  Keeping them apart lets ONE load instruction bring the rope bytes of 4 rows (32
+// lanes x 16 bytes, the lane picks row and chunk through its global offset) instead of one
+// 8-lane instruction per row: a wavefront issues 5 loads per sub-tile instead of 8 (an 8-lane
+// load costs its wavefront as much issue time as a 64-lane one).  With 128 heads that time is
+// covered by the other wavefront of the SIMD and the layout changes nothing; with the few heads
+// of a tensor-parallel shard the computing wavefronts also issue loads and it is on their path.
+constexpr int kRow16 = kDL * 2 + 32;
 constexpr int kSubTok = 32;                      // tokens per sub-tile
 constexpr int kRing16 = 4;                       // ring slots
-constexpr int kSubBytes = kSubTok * kRow16;      // 37888
+constexpr int kRope16Off = kSubTok * kRow16;     // rope area of a sub-tile
+constexpr int kSubBytes = kRope16Off + kSubTok * kDR * 2;  // 37888
+constexpr int kLoadsPerSub16 = 5;                // per wavefront
 constexpr int kThreads16 = 512;
 constexpr int kHeadsPerWg16 = 128;
 constexpr int kPage16Off = kRing16 * kSubBytes;  // LDS: ring | page-table chunks [2][64] | prefix
@@ -480,39 +489,22 @@ __device__ __forceinline__ void dma4(const void* gptr, u32 lds_addr) {
   const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(base), "v"(gptr) : "memory");
 }
-// Four adjacent cache rows (1152 bytes apart) of one page into four LDS rows (kRow16 apart): per
-// row the 1024 latent bytes with all lanes, then the 128 rope bytes with the lanes of `rope`.
-// The instruction offset is added to the global AND to the LDS address (LDS address = M0 +
-// offset + lane * 16), so M0 only carries the difference of the two row strides.
-__device__ __forceinline__ void dma_rows4(uint64_t base, u32 lane_off, u32 lds_addr, bool rope) {
-  constexpr int kPad = kRow16 - kRowBytes;  // 32
-#define XLLM_DMA(lds, gbase, m0_add, goff)                                                               \
-  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%4 nt" ::"s"(lds), \
-               "v"(lane_off), "s"(gbase), "n"(m0_add), "n"(goff)                                         \
-               : "memory", "scc")
-  // instruction offsets reach 4095: rows 2 and 3 go through a second base
-  const uint64_t base2 = base + 2 * kRowBytes;
-  const u32 lds2 = lds_addr + 2 * kRow16;
-  XLLM_DMA(lds_addr, base, 0, 0);
-  XLLM_DMA(lds_addr, base, kPad, kRowBytes);
-  XLLM_DMA(lds2, base2, 0, 0);
-  XLLM_DMA(lds2, base2, kPad, kRowBytes);
-  if (rope) {
-    XLLM_DMA(lds_addr, base, 0, kDL * 2);
-    XLLM_DMA(lds_addr, base, kPad, kRowBytes + kDL * 2);
-    XLLM_DMA(lds2, base2, 0, kDL * 2);
-    XLLM_DMA(lds2, base2, kPad, kRowBytes + kDL * 2);
-  }
-#undef XLLM_DMA
-}
-// Wait until at most 8 * subs of the wavefront's vector memory operations are outstanding
-// (a wavefront issues 8 loads per sub-tile).
+// Wait until at most kLoadsPerSub16 * subs of the wavefront's vector memory operations are outstanding.
 __device__ __forceinline__ void wait_younger_subs(int subs) {
+  static_assert(kLoadsPerSub16 == 5, "the immediates below are multiples of the loads per sub-tile");
   if (subs <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  else if (subs == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else if (subs == 1) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
 }
 
+//
+// SPLIT (at most 64 heads per GPU, the head counts of tensor-parallel shards): with 16 heads per
+// wavefront only H / 16 wavefronts would compute and the loop would run at the pace of one
+// wavefront's chain of reads and MFMAs, well below what HBM delivers.  The two 16-token blocks of
+// every sub-tile then go to different wavefronts: wavefront (head block w % 4, token block w / 4)
+// keeps its own maximum, sum and O^T, and at the end of a run the token-block-1 wavefronts hand
+// theirs to their partners through the (then idle) ring, merged like two partials.
+template <bool SPLIT>
 __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kPrefix16Off);
@@ -531,9 +523,11 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
   const int y = blockIdx.x >> 3;
   const int hb128 = y % a.n_hb;
   const int team = (y / a.n_hb) * 8 + xcd;
-  const int head = hb128 * kHeadsPerWg16 + wave * 16 + c16;
+  const int hblk = SPLIT ? (wave & 3) : wave;  // 16-head block of the wavefront
+  const int tb = SPLIT ? (wave >> 2) : 0;      // SPLIT: its 16-token block of every sub-tile
+  const int head = hb128 * kHeadsPerWg16 + hblk * 16 + c16;
   const bool head_ok = head < H;
-  const bool wave_ok = hb128 * kHeadsPerWg16 + wave * 16 < H;
+  const bool wave_ok = hb128 * kHeadsPerWg16 + hblk * 16 < H;
 
   // ---- tile prefix over the batch (every workgroup computes it; no extra launch)
   {
@@ -577,6 +571,15 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
   const int v_row0 = (4 * g + (c16 >> 2)) * kRow16 + ((((c16 & 3) >> 1) ^ (g & 1)) * 16) + (c16 & 1) * 8;
   // tile loads: this wavefront moves rows wave*4 .. +3 of a sub-tile; bit 2 of those rows is wave & 1
   const u32 lane_off = (lane ^ (wave & 1)) * 16;
+  // The kernel runs at the register limit, and a per-lane constant more costs the operand reads of
+  // the loop a buffer of their pipeline: the few per-lane offsets of the rope area are therefore
+  // recomputed where they are used, from this copy of the lane number that the compiler cannot
+  // trace back to the thread index (it would otherwise hoist them into registers of their own).
+  auto lane_again = [&]() {
+    u32 x = lane_off;
+    asm volatile("" : "+v"(x));
+    return static_cast<int>(x >> 4) ^ (wave & 1);
+  };
 
   while (cur < end) {
     int lo = 0, hi = a.batch;
@@ -620,37 +623,35 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
       dma4(pages + min(ck * kWave + lane, n_pages - 1), page_lds + (ck & 1) * kWave * 4);
     };
     int ck_cur = (t_begin >> a.bs_shift) >> 6;  // chunk of the sub-tile being issued
-    // Rows go from global memory straight into LDS: one 64-lane load moves the 1024 latent bytes
-    // of a row, a second one with 8 lanes the 128 rope bytes; 8 loads per wavefront and sub-tile.
+    // Rows go from global memory straight into LDS: one 64-lane load per row moves its 1024 latent
+    // bytes, a fifth load with 32 lanes the 128 rope bytes of all 4 rows.
     auto issue_sub = [&](int sub) {
       const int tok0 = t_begin + sub * kSubTok + wave * 4;  // block_size >= 16: the 4 rows share a page
-      const u32 dst = __builtin_amdgcn_readfirstlane(lds_base + (sub & (kRing16 - 1)) * kSubBytes + wave * 4 * kRow16);
+      const u32 slot = lds_base + (sub & (kRing16 - 1)) * kSubBytes;
+      const u32 dst = __builtin_amdgcn_readfirstlane(slot + wave * 4 * kRow16);
+      const u32 dst_rope = __builtin_amdgcn_readfirstlane(slot + kRope16Off + wave * 4 * (kDR * 2));
       const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
-      const int ck = (min(tok0, L - 1) >> a.bs_shift) >> 6;
+      const int tb = min(tok0, L - 1);  // rows past the end of the context repeat the last valid row
+      const int ck = (tb >> a.bs_shift) >> 6;
       if (ck != ck_cur) {  // first sub-tile of a chunk: wavefront 0 fetches the one after it
         ck_cur = ck;
         if (wave == 0 && (ck + 1) * kWave < n_pages) issue_chunk(ck + 1);
       }
-      if (tok0 + 3 < L) {
-        int page = __builtin_amdgcn_readfirstlane(pagebuf[(ck & 1) * kWave + ((tok0 >> a.bs_shift) & 63)]);
-        page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
-        const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tok0 & (a.block_size - 1))) * kRowBytes;
-        const u32 lo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row)));
-        const u32 hi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row >> 32)));
-        const uint64_t sb = (static_cast<uint64_t>(hi) << 32) | lo;
-        // the 4 rows are adjacent in the page: one base, the row offset in the instruction
-        dma_rows4(sb, lane_off, dst, lane < kDR * 2 / 16);
-      } else {  // ragged end of the context: rows past it repeat the last valid row
+      int page = __builtin_amdgcn_readfirstlane(pagebuf[(ck & 1) * kWave + ((tb >> a.bs_shift) & 63)]);
+      page = max(0, min(page, a.num_blocks - 1));  // a corrupt table must not fault the GPU
+      const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tb & (a.block_size - 1))) * kRowBytes;
+      const u32 lo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row)));
+      const u32 hi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row >> 32)));
+      const uint64_t sb = (static_cast<uint64_t>(hi) << 32) | lo;
+      const int last = __builtin_amdgcn_readfirstlane(L - 1 - tb);  // valid rows after the first: >= 0
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tok = min(tok0 + i, L - 1);
-          int page = __builtin_amdgcn_readfirstlane(pagebuf[(((tok >> a.bs_shift) >> 6) & 1) * kWave + ((tok >> a.bs_shift) & 63)]);
-          page = max(0, min(page, a.num_blocks - 1));
-          const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tok & (a.block_size - 1))) * kRowBytes;
-          dma16_row(row, lane_off, dst + i * kRow16);
-          if (lane < kDR * 2 / 16) dma16_row(row + kDL * 2, lane_off, dst + i * kRow16 + kDL * 2);
-        }
-      }
+      for (int i = 0; i < 4; ++i) dma16_row(sb + static_cast<uint64_t>(min(i, last)) * kRowBytes, lane_off, dst + i * kRow16);
+      // rope load: lane (row r = lane / 8 of the 4, position p = lane % 8) lands at rope row wave*4 + r,
+      // position p, and so fetches chunk p ^ (low 3 bits of that row)
+      const int ln = lane_again();
+      const int rope_r = (ln >> 3) & 3;
+      const u32 rope_off = min(rope_r, last) * kRowBytes + kDL * 2 + (((ln & 7) ^ ((wave & 1) * 4 + rope_r)) * 16);
+      if (lane < 4 * kDR * 2 / 16) dma16_row(sb, rope_off, dst_rope);
     };
 
     // make the compiler wait for the Q loads here, not inside the loop
@@ -671,92 +672,190 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
       // Wavefronts 0-3 issue their rows of sub-tile sub + 3 (into the slot released just now)
       // before they compute, wavefronts 4-7 (the second wavefront of each SIMD) after: the phases
       // of the two groups then interleave instead of all eight hitting LDS at the same time.
-      if (wave < 4 && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
+      const bool early = wave < 4;
+      if (early && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
       const char* kb = smem + (sub & (kRing16 - 1)) * kSubBytes;
       if (wave_ok) {
-        // ---- S^T of the sub-tile, two blocks of 16 tokens: lane (head c16, tokens 16 tb + 4g + r)
-        f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
-        const char* ka = kb + k_row0;
-        __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the Q.K reads only
+        // rope k-steps: row c16 of the rope area, chunk (kk - 16) * 4 + g XOR-ed with the low 3 bits of the row
+        const int ln = lane_again();
+        const char* kr = kb + kRope16Off + (ln & 15) * (kDR * 2);
+        const int kr_x = (ln >> 4) ^ (ln & 7);
+        if constexpr (SPLIT) {
+          // ---- S^T of the wavefront's 16 tokens: lane (head c16, tokens 16 tb + 4g + r)
+          f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f};
+          const char* ka = kb + k_row0 + tb * 16 * kRow16;
+          __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the Q.K reads only
 #pragma unroll
-        for (int kk = 0; kk < kKSteps32; ++kk) {
-          const u32x4 x0 = *reinterpret_cast<const u32x4*>(ka + kk * 64);
-          const u32x4 x1 = *reinterpret_cast<const u32x4*>(ka + 16 * kRow16 + kk * 64);
-          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x0), __builtin_bit_cast(bf16x8, q[kk]), s0, 0, 0, 0);
-          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x1), __builtin_bit_cast(bf16x8, q[kk]), s1, 0, 0, 0);
-        }
-        // pipeline the LDS operand reads kAhead MFMAs ahead of their use
-        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
-#pragma unroll
-        for (int i = 0; i < 2 * kKSteps32 - kAhead; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        float sv[8];
-        const int tok_base = t_begin + sub * kSubTok + 4 * g;
-        bool over = false;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          sv[r] = tok_base + r < L ? s0[r] * a.scale_log2 : -INFINITY;
-          sv[4 + r] = tok_base + 16 + r < L ? s1[r] * a.scale_log2 : -INFINITY;
-        }
-#pragma unroll
-        for (int r = 0; r < 8; ++r) over |= sv[r] > m + kSlack;
-        if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
-          float mx = sv[0];
-#pragma unroll
-          for (int r = 1; r < 8; ++r) mx = fmaxf(mx, sv[r]);
-          mx = quad_rows_max(mx);
-          if (mx > m + kSlack) {
-            const float alpha = fast_exp2(m - mx);
-            m = mx;
-            l *= alpha;
-#pragma unroll
-            for (int i = 0; i < 32; ++i) o[i] *= alpha;
+          for (int kk = 0; kk < kKSteps32; ++kk) {
+            const char* k0 = kk < kDL / 32 ? ka + kk * 64 : kr + tb * 16 * (kDR * 2) + (kk == kDL / 32 ? kr_x : kr_x ^ 4) * 16;
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(k0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x0), __builtin_bit_cast(bf16x8, q[kk]), s0, 0, 0, 0);
           }
-        }
-        float p[8];
+          __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          p[r] = fast_exp2(sv[r] - m);
-          l += p[r];
-        }
-        // k-slot g*8 + j of the P.V MFMA <-> token 4g + j of block 0 (j < 4), of block 1 (j >= 4)
-        const u32x4 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3]), BF16::pack(p[4], p[5]), BF16::pack(p[6], p[7])};
-        const bf16x8 pb = __builtin_bit_cast(bf16x8, pbw);
-        // ---- O^T += V^T . P^T over the 32 tokens and all 512 dims.  The transposing LDS load works on
-        // groups of 16 lanes: lane p of a group supplies the address of 4 dims of token row p/4 and
-        // receives the 4 tokens of dim column p.
-        const char* va = kb + v_row0;
-        __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the P.V reads only
+          for (int i = 0; i < kKSteps32 - kAhead; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          float sv[4];
+          const int tok_base = t_begin + sub * kSubTok + tb * 16 + 4 * g;
+          bool over = false;
 #pragma unroll
-        for (int mb = 0; mb < 32; ++mb) {
-          const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
-          const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + 16 * kRow16 + mb * 32));
-          const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-          o[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, o[mb], 0, 0, 0);
-        }
-        // pipeline the transposing reads (two per MFMA) kAhead MFMAs ahead of their use
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+          for (int r = 0; r < 4; ++r) {
+            sv[r] = tok_base + r < L ? s0[r] * a.scale_log2 : -INFINITY;
+            over |= sv[r] > m + kSlack;
+          }
+          if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+            const float mx = quad_rows_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+            if (mx > m + kSlack) {
+              const float alpha = fast_exp2(m - mx);
+              m = mx;
+              l *= alpha;
 #pragma unroll
-        for (int i = 0; i < 32 - kAhead; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+              for (int i = 0; i < 32; ++i) o[i] *= alpha;
+            }
+          }
+          float p[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            p[r] = fast_exp2(sv[r] - m);
+            l += p[r];
+          }
+          const u32x2 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3])};
+          const s16x4 pb = __builtin_bit_cast(s16x4, pbw);
+          // ---- O^T += V^T . P^T over the 16 tokens: k-slot 4g + j of the MFMA <-> token 4g + j of the block
+          const char* va = kb + v_row0 + tb * 16 * kRow16;
+          __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the P.V reads only
+#pragma unroll
+          for (int mb = 0; mb < 32; ++mb) {
+            const s16x4 v4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
+            o[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v4, pb, o[mb], 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+          for (int i = 0; i < 32 - kAhead; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          // ---- S^T of the sub-tile, two blocks of 16 tokens: lane (head c16, tokens 16 tb + 4g + r)
+          f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+          const char* ka = kb + k_row0;
+          __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the Q.K reads only
+#pragma unroll
+          for (int kk = 0; kk < kKSteps32; ++kk) {
+            const char* k0 = kk < kDL / 32 ? ka + kk * 64 : kr + (kk == kDL / 32 ? kr_x : kr_x ^ 4) * 16;
+            const u32x4 x0 = *reinterpret_cast<const u32x4*>(k0);
+            const u32x4 x1 = *reinterpret_cast<const u32x4*>(k0 + 16 * (kk < kDL / 32 ? kRow16 : kDR * 2));
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x0), __builtin_bit_cast(bf16x8, q[kk]), s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x1), __builtin_bit_cast(bf16x8, q[kk]), s1, 0, 0, 0);
+          }
+          // pipeline the LDS operand reads kAhead MFMAs ahead of their use
+          __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+          for (int i = 0; i < 2 * kKSteps32 - kAhead; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          float sv[8];
+          const int tok_base = t_begin + sub * kSubTok + 4 * g;
+          bool over = false;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            sv[r] = tok_base + r < L ? s0[r] * a.scale_log2 : -INFINITY;
+            sv[4 + r] = tok_base + 16 + r < L ? s1[r] * a.scale_log2 : -INFINITY;
+          }
+#pragma unroll
+          for (int r = 0; r < 8; ++r) over |= sv[r] > m + kSlack;
+          if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+            float mx = sv[0];
+#pragma unroll
+            for (int r = 1; r < 8; ++r) mx = fmaxf(mx, sv[r]);
+            mx = quad_rows_max(mx);
+            if (mx > m + kSlack) {
+              const float alpha = fast_exp2(m - mx);
+              m = mx;
+              l *= alpha;
+#pragma unroll
+              for (int i = 0; i < 32; ++i) o[i] *= alpha;
+            }
+          }
+          float p[8];
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            p[r] = fast_exp2(sv[r] - m);
+            l += p[r];
+          }
+          // k-slot g*8 + j of the P.V MFMA <-> token 4g + j of block 0 (j < 4), of block 1 (j >= 4)
+          const u32x4 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3]), BF16::pack(p[4], p[5]), BF16::pack(p[6], p[7])};
+          const bf16x8 pb = __builtin_bit_cast(bf16x8, pbw);
+          // ---- O^T += V^T . P^T over the 32 tokens and all 512 dims.  The transposing LDS load works on
+          // groups of 16 lanes: lane p of a group supplies the address of 4 dims of token row p/4 and
+          // receives the 4 tokens of dim column p.
+          const char* va = kb + v_row0;
+          __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the P.V reads only
+#pragma unroll
+          for (int mb = 0; mb < 32; ++mb) {
+            const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
+            const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + 16 * kRow16 + mb * 32));
+            const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+            o[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, o[mb], 0, 0, 0);
+          }
+          // pipeline the transposing reads (two per MFMA) kAhead MFMAs ahead of their use
+          __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+          for (int i = 0; i < 32 - kAhead; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
-        __builtin_amdgcn_sched_barrier(0);
       }
-      if (wave >= 4 && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
+      if (!early && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
     }
 
-    // ---- end of the run: every wavefront writes its own heads
+    if constexpr (SPLIT) {
+      // the token-block-1 wavefronts hand their state to their partners: [head block][value][lane] floats
+      // in the ring, which nobody reads or writes between the last sub-tile and the next run
+      constexpr int kState = 32 * 4 + 2;
+      float* xch = reinterpret_cast<float*>(smem) + hblk * kState * kWave + lane;
+      static_assert(4 * kState * kWave * 4 <= kRing16 * kSubBytes, "the exchange fits the ring");
+      __syncthreads();
+      if (tb == 1 && wave_ok) {
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) xch[(i * 4 + r) * kWave] = o[i][r];
+        xch[128 * kWave] = m;
+        xch[129 * kWave] = l;
+      }
+      __syncthreads();
+      if (tb == 0 && wave_ok) {
+        const float m1 = xch[128 * kWave], l1 = xch[129 * kWave];
+        const float mm = fmaxf(m, m1);
+        const float a0 = fast_exp2(m - mm), a1 = fast_exp2(m1 - mm);
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[i][r] = o[i][r] * a0 + xch[(i * 4 + r) * kWave] * a1;
+        l = l * a0 + l1 * a1;
+        m = mm;
+      }
+    }
+    // ---- end of the run: every wavefront (SPLIT: of token block 0) writes its own heads
+    const bool writer = head_ok && tb == 0;
     const float lsum = quad_rows_sum(l);
     const float inv = 1.0f / lsum;
     const float lse2 = m + fast_log2(lsum);
     const int64_t ps = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H + head;
-    if (head_ok && complete) {
+    if (writer && complete) {
       char* op = a.out + ((static_cast<int64_t>(b) * H + head) * kDL + 4 * g) * 2;
 #pragma unroll
       for (int mb = 0; mb < 32; ++mb) {
@@ -764,7 +863,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
         *reinterpret_cast<u32x2*>(op + mb * 32) = w;
       }
     }
-    if (head_ok && !complete) {
+    if (writer && !complete) {
       float* wp = a.ws_out + ps * kDL + 4 * g;
 #pragma unroll
       for (int mb = 0; mb < 32; ++mb) {
@@ -772,8 +871,8 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
         *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
       }
     }
-    if (head_ok && g == 0 && complete && a.lse != nullptr) a.lse[b * H + head] = lse2 * kLn2;
-    if (head_ok && g == 0 && !complete) a.ws_lse[ps] = lse2;
+    if (writer && g == 0 && complete && a.lse != nullptr) a.lse[b * H + head] = lse2 * kLn2;
+    if (writer && g == 0 && !complete) a.ws_lse[ps] = lse2;
     first_run = false;
   }
 }
@@ -1484,7 +1583,11 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
                                        hipFuncAttributeMaxDynamicSharedMemorySize,
                                        static_cast<int>(kPrefixOff + (kMaxBatchMla + 1) * 4));
     if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode16_kernel),
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode16_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(kPrefix16Off + (kMaxBatchMla + 1) * 4));
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode16_kernel<true>),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(kPrefix16Off + (kMaxBatchMla + 1) * 4));
     if (e == hipSuccess)
@@ -1523,8 +1626,10 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       launch_timed(mla_decode_kernel, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kMlaThreads), smem, stream, a);
     else if (use_p)
       launch_timed(mla_decode32w_kernel, dim3(static_cast<unsigned>(a.n_teams * a.n_hb)), dim3(kWThreads), kPLdsBytes, stream, a);
+    else if (n_heads <= 64)  // head counts of tensor-parallel shards: two wavefronts per 16 heads
+      launch_timed(mla_decode16_kernel<true>, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kThreads16), smem, stream, a);
     else
-      launch_timed(mla_decode16_kernel, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kThreads16), smem, stream, a);
+      launch_timed(mla_decode16_kernel<false>, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kThreads16), smem, stream, a);
     int rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
     mla_merge_kernel<<<dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb)), 128, 0, stream>>>(a);
