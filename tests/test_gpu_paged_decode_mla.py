@@ -105,11 +105,22 @@ def test_small_and_odd_block_sizes_and_page_table_chunks(device):
     _check(_mla_cfg("short", 96, 16, 1, 200, bs=16), 13, device)
 
 
+def test_token_blocks_on_different_wavefronts_for_few_heads(device):
+    # at most 64 heads: the two 16-token blocks of a sub-tile go to different wavefronts whose states are merged
+    # at the end of a run.  Contexts long enough to span several workgroups (partials of merged states), head
+    # counts that leave the last head block partly or wholly empty, and lengths whose last sub-tile has nothing
+    # for the second token block.
+    for heads, seed in ((48, 3), (64, 4), (24, 5), (16, 6)):
+        _check(_mla_cfg(f"few{heads}", 5, heads, 1200, 4000), seed, device)
+    for L in (1, 16, 17, 33, 48, 65):  # the generator draws lengths from [lo, hi]: pin them one by one
+        _check(_mla_cfg(f"few32_L{L}", 2, 32, L, L), 50 + L, device)
+
+
 def test_scores_that_rise_along_the_context(device):
     # the rope dims of K carry a ramp and those of Q a constant, so the scores rise by about 120 log2 units from
     # the first token to the last: every running maximum is overtaken many times and whatever was accumulated
     # before has to be rescaled (or restarted) again and again; V = K[..., :512] is unaffected
-    for heads, lo, hi, bs in ((128, 1500, 2500, 64), (16, 700, 900, 16)):
+    for heads, lo, hi, bs in ((128, 1500, 2500, 64), (16, 700, 900, 16), (32, 1500, 2500, 64)):
         cfg = _mla_cfg(f"ramp{heads}", 3, heads, lo, hi, bs=bs)
         inp = workloads.make_inputs(cfg, 31)
         lay = inp.layout
