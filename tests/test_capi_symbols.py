@@ -48,6 +48,23 @@ def test_host_only_entry_points_without_a_gpu():
     assert lib.xllm_mi355_lse_merge(None, None, None, None, 2, 1, 1, 8, capi.FP32, None) == -1
     assert lib.xllm_mi355_reshape_and_cache(None, None, None, None, None, None, None, 0, 8, 128, 16, 10,
                                             1024, 1024, capi.BF16, capi.BF16, None) == 0  # no tokens: no-op
+    # the entry points either side of the path: null pointers, shapes and alignments they do not take
+    fake = 1 << 20  # an aligned non-null address: the calls below return before anything is launched
+    bmm = lib.xllm_mi355_mla_absorbed_bmm
+    assert bmm(None, None, None, 4, 16, 128, 512, 2048, 128, 8192, 512, capi.BF16, None) == -1
+    assert bmm(fake, fake, fake, 0, 16, 128, 512, 2048, 128, 8192, 512, capi.BF16, None) == 0      # no tokens: no-op
+    assert bmm(fake, fake, fake, 4, 16, 96, 512, 1536, 96, 8192, 512, capi.BF16, None) == -3       # K not a multiple of 128
+    assert bmm(fake, fake, fake, 4, 16, 128, 48, 2048, 128, 768, 48, capi.BF16, None) == -3        # N not a multiple of 64
+    assert bmm(fake, fake, fake, 4, 16, 128, 512, 2048, 128, 8192, 512, capi.FP16, None) == -2     # bf16 only
+    assert bmm(fake + 2, fake, fake, 4, 16, 128, 512, 2048, 128, 8192, 512, capi.BF16, None) == -5
+    assert bmm(fake, fake, fake, 4, 16, 128, 512, 2048, 64, 8192, 512, capi.BF16, None) == -1      # heads overlap in x
+    mask = lib.xllm_mi355_mask_block_table_padding
+    assert mask(None, 8, None, None, 8, 4, 8, 16, None) == -1
+    assert mask(fake, 4, fake, fake, 8, 4, 8, 16, None) == -1                                      # row stride below the width
+    assert mask(fake, 8, fake, fake, 8, 4, 8, 0, None) == -1                                       # block size
+    assert mask(fake, 8, fake, fake, 8, 0, 8, 16, None) == 0                                       # empty batch: no-op
+    assert lib.xllm_mi355_rope_and_cache(fake, None, None, fake + 4, fake, None, None, None, None, None, 4, 6144, 32, 8,
+                                         8, 128, 128, 1e-6, 0, 16, 10, capi.BF16, capi.FP32, capi.BF16, None) == -5
     # workspace sizes are positive and grow with the head dim
     a = lib.xllm_mi355_paged_decode_workspace_bytes(64, 32, 128, 4096)
     b = lib.xllm_mi355_paged_decode_workspace_bytes(64, 32, 256, 4096)
