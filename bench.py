@@ -261,7 +261,8 @@ def main():
         achieved = nbytes / (kernel_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                    "kernel": "gqa_mfma_kernel" if cfg.head_dim == 128 else "gqa_decode_kernel",
+                    "kernel": ("gqa_mfma_kernel" if cfg.head_dim == 128 or (cfg.head_dim == 64 and cfg.cache_dtype != "fp8")
+                               else "gqa_decode_kernel"),
                     "kernel_ms": kernel_ms, "algorithmic_bytes": nbytes}
 
     # the same number of bytes through the plain read kernel: the rate this GPU sustains at this size

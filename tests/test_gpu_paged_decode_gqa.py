@@ -59,6 +59,20 @@ def test_fp16_and_other_head_dims(device):
         _check_config(cfg, 100 + D + Hq, device, dtype=dt)
 
 
+def test_head_dim_64_on_the_matrix_core_kernel(device):
+    # head dim 64 with a power-of-two block size >= 16: rows of 128 bytes, 32 tokens per stage, two score blocks.
+    # Group sizes that fill 1, 4 and all 16 columns and one that needs two head blocks; block sizes 16 / 64 / 128;
+    # contexts from one token to several workers' worth; lengths around the 16- and 32-token boundaries; fp16.
+    for name, batch, Hq, Hkv, bs, lo, hi, dt in (("g1", 4, 4, 4, 32, 1, 700, torch.bfloat16),
+                                                 ("g4", 5, 32, 8, 16, 1, 3000, torch.bfloat16),
+                                                 ("g16", 3, 16, 1, 128, 100, 2500, torch.float16),
+                                                 ("g20", 3, 40, 2, 64, 50, 1200, torch.bfloat16),
+                                                 ("long", 3, 8, 2, 16, 20000, 40000, torch.bfloat16)):
+        _check_config(workloads.DecodeConfig(f"d64_{name}", batch, Hq, Hkv, 64, bs, lo, hi), 300 + Hq, device, dtype=dt)
+    for L in (1, 15, 16, 17, 31, 32, 33, 48, 64, 65):
+        _check_config(workloads.DecodeConfig(f"d64_L{L}", 2, 8, 2, 64, 16, L, L), 400 + L, device)
+
+
 def test_reference_npu_case_130_tokens_block128(device):
     # Qwen35_27B_TP4_KvCacheCrosses128TokenBoundary (tests/core/kernels/npu/npu_xllm_ops_test.cpp:305-394):
     # seq 130, block 128, 3 blocks, Hq 6 / Hkv 1 / D 256, scale 1/16, table [[2, 0]], tolerance 5e-2

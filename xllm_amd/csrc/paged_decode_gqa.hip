@@ -10,8 +10,8 @@
 // writes a normalised fp32 partial + log2-domain LSE, and a small merge kernel folds those.
 // The item counts are prefix-summed inside every workgroup (no extra launch, no host read).
 //
-// gqa_mfma_kernel (head_dim 128, block size a power of two >= 16): worker = a loading and a computing
-// wavefront, item = 16 tokens (32 for fp8 pages); rows travel global memory -> LDS directly into a
+// gqa_mfma_kernel (head_dim 128, or 64 with 16-bit pages; block size a power of two >= 16): worker = a loading
+// and a computing wavefront, item = 16 tokens (32 for rows of 128 bytes: fp8 pages, head_dim 64); rows travel global memory -> LDS directly into a
 // private ring per worker and both products run on the matrix cores.  Its own comment below has the
 // details.
 //
@@ -490,7 +490,8 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Matrix-core variant for D = 128 with 16-bit pages.
+// Matrix-core variant, described for D = 128 with 16-bit pages (fp8 pages and D = 64 differ in the
+// number of tokens per stage and are noted where they do).
 //
 // A worker is a PAIR of wavefronts that share a SIMD: wavefront w of the workgroup loads, wavefront
 // kWaves + w computes.  A wavefront cannot issue more than one load-to-LDS instruction per 90 ns or
@@ -675,12 +676,19 @@ struct MfmaLayout {
 // columns hold (token j, head h) pairs, column j * group + h, all against the same pages: 16 / group tokens
 // per column block, chunk_blocks column blocks per KV head, so a chunk costs the page traffic of
 // ceil(tokens * group / 16) single tokens; column j is masked beyond its own length.
-template <typename QT, bool FP8, int NS, bool VL>
+// D = 64 (16-bit pages only): rows of 128 bytes, so a stage holds 32 tokens and is multiplied as two blocks
+// of 16 like an fp8 stage, with 2 k-steps per score block and 4 dim blocks.
+template <typename QT, bool FP8, int NS, bool VL, int D>
 __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   static_assert(NS >= 2 && NS <= 4, "wait_younger_stages covers up to three stages in flight");
+  static_assert(D == 128 || (D == 64 && !FP8), "head dims of the matrix-core loop");
   using Lay = MfmaLayout<NS>;
-  constexpr int D = 128, G = kMfmaHeads;
-  constexpr int RB = FP8 ? 128 : 256;      // bytes of one token row of one KV head
+  constexpr int G = kMfmaHeads;
+  constexpr int KS = D / 32;               // k-steps of a score block
+  constexpr int MB = D / 16;               // dim blocks of the output
+  constexpr int QLPR = D * 2 / 16;         // 16-byte chunks of a Q row
+  constexpr int QRPI = kWave / QLPR;       // Q rows per load instruction
+  constexpr int RB = FP8 ? D : 2 * D;      // bytes of one token row of one KV head
   constexpr int T = kStageBytes / 2 / RB;  // tokens per stage
   constexpr int LPR = RB / 16;             // lanes (16-byte chunks) per row in a load instruction
   constexpr int RPI = kWave / LPR;         // rows per load instruction
@@ -826,7 +834,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     lane_v[i] = static_cast<u32>((row & 15) * a.row_bytes) + ((dc ^ swz_v(row)) * 16);
   }
   // per-lane constants of the operand reads
-  const int q_read = c16 * 256;  // Q rows (16-bit): + ((chunk ^ c16) * 16)
+  const int q_read = c16 * (D * 2);  // Q rows (16-bit): + ((chunk ^ (c16 % QLPR)) * 16)
   // 16-bit pages.  K: row c16, + ((chunk ^ c16) * 16).  V: lane c16 of a 16-lane group addresses 4 dims
   // (8 bytes) of token row 4g + c16/4; + (v_y ^ (mb << 5)) selects dims 16 mb ..
   const int k_read = c16 * RB;
@@ -895,18 +903,18 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       if constexpr (VL) {
         const int nhp = pc.qn * a.group;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int row = 4 * i + g;
-          dma16(a.q + q_row_offset(pc, kvh, max(0, min(row, nhp - 1))) + ((c16 ^ row) * 16), q_lds + i * 1024);
+        for (int i = 0; i < G / QRPI; ++i) {
+          const int row = QRPI * i + lane / QLPR;
+          dma16(a.q + q_row_offset(pc, kvh, max(0, min(row, nhp - 1))) + (((lane % QLPR) ^ (row % QLPR)) * 16), q_lds + i * 1024);
         }
       } else {
         const int h0p = kvh * a.group + (pc.hbk % hb_per_kv) * G;
         const int nhp = min(G, (kvh + 1) * a.group - h0p);
         const char* qb = a.q + pc.b * a.q_stride_bytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int row = 4 * i + g;
-          dma16(qb + (static_cast<int64_t>(h0p + min(row, nhp - 1)) * D) * 2 + ((c16 ^ row) * 16), q_lds + i * 1024);
+        for (int i = 0; i < G / QRPI; ++i) {
+          const int row = QRPI * i + lane / QLPR;
+          dma16(qb + (static_cast<int64_t>(h0p + min(row, nhp - 1)) * D) * 2 + (((lane % QLPR) ^ (row % QLPR)) * 16), q_lds + i * 1024);
         }
       }
     }
@@ -1012,8 +1020,8 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   int Lc = 0;                 // tokens the lane's column attends to (the context length unless VL and causal)
   int64_t out_off = 0;        // VL: byte offset of the lane's output row
   int c_ctx_first = 0, c_prev_len = 0;
-  u32x4 q[4];
-  f32x4 o[8];
+  u32x4 q[KS];
+  f32x4 o[MB];
   float m = kNegBig, l = 0.0f;
   float score_scale = a.scale_log2, out_scale = 1.0f;
 
@@ -1045,11 +1053,11 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       complete = cc.st == 0 && cc.n_st <= n_stages - s;
       if (s == 0 || c_prev_len >= NS) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk)  // the rows landed before this stage's tiles did
-          q[kk] = *reinterpret_cast<const u32x4*>(qbuf + q_read + (((kk * 4 + g) ^ c16) * 16));
+        for (int kk = 0; kk < KS; ++kk)  // the rows landed before this stage's tiles did
+          q[kk] = *reinterpret_cast<const u32x4*>(qbuf + q_read + (((kk * 4 + g) ^ (c16 % QLPR)) * 16));
       } else {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < KS; ++kk) {
           if constexpr (VL)
             q[kk] = ldg16(a.q + q_row_offset(cc, kvh, max(0, min(c16, nh - 1))) + (kk * 32 + g * 8) * 2);
           else
@@ -1058,14 +1066,15 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         }
         // The wait for these loads (it also drains the stages in flight) must stay on this path:
         // left to the first use after the join it would run on every stage.
-        asm volatile("" : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]));
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) asm volatile("" : "+v"(q[kk]));
       }
       if (c16 >= nh) {
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) q[kk] = u32x4{0u, 0u, 0u, 0u};
+        for (int kk = 0; kk < KS; ++kk) q[kk] = u32x4{0u, 0u, 0u, 0u};
       }
 #pragma unroll
-      for (int mb = 0; mb < 8; ++mb) o[mb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int mb = 0; mb < MB; ++mb) o[mb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
       m = kNegBig;
       l = 0.0f;
       c_ctx_first = s;
@@ -1076,7 +1085,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     }
 
     const char* st = ring + (s % NS) * kStageBytes;
-    if constexpr (!FP8) {
+    if constexpr (!FP8 && T == 16) {
       // ---- all operand reads of the stage first: the latency of the V^T reads passes behind the score
       // MFMAs and the softmax (the scheduler would otherwise place them next to their use)
       u32x4 kr[4];
@@ -1108,7 +1117,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
           m = mx;
           l *= alpha;
 #pragma unroll
-          for (int mb = 0; mb < 8; ++mb) o[mb] *= alpha;
+          for (int mb = 0; mb < MB; ++mb) o[mb] *= alpha;
         }
       }
       float pr[4];
@@ -1122,6 +1131,64 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       // row 4g + c16/4 and receives the 4 tokens of dim column 16 mb + c16
 #pragma unroll
       for (int mb = 0; mb < 8; ++mb) o[mb] = Mfma<QT>::k16(vt[mb], pb, o[mb]);
+    } else if constexpr (!FP8) {
+      // ---- 16-bit pages with 32 tokens per stage (head dim 64): two score blocks of 16 tokens,
+      // lane (head c16, tokens 16 tb + 4g ..), then all 32 tokens in one P.V MFMA per dim block
+      u32x4 kr[2][KS];
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb) {
+        const int tok = tb * 16 + c16;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk)
+          kr[tb][kk] = *reinterpret_cast<const u32x4*>(st + tok * RB + (((kk * 4 + g) ^ (tok & (LPR - 1))) * 16));
+      }
+      s16x4 vlo[MB], vhi[MB];
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        vlo[mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + v_read + (v_y ^ (mb << 5))));
+        vhi[mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + v_read + 16 * RB + (v_y ^ (mb << 5))));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      float sv[8];
+      bool over = false;
+#pragma unroll
+      for (int tb = 0; tb < 2; ++tb) {
+        f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) sc = Mfma<QT>::k32(kr[tb][kk], q[kk], sc);
+        const int tok0 = cc.st * T + tb * 16 + 4 * g;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          sv[tb * 4 + r] = tok0 + r < Lc ? sc[r] * score_scale : -INFINITY;
+          over |= sv[tb * 4 + r] > m + kSlack;
+        }
+      }
+      if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+        float mx = sv[0];
+#pragma unroll
+        for (int r = 1; r < 8; ++r) mx = fmaxf(mx, sv[r]);
+        mx = quad_rows_max(mx);
+        if (mx > m + kSlack) {
+          const float alpha = fast_exp2(m - mx);
+          m = mx;
+          l *= alpha;
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) o[mb] *= alpha;
+        }
+      }
+      float pr[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        pr[r] = fast_exp2(sv[r] - m);
+        l += pr[r];
+      }
+      // k-slot 8g + j of the P.V MFMA <-> token 4g + j of block 0 (j < 4), of block 1 (j >= 4)
+      const u32x4 pb = {QT::pack(pr[0], pr[1]), QT::pack(pr[2], pr[3]), QT::pack(pr[4], pr[5]), QT::pack(pr[6], pr[7])};
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const u32x2 lo = __builtin_bit_cast(u32x2, vlo[mb]), hi = __builtin_bit_cast(u32x2, vhi[mb]);
+        o[mb] = Mfma<QT>::k32(u32x4{lo[0], lo[1], hi[0], hi[1]}, pb, o[mb]);
+      }
     } else {
       // ---- scores of the stage's 32 tokens, two blocks of 16: lane (head c16, tokens 16 tb + 4g ..)
       float sv[8];
@@ -1155,7 +1222,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
           m = mx;
           l *= alpha;
 #pragma unroll
-          for (int mb = 0; mb < 8; ++mb) o[mb] *= alpha;
+          for (int mb = 0; mb < MB; ++mb) o[mb] *= alpha;
         }
       }
       float pr[8];
@@ -1168,7 +1235,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       // ---- O^T += V^T . P^T over the 32 tokens: the 8-bit transposing read hands lane c16 the
       // eight tokens of its group's k-slots for dim column 16 mb + c16
 #pragma unroll
-      for (int mb = 0; mb < 8; ++mb) {
+      for (int mb = 0; mb < MB; ++mb) {
         const i32x2 v8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(st + v8_read + (v8_y ^ (mb << 4))));
         const u32x4 vt = {QT::template from_fp8x2<false>(static_cast<u32>(v8[0])),
                           QT::template from_fp8x2<true>(static_cast<u32>(v8[0])),
@@ -1192,7 +1259,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         char* op = VL ? a.out + out_off + 4 * g * 2
                       : a.out + cc.b * a.out_stride_bytes + (static_cast<int64_t>(hq) * D + 4 * g) * 2;
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
+        for (int mb = 0; mb < MB; ++mb) {
           const u32x2 w = {QT::pack(o[mb][0] * inv, o[mb][1] * inv), QT::pack(o[mb][2] * inv, o[mb][3] * inv)};
           *reinterpret_cast<u32x2*>(op + mb * 32) = w;
         }
@@ -1200,7 +1267,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       if (head_on && !complete) {
         float* wp = a.ws_out + pidx * D + 4 * g;
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
+        for (int mb = 0; mb < MB; ++mb) {
           const f32x4 w = {o[mb][0] * inv, o[mb][1] * inv, o[mb][2] * inv, o[mb][3] * inv};
           *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
         }
@@ -1373,11 +1440,10 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
 
 constexpr int kMfmaStages = 4;
 
-template <typename QT, bool FP8, bool VL = false>
+template <typename QT, bool FP8, bool VL = false, int D = 128>
 int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
   using Lay = MfmaLayout<kMfmaStages>;
-  constexpr int D = 128;
-  auto kern = gqa_mfma_kernel<QT, FP8, kMfmaStages, VL>;
+  auto kern = gqa_mfma_kernel<QT, FP8, kMfmaStages, VL, D>;
   static std::atomic<uint64_t> configured{0};
   if (first_use_on_current_device(configured)) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1400,7 +1466,7 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   return static_cast<int>(hipGetLastError());
 }
 
-// Which kernel serves head_dim 128 with 16-bit pages and a power-of-two block size: the
+// Which kernel serves head_dim 128 (or 64 with 16-bit pages) and a power-of-two block size: the
 // matrix-core one ("mfma", default) or the dot-product one ("rows").
 bool use_mfma_kernel() {
   static const bool v = [] {
@@ -1438,6 +1504,8 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
     const bool out_aligned = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
     if (head_dim == 128 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
       return launch_gqa_mfma<QT, false>(a, wsb, s, plan_only, need);
+    if (head_dim == 64 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
+      return launch_gqa_mfma<QT, false, false, 64>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, false, 64, 8, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, false, 128, 16, 4>(a, wsb, s, plan_only, need);
