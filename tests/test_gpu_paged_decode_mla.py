@@ -258,6 +258,83 @@ def test_step_captured_in_a_graph_follows_new_metadata(device):
         assert_close_to_reference(replayed.view(cfg.batch, cfg.n_q_heads, 512), ref, f"mla graph replay {rep}")
 
 
+def test_absorbed_attention_layer_captured_in_a_graph(device):
+    # The decode branch of the reference's absorbed MLA attention (layers/dcu/deepseek_v2_attention.cpp:221-263,
+    # 428-432) as one captured step: q_nope . w_kc, latent store, dense decode, output . w_vc -- replayed over
+    # rewritten persistent buffers with eager work between the replays, every replay equal to the eager step bit
+    # for bit and within the path's tolerance of the same chain on the oracle.  16 heads: a tensor-parallel shard.
+    H = 16
+    cfg = _mla_cfg("layer", 5, H, 100, 1500)
+    g = torch.Generator().manual_seed(77)
+    w_kc = (torch.randn(H, 128, 512, generator=g) / math.sqrt(128)).bfloat16()
+    w_vc = (torch.randn(H, 512, 128, generator=g) / math.sqrt(512)).bfloat16()
+    inputs = [workloads.make_inputs(cfg, 500 + i) for i in range(2)]
+    qs = [(0.5 * torch.randn(cfg.batch, H, 192, generator=g)).bfloat16() for _ in inputs]
+    width = max(inp.layout.block_table.shape[1] for inp in inputs)
+    blocks = max(inp.layout.num_blocks for inp in inputs)
+    k_cache = torch.zeros(blocks, cfg.block_size, 1, 576, dtype=torch.bfloat16, device=device)
+    table = torch.zeros(cfg.batch, width, dtype=torch.int32, device=device)
+    lens = torch.zeros(cfg.batch, dtype=torch.int32, device=device)
+    slots = torch.zeros(cfg.batch, dtype=torch.int32, device=device)
+    q = torch.zeros(cfg.batch, H, 192, dtype=torch.bfloat16, device=device)
+    q_pe = torch.zeros(cfg.batch, 1, H, 64, dtype=torch.bfloat16, device=device)
+    q_abs = torch.zeros(cfg.batch, H, 512, dtype=torch.bfloat16, device=device)
+    proj = torch.zeros(cfg.batch, H, 128, dtype=torch.bfloat16, device=device)
+    k_new = torch.zeros(cfg.batch, 1, 576, dtype=torch.bfloat16, device=device)
+    wk, wv = w_kc.to(device), w_vc.to(device)
+
+    def load(inp, qi):
+        lay = inp.layout
+        k_cache.zero_()
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=inp.k_ctx.to(device), value=None, k_cache=k_cache,
+                                                            v_cache=None, slot_mapping=lay.ctx_slots.to(device)))
+        table.zero_()
+        table[:, : lay.block_table.shape[1]] = lay.block_table.to(device)
+        lens.copy_(lay.seq_lens.to(device))
+        slots.copy_(lay.new_slots.to(device))
+        q.copy_(qi.to(device))
+        q_pe.copy_(qi[:, :, 128:].reshape(cfg.batch, 1, H, 64).to(device))
+        k_new.copy_(inp.k_new.to(device))
+
+    def step():
+        ops.absorbed_bmm(q[:, :, :128], wk, out=q_abs)
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=k_new, value=None, k_cache=k_cache, v_cache=None,
+                                                            slot_mapping=slots))
+        p = ops.DenseDecodeParams(q_nope=q_abs.view(cfg.batch, 1, H, 512), q_pe=q_pe, k_cache=k_cache, seqlens_k=lens,
+                                  block_table=table, head_size_v=512, softmax_scale=cfg.scale)
+        att = ops.dense_decode(p, max_seq_len=width * cfg.block_size)
+        ops.absorbed_bmm(att.view(cfg.batch, H, 512), wv, out=proj)
+
+    load(inputs[0], qs[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture: workspace allocation, kernel attributes
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(4):
+        inp, qi = inputs[rep % 2], qs[rep % 2]
+        load(inp, qi)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = proj.clone()
+        load(inp, qi)
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, proj), f"replay {rep}"
+        kc, _ = fill_caches_cpu(inp)
+        lay = inp.layout
+        qa, _ = oracle.absorbed_bmm(qi[:, :, :128], w_kc)
+        att = oracle.aten_paged_decode(torch.cat([qa, qi[:, :, 128:]], dim=-1), kc, None, lay.block_table, lay.seq_lens,
+                                       cfg.scale, dv=512)
+        _, want = oracle.absorbed_bmm(att, w_vc)
+        assert_close_to_reference(replayed, want, f"absorbed layer replay {rep}")
+
+
 def _bmm_case(T, H, K, N, seed, wide=0):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(T, H, K + wide, generator=g).bfloat16()
