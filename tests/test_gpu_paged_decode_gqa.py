@@ -485,3 +485,81 @@ def test_step_captured_in_a_graph_follows_new_metadata(device):
         lay = inp.layout
         ref = oracle.aten_paged_decode(inp.q, kc[: blocks], vc[: blocks], lay.block_table, lay.seq_lens, cfg.scale)
         assert_close_to_reference(replayed, ref, f"graph replay {rep}")
+
+
+def test_norm_rope_cache_write_and_decode_captured_in_a_graph(device):
+    # The attention layer's decode step as the reference runs it (layers/common/qwen2_attention.cpp:144-186 then the
+    # attention op): fused q/k norm + RoPE on the qkv buffer with the cache write folded in, then the paged decode
+    # reading q as a strided view of that buffer.  Captured once, replayed over rewritten buffers, every replay
+    # equal to the eager step bit for bit and within the path's tolerance of the same chain on the oracle.
+    cfg = workloads.DecodeConfig("layer", 9, 32, 8, 128, 16, 50, 1200)
+    Hq, Hkv, D, B = cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.batch
+    g = torch.Generator().manual_seed(9)
+    qw, kw = (1 + 0.1 * torch.randn(D, generator=g)).bfloat16(), (1 + 0.1 * torch.randn(D, generator=g)).bfloat16()
+    ang = torch.rand(2048, D // 2, generator=g) * 6.28
+    cos_sin = torch.cat([ang.cos(), ang.sin()], 1)
+    inputs = [workloads.make_inputs(cfg, 600 + i) for i in range(2)]
+    raws = [torch.cat([inp.q.reshape(B, -1), inp.k_new.reshape(B, -1), inp.v_new.reshape(B, -1)], 1).contiguous() for inp in inputs]
+    width = max(inp.layout.block_table.shape[1] for inp in inputs)
+    blocks = max(inp.layout.num_blocks for inp in inputs)
+    k_cache = torch.zeros(blocks, cfg.block_size, Hkv, D, dtype=torch.bfloat16, device=device)
+    v_cache = torch.zeros_like(k_cache)
+    table = torch.zeros(B, width, dtype=torch.int32, device=device)
+    lens = torch.zeros(B, dtype=torch.int32, device=device)
+    slots = torch.zeros(B, dtype=torch.int32, device=device)
+    pos = torch.zeros(B, dtype=torch.int64, device=device)
+    qkv = torch.zeros(B, (Hq + 2 * Hkv) * D, dtype=torch.bfloat16, device=device)
+    out = torch.zeros(B, Hq, D, dtype=torch.bfloat16, device=device)
+    qwd, kwd, csd = qw.to(device), kw.to(device), cos_sin.to(device)
+
+    def load(inp, raw):
+        lay = inp.layout
+        k_cache.zero_()
+        v_cache.zero_()
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(
+            key=inp.k_ctx.to(device), value=inp.v_ctx.to(device), k_cache=k_cache, v_cache=v_cache,
+            slot_mapping=lay.ctx_slots.to(device)))
+        table.zero_()
+        table[:, : lay.block_table.shape[1]] = lay.block_table.to(device)
+        lens.copy_(lay.seq_lens.to(device))
+        slots.copy_(lay.new_slots.to(device))
+        pos.copy_((lay.seq_lens - 1).long().to(device))
+        qkv.copy_(raw.to(device))
+
+    def step():
+        ops.fused_qk_norm_rope(qkv, Hq, Hkv, Hkv, D, 1e-6, qwd, kwd, csd, False, pos, k_cache=k_cache, v_cache=v_cache,
+                               slot_mapping=slots)
+        ops.batch_decode(qkv[:, : Hq * D].view(B, Hq, D), k_cache, out, table, lens, v_cache=v_cache, scale=cfg.scale,
+                         max_seq_len=width * cfg.block_size)
+
+    load(inputs[0], raws[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture: workspace allocation, kernel attributes
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(4):
+        inp, raw = inputs[rep % 2], raws[rep % 2]
+        load(inp, raw)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out.clone()
+        out.zero_()
+        load(inp, raw)
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, out), f"replay {rep}"
+        lay = inp.layout
+        want = oracle.fused_qk_norm_rope(raw, Hq, Hkv, Hkv, D, 1e-6, qw, kw, cos_sin, False, (lay.seq_lens - 1).long())
+        kc, vc = fill_caches_cpu(inp)
+        new = lay.new_slots.long()
+        kc.view(-1, Hkv, D)[new] = want[:, Hq * D : (Hq + Hkv) * D].view(B, Hkv, D)
+        vc.view(-1, Hkv, D)[new] = want[:, (Hq + Hkv) * D :].view(B, Hkv, D)
+        ref = oracle.aten_paged_decode(want[:, : Hq * D].view(B, Hq, D).contiguous(), kc, vc, lay.block_table, lay.seq_lens,
+                                       cfg.scale)
+        assert_close_to_reference(replayed, ref, f"layer step replay {rep}")
