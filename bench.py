@@ -27,7 +27,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="llama3_8b",
-                    help="tiny | llama3_8b | long_b256 | fp8_kv | mla_dsv3")
+                    help="tiny | llama3_8b | long_b256 | fp8_kv | mla_dsv3 (the five configurations); gqa_d64 | mla_tp8 (side workloads)")
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
@@ -248,7 +248,14 @@ def main():
             traffic = json.load(f).get(args.workload, {}).get("hbm_bytes_per_launch")
     except (OSError, ValueError):
         pass
-    if cfg.mla:
+    if cfg.mla and cfg.n_q_heads <= 64:
+        # the few heads of a tensor-parallel shard: 30-120 flop per cache byte, far below the ridge: HBM bound
+        nbytes, flops = workloads.mla_bytes_flops(cfg, lay.seq_lens)
+        achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": "mla_decode16_kernel",
+                    "kernel_ms": kernel_ms, "algorithmic_bytes": nbytes, "algorithmic_flops": flops}
+    elif cfg.mla:
         nbytes, flops = workloads.mla_bytes_flops(cfg, lay.seq_lens)
         achieved = flops / (kernel_ms * 1e-3) / 1e12
         roofline = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
