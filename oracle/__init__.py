@@ -71,10 +71,13 @@ def c_lib():
 
 
 def aten_lib():
-    """The ATen-op-order oracle, built on first use if missing or older than its source."""
+    """The ATen-op-order oracle, built on first use if missing (a minute of compilation: a stale one is
+    rebuilt by the build step, not inside a test)."""
     global _aten
     if _aten is None:
-        path = _build.build_aten(force=False)
+        path = _build.ATEN_LIB
+        if not os.path.exists(path):
+            _build.build_aten()
         lib = ctypes.CDLL(path)
         lib.aten_oracle_num_threads.restype = _i32
         lib.aten_oracle_set_num_threads.argtypes = [_i32]
