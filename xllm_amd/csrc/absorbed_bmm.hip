@@ -122,7 +122,8 @@ __global__ __launch_bounds__(kBmmThreads) void absorbed_bmm_kernel(BmmArgs a) {
       const int row = half * 8 + (lane >> 3);
       const int t = t0 + i * 16 + row;
       const u32x4 v = *reinterpret_cast<const u32x4*>(mine + row * kBmmRow + (lane & 7) * 16);
-      if (t < a.n_tokens) stg16(a.y + t * a.y_token_stride + h * a.y_head_stride + n0 * 2 + (lane & 7) * 16, v);
+      if (t < a.n_tokens)
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(a.y + t * a.y_token_stride + h * a.y_head_stride + n0 * 2 + (lane & 7) * 16));
     }
   }
 }
