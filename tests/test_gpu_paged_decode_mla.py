@@ -350,6 +350,8 @@ def _bmm_case(T, H, K, N, seed, wide=0):
     (100, 4, 128, 128, 0),     # two token blocks per wavefront, the second one ragged
     (200, 3, 128, 64, 8),      # four token blocks per wavefront
     (700, 2, 256, 64, 0),      # several workgroups along the tokens
+    (300, 4, 128, 512, 64),    # many tokens: 128 output columns per workgroup
+    (261, 3, 512, 128, 0),
 ])
 def test_absorbed_products_either_side_of_the_decode(device, T, H, K, N, wide):
     # bmm(x.transpose(0, 1), w).transpose(0, 1) of layers/dcu/deepseek_v2_attention.cpp:428-430 and 231-238.
