@@ -669,11 +669,10 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
     for (int sub = 0; sub < n_sub; ++sub) {
       wait_younger_subs(min(kRing16 - 2, n_sub - 1 - sub));
       __syncthreads();  // this sub-tile has landed in LDS; every wavefront is past the previous one
-      // Wavefronts 0-3 issue their rows of sub-tile sub + 3 (into the slot released just now)
-      // before they compute, wavefronts 4-7 (the second wavefront of each SIMD) after: the phases
-      // of the two groups then interleave instead of all eight hitting LDS at the same time.
-      const bool early = wave < 4;
-      if (early && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
+      // Every wavefront issues its rows of sub-tile sub + 3 (into the slot released just now) before it
+      // computes.  (With 8 loads per wavefront it paid to let the second wavefront of each SIMD issue after
+      // its arithmetic; with 5 it no longer does.)
+      if (sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
       const char* kb = smem + (sub & (kRing16 - 1)) * kSubBytes;
       if (wave_ok) {
         // rope k-steps: row c16 of the rope area, chunk (kk - 16) * 4 + g XOR-ed with the low 3 bits of the row
@@ -818,7 +817,6 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      if (!early && sub + kRing16 - 1 < n_sub) issue_sub(sub + kRing16 - 1);
     }
 
     if constexpr (SPLIT) {
