@@ -87,3 +87,18 @@ def test_python_ops_refuse_cpu_tensors():
     with pytest.raises(ValueError):
         ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=k, value=k, k_cache=cache, v_cache=cache,
                                                             slot_mapping=torch.zeros(2, dtype=torch.int32)))
+    # every op of the mirror refuses host tensors: there is no CPU path behind it
+    x = torch.zeros(2, 4, 128, dtype=torch.bfloat16)
+    w = torch.zeros(4, 128, 64, dtype=torch.bfloat16)
+    table = torch.zeros(2, 3, dtype=torch.int32)
+    lens = torch.ones(2, dtype=torch.int32)
+    qkv = torch.zeros(2, 6 * 64, dtype=torch.bfloat16)
+    for call in (lambda: ops.absorbed_bmm(x, w),
+                 lambda: ops.mask_block_table_padding(table, lens, 16),
+                 lambda: ops.fused_qk_norm_rope(qkv, 4, 1, 1, 64, 1e-6, torch.ones(64, dtype=torch.bfloat16),
+                                                torch.ones(64, dtype=torch.bfloat16), torch.zeros(8, 64), False,
+                                                torch.zeros(2, dtype=torch.int64)),
+                 lambda: ops.gather_mla_latent_cache(torch.zeros(1, 16, 1, 576, dtype=torch.bfloat16), table,
+                                                     torch.zeros(3, dtype=torch.int32), 4)):
+        with pytest.raises(ValueError):
+            call()
