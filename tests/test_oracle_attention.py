@@ -305,3 +305,57 @@ def test_absorbed_bmm_oracle_against_loops_and_selections():
     y_slice, _ = oracle.absorbed_bmm(q[..., :K], w)
     ref = torch.bmm(q[..., :K].float().transpose(0, 1), w.float()).transpose(0, 1)
     assert torch.equal(y_slice, ref.bfloat16())
+
+
+def test_fp8_dequant_branch_of_both_oracles():
+    """Decode on an fp8 cache with per-head scales must equal, bit for bit, decode on a 16-bit cache that
+    holds (decode_table[code] * scale[h]).to(q dtype): the dequantisation rule stated for the fp8 pages
+    (the int8 precedent of xllm/core/layers/mlu/attention.cpp:171-222).  A scale applied to the wrong head,
+    taken from the other tensor, squared or dropped changes the 16-bit cache and fails the comparison."""
+    cfg = workloads.DecodeConfig("fp8pin", 3, 8, 4, 128, 16, 33, 150)
+    inp = workloads.make_inputs(cfg, 21)
+    lay = inp.layout
+    k_scale = oracle.kv_head_scales(torch.cat([inp.k_ctx, inp.k_new]))
+    v_scale = oracle.kv_head_scales(torch.cat([inp.v_ctx, inp.v_new])) * 1.5   # K and V scales differ per head
+    assert len(set(k_scale.tolist())) == cfg.n_kv_heads and not torch.equal(k_scale, v_scale)
+    kc8, vc8 = fill_caches_cpu(inp, torch.uint8, k_scale, v_scale)
+    table = oracle.fp8_decode_table()
+    for dt in (torch.bfloat16, torch.float16):
+        q = inp.q.to(dt)
+        kc16 = (table[kc8.long()] * k_scale.view(1, 1, -1, 1)).to(dt)
+        vc16 = (table[vc8.long()] * v_scale.view(1, 1, -1, 1)).to(dt)
+        a8 = oracle.aten_paged_decode(q, kc8, vc8, lay.block_table, lay.seq_lens, cfg.scale, k_scale, v_scale)
+        a16 = oracle.aten_paged_decode(q, kc16, vc16, lay.block_table, lay.seq_lens, cfg.scale)
+        assert torch.equal(a8.view(torch.int16), a16.view(torch.int16))
+        f8, l8 = oracle.paged_decode_f64(q, kc8, vc8, lay.block_table, lay.seq_lens, cfg.scale, k_scale, v_scale)
+        f16, l16 = oracle.paged_decode_f64(q, kc16, vc16, lay.block_table, lay.seq_lens, cfg.scale)
+        assert torch.equal(f8, f16) and torch.equal(l8, l16)
+        lse8 = oracle.aten_paged_decode_lse(q, kc8, lay.block_table, lay.seq_lens, cfg.scale, k_scale)
+        lse16 = oracle.aten_paged_decode_lse(q, kc16, lay.block_table, lay.seq_lens, cfg.scale)
+        assert torch.equal(lse8, lse16)
+    # the torch view of the same bytes is the same cache
+    a8v = oracle.aten_paged_decode(inp.q, kc8.view(torch.float8_e4m3fn), vc8.view(torch.float8_e4m3fn),
+                                   lay.block_table, lay.seq_lens, cfg.scale, k_scale, v_scale)
+    a8u = oracle.aten_paged_decode(inp.q, kc8, vc8, lay.block_table, lay.seq_lens, cfg.scale, k_scale, v_scale)
+    assert torch.equal(a8v, a8u)
+
+
+def test_fp8_decode_known_answer():
+    """All codes 0x38 (= 1.0) in K and V, V scale 0.5: every score is equal, so the output is 0.5 exactly and
+    the LSE is log(L) + scale * k_scale * sum(q)."""
+    B, Hq, Hkv, D, bs, L = 2, 4, 2, 64, 16, 37
+    kc = torch.full((8, bs, Hkv, D), 0x38, dtype=torch.uint8)
+    vc = kc.clone()
+    q = torch.ones(B, Hq, D, dtype=torch.bfloat16)
+    table = torch.arange(8, dtype=torch.int32).view(2, 4)
+    lens = torch.tensor([L, 5], dtype=torch.int32)
+    ks = torch.tensor([2.0, 0.25])
+    vs = torch.tensor([0.5, 0.125])
+    out = oracle.aten_paged_decode(q, kc, vc, table, lens, 0.125, ks, vs)
+    out64, lse64 = oracle.paged_decode_f64(q, kc, vc, table, lens, 0.125, ks, vs)
+    for o in (out.float(), out64):
+        assert torch.all(o[:, :2] == 0.5) and torch.all(o[:, 2:] == 0.125)
+    expect = torch.log(lens.double()).view(2, 1) + 0.125 * D * ks.double().repeat_interleave(2).view(1, 4)
+    assert torch.allclose(lse64.double(), expect, atol=1e-5)
+    lse = oracle.aten_paged_decode_lse(q, kc, table, lens, 0.125, ks)
+    assert torch.allclose(lse.double(), expect, atol=1e-4)
