@@ -57,7 +57,8 @@ enum {
   XLLM_MI355_EDTYPE = -2,      /* dtype combination not implemented             */
   XLLM_MI355_ESHAPE = -3,      /* head_dim / group / block size not implemented */
   XLLM_MI355_EWORKSPACE = -4,  /* workspace missing or too small                */
-  XLLM_MI355_EALIGN = -5       /* pointer or stride not 16-byte aligned         */
+  XLLM_MI355_EALIGN = -5,      /* pointer or stride not 16-byte aligned         */
+  XLLM_MI355_ESTALLED = -6     /* xllm_mi355_decode_status: a bounded wait inside a decode kernel gave up */
 };
 
 /* Human-readable text for a return code of this library (host pointer, static). */
@@ -109,6 +110,33 @@ int xllm_mi355_kv_head_scales(const void* x, float* scales,
  */
 size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads,
                                                int64_t v_head_dim, int64_t max_seq_len);
+
+/*
+ * The decode workspace.  Counterpart of the process-wide FlashInfer workspace of the reference
+ * (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41: allocated once, handed to every layer's decode call).
+ * Layout, the same for every decode entry point and independent of the batch, so that a launch recorded in a
+ * HIP graph keeps meaning the same addresses whatever later calls ask for:
+ *     256 bytes of header (word 0: status flags) | item prefix of up to 2048 sequences | fp32 partial slots
+ * xllm_mi355_decode_workspace_bound() is a size that serves every GQA call, MLA calls with up to 1024 heads and
+ * varlen calls of up to 65536 query tokens (about 135 MB on a GPU with 256 CUs): allocate that much once per
+ * device and never replace it while graphs that captured a decode call are alive.
+ * xllm_mi355_decode_workspace_init clears the header; call it once after allocating (it is a small fill kernel
+ * on `stream`, legal under capture).
+ * ONE workspace serves ONE stream at a time: two decode calls that use the same workspace and overlap in time
+ * (two streams of one device, or two graphs replayed concurrently) overwrite each other's partial results.
+ * Give every stream that decodes concurrently a workspace of its own.  The reference has the same rule: its
+ * workspace is a per-process singleton used from the one worker thread and stream of a device.
+ *
+ * xllm_mi355_decode_status is the voice of the kernels: the wavefronts of the matrix-core GQA kernel wait for
+ * each other with bounded polls; if a poll ever runs out, the wavefront sets a flag in the header and exits,
+ * and the outputs of that launch are invalid.  The call waits for `stream`, reads the flag from the host and
+ * clears it: 0 = no launch since the last call gave up, XLLM_MI355_ESTALLED otherwise.  It synchronises, so it
+ * is for use outside graph capture (for example once per step, or when a result looks wrong).  The reference
+ * has no counterpart (its fast paths are closed libraries that abort on error).
+ */
+size_t xllm_mi355_decode_workspace_bound(void);
+int xllm_mi355_decode_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+int xllm_mi355_decode_status(void* workspace, void* stream);
 
 /*
  * Paged decode attention, GQA, block-table addressing.
@@ -203,7 +231,8 @@ int xllm_mi355_mla_absorbed_bmm(const void* x, const void* w, void* y,
  * are read once per 16 / (Hq / Hkv) query tokens, and a chunk longer than the bound is cut to it.  Otherwise
  * every query token is decoded as an entry of its own against its sequence's pages (read once per token,
  * partly from L2), which is correct for any length.
- * Workspace: xllm_mi355_paged_decode_varlen_workspace_bytes(max(n_tokens, batch), ...).
+ * Workspace: xllm_mi355_paged_decode_varlen_workspace_bytes(max(n_tokens, batch), ...); the per-token arrays
+ * take its last bytes, so pass the same workspace_bytes on every call that shares a captured graph.
  */
 size_t xllm_mi355_paged_decode_varlen_workspace_bytes(int64_t n_tokens, int64_t n_q_heads,
                                                       int64_t head_dim);
@@ -342,6 +371,16 @@ int xllm_mi355_decode_metadata_update(const int32_t* src_tokens, const int32_t* 
  */
 int xllm_mi355_profile_enable(int capacity);
 int xllm_mi355_profile_collect(float* ms_out, int max_n);
+
+/*
+ * Test hooks.  No counterpart in the reference.  XLLM_MI355_DEBUG_WAIT_SPINS: the bound of the polls described
+ * at xllm_mi355_decode_status (negative = default, 2^22; 0 makes the first wait of a launch give up, which is
+ * how the status path is tested: every wavefront still exits normally).  XLLM_MI355_DEBUG_MLA_KERNEL: the MLA
+ * kernel choice, as the first letter of the environment variable XLLM_MI355_MLA_KERNEL, which the library reads
+ * once per process (0 default, 'p' pairs, 's' split).
+ */
+enum { XLLM_MI355_DEBUG_WAIT_SPINS = 0, XLLM_MI355_DEBUG_MLA_KERNEL = 1 };
+int xllm_mi355_debug_set(int what, int value);
 
 /*
  * Plain streaming kernels of known size, the yardstick for the decode kernels.  No

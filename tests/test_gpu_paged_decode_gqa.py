@@ -563,3 +563,62 @@ def test_norm_rope_cache_write_and_decode_captured_in_a_graph(device):
         ref = oracle.aten_paged_decode(want[:, : Hq * D].view(B, Hq, D).contiguous(), kc, vc, lay.block_table, lay.seq_lens,
                                        cfg.scale)
         assert_close_to_reference(replayed, ref, f"layer step replay {rep}")
+
+
+def test_graph_captured_at_a_small_batch_survives_a_larger_eager_call(device):
+    """The workspace is allocated once and its layout does not depend on the batch: a graph captured at batch 32
+    replays correctly after an eager call at batch 128 (and after MLA and varlen calls) has used the same
+    workspace."""
+    small = workloads.DecodeConfig("ws_small", 32, 32, 8, 128, 16, 600, 2500)
+    large = workloads.DecodeConfig("ws_large", 128, 32, 8, 128, 16, 600, 2500)
+    inp_s, inp_l = workloads.make_inputs(small, 31), workloads.make_inputs(large, 32)
+    ks_, vs_, _, _ = fill_caches_gpu(inp_s, device)
+    kl_, vl_, _, _ = fill_caches_gpu(inp_l, device)
+    q = inp_s.q.to(device)
+    table, lens = inp_s.layout.block_table.to(device), inp_s.layout.seq_lens.to(device)
+    out = torch.empty_like(q)
+    eager, _ = _decode_gpu(inp_s, ks_, vs_, device)
+    ws_before = ops.decode_workspace(device, 0).data_ptr()
+    side = torch.cuda.Stream(device)
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        ops.batch_decode(q, ks_, out, table, lens, v_cache=vs_, scale=small.scale, max_seq_len=2500)  # warm-up
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            ops.batch_decode(q, ks_, out, table, lens, v_cache=vs_, scale=small.scale, max_seq_len=2500)
+    torch.cuda.current_stream(device).wait_stream(side)
+    torch.cuda.synchronize()
+    for _ in range(2):
+        big, _ = _decode_gpu(inp_l, kl_, vl_, device)
+        ref = oracle.aten_paged_decode(inp_l.q[:4].contiguous(), kl_.cpu(), vl_.cpu(), inp_l.layout.block_table[:4].contiguous(),
+                                       inp_l.layout.seq_lens[:4].contiguous(), large.scale)
+        assert_close_to_reference(big[:4], ref, "large eager")
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+    assert ops.decode_workspace(device, 0).data_ptr() == ws_before
+    with pytest.raises(RuntimeError):
+        ops.decode_workspace(device, 1 << 40)
+
+
+def test_a_wait_that_gives_up_is_reported(device):
+    """With the poll bound at zero the first wait of a wavefront on its partner gives up: every wavefront still
+    exits normally, the launch returns, and xllm_mi355_decode_status reports it once."""
+    from xllm_amd import capi
+    lib = capi.lib()
+    cfg = workloads.DecodeConfig("stall", 8, 32, 8, 128, 16, 400, 1200)
+    inp = workloads.make_inputs(cfg, 5)
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    good, _ = _decode_gpu(inp, kg, vg, device)
+    assert ops.decode_status(device) == 0
+    try:
+        assert lib.xllm_mi355_debug_set(0, 0) == 0
+        _decode_gpu(inp, kg, vg, device)
+    finally:
+        assert lib.xllm_mi355_debug_set(0, -1) == 0
+    with pytest.raises(capi.XllmMi355Error, match="gave up"):
+        ops.decode_status(device)
+    assert ops.decode_status(device) == 0   # reported once, then cleared
+    again, _ = _decode_gpu(inp, kg, vg, device)
+    assert torch.equal(again, good) and ops.decode_status(device) == 0

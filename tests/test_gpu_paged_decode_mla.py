@@ -58,13 +58,21 @@ def test_head_counts_of_tp_shards_and_reference_test_shape(device):
         _check(_mla_cfg(f"mla{heads}", 2, heads, 1, 400), 40 + heads, device)
 
 
-def test_batches_larger_than_a_workgroup_and_than_a_launch(device, monkeypatch):
+def _select_kernel(name):
+    """The MLA kernel choice (the library reads the environment variable once per process)."""
+    from xllm_amd import capi
+    assert capi.lib().xllm_mi355_debug_set(1, ord(name[0]) if name else 0) == 0
+
+
+def test_batches_larger_than_a_workgroup_and_than_a_launch(device):
     # more sequences than threads in a workgroup (several per thread in the tile prefix) and more than one launch
     # holds (1024), in all three kernels
     for knob in ("", "pairs", "split"):
-        monkeypatch.setenv("XLLM_MI355_MLA_KERNEL", knob)
-        _check(_mla_cfg(f"mla_b600_{knob}", 600, 16, 1, 150), 90, device)
-    monkeypatch.delenv("XLLM_MI355_MLA_KERNEL")
+        _select_kernel(knob)
+        try:
+            _check(_mla_cfg(f"mla_b600_{knob}", 600, 16, 1, 150), 90, device)
+        finally:
+            _select_kernel("")
     _check(_mla_cfg("mla_b1100", 1100, 8, 1, 80), 91, device)
 
 
@@ -140,9 +148,16 @@ def test_scores_that_rise_along_the_context(device):
         assert torch.allclose(lse.cpu(), ref_lse, rtol=1e-3, atol=1e-3)
 
 
-def test_producer_consumer_kernel(device, monkeypatch):
+def test_producer_consumer_kernel(device):
     # the kernel with the two products on different wavefronts, selected by the tuning knob
-    monkeypatch.setenv("XLLM_MI355_MLA_KERNEL", "split")
+    _select_kernel("split")
+    try:
+        _producer_consumer_cases(device)
+    finally:
+        _select_kernel("")
+
+
+def _producer_consumer_cases(device):
     _check(_mla_cfg("split128", 3, 128, 100, 1500), 5, device)
     for heads in (2, 16, 80):
         _check(_mla_cfg(f"split{heads}", 2, heads, 1, 400), 60 + heads, device)

@@ -3,6 +3,15 @@
 
 using namespace xllm_mi355;
 
+namespace xllm_mi355 {
+namespace {
+constexpr int kDefaultWaitSpins = 1 << 22;
+std::atomic<int> g_wait_spins{kDefaultWaitSpins};
+}  // namespace
+int wait_spin_limit() { return g_wait_spins.load(std::memory_order_relaxed); }
+void set_mla_kernel_knob(int first_letter);  // paged_decode_mla.hip
+}  // namespace xllm_mi355
+
 extern "C" {
 
 const char* xllm_mi355_version(void) { return "0.1.0"; }
@@ -15,6 +24,7 @@ const char* xllm_mi355_error_string(int code) {
     case XLLM_MI355_ESHAPE: return "head dim, group size or block size not implemented";
     case XLLM_MI355_EWORKSPACE: return "split-K workspace missing, misaligned or too small";
     case XLLM_MI355_EALIGN: return "pointer or stride not 16-byte aligned";
+    case XLLM_MI355_ESTALLED: return "a bounded wait inside a decode kernel gave up: the outputs of that launch are invalid";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -44,6 +54,39 @@ size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads,
   // 512 is the latent width of the MLA kernel; every other width is a GQA head dim
   if (v_head_dim == 512) return mla_workspace_bytes(batch, n_q_heads, max_seq_len);
   return gqa_workspace_bytes(batch, n_q_heads, v_head_dim);
+}
+
+size_t xllm_mi355_decode_workspace_bound(void) { return decode_workspace_bound(); }
+
+int xllm_mi355_decode_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+  return decode_workspace_init(workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_decode_status(void* workspace, void* stream) {
+  if (workspace == nullptr) return XLLM_MI355_EINVAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int status = 0;
+  hipError_t e = hipMemcpyAsync(&status, workspace, sizeof(int), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (status == 0) return XLLM_MI355_OK;
+  const int zero = 0;
+  e = hipMemcpyAsync(workspace, &zero, sizeof(int), hipMemcpyHostToDevice, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return static_cast<int>(e);
+  return XLLM_MI355_ESTALLED;
+}
+
+int xllm_mi355_debug_set(int what, int value) {
+  switch (what) {
+    case XLLM_MI355_DEBUG_WAIT_SPINS:
+      g_wait_spins.store(value < 0 ? kDefaultWaitSpins : value, std::memory_order_relaxed);
+      return XLLM_MI355_OK;
+    case XLLM_MI355_DEBUG_MLA_KERNEL:
+      set_mla_kernel_knob(value);
+      return XLLM_MI355_OK;
+    default: return XLLM_MI355_EINVAL;
+  }
 }
 
 int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out,
@@ -108,7 +151,7 @@ int xllm_mi355_mla_absorbed_bmm(const void* x, const void* w, void* y, int64_t n
 
 size_t xllm_mi355_paged_decode_varlen_workspace_bytes(int64_t n_tokens, int64_t n_q_heads, int64_t head_dim) {
   if (n_tokens <= 0 || n_q_heads <= 0 || head_dim <= 0) return 0;
-  return varlen_extra_bytes(n_tokens) + gqa_workspace_bytes(n_tokens, n_q_heads, head_dim);
+  return gqa_workspace_bytes(n_tokens, n_q_heads, head_dim) + varlen_extra_bytes(n_tokens) + 256;
 }
 
 int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_cache, void* out,

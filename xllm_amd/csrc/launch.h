@@ -38,10 +38,28 @@ struct PageAddressing {
   const int32_t* last_page_len = nullptr;
 };
 
-// Workspace bytes of the GQA decode (item prefix + two partial slots per persistent workgroup).
+// Layout of a decode workspace, the same for every decode entry point and independent of the batch, so that
+// a launch recorded in a HIP graph keeps meaning the same addresses whatever later calls ask for:
+//   [0, kWsHeaderBytes)                 header: word 0 = status flags (kStatus*), the rest reserved
+//   [kWsHeaderBytes, kWsPartialsOff)    item prefix of up to kWsMaxBatch sequences per launch
+//   [kWsPartialsOff, ...)               two fp32 partial slots per persistent worker
+//   the last varlen_extra_bytes(n)      per-token lengths and table rows of the varlen entry point
+constexpr size_t kWsHeaderBytes = 256;
+constexpr int kWsMaxBatch = 2048;
+constexpr size_t kWsPartialsOff = kWsHeaderBytes + (static_cast<size_t>(kWsMaxBatch + 1) * 4 + 255) / 256 * 256;
+constexpr int kStatusWaitGaveUp = 1;  // a bounded wait of one wavefront on another ran out: the launch's output is invalid
+
+// Bound of the polls of one wavefront on another (test hook: xllm_mi355_debug_set_wait_spins).
+int wait_spin_limit();
+
+// Workspace bytes of the GQA decode (header + item prefix + two partial slots per persistent worker).
 size_t gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim);
-// Workspace bytes of the MLA decode for an upper bound of the context length.
+// Workspace bytes of the MLA decode.
 size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len);
+// Bytes that serve every GQA call, MLA calls with up to 1024 heads and varlen calls of up to 65536 query tokens.
+size_t decode_workspace_bound();
+// Clears the header of a workspace (a fill kernel: legal under graph capture).
+int decode_workspace_init(void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out, float* lse,
                      const PageAddressing& addr, const float* k_scale, const float* v_scale,

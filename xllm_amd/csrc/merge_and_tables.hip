@@ -216,6 +216,28 @@ int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t tab
   return static_cast<int>(hipGetLastError());
 }
 
+namespace {
+__global__ __launch_bounds__(64) void clear_words_kernel(int* p, int n) {
+  if (static_cast<int>(threadIdx.x) < n) p[threadIdx.x] = 0;
+}
+}  // namespace
+
+int decode_workspace_init(void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 || workspace_bytes < kWsHeaderBytes)
+    return XLLM_MI355_EWORKSPACE;
+  clear_words_kernel<<<dim3(1), 64, 0, stream>>>(static_cast<int*>(workspace), static_cast<int>(kWsHeaderBytes / 4));
+  return static_cast<int>(hipGetLastError());
+}
+
+size_t decode_workspace_bound() {
+  size_t need = gqa_workspace_bytes(1, 1, 256);
+  for (int64_t heads = 128; heads <= 1024; heads += 128) {
+    const size_t m = mla_workspace_bytes(1, heads, 0);
+    need = m > need ? m : need;
+  }
+  return need + varlen_extra_bytes(65536) + 256;
+}
+
 size_t varlen_extra_bytes(int64_t n_tokens) {
   return n_tokens <= 0 ? 0 : (static_cast<size_t>(n_tokens) * 2 * 4 + 255) / 256 * 256;
 }
@@ -257,11 +279,13 @@ int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_ca
                             n_kv_heads, head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
                             max_seq_len, sm_scale, workspace, workspace_bytes, q_dtype, cache_dtype, stream);
   }
-  // Otherwise every query token becomes a decode entry of its own.
+  // Otherwise every query token becomes a decode entry of its own; their lengths and table rows take the
+  // last bytes of the workspace (the header, prefix and partials keep their places at its start).
   const size_t extra = varlen_extra_bytes(n_tokens);
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 || workspace_bytes < extra)
     return XLLM_MI355_EWORKSPACE;
-  int32_t* tok_lens = static_cast<int32_t*>(workspace);
+  const size_t usable = (workspace_bytes - extra) / 256 * 256;
+  int32_t* tok_lens = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + usable);
   int32_t* tok_rows = tok_lens + n_tokens;
   const unsigned grid = static_cast<unsigned>((n_tokens + 255) / 256);
   expand_varlen_kernel<<<dim3(grid), 256, 0, stream>>>(cu_seqlens_q, kv_seq_lens, tok_lens, tok_rows,
@@ -275,8 +299,7 @@ int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_ca
   addr.table_rows = tok_rows;
   return paged_decode_gqa(q, k_cache, v_cache, out, nullptr, addr, k_scale, v_scale, n_tokens, n_q_heads,
                           n_kv_heads, head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
-                          max_seq_len, sm_scale, static_cast<char*>(workspace) + extra, workspace_bytes - extra,
-                          q_dtype, cache_dtype, stream);
+                          max_seq_len, sm_scale, workspace, usable, q_dtype, cache_dtype, stream);
 }
 
 int lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,

@@ -50,7 +50,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / kWave;
 constexpr int kItem = 64;      // tokens per schedulable item
 constexpr int kSub = 2048;     // tokens whose slot ids are staged in LDS at a time
-constexpr int kMaxBatch = 2048;  // sequences per launch (their item prefix lives in LDS)
+constexpr int kMaxBatch = kWsMaxBatch;  // sequences per launch (their item prefix lives in LDS)
 
 struct GqaArgs {
   const char* q;
@@ -70,6 +70,7 @@ struct GqaArgs {
   const int32_t* last_page_len;
   const float* k_scale;
   const float* v_scale;
+  int* ws_status;  // status flags of the workspace (kStatus*), only ever OR-ed into
   int* ws_prefix;  // [batch + 1] item prefix, written by workgroup 0 for the merge kernel
   float* ws_out;   // [2 * n_workgroups][G][D]
   float* ws_lse;   // [2 * n_workgroups][G]
@@ -86,6 +87,7 @@ struct GqaArgs {
   int bs_shift;       // log2(block_size) or -1
   int num_blocks;
   int n_workgroups;   // workers of the decode kernel (workgroups; wavefront pairs of the matrix-core kernel)
+  int wait_spins;     // bound of the polls of one wavefront of a pair on the other
   float scale_log2;   // sm_scale * log2(e)
 };
 
@@ -655,7 +657,6 @@ __device__ __forceinline__ void copy_cursor(CtxCursor& d, const CtxCursor& s) {
   }
 }
 
-constexpr int kPairSpins = 1 << 22;          // bound of every wait of one wavefront of a pair on the other
 constexpr int kMfmaThreads = 2 * kThreads;   // kWaves loading wavefronts and kWaves computing wavefronts
 
 template <int NS>
@@ -997,7 +998,11 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     for (int spin = 0; i - released >= NS; ++spin) {
       released = __builtin_amdgcn_readfirstlane(*freed);
       if (i - released < NS) break;
-      if (spin > kPairSpins) return;  // (never: the computing wavefront gives every slot back)
+      if (spin >= a.wait_spins) {  // (never in a correct run: the computing wavefront gives every slot back)
+        if (lane == 0) atomicOr(a.ws_status, kStatusWaitGaveUp);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stages in flight land before the LDS is handed back
+        return;
+      }
       __builtin_amdgcn_s_sleep(1);
     }
     issue_stage();
@@ -1030,7 +1035,10 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     for (int spin = 0; arrived <= s; ++spin) {
       arrived = __builtin_amdgcn_readfirstlane(*landed);
       if (arrived > s) break;
-      if (spin > kPairSpins) return;  // (never: the loading wavefront announces every stage)
+      if (spin >= a.wait_spins) {  // (never in a correct run: the loading wavefront announces every stage)
+        if (lane == 0) atomicOr(a.ws_status, kStatusWaitGaveUp);
+        return;
+      }
       __builtin_amdgcn_s_sleep(1);
     }
     asm volatile("" ::: "memory");  // no read of the stage moves above the poll
@@ -1427,12 +1435,11 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
     return n;
   }();
   a.n_workgroups = device_cu_count() * per_cu;
-  const size_t prefix_bytes = ((static_cast<size_t>(a.batch) + 1) * 4 + 255) / 256 * 256;
   const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * G * (D + 1);
-  *need = prefix_bytes + part_floats * 4;
+  *need = kWsPartialsOff + part_floats * 4;
   if (plan_only) return XLLM_MI355_OK;
   if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
-  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_prefix) + prefix_bytes);
+  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_status) + kWsPartialsOff);
   a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * G * D;
   launch_timed(kern, dim3(static_cast<unsigned>(a.n_workgroups)), dim3(kThreads), smem, stream, a);
   return static_cast<int>(hipGetLastError());
@@ -1454,12 +1461,11 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   a.g_block = kMfmaHeads;
   const int n_wg = device_cu_count();  // the ring fills a CU's LDS: one workgroup each
   a.n_workgroups = n_wg * kWaves;      // independent workers = wavefronts
-  const size_t prefix_bytes = ((static_cast<size_t>(a.batch) + 1) * 4 + 255) / 256 * 256;
   const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * (D + 1);
-  *need = prefix_bytes + part_floats * 4;
+  *need = kWsPartialsOff + part_floats * 4;
   if (plan_only) return XLLM_MI355_OK;
   if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
-  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_prefix) + prefix_bytes);
+  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_status) + kWsPartialsOff);
   a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
   const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 1) * 4;
   launch_timed(kern, dim3(static_cast<unsigned>(n_wg)), dim3(kMfmaThreads), smem, stream, a);
@@ -1525,11 +1531,11 @@ int group_block(int group) {
 }  // namespace
 
 size_t gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim) {
-  // Upper bound over every kernel variant: at most 8 workgroups per CU, 8 heads per block.
+  // Upper bound over every kernel variant, independent of the batch: at most 8 workgroups per CU, 8 heads
+  // per block (the matrix-core kernel: 4 workers per CU, 16 heads).
+  (void)batch;
   (void)n_q_heads;
-  const size_t b = static_cast<size_t>(batch < kMaxBatch ? batch : kMaxBatch);
-  const size_t prefix_bytes = ((b + 1) * 4 + 255) / 256 * 256;
-  return prefix_bytes + static_cast<size_t>(device_cu_count()) * 8 * 2 * 8 * (head_dim + 1) * 4;
+  return kWsPartialsOff + static_cast<size_t>(device_cu_count()) * 8 * 2 * 8 * (head_dim + 1) * 4;
 }
 
 int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out, float* lse,
@@ -1593,7 +1599,9 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     a.last_page_len = csr ? addr.last_page_len + b0 : nullptr;
     a.k_scale = k_scale;
     a.v_scale = v_scale;
-    a.ws_prefix = static_cast<int*>(workspace);
+    a.ws_status = static_cast<int*>(workspace);
+    a.ws_prefix = reinterpret_cast<int*>(static_cast<char*>(workspace) + kWsHeaderBytes);
+    a.wait_spins = wait_spin_limit();
     a.table_stride = addr.table_stride;
     a.q_stride_bytes = q_token_stride * 2;
     a.out_stride_bytes = out_token_stride * 2;

@@ -1531,15 +1531,29 @@ int mla_teams(int n_hb) {
   return teams < 8 ? 8 : teams;
 }
 
+// Tuning knob XLLM_MI355_MLA_KERNEL, read once per process (first letter: 'p' pairs, 's' split); a test may
+// override it through set_mla_kernel_knob.
+std::atomic<int> g_mla_knob{-1};
+int mla_kernel_knob() {
+  int v = g_mla_knob.load(std::memory_order_relaxed);
+  if (v < 0) {
+    const char* e = getenv("XLLM_MI355_MLA_KERNEL");
+    v = e != nullptr ? static_cast<unsigned char>(e[0]) : 0;
+    g_mla_knob.store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
 }  // namespace
 
+void set_mla_kernel_knob(int first_letter) { g_mla_knob.store(first_letter < 0 ? 0 : first_letter, std::memory_order_relaxed); }
+
 size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) {
+  (void)batch;  // (the layout does not depend on it)
   (void)max_seq_len;
-  const size_t b = static_cast<size_t>(batch < kMaxBatchMla ? batch : kMaxBatchMla);
-  const size_t prefix_bytes = ((b + 1) * 4 + 255) / 256 * 256;
   // the kernel with 128 heads per workgroup has the fewer workgroups per team, hence the more teams
   const int n_hb = static_cast<int>((n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
-  return prefix_bytes + static_cast<size_t>(mla_teams(n_hb)) * 2 * n_heads * (kDL + 1) * 4;
+  return kWsPartialsOff + static_cast<size_t>(mla_teams(n_hb)) * 2 * n_heads * (kDL + 1) * 4;
 }
 
 int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out, float* lse,
@@ -1565,12 +1579,12 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       workspace_bytes < mla_workspace_bytes(batch, n_heads, 0))
     return XLLM_MI355_EWORKSPACE;
 
-  // tuning knob, read on every call: "pairs" selects the kernel with the per-tile exchange (also taken for
-  // block sizes below 16 or not a power of two: the other kernels look pages up per group of 4 tokens inside
-  // chunks of 64 pages), "split" the producer / consumer kernel
-  const char* knob = getenv("XLLM_MI355_MLA_KERNEL");
-  const bool pairs = (knob != nullptr && knob[0] == 'p') || block_size < 16 || (block_size & (block_size - 1)) != 0;
-  const bool split = knob != nullptr && knob[0] == 's' && !pairs;
+  // "pairs" selects the kernel with the per-tile exchange (also taken for block sizes below 16 or not a power
+  // of two: the other kernels look pages up per group of 4 tokens inside chunks of 64 pages), "split" the
+  // producer / consumer kernel
+  const int knob = mla_kernel_knob();
+  const bool pairs = knob == 'p' || block_size < 16 || (block_size & (block_size - 1)) != 0;
+  const bool split = knob == 's' && !pairs;
   const int n_hb = static_cast<int>(pairs ? (n_heads + kHeadsPerWg - 1) / kHeadsPerWg
                                           : (n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
   const int n_hb_p = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
@@ -1615,9 +1629,8 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       if ((1LL << s) == block_size) a.bs_shift = s;
     a.num_blocks = static_cast<int>(num_blocks);
     a.scale_log2 = sm_scale * kLog2e;
-    const size_t prefix_bytes = ((static_cast<size_t>(nb) + 1) * 4 + 255) / 256 * 256;
-    a.ws_prefix = static_cast<int*>(workspace);
-    a.ws_out = reinterpret_cast<float*>(static_cast<char*>(workspace) + prefix_bytes);
+    a.ws_prefix = reinterpret_cast<int*>(static_cast<char*>(workspace) + kWsHeaderBytes);
+    a.ws_out = reinterpret_cast<float*>(static_cast<char*>(workspace) + kWsPartialsOff);
     a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * n_heads * kDL;
 
     if (pairs)

@@ -80,10 +80,25 @@ torch::Tensor decode_workspace(const torch::Device& device, size_t nbytes) {
   static std::unordered_map<int, torch::Tensor> ws;
   std::lock_guard<std::mutex> lock(mu);
   torch::Tensor& t = ws[device.index()];
-  if (!t.defined() || static_cast<size_t>(t.numel()) < nbytes)
-    t = torch::empty({static_cast<int64_t>(std::max<size_t>(nbytes, 1 << 20))},
-                     torch::TensorOptions().dtype(torch::kUInt8).device(device));
+  if (!t.defined()) {
+    // once per device, at the library's bound over every supported shape, and never replaced: a launch
+    // recorded in a HIP graph keeps the address it was captured with
+    const size_t want = std::max<size_t>(nbytes, xllm_mi355_decode_workspace_bound());
+    t = torch::empty({static_cast<int64_t>(want)}, torch::TensorOptions().dtype(torch::kUInt8).device(device));
+    check_rc(xllm_mi355_decode_workspace_init(t.data_ptr(), want, c10::hip::getCurrentHIPStream(device.index()).stream()),
+             "xllm_mi355_decode_workspace_init");
+  }
+  TORCH_CHECK(static_cast<size_t>(t.numel()) >= nbytes, "the decode workspace of device ", device.index(), " holds ",
+              t.numel(), " bytes and ", nbytes,
+              " are needed: it cannot grow once handed out (captured graphs hold its address); call "
+              "decode_workspace(device, nbytes) with the largest need before the first decode call");
   return t;
+}
+
+void decode_status(const torch::Device& device) {
+  torch::Tensor ws = decode_workspace(device, 0);
+  check_rc(xllm_mi355_decode_status(ws.data_ptr(), c10::hip::getCurrentHIPStream(device.index()).stream()),
+           "xllm_mi355_decode_status");
 }
 
 void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torch::Tensor& output,

@@ -35,9 +35,14 @@ void quant_to_paged_cache(ReshapePagedCacheParams& params);
 
 namespace mi355 {
 
-// Per-device split workspace, grown on demand; same lifetime as the reference's
-// FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41).
+// Per-device split workspace, allocated once (at the library's bound over every supported shape, or nbytes if
+// that is more) and never replaced; same lifetime as the reference's FlashinferWorkspace singleton
+// (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41).  A request beyond its size throws.  It serves one
+// stream at a time: decode calls on two streams of one device must not overlap.
 torch::Tensor decode_workspace(const torch::Device& device, size_t nbytes);
+// Throws if a bounded wait inside a decode kernel gave up since the last call (that launch's outputs are
+// invalid).  Synchronises the current stream: not for use under graph capture.
+void decode_status(const torch::Device& device);
 
 void batch_decode(const torch::Tensor& query,        // [B, Hq, D]
                   const torch::Tensor& k_cache,      // [P, bs, Hkv, D]

@@ -61,18 +61,50 @@ def _require_cuda(*tensors):
 
 
 # ------------------------------------------------------------------------------------------
-# workspace: one per device, grown on demand, same lifetime as the reference's
-# FlashinferWorkspace singleton (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41)
+# workspace: one per device, allocated once and never replaced (a launch recorded in a HIP graph keeps the
+# address it was captured with), same lifetime as the reference's FlashinferWorkspace singleton
+# (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41).  It serves one stream at a time: decode calls on two
+# streams of one device must not overlap.
 
 _workspaces = {}
 
 
-def decode_workspace(device, nbytes):
+def reserve_decode_workspace(device, nbytes=0):
+    """Allocate the device's decode workspace (at least the library's bound over every supported shape, or
+    nbytes if that is more).  Call it before the first decode of a process that needs more than the bound;
+    a second call that would have to grow the workspace raises."""
+    device = torch.device(device)
+    lib = capi.lib()
+    want = max(int(nbytes), int(lib.xllm_mi355_decode_workspace_bound()))
     ws = _workspaces.get(device)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[device] = ws
+    if ws is not None:
+        if ws.numel() < nbytes:
+            raise RuntimeError(
+                f"the decode workspace of {device} holds {ws.numel()} bytes and {nbytes} are needed: it cannot grow "
+                "once handed out (captured graphs hold its address); reserve_decode_workspace(device, nbytes) "
+                "before the first decode call")
+        return ws
+    with torch.cuda.device(device):
+        ws = torch.empty(want, dtype=torch.uint8, device=device)
+        capi.check(lib.xllm_mi355_decode_workspace_init(ws.data_ptr(), ws.numel(), _stream(device)),
+                   "xllm_mi355_decode_workspace_init")
+    _workspaces[device] = ws
     return ws
+
+
+def decode_workspace(device, nbytes):
+    return reserve_decode_workspace(device, nbytes)
+
+
+def decode_status(device):
+    """0, or raises if a bounded wait inside a decode kernel gave up since the last call (the outputs of that
+    launch are invalid).  Synchronises the current stream: not for use under graph capture."""
+    ws = _workspaces.get(torch.device(device))
+    if ws is None:
+        return 0
+    capi.check(capi.lib().xllm_mi355_decode_status(ws.data_ptr(), _stream(torch.device(device))),
+               "xllm_mi355_decode_status")
+    return 0
 
 
 # ------------------------------------------------------------------------------------------
