@@ -58,7 +58,8 @@ enum {
   XLLM_MI355_ESHAPE = -3,      /* head_dim / group / block size not implemented */
   XLLM_MI355_EWORKSPACE = -4,  /* workspace missing or too small                */
   XLLM_MI355_EALIGN = -5,      /* pointer or stride not 16-byte aligned         */
-  XLLM_MI355_ESTALLED = -6     /* xllm_mi355_decode_status: a bounded wait inside a decode kernel gave up */
+  XLLM_MI355_ESTALLED = -6,    /* xllm_mi355_decode_status: a bounded wait inside a decode kernel gave up */
+  XLLM_MI355_ESCRATCH = -7     /* the problem does not fit the static scratch of the no-allocation entry point */
 };
 
 /* Human-readable text for a return code of this library (host pointer, static). */
@@ -161,6 +162,30 @@ int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* 
                                 int64_t max_seq_len, float sm_scale,
                                 void* workspace, size_t workspace_bytes,
                                 int q_dtype, int cache_dtype, void* stream);
+
+/*
+ * xllm_mi355_paged_decode_gqa without a workspace argument and without any allocation, for callers that
+ * cannot allocate: code under HIP graph capture whose workspace was not set up beforehand, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same
+ * kernels and bit-identical results; the partial results of contexts that span several workers go to a
+ * scratch array inside the library's code object (XLLM_MI355_STATIC_SCRATCH_BYTES per GPU, held until the
+ * process ends).  Limits: batch <= 2048, and a shape whose partial slots fit the scratch (every shape of the
+ * matrix-core kernel does; XLLM_MI355_ESCRATCH otherwise).  Every call on a GPU shares that GPU's scratch:
+ * calls that overlap in time on one GPU (two streams, two threads) race on it.  Nothing in it needs to start
+ * at zero except the status word, which only xllm_mi355_decode_status(NULL, stream) clears.  The first call on
+ * a device looks the scratch address up (hipGetSymbolAddress): make it outside graph capture.
+ */
+#define XLLM_MI355_STATIC_SCRATCH_BYTES (20u << 20)
+int xllm_mi355_paged_decode_gqa_static(const void* q, const void* k_cache, const void* v_cache,
+                                       void* out, float* lse,
+                                       const int32_t* block_table, int64_t table_stride,
+                                       const int32_t* seq_lens,
+                                       const float* k_scale, const float* v_scale,
+                                       int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
+                                       int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                       int64_t q_token_stride, int64_t out_token_stride,
+                                       int64_t max_seq_len, float sm_scale,
+                                       int q_dtype, int cache_dtype, void* stream);
 
 /*
  * Same, CSR addressing.  Replaces xllm::kernel::cuda::batch_decode
@@ -364,10 +389,12 @@ int xllm_mi355_decode_metadata_update(const int32_t* src_tokens, const int32_t* 
  * Opt-in timing of the dominant decode kernel.  No counterpart in the reference, which
  * relies on external profilers (xllm/core/platform/cuda_profiler.cpp,
  * xllm/core/platform/torch_profiler.cpp).  After xllm_mi355_profile_enable(n) the next n
- * calls of a decode entry point record a HIP event pair around their main kernel on the
- * caller's stream; xllm_mi355_profile_collect waits for them, writes the elapsed
- * milliseconds of each (host pointer) and returns how many, or a value < -1000 on a HIP
- * error.  Process-wide, single caller thread, not usable under graph capture.
+ * timed kernels carry a HIP event pair that the runtime fills with the kernel's own start and
+ * end; a decode entry point times two kernels per launch pair, in this order: the decode kernel,
+ * then the merge kernel (a batch of more than 2048 sequences is several launch pairs).
+ * xllm_mi355_profile_collect waits for them, writes the elapsed milliseconds of each (host
+ * pointer) and returns how many, or a value < -1000 on a HIP error.  Process-wide, single
+ * caller thread, not usable under graph capture.
  */
 int xllm_mi355_profile_enable(int capacity);
 int xllm_mi355_profile_collect(float* ms_out, int max_n);

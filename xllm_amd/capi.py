@@ -28,6 +28,8 @@ SIGNATURES = {
     "xllm_mi355_paged_decode_gqa": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64,
                                            _i64, _i64, _i64, _i64, _i64, _i64, _f32, _p, _sz, _i32,
                                            _i32, _p]),
+    "xllm_mi355_paged_decode_gqa_static": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64,
+                                                  _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _i32, _p]),
     "xllm_mi355_decode_workspace_bound": (_sz, []),
     "xllm_mi355_decode_workspace_init": (_i32, [_p, _sz, _p]),
     "xllm_mi355_decode_status": (_i32, [_p, _p]),

@@ -1,6 +1,8 @@
 // extern "C" surface of libxllm_mi355.so: plain pointers and sizes in, enqueue only.
 #include "launch.h"
 
+#include <mutex>
+
 using namespace xllm_mi355;
 
 namespace xllm_mi355 {
@@ -11,6 +13,35 @@ std::atomic<int> g_wait_spins{kDefaultWaitSpins};
 int wait_spin_limit() { return g_wait_spins.load(std::memory_order_relaxed); }
 void set_mla_kernel_knob(int first_letter);  // paged_decode_mla.hip
 }  // namespace xllm_mi355
+
+// Scratch of xllm_mi355_paged_decode_gqa_static: a decode workspace that lives in the code object, one copy
+// per GPU that loads the library, held until the process ends.  In host code the name is only a handle for
+// hipGetSymbolAddress; kernels and fills take the per-device address kept in static_scratch().
+constexpr size_t kStaticScratchBytes = XLLM_MI355_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+// The device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kMaxDevices) return XLLM_MI355_EINVAL;
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 255) != 0) return XLLM_MI355_EWORKSPACE;
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return XLLM_MI355_OK;
+}
+}  // namespace
 
 extern "C" {
 
@@ -25,6 +56,7 @@ const char* xllm_mi355_error_string(int code) {
     case XLLM_MI355_EWORKSPACE: return "split-K workspace missing, misaligned or too small";
     case XLLM_MI355_EALIGN: return "pointer or stride not 16-byte aligned";
     case XLLM_MI355_ESTALLED: return "a bounded wait inside a decode kernel gave up: the outputs of that launch are invalid";
+    case XLLM_MI355_ESCRATCH: return "the problem needs more scratch than the static scratch of the no-allocation entry point holds";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -63,7 +95,10 @@ int xllm_mi355_decode_workspace_init(void* workspace, size_t workspace_bytes, vo
 }
 
 int xllm_mi355_decode_status(void* workspace, void* stream) {
-  if (workspace == nullptr) return XLLM_MI355_EINVAL;
+  if (workspace == nullptr) {
+    const int rc = static_scratch(&workspace);
+    if (rc != 0) return rc;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   int status = 0;
   hipError_t e = hipMemcpyAsync(&status, workspace, sizeof(int), hipMemcpyDeviceToHost, s);
@@ -105,6 +140,27 @@ int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* 
                           n_kv_heads, head_dim, block_size, num_blocks, q_token_stride,
                           out_token_stride, max_seq_len, sm_scale, workspace, workspace_bytes, q_dtype,
                           cache_dtype, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_paged_decode_gqa_static(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                       float* lse, const int32_t* block_table, int64_t table_stride,
+                                       const int32_t* seq_lens, const float* k_scale, const float* v_scale,
+                                       int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim,
+                                       int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
+                                       int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
+                                       int q_dtype, int cache_dtype, void* stream) {
+  if (batch > kWsMaxBatch) return XLLM_MI355_ESCRATCH;  // (a longer batch would be decoded in slices that share the scratch)
+  void* ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc != 0) return rc;
+  PageAddressing addr;
+  addr.block_table = block_table;
+  addr.table_stride = table_stride;
+  addr.seq_lens = seq_lens;
+  rc = paged_decode_gqa(q, k_cache, v_cache, out, lse, addr, k_scale, v_scale, batch, n_q_heads, n_kv_heads,
+                        head_dim, block_size, num_blocks, q_token_stride, out_token_stride, max_seq_len, sm_scale,
+                        ws, kStaticScratchBytes, q_dtype, cache_dtype, static_cast<hipStream_t>(stream));
+  return rc == XLLM_MI355_EWORKSPACE ? XLLM_MI355_ESCRATCH : rc;
 }
 
 int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const void* v_cache, void* out,
