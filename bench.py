@@ -3,11 +3,18 @@
 
 A step = one pass of the hot path over one synthetic decode batch that is already resident in
 HBM: reshape_and_cache of the step's new K/V rows, then the paged decode attention over the
-whole context.  Prints ONE JSON line (see README of the contract in the repository docs).
+whole context.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+Without --workload every benchmark configuration runs: `tiny` as the correctness gate, then
+llama3_8b, long_b256, fp8_kv and mla_dsv3, each timed over K steps after W warm-up steps.  The
+headline fields of the line are those of long_b256 (the largest configuration that fits one GPU);
+`per_config` carries the same fields for each of the four.  Every configuration's GPU output is
+compared with the CPU checker on the sequences the CPU baseline samples (`parity`).
 """
 import argparse
+import ctypes
 import json
 import os
 import statistics
@@ -19,17 +26,22 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+METRIC = "paged-decode tokens/s + achieved HBM GB/s (% of 8 TB/s) on 1 MI355X"
+ALL = ("llama3_8b", "long_b256", "fp8_kv", "mla_dsv3")
+HEADLINE = "long_b256"
+MAX_ABS_TOL, MEAN_ABS_TOL = 2e-2, 2e-3   # attention output against the reference's libtorch CPU path, bf16
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="llama3_8b",
-                    help="tiny | llama3_8b | long_b256 | fp8_kv | mla_dsv3 (the five configurations); gqa_d64 | mla_tp8 (side workloads)")
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="all",
+                    help="all (default) | tiny | llama3_8b | long_b256 | fp8_kv | mla_dsv3 (the five configurations); "
+                         "gqa_d64 | gqa_d256 | mla_tp8 (side workloads)")
     ap.add_argument("--seed", type=int, default=2)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline (and with it the parity check)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run only the plain stream_read / stream_copy kernels over 1 GiB (counter calibration)")
@@ -38,55 +50,72 @@ def parse_args():
     return ap.parse_args()
 
 
-def cpu_baseline(inp, k_cache, v_cache, k_scale, v_scale, n_sample, budget_s=6.0):
-    """Time the checker (the ATen-op-order restatement of the reference's libtorch CPU path) on the
-    first n_sample sequences of the same workload (0 = as many as fit ~budget_s per pass).  A reported
-    baseline, never the product path."""
+def cpu_baseline(inp, k_cache, v_cache, k_scale, v_scale, gpu_out, n_sample, budget_s):
+    """Time the checker (the ATen-op-order restatement of the reference's libtorch CPU path) on the first
+    n_sample sequences of the same workload (0 = as many as fit ~budget_s per pass), and compare what it
+    computes with what the GPU computed for the same sequences: the rows the step's reshape_and_cache wrote
+    (bit for bit) and the attention output (max / mean absolute difference).  A reported baseline and a
+    checker, never the product path."""
     import torch
     import oracle
     cfg, lay = inp.cfg, inp.layout
+    kc = k_cache.cpu()
+    vc = None if v_cache is None else v_cache.cpu()
+    ks = None if k_scale is None else k_scale.cpu()
+    vs = None if v_scale is None else v_scale.cpu()
     if n_sample <= 0:
         # size the sample from one sequence's cost
         probe_q = inp.q[:1].cpu().contiguous()
-        kc0 = k_cache.cpu()
-        vc0 = None if v_cache is None else v_cache.cpu()
-        ks0 = None if k_scale is None else k_scale.cpu()
-        vs0 = None if v_scale is None else v_scale.cpu()
         t0 = time.perf_counter()
         for _ in range(2):
-            oracle.aten_paged_decode(probe_q, kc0, vc0, lay.block_table[:1].contiguous(),
-                                     lay.seq_lens[:1].contiguous(), cfg.scale, ks0, vs0, dv=cfg.dv)
+            oracle.aten_paged_decode(probe_q, kc, vc, lay.block_table[:1].contiguous(),
+                                     lay.seq_lens[:1].contiguous(), cfg.scale, ks, vs, dv=cfg.dv)
         per_token = (time.perf_counter() - t0) / 2 / max(1, int(lay.seq_lens[0]))
         mean_len = float(lay.seq_lens.float().mean())
         n_sample = max(1, min(cfg.batch, int(budget_s / (per_token * mean_len))))
     idx = list(range(min(n_sample, cfg.batch)))
     q = inp.q[idx].cpu().contiguous()
-    kc = k_cache.cpu()
-    vc = None if v_cache is None else v_cache.cpu()
     table = lay.block_table[idx].contiguous()
     lens = lay.seq_lens[idx].contiguous()
-    ks = None if k_scale is None else k_scale.cpu()
-    vs = None if v_scale is None else v_scale.cpu()
     k_new = inp.k_new[idx].cpu().contiguous()
     v_new = None if inp.v_new is None else inp.v_new[idx].cpu().contiguous()
     slots = lay.new_slots[idx].contiguous()
-    kc_store = kc.view(torch.uint8) if kc.dtype == torch.float8_e4m3fn else kc
-    vc_store = None if vc is None else (vc.view(torch.uint8) if vc.dtype == torch.float8_e4m3fn else vc)
+    fp8 = kc.dtype == torch.float8_e4m3fn
+    kc_store = kc.view(torch.uint8) if fp8 else kc
+    vc_store = None if vc is None else (vc.view(torch.uint8) if fp8 else vc)
+    # the GPU wrote these rows in every step; blank them in the copy so that the checker's write is what is compared
+    gpu_k_rows = kc_store.view(-1, kc_store.shape[-2] * kc_store.shape[-1])[slots.long()].clone()
+    gpu_v_rows = None if vc_store is None else vc_store.view(-1, vc_store.shape[-2] * vc_store.shape[-1])[slots.long()].clone()
+    kc_store.view(-1, kc_store.shape[-2] * kc_store.shape[-1])[slots.long()] = 0
+    if vc_store is not None:
+        vc_store.view(-1, vc_store.shape[-2] * vc_store.shape[-1])[slots.long()] = 0
 
     def one():
         oracle.reshape_and_cache(k_new, v_new, kc_store, vc_store, slots, ks, vs)
         return oracle.aten_paged_decode(q, kc, vc, table, lens, cfg.scale, ks, vs, dv=cfg.dv)
 
-    one()  # warm-up
+    ref = one()  # warm-up; also the reference output
+    cache_equal = torch.equal(kc_store.view(-1, gpu_k_rows.shape[1])[slots.long()], gpu_k_rows)
+    if vc_store is not None:
+        cache_equal = cache_equal and torch.equal(vc_store.view(-1, gpu_v_rows.shape[1])[slots.long()], gpu_v_rows)
     times = []
     for _ in range(3):
         t0 = time.perf_counter()
         one()
         times.append(time.perf_counter() - t0)
-        if sum(times) > 30:
+        if sum(times) > 3 * budget_s:
             break
     t = statistics.median(times)
-    return {
+    diff = (gpu_out[idx].float().cpu().reshape(ref.shape) - ref.float()).abs()
+    finite = bool(torch.isfinite(gpu_out.float()).all())
+    parity = {
+        "max_abs": float(diff.max()), "mean_abs": float(diff.mean()), "cache_bytes_equal": bool(cache_equal),
+        "tolerance": {"max_abs": MAX_ABS_TOL, "mean_abs": MEAN_ABS_TOL},
+        "sequences": len(idx),
+        "ok": bool(finite and cache_equal and diff.max() <= MAX_ABS_TOL and diff.mean() <= MEAN_ABS_TOL),
+        "against": "ATen-op-order restatement of the reference's libtorch CPU decode, same bytes",
+    }
+    baseline = {
         "value": len(idx) / t,
         "unit": "tokens/s",
         "cores": oracle.aten_lib().aten_oracle_num_threads(),
@@ -95,12 +124,20 @@ def cpu_baseline(inp, k_cache, v_cache, k_scale, v_scale, n_sample, budget_s=6.0
                   f"({int(lens.sum())} context tokens), median of {len(times)} runs, "
                   f"{t * 1e3:.1f} ms per pass",
     }
+    return baseline, parity
+
+
+def collect_ms(lib, n):
+    ms = (ctypes.c_float * n)()
+    got = lib.xllm_mi355_profile_collect(ms, n)
+    if got < 0:
+        raise RuntimeError(f"xllm_mi355_profile_collect failed: {got}")
+    return [ms[i] for i in range(got)]
 
 
 def stream_rate(lib, capi, torch, dev, nbytes, copy=False, reps=10):
     """GB/s of the library's plain read (or copy) kernel over nbytes: what this GPU sustains for a
     working set of that size, measured with the same event hook as the decode kernel."""
-    import ctypes
     nbytes = max(16, nbytes // 16 * 16)
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev).fill_(1)
     dst = torch.empty(nbytes, dtype=torch.uint8, device=dev) if copy else None
@@ -117,9 +154,8 @@ def stream_rate(lib, capi, torch, dev, nbytes, copy=False, reps=10):
     capi.check(lib.xllm_mi355_profile_enable(reps), "profile_enable")
     for _ in range(reps):
         run()
-    ms = (ctypes.c_float * reps)()
-    n = lib.xllm_mi355_profile_collect(ms, reps)
-    avg = sum(ms[i] for i in range(n)) / max(n, 1)
+    ms = collect_ms(lib, reps)
+    avg = sum(ms) / max(len(ms), 1)
     return (2 if copy else 1) * nbytes / (avg * 1e-3) / 1e9, avg
 
 
@@ -131,27 +167,16 @@ def calibrate(lib, capi, torch, dev):
             "stream_copy_gbs_read_plus_write": copy_gbs, "stream_copy_ms": copy_ms}
 
 
-def main():
-    args = parse_args()
-    world = int(os.environ.get("WORLD_SIZE", "1"))
-    if args.gpus != 1 or world != 1:
-        print("bench.py: this build runs on ONE GPU (every box has one); --gpus N with N > 1 is not "
-              "supported. The path shards by sequence or KV head with no exchange inside the op.",
-              file=sys.stderr)
-        sys.exit(2)
+def decode_kernel_name(cfg):
+    if cfg.mla:
+        return "mla_decode16_kernel"
+    mfma = (cfg.head_dim == 128 or (cfg.head_dim == 64 and cfg.cache_dtype != "fp8")) and cfg.block_size >= 16 \
+        and cfg.block_size & (cfg.block_size - 1) == 0
+    return "gqa_mfma_kernel" if mfma else "gqa_decode_kernel"
 
-    import torch
-    from xllm_amd import capi, ops, workloads
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    lib = capi.lib()  # raises if the HIP library has not been built
-    dev = torch.device("cuda:0")
-    if args.calibrate:
-        print(json.dumps(calibrate(lib, capi, torch, dev)))
-        return
-    cfg = workloads.CONFIGS[args.workload]
+def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s):
+    cfg = workloads.CONFIGS[name]
     fp8 = cfg.cache_dtype == "fp8"
 
     # ---- build the resident workload: context rows go into the cache through the op itself
@@ -170,6 +195,7 @@ def main():
     new_slots = lay.new_slots.to(dev)
     store(ops.ReshapePagedCacheParams(key=inp.k_ctx, value=inp.v_ctx, k_cache=k_cache, v_cache=v_cache,
                                       slot_mapping=ctx_slots, k_cache_scale=k_scale, v_cache_scale=v_scale))
+    inp.k_ctx = inp.v_ctx = None   # (the context now lives in the cache)
     table = lay.block_table.to(dev)
     seq_lens = lay.seq_lens.to(dev)
     max_len = int(lay.seq_lens.max())
@@ -227,16 +253,16 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    capi.check(lib.xllm_mi355_profile_enable(args.steps), "profile_enable")
+    capi.check(lib.xllm_mi355_profile_enable(2 * args.steps), "profile_enable")
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    import ctypes
-    ms = (ctypes.c_float * args.steps)()
-    n = lib.xllm_mi355_profile_collect(ms, args.steps)
-    kernel_ms = sum(ms[i] for i in range(n)) / max(n, 1)
+    ms = collect_ms(lib, 2 * args.steps)   # per step: the decode kernel, then the merge kernel
+    kernel_ms = sum(ms[0::2]) / max(len(ms[0::2]), 1)
+    merge_ms = sum(ms[1::2]) / max(len(ms[1::2]), 1)
+    ops.decode_status(dev)                 # raises if a wait inside a decode kernel gave up
 
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = cfg.batch / (ms_per_step * 1e-3)
@@ -245,38 +271,35 @@ def main():
     traffic = None
     try:
         with open(args.traffic_json) as f:
-            traffic = json.load(f).get(args.workload, {}).get("hbm_bytes_per_launch")
+            traffic = json.load(f).get(name, {}).get("hbm_bytes_per_launch")
     except (OSError, ValueError):
         pass
-    if cfg.mla and cfg.n_q_heads <= 64:
-        # the few heads of a tensor-parallel shard: 30-120 flop per cache byte, far below the ridge: HBM bound
+    op_ms = kernel_ms + merge_ms
+    if cfg.mla:
         nbytes, flops = workloads.mla_bytes_flops(cfg, lay.seq_lens)
-        achieved = nbytes / (kernel_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": "mla_decode16_kernel",
-                    "kernel_ms": kernel_ms, "algorithmic_bytes": nbytes, "algorithmic_flops": flops}
-    elif cfg.mla:
-        nbytes, flops = workloads.mla_bytes_flops(cfg, lay.seq_lens)
+    else:
+        nbytes, flops = workloads.gqa_bytes(cfg, lay.seq_lens, 1 if fp8 else 2), None
+    if cfg.mla and cfg.n_q_heads > 64:
         achieved = flops / (kernel_ms * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS,
-                    "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic,
-                    "kernel": "mla_decode16_kernel", "kernel_ms": kernel_ms, "algorithmic_flops": flops,
-                    "algorithmic_bytes": nbytes,
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": traffic,
+                    "op_frac": flops / (op_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                     "hbm_gbs": nbytes / (kernel_ms * 1e-3) / 1e9}
     else:
-        nbytes = workloads.gqa_bytes(cfg, lay.seq_lens, 1 if fp8 else 2)
+        # GQA, and MLA with the few heads of a tensor-parallel shard (30-120 flop per cache byte, far below the ridge)
         achieved = nbytes / (kernel_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                    "kernel": ("gqa_mfma_kernel" if cfg.head_dim == 128 or (cfg.head_dim == 64 and cfg.cache_dtype != "fp8")
-                               else "gqa_decode_kernel"),
-                    "kernel_ms": kernel_ms, "algorithmic_bytes": nbytes}
-
+                    "op_frac": nbytes / (op_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    roofline.update({"kernel": decode_kernel_name(cfg), "kernel_ms": kernel_ms, "merge_kernel_ms": merge_ms,
+                     "algorithmic_bytes": nbytes})
+    if flops is not None:
+        roofline["algorithmic_flops"] = flops
     # the same number of bytes through the plain read kernel: the rate this GPU sustains at this size
     roofline["stream_read_gbs_same_bytes"], _ = stream_rate(lib, capi, torch, dev, nbytes)
 
     result = {
-        "metric": "paged-decode tokens/s + achieved HBM GB/s (% of 8 TB/s) on 1 MI355X",
+        "metric": METRIC,
         "value": tokens_per_s,
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -289,7 +312,7 @@ def main():
         "dtype": "fp8_e4m3 KV, bf16 Q/O, fp32 accumulate" if fp8 else "bf16 (fp32 accumulate)",
         "data": "synthetic",
         "config": {
-            "workload": args.workload,
+            "workload": name,
             "batch": cfg.batch, "n_q_heads": cfg.n_q_heads, "n_kv_heads": cfg.n_kv_heads,
             "head_dim": cfg.head_dim, "block_size": cfg.block_size,
             "context_tokens": int(lay.seq_lens.sum()), "max_context": max_len,
@@ -301,8 +324,62 @@ def main():
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(inp, k_cache, v_cache, k_scale, v_scale, args.cpu_sample)
+        result["cpu_baseline"], result["parity"] = cpu_baseline(
+            inp, k_cache, v_cache, k_scale, v_scale, out.view(cfg.batch, cfg.n_q_heads, cfg.dv), args.cpu_sample,
+            cpu_budget_s)
+    del k_cache, v_cache, inp, out
+    torch.cuda.empty_cache()
+    return result
+
+
+def main():
+    args = parse_args()
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        print("bench.py: this build runs on ONE GPU (every box has one); --gpus N with N > 1 is not "
+              "supported. The path shards by sequence or KV head with no exchange inside the op.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from xllm_amd import capi, ops, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = capi.lib()  # raises if the HIP library has not been built
+    dev = torch.device("cuda:0")
+    if args.calibrate:
+        print(json.dumps(calibrate(lib, capi, torch, dev)))
+        return
+    run = lambda name, budget: run_workload(name, args, lib, capi, ops, workloads, torch, dev, budget)
+    if args.workload != "all":
+        result = run(args.workload, 6.0)
+    else:
+        # the correctness gate first: a wrong path is not timed
+        gate = run("tiny", 1.0)
+        if not args.no_cpu_baseline and not gate["parity"]["ok"]:
+            print(f"bench.py: the tiny configuration fails parity: {gate['parity']}", file=sys.stderr)
+            sys.exit(3)
+        per = {}
+        for name in ALL:
+            per[name] = run(name, 5.0 if name == HEADLINE else 2.0)
+            print(f"bench.py: {name}: {per[name]['ms_per_step']:.4f} ms/step, roofline {per[name]['roofline']['frac']:.3f}",
+                  file=sys.stderr, flush=True)
+        result = dict(per[HEADLINE])
+        result["gate"] = {"workload": "tiny", "parity": gate.get("parity")}
+        keep = ("value", "unit", "ms_per_step", "dtype", "config", "hbm_gbs_whole_step", "roofline", "cpu_baseline",
+                "parity")
+        result["per_config"] = [{k: per[name][k] for k in keep if k in per[name]} for name in ALL]
+        if not args.no_cpu_baseline:
+            result["parity_all_ok"] = all(per[name]["parity"]["ok"] for name in ALL) and gate["parity"]["ok"]
     print(json.dumps(result))
+    if not args.no_cpu_baseline:
+        bad = [name for name, ok in ((result["config"]["workload"], result["parity"]["ok"]),) if not ok]
+        bad += [p["config"]["workload"] for p in result.get("per_config", []) if not p["parity"]["ok"]]
+        if bad:
+            print(f"bench.py: parity FAILED for {sorted(set(bad))}", file=sys.stderr)
+            sys.exit(3)
 
 
 if __name__ == "__main__":

@@ -1630,9 +1630,9 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
       if (rc != 0) return rc;
       dim3 grid(static_cast<unsigned>(n_kv_heads * addr.chunk_blocks), static_cast<unsigned>(nb));
       if (q_dtype == XLLM_MI355_BF16)
-        merge_partials_kernel<BF16, true><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+        launch_timed(merge_partials_kernel<BF16, true>, grid, dim3(kThreads), 0, stream, a, static_cast<int>(head_dim));
       else
-        merge_partials_kernel<FP16, true><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+        launch_timed(merge_partials_kernel<FP16, true>, grid, dim3(kThreads), 0, stream, a, static_cast<int>(head_dim));
       rc = static_cast<int>(hipGetLastError());
       if (rc != 0) return rc;
       continue;
@@ -1647,9 +1647,9 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     const int hb_per_kv = (group + a.g_block - 1) / a.g_block;
     dim3 grid(static_cast<unsigned>(n_kv_heads * hb_per_kv), static_cast<unsigned>(nb));
     if (q_dtype == XLLM_MI355_BF16)
-      merge_partials_kernel<BF16, false><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+      launch_timed(merge_partials_kernel<BF16, false>, grid, dim3(kThreads), 0, stream, a, static_cast<int>(head_dim));
     else
-      merge_partials_kernel<FP16, false><<<grid, kThreads, 0, stream>>>(a, static_cast<int>(head_dim));
+      launch_timed(merge_partials_kernel<FP16, false>, grid, dim3(kThreads), 0, stream, a, static_cast<int>(head_dim));
     rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
   }

@@ -1643,7 +1643,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       launch_timed(mla_decode16_kernel<false>, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kThreads16), smem, stream, a);
     int rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
-    mla_merge_kernel<<<dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb)), 128, 0, stream>>>(a);
+    launch_timed(mla_merge_kernel, dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb)), dim3(128), 0, stream, a);
     rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
   }

@@ -44,9 +44,10 @@ CONFIGS = {
     "fp8_kv": DecodeConfig("fp8_kv", 128, 32, 8, 128, 16, 2048, 16384, cache_dtype="fp8"),
     "mla_dsv3": DecodeConfig("mla_dsv3", 64, 128, 1, 576, 64, 2048, 16384, mla=True, v_dim=512,
                              sigma=0.5, sm_scale=1.0 / math.sqrt(192.0)),
-    # side workloads (not among the five configurations above): 64-dim heads, and the MLA head count of an
+    # side workloads (not among the five configurations above): 64-dim and 256-dim heads, and the MLA head count of an
     # 8-way tensor-parallel shard
     "gqa_d64": DecodeConfig("gqa_d64", 64, 32, 8, 64, 16, 1024, 8192),
+    "gqa_d256": DecodeConfig("gqa_d256", 64, 16, 4, 256, 16, 512, 4096),
     "mla_tp8": DecodeConfig("mla_tp8", 64, 16, 1, 576, 64, 2048, 16384, mla=True, v_dim=512,
                             sigma=0.5, sm_scale=1.0 / math.sqrt(192.0)),
 }
