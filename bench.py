@@ -240,7 +240,7 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
         decode_args = (ptr(inp.q), ptr(k_cache), ptr(v_cache), ptr(out), None, ptr(table),
                        table.stride(0), ptr(seq_lens), ptr(k_scale), ptr(v_scale), cfg.batch,
                        cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, lay.num_blocks,
-                       inp.q.stride(0), out.stride(0), max_len, cfg.scale, ptr(ws), ws.numel(),
+                       inp.q.stride(0), out.stride(0), max_len, -1, cfg.scale, ptr(ws), ws.numel(),
                        capi.BF16, code[cache_dt], stream)
     reshape_fn = lib.xllm_mi355_reshape_and_cache
 

@@ -149,6 +149,9 @@ int xllm_mi355_decode_status(void* workspace, void* stream);
  * k_scale / v_scale: [Hkv] fp32, required iff cache_dtype is fp8 (dequantised value
  * = float(code) * scale[h]).  q_dtype also is the dtype of `out`.
  * max_seq_len <= 0 means "table_stride * block_size".
+ * window_left: sliding window (window_left of xllm/core/kernels/cuda/cuda_ops_api.h:139; sliding_window_ of
+ * xllm/core/layers/dcu/flash_attention.cpp:484): the query, at position L - 1, attends to positions
+ * >= L - 1 - window_left; negative = the whole context.  Pages that lie wholly before the window are not read.
  * A sequence with seq_lens[b] <= 0 gets out = 0 and lse = -inf.
  */
 int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache,
@@ -159,7 +162,7 @@ int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* 
                                 int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
                                 int64_t head_dim, int64_t block_size, int64_t num_blocks,
                                 int64_t q_token_stride, int64_t out_token_stride,
-                                int64_t max_seq_len, float sm_scale,
+                                int64_t max_seq_len, int64_t window_left, float sm_scale,
                                 void* workspace, size_t workspace_bytes,
                                 int q_dtype, int cache_dtype, void* stream);
 
@@ -184,7 +187,7 @@ int xllm_mi355_paged_decode_gqa_static(const void* q, const void* k_cache, const
                                        int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
                                        int64_t head_dim, int64_t block_size, int64_t num_blocks,
                                        int64_t q_token_stride, int64_t out_token_stride,
-                                       int64_t max_seq_len, float sm_scale,
+                                       int64_t max_seq_len, int64_t window_left, float sm_scale,
                                        int q_dtype, int cache_dtype, void* stream);
 
 /*
@@ -204,7 +207,7 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                                     int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
                                     int64_t head_dim, int64_t block_size, int64_t num_blocks,
                                     int64_t q_token_stride, int64_t out_token_stride,
-                                    int64_t max_seq_len, float sm_scale,
+                                    int64_t max_seq_len, int64_t window_left, float sm_scale,
                                     void* workspace, size_t workspace_bytes,
                                     int q_dtype, int cache_dtype, void* stream);
 
@@ -253,9 +256,11 @@ int xllm_mi355_mla_absorbed_bmm(const void* x, const void* w, void* y,
  * max_q_len is the caller's bound on the chunk lengths (AttentionMetadata::max_query_len), 0 if unknown.
  * With a bound (head dim 128, block size a power of two >= 16, Hq / Hkv <= 8 or the whole chunk in 16 columns)
  * the (token, head) pairs of a chunk share the 16 columns of the matrix-core kernel: the pages of a sequence
- * are read once per 16 / (Hq / Hkv) query tokens, and a chunk longer than the bound is cut to it.  Otherwise
- * every query token is decoded as an entry of its own against its sequence's pages (read once per token,
- * partly from L2), which is correct for any length.
+ * are read once per 16 / (Hq / Hkv) query tokens; the tokens of a chunk beyond the bound are left unwritten (the
+ * others still attend to the right prefix), so the bound must hold.  Otherwise
+ * (and always with a sliding window, window_left >= 0, which then counts from each token's own last attended
+ * position) every query token is decoded as an entry of its own against its sequence's pages (read once per
+ * token, partly from L2), which is correct for any length.
  * Workspace: xllm_mi355_paged_decode_varlen_workspace_bytes(max(n_tokens, batch), ...); the per-token arrays
  * take its last bytes, so pass the same workspace_bytes on every call that shares a captured graph.
  */
@@ -270,8 +275,8 @@ int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const
                                        int64_t n_q_heads,
                                        int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
                                        int64_t num_blocks, int64_t q_token_stride,
-                                       int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
-                                       int causal, void* workspace, size_t workspace_bytes,
+                                       int64_t out_token_stride, int64_t max_seq_len, int64_t window_left,
+                                       float sm_scale, int causal, void* workspace, size_t workspace_bytes,
                                        int q_dtype, int cache_dtype, void* stream);
 
 /*
@@ -280,8 +285,10 @@ int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const
  * (xllm/core/kernels/dcu/flash_mla_adapter.h:40-53, flash_mla_adapter.cpp:104-153):
  *     out[b, h, :] = softmax(sm_scale * [q_nope | q_pe][b, h, :] . C_b^T) . C_b[:, :d_latent]
  * with C_b the latent rows of sequence b, [L_b, d_latent + d_rope].
- * q_nope: [B, H, d_latent], q_pe: [B, H, d_rope], out: [B, H, d_latent], all
- * contiguous bf16; k_cache: [P, bs, 1, d_latent + d_rope] bf16.
+ * q_nope: [B, H, d_latent], q_pe: [B, H, d_rope], out: [B, H, d_latent], all contiguous and of `dtype`
+ * (XLLM_MI355_BF16 or XLLM_MI355_FP16: "BF16/FP16", flash_mla_adapter.cpp:105-107); k_cache:
+ * [P, bs, 1, d_latent + d_rope] of the same type.  d_latent 512, d_rope 64.  The S_q query tokens of a
+ * multi-token step are passed as S_q * H heads (the adapter folds them the same way, :119-123).
  */
 int xllm_mi355_paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache,
                                 void* out, float* lse,
@@ -308,6 +315,20 @@ int xllm_mi355_lse_merge(const void* partial_out, const float* partial_lse,
                          void* out, float* lse,
                          int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim,
                          int dtype, void* stream);
+
+/*
+ * Two-way combine of attention results whose LSEs are in base 2 (the convention of FlashInfer).  Replaces
+ * xllm::kernel::cuda::lse_combine (xllm/core/kernels/cuda/xattention/lse_combine.cu:41-85,99-166; caller
+ * xllm/core/layers/cuda/xattention.cpp:315), in the reference's arithmetic order:
+ *     m = max(a, b);  merged = m + log2(exp2(a - m) + exp2(b - m));
+ *     out = exp2(a - merged) * shared_o + exp2(b - merged) * unshared_o
+ * shared_o / unshared_o: [rows, head_dim] of in_dtype (rows = batch * heads); the LSEs: [rows] fp32;
+ * out: [rows, head_dim] of out_dtype.  Like the reference it returns no merged LSE, and two empty inputs
+ * (both LSEs -inf) give NaN.  A natural-log LSE of this library is this base-2 LSE times ln 2.
+ */
+int xllm_mi355_lse_combine(void* out, const void* shared_o, const float* shared_lse,
+                           const void* unshared_o, const float* unshared_lse,
+                           int64_t rows, int64_t head_dim, int in_dtype, int out_dtype, void* stream);
 
 /*
  * CSR -> padded block table.  Replaces build_block_table_from_paged_kv

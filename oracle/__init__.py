@@ -60,6 +60,8 @@ def c_lib():
                                                 _i64, _i64, _i64, _i64, _f64, _i32, _i32, _i32]
         lib.oracle_lse_merge.restype = None
         lib.oracle_lse_merge.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64]
+        lib.oracle_lse_combine.restype = None
+        lib.oracle_lse_combine.argtypes = [_p, _p, _p, _p, _p, _p, _i64, _i64]
         lib.oracle_build_block_table.restype = None
         lib.oracle_build_block_table.argtypes = [_p, _p, _p, _p, _i64, _p, _i64, _i64]
         lib.oracle_mask_block_table_padding.restype = None
@@ -240,6 +242,18 @@ def lse_merge(partial_out_f32, partial_lse):
     lse = torch.empty(B, H, dtype=torch.float32)
     c_lib().oracle_lse_merge(_ptr(partial_out_f32), _ptr(partial_lse), _ptr(out), _ptr(lse), S, B, H, Dv)
     return out, lse
+
+
+def lse_combine(shared_o, shared_lse, unshared_o, unshared_lse):
+    """C oracle of the two-way base-2 combine.  shared_o / unshared_o [B, H, D] (any float type; computed in fp32),
+    the LSEs [B, H, 1] fp32 in base 2.  Returns (out fp32 [B, H, D], merged base-2 LSE [B, H, 1])."""
+    B, H, D = shared_o.shape
+    so, uo = shared_o.float().contiguous(), unshared_o.float().contiguous()
+    sl, ul = shared_lse.float().contiguous(), unshared_lse.float().contiguous()
+    out = torch.empty(B, H, D, dtype=torch.float32)
+    merged = torch.empty(B, H, 1, dtype=torch.float32)
+    c_lib().oracle_lse_combine(_ptr(out), _ptr(merged), _ptr(so), _ptr(sl), _ptr(uo), _ptr(ul), B * H, D)
+    return out, merged
 
 
 def aten_lse_merge(partial_out, partial_lse):

@@ -328,6 +328,25 @@ void oracle_lse_merge(const float* partial_out, const float* partial_lse, float*
   }
 }
 
+/*
+ * Follows lse_combine_kernel (kernels/cuda/xattention/lse_combine.cu:41-85) in fp32, step for step, with the
+ * LSEs in base 2: max; exp2 of both against it; merged = max + log2(sum); weights exp2(lse - merged);
+ * out = w_shared * shared_o + w_unshared * unshared_o.  All arrays fp32: shared_o / unshared_o / out [rows, d],
+ * the LSEs [rows].  The reference writes no merged LSE; `merged` (may be null) receives it for the tests.
+ */
+void oracle_lse_combine(float* out, float* merged, const float* shared_o, const float* shared_lse,
+                        const float* unshared_o, const float* unshared_lse, int64_t rows, int64_t d) {
+  for (int64_t i = 0; i < rows; ++i) {
+    const float a = shared_lse[i], b = unshared_lse[i];
+    const float lse_max = fmaxf(a, b);
+    const float ea = exp2f(a - lse_max), eb = exp2f(b - lse_max);
+    const float lse_new = lse_max + log2f(ea + eb);
+    const float wa = exp2f(a - lse_new), wb = exp2f(b - lse_new);
+    for (int64_t k = 0; k < d; ++k) out[i * d + k] = wa * shared_o[i * d + k] + wb * unshared_o[i * d + k];
+    if (merged) merged[i] = lse_new;
+  }
+}
+
 /* ---- CSR -> block table ------------------------------------------------------------ */
 
 /*

@@ -55,3 +55,31 @@ def assert_close_to_reference(actual, expected, what=""):
     mx, mean = diff.max().item(), diff.mean().item()
     assert mx <= MAX_ABS_TOL and mean <= MEAN_ABS_TOL, f"{what}: max-abs {mx:.3e}, mean-abs {mean:.3e}"
     return mx, mean
+
+
+def trimmed_context(k_cache, v_cache, block_table, seq_lens, first_tokens):
+    """The paged caches of the contexts cut to their tokens [first_tokens[b], seq_lens[b]): new caches whose pages
+    hold those rows from row 0 on, with their table and lengths.  The block-table oracle on this layout is the
+    reference of a sliding-window decode."""
+    P, bs = k_cache.shape[0], k_cache.shape[1]
+    B = seq_lens.numel()
+    kf = k_cache.reshape(P * bs, *k_cache.shape[2:])
+    vf = None if v_cache is None else v_cache.reshape(P * bs, *v_cache.shape[2:])
+    new_lens = (seq_lens - first_tokens).to(torch.int32)
+    n_pages = (new_lens.long() + bs - 1) // bs
+    total = int(n_pages.sum())
+    nk = torch.zeros(total * bs, *k_cache.shape[2:], dtype=k_cache.dtype)
+    nv = None if v_cache is None else torch.zeros_like(nk)
+    table = torch.zeros(B, max(1, int(n_pages.max())), dtype=torch.int32)
+    page = 0
+    for b in range(B):
+        t = torch.arange(int(first_tokens[b]), int(seq_lens[b]))
+        slots = block_table[b, t // bs].long() * bs + t % bs
+        n = t.numel()
+        nk[page * bs : page * bs + n] = kf[slots]
+        if nv is not None:
+            nv[page * bs : page * bs + n] = vf[slots]
+        table[b, : int(n_pages[b])] = torch.arange(page, page + int(n_pages[b]), dtype=torch.int32)
+        page += int(n_pages[b])
+    shape = (total, bs, *k_cache.shape[2:])
+    return nk.view(shape), None if nv is None else nv.view(shape), table, new_lens

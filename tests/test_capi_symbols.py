@@ -35,13 +35,13 @@ def test_host_only_entry_points_without_a_gpu():
     lib = capi.lib()
     assert re.fullmatch(rb"\d+\.\d+\.\d+", lib.xllm_mi355_version())
     assert lib.xllm_mi355_error_string(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert len(lib.xllm_mi355_error_string(code)) > 4
     # argument validation happens before any HIP call
     assert lib.xllm_mi355_reshape_and_cache(None, None, None, None, None, None, None, 4, 8, 128, 16, 10,
                                             1024, 1024, capi.BF16, capi.BF16, None) == -1
     assert lib.xllm_mi355_paged_decode_gqa(None, None, None, None, None, None, 0, None, None, None, 4, 32,
-                                           8, 128, 16, 10, 4096, 4096, 100, 0.1, None, 0, capi.BF16,
+                                           8, 128, 16, 10, 4096, 4096, 100, -1, 0.1, None, 0, capi.BF16,
                                            capi.BF16, None) == -1
     assert lib.xllm_mi355_paged_decode_mla(None, None, None, None, None, None, 0, None, 4, 128, 512, 64, 64,
                                            10, 100, 0.1, None, 0, capi.BF16, None) == -1

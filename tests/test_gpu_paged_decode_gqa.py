@@ -160,7 +160,7 @@ def test_csr_form_matches_block_table_form_and_csr_oracle(device):
     q = inp.q.to(device)
     out_b = torch.empty_like(q)
     ops.batch_decode_csr(q, kg, vg, lay.indptr.to(device), lay.indices.to(device),
-                         lay.last_page_len.to(device), cfg.scale, out_b, max_seq_len=int(lay.seq_lens.max()))
+                         lay.last_page_len.to(device), -1, cfg.scale, out_b, max_seq_len=int(lay.seq_lens.max()))
     assert torch.equal(out_a, out_b)
     ref = oracle.aten_paged_decode_csr(inp.q, kg.cpu(), vg.cpu(), lay.indptr, lay.indices, lay.last_page_len)
     assert_close_to_reference(out_b, ref, "csr")

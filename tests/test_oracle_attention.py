@@ -359,3 +359,32 @@ def test_fp8_decode_known_answer():
     assert torch.allclose(lse64.double(), expect, atol=1e-5)
     lse = oracle.aten_paged_decode_lse(q, kc, table, lens, 0.125, ks)
     assert torch.allclose(lse.double(), expect, atol=1e-4)
+
+
+def test_base2_two_way_combine_oracle():
+    """The known answers of the reference's merge tests (dcp_attention_merge_test.cpp:34-63) with the LSEs
+    rescaled to base 2 (natural-log LSE / ln 2), the natural-log merge oracle on random inputs, and the
+    equal-weights and one-sided special cases.  A swapped weight, a natural-log exponential or a missing
+    normalisation fails one of them."""
+    ln2 = math.log(2.0)
+    o_a = torch.tensor([[[2.0, 4.0]]]); o_b = torch.tensor([[[6.0, 8.0]]])
+    out, merged = oracle.lse_combine(o_a, torch.tensor([[[math.log(2.0) / ln2]]]), o_b, torch.tensor([[[math.log(6.0) / ln2]]]))
+    assert torch.allclose(out, torch.tensor([[[5.0, 7.0]]]), atol=1e-6)
+    assert torch.allclose(merged, torch.tensor([[[math.log(8.0) / ln2]]]), atol=1e-6)
+    out, merged = oracle.lse_combine(torch.zeros(1, 1, 2), torch.tensor([[[-math.inf]]]), torch.tensor([[[3.0, 9.0]]]),
+                                     torch.tensor([[[2.0]]]))
+    assert torch.equal(out, torch.tensor([[[3.0, 9.0]]])) and torch.equal(merged, torch.tensor([[[2.0]]]))
+    # equal LSEs: the mean; the merged LSE is one more (base 2)
+    out, merged = oracle.lse_combine(o_a, torch.tensor([[[3.0]]]), o_b, torch.tensor([[[3.0]]]))
+    assert torch.equal(out, torch.tensor([[[4.0, 6.0]]])) and torch.equal(merged, torch.tensor([[[4.0]]]))
+    # random inputs against the natural-log merge oracle (two shards)
+    g = torch.Generator().manual_seed(3)
+    a, b = torch.randn(3, 5, 16, generator=g), torch.randn(3, 5, 16, generator=g)
+    la, lb = torch.randn(3, 5, 1, generator=g) * 4, torch.randn(3, 5, 1, generator=g) * 4
+    out, merged = oracle.lse_combine(a, la, b, lb)
+    ref, ref_lse = oracle.lse_merge(torch.stack([a, b]), torch.stack([la, lb]).squeeze(-1) * ln2)
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(merged.squeeze(-1) * ln2, ref_lse, rtol=1e-5, atol=1e-5)
+    # both inputs empty: NaN, as the reference's arithmetic gives
+    out, _ = oracle.lse_combine(o_a, torch.tensor([[[-math.inf]]]), o_b, torch.tensor([[[-math.inf]]]))
+    assert torch.isnan(out).all()

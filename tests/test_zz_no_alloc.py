@@ -22,7 +22,7 @@ def _call(lib, static, inp, kg, vg, ks, vs, device):
     ptr = lambda t: None if t is None else t.data_ptr()
     head = (q.data_ptr(), kg.data_ptr(), vg.data_ptr(), out.data_ptr(), lse.data_ptr(), table.data_ptr(),
             table.stride(0), lens.data_ptr(), ptr(ks), ptr(vs), cfg.batch, cfg.n_q_heads, cfg.n_kv_heads,
-            cfg.head_dim, cfg.block_size, lay.num_blocks, q.stride(0), out.stride(0), int(lay.seq_lens.max()),
+            cfg.head_dim, cfg.block_size, lay.num_blocks, q.stride(0), out.stride(0), int(lay.seq_lens.max()), -1,
             cfg.scale)
     code = capi.FP8_E4M3 if kg.dtype == torch.float8_e4m3fn else capi.BF16
     if static:
@@ -64,5 +64,5 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(device):
     fake = 1 << 20
     # more sequences than one launch holds: the slices of a longer batch would share the scratch
     rc = lib.xllm_mi355_paged_decode_gqa_static(fake, fake, fake, fake, None, fake, 8, fake, None, None, 2049, 32, 8,
-                                                128, 16, 100, 4096, 4096, 100, 0.1, capi.BF16, capi.BF16, None)
+                                                128, 16, 100, 4096, 4096, 100, -1, 0.1, capi.BF16, capi.BF16, None)
     assert rc == -7 and b"scratch" in lib.xllm_mi355_error_string(rc)

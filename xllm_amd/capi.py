@@ -26,25 +26,26 @@ SIGNATURES = {
     "xllm_mi355_kv_head_scales": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "xllm_mi355_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
     "xllm_mi355_paged_decode_gqa": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64,
-                                           _i64, _i64, _i64, _i64, _i64, _i64, _f32, _p, _sz, _i32,
+                                           _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _p, _sz, _i32,
                                            _i32, _p]),
     "xllm_mi355_paged_decode_gqa_static": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64,
-                                                  _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _i32, _p]),
+                                                  _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _i32, _p]),
     "xllm_mi355_decode_workspace_bound": (_sz, []),
     "xllm_mi355_decode_workspace_init": (_i32, [_p, _sz, _p]),
     "xllm_mi355_decode_status": (_i32, [_p, _p]),
     "xllm_mi355_debug_set": (_i32, [_i32, _i32]),
     "xllm_mi355_paged_decode_gqa_csr": (_i32, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64,
-                                               _i64, _i64, _i64, _i64, _i64, _i64, _f32, _p, _sz, _i32,
+                                               _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _p, _sz, _i32,
                                                _i32, _p]),
     "xllm_mi355_gather_paged_rows": (_i32, [_p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "xllm_mi355_paged_decode_varlen_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "xllm_mi355_paged_decode_gqa_varlen": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64,
-                                                  _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _p,
+                                                  _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i32, _p,
                                                   _sz, _i32, _i32, _p]),
     "xllm_mi355_paged_decode_mla": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64,
                                            _i64, _i64, _i64, _f32, _p, _sz, _i32, _p]),
     "xllm_mi355_lse_merge": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
+    "xllm_mi355_lse_combine": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p]),
     "xllm_mi355_build_block_table": (_i32, [_p, _p, _p, _p, _i64, _p, _i64, _i64, _p]),
     "xllm_mi355_decode_metadata_update": (_i32, [_p] * 15 + [_i64] * 4 + [_p]),
     "xllm_mi355_mask_block_table_padding": (_i32, [_p, _i64, _p, _p, _i64, _i64, _i64, _i64, _p]),

@@ -129,13 +129,14 @@ int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* 
                                 const int32_t* seq_lens, const float* k_scale, const float* v_scale,
                                 int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim,
                                 int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
-                                int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
+                                int64_t out_token_stride, int64_t max_seq_len, int64_t window_left, float sm_scale,
                                 void* workspace, size_t workspace_bytes, int q_dtype, int cache_dtype,
                                 void* stream) {
   PageAddressing addr;
   addr.block_table = block_table;
   addr.table_stride = table_stride;
   addr.seq_lens = seq_lens;
+  addr.window_left = window_left;
   return paged_decode_gqa(q, k_cache, v_cache, out, lse, addr, k_scale, v_scale, batch, n_q_heads,
                           n_kv_heads, head_dim, block_size, num_blocks, q_token_stride,
                           out_token_stride, max_seq_len, sm_scale, workspace, workspace_bytes, q_dtype,
@@ -147,8 +148,8 @@ int xllm_mi355_paged_decode_gqa_static(const void* q, const void* k_cache, const
                                        const int32_t* seq_lens, const float* k_scale, const float* v_scale,
                                        int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim,
                                        int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
-                                       int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
-                                       int q_dtype, int cache_dtype, void* stream) {
+                                       int64_t out_token_stride, int64_t max_seq_len, int64_t window_left,
+                                       float sm_scale, int q_dtype, int cache_dtype, void* stream) {
   if (batch > kWsMaxBatch) return XLLM_MI355_ESCRATCH;  // (a longer batch would be decoded in slices that share the scratch)
   void* ws = nullptr;
   int rc = static_scratch(&ws);
@@ -157,6 +158,7 @@ int xllm_mi355_paged_decode_gqa_static(const void* q, const void* k_cache, const
   addr.block_table = block_table;
   addr.table_stride = table_stride;
   addr.seq_lens = seq_lens;
+  addr.window_left = window_left;
   rc = paged_decode_gqa(q, k_cache, v_cache, out, lse, addr, k_scale, v_scale, batch, n_q_heads, n_kv_heads,
                         head_dim, block_size, num_blocks, q_token_stride, out_token_stride, max_seq_len, sm_scale,
                         ws, kStaticScratchBytes, q_dtype, cache_dtype, static_cast<hipStream_t>(stream));
@@ -170,11 +172,12 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                                     const float* v_scale, int64_t batch, int64_t n_q_heads,
                                     int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
                                     int64_t num_blocks, int64_t q_token_stride,
-                                    int64_t out_token_stride, int64_t max_seq_len, float sm_scale,
-                                    void* workspace, size_t workspace_bytes, int q_dtype,
+                                    int64_t out_token_stride, int64_t max_seq_len, int64_t window_left,
+                                    float sm_scale, void* workspace, size_t workspace_bytes, int q_dtype,
                                     int cache_dtype, void* stream) {
   if (paged_kv_indptr == nullptr) return XLLM_MI355_EINVAL;
   PageAddressing addr;
+  addr.window_left = window_left;
   addr.indptr = paged_kv_indptr;
   addr.indices = paged_kv_indices;
   addr.last_page_len = paged_kv_last_page_len;
@@ -217,12 +220,13 @@ int xllm_mi355_paged_decode_gqa_varlen(const void* q, const void* k_cache, const
                                        int64_t n_tokens, int64_t max_q_len, int64_t n_q_heads, int64_t n_kv_heads,
                                        int64_t head_dim, int64_t block_size, int64_t num_blocks,
                                        int64_t q_token_stride, int64_t out_token_stride,
-                                       int64_t max_seq_len, float sm_scale, int causal, void* workspace,
-                                       size_t workspace_bytes, int q_dtype, int cache_dtype, void* stream) {
+                                       int64_t max_seq_len, int64_t window_left, float sm_scale, int causal,
+                                       void* workspace, size_t workspace_bytes, int q_dtype, int cache_dtype,
+                                       void* stream) {
   return paged_decode_gqa_varlen(q, k_cache, v_cache, out, cu_seqlens_q, kv_seq_lens, block_table,
                                  table_stride, k_scale, v_scale, batch, n_tokens, max_q_len, n_q_heads, n_kv_heads,
                                  head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
-                                 max_seq_len, sm_scale, causal, workspace, workspace_bytes, q_dtype,
+                                 max_seq_len, window_left, sm_scale, causal, workspace, workspace_bytes, q_dtype,
                                  cache_dtype, static_cast<hipStream_t>(stream));
 }
 
@@ -246,6 +250,13 @@ int xllm_mi355_lse_merge(const void* partial_out, const float* partial_lse, void
                          int dtype, void* stream) {
   return lse_merge(partial_out, partial_lse, out, lse, n_shards, batch, n_heads, v_head_dim, dtype,
                    static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_lse_combine(void* out, const void* shared_o, const float* shared_lse, const void* unshared_o,
+                           const float* unshared_lse, int64_t rows, int64_t head_dim, int in_dtype, int out_dtype,
+                           void* stream) {
+  return lse_combine(out, shared_o, shared_lse, unshared_o, unshared_lse, rows, head_dim, in_dtype, out_dtype,
+                     static_cast<hipStream_t>(stream));
 }
 
 int xllm_mi355_rope_and_cache(void* qkv, const void* q_weight, const void* k_weight, const void* cos_sin_cache,

@@ -36,6 +36,8 @@ struct PageAddressing {
   const int32_t* indptr = nullptr;       // CSR when non-null: [B+1]
   const int32_t* indices = nullptr;
   const int32_t* last_page_len = nullptr;
+  // sliding window: the query at position L - 1 attends to positions >= L - 1 - window_left; negative: all
+  int64_t window_left = -1;
 };
 
 // Layout of a decode workspace, the same for every decode entry point and independent of the batch, so that
@@ -84,12 +86,16 @@ int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_ca
                             const float* v_scale, int64_t batch, int64_t n_tokens, int64_t max_q_len,
                             int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
                             int64_t num_blocks, int64_t q_token_stride, int64_t out_token_stride,
-                            int64_t max_seq_len, float sm_scale, int causal, void* workspace,
+                            int64_t max_seq_len, int64_t window_left, float sm_scale, int causal, void* workspace,
                             size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream);
 
 int lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,
               int64_t n_shards, int64_t batch, int64_t n_heads, int64_t v_head_dim, int dtype,
               hipStream_t stream);
+
+int lse_combine(void* out, const void* shared_o, const float* shared_lse, const void* unshared_o,
+                const float* unshared_lse, int64_t rows, int64_t head_dim, int in_dtype, int out_dtype,
+                hipStream_t stream);
 
 int build_block_table(const int32_t* indptr, const int32_t* indices, const int32_t* last_page_len,
                       int32_t* block_table, int64_t table_stride, int32_t* seq_lens, int64_t batch,

@@ -56,6 +56,32 @@ __global__ __launch_bounds__(128) void lse_merge_kernel(const char* partial_out,
   if (lse != nullptr && threadIdx.x == 0) lse[i] = wsum > 0.0f ? safe_max + logf(wsum) : -INFINITY;
 }
 
+// Two-way combine with base-2 LSEs, one workgroup per (batch, head) row, the arithmetic of the reference kernel
+// in its order (xllm/core/kernels/cuda/xattention/lse_combine.cu:41-85): maximum, exp2 of both against it, merged
+// LSE = max + log2(sum), weights exp2(lse - merged), weighted sum, one rounding to the output type.
+template <int IN, int OUT>
+__global__ __launch_bounds__(128) void lse_combine_kernel(char* out, const char* shared_o, const float* shared_lse,
+                                                          const char* unshared_o, const float* unshared_lse, int d_total) {
+  const int64_t idx = blockIdx.x;
+  const float a = shared_lse[idx], b = unshared_lse[idx];
+  const float lse_max = fmaxf(a, b);
+  const float ea = exp2f(a - lse_max), eb = exp2f(b - lse_max);
+  const float lse_new = lse_max + log2f(ea + eb);
+  const float wa = exp2f(a - lse_new), wb = exp2f(b - lse_new);
+  auto load = [](const char* p, int64_t i) -> float {
+    if constexpr (IN == XLLM_MI355_FP32) return reinterpret_cast<const float*>(p)[i];
+    else if constexpr (IN == XLLM_MI355_BF16) return BF16::to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+    else return FP16::to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  };
+  for (int d = threadIdx.x; d < d_total; d += 128) {
+    const int64_t i = idx * d_total + d;
+    const float v = wa * load(shared_o, i) + wb * load(unshared_o, i);
+    if constexpr (OUT == XLLM_MI355_FP32) reinterpret_cast<float*>(out)[i] = v;
+    else if constexpr (OUT == XLLM_MI355_BF16) reinterpret_cast<uint16_t*>(out)[i] = BF16::from_f32(v);
+    else reinterpret_cast<uint16_t*>(out)[i] = FP16::from_f32(v);
+  }
+}
+
 __global__ __launch_bounds__(256) void build_block_table_kernel(const int32_t* indptr,
                                                                 const int32_t* indices,
                                                                 const int32_t* last_page_len,
@@ -248,7 +274,7 @@ int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_ca
                             const float* v_scale, int64_t batch, int64_t n_tokens, int64_t max_q_len,
                             int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
                             int64_t num_blocks, int64_t q_token_stride, int64_t out_token_stride,
-                            int64_t max_seq_len, float sm_scale, int causal, void* workspace,
+                            int64_t max_seq_len, int64_t window_left, float sm_scale, int causal, void* workspace,
                             size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream) {
   if (batch == 0 || n_tokens == 0) return XLLM_MI355_OK;
   if (cu_seqlens_q == nullptr || kv_seq_lens == nullptr || block_table == nullptr || table_stride <= 0)
@@ -266,7 +292,8 @@ int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_ca
   // blocks an entry per token is cheaper, its repeated page reads being served partly by L2
   const int64_t per = group <= 16 ? 16 / group : 0;
   const int64_t blocks = per > 0 && max_q_len > 0 ? (max_q_len + per - 1) / per : 0;
-  if (blocks >= 1 && blocks <= 16 && (per >= 2 || blocks == 1) && head_dim == 128 && pow2 && out_aligned) {
+  // (with a sliding window every token has its own first position: the per-token path below serves that)
+  if (window_left < 0 && blocks >= 1 && blocks <= 16 && (per >= 2 || blocks == 1) && head_dim == 128 && pow2 && out_aligned) {
     PageAddressing addr;
     addr.chunk_blocks = static_cast<int>(blocks);
     addr.block_table = block_table;
@@ -297,6 +324,7 @@ int paged_decode_gqa_varlen(const void* q, const void* k_cache, const void* v_ca
   addr.table_stride = table_stride;
   addr.seq_lens = tok_lens;
   addr.table_rows = tok_rows;
+  addr.window_left = window_left;   // token j sits at position tok_lens[j] - 1 of its own attended range
   return paged_decode_gqa(q, k_cache, v_cache, out, nullptr, addr, k_scale, v_scale, n_tokens, n_q_heads,
                           n_kv_heads, head_dim, block_size, num_blocks, q_token_stride, out_token_stride,
                           max_seq_len, sm_scale, workspace, usable, q_dtype, cache_dtype, stream);
@@ -326,6 +354,37 @@ int lse_merge(const void* partial_out, const float* partial_lse, void* out, floa
       break;
     default: return XLLM_MI355_EDTYPE;
   }
+  return static_cast<int>(hipGetLastError());
+}
+
+int lse_combine(void* out, const void* shared_o, const float* shared_lse, const void* unshared_o,
+                const float* unshared_lse, int64_t rows, int64_t head_dim, int in_dtype, int out_dtype,
+                hipStream_t stream) {
+  if (rows == 0 || head_dim == 0) return XLLM_MI355_OK;
+  if (out == nullptr || shared_o == nullptr || shared_lse == nullptr || unshared_o == nullptr || unshared_lse == nullptr)
+    return XLLM_MI355_EINVAL;
+  if (rows < 0 || rows > 0x7fffffffLL || head_dim < 0 || head_dim > 0x7fffffffLL) return XLLM_MI355_EINVAL;
+  const dim3 grid(static_cast<unsigned>(rows));
+  char* o = static_cast<char*>(out);
+  const char* s = static_cast<const char*>(shared_o);
+  const char* u = static_cast<const char*>(unshared_o);
+  const int d = static_cast<int>(head_dim);
+#define XLLM_COMBINE(IN, OUT) lse_combine_kernel<IN, OUT><<<grid, 128, 0, stream>>>(o, s, shared_lse, u, unshared_lse, d)
+#define XLLM_COMBINE_OUT(IN)                                                    \
+  switch (out_dtype) {                                                          \
+    case XLLM_MI355_BF16: XLLM_COMBINE(IN, XLLM_MI355_BF16); break;             \
+    case XLLM_MI355_FP16: XLLM_COMBINE(IN, XLLM_MI355_FP16); break;             \
+    case XLLM_MI355_FP32: XLLM_COMBINE(IN, XLLM_MI355_FP32); break;             \
+    default: return XLLM_MI355_EDTYPE;                                          \
+  }
+  switch (in_dtype) {
+    case XLLM_MI355_BF16: XLLM_COMBINE_OUT(XLLM_MI355_BF16); break;
+    case XLLM_MI355_FP16: XLLM_COMBINE_OUT(XLLM_MI355_FP16); break;
+    case XLLM_MI355_FP32: XLLM_COMBINE_OUT(XLLM_MI355_FP32); break;
+    default: return XLLM_MI355_EDTYPE;
+  }
+#undef XLLM_COMBINE_OUT
+#undef XLLM_COMBINE
   return static_cast<int>(hipGetLastError());
 }
 

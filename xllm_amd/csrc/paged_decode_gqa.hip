@@ -88,6 +88,7 @@ struct GqaArgs {
   int num_blocks;
   int n_workgroups;   // workers of the decode kernel (workgroups; wavefront pairs of the matrix-core kernel)
   int wait_spins;     // bound of the polls of one wavefront of a pair on the other
+  int window_left;    // sliding window: the query (position L - 1) attends to positions >= L - 1 - window_left; < 0: all
   float scale_log2;   // sm_scale * log2(e)
 };
 
@@ -103,8 +104,15 @@ __device__ __forceinline__ void sequence_of(const GqaArgs& a, int b, const int32
   }
 }
 
+// First token a query at position L - 1 attends to (0 without a sliding window).
+__device__ __forceinline__ int first_token(const GqaArgs& a, int L) {
+  return a.window_left < 0 ? 0 : max(0, L - 1 - a.window_left);
+}
+// Items of a context: those that hold a token of the attended range [first_token, L).
 template <int ITEM>
-__device__ __forceinline__ int items_of(int L) { return L > 0 ? (L + ITEM - 1) / ITEM : 0; }
+__device__ __forceinline__ int items_of(const GqaArgs& a, int L) {
+  return L > 0 ? (L + ITEM - 1) / ITEM - first_token(a, L) / ITEM : 0;
+}
 
 // First flat item of workgroup w when `total` items are dealt to `n` workgroups.
 __device__ __forceinline__ int64_t range_start(int64_t w, int64_t total, int64_t n) { return w * total / n; }
@@ -130,7 +138,7 @@ __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* 
     const int32_t* pages;
     int L;
     sequence_of(a, b, pages, L);
-    local += items_of<ITEM>(L);
+    local += items_of<ITEM>(a, L);
     last_len = L;
   }
   if (on) tmp[tid] = local;
@@ -148,7 +156,7 @@ __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* 
         int L;
         sequence_of(a, b, pages, L);
         prefix[b] = excl;
-        excl += items_of<ITEM>(L);
+        excl += items_of<ITEM>(a, L);
       }
     }
     if (hi == a.batch) prefix[a.batch] = excl;  // the last non-empty slice holds the total
@@ -258,8 +266,10 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
     const int kvh = hbk / hb_per_kv;
     const int h0 = kvh * a.group + (hbk % hb_per_kv) * G;
     const int nh = min(G, (kvh + 1) * a.group - h0);
-    const int run_t0 = item0 * kItem;
-    const int run_t1 = min(L, (item0 + run_items) * kItem);
+    const int win_lo = first_token(a, L);   // tokens before it lie outside the sliding window
+    const int item_lo = win_lo / kItem;     // first item of the context that is scheduled
+    const int run_t0 = (item_lo + item0) * kItem;
+    const int run_t1 = min(L, (item_lo + item0 + run_items) * kItem);
 
     // query registers: for each head the 16-bit pairs matching this lane's cache columns
     u32 qreg[G][NLD][EPL / 2];
@@ -363,7 +373,7 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
             s[u][h] = group_sum<LPT>(d);
           }
           if constexpr (MASKED) {
-            if (t0 + step * STEP + u * TPP + r >= t1) {
+            if (t0 + step * STEP + u * TPP + r >= t1 || t0 + step * STEP + u * TPP + r < win_lo) {
 #pragma unroll
               for (int h = 0; h < G; ++h) s[u][h] = -INFINITY;
             }
@@ -432,7 +442,7 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
       };
 
       auto compute = [&](const Tile& t, int step) {
-        if (ragged && step == n_steps - 1) compute_tile(t, step, std::true_type{});
+        if ((ragged && step == n_steps - 1) || t0 + step * STEP < win_lo) compute_tile(t, step, std::true_type{});
         else compute_tile(t, step, std::false_type{});
       };
 
@@ -533,34 +543,10 @@ constexpr float kSlack = 8.0f;
 constexpr int kStageBytes = 8192;  // K rows then V rows: 16 tokens of 16-bit pages, 32 of fp8 pages
 constexpr int kMfmaHeads = 16;                        // head columns of one MFMA
 
-typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((ext_vector_type(2))) int i32x2;
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
 typedef __attribute__((address_space(3))) volatile int lds_vint;  // a word of LDS that other wavefronts write
-typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-
-template <typename QT>
-struct Mfma;
-template <>
-struct Mfma<BF16> {
-  static __device__ __forceinline__ f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ f32x4 k16(s16x4 a, u32x2 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
-  }
-};
-template <>
-struct Mfma<FP16> {
-  static __device__ __forceinline__ f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ f32x4 k16(s16x4 a, u32x2 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
-  }
-};
 
 // 16 (4) bytes per lane from global memory straight into LDS at lds_addr + lane * 16 (4);
 // lds_addr is wave-uniform and travels in M0.
@@ -628,6 +614,7 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
 // Position of a stage in the flat list (sequence, head block, stage of 16 tokens).
 struct CtxCursor {
   int b, hbk, st, n_st;
+  int st0;  // first scheduled stage of the context (stages before it lie outside the sliding window)
   int kvh;  // KV head of the head block: hbk / (head blocks per KV head)
   int L;
   const int32_t* pages;
@@ -635,6 +622,7 @@ struct CtxCursor {
   // the column block hbk % chunk_blocks holds: its first token, its number of tokens, and the index of its
   // first token inside the chunk
   int Q0, QN, q0, qn, jb;
+  int QF;  // the chunk's full length (QN is cut to what the column blocks hold): the causal offset counts from it
 };
 // Field by field, and the chunk fields only where they are in use: a whole-struct copy with fields that
 // were never written goes through scratch memory, whose loads count on the same counter as the stages
@@ -645,12 +633,14 @@ __device__ __forceinline__ void copy_cursor(CtxCursor& d, const CtxCursor& s) {
   d.hbk = s.hbk;
   d.kvh = s.kvh;
   d.st = s.st;
+  d.st0 = s.st0;
   d.n_st = s.n_st;
   d.L = s.L;
   d.pages = s.pages;
   if constexpr (VL) {
     d.Q0 = s.Q0;
     d.QN = s.QN;
+    d.QF = s.QF;
     d.q0 = s.q0;
     d.qn = s.qn;
     d.jb = s.jb;
@@ -723,7 +713,8 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   auto chunk_of = [&](CtxCursor& cu) {
     if constexpr (VL) {
       cu.Q0 = sload32(a.cu_q + cu.b);
-      cu.QN = max(0, min(sload32(a.cu_q + cu.b + 1) - cu.Q0, hb_per_kv * (G / a.group)));
+      cu.QF = max(0, sload32(a.cu_q + cu.b + 1) - cu.Q0);
+      cu.QN = min(cu.QF, hb_per_kv * (G / a.group));
       chunk_part(cu);
     }
   };
@@ -801,6 +792,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     cu.st = __builtin_amdgcn_readfirstlane(static_cast<int>(rem - static_cast<int64_t>(cu.hbk) * cu.n_st));
     cu.kvh = cu.hbk / hb_per_kv;
     sequence_at(cu.b, cu.pages, cu.L);
+    cu.st0 = first_token(a, cu.L) / T;
     chunk_of(cu);
   };
   auto next_context = [&](CtxCursor& cu) {  // the caller never steps past the last context of the batch
@@ -817,6 +809,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       cu.n_st = __builtin_amdgcn_readfirstlane(prefix[cu.b + 1] - prefix[cu.b]);
     } while (cu.n_st == 0);
     sequence_at(cu.b, cu.pages, cu.L);
+    cu.st0 = first_token(a, cu.L) / T;
     chunk_of(cu);
   };
   // 64 entries of the context's page table, from page 64 ck on (the tail repeats the last page),
@@ -869,14 +862,14 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   };
   auto begin_context = [&](bool first) {
     if (first) {
-      ck_a = ((pc.st * T) >> a.bs_shift) >> 6;
+      ck_a = (((pc.st0 + pc.st) * T) >> a.bs_shift) >> 6;
       issue_chunk(pc, ck_a, off_a);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     } else {
       const u32 t = off_a;
       off_a = off_c;
       off_c = t;
-      ck_a = 0;
+      ck_a = ((pc.st0 * T) >> a.bs_shift) >> 6;   // the chunk that was fetched ahead: the one of the first stage
       ensure_landed(has_c, t_c);
     }
     has_b = has_c = false;
@@ -884,7 +877,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     if (pc.n_st - pc.st < n_stages - p) {  // the range goes on into another context
       copy_cursor<VL>(pn, pc);
       next_context(pn);
-      issue_chunk(pn, 0, off_c);
+      issue_chunk(pn, ((pn.st0 * T) >> a.bs_shift) >> 6, off_c);
       t_c = p;
       has_c = true;
     }
@@ -928,7 +921,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       copy_cursor<VL>(pc, pn);
       begin_context(false);
     }
-    const int tok0 = pc.st * T;
+    const int tok0 = (pc.st0 + pc.st) * T;
     const int lim = pc.L - tok0 - 1;  // last valid row of the stage
     // block size >= 16: a sub-block of 16 tokens lies in one page
     constexpr int NSUB = T / 16;
@@ -1023,6 +1016,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   bool complete = false;
   int h0 = 0, nh = 0;
   int Lc = 0;                 // tokens the lane's column attends to (the context length unless VL and causal)
+  int Lo = 0;                 // first token it attends to (0 without a sliding window)
   int64_t out_off = 0;        // VL: byte offset of the lane's output row
   int c_ctx_first = 0, c_prev_len = 0;
   u32x4 q[KS];
@@ -1050,7 +1044,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         nh = cc.qn * a.group;
         const int col = max(0, min(c16, nh - 1));
         const int j = col / a.group;
-        Lc = a.causal != 0 ? cc.L - (cc.QN - 1 - (cc.jb + j)) : cc.L;
+        Lc = a.causal != 0 ? cc.L - (cc.QF - 1 - (cc.jb + j)) : cc.L;
         const int tok = max(0, min(cc.q0 + j, a.n_tokens - 1));
         out_off = tok * a.out_stride_bytes + (static_cast<int64_t>(kvh * a.group + (col - j * a.group)) * D) * 2;
       } else {
@@ -1058,6 +1052,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         nh = min(G, (kvh + 1) * a.group - h0);
         Lc = cc.L;
       }
+      Lo = first_token(a, cc.L);
       complete = cc.st == 0 && cc.n_st <= n_stages - s;
       if (s == 0 || c_prev_len >= NS) {
 #pragma unroll
@@ -1110,12 +1105,12 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       sc = Mfma<QT>::k32(kr[2], q[2], sc);
       sc1 = Mfma<QT>::k32(kr[3], q[3], sc1);
       sc += sc1;
-      const int tok0 = cc.st * T + 4 * g;
+      const int tok0 = (cc.st0 + cc.st) * T + 4 * g;
       float sv[4];
       bool over = false;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        sv[r] = tok0 + r < Lc ? sc[r] * score_scale : -INFINITY;
+        sv[r] = tok0 + r < Lc && tok0 + r >= Lo ? sc[r] * score_scale : -INFINITY;
         over |= sv[r] > m + kSlack;
       }
       if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
@@ -1164,10 +1159,10 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) sc = Mfma<QT>::k32(kr[tb][kk], q[kk], sc);
-        const int tok0 = cc.st * T + tb * 16 + 4 * g;
+        const int tok0 = (cc.st0 + cc.st) * T + tb * 16 + 4 * g;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          sv[tb * 4 + r] = tok0 + r < Lc ? sc[r] * score_scale : -INFINITY;
+          sv[tb * 4 + r] = tok0 + r < Lc && tok0 + r >= Lo ? sc[r] * score_scale : -INFINITY;
           over |= sv[tb * 4 + r] > m + kSlack;
         }
       }
@@ -1213,10 +1208,10 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
                             QT::template from_fp8x2<false>(k8[1]), QT::template from_fp8x2<true>(k8[1])};
           sc = Mfma<QT>::k32(kr, q[kk], sc);
         }
-        const int tok0 = cc.st * T + tb * 16 + 4 * g;
+        const int tok0 = (cc.st0 + cc.st) * T + tb * 16 + 4 * g;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          sv[tb * 4 + r] = tok0 + r < Lc ? sc[r] * score_scale : -INFINITY;
+          sv[tb * 4 + r] = tok0 + r < Lc && tok0 + r >= Lo ? sc[r] * score_scale : -INFINITY;
           over |= sv[tb * 4 + r] > m + kSlack;
         }
       }
@@ -1574,7 +1569,8 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     bool pow2 = false;
     for (int s = 4; s < 31; ++s) pow2 |= (1LL << s) == block_size;
     if (csr || lse != nullptr || head_dim != 128 || !pow2 || !out_aligned || group > kMfmaHeads ||
-        addr.n_tokens <= 0 || addr.n_tokens > 0x7fffffffLL || addr.chunk_blocks <= 0 || addr.chunk_blocks > kMfmaHeads)
+        addr.n_tokens <= 0 || addr.n_tokens > 0x7fffffffLL || addr.chunk_blocks <= 0 || addr.chunk_blocks > kMfmaHeads ||
+        addr.window_left >= 0)
       return XLLM_MI355_EINVAL;
   }
   // Batches beyond the LDS prefix capacity are decoded in slices; each slice is an
@@ -1602,6 +1598,7 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     a.ws_status = static_cast<int*>(workspace);
     a.ws_prefix = reinterpret_cast<int*>(static_cast<char*>(workspace) + kWsHeaderBytes);
     a.wait_spins = wait_spin_limit();
+    a.window_left = addr.window_left < 0 ? -1 : static_cast<int>(addr.window_left < 0x7fffffffLL ? addr.window_left : 0x7fffffffLL);
     a.table_stride = addr.table_stride;
     a.q_stride_bytes = q_token_stride * 2;
     a.out_stride_bytes = out_token_stride * 2;

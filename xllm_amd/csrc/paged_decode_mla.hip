@@ -57,14 +57,11 @@ constexpr int kXchPOff = 2 * kTileBytes;
 constexpr int kXchMOff = kXchPOff + 4 * 8 * 64 * 4;
 constexpr int kPrefixOff = kXchMOff + 4 * 32 * 4;
 
-typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 typedef __attribute__((address_space(3))) float lds_f32;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-
 struct MlaArgs {
   const char* q_nope;
   const char* q_pe;
@@ -118,6 +115,7 @@ __device__ __forceinline__ void dma16_row(uint64_t row_base, u32 lane_off, u32 l
 }
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+template <typename QT>
 __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
   extern __shared__ __align__(16) char smem[];
   u32* xch_p = reinterpret_cast<u32*>(smem + kXchPOff);
@@ -193,7 +191,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     const int L = a.seq_lens[b];
 
     // Q^T operand: lane (head c32, k-group g) keeps dims ks*16 + g*8 .. +8 of every k-step
-    bf16x8 q[kKSteps];
+    u32x4 q[kKSteps];
     {
       const char* qn = a.q_nope + (static_cast<int64_t>(b) * H + head) * kDL * 2;
       const char* qp = a.q_pe + (static_cast<int64_t>(b) * H + head) * kDR * 2;
@@ -202,7 +200,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         u32x4 x = {0u, 0u, 0u, 0u};
         if (head_ok)
           x = ks < kDL / 16 ? ldg16(qn + (ks * 16 + g * 8) * 2) : ldg16(qp + ((ks - kDL / 16) * 16 + g * 8) * 2);
-        q[ks] = __builtin_bit_cast(bf16x8, x);
+        q[ks] = x;
       }
     }
     f32x16 o[8];  // O^T blocks: dims tblk*256 + mb*32 + (8*(r/4) + 4g + r%4), head c32
@@ -253,7 +251,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
     for (int ks = 0; ks < kKSteps; ++ks) {
       u32x4 x = __builtin_bit_cast(u32x4, q[ks]);
       asm volatile("" : "+v"(x));
-      q[ks] = __builtin_bit_cast(bf16x8, x);
+      q[ks] = x;
     }
     __syncthreads();  // the previous run no longer reads the tiles or the exchange buffers
     int off_next = 0;
@@ -284,8 +282,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         for (int ks = 0; ks < kKSteps; ks += 2) {
           const u32x4 x0 = *reinterpret_cast<const u32x4*>(ka + ks * 32);
           const u32x4 x1 = *reinterpret_cast<const u32x4*>(ka + ks * 32 + 32);
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x0), q[ks], s, 0, 0, 0);
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x1), q[ks + 1], s, 0, 0, 0);
+          s = Mfma<QT>::w32(x0, q[ks], s);
+          s = Mfma<QT>::w32(x1, q[ks + 1], s);
         }
         // pipeline the LDS operand reads four MFMAs ahead of their use
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -311,7 +309,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
           sum_own += s[r];
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) pk_own[i] = BF16::pack(s[2 * i], s[2 * i + 1]);
+        for (int i = 0; i < 8; ++i) pk_own[i] = QT::pack(s[2 * i], s[2 * i + 1]);
 #pragma unroll
         for (int i = 0; i < 8; ++i) xch_p[(wave * 8 + i) * 64 + lane] = pk_own[i];
         if (g == 0) xch_m[wave * 32 + c32] = m_own;
@@ -342,19 +340,19 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
         }
         // B operands per k-step: k-slot g*8 + j <-> rows 16*kk + 4g + j (j < 4), + 8 more (j >= 4)
         // of the own token block (pb_own) and of the partner's (pb_other)
-        bf16x8 pb_own[2], pb_other[2];
+        u32x4 pb_own[2], pb_other[2];
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
           u32x4 mine, theirs;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const u32 w = pk_own[4 * kk + i];
-            mine[i] = BF16::pack(BF16::lo(w) * f_own, BF16::hi(w) * f_own);
+            mine[i] = QT::pack(QT::lo(w) * f_own, QT::hi(w) * f_own);
             const u32 t = theirs_raw[4 * kk + i];
-            theirs[i] = BF16::pack(BF16::lo(t) * f_other, BF16::hi(t) * f_other);
+            theirs[i] = QT::pack(QT::lo(t) * f_other, QT::hi(t) * f_other);
           }
-          pb_own[kk] = __builtin_bit_cast(bf16x8, mine);
-          pb_other[kk] = __builtin_bit_cast(bf16x8, theirs);
+          pb_own[kk] = mine;
+          pb_other[kk] = theirs;
         }
         // ---- O^T += V^T . P^T over the 64 tokens, dims tblk*256 .. +256.  The transposing
         // LDS load works on groups of 16 lanes: lane p of a group supplies the address of 4
@@ -373,8 +371,7 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
             const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows));
             const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows + 8 * kLdsRow));
             const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-            o[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                __builtin_bit_cast(bf16x8, v), ks < 2 ? pb_own[ks & 1] : pb_other[ks & 1], o[mb], 0, 0, 0);
+            o[mb] = Mfma<QT>::w32(__builtin_bit_cast(u32x4, v), ks < 2 ? pb_own[ks & 1] : pb_other[ks & 1], o[mb]);
           }
         }
         // pipeline the transposing reads (two per MFMA) four MFMAs ahead of their use
@@ -404,8 +401,8 @@ __global__ __launch_bounds__(kMlaThreads) void mla_decode_kernel(MlaArgs a) {
 #pragma unroll
           for (int qd = 0; qd < 4; ++qd) {
             u32x2 w;
-            w[0] = BF16::pack(o[mb][4 * qd] * inv, o[mb][4 * qd + 1] * inv);
-            w[1] = BF16::pack(o[mb][4 * qd + 2] * inv, o[mb][4 * qd + 3] * inv);
+            w[0] = QT::pack(o[mb][4 * qd] * inv, o[mb][4 * qd + 1] * inv);
+            w[1] = QT::pack(o[mb][4 * qd + 2] * inv, o[mb][4 * qd + 3] * inv);
             *reinterpret_cast<u32x2*>(op + (mb * 32 + 8 * qd + 4 * g) * 2) = w;
           }
         if (a.lse != nullptr && g == 0 && tblk == 0) a.lse[b * H + head] = (m + fast_log2(lsum)) * kLn2;
@@ -504,7 +501,7 @@ __device__ __forceinline__ void wait_younger_subs(int subs) {
 // every sub-tile then go to different wavefronts: wavefront (head block w % 4, token block w / 4)
 // keeps its own maximum, sum and O^T, and at the end of a run the token-block-1 wavefronts hand
 // theirs to their partners through the (then idle) ring, merged like two partials.
-template <bool SPLIT>
+template <typename QT, bool SPLIT>
 __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kPrefix16Off);
@@ -688,7 +685,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
           for (int kk = 0; kk < kKSteps32; ++kk) {
             const char* k0 = kk < kDL / 32 ? ka + kk * 64 : kr + tb * 16 * (kDR * 2) + (kk == kDL / 32 ? kr_x : kr_x ^ 4) * 16;
             const u32x4 x0 = *reinterpret_cast<const u32x4*>(k0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x0), __builtin_bit_cast(bf16x8, q[kk]), s0, 0, 0, 0);
+            s0 = Mfma<QT>::k32(x0, q[kk], s0);
           }
           __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
@@ -722,15 +719,14 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
             p[r] = fast_exp2(sv[r] - m);
             l += p[r];
           }
-          const u32x2 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3])};
-          const s16x4 pb = __builtin_bit_cast(s16x4, pbw);
+          const u32x2 pb = {QT::pack(p[0], p[1]), QT::pack(p[2], p[3])};
           // ---- O^T += V^T . P^T over the 16 tokens: k-slot 4g + j of the MFMA <-> token 4g + j of the block
           const char* va = kb + v_row0 + tb * 16 * kRow16;
           __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the P.V reads only
 #pragma unroll
           for (int mb = 0; mb < 32; ++mb) {
             const s16x4 v4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
-            o[mb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(v4, pb, o[mb], 0, 0, 0);
+            o[mb] = Mfma<QT>::k16(v4, pb, o[mb]);
           }
           __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
@@ -750,8 +746,8 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
             const char* k0 = kk < kDL / 32 ? ka + kk * 64 : kr + (kk == kDL / 32 ? kr_x : kr_x ^ 4) * 16;
             const u32x4 x0 = *reinterpret_cast<const u32x4*>(k0);
             const u32x4 x1 = *reinterpret_cast<const u32x4*>(k0 + 16 * (kk < kDL / 32 ? kRow16 : kDR * 2));
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x0), __builtin_bit_cast(bf16x8, q[kk]), s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x1), __builtin_bit_cast(bf16x8, q[kk]), s1, 0, 0, 0);
+            s0 = Mfma<QT>::k32(x0, q[kk], s0);
+            s1 = Mfma<QT>::k32(x1, q[kk], s1);
           }
           // pipeline the LDS operand reads kAhead MFMAs ahead of their use
           __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
@@ -792,8 +788,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
             l += p[r];
           }
           // k-slot g*8 + j of the P.V MFMA <-> token 4g + j of block 0 (j < 4), of block 1 (j >= 4)
-          const u32x4 pbw = {BF16::pack(p[0], p[1]), BF16::pack(p[2], p[3]), BF16::pack(p[4], p[5]), BF16::pack(p[6], p[7])};
-          const bf16x8 pb = __builtin_bit_cast(bf16x8, pbw);
+          const u32x4 pb = {QT::pack(p[0], p[1]), QT::pack(p[2], p[3]), QT::pack(p[4], p[5]), QT::pack(p[6], p[7])};
           // ---- O^T += V^T . P^T over the 32 tokens and all 512 dims.  The transposing LDS load works on
           // groups of 16 lanes: lane p of a group supplies the address of 4 dims of token row p/4 and
           // receives the 4 tokens of dim column p.
@@ -804,7 +799,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
             const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + mb * 32));
             const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + 16 * kRow16 + mb * 32));
             const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-            o[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, v), pb, o[mb], 0, 0, 0);
+            o[mb] = Mfma<QT>::k32(__builtin_bit_cast(u32x4, v), pb, o[mb]);
           }
           // pipeline the transposing reads (two per MFMA) kAhead MFMAs ahead of their use
           __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
@@ -857,7 +852,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
       char* op = a.out + ((static_cast<int64_t>(b) * H + head) * kDL + 4 * g) * 2;
 #pragma unroll
       for (int mb = 0; mb < 32; ++mb) {
-        const u32x2 w = {BF16::pack(o[mb][0] * inv, o[mb][1] * inv), BF16::pack(o[mb][2] * inv, o[mb][3] * inv)};
+        const u32x2 w = {QT::pack(o[mb][0] * inv, o[mb][1] * inv), QT::pack(o[mb][2] * inv, o[mb][3] * inv)};
         *reinterpret_cast<u32x2*>(op + mb * 32) = w;
       }
     }
@@ -1448,6 +1443,7 @@ __global__ __launch_bounds__(kWThreads) void mla_decode32w_kernel(MlaArgs a) {
 
 // Merge of the partials of contexts that span several teams; also writes the output of
 // empty sequences.  One workgroup per (head, sequence).
+template <typename QT>
 __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
   // One workgroup per (head, sequence); thread t owns dims 4t .. 4t+3, read from the fp32 partials
   // with 16-byte loads.  Two dependent round trips to memory: the tile prefix, then the LSEs and
@@ -1506,7 +1502,7 @@ __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
     M = m_new;
   }
   const float inv = 1.0f / W;
-  *reinterpret_cast<u32x2*>(out) = u32x2{BF16::pack(O[0] * inv, O[1] * inv), BF16::pack(O[2] * inv, O[3] * inv)};
+  *reinterpret_cast<u32x2*>(out) = u32x2{QT::pack(O[0] * inv, O[1] * inv), QT::pack(O[2] * inv, O[3] * inv)};
   if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = (M + fast_log2(W)) * kLn2;
 }
 
@@ -1570,7 +1566,8 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       !(sm_scale > 0.0f))
     return XLLM_MI355_EINVAL;
   if (d_latent != kDL || d_rope != kDR) return XLLM_MI355_ESHAPE;
-  if (dtype != XLLM_MI355_BF16) return XLLM_MI355_EDTYPE;
+  if (dtype != XLLM_MI355_BF16 && dtype != XLLM_MI355_FP16) return XLLM_MI355_EDTYPE;
+  const bool f16 = dtype == XLLM_MI355_FP16;
   if (num_blocks * block_size > 0x7fffffffLL) return XLLM_MI355_ESHAPE;
   auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   if (!aligned16(q_nope) || !aligned16(q_pe) || !aligned16(k_cache) || !aligned16(out))
@@ -1584,24 +1581,26 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   // producer / consumer kernel
   const int knob = mla_kernel_knob();
   const bool pairs = knob == 'p' || block_size < 16 || (block_size & (block_size - 1)) != 0;
-  const bool split = knob == 's' && !pairs;
+  const bool split = knob == 's' && !pairs && !f16;  // (the producer / consumer kernel is written for bf16)
   const int n_hb = static_cast<int>(pairs ? (n_heads + kHeadsPerWg - 1) / kHeadsPerWg
                                           : (n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
   const int n_hb_p = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
   static std::atomic<uint64_t> configured{0};
   const size_t smem = pairs ? kPrefixOff + (kMaxBatchMla + 1) * 4 : kPrefix16Off + (kMaxBatchMla + 1) * 4;
   if (first_use_on_current_device(configured)) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       static_cast<int>(kPrefixOff + (kMaxBatchMla + 1) * 4));
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode16_kernel<false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kPrefix16Off + (kMaxBatchMla + 1) * 4));
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode16_kernel<true>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kPrefix16Off + (kMaxBatchMla + 1) * 4));
+    hipError_t e = hipSuccess;
+    const int lds_pairs = static_cast<int>(kPrefixOff + (kMaxBatchMla + 1) * 4);
+    const int lds_16 = static_cast<int>(kPrefix16Off + (kMaxBatchMla + 1) * 4);
+    const void* pairs_kernels[] = {reinterpret_cast<const void*>(mla_decode_kernel<BF16>),
+                                   reinterpret_cast<const void*>(mla_decode_kernel<FP16>)};
+    const void* kernels_16[] = {reinterpret_cast<const void*>(mla_decode16_kernel<BF16, false>),
+                                reinterpret_cast<const void*>(mla_decode16_kernel<BF16, true>),
+                                reinterpret_cast<const void*>(mla_decode16_kernel<FP16, false>),
+                                reinterpret_cast<const void*>(mla_decode16_kernel<FP16, true>)};
+    for (const void* k : pairs_kernels)
+      if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_pairs);
+    for (const void* k : kernels_16)
+      if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_16);
     if (e == hipSuccess)
       e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode32w_kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
@@ -1633,17 +1632,24 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.ws_out = reinterpret_cast<float*>(static_cast<char*>(workspace) + kWsPartialsOff);
     a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * n_heads * kDL;
 
-    if (pairs)
-      launch_timed(mla_decode_kernel, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kMlaThreads), smem, stream, a);
-    else if (use_p)
-      launch_timed(mla_decode32w_kernel, dim3(static_cast<unsigned>(a.n_teams * a.n_hb)), dim3(kWThreads), kPLdsBytes, stream, a);
-    else if (n_heads <= 64)  // head counts of tensor-parallel shards: two wavefronts per 16 heads
-      launch_timed(mla_decode16_kernel<true>, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kThreads16), smem, stream, a);
-    else
-      launch_timed(mla_decode16_kernel<false>, dim3(static_cast<unsigned>(a.n_teams * n_hb)), dim3(kThreads16), smem, stream, a);
+    const dim3 grid(static_cast<unsigned>(a.n_teams * a.n_hb));
+    if (pairs) {
+      if (f16) launch_timed(mla_decode_kernel<FP16>, grid, dim3(kMlaThreads), smem, stream, a);
+      else launch_timed(mla_decode_kernel<BF16>, grid, dim3(kMlaThreads), smem, stream, a);
+    } else if (use_p) {
+      launch_timed(mla_decode32w_kernel, grid, dim3(kWThreads), kPLdsBytes, stream, a);
+    } else if (n_heads <= 64) {  // head counts of tensor-parallel shards: two wavefronts per 16 heads
+      if (f16) launch_timed(mla_decode16_kernel<FP16, true>, grid, dim3(kThreads16), smem, stream, a);
+      else launch_timed(mla_decode16_kernel<BF16, true>, grid, dim3(kThreads16), smem, stream, a);
+    } else {
+      if (f16) launch_timed(mla_decode16_kernel<FP16, false>, grid, dim3(kThreads16), smem, stream, a);
+      else launch_timed(mla_decode16_kernel<BF16, false>, grid, dim3(kThreads16), smem, stream, a);
+    }
     int rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
-    launch_timed(mla_merge_kernel, dim3(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb)), dim3(128), 0, stream, a);
+    const dim3 mgrid(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb));
+    if (f16) launch_timed(mla_merge_kernel<FP16>, mgrid, dim3(128), 0, stream, a);
+    else launch_timed(mla_merge_kernel<BF16>, mgrid, dim3(128), 0, stream, a);
     rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
   }

@@ -47,12 +47,32 @@ void reshape_impl(xllm::kernel::ReshapePagedCacheParams& p, bool quantized) {
                     p.value->sizes() == key.sizes(),
                 "value: last two dims must be contiguous and the shape must match key");
   }
-  TORCH_CHECK(p.k_cache.dim() == 4 && p.k_cache.is_contiguous(), "k_cache must be contiguous [P, bs, Hkv, D]");
+  TORCH_CHECK(p.k_cache.is_cuda() && p.k_cache.dim() == 4 && p.k_cache.is_contiguous(),
+              "k_cache must be a contiguous device tensor [P, bs, Hkv, D]");
+  TORCH_CHECK(p.k_cache.size(2) == key.size(1) && p.k_cache.size(3) == key.size(2),
+              "k_cache heads / head_dim do not match key");
+  if (has_v) {
+    TORCH_CHECK(p.v_cache->is_cuda() && p.v_cache->is_contiguous() && p.v_cache->sizes() == p.k_cache.sizes() &&
+                    p.v_cache->scalar_type() == p.k_cache.scalar_type() && p.value->scalar_type() == key.scalar_type(),
+                "v_cache must match k_cache in shape and dtype (contiguous), value must match key in dtype");
+  }
+  TORCH_CHECK(p.slot_mapping.is_cuda(), "slot_mapping must be a device tensor");
   TORCH_CHECK(p.slot_mapping.scalar_type() == torch::kInt32 && p.slot_mapping.is_contiguous() &&
                   p.slot_mapping.numel() == key.size(0),
               "slot_mapping must be contiguous int32 [T]");
   if (quantized) {
-    TORCH_CHECK(p.k_cache_scale.has_value(), "k_cache_scale is required for quant_to_paged_cache");
+    TORCH_CHECK(p.k_cache_scale.has_value() && p.k_cache_scale->defined(),
+                "k_cache_scale is required for quant_to_paged_cache");
+    TORCH_CHECK(!has_v || (p.v_cache_scale.has_value() && p.v_cache_scale->defined()),
+                "v_cache_scale is required with a v_cache");
+    for (const std::optional<torch::Tensor>* s : {&p.k_cache_scale, &p.v_cache_scale}) {
+      if (!s->has_value() || !(*s)->defined()) continue;
+      TORCH_CHECK((*s)->is_cuda() && (*s)->scalar_type() == torch::kFloat32 && (*s)->is_contiguous() &&
+                      (*s)->numel() == key.size(1),
+                  "cache scales must be contiguous fp32 device tensors [Hkv]");
+    }
+    TORCH_CHECK(p.k_cache.scalar_type() == torch::kFloat8_e4m3fn || p.k_cache.scalar_type() == torch::kUInt8,
+                "quant_to_paged_cache writes an fp8 e4m3fn (or uint8) cache");
   } else {
     TORCH_CHECK(p.k_cache.scalar_type() == key.scalar_type(), "key and k_cache must have the same dtype");
   }
@@ -64,6 +84,33 @@ void reshape_impl(xllm::kernel::ReshapePagedCacheParams& p, bool quantized) {
       key.size(2), p.k_cache.size(1), p.k_cache.size(0), key.stride(0), has_v ? p.value->stride(0) : 0,
       dtype_code(key), dtype_code(p.k_cache), current_stream(key));
   check_rc(rc, "xllm_mi355_reshape_and_cache");
+}
+
+// What every GQA decode entry needs of its operands before their pointers reach a kernel.
+void check_decode_operands(const torch::Tensor& query, const torch::Tensor& output, const torch::Tensor& k_cache,
+                           const torch::Tensor& v_cache, const std::optional<torch::Tensor>& k_scale,
+                           const std::optional<torch::Tensor>& v_scale) {
+  TORCH_CHECK(query.is_cuda() && query.dim() == 3, "query must be a device tensor [B, Hq, D]");
+  TORCH_CHECK(query.stride(-1) == 1 && query.stride(-2) == query.size(-1), "query: last two dims must be contiguous");
+  TORCH_CHECK(output.is_cuda() && output.sizes() == query.sizes() && output.scalar_type() == query.scalar_type(),
+              "output must be a device tensor of query's shape and dtype");
+  TORCH_CHECK(output.stride(-1) == 1 && output.stride(-2) == output.size(-1), "output: last two dims must be contiguous");
+  TORCH_CHECK(k_cache.is_cuda() && k_cache.dim() == 4 && k_cache.is_contiguous(),
+              "k_cache must be a contiguous device tensor [P, bs, Hkv, D]");
+  TORCH_CHECK(v_cache.is_cuda() && v_cache.is_contiguous() && v_cache.sizes() == k_cache.sizes() &&
+                  v_cache.scalar_type() == k_cache.scalar_type(),
+              "v_cache must match k_cache in shape and dtype, contiguous");
+  TORCH_CHECK(k_cache.size(3) == query.size(2) && k_cache.size(2) > 0 && query.size(1) % k_cache.size(2) == 0,
+              "cache head_dim / KV heads do not match query");
+  const bool fp8 = k_cache.scalar_type() == torch::kFloat8_e4m3fn || k_cache.scalar_type() == torch::kUInt8;
+  if (fp8) {
+    for (const std::optional<torch::Tensor>* s : {&k_scale, &v_scale})
+      TORCH_CHECK(s->has_value() && (*s)->defined() && (*s)->is_cuda() && (*s)->scalar_type() == torch::kFloat32 &&
+                      (*s)->is_contiguous() && (*s)->numel() == k_cache.size(2),
+                  "an fp8 cache needs contiguous fp32 device scales [Hkv] for K and V");
+  } else {
+    TORCH_CHECK(k_cache.scalar_type() == query.scalar_type(), "cache dtype must equal the query dtype (or be fp8)");
+  }
 }
 
 }  // namespace
@@ -106,12 +153,9 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
                   const std::optional<torch::Tensor>& v_cache, std::optional<torch::Tensor>& output_lse,
                   const std::optional<torch::Tensor>& k_cache_quant_scale,
                   const std::optional<torch::Tensor>& v_cache_quant_scale, int64_t max_seq_len,
-                  float scale, bool return_lse) {
+                  int64_t window_size_left, float scale, bool return_lse) {
   TORCH_CHECK(v_cache.has_value() && v_cache->defined(), "GQA decode needs v_cache");
-  TORCH_CHECK(query.is_cuda() && query.dim() == 3, "query must be a device tensor [B, Hq, D]");
-  TORCH_CHECK(query.stride(-1) == 1 && query.stride(-2) == query.size(-1), "query: last two dims contiguous");
-  TORCH_CHECK(output.stride(-1) == 1 && output.stride(-2) == output.size(-1), "output: last two dims contiguous");
-  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && v_cache->is_contiguous(), "caches contiguous");
+  check_decode_operands(query, output, k_cache, *v_cache, k_cache_quant_scale, v_cache_quant_scale);
   TORCH_CHECK(block_table.scalar_type() == torch::kInt32 && block_table.dim() == 2 && block_table.stride(1) == 1 &&
                   block_table.size(0) == query.size(0),
               "block_table must be int32 [B, W]");
@@ -135,21 +179,28 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
       block_table.data_ptr<int32_t>(), block_table.stride(0), seq_lens.data_ptr<int32_t>(),
       static_cast<const float*>(ptr_or_null(k_cache_quant_scale)),
       static_cast<const float*>(ptr_or_null(v_cache_quant_scale)), B, Hq, k_cache.size(2), D, k_cache.size(1),
-      k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, scale, ws.data_ptr(),
+      k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, window_size_left, scale, ws.data_ptr(),
       static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
   check_rc(rc, "xllm_mi355_paged_decode_gqa");
 }
 
 void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache,
                       torch::Tensor paged_kv_indptr, torch::Tensor paged_kv_indices,
-                      torch::Tensor paged_kv_last_page_len, double sm_scale, torch::Tensor output,
-                      std::optional<torch::Tensor>& output_lse, int64_t max_seq_len) {
-  TORCH_CHECK(query.is_cuda() && query.dim() == 3, "query must be a device tensor [B, Hq, D]");
+                      torch::Tensor paged_kv_last_page_len, int64_t window_left, double sm_scale,
+                      torch::Tensor output, std::optional<torch::Tensor>& output_lse, int64_t max_seq_len) {
+  check_decode_operands(query, output, k_cache, v_cache, std::nullopt, std::nullopt);
   const int64_t B = query.size(0), Hq = query.size(1), D = query.size(2);
   for (const torch::Tensor* t : {&paged_kv_indptr, &paged_kv_indices, &paged_kv_last_page_len})
-    TORCH_CHECK(t->scalar_type() == torch::kInt32 && t->is_contiguous(), "CSR arrays must be contiguous int32");
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == torch::kInt32 && t->is_contiguous(),
+                "CSR arrays must be contiguous int32 device tensors");
   TORCH_CHECK(paged_kv_indptr.numel() == B + 1 && paged_kv_last_page_len.numel() == B, "CSR sizes");
-  float* lse = output_lse.has_value() && output_lse->defined() ? output_lse->data_ptr<float>() : nullptr;
+  float* lse = nullptr;
+  if (output_lse.has_value() && output_lse->defined()) {
+    TORCH_CHECK(output_lse->is_cuda() && output_lse->scalar_type() == torch::kFloat32 && output_lse->is_contiguous() &&
+                    output_lse->numel() == B * Hq,
+                "output_lse must be contiguous fp32 [B, Hq, 1]");
+    lse = output_lse->data_ptr<float>();
+  }
   if (max_seq_len <= 0) max_seq_len = std::max<int64_t>(1, paged_kv_indices.numel()) * k_cache.size(1);
   const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len);
   torch::Tensor ws = decode_workspace(query.device(), nbytes);
@@ -157,7 +208,7 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
       query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), lse,
       paged_kv_indptr.data_ptr<int32_t>(), paged_kv_indices.data_ptr<int32_t>(),
       paged_kv_last_page_len.data_ptr<int32_t>(), nullptr, nullptr, B, Hq, k_cache.size(2), D, k_cache.size(1),
-      k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, static_cast<float>(sm_scale),
+      k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, window_left, static_cast<float>(sm_scale),
       ws.data_ptr(), static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache),
       current_stream(query));
   check_rc(rc, "xllm_mi355_paged_decode_gqa_csr");
@@ -166,15 +217,10 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
 void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torch::Tensor& k_cache,
                    const torch::Tensor& v_cache, const torch::Tensor& block_table,
                    const torch::Tensor& kv_seq_lens, const torch::Tensor& q_cu_seq_lens, float scale,
-                   bool is_causal, int64_t max_seq_len, int64_t max_query_len) {
-  TORCH_CHECK(query.is_cuda() && query.dim() == 3 && query.stride(2) == 1 && query.stride(1) == query.size(2),
-              "query must be a device tensor [T, Hq, D] with contiguous heads");
-  TORCH_CHECK(output.dim() == 3 && output.sizes() == query.sizes() && output.stride(2) == 1 &&
-                  output.stride(1) == output.size(2),
-              "output must match query");
-  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.sizes() == k_cache.sizes() &&
-                  v_cache.is_contiguous(),
-              "caches must be contiguous [P, bs, Hkv, D]");
+                   bool is_causal, int64_t max_seq_len, int64_t max_query_len, int64_t window_left,
+                   const std::optional<torch::Tensor>& k_cache_quant_scale,
+                   const std::optional<torch::Tensor>& v_cache_quant_scale) {
+  check_decode_operands(query, output, k_cache, v_cache, k_cache_quant_scale, v_cache_quant_scale);
   const int64_t T = query.size(0), Hq = query.size(1), D = query.size(2), B = kv_seq_lens.numel();
   TORCH_CHECK(block_table.scalar_type() == torch::kInt32 && block_table.dim() == 2 && block_table.stride(1) == 1 &&
                   block_table.size(0) == B,
@@ -189,8 +235,10 @@ void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torc
   const int rc = xllm_mi355_paged_decode_gqa_varlen(
       query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
       q_cu_seq_lens.data_ptr<int32_t>(), kv_seq_lens.data_ptr<int32_t>(), block_table.data_ptr<int32_t>(),
-      block_table.stride(0), nullptr, nullptr, B, T, max_query_len, Hq, k_cache.size(2), D, k_cache.size(1), k_cache.size(0),
-      query.stride(0), output.stride(0), max_seq_len, scale, is_causal ? 1 : 0, ws.data_ptr(),
+      block_table.stride(0), static_cast<const float*>(ptr_or_null(k_cache_quant_scale)),
+      static_cast<const float*>(ptr_or_null(v_cache_quant_scale)), B, T, max_query_len, Hq, k_cache.size(2), D,
+      k_cache.size(1), k_cache.size(0),
+      query.stride(0), output.stride(0), max_seq_len, window_left, scale, is_causal ? 1 : 0, ws.data_ptr(),
       static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
   check_rc(rc, "xllm_mi355_paged_decode_gqa_varlen");
 }
@@ -288,8 +336,25 @@ void rope_launch(torch::Tensor& qkv, int64_t num_heads_q, int64_t num_heads_k, i
   int cache_dtype = dtype_code(qkv);
   torch::Tensor slot32;
   if (cache != nullptr) {
-    TORCH_CHECK(cache->v_cache.has_value(), "the fused cache write needs k_cache and v_cache");
+    TORCH_CHECK(cache->v_cache.has_value() && cache->v_cache->defined() && cache->k_cache.defined(),
+                "the fused cache write needs k_cache and v_cache");
+    TORCH_CHECK(cache->k_cache.is_cuda() && cache->v_cache->is_cuda() && cache->slot_mapping.is_cuda(),
+                "caches and slot_mapping must be device tensors");
     TORCH_CHECK(cache->k_cache.is_contiguous() && cache->v_cache->is_contiguous(), "caches must be contiguous");
+    TORCH_CHECK(cache->k_cache.dim() == 4 && cache->k_cache.size(2) == num_heads_k && cache->k_cache.size(3) == head_dim &&
+                    cache->v_cache->sizes() == cache->k_cache.sizes() &&
+                    cache->v_cache->scalar_type() == cache->k_cache.scalar_type() && num_heads_v == num_heads_k,
+                "caches must be [P, bs, num_heads_k, head_dim], v_cache like k_cache");
+    TORCH_CHECK(cache->slot_mapping.numel() == qkv.size(0), "one slot per token");
+    const bool fp8 = cache->k_cache.scalar_type() == torch::kFloat8_e4m3fn || cache->k_cache.scalar_type() == torch::kUInt8;
+    if (fp8) {
+      for (const std::optional<torch::Tensor>* s : {&cache->k_cache_scale, &cache->v_cache_scale})
+        TORCH_CHECK(s->has_value() && (*s)->defined() && (*s)->is_cuda() && (*s)->scalar_type() == torch::kFloat32 &&
+                        (*s)->is_contiguous() && (*s)->numel() == num_heads_k,
+                    "an fp8 cache needs contiguous fp32 device scales [num_heads_k]");
+    } else {
+      TORCH_CHECK(cache->k_cache.scalar_type() == qkv.scalar_type(), "cache dtype must equal the qkv dtype (or be fp8)");
+    }
     slot32 = (cache->slot_mapping.scalar_type() == torch::kInt32 ? cache->slot_mapping
                                                                    : cache->slot_mapping.to(torch::kInt32)).contiguous();
     kc = cache->k_cache.data_ptr();
@@ -335,46 +400,125 @@ void update_llm_decode_metadata(const LlmDecodeMetadataUpdateParams& p, void* st
   check_rc(rc, "xllm_mi355_decode_metadata_update");
 }
 
+void lse_combine(torch::Tensor output, torch::Tensor shared_o, torch::Tensor shared_lse, torch::Tensor unshared_o,
+                 torch::Tensor unshared_lse) {
+  // the checks of xllm/core/kernels/cuda/xattention/lse_combine.cu:104-131
+  TORCH_CHECK(shared_o.dim() == 3, "shared_o must be 3D [B, H, D]");
+  TORCH_CHECK(unshared_o.dim() == 3, "unshared_o must be 3D [B, H, D]");
+  TORCH_CHECK(shared_lse.dim() == 3, "shared_lse must be 3D [B, H, 1]");
+  TORCH_CHECK(unshared_lse.dim() == 3, "unshared_lse must be 3D [B, H, 1]");
+  const int64_t B = shared_o.size(0), H = shared_o.size(1), D = shared_o.size(2);
+  TORCH_CHECK(shared_o.sizes() == unshared_o.sizes() && shared_o.scalar_type() == unshared_o.scalar_type(),
+              "shared_o and unshared_o must have same shape");
+  TORCH_CHECK(shared_lse.scalar_type() == torch::kFloat32, "shared_lse must be float32");
+  TORCH_CHECK(unshared_lse.scalar_type() == torch::kFloat32, "unshared_lse must be float32");
+  for (const torch::Tensor* t : {&shared_lse, &unshared_lse})
+    TORCH_CHECK(t->size(0) == B && t->size(1) == H && t->size(2) == 1, "lse shape mismatch, expected [B, H, 1]");
+  TORCH_CHECK(shared_o.is_cuda() && unshared_o.is_cuda() && shared_lse.is_cuda() && unshared_lse.is_cuda(),
+              "tensors must be on the device");
+  // (like the reference, a missing or misshapen output is replaced by a local tensor the caller never sees)
+  if (!output.defined() || output.sizes() != shared_o.sizes()) output = torch::empty_like(shared_o);
+  TORCH_CHECK(output.is_cuda() && output.is_contiguous(), "output must be a contiguous device tensor");
+  const torch::Tensor so = shared_o.contiguous(), uo = unshared_o.contiguous();
+  const torch::Tensor sl = shared_lse.contiguous(), ul = unshared_lse.contiguous();
+  const int rc = xllm_mi355_lse_combine(output.data_ptr(), so.data_ptr(), sl.data_ptr<float>(), uo.data_ptr(),
+                                        ul.data_ptr<float>(), B * H, D, dtype_code(so), dtype_code(output),
+                                        current_stream(so));
+  check_rc(rc, "xllm_mi355_lse_combine");
+}
+
+}  // namespace mi355
+
+namespace dcu {
 namespace flash_mla {
 
-torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {
-  // the checks of check_dense_decode_inputs, xllm/core/kernels/dcu/flash_mla_adapter.cpp:55-100
-  TORCH_CHECK(p.q_nope.defined() && p.q_pe.defined() && p.k_cache.defined() && p.seqlens_k.defined() &&
-                  p.block_table.defined(),
-              "flash_mla: all tensors must be defined");
-  TORCH_CHECK(p.q_nope.dim() == 4 && p.q_pe.dim() == 4, "flash_mla: q_nope / q_pe must be 4D [B,S_q,H_q,D]");
-  TORCH_CHECK(p.k_cache.dim() == 4 && p.k_cache.size(2) == 1,
-              "flash_mla: k_cache must be 4D [blocks,page,1,D] with a single KV head");
+namespace {
+// check_dense_decode_inputs, xllm/core/kernels/dcu/flash_mla_adapter.cpp:55-100 (the page size is not pinned to
+// 64 here: the kernels take any block size)
+void check_dense_decode_inputs(const DenseDecodeParams& p) {
+  TORCH_CHECK(p.q_nope.defined(), "flash_mla: q_nope must be defined");
+  TORCH_CHECK(p.q_pe.defined(), "flash_mla: q_pe must be defined");
+  TORCH_CHECK(p.k_cache.defined(), "flash_mla: k_cache must be defined");
+  TORCH_CHECK(p.seqlens_k.defined(), "flash_mla: seqlens_k must be defined");
+  TORCH_CHECK(p.block_table.defined(), "flash_mla: block_table must be defined");
+  const torch::Device dev = p.k_cache.device();
+  TORCH_CHECK(dev.is_cuda(), "flash_mla: k_cache must be on the device");
+  TORCH_CHECK(p.q_nope.device() == dev, "flash_mla: q_nope must be on the device of k_cache");
+  TORCH_CHECK(p.q_pe.device() == dev, "flash_mla: q_pe must be on the device of k_cache");
+  TORCH_CHECK(p.seqlens_k.device() == dev, "flash_mla: seqlens_k must be on the device of k_cache");
+  TORCH_CHECK(p.block_table.device() == dev, "flash_mla: block_table must be on the device of k_cache");
+  TORCH_CHECK(p.q_nope.dim() == 4, "flash_mla: q_nope must be 4D [B,S_q,H_q,D]");
+  TORCH_CHECK(p.q_pe.dim() == 4, "flash_mla: q_pe must be 4D [B,S_q,H_q,D]");
+  TORCH_CHECK(p.k_cache.dim() == 4, "flash_mla: k_cache must be 4D [blocks,page,1,D]");
+  TORCH_CHECK(p.k_cache.size(2) == 1, "flash_mla: MLA expects a single KV head (num_heads_k == 1)");
+  TORCH_CHECK(p.seqlens_k.dim() == 1, "flash_mla: seqlens_k must be 1D [B]");
+  TORCH_CHECK(p.block_table.dim() == 2, "flash_mla: block_table must be 2D [B,max_blocks]");
   TORCH_CHECK(p.k_cache.size(3) == p.q_nope.size(3) + p.q_pe.size(3),
               "flash_mla: k_cache last dim must equal q_nope.dim + q_pe.dim");
+  TORCH_CHECK(p.q_nope.size(0) == p.q_pe.size(0), "flash_mla: q_nope/q_pe batch must match");
+  TORCH_CHECK(p.q_nope.size(1) == p.q_pe.size(1), "flash_mla: q_nope/q_pe seq must match");
+  TORCH_CHECK(p.q_nope.size(2) == p.q_pe.size(2), "flash_mla: q_nope/q_pe head count must match");
   TORCH_CHECK(p.head_size_v > 0, "flash_mla: head_size_v must be positive");
-  TORCH_CHECK(p.softmax_scale > 0.0F, "flash_mla: softmax_scale must be set by the MLA attention layer");
-  TORCH_CHECK(p.q_nope.size(1) == 1, "decode path: one query token per sequence");
-  TORCH_CHECK(p.head_size_v == p.q_nope.size(3), "V is the latent part of the cache");
+  // what the kernels behind this adapter add
+  TORCH_CHECK(p.seqlens_k.numel() == p.q_nope.size(0) && p.block_table.size(0) == p.q_nope.size(0),
+              "flash_mla: seqlens_k and block_table must have one row per sequence");
+  TORCH_CHECK(p.k_cache.is_contiguous(), "flash_mla: k_cache must be contiguous");
+  TORCH_CHECK(p.q_nope.scalar_type() == p.q_pe.scalar_type() && p.q_nope.scalar_type() == p.k_cache.scalar_type(),
+              "flash_mla: q_nope, q_pe and k_cache must have the same dtype");
+  TORCH_CHECK(p.q_nope.scalar_type() == torch::kBFloat16 || p.q_nope.scalar_type() == torch::kFloat16,
+              "flash_mla: BF16 / FP16 only");
+  TORCH_CHECK(p.head_size_v == p.q_nope.size(3), "flash_mla: V is the latent part of the cache (head_size_v == q_nope.dim)");
+}
+}  // namespace
+
+torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {
+  TORCH_CHECK(p.kind == DenseDecodeKind::kQNopePe,
+              "flash_mla: only DenseDecodeKind::kQNopePe (BF16/FP16 split-q) is supported");
+  check_dense_decode_inputs(p);
   torch::Tensor seqlens = p.seqlens_k.scalar_type() == torch::kInt32 ? p.seqlens_k : p.seqlens_k.to(torch::kInt32);
   torch::Tensor table = p.block_table.scalar_type() == torch::kInt32 ? p.block_table : p.block_table.to(torch::kInt32);
-  torch::Tensor q_nope = p.q_nope.contiguous(), q_pe = p.q_pe.contiguous();
-  const int64_t B = q_nope.size(0), H = q_nope.size(2);
-  torch::Tensor out = torch::empty({B, 1, H, p.head_size_v}, q_nope.options());
+  seqlens = seqlens.contiguous();
+  if (table.stride(1) != 1) table = table.contiguous();
+  TORCH_CHECK(p.softmax_scale > 0.0F, "flash_mla: softmax_scale must be set by the MLA attention layer");
+  const torch::Tensor q_nope = p.q_nope.contiguous(), q_pe = p.q_pe.contiguous();
+  const int64_t B = q_nope.size(0), Sq = q_nope.size(1), H = q_nope.size(2);
+  torch::Tensor out = torch::empty({B, Sq, H, p.head_size_v}, q_nope.options());
+  // The reference folds the S_q query tokens of a sequence into the head count (flash_mla_adapter.cpp:119-123):
+  // q [B, S_q * H, D] against the same pages.  With a causal mask token j sees S_q - 1 - j tokens less than the
+  // last one, so every (sequence, token) becomes a row of its own: [B * S_q, H, D] with its own length and the
+  // table row of its sequence.
+  const bool per_token = p.is_causal && Sq > 1;
+  int64_t rows = B, heads = Sq * H;
+  if (per_token) {
+    rows = B * Sq;
+    heads = H;
+    const torch::Tensor back = torch::arange(Sq - 1, -1, -1, seqlens.options());            // S_q - 1 - j
+    seqlens = (seqlens.unsqueeze(1) - back.unsqueeze(0)).clamp_min(0).reshape({rows}).contiguous();
+    table = table.repeat_interleave(Sq, 0).contiguous();
+  }
+  torch::Tensor lse_rows;  // [rows, heads]
   float* lse = nullptr;
   if (lse_out != nullptr) {
-    *lse_out = torch::empty({B, H, 1}, q_nope.options().dtype(torch::kFloat32));
-    lse = lse_out->data_ptr<float>();
+    lse_rows = torch::empty({rows, heads}, q_nope.options().dtype(torch::kFloat32));
+    lse = lse_rows.data_ptr<float>();
   }
   const int64_t max_seq_len = table.size(1) * p.k_cache.size(1);
-  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, H, p.head_size_v, max_seq_len);
-  torch::Tensor ws = decode_workspace(q_nope.device(), nbytes);
+  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(rows, heads, p.head_size_v, max_seq_len);
+  torch::Tensor ws = mi355::decode_workspace(q_nope.device(), nbytes);
   const int rc = xllm_mi355_paged_decode_mla(
       q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), lse, table.data_ptr<int32_t>(),
-      table.stride(0), seqlens.data_ptr<int32_t>(), B, H, q_nope.size(3), q_pe.size(3), p.k_cache.size(1),
+      table.stride(0), seqlens.data_ptr<int32_t>(), rows, heads, q_nope.size(3), q_pe.size(3), p.k_cache.size(1),
       p.k_cache.size(0), max_seq_len, p.softmax_scale, ws.data_ptr(), static_cast<size_t>(ws.numel()),
       dtype_code(q_nope), current_stream(q_nope));
   check_rc(rc, "xllm_mi355_paged_decode_mla");
+  if (lse_out != nullptr) *lse_out = lse_rows.view({B, Sq, H}).transpose(1, 2).contiguous();  // [B, H, S_q]
   return out;
 }
 
+torch::Tensor dense_decode(DenseDecodeParams& params) { return dense_decode(params, nullptr); }
+
 }  // namespace flash_mla
-}  // namespace mi355
+}  // namespace dcu
 }  // namespace xllm::kernel
 
 namespace xllm::layer {
@@ -397,6 +541,73 @@ DcpAttentionResult merge_dcp_attention_shards(const torch::Tensor& partial_outpu
                                       H, Dv, dtype_code(po), current_stream(po));
   check_rc(rc, "xllm_mi355_lse_merge");
   return {out, lse};
+}
+
+// The decode and short-chunk branches of FlashAttentionImpl::forward / paged_forward
+// (xllm/core/layers/dcu/flash_attention.cpp:547-660, 447-545) on this library's kernels.
+std::tuple<torch::Tensor, std::optional<torch::Tensor>> Mi355AttentionImpl::forward(
+    const AttentionMetadata& attn_metadata, torch::Tensor& query, torch::Tensor& key, torch::Tensor& value,
+    torch::Tensor& output, KVCache& kv_cache) {
+  std::optional<torch::Tensor> output_lse = std::nullopt;
+  if (attn_metadata.max_seq_len == 0) {
+    output = output.view({-1, num_heads_ * head_size_});
+    return std::make_tuple(output, output_lse);
+  }
+  query = query.view({-1, num_heads_, head_size_});
+  key = key.view({-1, num_kv_heads_, head_size_});
+  value = value.view({-1, num_kv_heads_, head_size_});
+  output = output.view({-1, num_heads_, head_size_});
+
+  torch::Tensor k_cache = kv_cache.get_k_cache();
+  torch::Tensor v_cache = kv_cache.get_v_cache();
+  const std::optional<torch::Tensor> k_scale = kv_cache.get_k_cache_scale();
+  const std::optional<torch::Tensor> v_scale = kv_cache.get_v_cache_scale();
+  const bool quantized = k_scale.has_value() && k_scale->defined();
+
+  // store the step's K / V rows; the quantising store where the cache carries scales
+  // (xllm/core/layers/mlu/attention.cpp:109-117)
+  if (k_cache.defined() && k_cache.dim() >= 2) {
+    xllm::kernel::ReshapePagedCacheParams params;
+    params.key = key;
+    params.value = value;
+    params.k_cache = k_cache;
+    params.v_cache = v_cache;
+    params.slot_mapping = attn_metadata.slot_mapping;
+    if (quantized) {
+      params.k_cache_scale = k_scale;
+      params.v_cache_scale = v_scale;
+      xllm::kernel::quant_to_paged_cache(params);
+    } else {
+      xllm::kernel::reshape_paged_cache(params);
+    }
+  }
+
+  TORCH_CHECK(!attn_metadata.is_prefill || attn_metadata.is_chunked_prefill,
+              "prefill is not part of the paged decode path");
+  // window_left: a positive sliding window, otherwise the whole context (flash_attention.cpp:484)
+  const int64_t window_left = sliding_window_ > 0 ? sliding_window_ : -1;
+  torch::Tensor kv_seq_lens = attn_metadata.kv_seq_lens.scalar_type() == torch::kInt32
+                                  ? attn_metadata.kv_seq_lens
+                                  : attn_metadata.kv_seq_lens.to(torch::kInt32);
+  kv_seq_lens = kv_seq_lens.contiguous();
+  torch::Tensor block_table = attn_metadata.block_table.scalar_type() == torch::kInt32
+                                  ? attn_metadata.block_table
+                                  : attn_metadata.block_table.to(torch::kInt32);
+  if (attn_metadata.is_chunked_prefill) {
+    constexpr int64_t kDecodeMaxQueryLen = 16;  // kHgPrefixDecodeMaxQueryLen, flash_attention.cpp:504
+    TORCH_CHECK(attn_metadata.max_query_len <= kDecodeMaxQueryLen,
+                "query chunks of more than 16 tokens belong to the prefill kernel, which is not part of this path");
+    const torch::Tensor cu = attn_metadata.q_cu_seq_lens.to(torch::kInt32).contiguous();
+    xllm::kernel::mi355::paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, cu, scale_,
+                                       attn_metadata.is_causal, attn_metadata.max_seq_len,
+                                       attn_metadata.max_query_len, window_left, k_scale, v_scale);
+  } else {
+    // decode: one query token per sequence, a token attends to its whole context whatever is_causal says
+    xllm::kernel::mi355::batch_decode(query, k_cache, output, block_table, kv_seq_lens, v_cache, output_lse, k_scale,
+                                      v_scale, attn_metadata.max_seq_len, window_left, scale_, return_lse_);
+  }
+  output = output.view({-1, num_heads_ * head_size_});
+  return std::make_tuple(output, output_lse);
 }
 
 }  // namespace xllm::layer
@@ -440,15 +651,46 @@ std::tuple<torch::Tensor, torch::Tensor> op_batch_decode(torch::Tensor query, to
                                                          double scale) {
   std::optional<torch::Tensor> lse;
   xllm::kernel::mi355::batch_decode(query, k_cache, output, block_table, seq_lens, v_cache, lse, k_scale, v_scale,
-                                    max_seq_len, static_cast<float>(scale), /*return_lse=*/true);
+                                    max_seq_len, /*window_size_left=*/-1, static_cast<float>(scale), /*return_lse=*/true);
   return {output, lse.value()};
+}
+
+torch::Tensor op_lse_combine(torch::Tensor output, torch::Tensor shared_o, torch::Tensor shared_lse,
+                             torch::Tensor unshared_o, torch::Tensor unshared_lse) {
+  xllm::kernel::mi355::lse_combine(output, shared_o, shared_lse, unshared_o, unshared_lse);
+  return output;
+}
+
+// The layer contract end to end: AttentionMetadata + KVCache + AttentionImpl::forward built from plain arguments
+// (xllm/core/layers/dcu/attention.cpp:55-112).  q_cu_seq_lens undefined: decode, one token per sequence.
+std::tuple<torch::Tensor, std::optional<torch::Tensor>> op_attention_layer_forward(
+    torch::Tensor query, torch::Tensor key, torch::Tensor value, torch::Tensor k_cache, torch::Tensor v_cache,
+    std::optional<torch::Tensor> k_cache_scale, std::optional<torch::Tensor> v_cache_scale, torch::Tensor slot_mapping,
+    torch::Tensor block_table, torch::Tensor kv_seq_lens, std::optional<torch::Tensor> q_cu_seq_lens, int64_t max_seq_len,
+    int64_t max_query_len, int64_t num_heads, int64_t head_size, int64_t num_kv_heads, double scale,
+    int64_t sliding_window, bool is_causal, bool return_lse) {
+  xllm::layer::AttentionMetadata meta;
+  meta.kv_seq_lens = kv_seq_lens;
+  meta.block_table = block_table;
+  meta.slot_mapping = slot_mapping;
+  meta.max_seq_len = max_seq_len;
+  meta.max_query_len = max_query_len;
+  meta.is_causal = is_causal;
+  if (q_cu_seq_lens.has_value() && q_cu_seq_lens->defined()) {
+    meta.q_cu_seq_lens = *q_cu_seq_lens;
+    meta.is_prefill = true;
+    meta.is_chunked_prefill = true;
+  }
+  xllm::KVCache cache(k_cache, v_cache, k_cache_scale, v_cache_scale);
+  xllm::layer::AttentionImpl attn(num_heads, head_size, static_cast<float>(scale), num_kv_heads, sliding_window, return_lse);
+  return attn.forward(meta, query, key, value, cache);
 }
 
 std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nope, torch::Tensor q_pe,
                                                              torch::Tensor k_cache, torch::Tensor seqlens_k,
                                                              torch::Tensor block_table, int64_t head_size_v,
-                                                             double softmax_scale) {
-  xllm::kernel::mi355::flash_mla::DenseDecodeParams p;
+                                                             double softmax_scale, bool is_causal) {
+  xllm::kernel::dcu::flash_mla::DenseDecodeParams p;
   p.q_nope = q_nope;
   p.q_pe = q_pe;
   p.k_cache = k_cache;
@@ -456,8 +698,10 @@ std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nop
   p.block_table = block_table;
   p.head_size_v = head_size_v;
   p.softmax_scale = static_cast<float>(softmax_scale);
+  p.is_causal = is_causal;
+  p.kind = xllm::kernel::dcu::flash_mla::DenseDecodeKind::kQNopePe;
   torch::Tensor lse;
-  torch::Tensor out = xllm::kernel::mi355::flash_mla::dense_decode(p, &lse);
+  torch::Tensor out = xllm::kernel::dcu::flash_mla::dense_decode(p, &lse);
   return {out, lse};
 }
 
@@ -561,7 +805,12 @@ TORCH_LIBRARY(xllm_ops, m) {
   m.def("batch_decode(Tensor query, Tensor k_cache, Tensor v_cache, Tensor(a!) output, Tensor block_table, "
         "Tensor seq_lens, Tensor? k_scale, Tensor? v_scale, int max_seq_len, float scale) -> (Tensor, Tensor)");
   m.def("mla_dense_decode(Tensor q_nope, Tensor q_pe, Tensor k_cache, Tensor seqlens_k, Tensor block_table, "
-        "int head_size_v, float softmax_scale) -> (Tensor, Tensor)");
+        "int head_size_v, float softmax_scale, bool is_causal=False) -> (Tensor, Tensor)");
+  m.def("lse_combine(Tensor(a!) output, Tensor shared_o, Tensor shared_lse, Tensor unshared_o, Tensor unshared_lse) -> Tensor");
+  m.def("attention_layer_forward(Tensor query, Tensor key, Tensor value, Tensor(a!) k_cache, Tensor(b!) v_cache, "
+        "Tensor? k_cache_scale, Tensor? v_cache_scale, Tensor slot_mapping, Tensor block_table, Tensor kv_seq_lens, "
+        "Tensor? q_cu_seq_lens, int max_seq_len, int max_query_len, int num_heads, int head_size, int num_kv_heads, "
+        "float scale, int sliding_window, bool is_causal, bool return_lse) -> (Tensor, Tensor?)");
   m.def("merge_dcp_attention_shards(Tensor partial_outputs, Tensor partial_lse) -> (Tensor, Tensor)");
   m.def("paged_forward(Tensor query, Tensor(a!) output, Tensor k_cache, Tensor v_cache, Tensor block_table, "
         "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len, int max_query_len) -> Tensor");
@@ -586,6 +835,8 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("quant_to_paged_cache", &op_quant_to_paged_cache);
   m.impl("batch_decode", &op_batch_decode);
   m.impl("mla_dense_decode", &op_mla_dense_decode);
+  m.impl("lse_combine", &op_lse_combine);
+  m.impl("attention_layer_forward", &op_attention_layer_forward);
   m.impl("merge_dcp_attention_shards", &op_merge);
   m.impl("paged_forward", &op_paged_forward);
   m.impl("gather_mla_latent_cache", &op_gather_mla_latent_cache);

@@ -7,14 +7,22 @@
 //   xllm::kernel::mi355::batch_decode (block table)   xllm/core/kernels/mlu/mlu_ops_api.h:127,
 //                                                     xllm/core/kernels/npu/npu_ops_api.h:46
 //   xllm::kernel::mi355::batch_decode_csr             xllm/core/kernels/cuda/cuda_ops_api.h:128-144
-//   xllm::kernel::mi355::flash_mla::dense_decode      xllm/core/kernels/dcu/flash_mla_adapter.h:40-53
+//   xllm::kernel::dcu::flash_mla::dense_decode        xllm/core/kernels/dcu/flash_mla_adapter.h:29-53
+//   xllm::kernel::mi355::lse_combine                  xllm/core/kernels/cuda/xattention/xattention_ops_api.h:38
 //   xllm::layer::merge_dcp_attention_shards           xllm/core/layers/mlu/dcp_attention_merge.h:28-34
+//   xllm::layer::AttentionMetadata (decode subset), xllm::KVCache (accessors), xllm::layer::BaseAttentionImpl,
+//   xllm::layer::AttentionImpl                        xllm/core/layers/common/attention_metadata.h:99-156,
+//                                                     xllm/core/framework/kv_cache/kv_cache.h:29-95,
+//                                                     xllm/core/layers/dcu/base_attention_impl.h:30-57,
+//                                                     xllm/core/layers/dcu/attention.cpp:28-112
 // A violated precondition throws c10::Error (TORCH_CHECK) where the reference CHECK-aborts.
 #pragma once
 
 #include <torch/torch.h>
 
+#include <memory>
 #include <optional>
+#include <string>
 #include <tuple>
 
 namespace xllm::kernel {
@@ -53,12 +61,15 @@ void batch_decode(const torch::Tensor& query,        // [B, Hq, D]
                   std::optional<torch::Tensor>& output_lse,  // [B, Hq, 1] fp32, natural log
                   const std::optional<torch::Tensor>& k_cache_quant_scale,
                   const std::optional<torch::Tensor>& v_cache_quant_scale,
-                  int64_t max_seq_len, float scale, bool return_lse);
+                  int64_t max_seq_len, int64_t window_size_left, float scale, bool return_lse);
 
+// The CSR form, with the arguments of xllm::kernel::cuda::batch_decode (cuda_ops_api.h:128-144) that are not
+// FlashInfer's own (uri, plan_info, the three workspace buffers, use_tensor_core, qo_indptr), in its order;
+// max_seq_len bounds the longest context (0 = unknown).
 void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache,
                       torch::Tensor paged_kv_indptr, torch::Tensor paged_kv_indices,
-                      torch::Tensor paged_kv_last_page_len, double sm_scale, torch::Tensor output,
-                      std::optional<torch::Tensor>& output_lse, int64_t max_seq_len);
+                      torch::Tensor paged_kv_last_page_len, int64_t window_left, double sm_scale,
+                      torch::Tensor output, std::optional<torch::Tensor>& output_lse, int64_t max_seq_len);
 
 // Short query chunks against paged KV: the decode branch of FlashAttentionImpl::paged_forward
 // (xllm/core/layers/dcu/flash_attention.cpp:447-545).  query / output packed [T, Hq, D]; kv_seq_lens [B] are the
@@ -67,7 +78,14 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
 void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torch::Tensor& k_cache,
                    const torch::Tensor& v_cache, const torch::Tensor& block_table,
                    const torch::Tensor& kv_seq_lens, const torch::Tensor& q_cu_seq_lens, float scale,
-                   bool is_causal, int64_t max_seq_len, int64_t max_query_len);
+                   bool is_causal, int64_t max_seq_len, int64_t max_query_len, int64_t window_left = -1,
+                   const std::optional<torch::Tensor>& k_cache_quant_scale = std::nullopt,
+                   const std::optional<torch::Tensor>& v_cache_quant_scale = std::nullopt);
+
+// xllm::kernel::cuda::lse_combine (xllm/core/kernels/cuda/xattention/xattention_ops_api.h:38,
+// lse_combine.cu:99-166), same arguments: the two-way combine with BASE-2 LSEs [B, H, 1] fp32.
+void lse_combine(torch::Tensor output, torch::Tensor shared_o, torch::Tensor shared_lse, torch::Tensor unshared_o,
+                 torch::Tensor unshared_lse);
 
 // xllm::kernel::dcu::gather_mla_latent_cache (xllm/core/kernels/dcu/dcu_ops_api.h:74), same arguments.
 torch::Tensor gather_mla_latent_cache(const torch::Tensor& k_cache, const torch::Tensor& block_table,
@@ -122,23 +140,156 @@ struct LlmDecodeMetadataUpdateParams {
 };
 void update_llm_decode_metadata(const LlmDecodeMetadataUpdateParams& params, void* stream);
 
+}  // namespace mi355
+
+// The reference's own namespace, types and signature (xllm/core/kernels/dcu/flash_mla_adapter.h:29-53): a caller
+// such as DeepseekV2AttentionImpl::decode_flash_mla (layers/dcu/deepseek_v2_attention.cpp:242-263) compiles against
+// this unchanged.
+namespace dcu {
 namespace flash_mla {
+
+enum class DenseDecodeKind {
+  kQNopePe,
+};
+
+// Inputs of the dense MLA decode.
+//   q_nope:      [B, S_q, H_q, kv_lora_rank]
+//   q_pe:        [B, S_q, H_q, qk_rope_head_dim]
+//   k_cache:     [num_blocks, block_size, 1, kv_lora_rank + qk_rope_head_dim]
+//   seqlens_k:   [B] int32
+//   block_table: [B, max_blocks] int32
 struct DenseDecodeParams {
-  torch::Tensor q_nope;       // [B, S_q, H, kv_lora_rank]
-  torch::Tensor q_pe;         // [B, S_q, H, rope]
-  torch::Tensor k_cache;      // [P, bs, 1, kv_lora_rank + rope]
-  torch::Tensor seqlens_k;    // [B] int32
-  torch::Tensor block_table;  // [B, W] int32
+  torch::Tensor q_nope;
+  torch::Tensor q_pe;
+  torch::Tensor k_cache;
+  torch::Tensor seqlens_k;
+  torch::Tensor block_table;
   int64_t head_size_v = 0;
   float softmax_scale = -1.0F;
   bool is_causal = false;
+  DenseDecodeKind kind = DenseDecodeKind::kQNopePe;
 };
-// Returns [B, S_q, H, head_size_v]; lse (if not null) receives [B, H, 1] fp32.
-torch::Tensor dense_decode(DenseDecodeParams& params, torch::Tensor* lse = nullptr);
-}  // namespace flash_mla
 
+// Returns [B, S_q, H_q, head_size_v].  BF16 and FP16.  S_q query tokens per sequence (multi-token speculative
+// steps) are folded into the head count as the reference folds them (flash_mla_adapter.cpp:119-123); with
+// is_causal and S_q > 1 token j attends to the first seqlens_k - (S_q - 1 - j) tokens.
+torch::Tensor dense_decode(DenseDecodeParams& params);
+// The same with the natural-log LSE, [B, H_q, S_q] fp32 (the layout of MluMlaDecodeLseTest,
+// tests/core/layers/mlu/dcp_attention_merge_test.cpp:127-143, for S_q = 1: [B, H, 1]).
+torch::Tensor dense_decode(DenseDecodeParams& params, torch::Tensor* lse);
+
+}  // namespace flash_mla
+}  // namespace dcu
+
+namespace mi355 {
+namespace flash_mla = ::xllm::kernel::dcu::flash_mla;
 }  // namespace mi355
 }  // namespace xllm::kernel
+
+// Minimal stand-ins for the two types the layer contract takes, with the reference's member names, holding only
+// what the decode path reads.
+namespace xllm {
+// xllm::KVCache (xllm/core/framework/kv_cache/kv_cache.h:29-95): the four accessors of the path.
+class KVCache final {
+ public:
+  KVCache() = default;
+  KVCache(torch::Tensor k_cache, torch::Tensor v_cache, std::optional<torch::Tensor> k_cache_scale = std::nullopt,
+          std::optional<torch::Tensor> v_cache_scale = std::nullopt)
+      : k_cache_(std::move(k_cache)), v_cache_(std::move(v_cache)), k_scale_(std::move(k_cache_scale)),
+        v_scale_(std::move(v_cache_scale)) {}
+  torch::Tensor get_k_cache() const { return k_cache_; }
+  torch::Tensor get_v_cache() const { return v_cache_; }
+  std::optional<torch::Tensor> get_k_cache_scale() const { return k_scale_; }
+  std::optional<torch::Tensor> get_v_cache_scale() const { return v_scale_; }
+
+ private:
+  torch::Tensor k_cache_, v_cache_;
+  std::optional<torch::Tensor> k_scale_, v_scale_;
+};
+
+namespace layer {
+// xllm::layer::AttentionMetadata (xllm/core/layers/common/attention_metadata.h:99-156), decode subset.
+struct AttentionMetadata {
+  torch::Tensor q_cu_seq_lens;
+  torch::Tensor kv_cu_seq_lens;
+  torch::Tensor kv_seq_lens;
+  torch::Tensor q_seq_lens;
+  torch::Tensor block_table;
+  torch::Tensor slot_mapping;
+  int64_t max_query_len = 1;
+  int64_t max_seq_len = 0;
+  int64_t total_kv_len = 0;
+  std::string compute_dtype;
+  bool is_prefill = false;
+  bool is_chunked_prefill = false;
+  bool is_dummy = false;
+  bool is_causal = true;
+  torch::Tensor paged_kv_indptr;
+  torch::Tensor paged_kv_indices;
+  torch::Tensor paged_kv_last_page_len;
+  bool enable_cuda_graph = false;
+};
+
+// xllm::layer::BaseAttentionImpl (xllm/core/layers/dcu/base_attention_impl.h:30-57), unchanged.
+class BaseAttentionImpl {
+ public:
+  BaseAttentionImpl(int64_t num_heads, int64_t head_size, float scale, int64_t num_kv_heads, int64_t sliding_window)
+      : num_heads_(num_heads), head_size_(head_size), scale_(scale), num_kv_heads_(num_kv_heads),
+        sliding_window_(sliding_window) {}
+  virtual ~BaseAttentionImpl() = default;
+  virtual std::tuple<torch::Tensor, std::optional<torch::Tensor>> forward(const AttentionMetadata& attn_metadata,
+                                                                          torch::Tensor& query, torch::Tensor& key,
+                                                                          torch::Tensor& value, torch::Tensor& output,
+                                                                          KVCache& kv_cache) = 0;
+
+ protected:
+  int64_t num_heads_;
+  int64_t head_size_;
+  float scale_;
+  int64_t num_kv_heads_;
+  int64_t sliding_window_;
+  bool decode_use_tensor_core_ = false;
+};
+
+// The MI355X implementation behind that interface: the write-then-attend step of FlashAttentionImpl::forward
+// (xllm/core/layers/dcu/flash_attention.cpp:547-660) for decode and for chunked prefill with chunks of up to 16
+// tokens, on this library's kernels.  The quantising store is chosen where the cache carries scales
+// (xllm/core/layers/mlu/attention.cpp:109-117).  Prefill is not part of this path and throws.
+// return_lse: also return the natural-log LSE [tokens, num_heads] fp32 (decode only).
+class Mi355AttentionImpl final : public BaseAttentionImpl {
+ public:
+  Mi355AttentionImpl(int64_t num_heads, int64_t head_size, float scale, int64_t num_kv_heads, int64_t sliding_window,
+                     bool return_lse = false)
+      : BaseAttentionImpl(num_heads, head_size, scale, num_kv_heads, sliding_window), return_lse_(return_lse) {}
+  std::tuple<torch::Tensor, std::optional<torch::Tensor>> forward(const AttentionMetadata& attn_metadata,
+                                                                  torch::Tensor& query, torch::Tensor& key,
+                                                                  torch::Tensor& value, torch::Tensor& output,
+                                                                  KVCache& kv_cache) override;
+
+ private:
+  bool return_lse_;
+};
+
+// xllm::layer::AttentionImpl (xllm/core/layers/dcu/attention.cpp:28-112): picks the implementation, allocates
+// output = empty_like(query) and forwards.
+class AttentionImpl final {
+ public:
+  AttentionImpl(int64_t num_heads, int64_t head_size, float scale, int64_t num_kv_heads, int64_t sliding_window,
+                bool return_lse = false)
+      : attention_impl_(std::make_shared<Mi355AttentionImpl>(num_heads, head_size, scale, num_kv_heads, sliding_window,
+                                                             return_lse)) {}
+  std::tuple<torch::Tensor, std::optional<torch::Tensor>> forward(const AttentionMetadata& attn_metadata,
+                                                                  torch::Tensor& query, torch::Tensor& key,
+                                                                  torch::Tensor& value, KVCache& kv_cache) {
+    torch::Tensor output = torch::empty_like(query);
+    return attention_impl_->forward(attn_metadata, query, key, value, output, kv_cache);
+  }
+
+ private:
+  std::shared_ptr<BaseAttentionImpl> attention_impl_;
+};
+}  // namespace layer
+}  // namespace xllm
 
 namespace xllm::layer {
 struct DcpAttentionResult {

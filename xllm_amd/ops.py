@@ -190,29 +190,44 @@ def kv_head_scales(x):
 # ------------------------------------------------------------------------------------------
 # op 2
 
-def _decode_common(query, k_cache, output):
+def _decode_common(query, k_cache, output, v_cache=None, k_scale=None, v_scale=None):
     if query.dim() != 3:
         raise ValueError("query must be [B, Hq, D]")
     if not (query.stride(-1) == 1 and query.stride(-2) == query.shape[-1]):
         raise ValueError("query: last two dims must be contiguous")
+    if output.shape != query.shape or output.dtype != query.dtype:
+        raise ValueError("output must have query's shape and dtype")
     if not (output.stride(-1) == 1 and output.stride(-2) == output.shape[-1]):
         raise ValueError("output: last two dims must be contiguous")
     if not k_cache.is_contiguous() or k_cache.dim() != 4:
         raise ValueError("k_cache must be contiguous [P, bs, Hkv, D]")
+    if k_cache.shape[3] != query.shape[2] or query.shape[1] % k_cache.shape[2] != 0:
+        raise ValueError("cache head_dim / KV heads do not match query")
+    if v_cache is not None and (v_cache.shape != k_cache.shape or v_cache.dtype != k_cache.dtype
+                                or not v_cache.is_contiguous()):
+        raise ValueError("v_cache must match k_cache in shape and dtype, contiguous")
+    if _dtype_code(k_cache) == capi.FP8_E4M3:
+        for s in (k_scale, v_scale):
+            if s is None or s.dtype != torch.float32 or s.numel() != k_cache.shape[2] or not s.is_contiguous():
+                raise ValueError("an fp8 cache needs contiguous fp32 scales [Hkv] for K and V")
+    elif k_cache.dtype != query.dtype:
+        raise TypeError("the cache dtype must equal the query dtype (or be fp8)")
 
 
 def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, output_lse=None,
                  k_cache_quant_scale=None, v_cache_quant_scale=None, scale=None, return_lse=False,
-                 max_seq_len=0):
+                 max_seq_len=0, window_left=-1):
     """Block-table paged decode.  Argument order and meaning follow mlu::batch_decode
     (mlu_ops_api.h:127) restricted to what npu::batch_decode (npu_ops_api.h:46) also has.
     query/output [B, Hq, D]; caches [P, bs, Hkv, D]; block_table [B, W] int32; seq_lens [B] int32.
+    window_left >= 0: sliding window, the query attends to the last window_left + 1 tokens of its context
+    (sliding_window_ of layers/dcu/flash_attention.cpp:484).
     Returns (output, lse or None) with lse [B, Hq, 1] fp32 natural log."""
     if v_cache is None:
         raise ValueError("GQA decode needs v_cache; the latent-KV variant is dense_decode")
     dev = _require_cuda(query, k_cache, v_cache, output, block_table, seq_lens, output_lse,
                         k_cache_quant_scale, v_cache_quant_scale)
-    _decode_common(query, k_cache, output)
+    _decode_common(query, k_cache, output, v_cache, k_cache_quant_scale, v_cache_quant_scale)
     B, Hq, D = query.shape
     P, bs, Hkv, _ = k_cache.shape
     if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
@@ -237,21 +252,21 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
         query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(lse),
         block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(),
         _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D, bs, P,
-        query.stride(0), output.stride(0), max_seq_len, float(scale), ws.data_ptr(), ws.numel(),
+        query.stride(0), output.stride(0), max_seq_len, int(window_left), float(scale), ws.data_ptr(), ws.numel(),
         _dtype_code(query), _dtype_code(k_cache), _stream(dev))
     capi.check(rc, "xllm_mi355_paged_decode_gqa")
     return output, lse
 
 
 def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
-                     paged_kv_last_page_len, sm_scale, output, output_lse=None, max_seq_len=0,
+                     paged_kv_last_page_len, window_left, sm_scale, output, output_lse=None, max_seq_len=0,
                      k_cache_quant_scale=None, v_cache_quant_scale=None):
     """CSR paged decode: cuda::batch_decode (cuda_ops_api.h:128-144) without the FlashInfer
-    uri / plan_info / workspace arguments.  max_seq_len bounds the longest context; 0 means
+    uri / plan_info / workspace arguments; window_left as there (-1 = the whole context).  max_seq_len bounds the longest context; 0 means
     "all pages of the call could belong to one sequence"."""
     dev = _require_cuda(query, k_cache, v_cache, output, paged_kv_indptr, paged_kv_indices,
-                        paged_kv_last_page_len, output_lse)
-    _decode_common(query, k_cache, output)
+                        paged_kv_last_page_len, output_lse, k_cache_quant_scale, v_cache_quant_scale)
+    _decode_common(query, k_cache, output, v_cache, k_cache_quant_scale, v_cache_quant_scale)
     B, Hq, D = query.shape
     P, bs, Hkv, _ = k_cache.shape
     for t, n in ((paged_kv_indptr, B + 1), (paged_kv_last_page_len, B)):
@@ -268,7 +283,7 @@ def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
         query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(output_lse),
         paged_kv_indptr.data_ptr(), paged_kv_indices.data_ptr(), paged_kv_last_page_len.data_ptr(),
         _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D, bs, P,
-        query.stride(0), output.stride(0), max_seq_len, float(sm_scale), ws.data_ptr(), ws.numel(),
+        query.stride(0), output.stride(0), max_seq_len, int(window_left), float(sm_scale), ws.data_ptr(), ws.numel(),
         _dtype_code(query), _dtype_code(k_cache), _stream(dev))
     capi.check(rc, "xllm_mi355_paged_decode_gqa_csr")
     return output
@@ -276,7 +291,7 @@ def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
 
 def paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_cu_seq_lens, scale=None,
                   is_causal=True, max_seq_len=0, k_cache_quant_scale=None, v_cache_quant_scale=None,
-                  max_query_len=0):
+                  max_query_len=0, window_left=-1):
     """Short query chunks (chunked prefill, speculative-decoding verification) against paged KV:
     the decode branch of FlashAttentionImpl::paged_forward (layers/dcu/flash_attention.cpp:447-545).
     query/output packed [T, Hq, D]; q_cu_seq_lens [B + 1] int32 from 0 to T; kv_seq_lens [B] int32 are
@@ -285,7 +300,7 @@ def paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_c
     chunk lengths; 0 = unknown.  Returns output."""
     dev = _require_cuda(query, k_cache, v_cache, output, block_table, kv_seq_lens, q_cu_seq_lens,
                         k_cache_quant_scale, v_cache_quant_scale)
-    _decode_common(query, k_cache, output)
+    _decode_common(query, k_cache, output, v_cache, k_cache_quant_scale, v_cache_quant_scale)
     T, Hq, D = query.shape
     P, bs, Hkv, _ = k_cache.shape
     B = kv_seq_lens.numel()
@@ -300,6 +315,11 @@ def paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_c
         scale = D ** -0.5
     if max_seq_len <= 0:
         max_seq_len = block_table.shape[1] * bs
+    if max_query_len > 0 and not torch.cuda.is_current_stream_capturing():
+        # (a host read, so only outside capture: a chunk longer than the bound would leave its tail unwritten)
+        longest = int((q_cu_seq_lens[1:] - q_cu_seq_lens[:-1]).max()) if B > 0 else 0
+        if longest > max_query_len:
+            raise ValueError(f"max_query_len is {max_query_len} but a chunk has {longest} query tokens")
     lib = capi.lib()
     nbytes = lib.xllm_mi355_paged_decode_varlen_workspace_bytes(max(T, B), Hq, D)
     ws = decode_workspace(dev, nbytes)
@@ -307,15 +327,20 @@ def paged_forward(query, output, k_cache, v_cache, block_table, kv_seq_lens, q_c
         query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
         q_cu_seq_lens.data_ptr(), kv_seq_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
         _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, T, int(max_query_len), Hq, Hkv, D, bs, P,
-        query.stride(0), output.stride(0), max_seq_len, float(scale), 1 if is_causal else 0,
+        query.stride(0), output.stride(0), max_seq_len, int(window_left), float(scale), 1 if is_causal else 0,
         ws.data_ptr(), ws.numel(), _dtype_code(query), _dtype_code(k_cache), _stream(dev))
     capi.check(rc, "xllm_mi355_paged_decode_gqa_varlen")
     return output
 
 
+class DenseDecodeKind:
+    """flash_mla::DenseDecodeKind (xllm/core/kernels/dcu/flash_mla_adapter.h:29-31)."""
+    kQNopePe = 0
+
+
 @dataclass
 class DenseDecodeParams:
-    """flash_mla::DenseDecodeParams (xllm/core/kernels/dcu/flash_mla_adapter.h:40-53)."""
+    """flash_mla::DenseDecodeParams (xllm/core/kernels/dcu/flash_mla_adapter.h:40-50), field for field."""
     q_nope: torch.Tensor       # [B, S_q, H, kv_lora_rank]
     q_pe: torch.Tensor         # [B, S_q, H, rope]
     k_cache: torch.Tensor      # [P, bs, 1, kv_lora_rank + rope]
@@ -324,17 +349,24 @@ class DenseDecodeParams:
     head_size_v: int = 0
     softmax_scale: float = -1.0
     is_causal: bool = False
+    kind: int = DenseDecodeKind.kQNopePe
 
 
 def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0):
-    """flash_mla::dense_decode (flash_mla_adapter.cpp:104-153): returns [B, S_q, H, head_size_v]
-    (and lse [B, H, 1] when asked).  The same argument checks; S_q must be 1 on this path."""
+    """flash_mla::dense_decode (flash_mla_adapter.cpp:104-153): returns [B, S_q, H, head_size_v] (and the natural-log
+    lse [B, H, S_q] fp32 when asked).  The same argument checks.  BF16 and FP16.  The S_q query tokens of a sequence
+    are folded into the head count as the reference folds them (:119-123); with is_causal and S_q > 1 token j attends
+    to the first seqlens_k - (S_q - 1 - j) tokens and every (sequence, token) becomes a row of its own."""
     p = params
+    if p.kind != DenseDecodeKind.kQNopePe:
+        raise ValueError("flash_mla: only DenseDecodeKind::kQNopePe (BF16/FP16 split-q) is supported")
     dev = _require_cuda(p.q_nope, p.q_pe, p.k_cache, p.seqlens_k, p.block_table)
     if p.q_nope.dim() != 4 or p.q_pe.dim() != 4:
         raise ValueError("flash_mla: q_nope / q_pe must be 4D [B,S_q,H_q,D]")
     if p.k_cache.dim() != 4 or p.k_cache.shape[2] != 1:
         raise ValueError("flash_mla: k_cache must be 4D [blocks,page,1,D] with a single KV head")
+    if p.seqlens_k.dim() != 1 or p.block_table.dim() != 2:
+        raise ValueError("flash_mla: seqlens_k must be 1D [B] and block_table 2D [B,max_blocks]")
     B, Sq, H, d_latent = p.q_nope.shape
     d_rope = p.q_pe.shape[3]
     if p.q_pe.shape[:3] != p.q_nope.shape[:3]:
@@ -345,29 +377,43 @@ def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0):
         raise ValueError("flash_mla: head_size_v must be positive")
     if p.softmax_scale <= 0:
         raise ValueError("flash_mla: softmax_scale must be set by the MLA attention layer")
-    if Sq != 1:
-        raise NotImplementedError("decode path: one query token per sequence")
+    if p.seqlens_k.numel() != B or p.block_table.shape[0] != B:
+        raise ValueError("flash_mla: seqlens_k and block_table must have one row per sequence")
+    if not p.k_cache.is_contiguous():
+        raise ValueError("flash_mla: k_cache must be contiguous")
+    if not (p.q_nope.dtype == p.q_pe.dtype == p.k_cache.dtype) or p.q_nope.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError("flash_mla: q_nope, q_pe and k_cache must share one dtype, BF16 or FP16")
     if p.head_size_v != d_latent:
         raise NotImplementedError("V is the latent part of the cache: head_size_v must equal kv_lora_rank")
-    seqlens = p.seqlens_k if p.seqlens_k.dtype == torch.int32 else p.seqlens_k.to(torch.int32)
+    seqlens = (p.seqlens_k if p.seqlens_k.dtype == torch.int32 else p.seqlens_k.to(torch.int32)).contiguous()
     table = p.block_table if p.block_table.dtype == torch.int32 else p.block_table.to(torch.int32)
+    if table.stride(1) != 1:
+        table = table.contiguous()
     q_nope = p.q_nope.contiguous()
     q_pe = p.q_pe.contiguous()
     P, bs = p.k_cache.shape[0], p.k_cache.shape[1]
     out = torch.empty(B, Sq, H, p.head_size_v, dtype=q_nope.dtype, device=dev)
-    lse = torch.empty(B, H, 1, dtype=torch.float32, device=dev) if return_lse else None
+    rows, heads = B, Sq * H
+    if p.is_causal and Sq > 1:
+        rows, heads = B * Sq, H
+        back = torch.arange(Sq - 1, -1, -1, dtype=torch.int32, device=dev)
+        seqlens = (seqlens.unsqueeze(1) - back.unsqueeze(0)).clamp_min(0).reshape(rows).contiguous()
+        table = table.repeat_interleave(Sq, 0).contiguous()
+    lse = torch.empty(rows, heads, dtype=torch.float32, device=dev) if return_lse else None
     if max_seq_len <= 0:
         max_seq_len = table.shape[1] * bs
     lib = capi.lib()
-    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, H, d_latent, max_seq_len)
+    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(rows, heads, d_latent, max_seq_len)
     ws = decode_workspace(dev, nbytes)
     rc = lib.xllm_mi355_paged_decode_mla(
         q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), _ptr(lse),
-        table.data_ptr(), table.stride(0), seqlens.data_ptr(), B, H, d_latent, d_rope, bs, P,
+        table.data_ptr(), table.stride(0), seqlens.data_ptr(), rows, heads, d_latent, d_rope, bs, P,
         max_seq_len, float(p.softmax_scale), ws.data_ptr(), ws.numel(), _dtype_code(q_nope),
         _stream(dev))
     capi.check(rc, "xllm_mi355_paged_decode_mla")
-    return (out, lse) if return_lse else out
+    if return_lse:
+        return out, lse.view(B, Sq, H).transpose(1, 2).contiguous()
+    return out
 
 
 # ------------------------------------------------------------------------------------------
@@ -394,6 +440,33 @@ def merge_dcp_attention_shards(partial_outputs, partial_lse):
                                          S, B, H, Dv, _dtype_code(po), _stream(dev))
     capi.check(rc, "xllm_mi355_lse_merge")
     return out, lse
+
+
+def lse_combine(output, shared_o, shared_lse, unshared_o, unshared_lse):
+    """xllm::kernel::cuda::lse_combine (kernels/cuda/xattention/lse_combine.cu:99-166), same arguments: shared_o /
+    unshared_o [B, H, D], the LSEs [B, H, 1] fp32 in BASE 2; output [B, H, D] (allocated like shared_o when None or
+    of another shape).  Returns output."""
+    dev = _require_cuda(output, shared_o, shared_lse, unshared_o, unshared_lse)
+    if shared_o.dim() != 3 or unshared_o.dim() != 3:
+        raise ValueError("shared_o and unshared_o must be 3D [B, H, D]")
+    if shared_lse.dim() != 3 or unshared_lse.dim() != 3:
+        raise ValueError("shared_lse and unshared_lse must be 3D [B, H, 1]")
+    if shared_o.shape != unshared_o.shape or shared_o.dtype != unshared_o.dtype:
+        raise ValueError("shared_o and unshared_o must have same shape")
+    B, H, D = shared_o.shape
+    for t in (shared_lse, unshared_lse):
+        if t.dtype != torch.float32 or tuple(t.shape) != (B, H, 1):
+            raise ValueError("the LSEs must be float32 [B, H, 1]")
+    if output is None or output.shape != shared_o.shape:
+        output = torch.empty_like(shared_o)
+    so, uo = shared_o.contiguous(), unshared_o.contiguous()
+    if not output.is_contiguous():
+        raise ValueError("output must be contiguous")
+    rc = capi.lib().xllm_mi355_lse_combine(
+        output.data_ptr(), so.data_ptr(), shared_lse.contiguous().data_ptr(), uo.data_ptr(),
+        unshared_lse.contiguous().data_ptr(), B * H, D, _dtype_code(so), _dtype_code(output), _stream(dev))
+    capi.check(rc, "xllm_mi355_lse_combine")
+    return output
 
 
 def build_block_table_from_paged_kv(paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len,
@@ -437,22 +510,49 @@ def fused_qk_norm_rope(qkv, num_heads_q, num_heads_k, num_heads_v, head_dim, eps
     [T, (Hq + Hk + Hv) * D] is normalised and rotated in place.  With k_cache / v_cache / slot_mapping the same
     launch also writes the new k and v rows into the paged cache (the reshape_paged_cache call that follows in the
     reference); fp8 caches take the per-KV-head scales."""
-    dev = _require_cuda(qkv, cos_sin_cache, position_ids)
+    dev = _require_cuda(qkv, cos_sin_cache, position_ids, q_weight, k_weight, k_cache, v_cache, slot_mapping,
+                        k_cache_scale, v_cache_scale)
     if qkv.dim() != 2 or qkv.stride(1) != 1:
         raise ValueError("qkv must be [tokens, (Hq + Hk + Hv) * head_dim] with contiguous rows")
-    if position_ids.dtype != torch.int64 or not position_ids.is_contiguous():
-        raise ValueError("position_ids must be a contiguous int64 tensor")
+    if qkv.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError("qkv must be bf16 or fp16")
+    T = qkv.shape[0]
+    if qkv.shape[1] != (num_heads_q + num_heads_k + num_heads_v) * head_dim:
+        raise ValueError("qkv width must be (Hq + Hk + Hv) * head_dim")
+    if position_ids.dtype != torch.int64 or not position_ids.is_contiguous() or position_ids.numel() != T:
+        raise ValueError("position_ids must be a contiguous int64 tensor [tokens]")
     if cos_sin_cache.dim() != 2 or not cos_sin_cache.is_contiguous():
         raise ValueError("cos_sin_cache must be [max_position, rotary_dim], contiguous")
+    if (q_weight is None) != (k_weight is None):
+        raise ValueError("q_weight and k_weight go together")
+    for w in (q_weight, k_weight):
+        if w is not None and (w.dtype != qkv.dtype or w.numel() != head_dim or not w.is_contiguous()):
+            raise ValueError("q_weight / k_weight must be contiguous [head_dim] tensors of the qkv dtype")
     with_cache = k_cache is not None
-    fp8 = with_cache and k_cache.dtype == torch.float8_e4m3fn
+    cache_code = _dtype_code(qkv)
+    if with_cache:
+        if v_cache is None or slot_mapping is None:
+            raise ValueError("the fused cache write needs k_cache, v_cache and slot_mapping")
+        if (k_cache.dim() != 4 or tuple(k_cache.shape[2:]) != (num_heads_k, head_dim) or not k_cache.is_contiguous()
+                or v_cache.shape != k_cache.shape or v_cache.dtype != k_cache.dtype or not v_cache.is_contiguous()
+                or num_heads_v != num_heads_k):
+            raise ValueError("k_cache / v_cache must be contiguous [P, bs, num_heads_k, head_dim] of one dtype")
+        if slot_mapping.dtype != torch.int32 or not slot_mapping.is_contiguous() or slot_mapping.numel() != T:
+            raise ValueError("slot_mapping must be contiguous int32 [tokens]")
+        cache_code = _dtype_code(k_cache)   # fp8 caches are float8_e4m3fn or uint8 tensors
+        if cache_code == capi.FP8_E4M3:
+            for sc in (k_cache_scale, v_cache_scale):
+                if sc is None or sc.dtype != torch.float32 or sc.numel() != num_heads_k or not sc.is_contiguous():
+                    raise ValueError("an fp8 cache needs contiguous fp32 scales [num_heads_k] for K and V")
+        elif k_cache.dtype != qkv.dtype:
+            raise TypeError("the cache dtype must equal the qkv dtype (or be fp8)")
     rc = capi.lib().xllm_mi355_rope_and_cache(
         qkv.data_ptr(), _ptr(q_weight), _ptr(k_weight), cos_sin_cache.data_ptr(), position_ids.data_ptr(),
         _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), _ptr(k_cache_scale), _ptr(v_cache_scale),
         qkv.shape[0], qkv.stride(0), num_heads_q, num_heads_k, num_heads_v, head_dim, cos_sin_cache.shape[1],
         float(eps), 1 if interleave else 0, k_cache.shape[1] if with_cache else 0,
         k_cache.shape[0] if with_cache else 0, _dtype_code(qkv), _dtype_code(cos_sin_cache),
-        capi.FP8_E4M3 if fp8 else _dtype_code(qkv), _stream(dev))
+        cache_code, _stream(dev))
     capi.check(rc, "xllm_mi355_rope_and_cache")
     return qkv
 

@@ -7,8 +7,13 @@ over the C ABI, registered with the torch dispatcher as torch.ops.xllm_ops.*.
   torch.ops.xllm_ops.batch_decode(query, k_cache, v_cache, output, block_table, seq_lens,
                                   k_scale, v_scale, max_seq_len, scale) -> (output, lse)
   torch.ops.xllm_ops.mla_dense_decode(q_nope, q_pe, k_cache, seqlens_k, block_table,
-                                      head_size_v, softmax_scale) -> (out, lse)
+                                      head_size_v, softmax_scale, is_causal=False) -> (out, lse)
   torch.ops.xllm_ops.merge_dcp_attention_shards(partial_outputs, partial_lse) -> (out, lse)
+  torch.ops.xllm_ops.lse_combine(output, shared_o, shared_lse, unshared_o, unshared_lse) -> output   (base-2 LSEs)
+  torch.ops.xllm_ops.attention_layer_forward(query, key, value, k_cache, v_cache, k_cache_scale, v_cache_scale,
+        slot_mapping, block_table, kv_seq_lens, q_cu_seq_lens, max_seq_len, max_query_len, num_heads, head_size,
+        num_kv_heads, scale, sliding_window, is_causal, return_lse) -> (output [T, Hq * D], lse or None)
+      -- AttentionImpl::forward of the reference (xllm/core/layers/dcu/attention.cpp:55-112) end to end
 """
 import os
 
