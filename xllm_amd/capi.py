@@ -7,7 +7,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libxllm_mi355.so")
+# XLLM_MI355_LIBRARY names another build of the same library (A/B measurements of kernel variants)
+LIB_PATH = os.environ.get("XLLM_MI355_LIBRARY") or os.path.join(_HERE, "libxllm_mi355.so")
 
 BF16, FP16, FP32, FP8_E4M3 = 0, 1, 2, 3
 

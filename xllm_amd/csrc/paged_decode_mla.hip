@@ -62,6 +62,7 @@ typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 typedef __attribute__((address_space(3))) float lds_f32;
+typedef __attribute__((address_space(3))) volatile int lds_vint;  // a word of LDS that other wavefronts write
 struct MlaArgs {
   const char* q_nope;
   const char* q_pe;
@@ -503,6 +504,10 @@ __device__ __forceinline__ void wait_younger_subs(int subs) {
 // theirs to their partners through the (then idle) ring, merged like two partials.
 template <typename QT, bool SPLIT>
 __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
+#ifdef XLLM_DS_TIMING
+  const unsigned long long w_entry16 = wall_clock64();
+  const unsigned long long t_entry16 = __builtin_readcyclecounter();
+#endif
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kPrefix16Off);
   const int* pagebuf = reinterpret_cast<const int*>(smem + kPage16Off);
@@ -868,6 +873,484 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
     if (writer && g == 0 && !complete) a.ws_lse[ps] = lse2;
     first_run = false;
   }
+#ifdef XLLM_DS_TIMING
+  if ((threadIdx.x & 63) == 0) {
+    unsigned long long* dst = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * a.n_heads) +
+                              (blockIdx.x * 8 + (threadIdx.x >> 6)) * 10;
+    dst[0] = w_entry16;
+    dst[1] = wall_clock64();
+    dst[8] = __builtin_readcyclecounter() - t_entry16;
+    dst[9] = (dst[1] - dst[0]) << 32;
+  }
+#endif
+}
+
+// ---------------------------------------------------------------------------------------------
+// The kernel for more than 64 heads: scores by head block, P.V by DIM block, the two out of phase on a SIMD.
+//
+// In mla_decode16_kernel every wavefront reads the whole K tile AND the whole V tile from LDS for its 16 heads:
+// 68 KB per wavefront and sub-tile, 544 KB per workgroup, against an LDS that delivers 128 bytes per cycle and
+// a matrix pipe that needs 2176 cycles for the same sub-tile: the loop runs at the pace of the LDS.  Here the
+// second product is cut the other way.  Wavefront w still computes S^T for heads 16w .. 16w+15 (Q^T stays in 72
+// registers, K operands from LDS as before) and their softmax, and leaves its P^T block (32 tokens x 16 heads,
+// 1 KB, already in the B-operand layout) in LDS.  After the barrier every wavefront multiplies ALL 8 P^T blocks
+// with ITS 64 output dims: O^T[dims 64w .. 64w+63, all 128 heads] in the same 128 accumulator registers.  Its
+// A operands are 4 KB of V^T instead of 32 KB, its B operands the 8 KB of P^T: 49 KB per wavefront and sub-tile
+// instead of 68, 392 KB per workgroup instead of 544.
+//
+// One barrier per sub-tile.  Between barrier t and barrier t + 1 a wavefront has two independent jobs: P.V of
+// sub-tile t (its V^T operands are already in registers, P^T of t is complete) and the scores + softmax of
+// sub-tile t + 1 (into the other P^T buffer).  Wavefronts 0-3 take them in this order, wavefronts 4-7 in the
+// other: a SIMD holds one of each, so while one keeps the matrix pipe busy with P.V (light on LDS) the other
+// streams K operands from LDS for its scores (light on the matrix pipe), and their tile loads go out at different
+// times.  A wavefront reads the V^T operands of a sub-tile right after it is done with its scores, so after the
+// next barrier nobody needs the sub-tile any more and its ring slot is refilled at once: three slots keep two
+// sub-tiles in flight.
+//
+// The running maximum and sum of a head stay with the wavefront that owns its scores; when a maximum moves
+// (rare, the maxima carry kSlack of head room) the owner leaves the factor in LDS and raises a flag, and every
+// wavefront rescales that head block's accumulators before it adds the sub-tile.  At the end of a run the
+// owners publish 1 / sum and every wavefront writes its dims.
+// LDS: ring [3 sub-tiles] | P^T [2][8 blocks] | factors [2][128] | flags [3] | page chunks [2][64] | prefix.
+#ifndef XLLM_DS_AHEAD
+#define XLLM_DS_AHEAD 2
+#endif
+constexpr int kDsRing = 3;
+constexpr int kDsPOff = kDsRing * kSubBytes;               // P^T blocks: [2][8][64 lanes][16 bytes]
+constexpr int kDsFacOff = kDsPOff + 2 * 8 * 1024;          // [2][128] rescale factors of a sub-tile; [128] 1 / sum at the end
+constexpr int kDsFlagOff = kDsFacOff + 2 * kHeadsPerWg16 * 4;  // [3] head blocks whose maximum moved, by sub-tile % 3
+constexpr int kDsPageOff = kDsFlagOff + 16;
+constexpr int kDsStashOff = kDsPageOff + 2 * kWave * 4;   // V^T operands of wavefronts 4-7 between two windows: [4][4 KB]
+constexpr int kDsPrefixOff = kDsStashOff + 4 * 4096;
+constexpr int kDsMaxBatch = kMaxBatchMla;
+constexpr int kDsLdsBytes = kDsPrefixOff + (kDsMaxBatch + 1) * 4;
+static_assert(kDsLdsBytes <= 160 * 1024, "LDS of a CU");
+
+template <typename QT>
+__global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
+#ifdef XLLM_DS_TIMING
+  const unsigned long long t_entry = __builtin_readcyclecounter();
+  const unsigned long long w_entry = wall_clock64();
+#endif
+  extern __shared__ __align__(16) char smem[];
+  int* prefix = reinterpret_cast<int*>(smem + kDsPrefixOff);
+  const int* pagebuf = reinterpret_cast<const int*>(smem + kDsPageOff);
+  float* fac = reinterpret_cast<float*>(smem + kDsFacOff);
+  int* flags = reinterpret_cast<int*>(smem + kDsFlagOff);
+  int* tmp = reinterpret_cast<int*>(smem);  // prologue only
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15;    // MFMA row / column index owned by the lane
+  const int g = lane >> 4;      // MFMA k-group of the lane
+  const int H = a.n_heads;
+#ifdef XLLM_DS_SAME_ORDER
+  constexpr bool pv_first = true;
+#else
+  const bool pv_first = wave < 4;  // order of the two jobs between barriers (the SIMD's other wavefront has the other)
+#endif
+
+  // block id -> (team, head block of 128): members of a team are 8 ids apart (same XCD)
+  const int xcd = blockIdx.x & 7;
+  const int y = blockIdx.x >> 3;
+  const int hb128 = y % a.n_hb;
+  const int team = (y / a.n_hb) * 8 + xcd;
+  const int head0 = hb128 * kHeadsPerWg16;
+  const int n16 = min(8, (H - head0 + 15) >> 4);       // 16-head blocks of this workgroup that hold heads
+  const int head = head0 + wave * 16 + c16;            // the head whose scores this lane owns
+  const bool head_ok = head < H;
+  const bool wave_ok = wave < n16;
+
+  // ---- tile prefix over the batch (every workgroup computes it; no extra launch)
+  {
+    const int per = (a.batch + kThreads16 - 1) / kThreads16;
+    const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
+    int local = 0;
+    for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
+    tmp[tid] = local;
+    __syncthreads();
+    if (lo < hi) {
+      int excl = 0;
+      for (int j = 0; j < tid; ++j) excl += tmp[j];
+      if (per == 1) {
+        prefix[lo] = excl;
+        excl += local;
+      } else {
+        for (int b = lo; b < hi; ++b) {
+          prefix[b] = excl;
+          excl += tiles_of(a.seq_lens[b]);
+        }
+      }
+      if (hi == a.batch) prefix[a.batch] = excl;
+    }
+    __syncthreads();
+  }
+  const int64_t total = prefix[a.batch];
+  if (blockIdx.x == 0)
+    for (int i = tid; i <= a.batch; i += kThreads16) a.ws_prefix[i] = prefix[i];
+  if (total == 0) return;
+  int64_t cur = team_start(team, total, a.n_teams);
+  const int64_t end = team_start(team + 1, total, a.n_teams);
+  bool first_run = true;
+  if (!wave_ok) {  // a head block without heads: its P^T blocks stay zero, P.V multiplies all eight
+    *reinterpret_cast<u32x4*>(smem + kDsPOff + wave * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(smem + kDsPOff + (8 + wave) * 1024 + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+  }
+
+  const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
+  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + kDsPageOff);
+  // per-lane constants of the operand reads (byte offsets inside a sub-tile), as in mla_decode16_kernel
+  const int k_row0 = c16 * kRow16 + ((g ^ ((c16 >> 2) & 1)) * 16);
+  const int v_row0 = (4 * g + (c16 >> 2)) * kRow16 + ((((c16 & 3) >> 1) ^ (g & 1)) * 16) + (c16 & 1) * 8 + wave * (4 * 32);
+  const u32 lane_off = (lane ^ (wave & 1)) * 16;
+  auto lane_again = [&]() {
+    u32 x = lane_off;
+    asm volatile("" : "+v"(x));
+    return static_cast<int>(x >> 4) ^ (wave & 1);
+  };
+
+#ifdef XLLM_DS_TIMING
+  unsigned long long tm[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned long long tk = __builtin_readcyclecounter();
+  const unsigned long long t_start = t_entry;
+  const unsigned long long w_start = w_entry;
+  tm[7] += tk - t_entry;   // (the time before the first run is booked as epilogue)
+#define DS_TICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; }
+#else
+#define DS_TICK(i)
+#endif
+  while (cur < end) {
+    int lo = 0, hi = a.batch;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (prefix[mid] <= cur) lo = mid; else hi = mid;
+    }
+    const int b = __builtin_amdgcn_readfirstlane(lo);
+    const int n_tiles_seq = prefix[b + 1] - prefix[b];
+    const int tile0 = static_cast<int>(cur - prefix[b]);
+    const int run_tiles = static_cast<int>(min<int64_t>(n_tiles_seq - tile0, end - cur));
+    const bool complete = tile0 == 0 && run_tiles == n_tiles_seq;
+    cur += run_tiles;
+    const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
+    const int L = __builtin_amdgcn_readfirstlane(a.seq_lens[b]);
+    const int t_begin = tile0 * kTile;
+    const int t_end = min(L, (tile0 + run_tiles) * kTile);
+    const int n_sub = (t_end - t_begin + kSubTok - 1) / kSubTok;
+    const int n_pages = (L + a.block_size - 1) >> a.bs_shift;
+
+    auto issue_chunk = [&](int ck) {
+      dma4(pages + min(ck * kWave + lane, n_pages - 1), page_lds + (ck & 1) * kWave * 4);
+    };
+    int ck_cur = (t_begin >> a.bs_shift) >> 6;
+    __syncthreads();  // the previous run no longer reads the ring, the chunks, the factors or the flags
+    // the page-table chunks of the run's first sub-tiles travel while the Q rows do
+    if (wave == 0) {
+      issue_chunk(ck_cur);
+      if ((ck_cur + 1) * kWave < n_pages) issue_chunk(ck_cur + 1);
+    }
+    if (tid < 3) flags[tid] = 0;
+
+    // Q^T operand: lane (head c16, k-group g) keeps dims kk*32 + g*8 .. +8 of every k-step
+    u32x4 q[kKSteps32];
+    {
+      const char* qn = a.q_nope + (static_cast<int64_t>(b) * H + head) * kDL * 2;
+      const char* qp = a.q_pe + (static_cast<int64_t>(b) * H + head) * kDR * 2;
+#pragma unroll
+      for (int kk = 0; kk < kKSteps32; ++kk) {
+        u32x4 x = {0u, 0u, 0u, 0u};
+        if (head_ok)
+          x = kk < kDL / 32 ? ldg16(qn + (kk * 32 + g * 8) * 2) : ldg16(qp + ((kk - kDL / 32) * 32 + g * 8) * 2);
+        q[kk] = x;
+      }
+    }
+    // O^T blocks of the wavefront's 64 dims: o[db][hb] = dims 64 wave + 16 db + 4g + r, head 16 hb + c16
+    f32x4 o[4][8];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int hb = 0; hb < 8; ++hb) o[db][hb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = kNegBig, l = 0.0f;
+
+    auto issue_sub = [&](int sub) {
+      const int tok0 = t_begin + sub * kSubTok + wave * 4;
+      const u32 slot = lds_base + (sub % kDsRing) * kSubBytes;
+      const u32 dst = __builtin_amdgcn_readfirstlane(slot + wave * 4 * kRow16);
+      const u32 dst_rope = __builtin_amdgcn_readfirstlane(slot + kRope16Off + wave * 4 * (kDR * 2));
+      const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
+      const int tb = min(tok0, L - 1);
+      const int ck = (tb >> a.bs_shift) >> 6;
+      if (ck != ck_cur) {
+        ck_cur = ck;
+        if (wave == 0 && (ck + 1) * kWave < n_pages) issue_chunk(ck + 1);
+      }
+      int page = __builtin_amdgcn_readfirstlane(pagebuf[(ck & 1) * kWave + ((tb >> a.bs_shift) & 63)]);
+      page = max(0, min(page, a.num_blocks - 1));
+      const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tb & (a.block_size - 1))) * kRowBytes;
+      const u32 rlo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row)));
+      const u32 rhi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row >> 32)));
+      const uint64_t sb = (static_cast<uint64_t>(rhi) << 32) | rlo;
+      const int last = __builtin_amdgcn_readfirstlane(L - 1 - tb);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dma16_row(sb + static_cast<uint64_t>(min(i, last)) * kRowBytes, lane_off, dst + i * kRow16);
+      const int ln = lane_again();
+      const int rope_r = (ln >> 3) & 3;
+      const u32 rope_off = min(rope_r, last) * kRowBytes + kDL * 2 + (((ln & 7) ^ ((wave & 1) * 4 + rope_r)) * 16);
+      if (lane < 4 * kDR * 2 / 16) dma16_row(sb, rope_off, dst_rope);
+    };
+
+    // ---- scores and softmax of sub-tile `sub` for the wavefront's 16 heads; P^T block, factor and flag to LDS
+    auto scores = [&](int sub) {
+      if (!wave_ok) return;
+      const char* kb = smem + (sub % kDsRing) * kSubBytes;
+      const int ln = lane_again();
+      const char* kr = kb + kRope16Off + (ln & 15) * (kDR * 2);
+      const int kr_x = (ln >> 4) ^ (ln & 7);
+      f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+      const char* ka = kb + k_row0;
+      // K operands kDsAhead k-steps ahead of the MFMAs that take them, in an order the scheduler may not change:
+      // left to itself it puts every read right in front of its MFMA, and a k-step then costs a whole LDS round
+      // trip (about 120 cycles against the 32 of its two MFMAs).
+      constexpr int kDsAhead = XLLM_DS_AHEAD;
+      auto k_addr = [&](int kk) -> const char* {
+        return kk < kDL / 32 ? ka + kk * 64 : kr + (kk == kDL / 32 ? kr_x : kr_x ^ 4) * 16;
+      };
+      u32x4 xa[kDsAhead], xb[kDsAhead];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < kDsAhead; ++i) {
+        xa[i] = *reinterpret_cast<const u32x4*>(k_addr(i));
+        xb[i] = *reinterpret_cast<const u32x4*>(k_addr(i) + 16 * (i < kDL / 32 ? kRow16 : kDR * 2));
+      }
+#pragma unroll
+      for (int kk = 0; kk < kKSteps32; ++kk) {
+        __builtin_amdgcn_sched_barrier(0);
+#ifdef XLLM_DS_WHATIF_NO_QK_MFMA   // (measurement only: wrong results)
+        s0[0] += as_f32(xa[kk % kDsAhead][0]);
+        s1[0] += as_f32(xb[kk % kDsAhead][0]);
+#else
+        s0 = Mfma<QT>::k32(xa[kk % kDsAhead], q[kk], s0);
+        s1 = Mfma<QT>::k32(xb[kk % kDsAhead], q[kk], s1);
+#endif
+#ifdef XLLM_DS_WHATIF_NO_K_READS   // (measurement only: wrong results)
+        if (false) {
+#else
+        if (kk + kDsAhead < kKSteps32) {
+#endif
+          const int kn = kk + kDsAhead;
+          xa[kk % kDsAhead] = *reinterpret_cast<const u32x4*>(k_addr(kn));
+          xb[kk % kDsAhead] = *reinterpret_cast<const u32x4*>(k_addr(kn) + 16 * (kn < kDL / 32 ? kRow16 : kDR * 2));
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      float sv[8];
+      const int tok_base = t_begin + sub * kSubTok + 4 * g;
+      bool over = false;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        sv[r] = tok_base + r < L ? s0[r] * a.scale_log2 : -INFINITY;
+        sv[4 + r] = tok_base + 16 + r < L ? s1[r] * a.scale_log2 : -INFINITY;
+      }
+#pragma unroll
+      for (int r = 0; r < 8; ++r) over |= sv[r] > m + kSlack;
+      if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
+        float mx = sv[0];
+#pragma unroll
+        for (int r = 1; r < 8; ++r) mx = fmaxf(mx, sv[r]);
+        mx = quad_rows_max(mx);
+        float alpha = 1.0f;
+        if (mx > m + kSlack) {
+          alpha = fast_exp2(m - mx);
+          m = mx;
+          l *= alpha;
+        }
+        // the factor of every head of the block (1 where the maximum stayed), and the block's flag (the lane's
+        // position is recomputed here: kept in registers of their own for this rare path, the addresses get spilled,
+        // and a reload from scratch waits for every tile load in flight)
+        const int lnx = lane_again();
+        if ((lnx >> 4) == 0) fac[(sub & 1) * kHeadsPerWg16 + wave * 16 + (lnx & 15)] = alpha;
+        if (lnx == 0) {
+          int bit;
+          asm volatile("s_lshl_b32 %0, 1, %1" : "=s"(bit) : "s"(wave));
+          atomicOr(flags + sub % 3, bit);
+        }
+      }
+      float p[8];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        p[r] = fast_exp2(sv[r] - m);
+        l += p[r];
+      }
+      // k-slot g*8 + j of the P.V MFMA <-> token 4g + j of block 0 (j < 4), of block 1 (j >= 4): the lane's
+      // eight probabilities are its 16 bytes of the B operand
+      const u32x4 pb = {QT::pack(p[0], p[1]), QT::pack(p[2], p[3]), QT::pack(p[4], p[5]), QT::pack(p[6], p[7])};
+      *reinterpret_cast<u32x4*>(smem + kDsPOff + ((sub & 1) * 8 + wave) * 1024 + lane * 16) = pb;
+    };
+    // ---- the V^T operands of sub-tile `sub` for the wavefront's dims, into registers
+    auto read_vt = [&](int sub, u32x4 (&vt)[4]) {
+      const char* va = smem + (sub % kDsRing) * kSubBytes + v_row0;
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+        const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + db * 32));
+        const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + 16 * kRow16 + db * 32));
+        const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+        vt[db] = __builtin_bit_cast(u32x4, v);
+      }
+    };
+    // ---- O^T[64 dims of the wavefront, all heads] += V^T . P^T of sub-tile `sub` (its P^T blocks are complete)
+    auto pv = [&](int sub, const u32x4 (&vt)[4]) {
+      // (read as LDS on purpose: a generic volatile pointer becomes a flat load, whose wait drains the tile loads in flight)
+      const int moved = __builtin_amdgcn_readfirstlane(*((lds_vint*)(smem + kDsFlagOff) + sub % 3));
+      if (moved != 0) {
+#pragma unroll
+        for (int hb = 0; hb < 8; ++hb) {
+          if ((moved >> hb) & 1) {
+            const float f = fac[(sub & 1) * kHeadsPerWg16 + hb * 16 + c16];
+#pragma unroll
+            for (int db = 0; db < 4; ++db) o[db][hb] *= f;
+          }
+        }
+      }
+      // all P^T blocks first: their reads return in order, so the MFMAs of a block start as soon as it is there
+      // while the later blocks are still on their way (a read per block in front of its MFMAs would put the LDS
+      // latency on the path eight times).  Blocks without heads hold zeros.
+      const char* pbase = smem + kDsPOff + (sub & 1) * 8 * 1024 + lane * 16;
+      u32x4 pb[8];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int hb = 0; hb < 8; ++hb) pb[hb] = *reinterpret_cast<const u32x4*>(pbase + hb * 1024);
+#pragma unroll
+      for (int hb = 0; hb < 8; ++hb)
+#pragma unroll
+        for (int db = 0; db < 4; ++db) o[db][hb] = Mfma<QT>::k32(vt[db], pb[hb], o[db][hb]);
+      // kPvAhead block reads ahead of the MFMAs that use them (registers allow three blocks in flight)
+      constexpr int kPvAhead = 3;
+      __builtin_amdgcn_sched_group_barrier(0x100, kPvAhead, 0);
+#pragma unroll
+      for (int i = 0; i < 8 - kPvAhead; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * kPvAhead, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // the chunk loads and the Q loads have landed (one wait for both latencies)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int kk = 0; kk < kKSteps32; ++kk) asm volatile("" : "+v"(q[kk]));
+    __syncthreads();
+    for (int sub = 0; sub < kDsRing && sub < n_sub; ++sub) issue_sub(sub);
+    // sub-tile 0 before the loop
+    wait_younger_subs(min(kDsRing - 1, n_sub - 1));
+    __syncthreads();
+    scores(0);
+    if (pv_first) {
+      // ---- wavefronts 0-3: P.V of `sub`, then the scores of sub + 1; the V^T operands wait in registers
+      u32x4 vt[4];  // V^T operands of the sub-tile whose P.V comes next: dims 64 wave + 16 db .., its 32 tokens
+      read_vt(0, vt);
+      DS_TICK(0)   // run prologue
+      for (int sub = 0; sub < n_sub; ++sub) {
+        // the wavefront's rows of sub-tile sub + 1 have landed (sub + 2 may still be in flight)
+        wait_younger_subs(min(kDsRing - 2, n_sub - 2 - sub));
+        DS_TICK(1)
+        __syncthreads();  // P^T of `sub` is complete; sub + 1 has landed; nobody reads sub-tile `sub` in LDS any more
+        DS_TICK(2)
+        if (tid == 0) flags[(sub + 2) % 3] = 0;   // (last read before this barrier, next raised after the next one)
+        if (sub + kDsRing < n_sub) issue_sub(sub + kDsRing);
+        DS_TICK(3)
+        pv(sub, vt);
+        DS_TICK(6)
+        if (sub + 1 < n_sub) {
+          scores(sub + 1);
+          read_vt(sub + 1, vt);
+        }
+        DS_TICK(4)
+      }
+    } else {
+      // ---- wavefronts 4-7: the scores of sub + 1, then P.V of `sub`.  They park the V^T operands (read while the
+      // sub-tile is still in the ring) in a private piece of LDS instead of holding 16 registers across the scores.
+      char* stash = smem + kDsStashOff + (wave & 3) * 4096 + lane * 16;
+      {
+        u32x4 vt[4];
+        read_vt(0, vt);
+#pragma unroll
+        for (int db = 0; db < 4; ++db) *reinterpret_cast<u32x4*>(stash + db * 1024) = vt[db];
+      }
+      DS_TICK(0)
+      for (int sub = 0; sub < n_sub; ++sub) {
+        wait_younger_subs(min(kDsRing - 2, n_sub - 2 - sub));
+        DS_TICK(1)
+        __syncthreads();
+        DS_TICK(2)
+        const bool more = sub + 1 < n_sub;
+        if (more) scores(sub + 1);
+        DS_TICK(4)
+        if (sub + kDsRing < n_sub) issue_sub(sub + kDsRing);
+        DS_TICK(3)
+        u32x4 vt[4];
+#pragma unroll
+        for (int db = 0; db < 4; ++db) vt[db] = *reinterpret_cast<const u32x4*>(stash + db * 1024);
+        pv(sub, vt);
+        if (more) {
+          read_vt(sub + 1, vt);
+#pragma unroll
+          for (int db = 0; db < 4; ++db) *reinterpret_cast<u32x4*>(stash + db * 1024) = vt[db];
+        }
+        DS_TICK(6)
+      }
+    }
+
+    // ---- end of the run: the owners publish 1 / sum per head, every wavefront writes its dims of every head
+    const float lsum = quad_rows_sum(l);
+    const float lse2 = m + fast_log2(lsum);
+    const int64_t ps_base = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H;
+    __syncthreads();  // the last sub-tile's factors have been read
+    if (wave_ok && g == 0) fac[wave * 16 + c16] = 1.0f / lsum;
+    if (wave_ok && head_ok && g == 0) {
+      if (complete && a.lse != nullptr) a.lse[b * H + head] = lse2 * kLn2;
+      if (!complete) a.ws_lse[ps_base + head] = lse2;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int hb = 0; hb < 8; ++hb) {
+      const int hd = head0 + hb * 16 + c16;
+      if (hb < n16 && hd < H) {
+        const float inv = fac[hb * 16 + c16];
+        if (complete) {
+          char* op = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + wave * 64 + 4 * g) * 2;
+#pragma unroll
+          for (int db = 0; db < 4; ++db) {
+            const u32x2 w = {QT::pack(o[db][hb][0] * inv, o[db][hb][1] * inv), QT::pack(o[db][hb][2] * inv, o[db][hb][3] * inv)};
+            *reinterpret_cast<u32x2*>(op + db * 32) = w;
+          }
+        } else {
+          float* wp = a.ws_out + (ps_base + hd) * kDL + wave * 64 + 4 * g;
+#pragma unroll
+          for (int db = 0; db < 4; ++db) {
+            const f32x4 w = {o[db][hb][0] * inv, o[db][hb][1] * inv, o[db][hb][2] * inv, o[db][hb][3] * inv};
+            *reinterpret_cast<f32x4*>(wp + db * 16) = w;
+          }
+        }
+      }
+    }
+    first_run = false;
+    DS_TICK(7)   // run epilogue
+  }
+#ifdef XLLM_DS_TIMING
+  // (measurement build only) per-phase cycle sums of every wavefront of every workgroup, behind the partials
+  if (lane == 0) {
+    unsigned long long* dst = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H) +
+                              (blockIdx.x * 8 + wave) * 10;
+    for (int i = 0; i < 8; ++i) dst[i] = tm[i];
+    dst[0] = w_entry;            // (absolute 100 MHz time stamps of entry and exit instead of two of the sums)
+    dst[1] = wall_clock64();
+    dst[8] = __builtin_readcyclecounter() - t_start;
+    dst[9] = static_cast<unsigned long long>(end - team_start(team, total, a.n_teams)) |
+             ((wall_clock64() - w_start) << 32);   // high half: the same span on the constant 100 MHz clock
+  }
+#endif
+#undef DS_TICK
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1452,6 +1935,10 @@ __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
   const int b = blockIdx.y;
   const int H = a.n_heads;
   const int d = threadIdx.x * 4;
+#ifdef XLLM_DS_TIMING
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)   // (measurement build only) when the merge kernel starts
+    reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H)[2048 * 10] = wall_clock64();
+#endif
   const int64_t first = a.ws_prefix[b];
   const int64_t last = static_cast<int64_t>(a.ws_prefix[b + 1]) - 1;
   const int64_t total = a.ws_prefix[a.batch];
@@ -1582,6 +2069,9 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   const int knob = mla_kernel_knob();
   const bool pairs = knob == 'p' || block_size < 16 || (block_size & (block_size - 1)) != 0;
   const bool split = knob == 's' && !pairs && !f16;  // (the producer / consumer kernel is written for bf16)
+  // more than 64 heads: scores by head block, P.V by dim block ("heads" keeps P.V by head block, for comparison)
+  const bool by_dims = !pairs && !split && knob != 'h' && n_heads > 64;
+  const int64_t max_batch = by_dims ? (kDsMaxBatch < kMaxBatchMla ? kDsMaxBatch : kMaxBatchMla) : kMaxBatchMla;
   const int n_hb = static_cast<int>(pairs ? (n_heads + kHeadsPerWg - 1) / kHeadsPerWg
                                           : (n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
   const int n_hb_p = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
@@ -1601,13 +2091,17 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_pairs);
     for (const void* k : kernels_16)
       if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_16);
+    const void* kernels_ds[] = {reinterpret_cast<const void*>(mla_decode_ds_kernel<BF16>),
+                                reinterpret_cast<const void*>(mla_decode_ds_kernel<FP16>)};
+    for (const void* k : kernels_ds)
+      if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kDsLdsBytes);
     if (e == hipSuccess)
       e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode32w_kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
     if (e != hipSuccess) return static_cast<int>(e);
   }
-  for (int64_t b0 = 0; b0 < batch; b0 += kMaxBatchMla) {
-    const int64_t nb = batch - b0 < kMaxBatchMla ? batch - b0 : kMaxBatchMla;
+  for (int64_t b0 = 0; b0 < batch; b0 += max_batch) {
+    const int64_t nb = batch - b0 < max_batch ? batch - b0 : max_batch;
     MlaArgs a = {};
     a.q_nope = static_cast<const char*>(q_nope) + b0 * n_heads * kDL * 2;
     a.q_pe = static_cast<const char*>(q_pe) + b0 * n_heads * kDR * 2;
@@ -1638,6 +2132,9 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       else launch_timed(mla_decode_kernel<BF16>, grid, dim3(kMlaThreads), smem, stream, a);
     } else if (use_p) {
       launch_timed(mla_decode32w_kernel, grid, dim3(kWThreads), kPLdsBytes, stream, a);
+    } else if (by_dims) {
+      if (f16) launch_timed(mla_decode_ds_kernel<FP16>, grid, dim3(kThreads16), kDsLdsBytes, stream, a);
+      else launch_timed(mla_decode_ds_kernel<BF16>, grid, dim3(kThreads16), kDsLdsBytes, stream, a);
     } else if (n_heads <= 64) {  // head counts of tensor-parallel shards: two wavefronts per 16 heads
       if (f16) launch_timed(mla_decode16_kernel<FP16, true>, grid, dim3(kThreads16), smem, stream, a);
       else launch_timed(mla_decode16_kernel<BF16, true>, grid, dim3(kThreads16), smem, stream, a);
