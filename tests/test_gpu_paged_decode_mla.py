@@ -124,28 +124,47 @@ def test_token_blocks_on_different_wavefronts_for_few_heads(device):
         _check(_mla_cfg(f"few32_L{L}", 2, 32, L, L), 50 + L, device)
 
 
+def _rising_scores_case(heads, lo, hi, bs, device):
+    cfg = _mla_cfg(f"ramp{heads}", 3, heads, lo, hi, bs=bs)
+    inp = workloads.make_inputs(cfg, 31)
+    lay = inp.layout
+    inp.q[:, :, 512:] = 2.0
+    for b in range(cfg.batch):
+        o0, o1 = int(lay.ctx_offsets[b]), int(lay.ctx_offsets[b + 1])
+        n = o1 - o0
+        ramp = (torch.arange(n, dtype=torch.float32) * (9.0 / max(n, 1))).to(torch.bfloat16)
+        inp.k_ctx[o0:o1, 0, 512:] = ramp[:, None]
+    inp.k_new[:, 0, 512:] = 9.0
+    kg, _, _, _ = fill_caches_gpu(inp, device)
+    kc, _ = fill_caches_cpu(inp)
+    out, lse = _decode_gpu(inp, kg, device)
+    ref = oracle.aten_paged_decode(inp.q, kc, None, lay.block_table, lay.seq_lens, cfg.scale, dv=cfg.v_dim)
+    assert_close_to_reference(out, ref, cfg.name)
+    ref_lse = oracle.aten_paged_decode_lse(inp.q, kc, lay.block_table, lay.seq_lens, cfg.scale)
+    assert torch.allclose(lse.cpu(), ref_lse, rtol=1e-3, atol=1e-3)
+
+
 def test_scores_that_rise_along_the_context(device):
     # the rope dims of K carry a ramp and those of Q a constant, so the scores rise by about 120 log2 units from
     # the first token to the last: every running maximum is overtaken many times and whatever was accumulated
     # before has to be rescaled (or restarted) again and again; V = K[..., :512] is unaffected
     for heads, lo, hi, bs in ((128, 1500, 2500, 64), (16, 700, 900, 16), (32, 1500, 2500, 64)):
-        cfg = _mla_cfg(f"ramp{heads}", 3, heads, lo, hi, bs=bs)
-        inp = workloads.make_inputs(cfg, 31)
-        lay = inp.layout
-        inp.q[:, :, 512:] = 2.0
-        for b in range(cfg.batch):
-            o0, o1 = int(lay.ctx_offsets[b]), int(lay.ctx_offsets[b + 1])
-            n = o1 - o0
-            ramp = (torch.arange(n, dtype=torch.float32) * (9.0 / max(n, 1))).to(torch.bfloat16)
-            inp.k_ctx[o0:o1, 0, 512:] = ramp[:, None]
-        inp.k_new[:, 0, 512:] = 9.0
-        kg, _, _, _ = fill_caches_gpu(inp, device)
-        kc, _ = fill_caches_cpu(inp)
-        out, lse = _decode_gpu(inp, kg, device)
-        ref = oracle.aten_paged_decode(inp.q, kc, None, lay.block_table, lay.seq_lens, cfg.scale, dv=cfg.v_dim)
-        assert_close_to_reference(out, ref, cfg.name)
-        ref_lse = oracle.aten_paged_decode_lse(inp.q, kc, lay.block_table, lay.seq_lens, cfg.scale)
-        assert torch.allclose(lse.cpu(), ref_lse, rtol=1e-3, atol=1e-3)
+        _rising_scores_case(heads, lo, hi, bs, device)
+
+
+def test_other_kernels_for_more_than_64_heads(device):
+    # the default for more than 64 heads has 16 heads per wavefront and P.V by dim block; "wide" (four wavefronts
+    # of 512 registers, 32 heads each) and "heads" (16 heads per wavefront, both products by head block) stay
+    # selectable
+    for knob in ("wide", "heads"):
+        _select_kernel(knob)
+        try:
+            _check(_mla_cfg(f"mla128_{knob}", 3, 128, 100, 1500), 5, device)
+            _check(_mla_cfg(f"mla80_{knob}", 2, 80, 1, 400), 120, device)
+            _check(_mla_cfg(f"long_{knob}", 1, 128, 3000, 5000), 6, device)
+            _rising_scores_case(128, 1500, 2500, 64, device)
+        finally:
+            _select_kernel("")
 
 
 def test_producer_consumer_kernel(device):

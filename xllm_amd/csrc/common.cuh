@@ -29,6 +29,7 @@ __device__ __forceinline__ float as_f32(u32 u) { return __builtin_bit_cast(float
 // ---- 16-bit element traits -------------------------------------------------------------
 
 struct BF16 {
+  static constexpr bool kIsBf16 = true;
   // a.lo*b.lo + a.hi*b.hi + c with fp32 accumulation (v_dot2c_f32_bf16)
   static __device__ __forceinline__ float dot2(u32 a, u32 b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a),
@@ -53,6 +54,7 @@ struct BF16 {
 };
 
 struct FP16 {
+  static constexpr bool kIsBf16 = false;
   static __device__ __forceinline__ float dot2(u32 a, u32 b, float c) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
   }
@@ -161,11 +163,20 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 template <typename QT>
 struct Mfma;
+// wait states between an MFMA written as inline assembly and the first instruction that reads its result
+__device__ __forceinline__ void mfma_result_nops() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 template <>
 struct Mfma<BF16> {
   // v_mfma_f32_16x16x32_bf16: 8 elements of A and of B per lane
   static __device__ __forceinline__ f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  // The same with the accumulator in ordinary vector registers, whatever form the compiler picks for its own
+  // MFMAs (in a kernel with one wavefront per SIMD it puts every accumulator of the builtin into the 256
+  // accumulation registers, which a kernel may need in full for other products).  The compiler does not know
+  // this is an MFMA: the caller leaves kMfmaResultNops wait states before other instructions read the result.
+  static __device__ __forceinline__ void k32_v(u32x4 a, u32x4 b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
   // v_mfma_f32_16x16x16_bf16: 4 elements per lane
   static __device__ __forceinline__ f32x4 k16(s16x4 a, u32x2 b, f32x4 c) {
@@ -180,6 +191,9 @@ template <>
 struct Mfma<FP16> {
   static __device__ __forceinline__ f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ void k32_v(u32x4 a, u32x4 b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ f32x4 k16(s16x4 a, u32x2 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
