@@ -59,6 +59,21 @@ def test_fp16_and_other_head_dims(device):
         _check_config(cfg, 100 + D + Hq, device, dtype=dt)
 
 
+def test_head_dim_256_on_the_matrix_core_kernel(device):
+    # head dim 256 with a power-of-two block size >= 16: rows of 512 bytes, 8 tokens per stage in a 16-row score
+    # block whose upper half is masked.  Group sizes 1, 4, 16 and one that needs two head blocks; block sizes
+    # 16 / 64 / 128; contexts from one token to several workers' worth; lengths around the 8- and 16-token
+    # boundaries; fp16; a sliding window through the same entry.
+    for name, batch, Hq, Hkv, bs, lo, hi, dt in (("g1", 4, 4, 4, 32, 1, 700, torch.bfloat16),
+                                                 ("g4", 5, 16, 4, 16, 1, 3000, torch.bfloat16),
+                                                 ("g16", 3, 16, 1, 128, 100, 2500, torch.float16),
+                                                 ("g20", 3, 40, 2, 64, 50, 1200, torch.bfloat16),
+                                                 ("long", 3, 8, 2, 16, 10000, 20000, torch.bfloat16)):
+        _check_config(workloads.DecodeConfig(f"d256_{name}", batch, Hq, Hkv, 256, bs, lo, hi), 500 + Hq, device, dtype=dt)
+    for L in (1, 7, 8, 9, 15, 16, 17, 24, 33, 64, 65):
+        _check_config(workloads.DecodeConfig(f"d256_L{L}", 2, 8, 2, 256, 16, L, L), 600 + L, device)
+
+
 def test_head_dim_64_on_the_matrix_core_kernel(device):
     # head dim 64 with a power-of-two block size >= 16: rows of 128 bytes, 32 tokens per stage, two score blocks.
     # Group sizes that fill 1, 4 and all 16 columns and one that needs two head blocks; block sizes 16 / 64 / 128;

@@ -649,14 +649,15 @@ __device__ __forceinline__ void copy_cursor(CtxCursor& d, const CtxCursor& s) {
 
 constexpr int kMfmaThreads = 2 * kThreads;   // kWaves loading wavefronts and kWaves computing wavefronts
 
-template <int NS>
+template <int NS, int D = 128>
 struct MfmaLayout {
-  // LDS: ring [waves][NS][stage] | Q rows [waves][16][256 B] | page-table chunks [waves][3][64] |
+  // LDS: ring [waves][NS][stage] | Q rows [waves][16][kQRow B] | page-table chunks [waves][3][64] |
   //      scan scratch [kThreads] | progress counters [waves][2] | context lengths [kThreads] |
   //      stage prefix [batch + 1]
   static constexpr int kRingBytes = kWaves * NS * kStageBytes;
+  static constexpr int kQRow = D * 2 > 256 ? D * 2 : 256;
   static constexpr int kQOff = kRingBytes;
-  static constexpr int kPageOff = kQOff + kWaves * kMfmaHeads * 256;
+  static constexpr int kPageOff = kQOff + kWaves * kMfmaHeads * kQRow;
   static constexpr int kTmpOff = kPageOff + kWaves * 3 * kWave * 4;
   static constexpr int kSyncOff = kTmpOff + kThreads * 4;
   static constexpr int kLensOff = kSyncOff + 2 * kWaves * 4;   // context lengths of up to kThreads sequences
@@ -669,11 +670,14 @@ struct MfmaLayout {
 // ceil(tokens * group / 16) single tokens; column j is masked beyond its own length.
 // D = 64 (16-bit pages only): rows of 128 bytes, so a stage holds 32 tokens and is multiplied as two blocks
 // of 16 like an fp8 stage, with 2 k-steps per score block and 4 dim blocks.
+// D = 256 (16-bit pages only): rows of 512 bytes, a stage holds 8 tokens.  They take the first 8 rows of a
+// 16-token score block whose other rows repeat them under a mask (the matrix pipe has time to spare: a stage
+// is 8 KB of HBM traffic whatever the head dim), with 8 k-steps per score block and 16 dim blocks.
 template <typename QT, bool FP8, int NS, bool VL, int D>
 __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   static_assert(NS >= 2 && NS <= 4, "wait_younger_stages covers up to three stages in flight");
-  static_assert(D == 128 || (D == 64 && !FP8), "head dims of the matrix-core loop");
-  using Lay = MfmaLayout<NS>;
+  static_assert(D == 128 || ((D == 64 || D == 256) && !FP8), "head dims of the matrix-core loop");
+  using Lay = MfmaLayout<NS, D>;
   constexpr int G = kMfmaHeads;
   constexpr int KS = D / 32;               // k-steps of a score block
   constexpr int MB = D / 16;               // dim blocks of the output
@@ -763,8 +767,8 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   const char* ring = smem + pair * NS * kStageBytes;
   const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + pair * 3 * kWave * 4);
   const char* pagebuf = smem + Lay::kPageOff + pair * 3 * kWave * 4;
-  const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + pair * G * 256);
-  const char* qbuf = smem + Lay::kQOff + pair * G * 256;
+  const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + pair * G * Lay::kQRow);
+  const char* qbuf = smem + Lay::kQOff + pair * G * Lay::kQRow;
 
   auto locate = [&](int64_t f, CtxCursor& cu) {
     int lo = 0;
@@ -831,8 +835,11 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   const int q_read = c16 * (D * 2);  // Q rows (16-bit): + ((chunk ^ (c16 % QLPR)) * 16)
   // 16-bit pages.  K: row c16, + ((chunk ^ c16) * 16).  V: lane c16 of a 16-lane group addresses 4 dims
   // (8 bytes) of token row 4g + c16/4; + (v_y ^ (mb << 5)) selects dims 16 mb ..
-  const int k_read = c16 * RB;
-  const int v_read = T * RB + (4 * g + (c16 >> 2)) * RB + ((c16 & 3) >> 1) * 16 + (c16 & 1) * 8;
+  // (a stage of 8 tokens: rows 8 .. 15 of the score block and of the V^T operand repeat rows 0 .. 7)
+  constexpr int TR = T < 16 ? T : 16;      // distinct token rows of a 16-row block
+  const int k_row = c16 & (TR - 1);
+  const int k_read = k_row * RB;
+  const int v_read = T * RB + ((4 * g + (c16 >> 2)) & (TR - 1)) * RB + ((c16 & 3) >> 1) * 16 + (c16 & 1) * 8;
   const int v_y = (c16 >> 2) << 5;
   // fp8 pages.  K: rows c16 and 16 + c16, 8 bytes of chunk kk*2 + g/2.  V: lane c16 of a 16-lane group
   // addresses 8 dims (8 bytes) of the token in k-slot c16/2 of the group: tokens 4g .. 4g+3, then
@@ -924,7 +931,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     const int tok0 = (pc.st0 + pc.st) * T;
     const int lim = pc.L - tok0 - 1;  // last valid row of the stage
     // block size >= 16: a sub-block of 16 tokens lies in one page
-    constexpr int NSUB = T / 16;
+    constexpr int NSUB = T >= 16 ? T / 16 : 1;
     uint64_t kb[NSUB], vb[NSUB];
 #pragma unroll
     for (int sub = 0; sub < NSUB; ++sub) {
@@ -1088,29 +1095,33 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     }
 
     const char* st = ring + (s % NS) * kStageBytes;
-    if constexpr (!FP8 && T == 16) {
+    if constexpr (!FP8 && T <= 16) {
       // ---- all operand reads of the stage first: the latency of the V^T reads passes behind the score
       // MFMAs and the softmax (the scheduler would otherwise place them next to their use)
-      u32x4 kr[4];
+      u32x4 kr[KS];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) kr[kk] = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ c16) * 16));
-      s16x4 vt[8];
+      for (int kk = 0; kk < KS; ++kk) kr[kk] = *reinterpret_cast<const u32x4*>(st + k_read + (((kk * 4 + g) ^ k_row) * 16));
+      s16x4 vt[MB];
 #pragma unroll
-      for (int mb = 0; mb < 8; ++mb)
+      for (int mb = 0; mb < MB; ++mb)
         vt[mb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(st + v_read + (v_y ^ (mb << 5))));
       __builtin_amdgcn_sched_barrier(0);
-      // ---- scores of the stage's 16 tokens: lane (head c16, tokens 4g .. 4g+3); two chains of two MFMAs
+      // ---- scores of the stage's tokens: lane (head c16, tokens 4g .. 4g+3); two chains of KS / 2 MFMAs
       f32x4 sc = Mfma<QT>::k32(kr[0], q[0], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
       f32x4 sc1 = Mfma<QT>::k32(kr[1], q[1], f32x4{0.0f, 0.0f, 0.0f, 0.0f});
-      sc = Mfma<QT>::k32(kr[2], q[2], sc);
-      sc1 = Mfma<QT>::k32(kr[3], q[3], sc1);
+#pragma unroll
+      for (int kk = 2; kk < KS; kk += 2) {
+        sc = Mfma<QT>::k32(kr[kk], q[kk], sc);
+        sc1 = Mfma<QT>::k32(kr[kk + 1], q[kk + 1], sc1);
+      }
       sc += sc1;
       const int tok0 = (cc.st0 + cc.st) * T + 4 * g;
       float sv[4];
       bool over = false;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        sv[r] = tok0 + r < Lc && tok0 + r >= Lo ? sc[r] * score_scale : -INFINITY;
+        const bool in_stage = T >= 16 || 4 * g + r < T;   // (rows past a short stage repeat its tokens)
+        sv[r] = in_stage && tok0 + r < Lc && tok0 + r >= Lo ? sc[r] * score_scale : -INFINITY;
         over |= sv[r] > m + kSlack;
       }
       if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
@@ -1133,7 +1144,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       // ---- O^T += V^T . P^T: lane c16 of a 16-lane group supplies the address of 4 dims of token
       // row 4g + c16/4 and receives the 4 tokens of dim column 16 mb + c16
 #pragma unroll
-      for (int mb = 0; mb < 8; ++mb) o[mb] = Mfma<QT>::k16(vt[mb], pb, o[mb]);
+      for (int mb = 0; mb < MB; ++mb) o[mb] = Mfma<QT>::k16(vt[mb], pb, o[mb]);
     } else if constexpr (!FP8) {
       // ---- 16-bit pages with 32 tokens per stage (head dim 64): two score blocks of 16 tokens,
       // lane (head c16, tokens 16 tb + 4g ..), then all 32 tokens in one P.V MFMA per dim block
@@ -1444,8 +1455,11 @@ constexpr int kMfmaStages = 4;
 
 template <typename QT, bool FP8, bool VL = false, int D = 128>
 int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
-  using Lay = MfmaLayout<kMfmaStages>;
-  auto kern = gqa_mfma_kernel<QT, FP8, kMfmaStages, VL, D>;
+  // (head dim 256: the Q rows of the four pairs take 32 KB of the LDS, which leaves room for three stages each)
+  constexpr int NS = D == 256 ? kMfmaStages - 1 : kMfmaStages;
+  using Lay = MfmaLayout<NS, D>;
+  static_assert(Lay::kPrefixOff + (kMaxBatch + 1) * 4 <= 160 * 1024, "LDS of a CU");
+  auto kern = gqa_mfma_kernel<QT, FP8, NS, VL, D>;
   static std::atomic<uint64_t> configured{0};
   if (first_use_on_current_device(configured)) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1507,6 +1521,8 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
       return launch_gqa_mfma<QT, false>(a, wsb, s, plan_only, need);
     if (head_dim == 64 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
       return launch_gqa_mfma<QT, false, false, 64>(a, wsb, s, plan_only, need);
+    if (head_dim == 256 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
+      return launch_gqa_mfma<QT, false, false, 256>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, false, 64, 8, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, false, 128, 16, 4>(a, wsb, s, plan_only, need);
