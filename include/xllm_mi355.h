@@ -178,7 +178,7 @@ int xllm_mi355_paged_decode_gqa(const void* q, const void* k_cache, const void* 
  * at zero except the status word, which only xllm_mi355_decode_status(NULL, stream) clears.  The first call on
  * a device looks the scratch address up (hipGetSymbolAddress): make it outside graph capture.
  */
-#define XLLM_MI355_STATIC_SCRATCH_BYTES (20u << 20)
+#define XLLM_MI355_STATIC_SCRATCH_BYTES (36u << 20)
 int xllm_mi355_paged_decode_gqa_static(const void* q, const void* k_cache, const void* v_cache,
                                        void* out, float* lse,
                                        const int32_t* block_table, int64_t table_stride,
@@ -425,9 +425,11 @@ int xllm_mi355_profile_collect(float* ms_out, int max_n);
  * at xllm_mi355_decode_status (negative = default, 2^22; 0 makes the first wait of a launch give up, which is
  * how the status path is tested: every wavefront still exits normally).  XLLM_MI355_DEBUG_MLA_KERNEL: the MLA
  * kernel choice, as the first letter of the environment variable XLLM_MI355_MLA_KERNEL, which the library reads
- * once per process (0 default, 'p' pairs, 's' split).
+ * once per process (0 default, 'p' pairs, 's' split, 'h' heads, 'w' wide).  XLLM_MI355_DEBUG_GQA_FOLD: 1 makes
+ * the matrix-core GQA kernel merge the partial results itself instead of leaving them to a second launch (same
+ * as XLLM_MI355_GQA_FOLD=1 in the environment; off by default because it measures slower).
  */
-enum { XLLM_MI355_DEBUG_WAIT_SPINS = 0, XLLM_MI355_DEBUG_MLA_KERNEL = 1 };
+enum { XLLM_MI355_DEBUG_WAIT_SPINS = 0, XLLM_MI355_DEBUG_MLA_KERNEL = 1, XLLM_MI355_DEBUG_GQA_FOLD = 2 };
 int xllm_mi355_debug_set(int what, int value);
 
 /*

@@ -74,6 +74,36 @@ def test_head_dim_256_on_the_matrix_core_kernel(device):
         _check_config(workloads.DecodeConfig(f"d256_L{L}", 2, 8, 2, 256, 16, L, L), 600 + L, device)
 
 
+def test_merge_inside_the_decode_kernel(device):
+    # the opt-in path where the worker that brings a context's last piece merges the partials (no merge launch):
+    # contexts that span many workers, short ones that no worker splits, empty sequences, LSE, fp8, head dim 256,
+    # and twice in a row on the same workspace (the arrival counters return to zero by themselves)
+    from xllm_amd import capi
+    lib = capi.lib()
+    assert lib.xllm_mi355_debug_set(2, 1) == 0
+    try:
+        for rep in range(2):
+            _check_config(workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=8), 2024 + rep, device)
+            _check_config(workloads.DecodeConfig("fold_long", 2, 8, 2, 128, 16, 20000, 30000), 11 + rep, device)
+            _check_config(workloads.DecodeConfig("fold_short", 300, 8, 2, 128, 16, 1, 40), 12 + rep, device)
+            _check_config(workloads.DecodeConfig("fold_d256", 3, 8, 2, 256, 16, 500, 6000), 13 + rep, device)
+            _check_fp8(workloads.DecodeConfig("fold_fp8", 4, 32, 8, 128, 16, 300, 5000, cache_dtype="fp8"), 14 + rep, device)
+        cfg = workloads.DecodeConfig("fold_empty", 5, 8, 2, 128, 16, 100, 3000)
+        inp = workloads.make_inputs(cfg, 15)
+        inp.layout.seq_lens[1] = 0
+        inp.layout.seq_lens[4] = 0
+        kg, vg, _, _ = fill_caches_gpu(inp, device)
+        out, lse = _decode_gpu(inp, kg, vg, device)
+        lay = inp.layout
+        keep = torch.tensor([0, 2, 3])
+        ref = oracle.aten_paged_decode(inp.q[keep], kg.cpu(), vg.cpu(), lay.block_table[keep], lay.seq_lens[keep], cfg.scale)
+        assert_close_to_reference(out[keep.to(out.device)], ref, cfg.name)
+        assert torch.all(out[1] == 0) and torch.all(out[4] == 0) and torch.all(torch.isneginf(lse[1])) and torch.all(torch.isneginf(lse[4]))
+        assert ops.decode_status(device) == 0
+    finally:
+        assert lib.xllm_mi355_debug_set(2, 0) == 0
+
+
 def test_head_dim_64_on_the_matrix_core_kernel(device):
     # head dim 64 with a power-of-two block size >= 16: rows of 128 bytes, 32 tokens per stage, two score blocks.
     # Group sizes that fill 1, 4 and all 16 columns and one that needs two head blocks; block sizes 16 / 64 / 128;

@@ -12,6 +12,7 @@ std::atomic<int> g_wait_spins{kDefaultWaitSpins};
 }  // namespace
 int wait_spin_limit() { return g_wait_spins.load(std::memory_order_relaxed); }
 void set_mla_kernel_knob(int first_letter);  // paged_decode_mla.hip
+void set_fold_merge(int on);                 // paged_decode_gqa.hip
 }  // namespace xllm_mi355
 
 // Scratch of xllm_mi355_paged_decode_gqa_static: a decode workspace that lives in the code object, one copy
@@ -105,9 +106,10 @@ int xllm_mi355_decode_status(void* workspace, void* stream) {
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   if (e != hipSuccess) return static_cast<int>(e);
   if (status == 0) return XLLM_MI355_OK;
-  const int zero = 0;
-  e = hipMemcpyAsync(workspace, &zero, sizeof(int), hipMemcpyHostToDevice, s);
-  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  // the launch that gave up may also have left arrival counters behind: the whole header starts over
+  const int rc = decode_workspace_init(workspace, kWsHeaderBytes, s);
+  if (rc != 0) return rc;
+  e = hipStreamSynchronize(s);
   if (e != hipSuccess) return static_cast<int>(e);
   return XLLM_MI355_ESTALLED;
 }
@@ -119,6 +121,9 @@ int xllm_mi355_debug_set(int what, int value) {
       return XLLM_MI355_OK;
     case XLLM_MI355_DEBUG_MLA_KERNEL:
       set_mla_kernel_knob(value);
+      return XLLM_MI355_OK;
+    case XLLM_MI355_DEBUG_GQA_FOLD:
+      set_fold_merge(value);
       return XLLM_MI355_OK;
     default: return XLLM_MI355_EINVAL;
   }

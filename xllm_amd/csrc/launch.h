@@ -42,11 +42,14 @@ struct PageAddressing {
 
 // Layout of a decode workspace, the same for every decode entry point and independent of the batch, so that
 // a launch recorded in a HIP graph keeps meaning the same addresses whatever later calls ask for:
-//   [0, kWsHeaderBytes)                 header: word 0 = status flags (kStatus*), the rest reserved
+//   [0, kWsHeaderBytes)                 header: word 0 = status flags (kStatus*); from byte kWsCountersOff on,
+//                                       one arrival counter per persistent worker (zero between launches)
 //   [kWsHeaderBytes, kWsPartialsOff)    item prefix of up to kWsMaxBatch sequences per launch
 //   [kWsPartialsOff, ...)               two fp32 partial slots per persistent worker
-//   the last varlen_extra_bytes(n)      per-token lengths and table rows of the varlen entry point
-constexpr size_t kWsHeaderBytes = 256;
+// (xllm_mi355_decode_workspace_init clears the header.)
+constexpr size_t kWsCountersOff = 256;
+constexpr int kWsMaxWorkers = 4096;
+constexpr size_t kWsHeaderBytes = kWsCountersOff + static_cast<size_t>(kWsMaxWorkers) * 4;
 constexpr int kWsMaxBatch = 2048;
 constexpr size_t kWsPartialsOff = kWsHeaderBytes + (static_cast<size_t>(kWsMaxBatch + 1) * 4 + 255) / 256 * 256;
 constexpr int kStatusWaitGaveUp = 1;  // a bounded wait of one wavefront on another ran out: the launch's output is invalid
@@ -147,6 +150,9 @@ inline bool first_use_on_current_device(std::atomic<uint64_t>& seen) {
 // would also count the 2-3 us each that their own packets take, 5 % of a 100 us kernel.
 bool profile_events(hipEvent_t* start, hipEvent_t* stop);
 void profile_commit();
+// A launch that a caller of xllm_mi355_profile_collect counts on did not take place (its work was done by the
+// launch before): recorded as an entry of 0 ms.
+void profile_skip();
 
 template <typename Kernel, typename... Args>
 inline void launch_timed(Kernel kernel, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, Args... args) {

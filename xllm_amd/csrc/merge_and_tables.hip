@@ -243,15 +243,15 @@ int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t tab
 }
 
 namespace {
-__global__ __launch_bounds__(64) void clear_words_kernel(int* p, int n) {
-  if (static_cast<int>(threadIdx.x) < n) p[threadIdx.x] = 0;
+__global__ __launch_bounds__(256) void clear_words_kernel(int* p, int n) {
+  for (int i = threadIdx.x; i < n; i += 256) p[i] = 0;
 }
 }  // namespace
 
 int decode_workspace_init(void* workspace, size_t workspace_bytes, hipStream_t stream) {
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 || workspace_bytes < kWsHeaderBytes)
     return XLLM_MI355_EWORKSPACE;
-  clear_words_kernel<<<dim3(1), 64, 0, stream>>>(static_cast<int*>(workspace), static_cast<int>(kWsHeaderBytes / 4));
+  clear_words_kernel<<<dim3(1), 256, 0, stream>>>(static_cast<int*>(workspace), static_cast<int>(kWsHeaderBytes / 4));
   return static_cast<int>(hipGetLastError());
 }
 

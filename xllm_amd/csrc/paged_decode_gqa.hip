@@ -71,6 +71,8 @@ struct GqaArgs {
   const float* k_scale;
   const float* v_scale;
   int* ws_status;  // status flags of the workspace (kStatus*), only ever OR-ed into
+  unsigned* ws_arrivals;  // one counter per worker (zero between launches): pieces of the context that starts in its range
+  int fold_merge;  // the matrix-core kernel merges a context's partials itself (last piece to arrive) and writes empty rows
   int* ws_prefix;  // [batch + 1] item prefix, written by workgroup 0 for the merge kernel
   float* ws_out;   // [2 * n_workgroups][G][D]
   float* ws_lse;   // [2 * n_workgroups][G]
@@ -649,6 +651,19 @@ __device__ __forceinline__ void copy_cursor(CtxCursor& d, const CtxCursor& s) {
 
 constexpr int kMfmaThreads = 2 * kThreads;   // kWaves loading wavefronts and kWaves computing wavefronts
 
+template <typename QT, bool VL, bool COHERENT = false>
+__device__ __forceinline__ void merge_context(const GqaArgs& a, int dv, int hbk, int b, int tid, int nthreads,
+                                              int p0, int p1, int pt);
+// Words of the partials that workers exchange inside one launch: relaxed atomics at device scope, which go to
+// the level of the memory system that all CUs share (the L2 of an XCD is not coherent with the other seven; a
+// fence that makes it so writes back and invalidates the whole L2, 60 us per launch when 1024 workers do it).
+__device__ __forceinline__ void store_shared(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_shared(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int NS, int D = 128>
 struct MfmaLayout {
   // LDS: ring [waves][NS][stage] | Q rows [waves][16][kQRow B] | page-table chunks [waves][3][64] |
@@ -688,6 +703,9 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   constexpr int LPR = RB / 16;             // lanes (16-byte chunks) per row in a load instruction
   constexpr int RPI = kWave / LPR;         // rows per load instruction
 
+#ifdef XLLM_GQA_TIMING
+  const unsigned long long t_entry = wall_clock64();
+#endif
   extern __shared__ __align__(16) char smem[];
   int* tmp = reinterpret_cast<int*>(smem + Lay::kTmpOff);
   int* prefix = reinterpret_cast<int*>(smem + Lay::kPrefixOff);
@@ -749,6 +767,13 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       sequence_of_scalar(a, b, pages, L);
     }
   };
+  if constexpr (!VL) {
+    if (a.fold_merge != 0) {  // rows of empty sequences (no item, so no worker ever meets them)
+      for (int b = blockIdx.x; b < a.batch; b += gridDim.x)
+        if (prefix[b + 1] == prefix[b])
+          for (int hbk = 0; hbk < n_hb; ++hbk) merge_context<QT, false>(a, D, hbk, b, tid, kMfmaThreads, 0, 0, 0);
+    }
+  }
   if (total == 0) return;
   // ---- from here on the pairs are independent: no workgroup barrier below this line
   const bool loader = wave < kWaves;   // wavefronts 0 .. kWaves - 1 load, wavefront kWaves + w computes what w loads
@@ -1016,6 +1041,10 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   }  // loader
 
   // ---- the computing wavefront
+#ifdef XLLM_GQA_TIMING   // (measurement build only) wall-clock stamps of every worker, behind the partials
+  const unsigned long long t_compute = wall_clock64();
+  unsigned long long t_first = 0;
+#endif
   CtxCursor cc;
   locate(cur, cc);
   bool run_start = true;
@@ -1026,6 +1055,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   int Lo = 0;                 // first token it attends to (0 without a sliding window)
   int64_t out_off = 0;        // VL: byte offset of the lane's output row
   int c_ctx_first = 0, c_prev_len = 0;
+  int n_pend = 0, pend_b0 = 0, pend_h0 = 0, pend_b1 = 0, pend_h1 = 0;  // pieces of contexts this worker left as partials
   u32x4 q[KS];
   f32x4 o[MB];
   float m = kNegBig, l = 0.0f;
@@ -1043,6 +1073,9 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       __builtin_amdgcn_s_sleep(1);
     }
     asm volatile("" ::: "memory");  // no read of the stage moves above the poll
+#ifdef XLLM_GQA_TIMING
+    if (s == 0) t_first = wall_clock64();
+#endif
 
     if (run_start) {  // first stage of a run: the (sequence, head block) changes
       run_start = false;
@@ -1278,7 +1311,8 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
           *reinterpret_cast<u32x2*>(op + mb * 32) = w;
         }
       }
-      if (head_on && !complete) {
+      const bool shared = !VL && a.fold_merge != 0;  // another worker of this launch reads the partial
+      if (head_on && !complete && !shared) {
         float* wp = a.ws_out + pidx * D + 4 * g;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
@@ -1286,8 +1320,28 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
           *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
         }
       }
+      if (head_on && !complete && shared) {
+        float* wp = a.ws_out + pidx * D + 4 * g;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) store_shared(wp + mb * 16 + r, o[mb][r] * inv);
+      }
       if (!VL && head_on && g == 0 && complete && a.lse != nullptr) a.lse[cc.b * a.n_q_heads + hq] = lse2 * kLn2;
-      if (head_on && g == 0 && !complete) a.ws_lse[pidx] = lse2;
+      if (head_on && g == 0 && !complete && !shared) a.ws_lse[pidx] = lse2;
+      if (head_on && g == 0 && !complete && shared) store_shared(a.ws_lse + pidx, lse2);
+      if constexpr (!VL) {
+        if (!complete) {  // (only the first and the last run of a range can be pieces)
+          if (n_pend == 0) {
+            pend_b0 = cc.b;
+            pend_h0 = cc.hbk;
+          } else {
+            pend_b1 = cc.b;
+            pend_h1 = cc.hbk;
+          }
+          ++n_pend;
+        }
+      }
       first_run = false;
     }
     // The operand reads of the stage have returned (the MFMAs that take them have been issued) and LDS
@@ -1302,6 +1356,43 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef XLLM_GQA_TIMING
+  if (lane == 0) {
+    unsigned long long* dst = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_workgroups) * 2 * G) + worker * 4;
+    dst[0] = t_entry;
+    dst[1] = t_compute;
+    dst[2] = t_first;
+    dst[3] = wall_clock64();
+  }
+#endif
+  // ---- the pieces this worker wrote as partials: the worker that brings a context's last piece merges them.
+  // One counter per context that spans workers, kept with the worker in whose range it starts (at most one
+  // such context per worker); atomicInc wraps it back to zero with the last arrival.  The partials were
+  // stored with store_shared and those stores have completed (the wait above), so the worker that sees the
+  // last arrival finds all of them with load_shared.
+  if constexpr (!VL) {
+    if (a.fold_merge != 0 && n_pend > 0) {
+      for (int i = 0; i < n_pend; ++i) {
+        const int b = i == 0 ? pend_b0 : pend_b1, hbk = i == 0 ? pend_h0 : pend_h1;
+        const int p0 = prefix[b], p1 = prefix[b + 1];
+        const int n_items = p1 - p0;
+        const int64_t first = static_cast<int64_t>(p0) * n_hb + static_cast<int64_t>(hbk) * n_items;
+        const int64_t last = first + n_items - 1;
+        const int w_first = workgroup_of(first, total, n_workers), w_last = workgroup_of(last, total, n_workers);
+        int pieces = 0;  // workers of w_first .. w_last whose range is not empty
+        for (int w0 = w_first; w0 <= w_last; w0 += kWave) {
+          const int w = w0 + lane;
+          const bool on = w <= w_last && range_start(w + 1, total, n_workers) > range_start(w, total, n_workers);
+          pieces += __builtin_popcountll(__builtin_amdgcn_ballot_w64(on));
+        }
+        unsigned old = 0;
+        if (lane == 0) old = atomicInc(a.ws_arrivals + w_first, static_cast<unsigned>(pieces - 1));
+        old = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(old)));
+        if (static_cast<int>(old) == pieces - 1)
+          merge_context<QT, false, true>(a, D, hbk, b, lane, kWave, p0, p1, prefix[a.batch]);
+      }
+    }
+  }
 }
 
 // Merge of the partials of contexts that span several workers (workgroups of the dot-product
@@ -1312,13 +1403,13 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
 // prefix, then the LSEs and accumulators of four consecutive workers at a time, all loads of a
 // group issued together.
 // VL: the columns of a partial are (query token, head) pairs of the sequence's chunk (see gqa_mfma_kernel).
-template <typename QT, bool VL>
-__global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int dv) {
-  const int hbk = blockIdx.x;
-  const int b = blockIdx.y;
-  const int tid = threadIdx.x;
+// The merge of one (head block hbk, sequence b) by `nthreads` threads (this one is `tid`); p0, p1, pt = item
+// prefix of the sequence, of the next one, and the batch total.  COHERENT: the partials were written by
+// other workers of the same launch (store_shared) and are read the same way.
+template <typename QT, bool VL, bool COHERENT>
+__device__ __forceinline__ void merge_context(const GqaArgs& a, int dv, int hbk, int b, int tid, int nthreads,
+                                              int p0, int p1, int pt) {
   const int G = a.g_block;
-  const int p0 = a.ws_prefix[b], p1 = a.ws_prefix[b + 1], pt = a.ws_prefix[a.batch];
   const int hb_per_kv = VL ? a.chunk_blocks : (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
   const int kvh = hbk / hb_per_kv;
@@ -1356,7 +1447,7 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
   };
   const int n_items = p1 - p0;
   if (n_items <= 0) {  // empty sequence
-    for (int v = tid; v < n_vec; v += kThreads) {
+    for (int v = tid; v < n_vec; v += nthreads) {
       store4(v / dv4, (v % dv4) * 4, 0.0f, 0.0f, 0.0f, 0.0f);
       if (!VL && a.lse != nullptr && v % dv4 == 0) a.lse[b * a.n_q_heads + h0 + v / dv4] = -INFINITY;
     }
@@ -1376,7 +1467,7 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
   // the first worker holds this context as its last run (slot 1) unless its range starts
   // exactly here; every later one holds it as its first run (slot 0)
   const int slot_first = range_start(w_first, total, n) < first ? 1 : 0;
-  for (int v = tid; v < n_vec; v += kThreads) {
+  for (int v = tid; v < n_vec; v += nthreads) {
     const int h = v / dv4, d = (v - h * dv4) * 4;
     int64_t acc = acc0;
     float M = kNegBig, W = 0.0f;
@@ -1394,8 +1485,15 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
         // with fewer items than workers some ranges in between are empty and own no partial
         on[k] = w <= w_last && step > 0;
         const int64_t ps = (static_cast<int64_t>(w) * 2 + (w == w_first ? slot_first : 0)) * G + h;
-        lse[k] = on[k] ? a.ws_lse[ps] : kNegBig;
-        x[k] = on[k] ? *reinterpret_cast<const f32x4*>(a.ws_out + ps * dv + d) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (COHERENT) {
+          const float* xp = a.ws_out + ps * dv + d;
+          lse[k] = on[k] ? load_shared(a.ws_lse + ps) : kNegBig;
+          x[k] = on[k] ? f32x4{load_shared(xp), load_shared(xp + 1), load_shared(xp + 2), load_shared(xp + 3)}
+                       : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        } else {
+          lse[k] = on[k] ? a.ws_lse[ps] : kNegBig;
+          x[k] = on[k] ? *reinterpret_cast<const f32x4*>(a.ws_out + ps * dv + d) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
       }
       const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
       const float keep = fast_exp2(M - m_new);
@@ -1413,6 +1511,13 @@ __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int
     store4(h, d, O[0] * inv, O[1] * inv, O[2] * inv, O[3] * inv);
     if (!VL && a.lse != nullptr && d == 0) a.lse[b * a.n_q_heads + h0 + h] = (M + fast_log2(W)) * kLn2;
   }
+}
+
+template <typename QT, bool VL>
+__global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int dv) {
+  const int b = blockIdx.y;
+  merge_context<QT, VL>(a, dv, blockIdx.x, b, threadIdx.x, kThreads, a.ws_prefix[b], a.ws_prefix[b + 1],
+                        a.ws_prefix[a.batch]);
 }
 
 int device_cu_count() {
@@ -1453,6 +1558,23 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
 
 constexpr int kMfmaStages = 4;
 
+// Whether the matrix-core kernel merges the partials itself: the worker that brings a context's last piece
+// reads the others' partials and writes the output, and no merge kernel is launched.  Off by default: the
+// exchange inside one launch has to go through the memory level that all XCDs share (store_shared /
+// load_shared), and its chain of three round trips at the tail of the launch costs more (about 12 us on the
+// 64-sequence configuration) than the separate merge launch it saves (4.5 us).  "1" in XLLM_MI355_GQA_FOLD, read
+// once per process, or set_fold_merge (test hook) turn it on.
+std::atomic<int> g_fold_merge{-1};
+bool fold_merge_enabled() {
+  int v = g_fold_merge.load(std::memory_order_relaxed);
+  if (v < 0) {
+    const char* e = getenv("XLLM_MI355_GQA_FOLD");  // tuning knob
+    v = e != nullptr && e[0] == '1' ? 1 : 0;
+    g_fold_merge.store(v, std::memory_order_relaxed);
+  }
+  return v != 0;
+}
+
 template <typename QT, bool FP8, bool VL = false, int D = 128>
 int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
   // (head dim 256: the Q rows of the four pairs take 32 KB of the LDS, which leaves room for three stages each)
@@ -1476,6 +1598,8 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
   a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_status) + kWsPartialsOff);
   a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
+  a.ws_arrivals = reinterpret_cast<unsigned*>(reinterpret_cast<char*>(a.ws_status) + kWsCountersOff);
+  a.fold_merge = !VL && a.n_workgroups <= kWsMaxWorkers && fold_merge_enabled() ? 1 : 0;
   const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 1) * 4;
   launch_timed(kern, dim3(static_cast<unsigned>(n_wg)), dim3(kMfmaThreads), smem, stream, a);
   return static_cast<int>(hipGetLastError());
@@ -1540,6 +1664,8 @@ int group_block(int group) {
 }
 
 }  // namespace
+
+void set_fold_merge(int on) { g_fold_merge.store(on != 0 ? 1 : 0, std::memory_order_relaxed); }
 
 size_t gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim) {
   // Upper bound over every kernel variant, independent of the batch: at most 8 workgroups per CU, 8 heads
@@ -1657,6 +1783,10 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
       rc = fp8 ? dispatch_dim<FP16, true>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need)
                : dispatch_dim<FP16, false>(a, static_cast<int>(head_dim), workspace_bytes, stream, false, &need);
     if (rc != 0) return rc;
+    if (a.fold_merge != 0) {  // the decode kernel merged
+      profile_skip();
+      continue;
+    }
     const int hb_per_kv = (group + a.g_block - 1) / a.g_block;
     dim3 grid(static_cast<unsigned>(n_kv_heads * hb_per_kv), static_cast<unsigned>(nb));
     if (q_dtype == XLLM_MI355_BF16)
