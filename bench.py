@@ -47,6 +47,9 @@ def parse_args():
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run only the plain stream_read / stream_copy kernels over 1 GiB (counter calibration)")
+    ap.add_argument("--neighbours", action="store_true",
+                    help="time the ops on either side of the decode (reshape_and_cache, fused norm + rope + cache write, "
+                         "the absorbed-weight batched matmuls of MLA, the gather of paged rows) and print their line")
     ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "traffic.json"),
                     help="measured HBM bytes per launch by workload (written from rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -167,6 +170,74 @@ def calibrate(lib, capi, torch, dev):
     copy_gbs, copy_ms = stream_rate(lib, capi, torch, dev, nbytes, copy=True)
     return {"bytes": nbytes, "stream_read_gbs": read_gbs, "stream_read_ms": read_ms,
             "stream_copy_gbs_read_plus_write": copy_gbs, "stream_copy_ms": copy_ms}
+
+
+def neighbours(ops, workloads, torch, dev, steps):
+    """The ops that feed the decode and take its result, at the shapes of the benchmark configurations: every one is
+    HBM-bound integer / byte movement or a skinny batched matmul, so each is priced by its algorithmic bytes."""
+    import math
+    g = torch.Generator().manual_seed(0)
+
+    def timed(fn):
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps * 1e3
+
+    rows = []
+
+    def row(op, kernel, shape, us, nbytes):
+        rows.append({"op": op, "kernel": kernel, "shape": shape, "us": us, "algorithmic_bytes": nbytes,
+                     "gbs": nbytes / us / 1e3, "frac_of_hbm_peak": nbytes / us / 1e3 / HBM_PEAK_GBS})
+
+    # reshape_and_cache: a prefill chunk of 8192 tokens into bf16 pages (configuration 2's heads), read + write
+    T, nk, D = 8192, 8, 128
+    k = torch.randn(T, nk, D, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(T, nk, D, generator=g).to(torch.bfloat16).to(dev)
+    P = T // 16 + 8
+    kc = torch.zeros(P, 16, nk, D, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    slots = torch.randperm(P * 16, generator=g)[:T].to(torch.int32).to(dev)
+    prm = ops.ReshapePagedCacheParams(key=k, value=v, k_cache=kc, v_cache=vc, slot_mapping=slots)
+    row("reshape_and_cache", "reshape_vec_kernel", f"{T} tokens x {nk} KV heads x {D}, bf16 pages of 16",
+        timed(lambda: ops.reshape_paged_cache(prm)), workloads.reshape_bytes(T, nk * D, 2, 2, 2))
+    # fused q/k norm + rope + cache write of the same chunk: reads q, k, v once, writes q, k and the two cache rows
+    nq = 32
+    qkv = (torch.randn(T, (nq + 2 * nk) * D, generator=g) * 0.3).to(torch.bfloat16).to(dev)
+    qw = torch.ones(D, dtype=torch.bfloat16, device=dev)
+    ang = torch.rand(4096, D // 2, generator=g) * 6.28
+    cs = torch.cat([ang.cos(), ang.sin()], 1).to(dev)
+    pos = torch.randint(0, 4096, (T,), generator=g).to(dev)
+    row("fused_qk_norm_rope + cache write", "rope_and_cache_kernel", f"{T} tokens, {nq}/{nk} heads x {D}",
+        timed(lambda: ops.fused_qk_norm_rope(qkv, nq, nk, nk, D, 1e-6, qw, qw, cs, False, pos, k_cache=kc, v_cache=vc,
+                                             slot_mapping=slots)),
+        T * (nq + nk) * D * 2 * 2 + T * 2 * nk * D * 2 * 2)
+    # the two absorbed-weight matmuls around the MLA decode of configuration 5 (64 tokens, 128 heads)
+    for K, N in ((128, 512), (512, 128)):
+        H, Tq = 128, 64
+        x = torch.randn(Tq, H, K, generator=g).to(torch.bfloat16).to(dev)
+        w = (torch.randn(H, K, N, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(dev)
+        out = torch.empty(Tq, H, N, dtype=torch.bfloat16, device=dev)
+        row("absorbed_bmm", "absorbed_bmm_kernel", f"{Tq} tokens x {H} heads, [{K}] x [{K}, {N}]",
+            timed(lambda: ops.absorbed_bmm(x, w, out=out)), H * K * N * 2 + Tq * H * (K + N) * 2)
+    # gather of the paged latent rows of configuration 5 into a packed tensor (chunked prefill reads it)
+    cfg = workloads.CONFIGS["mla_dsv3"]
+    lay = workloads.make_layout(cfg, 1)
+    lat = torch.randn(lay.num_blocks, cfg.block_size, 1, 576, generator=g).to(torch.bfloat16).to(dev)
+    cu = torch.zeros(cfg.batch + 1, dtype=torch.int32)
+    cu[1:] = lay.seq_lens.cumsum(0)
+    total = int(cu[-1])
+    tab, cu = lay.block_table.to(dev), cu.to(dev)
+    row("gather_mla_latent_cache", "gather_paged_rows_kernel", f"{total} rows of 1152 bytes from pages of {cfg.block_size}",
+        timed(lambda: ops.gather_mla_latent_cache(lat, tab, cu, total)), 2 * total * 1152)
+    return {"neighbour_ops": rows, "steps": steps, "peak_gbs": HBM_PEAK_GBS,
+            "note": "torch events around the loop of calls (launch gaps included)"}
 
 
 def decode_kernel_name(cfg):
@@ -363,6 +434,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.calibrate:
         print(json.dumps(calibrate(lib, capi, torch, dev)))
+        return
+    if args.neighbours:
+        print(json.dumps(neighbours(ops, workloads, torch, dev, max(args.steps, 1))))
         return
     run = lambda name, budget: run_workload(name, args, lib, capi, ops, workloads, torch, dev, budget)
     if args.workload != "all":
