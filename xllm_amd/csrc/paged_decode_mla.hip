@@ -1547,32 +1547,41 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       int last;        // rows of the context after that one
       u32 dst, dst_rope;
     };
-    auto issue_prepare = [&](int sub) -> Send {
-      const int tok0 = t_begin + sub * kSubTok + wave * 8;   // block_size >= 16: the 8 rows share a page
-      const u32 slot = lds_base + (sub % kDsRing) * kSubBytes;
-      Send sd;
-      sd.dst = __builtin_amdgcn_readfirstlane(slot + wave * 8 * kRow16);
-      sd.dst_rope = __builtin_amdgcn_readfirstlane(slot + kRope16Off + wave * 8 * (kDR * 2));
-      const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
-      const int tb = min(tok0, L - 1);
+    // (filled field by field: a struct that is copied as a whole goes through scratch memory, whose loads count
+    // on the same counter as the tile loads in flight)
+    // in two steps, so that the trip to LDS for the page id passes behind other work: the read ...
+    auto issue_prepare_read = [&](int sub) -> int {
+      const int tb = min(t_begin + sub * kSubTok + wave * 8, L - 1);   // block_size >= 16: the 8 rows share a page
       const int ck = (tb >> a.bs_shift) >> 6;
       if (ck != ck_cur) {
         ck_cur = ck;
         if (wave == 0 && (ck + 1) * kWave < n_pages) issue_chunk(ck + 1);
       }
-      int page = __builtin_amdgcn_readfirstlane(pagebuf[(ck & 1) * kWave + ((tb >> a.bs_shift) & 63)]);
+      return pagebuf[(ck & 1) * kWave + ((tb >> a.bs_shift) & 63)];
+    };
+    // ... and the addresses
+    auto issue_prepare_finish = [&](int sub, int page_read, Send& sd) {
+      const int tb = min(t_begin + sub * kSubTok + wave * 8, L - 1);
+      const u32 slot = lds_base + (sub % kDsRing) * kSubBytes;
+      sd.dst = __builtin_amdgcn_readfirstlane(slot + wave * 8 * kRow16);
+      sd.dst_rope = __builtin_amdgcn_readfirstlane(slot + kRope16Off + wave * 8 * (kDR * 2));
+      const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
+      int page = __builtin_amdgcn_readfirstlane(page_read);
       page = max(0, min(page, a.num_blocks - 1));
+#ifdef XLLM_W4_WHATIF_ONE_PAGE   // (measurement only: wrong results) every tile from the same pages: the loads hit in L2
+      page = page & 7;
+#endif
       const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tb & (a.block_size - 1))) * kRowBytes;
       const u32 rlo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row)));
       const u32 rhi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row >> 32)));
       sd.sb = (static_cast<uint64_t>(rhi) << 32) | rlo;
       sd.last = __builtin_amdgcn_readfirstlane(L - 1 - tb);
-      return sd;
     };
-    // 16-byte chunks of a latent row are XOR-ed with bit 2 of the row: rows 4-7 of the eight swap chunk pairs
+    auto issue_prepare = [&](int sub, Send& sd) { issue_prepare_finish(sub, issue_prepare_read(sub), sd); };
+    // (the row's distance from the first one rides in the per-lane offset: one vector add instead of five
+    // scalar instructions for a 64-bit base)
     auto issue_row = [&](const Send& sd, int i) {
-      dma16_row(sd.sb + static_cast<uint64_t>(min(i, sd.last)) * kRowBytes, i < 4 ? lane_off : lane_off ^ 16u,
-                sd.dst + i * kRow16);
+      dma16_row(sd.sb, (i < 4 ? lane_off : lane_off ^ 16u) + static_cast<u32>(min(i, sd.last)) * kRowBytes, sd.dst + i * kRow16);
     };
     auto issue_rope = [&](const Send& sd) {
       const int ln = lane_again();
@@ -1581,7 +1590,8 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       dma16_row(sd.sb, rope_off, sd.dst_rope);
     };
     auto issue_sub = [&](int sub) {
-      const Send sd = issue_prepare(sub);
+      Send sd;
+      issue_prepare(sub, sd);
 #pragma unroll
       for (int i = 0; i < 8; ++i) issue_row(sd, i);
       issue_rope(sd);
@@ -1726,9 +1736,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       }
     };
     // ---- the accumulators follow the maxima that moved in sub-tile `sub`
-    auto rescale = [&](int sub) {
-      // (read as LDS on purpose: a generic volatile pointer becomes a flat load, whose wait drains the tile loads in flight)
-      const int moved = __builtin_amdgcn_readfirstlane(*((lds_vint*)(smem + kDsFlagOff) + sub % 3));
+    auto rescale = [&](int sub, int moved) {
       if (moved != 0) {
         mfma_result_nops();
 #define XLLM_W4_SCALE(DB, HB, R0, R1, R2, R3) \
@@ -1757,26 +1765,32 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       }
     };
     // ---- O^T[128 dims of the wavefront, all heads] += V^T . P^T of sub-tile `sub` (its P^T blocks are complete)
-    auto pv = [&](int sub, const u32x4 (&vt)[8], bool sends, const Send& sd) {
+    // (the first two P^T blocks are on their way when it is called: pv_begin)
+    auto pv_begin = [&](int sub, u32x4 (&pb)[2]) -> int {
       const char* pbase = smem + kDsPOff + (sub & 1) * 8 * 1024 + lane * 16;
-      // P^T blocks two ahead of the MFMAs that take them
-      u32x4 pb[2];
       __builtin_amdgcn_sched_barrier(0);
-#ifdef XLLM_W4_STAGGER   // (experiment) wavefronts 32 cycles apart, so that their loads do not meet in the address unit
-      if (wave & 1) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-      if (wave & 2) asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-#endif
       pb[0] = *reinterpret_cast<const u32x4*>(pbase);
       pb[1] = *reinterpret_cast<const u32x4*>(pbase + 1024);
+      __builtin_amdgcn_sched_barrier(0);
+      // the head blocks whose maxima moved in this sub-tile: read behind the two blocks, so that one trip to LDS
+      // covers all three (read as LDS on purpose: a generic volatile pointer becomes a flat load, whose wait drains
+      // the tile loads in flight)
+      return __builtin_amdgcn_readfirstlane(*((lds_vint*)(smem + kDsFlagOff) + sub % 3));
+    };
+    auto pv = [&](auto sends_tag, int sub, const u32x4 (&vt)[8], const Send& sd, u32x4 (&pb)[2]) {
+      constexpr bool sends = decltype(sends_tag)::value;   // (the loop exists twice: a branch per row of MFMAs costs 16 cycles)
+      const char* pbase = smem + kDsPOff + (sub & 1) * 8 * 1024 + lane * 16;
+      // P^T blocks two ahead of the MFMAs that take them
+      __builtin_amdgcn_sched_barrier(0);
 #define XLLM_W4_PV_BF16(DB, HB, R0, R1, R2, R3) XLLM_W4_MFMA("v_mfma_f32_16x16x32_bf16", R0, R1, R2, R3, vt[DB], pb[HB & 1]);
 #define XLLM_W4_PV_F16(DB, HB, R0, R1, R2, R3) XLLM_W4_MFMA("v_mfma_f32_16x16x32_f16", R0, R1, R2, R3, vt[DB], pb[HB & 1]);
 #define XLLM_W4_PV_ROW(HB, ROW)                                                              \
   __builtin_amdgcn_sched_barrier(0);                                                         \
   if constexpr (QT::kIsBf16) { ROW(XLLM_W4_PV_BF16) } else { ROW(XLLM_W4_PV_F16) }           \
   if (HB + 2 < 8) pb[HB & 1] = *reinterpret_cast<const u32x4*>(pbase + (HB + 2) * 1024);   \
-  if (sends) {                                                                               \
+  if constexpr (sends) { /* one load per row of MFMAs and wavefront: the address unit takes the CU's four in the time of the row */ \
     issue_row(sd, HB);                                                                       \
-    if (HB == 7) issue_rope(sd);                                                             \
+    if (HB == 3) issue_rope(sd);                                                             \
   }
       XLLM_W4_PV_ROW(0, XLLM_W4_ROW0)
       XLLM_W4_PV_ROW(1, XLLM_W4_ROW1)
@@ -1811,6 +1825,12 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       probabilities(0, sv);
       read_vt(0, vt);
     }
+    bool sends = kDsRing < n_sub;
+    Send sd;
+    sd.sb = 0;
+    sd.last = 0;
+    sd.dst = sd.dst_rope = 0;
+    if (sends) issue_prepare(kDsRing, sd);
     W4_TICK(1)   // run prologue
     for (int sub = 0; sub < n_sub; ++sub) {
       const bool more = sub + 1 < n_sub;
@@ -1819,22 +1839,29 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       __syncthreads();  // P^T of `sub` is complete; sub + 1 has landed; nobody reads sub-tile `sub` in LDS any more
       W4_TICK(2)
       if (tid == 0) flags[(sub + 2) % 3] = 0;   // (last read before this barrier, next raised after the next one)
-      const bool sends = sub + kDsRing < n_sub;
-      Send sd = {};
-      if (sends) sd = issue_prepare(sub + kDsRing);
       W4_TICK(3)
-      rescale(sub);
-      pv(sub, vt, sends, sd);
+      u32x4 pb[2];
+      const int moved = pv_begin(sub, pb);
+      rescale(sub, moved);
+      if (sends) pv(std::true_type{}, sub, vt, sd, pb);
+      else pv(std::false_type{}, sub, vt, sd, pb);
       W4_TICK(4)
       if (more) {
         f32x4 s[2][2];
         float sv[2][8];
         scores(sub + 1, s);
         W4_TICK(5)
+        // the addresses of the loads that the next P.V sends: the page id is read here and used after the softmax
+        sends = sub + 1 + kDsRing < n_sub;
+        int page_read = 0;
+        if (sends) page_read = issue_prepare_read(sub + 1 + kDsRing);
         exponents(sub + 1, s, sv);
         probabilities(sub + 1, sv);
         read_vt(sub + 1, vt);
+        if (sends) issue_prepare_finish(sub + 1 + kDsRing, page_read, sd);
         W4_TICK(6)
+      } else {
+        sends = false;
       }
     }
 
