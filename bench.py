@@ -242,8 +242,10 @@ def neighbours(ops, workloads, torch, dev, steps):
 
 def decode_kernel_name(cfg):
     if cfg.mla:
-        old = os.environ.get("XLLM_MI355_MLA_KERNEL", "") == "heads" or cfg.n_q_heads <= 64
-        return "mla_decode16_kernel" if old else "mla_decode_ds_kernel"
+        knob = os.environ.get("XLLM_MI355_MLA_KERNEL", "")[:1]
+        if knob == "h" or cfg.n_q_heads <= 64:
+            return "mla_decode16_kernel"
+        return "mla_decode_ds_kernel" if knob == "n" else "mla_decode_w4_kernel"
     mfma = (cfg.head_dim == 128 or (cfg.head_dim in (64, 256) and cfg.cache_dtype != "fp8")) and cfg.block_size >= 16 \
         and cfg.block_size & (cfg.block_size - 1) == 0
     return "gqa_mfma_kernel" if mfma else "gqa_decode_kernel"

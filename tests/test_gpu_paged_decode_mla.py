@@ -153,10 +153,10 @@ def test_scores_that_rise_along_the_context(device):
 
 
 def test_other_kernels_for_more_than_64_heads(device):
-    # the default for more than 64 heads has 16 heads per wavefront and P.V by dim block; "wide" (four wavefronts
-    # of 512 registers, 32 heads each) and "heads" (16 heads per wavefront, both products by head block) stay
-    # selectable
-    for knob in ("wide", "heads"):
+    # the default for more than 64 heads has four wavefronts of 512 registers with 32 heads each; "narrow" (eight
+    # wavefronts, 16 heads each, P.V by dim block) and "heads" (16 heads per wavefront, both products by head
+    # block) stay selectable
+    for knob in ("narrow", "heads"):
         _select_kernel(knob)
         try:
             _check(_mla_cfg(f"mla128_{knob}", 3, 128, 100, 1500), 5, device)

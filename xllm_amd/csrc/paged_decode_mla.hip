@@ -1070,7 +1070,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int hb = 0; hb < 8; ++hb) o[db][hb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    float m = kNegBig, l = 0.0f;
+    float m = 0.0f, l = 0.0f;   // reference maximum (set by the run's first sub-tile) and sum of the lane's head
 
     auto issue_sub = [&](int sub) {
       const int tok0 = t_begin + sub * kSubTok + wave * 4;
@@ -1143,26 +1143,34 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      // exponents = scaled score - maximum in one fused multiply-add each; tokens past the end of the context are
+      // masked only in the sub-tile that has any (wave-uniform), and the test for a moved maximum is one compare
+      // of the block's top exponent
       float sv[8];
-      const int tok_base = t_begin + sub * kSubTok + 4 * g;
-      bool over = false;
+      const bool first = sub == 0;   // nothing accumulated yet: the maximum is set, whatever the scores
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        sv[r] = tok_base + r < L ? s0[r] * a.scale_log2 : -INFINITY;
-        sv[4 + r] = tok_base + 16 + r < L ? s1[r] * a.scale_log2 : -INFINITY;
+        sv[r] = __builtin_fmaf(s0[r], a.scale_log2, -m);
+        sv[4 + r] = __builtin_fmaf(s1[r], a.scale_log2, -m);
       }
+      if (t_begin + (sub + 1) * kSubTok > L) {
+        const int tok_base = t_begin + sub * kSubTok + 4 * g;
 #pragma unroll
-      for (int r = 0; r < 8; ++r) over |= sv[r] > m + kSlack;
-      if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare once the maxima have settled
-        float mx = sv[0];
-#pragma unroll
-        for (int r = 1; r < 8; ++r) mx = fmaxf(mx, sv[r]);
-        mx = quad_rows_max(mx);
+        for (int r = 0; r < 4; ++r) {
+          if (tok_base + r >= L) sv[r] = -INFINITY;
+          if (tok_base + 16 + r >= L) sv[4 + r] = -INFINITY;
+        }
+      }
+      const float top = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+      if (__builtin_amdgcn_ballot_w64(top > kSlack || first) != 0) {  // rare once the maxima have settled
+        const float rise = quad_rows_max(top);   // the head's highest score of the sub-tile, above its maximum
         float alpha = 1.0f;
-        if (mx > m + kSlack) {
-          alpha = fast_exp2(m - mx);
-          m = mx;
+        if (rise > kSlack || first) {
+          alpha = first ? 1.0f : fast_exp2(-rise);
+          m += rise;
           l *= alpha;
+#pragma unroll
+          for (int r = 0; r < 8; ++r) sv[r] -= rise;
         }
         // the factor of every head of the block (1 where the maximum stayed), and the block's flag (the lane's
         // position is recomputed here: kept in registers of their own for this rare path, the addresses get spilled,
@@ -1178,7 +1186,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
       float p[8];
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
-        p[r] = fast_exp2(sv[r] - m);
+        p[r] = fast_exp2(sv[r]);
         l += p[r];
       }
       // k-slot g*8 + j of the P.V MFMA <-> token 4g + j of block 0 (j < 4), of block 1 (j >= 4): the lane's
@@ -1608,7 +1616,20 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     };
 
     // ---- S^T of sub-tile `sub` for the wavefront's 32 heads: s[j][tb] = tokens 16 tb + 4g + r, head 16 j + c16
-    auto scores = [&](int sub, f32x4 (&s)[2][2]) {
+    constexpr int kAheadW = XLLM_W4_AHEAD;
+    // the K operands of the first kAheadW k-steps of sub-tile `sub` (its rows have landed): sent for before the first
+    // half of P.V, so that the scores start on operands that are there
+    auto scores_begin = [&](int sub, u32x4 (&xa)[kAheadW], u32x4 (&xb)[kAheadW]) {
+      const char* ka = smem + (sub % kDsRing) * kSubBytes + k_row0;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < kAheadW; ++i) {   // (kAheadW <= 16: latent k-steps)
+        xa[i] = *reinterpret_cast<const u32x4*>(ka + i * 64);
+        xb[i] = *reinterpret_cast<const u32x4*>(ka + i * 64 + 16 * kRow16);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto scores = [&](int sub, f32x4 (&s)[2][2], u32x4 (&xa)[kAheadW], u32x4 (&xb)[kAheadW]) {
       const char* kb = smem + (sub % kDsRing) * kSubBytes;
       const int ln = lane_again();
       const char* kr = kb + kRope16Off + (ln & 15) * (kDR * 2);
@@ -1619,17 +1640,10 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
         for (int tb = 0; tb < 2; ++tb) s[j][tb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
       const char* ka = kb + k_row0;
       // K operands kAheadW k-steps ahead of the MFMAs that take them, in an order the scheduler may not change
-      constexpr int kAheadW = XLLM_W4_AHEAD;
       auto k_addr = [&](int kk) -> const char* {
         return kk < kDL / 32 ? ka + kk * 64 : kr + (kk == kDL / 32 ? kr_x : kr_x ^ 4) * 16;
       };
-      u32x4 xa[kAheadW], xb[kAheadW];
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < kAheadW; ++i) {
-        xa[i] = *reinterpret_cast<const u32x4*>(k_addr(i));
-        xb[i] = *reinterpret_cast<const u32x4*>(k_addr(i) + 16 * (i < kDL / 32 ? kRow16 : kDR * 2));
-      }
 #pragma unroll
       for (int kk = 0; kk < kKSteps32; ++kk) {
         __builtin_amdgcn_sched_barrier(0);
@@ -1657,18 +1671,10 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     };
     // ---- exponents sv = scaled score - maximum of sub-tile `sub`; masks (last sub-tile of a context only), moved
     // maxima (rare), their factors and flag
-    auto exponents = [&](int sub, const f32x4 (&s)[2][2], float (&sv)[2][8]) {
+    auto exponents_rest = [&](int sub, float (&sv)[2][8]) {
       const bool first = sub == 0;   // nothing accumulated yet: the maxima are set, whatever the scores
       bool over = first;
       float top[2];
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          sv[j][r] = __builtin_fmaf(s[j][0][r], a.scale_log2, -m[j]);
-          sv[j][4 + r] = __builtin_fmaf(s[j][1][r], a.scale_log2, -m[j]);
-        }
-      }
       if (t_begin + (sub + 1) * kSubTok > L) {   // (wave-uniform) tokens past the end of the context
         const int tok_base = t_begin + sub * kSubTok + 4 * g;
 #pragma unroll
@@ -1708,6 +1714,17 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
         }
       }
     };
+    auto exponents = [&](int sub, const f32x4 (&s)[2][2], float (&sv)[2][8]) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          sv[j][r] = __builtin_fmaf(s[j][0][r], a.scale_log2, -m[j]);
+          sv[j][4 + r] = __builtin_fmaf(s[j][1][r], a.scale_log2, -m[j]);
+        }
+      }
+      exponents_rest(sub, sv);
+    };
     // ---- probabilities of sub-tile `sub` from its exponents; the wavefront's two P^T blocks to LDS
     auto probabilities = [&](int sub, const float (&sv)[2][8]) {
 #pragma unroll
@@ -1725,10 +1742,11 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       }
     };
     // ---- the V^T operands of sub-tile `sub` for the wavefront's dims, into registers
-    auto read_vt = [&](int sub, u32x4 (&vt)[8]) {
+    auto read_vt = [&](int sub, u32x4 (&vt)[8], int db0 = 0, int db1 = 8) {
       const char* va = smem + (sub % kDsRing) * kSubBytes + v_row0;
 #pragma unroll
       for (int db = 0; db < 8; ++db) {
+        if (db < db0 || db >= db1) continue;
         const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + db * 32));
         const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(va + 16 * kRow16 + db * 32));
         const s16x8 v = {lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
@@ -1777,20 +1795,64 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       // the tile loads in flight)
       return __builtin_amdgcn_readfirstlane(*((lds_vint*)(smem + kDsFlagOff) + sub % 3));
     };
-    auto pv = [&](auto sends_tag, int sub, const u32x4 (&vt)[8], const Send& sd, u32x4 (&pb)[2]) {
-      constexpr bool sends = decltype(sends_tag)::value;   // (the loop exists twice: a branch per row of MFMAs costs 16 cycles)
+    // Rows FIRST .. LAST - 1 (head blocks) of one half of the wavefront's dims (HALF 0: dim blocks 0-3, with the
+    // tile loads of a later sub-tile, one per row; HALF 1: dim blocks 4-7).  MODE says what rides in the shadow of
+    // the MFMAs of half 1, a few vector instructions behind each of them (a wavefront issues an MFMA every 16
+    // cycles and has 12 of them for other instructions): 1 = exponents and block maxima of the scores in `sc`
+    // (rows 0-2), 2 = exponentials, sums and the two P^T blocks (rows 3-7), 0 = nothing.
+    auto pv_rows = [&](auto half_tag, auto mode_tag, auto first_tag, auto last_tag, auto sends_tag, int sub,
+                       const u32x4 (&vt)[8], const Send& sd, u32x4 (&pb)[2], const f32x4 (&sc)[2][2], float (&sv)[2][8],
+                       float (&top)[2], bool prep = false, int page_read = 0, Send* sd_next = nullptr) {
+      constexpr int HALF = decltype(half_tag)::value, MODE = decltype(mode_tag)::value;
+      constexpr int FIRST = decltype(first_tag)::value, LAST = decltype(last_tag)::value;
+      constexpr bool sends = decltype(sends_tag)::value;
       const char* pbase = smem + kDsPOff + (sub & 1) * 8 * 1024 + lane * 16;
-      // P^T blocks two ahead of the MFMAs that take them
-      __builtin_amdgcn_sched_barrier(0);
-#define XLLM_W4_PV_BF16(DB, HB, R0, R1, R2, R3) XLLM_W4_MFMA("v_mfma_f32_16x16x32_bf16", R0, R1, R2, R3, vt[DB], pb[HB & 1]);
-#define XLLM_W4_PV_F16(DB, HB, R0, R1, R2, R3) XLLM_W4_MFMA("v_mfma_f32_16x16x32_f16", R0, R1, R2, R3, vt[DB], pb[HB & 1]);
-#define XLLM_W4_PV_ROW(HB, ROW)                                                              \
-  __builtin_amdgcn_sched_barrier(0);                                                         \
-  if constexpr (QT::kIsBf16) { ROW(XLLM_W4_PV_BF16) } else { ROW(XLLM_W4_PV_F16) }           \
-  if (HB + 2 < 8) pb[HB & 1] = *reinterpret_cast<const u32x4*>(pbase + (HB + 2) * 1024);   \
-  if constexpr (sends) { /* one load per row of MFMAs and wavefront: the address unit takes the CU's four in the time of the row */ \
-    issue_row(sd, HB);                                                                       \
-    if (HB == 3) issue_rope(sd);                                                             \
+      auto hook = [&](auto n_tag) {
+        constexpr int n = decltype(n_tag)::value;   // MFMA number within the half: 4 * row + dim block
+        if constexpr (HALF == 0 && n == 22) {   // the addresses of the loads that the next sub-tile's P.V sends (scalar work)
+          if (prep) issue_prepare_finish(sub + 1 + kDsRing, page_read, *sd_next);
+        }
+        if constexpr (MODE == 1 && n >= 2 && n < 10) {
+          constexpr int k = n - 2, v0 = 2 * k, v1 = 2 * k + 1, j = v0 >> 3, r0 = v0 & 7, r1 = v1 & 7;
+          sv[j][r0] = __builtin_fmaf(sc[j][r0 >> 2][r0 & 3], a.scale_log2, -m[j]);
+          sv[j][r1] = __builtin_fmaf(sc[j][r1 >> 2][r1 & 3], a.scale_log2, -m[j]);
+          const float t = fmaxf(sv[j][r0], sv[j][r1]);
+          top[j] = (k & 3) == 0 ? t : fmaxf(top[j], t);
+        }
+        if constexpr (MODE == 2 && n >= 12 && n < 28) {
+          constexpr int v = n - 12, j = v >> 3, r = v & 7;
+          sv[j][r] = fast_exp2(sv[j][r]);
+          l[j] += sv[j][r];
+        }
+        if constexpr (MODE == 2 && (n == 21 || n == 29)) {
+          // k-slot g*8 + i of the P.V MFMA <-> token 4g + i of block 0 (i < 4), of block 1 (i >= 4): the lane's
+          // eight probabilities are its 16 bytes of the B operand
+          constexpr int j = n == 21 ? 0 : 1;
+          const u32x4 w = {QT::pack(sv[j][0], sv[j][1]), QT::pack(sv[j][2], sv[j][3]), QT::pack(sv[j][4], sv[j][5]),
+                           QT::pack(sv[j][6], sv[j][7])};
+          *reinterpret_cast<u32x4*>(smem + kDsPOff + (((sub + 1) & 1) * 8 + wave * 2 + j) * 1024 + lane * 16) = w;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+#define XLLM_W4_PV_BF16(DB, HB, R0, R1, R2, R3)                                                 \
+  if constexpr ((DB >> 2) == HALF) {                                                            \
+    XLLM_W4_MFMA("v_mfma_f32_16x16x32_bf16", R0, R1, R2, R3, vt[DB], pb[HB & 1]);               \
+    hook(std::integral_constant<int, HB * 4 + (DB & 3)>{});                                     \
+  }
+#define XLLM_W4_PV_F16(DB, HB, R0, R1, R2, R3)                                                  \
+  if constexpr ((DB >> 2) == HALF) {                                                            \
+    XLLM_W4_MFMA("v_mfma_f32_16x16x32_f16", R0, R1, R2, R3, vt[DB], pb[HB & 1]);                \
+    hook(std::integral_constant<int, HB * 4 + (DB & 3)>{});                                     \
+  }
+#define XLLM_W4_PV_ROW(HB, ROW)                                                                 \
+  if constexpr (HB >= FIRST && HB < LAST) {                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                          \
+    if constexpr (QT::kIsBf16) { ROW(XLLM_W4_PV_BF16) } else { ROW(XLLM_W4_PV_F16) }            \
+    if (HB + 2 < 8) pb[HB & 1] = *reinterpret_cast<const u32x4*>(pbase + (HB + 2) * 1024);      \
+    if constexpr (sends) { /* the loads of a later sub-tile, one per row (spread over both halves they cost more: the */ \
+      issue_row(sd, HB);   /* second half is dense with the softmax arithmetic) */              \
+      if (HB == 3) issue_rope(sd);                                                              \
+    }                                                                                           \
   }
       XLLM_W4_PV_ROW(0, XLLM_W4_ROW0)
       XLLM_W4_PV_ROW(1, XLLM_W4_ROW1)
@@ -1804,6 +1866,12 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
 #undef XLLM_W4_PV_F16
 #undef XLLM_W4_PV_BF16
       __builtin_amdgcn_sched_barrier(0);
+    };
+    // the first two P^T blocks of `sub` again, for the second half of its P.V
+    auto pv_again = [&](int sub, u32x4 (&pb)[2]) {
+      const char* pbase = smem + kDsPOff + (sub & 1) * 8 * 1024 + lane * 16;
+      pb[0] = *reinterpret_cast<const u32x4*>(pbase);
+      pb[1] = *reinterpret_cast<const u32x4*>(pbase + 1024);
     };
 
     // the chunk loads and the Q loads have landed (one wait for both latencies)
@@ -1820,7 +1888,9 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     {
       f32x4 s[2][2];
       float sv[2][8];
-      scores(0, s);
+      u32x4 xa[kAheadW], xb[kAheadW];
+      scores_begin(0, xa, xb);
+      scores(0, s, xa, xb);
       exponents(0, s, sv);
       probabilities(0, sv);
       read_vt(0, vt);
@@ -1840,29 +1910,57 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       W4_TICK(2)
       if (tid == 0) flags[(sub + 2) % 3] = 0;   // (last read before this barrier, next raised after the next one)
       W4_TICK(3)
+      using I0 = std::integral_constant<int, 0>;
+      using I1 = std::integral_constant<int, 1>;
+      using I2 = std::integral_constant<int, 2>;
+      using I3 = std::integral_constant<int, 3>;
+      using I8 = std::integral_constant<int, 8>;
       u32x4 pb[2];
+      f32x4 sc[2][2];
+      float sv[2][8];
+      float top[2] = {0.0f, 0.0f};
+      // the page id behind the addresses of the loads that the NEXT sub-tile's P.V sends, and the first K operands of
+      // the scores: their trips to LDS pass behind the first half of P.V
+      const bool sends_next = more && sub + 1 + kDsRing < n_sub;
+      int page_read = 0;
+      if (sends_next) page_read = issue_prepare_read(sub + 1 + kDsRing);
+      Send sd_next;
+      sd_next.sb = 0;
+      sd_next.last = 0;
+      sd_next.dst = sd_next.dst_rope = 0;
       const int moved = pv_begin(sub, pb);
       rescale(sub, moved);
-      if (sends) pv(std::true_type{}, sub, vt, sd, pb);
-      else pv(std::false_type{}, sub, vt, sd, pb);
+      // ---- first half of P.V of `sub` (dim blocks 0-3), with the loads of sub + 3
+      if (sends) pv_rows(I0{}, I0{}, I0{}, I8{}, std::true_type{}, sub, vt, sd, pb, sc, sv, top, sends_next, page_read, &sd_next);
+      else pv_rows(I0{}, I0{}, I0{}, I8{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top, sends_next, page_read, &sd_next);
       W4_TICK(4)
       if (more) {
-        f32x4 s[2][2];
-        float sv[2][8];
-        scores(sub + 1, s);
+        u32x4 xa[kAheadW], xb[kAheadW];
+        scores_begin(sub + 1, xa, xb);
+        scores(sub + 1, sc, xa, xb);
         W4_TICK(5)
-        // the addresses of the loads that the next P.V sends: the page id is read here and used after the softmax
-        sends = sub + 1 + kDsRing < n_sub;
-        int page_read = 0;
-        if (sends) page_read = issue_prepare_read(sub + 1 + kDsRing);
-        exponents(sub + 1, s, sv);
-        probabilities(sub + 1, sv);
+        // ---- second half of P.V of `sub` (dim blocks 4-7) with the softmax of sub + 1 in the shadow of its MFMAs
+        pv_again(sub, pb);
+        pv_rows(I1{}, I1{}, I0{}, I3{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top);
+        const bool plain = t_begin + (sub + 2) * kSubTok <= L && !(top[0] > kSlack || top[1] > kSlack);
+        if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
+          pv_rows(I1{}, I2{}, I3{}, I8{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top);
+        } else {   // a maximum moves, or the sub-tile is the ragged end of a context: one thing after the other
+          pv_rows(I1{}, I0{}, I3{}, I8{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top);
+          exponents_rest(sub + 1, sv);
+          probabilities(sub + 1, sv);
+        }
         read_vt(sub + 1, vt);
-        if (sends) issue_prepare_finish(sub + 1 + kDsRing, page_read, sd);
         W4_TICK(6)
-      } else {
-        sends = false;
+      } else {   // (the last sub-tile of a run sends nothing: sub + 3 is past its end)
+        pv_again(sub, pb);
+        pv_rows(I1{}, I0{}, I0{}, I8{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top);
       }
+      sends = sends_next;
+      sd.sb = sd_next.sb;
+      sd.last = sd_next.last;
+      sd.dst = sd_next.dst;
+      sd.dst_rope = sd_next.dst_rope;
     }
 
     // ---- end of the run: the owners publish 1 / sum per head, every wavefront writes its dims of every head
@@ -2717,7 +2815,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       else launch_timed(mla_decode_kernel<BF16>, grid, dim3(kMlaThreads), smem, stream, a);
     } else if (use_p) {
       launch_timed(mla_decode32w_kernel, grid, dim3(kWThreads), kPLdsBytes, stream, a);
-    } else if (by_dims && knob == 'w') {  // (as fast as the default on 128 heads, with half the LDS traffic)
+    } else if (by_dims && knob != 'n') {  // ('n'arrow: the kernel with 16 heads per scoring wavefront, 3 % slower on 128 heads)
       if (f16) launch_timed(mla_decode_w4_kernel<FP16>, grid, dim3(kW4Threads), kW4LdsBytes, stream, a);
       else launch_timed(mla_decode_w4_kernel<BF16>, grid, dim3(kW4Threads), kW4LdsBytes, stream, a);
     } else if (by_dims) {
