@@ -59,6 +59,18 @@ def test_fp16_and_other_head_dims(device):
         _check_config(cfg, 100 + D + Hq, device, dtype=dt)
 
 
+def test_head_dim_64_with_fp8_pages_on_the_matrix_core_kernel(device):
+    # fp8 pages with head dim 64: rows of 64 bytes, 64 tokens per stage multiplied as two halves of 32.  Group sizes
+    # 1, 4, 16 and one that needs two head blocks; block sizes 16 / 64 / 128; lengths around the 16-, 32- and
+    # 64-token boundaries; contexts long enough to span workers.
+    for name, batch, Hq, Hkv, bs, lo, hi in (("g1", 4, 4, 4, 32, 1, 700), ("g4", 5, 32, 8, 16, 1, 3000),
+                                             ("g16", 3, 16, 1, 128, 100, 2500), ("g20", 3, 40, 2, 64, 50, 1200),
+                                             ("long", 3, 8, 2, 16, 20000, 40000)):
+        _check_fp8(workloads.DecodeConfig(f"d64_fp8_{name}", batch, Hq, Hkv, 64, bs, lo, hi, cache_dtype="fp8"), 700 + Hq, device)
+    for L in (1, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 96, 129):
+        _check_fp8(workloads.DecodeConfig(f"d64_fp8_L{L}", 2, 8, 2, 64, 16, L, L, cache_dtype="fp8"), 800 + L, device)
+
+
 def test_head_dim_256_on_the_matrix_core_kernel(device):
     # head dim 256 with a power-of-two block size >= 16: rows of 512 bytes, 8 tokens per stage in a 16-row score
     # block whose upper half is masked.  Group sizes 1, 4, 16 and one that needs two head blocks; block sizes

@@ -685,13 +685,15 @@ struct MfmaLayout {
 // ceil(tokens * group / 16) single tokens; column j is masked beyond its own length.
 // D = 64 (16-bit pages only): rows of 128 bytes, so a stage holds 32 tokens and is multiplied as two blocks
 // of 16 like an fp8 stage, with 2 k-steps per score block and 4 dim blocks.
+// D = 64 with fp8 pages: rows of 64 bytes, a stage holds 64 tokens and is multiplied as two halves of 32, each like
+// an fp8 stage of head dim 128 (2 k-steps per score block, 4 dim blocks).
 // D = 256 (16-bit pages only): rows of 512 bytes, a stage holds 8 tokens.  They take the first 8 rows of a
 // 16-token score block whose other rows repeat them under a mask (the matrix pipe has time to spare: a stage
 // is 8 KB of HBM traffic whatever the head dim), with 8 k-steps per score block and 16 dim blocks.
 template <typename QT, bool FP8, int NS, bool VL, int D>
 __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   static_assert(NS >= 2 && NS <= 4, "wait_younger_stages covers up to three stages in flight");
-  static_assert(D == 128 || ((D == 64 || D == 256) && !FP8), "head dims of the matrix-core loop");
+  static_assert(D == 128 || D == 64 || (D == 256 && !FP8), "head dims of the matrix-core loop");
   using Lay = MfmaLayout<NS, D>;
   constexpr int G = kMfmaHeads;
   constexpr int KS = D / 32;               // k-steps of a score block
@@ -719,7 +721,8 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // chunk swizzles within a row: K by the row number; V by twice its low two bits (16-bit pages,
   // whose transposing read takes 4 rows x 32 bytes per 16 lanes) or by its low three bits (fp8)
   auto swz_k = [](int row) { return row & (LPR - 1); };
-  auto swz_v = [](int row) { return FP8 ? (row & 7) : ((row & 3) << 1); };
+  constexpr int SW8 = LPR < 8 ? LPR - 1 : 7;   // fp8 rows: chunk swizzle by the low bits of the row, as many as the row has chunks
+  auto swz_v = [](int row) { return FP8 ? (row & SW8) : ((row & 3) << 1); };
   const int hb_per_kv = VL ? a.chunk_blocks : (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
   // packed query chunks: the part of the sequence's chunk that column block cu.hbk holds
@@ -871,7 +874,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // 16 + 4g .. 16 + 4g+3 -- the order in which the two score blocks leave the P^T registers
   const int v8_row = ((c16 >> 1) < 4 ? 0 : 12) + 4 * g + (c16 >> 1);
   const int v8_read = T * RB + v8_row * RB + (c16 & 1) * 8;
-  const int v8_y = (v8_row & 7) << 4;
+  const int v8_y = (v8_row & SW8) << 4;
 
   if (loader) {
   // ---- the loading wavefront: issues stage p of the worker's range; pc is the context of that stage
@@ -1002,8 +1005,16 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         const int row = RPI * i + dr;
         const int sub = min(RPI * i, lim) >> 4;  // sub-block of the rows this instruction reads
         const u32 ro = static_cast<u32>((min(row, lim) & 15) * a.row_bytes);
-        dma16_row(NSUB > 1 && sub > 0 ? kb[NSUB - 1] : kb[0], ro + ((dc ^ swz_k(row)) * 16), dst + i * 1024);
-        dma16_row(NSUB > 1 && sub > 0 ? vb[NSUB - 1] : vb[0], ro + ((dc ^ swz_v(row)) * 16), dst + T * RB + i * 1024);
+        uint64_t kbs = kb[0], vbs = vb[0];
+#pragma unroll
+        for (int s2 = 1; s2 < NSUB; ++s2) {
+          if (sub >= s2) {
+            kbs = kb[s2];
+            vbs = vb[s2];
+          }
+        }
+        dma16_row(kbs, ro + ((dc ^ swz_k(row)) * 16), dst + i * 1024);
+        dma16_row(vbs, ro + ((dc ^ swz_v(row)) * 16), dst + T * RB + i * 1024);
       }
     }
     ++p;
@@ -1237,7 +1248,11 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         o[mb] = Mfma<QT>::k32(u32x4{lo[0], lo[1], hi[0], hi[1]}, pb, o[mb]);
       }
     } else {
-      // ---- scores of the stage's 32 tokens, two blocks of 16: lane (head c16, tokens 16 tb + 4g ..)
+      // ---- fp8 pages: the stage's tokens in halves of 32 (one half at head dim 128, two at head dim 64)
+#pragma unroll
+      for (int hf = 0; hf < T / 32; ++hf) {
+      const char* sth = st + hf * 32 * RB;
+      // scores of the half's 32 tokens, two blocks of 16: lane (head c16, tokens 16 tb + 4g ..)
       float sv[8];
       bool over = false;
 #pragma unroll
@@ -1245,14 +1260,14 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
         const int tok = tb * 16 + c16;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < KS; ++kk) {
           const u32x2 k8 = *reinterpret_cast<const u32x2*>(
-              st + tok * RB + (((kk * 2 + (g >> 1)) ^ (tok & 7)) * 16) + (g & 1) * 8);
+              sth + tok * RB + (((kk * 2 + (g >> 1)) ^ (tok & SW8)) * 16) + (g & 1) * 8);
           const u32x4 kr = {QT::template from_fp8x2<false>(k8[0]), QT::template from_fp8x2<true>(k8[0]),
                             QT::template from_fp8x2<false>(k8[1]), QT::template from_fp8x2<true>(k8[1])};
           sc = Mfma<QT>::k32(kr, q[kk], sc);
         }
-        const int tok0 = (cc.st0 + cc.st) * T + tb * 16 + 4 * g;
+        const int tok0 = (cc.st0 + cc.st) * T + hf * 32 + tb * 16 + 4 * g;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           sv[tb * 4 + r] = tok0 + r < Lc && tok0 + r >= Lo ? sc[r] * score_scale : -INFINITY;
@@ -1283,13 +1298,14 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       // eight tokens of its group's k-slots for dim column 16 mb + c16
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const i32x2 v8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(st + v8_read + (v8_y ^ (mb << 4))));
+        const i32x2 v8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2*)(sth + v8_read + (v8_y ^ (mb << 4))));
         const u32x4 vt = {QT::template from_fp8x2<false>(static_cast<u32>(v8[0])),
                           QT::template from_fp8x2<true>(static_cast<u32>(v8[0])),
                           QT::template from_fp8x2<false>(static_cast<u32>(v8[1])),
                           QT::template from_fp8x2<true>(static_cast<u32>(v8[1]))};
         o[mb] = Mfma<QT>::k32(vt, pb, o[mb]);
       }
+      }  // halves
     }
 
     // ---- end of a run: last stage of the context or of the worker's range
@@ -1632,6 +1648,8 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
     const bool out_aligned8 = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
     if (head_dim == 128 && a.bs_shift >= 4 && out_aligned8 && use_mfma_kernel())
       return launch_gqa_mfma<QT, true>(a, wsb, s, plan_only, need);
+    if (head_dim == 64 && a.bs_shift >= 4 && out_aligned8 && use_mfma_kernel())
+      return launch_gqa_mfma<QT, true, false, 64>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, true, 64, 4, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, true, 128, 8, 2>(a, wsb, s, plan_only, need);
