@@ -167,6 +167,20 @@ def test_other_kernels_for_more_than_64_heads(device):
             _select_kernel("")
 
 
+def test_many_short_sequences_with_128_heads(device):
+    # more sequences than workgroups: a workgroup meets several contexts in one launch (whole ones written
+    # directly, the pieces at both ends of its range as partials), and a batch beyond what one launch holds;
+    # the default kernel and the eight-wavefront one
+    for knob in ("", "narrow"):
+        _select_kernel(knob)
+        try:
+            _check(_mla_cfg(f"mla128_b300_{knob}", 300, 128, 1, 150), 17, device)
+            _check(_mla_cfg(f"mla128_b600_{knob}", 600, 128, 40, 100), 18, device)
+        finally:
+            _select_kernel("")
+    _check(_mla_cfg("mla128_b1100", 1100, 128, 1, 40), 19, device)
+
+
 def test_producer_consumer_kernel(device):
     # the kernel with the two products on different wavefronts, selected by the tuning knob
     _select_kernel("split")
