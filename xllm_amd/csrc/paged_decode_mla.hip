@@ -72,11 +72,13 @@ struct MlaArgs {
   const int32_t* block_table;
   const int32_t* seq_lens;
   int* ws_prefix;  // [batch + 1]
-  float* ws_out;   // [2 * n_teams][H][512]
+  float* ws_out;   // [2 * n_teams][slot_heads][512]: partial rows, head by head, or as the tiles of the accumulators
+                   // (mla_decode_w4_kernel with mla_merge_tiles_kernel)
   float* ws_lse;   // [2 * n_teams][H]
   int64_t table_stride;
   int batch;
   int n_heads;
+  int slot_heads;  // n_heads rounded up to 16
   int n_hb;        // head blocks of 64 = workgroups per team
   int n_teams;
   int block_size;
@@ -1519,20 +1521,24 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       issue_chunk(ck_cur);
       if ((ck_cur + 1) * kWave < n_pages) issue_chunk(ck_cur + 1);
     }
-    if (tid < 3) flags[tid] = 0;
+    // (the lane's coordinates, opaque to the compiler: what it can compute from them before the first run it keeps in
+    // scratch memory through the loop, and a reload here waits for the chunk loads just issued)
+    const int lane_p = lane_again();
+    const int c16p = lane_p & 15, gp = lane_p >> 4;
+    if (wave == 0 && lane_p < 3) flags[lane_p] = 0;
 
     // Q^T operands of the two 16-head blocks: lane (head c16, k-group g) keeps dims kk*32 + g*8 .. +8 of every k-step
     u32x4 q[2][kKSteps32];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int head = head0 + wave * 32 + j * 16 + c16;
+      const int head = head0 + wave * 32 + j * 16 + c16p;
       const char* qn = a.q_nope + (static_cast<int64_t>(b) * H + head) * kDL * 2;
       const char* qp = a.q_pe + (static_cast<int64_t>(b) * H + head) * kDR * 2;
 #pragma unroll
       for (int kk = 0; kk < kKSteps32; ++kk) {
         u32x4 x = {0u, 0u, 0u, 0u};
         if (head < H)
-          x = kk < kDL / 32 ? ldg16(qn + (kk * 32 + g * 8) * 2) : ldg16(qp + ((kk - kDL / 32) * 32 + g * 8) * 2);
+          x = kk < kDL / 32 ? ldg16(qn + (kk * 32 + gp * 8) * 2) : ldg16(qp + ((kk - kDL / 32) * 32 + gp * 8) * 2);
         q[j][kk] = x;
       }
     }
@@ -1966,13 +1972,19 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     // ---- end of the run: the owners publish 1 / sum per head, every wavefront writes its dims of every head
     const float lsum0 = quad_rows_sum(l[0]), lsum1 = quad_rows_sum(l[1]);
     const int64_t ps_base = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H;
+    // The lane's coordinates once more, opaque to the compiler.  Address arithmetic of the epilogue that can be done
+    // before the loop is done there otherwise, and carried through the loop in scratch memory: every reload then waits
+    // for all the stores issued before it (one counter covers loads and stores), a round trip to memory per row.
+    const int ln = lane_again();
+    const int c16e = ln & 15, ge = ln >> 4;
+    mfma_result_nops();
     __syncthreads();  // the last sub-tile's factors have been read
-    if (g == 0) {
-      fac[wave * 32 + c16] = 1.0f / lsum0;
-      fac[wave * 32 + 16 + c16] = 1.0f / lsum1;
+    if (ge == 0) {
+      fac[wave * 32 + c16e] = 1.0f / lsum0;
+      fac[wave * 32 + 16 + c16e] = 1.0f / lsum1;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const int hd = head0 + wave * 32 + j * 16 + c16;
+        const int hd = head0 + wave * 32 + j * 16 + c16e;
         if (hd < H) {
           const float lse2 = m[j] + fast_log2(j == 0 ? lsum0 : lsum1);
           if (complete && a.lse != nullptr) a.lse[b * H + hd] = lse2 * kLn2;
@@ -1981,37 +1993,52 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       }
     }
     __syncthreads();
-    mfma_result_nops();
+    // Output rows of a whole context go out head by head (COMPLETE).  Partial rows go out as the tiles they are in the
+    // registers, [16-head block][wavefront][dim block][lane][4 floats]: every store instruction then writes 1 KB in
+    // one piece.  Head by head it writes sixteen pieces of 64 bytes, and the burst of partial rows that ends a launch
+    // takes twice as long to issue (it is bound by the number of write requests, not by their bytes).
 #define XLLM_W4_OUT(DB, HB, R0, R1, R2, R3)                                                          \
   {                                                                                                  \
     f32x4 t;                                                                                         \
     XLLM_W4_GET(R0, R1, R2, R3, t);                                                                  \
     t *= inv;                                                                                        \
-    if (complete) {                                                                                  \
+    if (COMPLETE) {                                                                                  \
       const u32x2 w = {QT::pack(t[0], t[1]), QT::pack(t[2], t[3])};                                  \
-      *reinterpret_cast<u32x2*>(op + DB * 32) = w;                                                   \
+      *reinterpret_cast<u32x2*>(dst + DB * 32) = w;                                                  \
     } else {                                                                                         \
-      *reinterpret_cast<f32x4*>(wp + DB * 16) = t;                                                   \
+      *reinterpret_cast<f32x4*>(dst + DB * 1024) = t;                                                \
     }                                                                                                \
   }
 #define XLLM_W4_OUT_ROW(HB, ROW)                                                                     \
   {                                                                                                  \
-    const int hd = head0 + HB * 16 + c16;                                                            \
+    const int hd = head0 + HB * 16 + c16e;                                                           \
     if (HB < n16 && hd < H) {                                                                        \
-      const float inv = fac[HB * 16 + c16];                                                          \
-      char* op = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + wave * 128 + 4 * g) * 2;        \
-      float* wp = a.ws_out + (ps_base + hd) * kDL + wave * 128 + 4 * g;                              \
+      const float inv = fac[HB * 16 + c16e];                                                         \
+      char* dst = COMPLETE ? a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + wave * 128 + 4 * ge) * 2 \
+                           : tiles + (HB * 4 + wave) * 8192;                                         \
       ROW(XLLM_W4_OUT)                                                                               \
     }                                                                                                \
   }
-    XLLM_W4_OUT_ROW(0, XLLM_W4_ROW0)
-    XLLM_W4_OUT_ROW(1, XLLM_W4_ROW1)
-    XLLM_W4_OUT_ROW(2, XLLM_W4_ROW2)
-    XLLM_W4_OUT_ROW(3, XLLM_W4_ROW3)
-    XLLM_W4_OUT_ROW(4, XLLM_W4_ROW4)
-    XLLM_W4_OUT_ROW(5, XLLM_W4_ROW5)
-    XLLM_W4_OUT_ROW(6, XLLM_W4_ROW6)
-    XLLM_W4_OUT_ROW(7, XLLM_W4_ROW7)
+#define XLLM_W4_OUT_ROWS                                                                             \
+  XLLM_W4_OUT_ROW(0, XLLM_W4_ROW0)                                                                   \
+  XLLM_W4_OUT_ROW(1, XLLM_W4_ROW1)                                                                   \
+  XLLM_W4_OUT_ROW(2, XLLM_W4_ROW2)                                                                   \
+  XLLM_W4_OUT_ROW(3, XLLM_W4_ROW3)                                                                   \
+  XLLM_W4_OUT_ROW(4, XLLM_W4_ROW4)                                                                   \
+  XLLM_W4_OUT_ROW(5, XLLM_W4_ROW5)                                                                   \
+  XLLM_W4_OUT_ROW(6, XLLM_W4_ROW6)                                                                   \
+  XLLM_W4_OUT_ROW(7, XLLM_W4_ROW7)
+    // (16-head blocks of this workgroup's 128 heads: block hb128 * 8 + HB of the slot)
+    char* tiles = reinterpret_cast<char*>(a.ws_out) +
+                  ((static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * a.slot_heads + head0) * (kDL * 4) + ln * 16;
+    if (complete) {
+      constexpr bool COMPLETE = true;
+      XLLM_W4_OUT_ROWS
+    } else {
+      constexpr bool COMPLETE = false;
+      XLLM_W4_OUT_ROWS
+    }
+#undef XLLM_W4_OUT_ROWS
 #undef XLLM_W4_OUT_ROW
 #undef XLLM_W4_OUT
     first_run = false;
@@ -2672,6 +2699,89 @@ __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
   if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = (M + fast_log2(W)) * kLn2;
 }
 
+// The same merge for partial rows kept as tiles (mla_decode_w4_kernel).  One workgroup per (block of 16 heads,
+// sequence), laid out like the four wavefronts that wrote the tiles: wavefront w, lane (head c16, k-group g) owns
+// dims 128 w + 16 db + 4 g .. + 3 of head 16 hb + c16 for the eight dim blocks db, and every load instruction reads
+// 1 KB in one piece.  Four teams at a time, their 32 loads per lane issued together.
+template <typename QT>
+__global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
+  const int hb = blockIdx.x;
+  const int b = blockIdx.y;
+  const int H = a.n_heads;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int w = threadIdx.x >> 6;
+  const int c16 = lane & 15, g = lane >> 4;
+  const int hd = hb * 16 + c16;
+  const bool head_ok = hd < H;
+#ifdef XLLM_DS_TIMING
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)   // (measurement build only) when the merge kernel starts
+    reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H)[2048 * 10] = wall_clock64();
+#endif
+  const int64_t first = a.ws_prefix[b];
+  const int64_t last = static_cast<int64_t>(a.ws_prefix[b + 1]) - 1;
+  const int64_t total = a.ws_prefix[a.batch];
+  char* out = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + w * 128 + 4 * g) * 2;
+  if (last < first) {  // empty sequence
+    if (head_ok) {
+#pragma unroll
+      for (int db = 0; db < 8; ++db) *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{0u, 0u};
+      if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * H + hd] = -INFINITY;
+    }
+    return;
+  }
+  const int64_t n = a.n_teams;
+  const int t_first = team_of(first, total, n);
+  const int t_last = team_of(last, total, n);
+  if (t_first == t_last) return;  // one team saw the whole context and wrote the output
+  // (team ranges stepped as in mla_merge_kernel)
+  const int64_t q = total / n, r = total - q * n;
+  int64_t acc = (static_cast<int64_t>(t_first) * r) % n;
+  const int slot_first = team_start(t_first, total, n) < first ? 1 : 0;
+  const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 4;
+  const char* tiles = reinterpret_cast<const char*>(a.ws_out) + (hb * 4 + w) * 8192 + lane * 16;
+  float M = kNegBig, W = 0.0f;
+  f32x4 O[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) O[db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int tb = t_first; tb <= t_last; tb += 4) {
+    float lse[4];
+    f32x4 x[4][8];
+    bool on[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = tb + k;
+      acc += r;
+      const int64_t step = q + (acc >= n ? 1 : 0);
+      acc -= acc >= n ? n : 0;
+      on[k] = t <= t_last && step > 0 && head_ok;
+      const int64_t slot = static_cast<int64_t>(t) * 2 + (t == t_first ? slot_first : 0);
+      lse[k] = on[k] ? a.ws_lse[slot * H + hd] : kNegBig;
+#pragma unroll
+      for (int db = 0; db < 8; ++db)
+        x[k][db] = on[k] ? *reinterpret_cast<const f32x4*>(tiles + slot * slot_bytes + db * 1024) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
+    const float keep = fast_exp2(M - m_new);
+    W *= keep;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) O[db] *= keep;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
+      W += e;
+#pragma unroll
+      for (int db = 0; db < 8; ++db) O[db] += e * x[k][db];
+    }
+    M = m_new;
+  }
+  if (!head_ok) return;
+  const float inv = 1.0f / W;
+#pragma unroll
+  for (int db = 0; db < 8; ++db)
+    *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{QT::pack(O[db][0] * inv, O[db][1] * inv), QT::pack(O[db][2] * inv, O[db][3] * inv)};
+  if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * H + hd] = (M + fast_log2(W)) * kLn2;
+}
+
 int mla_cu_count() {
   static const int n = [] {
     int dev = 0;
@@ -2715,7 +2825,9 @@ size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) 
   (void)max_seq_len;
   // the kernel with 128 heads per workgroup has the fewer workgroups per team, hence the more teams
   const int n_hb = static_cast<int>((n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
-  return kWsPartialsOff + static_cast<size_t>(mla_teams(n_hb)) * 2 * n_heads * (kDL + 1) * 4;
+  // (slots of whole 16-head blocks: the kernel with 128 heads per workgroup writes its partial rows as tiles)
+  const size_t slot_heads = static_cast<size_t>((n_heads + 15) / 16 * 16);
+  return kWsPartialsOff + static_cast<size_t>(mla_teams(n_hb)) * 2 * (slot_heads * kDL + n_heads) * 4;
 }
 
 int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out, float* lse,
@@ -2807,7 +2919,9 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.scale_log2 = sm_scale * kLog2e;
     a.ws_prefix = reinterpret_cast<int*>(static_cast<char*>(workspace) + kWsHeaderBytes);
     a.ws_out = reinterpret_cast<float*>(static_cast<char*>(workspace) + kWsPartialsOff);
-    a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * n_heads * kDL;
+    a.slot_heads = static_cast<int>((n_heads + 15) / 16 * 16);
+    a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * a.slot_heads * kDL;
+    const bool w4 = !pairs && !use_p && by_dims && knob != 'n';
 
     const dim3 grid(static_cast<unsigned>(a.n_teams * a.n_hb));
     if (pairs) {
@@ -2815,7 +2929,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       else launch_timed(mla_decode_kernel<BF16>, grid, dim3(kMlaThreads), smem, stream, a);
     } else if (use_p) {
       launch_timed(mla_decode32w_kernel, grid, dim3(kWThreads), kPLdsBytes, stream, a);
-    } else if (by_dims && knob != 'n') {  // ('n'arrow: the kernel with 16 heads per scoring wavefront, 3 % slower on 128 heads)
+    } else if (w4) {  // ('n'arrow: the kernel with 16 heads per scoring wavefront, 3 % slower on 128 heads)
       if (f16) launch_timed(mla_decode_w4_kernel<FP16>, grid, dim3(kW4Threads), kW4LdsBytes, stream, a);
       else launch_timed(mla_decode_w4_kernel<BF16>, grid, dim3(kW4Threads), kW4LdsBytes, stream, a);
     } else if (by_dims) {
@@ -2831,8 +2945,14 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     int rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
     const dim3 mgrid(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb));
-    if (f16) launch_timed(mla_merge_kernel<FP16>, mgrid, dim3(128), 0, stream, a);
-    else launch_timed(mla_merge_kernel<BF16>, mgrid, dim3(128), 0, stream, a);
+    if (w4) {   // (its partial rows are tiles)
+      const dim3 tgrid(static_cast<unsigned>(a.slot_heads / 16), static_cast<unsigned>(nb));
+      if (f16) launch_timed(mla_merge_tiles_kernel<FP16>, tgrid, dim3(256), 0, stream, a);
+      else launch_timed(mla_merge_tiles_kernel<BF16>, tgrid, dim3(256), 0, stream, a);
+    } else {
+      if (f16) launch_timed(mla_merge_kernel<FP16>, mgrid, dim3(128), 0, stream, a);
+      else launch_timed(mla_merge_kernel<BF16>, mgrid, dim3(128), 0, stream, a);
+    }
     rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
   }
