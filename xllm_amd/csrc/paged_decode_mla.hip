@@ -79,6 +79,10 @@ struct MlaArgs {
   int batch;
   int n_heads;
   int slot_heads;  // n_heads rounded up to 16
+  // mla_decode_w4_kernel and mla_merge_tiles_kernel: the schedule counts every context that holds tokens as its tiles
+  // plus this many, in front of them (the start of a run costs a workgroup about as much as four tiles; a range that
+  // holds the start of a context receives that many fewer).  0: the schedule counts tiles only
+  int run_cost;
   int n_hb;        // head blocks of 64 = workgroups per team
   int n_teams;
   int block_size;
@@ -1421,9 +1425,16 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
   const unsigned long long w_entry = wall_clock64();
   unsigned long long tm[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   unsigned long long tk = t_entry;
+#ifdef XLLM_W4_PROLOGUE_TIMING   // (slots 2-6 hold parts of the run prologue instead of the loop's phases)
+#define W4_PTICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; }
+#define W4_TICK(i) { if (i < 2 || i > 6) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; } }
+#else
+#define W4_PTICK(i)
 #define W4_TICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; }
+#endif
 #else
 #define W4_TICK(i)
+#define W4_PTICK(i)
 #endif
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kW4PrefixOff);
@@ -1439,20 +1450,25 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
   const int g = lane >> 4;      // MFMA k-group of the lane
   const int H = a.n_heads;
 
-  // block id -> (team, head block of 128): members of a team are 8 ids apart (same XCD)
+  // block id -> (team, head block of 128): members of a team are 8 ids apart (same XCD: they read the same pages),
+  // and so are consecutive teams: those that share a context read its Q rows from HBM once, then from their L2
+  // (one XCD after the other they fetch them four times over, 38 MB instead of 9 at the start of a launch of 64
+  // contexts)
   const int xcd = blockIdx.x & 7;
   const int y = blockIdx.x >> 3;
   const int hb128 = y % a.n_hb;
-  const int team = (y / a.n_hb) * 8 + xcd;
+  const int team = xcd * (a.n_teams >> 3) + y / a.n_hb;
   const int head0 = hb128 * kHeadsPerWg16;
   const int n16 = min(8, (H - head0 + 15) >> 4);       // 16-head blocks of this workgroup that hold heads
 
-  // ---- tile prefix over the batch (every workgroup computes it; no extra launch)
+  // ---- prefix over the batch of what the schedule divides: tiles, and run_cost more at the front of every context
+  // (every workgroup computes it; no extra launch)
   {
     const int per = (a.batch + kW4Threads - 1) / kW4Threads;
     const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
     int local = 0;
-    for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
+    auto span_of = [&](int len) { return len > 0 ? tiles_of(len) + a.run_cost : 0; };
+    for (int b = lo; b < hi; ++b) local += span_of(a.seq_lens[b]);
     tmp[tid] = local;
     __syncthreads();
     if (lo < hi) {
@@ -1464,7 +1480,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       } else {
         for (int b = lo; b < hi; ++b) {
           prefix[b] = excl;
-          excl += tiles_of(a.seq_lens[b]);
+          excl += span_of(a.seq_lens[b]);
         }
       }
       if (hi == a.batch) prefix[a.batch] = excl;
@@ -1499,11 +1515,13 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       if (prefix[mid] <= cur) lo = mid; else hi = mid;
     }
     const int b = __builtin_amdgcn_readfirstlane(lo);
-    const int n_tiles_seq = prefix[b + 1] - prefix[b];
-    const int tile0 = static_cast<int>(cur - prefix[b]);
-    const int run_tiles = static_cast<int>(min<int64_t>(n_tiles_seq - tile0, end - cur));
+    const int n_tiles_seq = prefix[b + 1] - prefix[b] - a.run_cost;
+    const int64_t piece_end = min<int64_t>(prefix[b + 1], end);
+    const int tile0 = max(0, static_cast<int>(cur - prefix[b]) - a.run_cost);
+    const int run_tiles = max(0, static_cast<int>(piece_end - prefix[b]) - a.run_cost) - tile0;
     const bool complete = tile0 == 0 && run_tiles == n_tiles_seq;
-    cur += run_tiles;
+    cur = piece_end;
+    if (run_tiles <= 0) continue;   // (the range ends inside the allowance in front of this context's tiles)
     const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
     const int L = __builtin_amdgcn_readfirstlane(a.seq_lens[b]);
     const int t_begin = tile0 * kTile;
@@ -1526,22 +1544,37 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     const int lane_p = lane_again();
     const int c16p = lane_p & 15, gp = lane_p >> 4;
     if (wave == 0 && lane_p < 3) flags[lane_p] = 0;
+    W4_PTICK(2)   // search, barrier, chunk loads issued
 
     // Q^T operands of the two 16-head blocks: lane (head c16, k-group g) keeps dims kk*32 + g*8 .. +8 of every k-step
     u32x4 q[2][kKSteps32];
+    auto load_q = [&]() {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int head = head0 + wave * 32 + j * 16 + c16p;
-      const char* qn = a.q_nope + (static_cast<int64_t>(b) * H + head) * kDL * 2;
-      const char* qp = a.q_pe + (static_cast<int64_t>(b) * H + head) * kDR * 2;
+#if defined(XLLM_W4_WHATIF_Q) && XLLM_W4_WHATIF_Q == 2
+      const int bq = 0;
+#else
+      const int bq = b;
+#endif
+      const char* qn = a.q_nope + (static_cast<int64_t>(bq) * H + head) * kDL * 2;
+      const char* qp = a.q_pe + (static_cast<int64_t>(bq) * H + head) * kDR * 2;
 #pragma unroll
       for (int kk = 0; kk < kKSteps32; ++kk) {
         u32x4 x = {0u, 0u, 0u, 0u};
+#if defined(XLLM_W4_WHATIF_Q) && XLLM_W4_WHATIF_Q == 1
+        if (head < H && kk == 0)
+#else
         if (head < H)
+#endif
           x = kk < kDL / 32 ? ldg16(qn + (kk * 32 + gp * 8) * 2) : ldg16(qp + ((kk - kDL / 32) * 32 + gp * 8) * 2);
         q[j][kk] = x;
       }
     }
+    };
+#ifndef XLLM_W4_TILES_FIRST
+    load_q();
+#endif
     // O^T blocks of the wavefront's 128 dims in the accumulation registers: block (db, hb) = dims 128 wave + 16 db
     // + 4g + r, head 16 hb + c16
     {
@@ -1880,6 +1913,23 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       pb[1] = *reinterpret_cast<const u32x4*>(pbase + 1024);
     };
 
+#ifdef XLLM_W4_TILES_FIRST
+    W4_PTICK(3)   // accumulators cleared
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    W4_PTICK(4)   // chunks landed, barrier
+    for (int sub = 0; sub < kDsRing && sub < n_sub; ++sub) issue_sub(sub);
+    W4_PTICK(5)   // three sub-tiles issued
+    load_q();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int kk = 0; kk < kKSteps32; ++kk) asm volatile("" : "+v"(q[j][kk]));
+    __syncthreads();
+    W4_PTICK(6)   // Q and sub-tiles landed, barrier
+#else
+    W4_PTICK(3)   // Q loads issued, accumulators cleared
     // the chunk loads and the Q loads have landed (one wait for both latencies)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
@@ -1887,9 +1937,13 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps32; ++kk) asm volatile("" : "+v"(q[j][kk]));
     __syncthreads();
+    W4_PTICK(4)   // Q and chunks landed, barrier
     for (int sub = 0; sub < kDsRing && sub < n_sub; ++sub) issue_sub(sub);
+    W4_PTICK(5)   // three sub-tiles issued
     wait_sent(min(kDsRing - 1, n_sub - 1));
     __syncthreads();
+    W4_PTICK(6)   // first sub-tile landed, barrier
+#endif
     u32x4 vt[8];  // V^T operands of the sub-tile whose P.V comes next: dims 128 wave + 16 db .., its 32 tokens
     {
       f32x4 s[2][2];
@@ -2057,6 +2111,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
   }
 #endif
 #undef W4_TICK
+#undef W4_PTICK
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2717,7 +2772,9 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)   // (measurement build only) when the merge kernel starts
     reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H)[2048 * 10] = wall_clock64();
 #endif
-  const int64_t first = a.ws_prefix[b];
+  // (a context's share of what the schedule divides: run_cost, then its tiles)
+  const int64_t front = a.ws_prefix[b];
+  const int64_t first = front + a.run_cost;
   const int64_t last = static_cast<int64_t>(a.ws_prefix[b + 1]) - 1;
   const int64_t total = a.ws_prefix[a.batch];
   char* out = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + w * 128 + 4 * g) * 2;
@@ -2736,7 +2793,8 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
   // (team ranges stepped as in mla_merge_kernel)
   const int64_t q = total / n, r = total - q * n;
   int64_t acc = (static_cast<int64_t>(t_first) * r) % n;
-  const int slot_first = team_start(t_first, total, n) < first ? 1 : 0;
+  // (a range that starts in front of the context holds the last tile of an earlier one)
+  const int slot_first = team_start(t_first, total, n) < front ? 1 : 0;
   const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 4;
   const char* tiles = reinterpret_cast<const char*>(a.ws_out) + (hb * 4 + w) * 8192 + lane * 16;
   float M = kNegBig, W = 0.0f;
@@ -2922,6 +2980,12 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.slot_heads = static_cast<int>((n_heads + 15) / 16 * 16);
     a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * a.slot_heads * kDL;
     const bool w4 = !pairs && !use_p && by_dims && knob != 'n';
+    static const int run_cost = [] {
+      const char* e = getenv("XLLM_MI355_MLA_RUN_COST");  // tuning knob: tiles charged for the start of a run
+      const int v = e ? atoi(e) : -1;
+      return v >= 0 && v <= 64 ? v : 4;
+    }();
+    a.run_cost = w4 ? run_cost : 0;
 
     const dim3 grid(static_cast<unsigned>(a.n_teams * a.n_hb));
     if (pairs) {
