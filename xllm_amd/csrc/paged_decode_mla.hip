@@ -1410,7 +1410,16 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
 #define XLLM_W4_ROW7(F) F(0, 7, 224, 225, 226, 227) F(1, 7, 228, 229, 230, 231) F(2, 7, 232, 233, 234, 235) F(3, 7, 236, 237, 238, 239) F(4, 7, 240, 241, 242, 243) F(5, 7, 244, 245, 246, 247) F(6, 7, 248, 249, 250, 251) F(7, 7, 252, 253, 254, 255)
 #define XLLM_W4_ALL(F) XLLM_W4_ROW0(F) XLLM_W4_ROW1(F) XLLM_W4_ROW2(F) XLLM_W4_ROW3(F) XLLM_W4_ROW4(F) XLLM_W4_ROW5(F) XLLM_W4_ROW6(F) XLLM_W4_ROW7(F)
 constexpr int kW4Threads = 256;
-constexpr int kW4PrefixOff = kDsPageOff + 2 * kWave * 4;
+// At the start of a run the Q rows of the 128 heads pass through the ring and the P^T area on their way into the
+// registers: latent parts at a pitch of 1040 bytes (16 lanes that read 16 bytes of 16 rows hit 64 different banks),
+// then the rope parts.  The small arrays sit behind them.
+constexpr int kW4QRow = kDL * 2 + 16;
+constexpr int kW4QRopeOff = kHeadsPerWg16 * kW4QRow;
+constexpr int kW4QEnd = kW4QRopeOff + kHeadsPerWg16 * kDR * 2;
+constexpr int kW4FacOff = kW4QEnd > kDsPOff + 2 * 8 * 1024 ? kW4QEnd : kDsPOff + 2 * 8 * 1024;   // as kDsFacOff
+constexpr int kW4FlagOff = kW4FacOff + 2 * kHeadsPerWg16 * 4;
+constexpr int kW4PageOff = kW4FlagOff + 16;
+constexpr int kW4PrefixOff = kW4PageOff + 2 * kWave * 4;
 constexpr int kW4LdsBytes = kW4PrefixOff + (kMaxBatchMla + 1) * 4;
 constexpr int kW4Loads = 9;   // loads a wavefront sends for a sub-tile: 8 rows and their rope parts
 static_assert(kW4LdsBytes <= 160 * 1024, "LDS of a CU");
@@ -1438,9 +1447,9 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
 #endif
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kW4PrefixOff);
-  const int* pagebuf = reinterpret_cast<const int*>(smem + kDsPageOff);
-  float* fac = reinterpret_cast<float*>(smem + kDsFacOff);
-  int* flags = reinterpret_cast<int*>(smem + kDsFlagOff);
+  const int* pagebuf = reinterpret_cast<const int*>(smem + kW4PageOff);
+  float* fac = reinterpret_cast<float*>(smem + kW4FacOff);
+  int* flags = reinterpret_cast<int*>(smem + kW4FlagOff);
   int* tmp = reinterpret_cast<int*>(smem);  // prologue only
 
   const int tid = threadIdx.x;
@@ -1496,7 +1505,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
   bool first_run = true;
 
   const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
-  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + kDsPageOff);
+  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + kW4PageOff);
   // per-lane constants of the operand reads (byte offsets inside a sub-tile), as in mla_decode16_kernel
   const int k_row0 = c16 * kRow16 + ((g ^ ((c16 >> 2) & 1)) * 16);
   const int v_row0 = (4 * g + (c16 >> 2)) * kRow16 + ((((c16 & 3) >> 1) ^ (g & 1)) * 16) + (c16 & 1) * 8 + wave * (8 * 32);
@@ -1546,35 +1555,28 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     if (wave == 0 && lane_p < 3) flags[lane_p] = 0;
     W4_PTICK(2)   // search, barrier, chunk loads issued
 
-    // Q^T operands of the two 16-head blocks: lane (head c16, k-group g) keeps dims kk*32 + g*8 .. +8 of every k-step
+    // Q^T operands of the two 16-head blocks: lane (head c16, k-group g) keeps dims kk*32 + g*8 .. +8 of every k-step.
+    // The rows of the wavefront's 32 heads travel through LDS, 36 loads of 1 KB (whole rows) and then 72 LDS reads per
+    // lane.  Gathered from memory by the lanes of that layout the same bytes take 72 loads that touch 16 rows each,
+    // and the four wavefronts keep the CU's address unit busy with them for 10 000 cycles.
     u32x4 q[2][kKSteps32];
-    auto load_q = [&]() {
+    {
+      const int head_w = head0 + wave * 32;
+#pragma unroll 4
+      for (int i = 0; i < 32; ++i) {   // (rows of heads beyond the last one: that one's again; their results go nowhere)
+        const int head = min(head_w + i, H - 1);
+        const uint64_t row = reinterpret_cast<uint64_t>(a.q_nope) + (static_cast<uint64_t>(b) * H + head) * (kDL * 2);
+        const u32 dst = __builtin_amdgcn_readfirstlane(lds_base + (wave * 32 + i) * kW4QRow);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(row) : "memory");
+      }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int head = head0 + wave * 32 + j * 16 + c16p;
-#if defined(XLLM_W4_WHATIF_Q) && XLLM_W4_WHATIF_Q == 2
-      const int bq = 0;
-#else
-      const int bq = b;
-#endif
-      const char* qn = a.q_nope + (static_cast<int64_t>(bq) * H + head) * kDL * 2;
-      const char* qp = a.q_pe + (static_cast<int64_t>(bq) * H + head) * kDR * 2;
-#pragma unroll
-      for (int kk = 0; kk < kKSteps32; ++kk) {
-        u32x4 x = {0u, 0u, 0u, 0u};
-#if defined(XLLM_W4_WHATIF_Q) && XLLM_W4_WHATIF_Q == 1
-        if (head < H && kk == 0)
-#else
-        if (head < H)
-#endif
-          x = kk < kDL / 32 ? ldg16(qn + (kk * 32 + gp * 8) * 2) : ldg16(qp + ((kk - kDL / 32) * 32 + gp * 8) * 2);
-        q[j][kk] = x;
+      for (int i = 0; i < 4; ++i) {    // rope parts, eight heads per load: lane -> head 8 i + lane / 8, piece lane % 8
+        const int head = min(head_w + 8 * i + (lane_p >> 3), H - 1);
+        const char* src = a.q_pe + (static_cast<int64_t>(b) * H + head) * (kDR * 2) + (lane_p & 7) * 16;
+        const u32 dst = __builtin_amdgcn_readfirstlane(lds_base + kW4QRopeOff + (wave * 32 + 8 * i) * (kDR * 2));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src) : "memory");
       }
     }
-    };
-#ifndef XLLM_W4_TILES_FIRST
-    load_q();
-#endif
     // O^T blocks of the wavefront's 128 dims in the accumulation registers: block (db, hb) = dims 128 wave + 16 db
     // + 4g + r, head 16 hb + c16
     {
@@ -1832,7 +1834,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       // the head blocks whose maxima moved in this sub-tile: read behind the two blocks, so that one trip to LDS
       // covers all three (read as LDS on purpose: a generic volatile pointer becomes a flat load, whose wait drains
       // the tile loads in flight)
-      return __builtin_amdgcn_readfirstlane(*((lds_vint*)(smem + kDsFlagOff) + sub % 3));
+      return __builtin_amdgcn_readfirstlane(*((lds_vint*)(smem + kW4FlagOff) + sub % 3));
     };
     // Rows FIRST .. LAST - 1 (head blocks) of one half of the wavefront's dims (HALF 0: dim blocks 0-3, with the
     // tile loads of a later sub-tile, one per row; HALF 1: dim blocks 4-7).  MODE says what rides in the shadow of
@@ -1913,37 +1915,25 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       pb[1] = *reinterpret_cast<const u32x4*>(pbase + 1024);
     };
 
-#ifdef XLLM_W4_TILES_FIRST
-    W4_PTICK(3)   // accumulators cleared
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    W4_PTICK(4)   // chunks landed, barrier
-    for (int sub = 0; sub < kDsRing && sub < n_sub; ++sub) issue_sub(sub);
-    W4_PTICK(5)   // three sub-tiles issued
-    load_q();
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int kk = 0; kk < kKSteps32; ++kk) asm volatile("" : "+v"(q[j][kk]));
-    __syncthreads();
-    W4_PTICK(6)   // Q and sub-tiles landed, barrier
-#else
     W4_PTICK(3)   // Q loads issued, accumulators cleared
-    // the chunk loads and the Q loads have landed (one wait for both latencies)
+    // the chunk loads and the Q rows have landed (one wait for both latencies); the wavefront reads the rows it sent
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < 2; ++j) {
+      const char* qrow = smem + (wave * 32 + j * 16 + c16p) * kW4QRow + gp * 16;
+      const char* qrope = smem + kW4QRopeOff + (wave * 32 + j * 16 + c16p) * (kDR * 2) + gp * 16;
 #pragma unroll
-      for (int kk = 0; kk < kKSteps32; ++kk) asm volatile("" : "+v"(q[j][kk]));
-    __syncthreads();
+      for (int kk = 0; kk < kKSteps32; ++kk)
+        q[j][kk] = kk < kDL / 32 ? *reinterpret_cast<const u32x4*>(qrow + kk * 64)
+                                 : *reinterpret_cast<const u32x4*>(qrope + (kk - kDL / 32) * 64);
+    }
+    __syncthreads();   // (the ring is free for the first sub-tiles)
     W4_PTICK(4)   // Q and chunks landed, barrier
     for (int sub = 0; sub < kDsRing && sub < n_sub; ++sub) issue_sub(sub);
     W4_PTICK(5)   // three sub-tiles issued
     wait_sent(min(kDsRing - 1, n_sub - 1));
     __syncthreads();
     W4_PTICK(6)   // first sub-tile landed, barrier
-#endif
     u32x4 vt[8];  // V^T operands of the sub-tile whose P.V comes next: dims 128 wave + 16 db .., its 32 tokens
     {
       f32x4 s[2][2];
