@@ -167,6 +167,14 @@ def test_other_kernels_for_more_than_64_heads(device):
             _select_kernel("")
 
 
+def test_head_counts_that_do_not_fill_their_blocks(device):
+    # more than 64 heads, not a multiple of 16 nor of 128: the last 16-head block of the partial tiles is part
+    # empty, the second workgroup of a team holds 72 heads; contexts long enough to be cut into partial runs
+    _check(_mla_cfg("mla100", 2, 100, 2000, 5000), 31, device)
+    _check(_mla_cfg("mla200", 2, 200, 1, 3000), 32, device)
+    _check(_mla_cfg("mla72_many", 70, 72, 1, 300), 33, device)
+
+
 def test_many_short_sequences_with_128_heads(device):
     # more sequences than workgroups: a workgroup meets several contexts in one launch (whole ones written
     # directly, the pieces at both ends of its range as partials), and a batch beyond what one launch holds;
