@@ -247,6 +247,20 @@ def test_fp8_kv_cache_decode(device):
     _check_fp8(cfg, 4242, device)
 
 
+def test_kv_head_counts_and_the_heads_read_side_by_side(device):
+    # The four workers of a workgroup read four adjacent KV heads side by side when the KV heads come in fours
+    # (12 = three groups), two when they come in pairs (6, 2), one otherwise (3, 1); contexts long enough to be cut
+    # into partial runs, and many short ones, so that the merge finds every head block's partials with the right
+    # member of every workgroup.
+    for Hq, Hkv in ((24, 12), (12, 6), (6, 3), (48, 12), (4, 2), (7, 1)):
+        cfg = workloads.DecodeConfig(f"lock_h{Hq}_{Hkv}", 6, Hq, Hkv, 128, 16, 900, 5000)
+        _check_config(cfg, 700 + Hq + Hkv, device)
+        cfg = workloads.DecodeConfig(f"lock_short_h{Hq}_{Hkv}", 200, Hq, Hkv, 128, 16, 1, 120)
+        _check_config(cfg, 800 + Hq + Hkv, device)
+    cfg = workloads.DecodeConfig("lock_fp8_h24_12", 6, 24, 12, 128, 16, 900, 5000, cache_dtype="fp8")
+    _check_fp8(cfg, 901, device)
+
+
 def test_whole_contexts_in_one_workgroup_every_group_size(device):
     # Few short sequences: every context is a single item, so one workgroup sees it whole and
     # writes the caller's output itself (no partials, no merge), with most wavefronts idle.
