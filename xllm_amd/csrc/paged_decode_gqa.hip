@@ -126,11 +126,18 @@ __device__ __forceinline__ int items_of(const GqaArgs& a, int L) {
 }
 
 // First flat item of workgroup w when `total` items are dealt to `n` workgroups.
-__device__ __forceinline__ int64_t range_start(int64_t w, int64_t total, int64_t n) { return w * total / n; }
+// (a 64-bit division is a long instruction sequence on this GPU, and these sit on the dependent chains at the start
+// of the decode and merge kernels: 32 bits whenever the products fit, which they do unless a batch holds more than a
+// million items)
+__device__ __forceinline__ int64_t range_start(int64_t w, int64_t total, int64_t n) {
+  if (total * n < (1LL << 31)) return static_cast<uint32_t>(w) * static_cast<uint32_t>(total) / static_cast<uint32_t>(n);
+  return w * total / n;
+}
 
 // The workgroup whose range holds flat item `id`.
 __device__ __forceinline__ int workgroup_of(int64_t id, int64_t total, int64_t n) {
-  int64_t w = id * n / total;
+  int64_t w = total * n < (1LL << 31) ? static_cast<int64_t>(static_cast<uint32_t>(id) * static_cast<uint32_t>(n) / static_cast<uint32_t>(total))
+                                      : id * n / total;
   while (w + 1 < n && range_start(w + 1, total, n) <= id) ++w;
   return static_cast<int>(w);
 }
@@ -1497,8 +1504,10 @@ __device__ __forceinline__ void merge_context(const GqaArgs& a, int dv, int hbk,
   if (w_first == w_last) return;  // one worker saw the whole context and wrote the output
   // range_start(w) = w * q + floor(w * r / n) with total = q * n + r: stepped from w to w + 1
   // without a division
-  const int64_t q = total / n, r = total - q * n;
-  const int64_t acc0 = (static_cast<int64_t>(w_first) * r) % n;
+  const bool fits32 = total * n < (1LL << 31);
+  const int64_t q = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(total) / static_cast<uint32_t>(n)) : total / n, r = total - q * n;
+  const int64_t acc0 = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(w_first) * static_cast<uint32_t>(r) % static_cast<uint32_t>(n))
+                              : (static_cast<int64_t>(w_first) * r) % n;
   // the first worker holds this context as its last run (slot 1) unless its range starts
   // exactly here; every later one holds it as its first run (slot 0)
   const int slot_first = range_start(w_first, total, n) < first ? 1 : 0;

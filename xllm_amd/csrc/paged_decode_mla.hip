@@ -92,9 +92,15 @@ struct MlaArgs {
 };
 
 __device__ __forceinline__ int tiles_of(int L) { return L > 0 ? (L + kTile - 1) / kTile : 0; }
-__device__ __forceinline__ int64_t team_start(int64_t t, int64_t total, int64_t n) { return t * total / n; }
+// (32-bit divisions whenever the products fit: a 64-bit one is a long instruction sequence, and these sit on the
+// dependent chains at the start of the decode and merge kernels)
+__device__ __forceinline__ int64_t team_start(int64_t t, int64_t total, int64_t n) {
+  if (total * n < (1LL << 31)) return static_cast<uint32_t>(t) * static_cast<uint32_t>(total) / static_cast<uint32_t>(n);
+  return t * total / n;
+}
 __device__ __forceinline__ int team_of(int64_t id, int64_t total, int64_t n) {
-  int64_t t = id * n / total;
+  int64_t t = total * n < (1LL << 31) ? static_cast<int64_t>(static_cast<uint32_t>(id) * static_cast<uint32_t>(n) / static_cast<uint32_t>(total))
+                                      : id * n / total;
   while (t + 1 < n && team_start(t + 1, total, n) <= id) ++t;
   return static_cast<int>(t);
 }
@@ -2704,8 +2710,10 @@ __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
   const int t_last = team_of(last, total, n);
   if (t_first == t_last) return;  // one team saw the whole context and wrote the output
   // team_start(t) = t * q + floor(t * r / n) with total = q * n + r: stepped without a division
-  const int64_t q = total / n, r = total - q * n;
-  int64_t acc = (static_cast<int64_t>(t_first) * r) % n;
+  const bool fits32 = total * n < (1LL << 31);
+  const int64_t q = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(total) / static_cast<uint32_t>(n)) : total / n, r = total - q * n;
+  int64_t acc = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(t_first) * static_cast<uint32_t>(r) % static_cast<uint32_t>(n))
+                       : (static_cast<int64_t>(t_first) * r) % n;
   // the first team holds this context as its last run (slot 1) unless its range starts exactly
   // here; every later one holds it as its first run (slot 0)
   const int slot_first = team_start(t_first, total, n) < first ? 1 : 0;
@@ -2781,8 +2789,10 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
   const int t_last = team_of(last, total, n);
   if (t_first == t_last) return;  // one team saw the whole context and wrote the output
   // (team ranges stepped as in mla_merge_kernel)
-  const int64_t q = total / n, r = total - q * n;
-  int64_t acc = (static_cast<int64_t>(t_first) * r) % n;
+  const bool fits32 = total * n < (1LL << 31);
+  const int64_t q = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(total) / static_cast<uint32_t>(n)) : total / n, r = total - q * n;
+  int64_t acc = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(t_first) * static_cast<uint32_t>(r) % static_cast<uint32_t>(n))
+                       : (static_cast<int64_t>(t_first) * r) % n;
   // (a range that starts in front of the context holds the last tile of an earlier one)
   const int slot_first = team_start(t_first, total, n) < front ? 1 : 0;
   const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 4;
