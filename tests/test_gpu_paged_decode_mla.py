@@ -175,6 +175,34 @@ def test_head_counts_that_do_not_fill_their_blocks(device):
     _check(_mla_cfg("mla72_many", 70, 72, 1, 300), 33, device)
 
 
+def test_random_batches_with_empty_sequences_on_the_default_kernel(device):
+    # Random batch sizes, head counts and length ranges; some sequences emptied (length 0: the output row is zero and
+    # the LSE -inf, and the schedule gives them no share).  The oracle takes non-empty sequences, so the emptied rows
+    # are checked by themselves and the others against a decode of the same batch without them.
+    g = torch.Generator().manual_seed(2025)
+    for case in range(6):
+        batch = int(torch.randint(1, 90, (1,), generator=g))
+        heads = (128, 96, 160, 256, 72, 112)[case]
+        lo = int(torch.randint(1, 300, (1,), generator=g))
+        hi = lo + int(torch.randint(1, 2000, (1,), generator=g))
+        cfg = _mla_cfg(f"rand{case}_b{batch}_h{heads}", batch, heads, lo, hi)
+        inp, kg, out, lse = _check(cfg, 1000 + case, device)
+        lens = inp.layout.seq_lens.clone()
+        empty = torch.rand(batch, generator=g) < 0.3
+        if not bool(empty.any()):
+            empty[0] = True
+        lens[empty] = 0
+        if int(lens.max()) == 0:
+            continue
+        out2, lse2 = _decode_gpu(inp, kg, device, seq_lens=lens)
+        keep = ~empty
+        assert torch.equal(out2[empty].cpu(), torch.zeros_like(out2[empty].cpu()))
+        assert bool(torch.isinf(lse2[empty]).all()) and bool((lse2[empty] < 0).all())
+        # the other rows: the same contexts, cut at other places by the schedule (fewer tiles to deal out)
+        assert torch.allclose(out2[keep].float().cpu(), out[keep].float().cpu(), atol=2e-2)
+        assert torch.allclose(lse2[keep].cpu(), lse[keep].cpu(), rtol=1e-3, atol=1e-3)
+
+
 def test_many_short_sequences_with_128_heads(device):
     # more sequences than workgroups: a workgroup meets several contexts in one launch (whole ones written
     # directly, the pieces at both ends of its range as partials), and a batch beyond what one launch holds;
