@@ -91,7 +91,7 @@ struct GqaArgs {
   int n_workgroups;   // workers of the decode kernel (workgroups; wavefront pairs of the matrix-core kernel)
   // Matrix-core kernel: this many workers of a workgroup (1, 2 or 4) walk the same stages of adjacent head blocks
   // side by side, so that the rows they ask for at the same time are neighbours in memory (a token's rows of all KV
-  // heads are contiguous in a page).  A plain streaming kernel reads 128-byte pieces that lie 1 KB apart at 5.8 TB/s
+  // heads are contiguous in a page), or the same rows (head blocks of one KV head).  A plain streaming kernel reads 128-byte pieces that lie 1 KB apart at 5.8 TB/s
   // when the neighbouring pieces are fetched at other times by other workgroups, at 6.7 TB/s when two wavefronts of a
   // workgroup fetch adjacent pieces together (the rate of 256-byte pieces) and at 7.0 TB/s with four.  The flat list
   // then holds (sequence, group of head blocks, stage) and is dealt to groups of workers.  The workers of a group
@@ -1654,12 +1654,17 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
   a.ws_arrivals = reinterpret_cast<unsigned*>(reinterpret_cast<char*>(a.ws_status) + kWsCountersOff);
   a.fold_merge = !VL && a.n_workgroups <= kWsMaxWorkers && fold_merge_enabled() ? 1 : 0;
-  // adjacent KV heads side by side (one head block per KV head; the in-kernel merge keeps its own bookkeeping per worker)
+  // Adjacent head blocks side by side: adjacent KV heads when a KV head has one head block; with several (more than
+  // 16 query heads per KV head, or packed query chunks of more than 16 / group tokens) the blocks of one KV head, which
+  // read the same rows, so that all but the first find them in L2.  (The in-kernel merge keeps its own bookkeeping
+  // per worker.)
   a.head_lock = 1;
-  if (!VL && a.fold_merge == 0 && a.group <= kMfmaHeads) {
+  if (a.fold_merge == 0) {
+    const int hb_per_kv = VL ? a.chunk_blocks : (a.group + kMfmaHeads - 1) / kMfmaHeads;
+    const int n_hb = a.n_kv_heads * hb_per_kv;
     const int want = head_lock_knob();
     for (int hl = kWaves; hl > 1; hl >>= 1)
-      if (hl <= want && a.n_kv_heads % hl == 0 && kWaves % hl == 0) {
+      if (hl <= want && n_hb % hl == 0 && kWaves % hl == 0) {
         a.head_lock = hl;
         break;
       }
