@@ -297,6 +297,39 @@ def test_block_sizes_and_page_table_chunks_of_both_kernels(device):
     _check_config(cfg, 900, device)
 
 
+def test_random_shapes_with_empty_sequences(device):
+    # Random head counts, block sizes, batch sizes and length ranges on the matrix-core kernel, each decoded a second
+    # time with some sequences emptied: their rows are zero with an LSE of -inf, the others agree with the first
+    # decode (the same contexts, cut at other places because fewer stages are dealt out).
+    g = torch.Generator().manual_seed(77)
+    shapes = ((32, 8, 128), (16, 4, 128), (24, 12, 128), (12, 6, 64), (40, 2, 128), (8, 8, 128), (9, 3, 128), (16, 4, 256))
+    for case, (Hq, Hkv, D) in enumerate(shapes):
+        batch = int(torch.randint(1, 150, (1,), generator=g))
+        bs = (16, 32, 64, 128)[int(torch.randint(0, 4, (1,), generator=g))]
+        lo = int(torch.randint(1, 200, (1,), generator=g))
+        hi = lo + int(torch.randint(1, 1500, (1,), generator=g))
+        cfg = workloads.DecodeConfig(f"rand{case}_h{Hq}_{Hkv}_d{D}_b{batch}_bs{bs}", batch, Hq, Hkv, D, bs, lo, hi)
+        _check_config(cfg, 1100 + case, device)
+        inp = workloads.make_inputs(cfg, 1100 + case)
+        lay = inp.layout
+        kg, vg, _, _ = fill_caches_gpu(inp, device)
+        out, lse = _decode_gpu(inp, kg, vg, device)
+        lens = lay.seq_lens.clone()
+        empty = torch.rand(batch, generator=g) < 0.3
+        empty[int(torch.randint(0, batch, (1,), generator=g))] = True
+        lens[empty] = 0
+        q = inp.q.to(device)
+        out2 = torch.full_like(q, 7.0)
+        out2, lse2 = ops.batch_decode(q, kg, out2, lay.block_table.to(device), lens.to(device), v_cache=vg,
+                                      scale=cfg.scale, return_lse=True)
+        torch.cuda.synchronize()
+        assert (out2[empty] == 0).all() and torch.isneginf(lse2[empty]).all()
+        keep = ~empty
+        if bool(keep.any()):
+            assert torch.allclose(out2[keep].float().cpu(), out[keep].float().cpu(), atol=2e-2)
+            assert torch.allclose(lse2[keep].cpu().view(-1), lse[keep].cpu().view(-1), rtol=1e-3, atol=1e-3)
+
+
 def test_empty_sequence_and_argument_errors(device):
     cfg = workloads.DecodeConfig("e", 3, 8, 2, 128, 16, 10, 50)
     inp = workloads.make_inputs(cfg, 2)
