@@ -98,6 +98,11 @@ struct GqaArgs {
   // start together and are left to themselves: made to wait for each other (stage i only after all have issued stage
   // i - 1, or i - 3, or i - 9) they were 1-2 % slower than free, which is 2-5 % faster than apart.
   int head_lock;
+  // Matrix-core kernel: the flat list is cut in two, in the ratio pool_even : pool_odd, and the first part dealt to
+  // the groups of workers on XCDs 0, 2, 4, 6, the second to those on XCDs 1, 3, 5, 7 (workgroup i runs on XCD i % 8).
+  // With equal shares the workgroups on the odd XCDs stream their rows 8-11 % slower and end a launch that much later
+  // (every MI355X measured, five of them); 9 : 8 ends the decode kernels 1.7-2.7 % earlier.  0 : 0 = one list.
+  int pool_even, pool_odd;
   int wait_spins;     // bound of the polls of one wavefront of a pair on the other
   int window_left;    // sliding window: the query (position L - 1) attends to positions >= L - 1 - window_left; < 0: all
   float scale_log2;   // sm_scale * log2(e)
@@ -134,12 +139,46 @@ __device__ __forceinline__ int64_t range_start(int64_t w, int64_t total, int64_t
   return w * total / n;
 }
 
+// With fewer items than workers only the first `total` workers take part (one item each): no range in the middle of
+// the list is ever empty, and the merge need not ask which ones are.
+__device__ __forceinline__ int64_t used_workers(int64_t n, int64_t total) { return total < n ? total : n; }
+
 // The workgroup whose range holds flat item `id`.
 __device__ __forceinline__ int workgroup_of(int64_t id, int64_t total, int64_t n) {
   int64_t w = total * n < (1LL << 31) ? static_cast<int64_t>(static_cast<uint32_t>(id) * static_cast<uint32_t>(n) / static_cast<uint32_t>(total))
                                       : id * n / total;
   while (w + 1 < n && range_start(w + 1, total, n) <= id) ++w;
   return static_cast<int>(w);
+}
+
+// The two pools of GqaArgs::pool_even / pool_odd.  Groups of workers ("teams", `per` of them in a workgroup) are
+// numbered pool by pool: index q of pool `par` (0: even XCDs, 1: odd XCDs) <-> team of_pool(par, q).
+struct Pools {
+  int64_t total, cut;  // the flat list and where the second pool's part begins
+  int half, per_shift; // teams per pool; log2 of the teams per workgroup (1, 2 or 4 of them)
+  __device__ __forceinline__ int64_t size(int par) const { return par ? total - cut : cut; }
+  __device__ __forceinline__ int64_t base(int par) const { return par ? cut : 0; }
+  __device__ __forceinline__ int of_pool(int par, int q) const {
+    const int r = q >> per_shift, o = q - (r << per_shift);
+    return (((r >> 2) * 8 + (r & 3) * 2 + par) << per_shift) + o;
+  }
+  __device__ __forceinline__ void of_team(int team, int& par, int& q) const {
+    const int g = team >> per_shift, o = team - (g << per_shift), xcd = g & 7;
+    par = xcd & 1;
+    q = (((g >> 3) * 4 + (xcd >> 1)) << per_shift) + o;
+  }
+};
+__device__ __forceinline__ int64_t pool_cut(const GqaArgs& a, int64_t total) {
+  return total * a.pool_even / (a.pool_even + a.pool_odd);
+}
+// (the merge kernel takes the cut that the decode kernel left behind the item prefix: no division there)
+__device__ __forceinline__ Pools make_pools(const GqaArgs& a, int64_t total, int64_t cut) {
+  Pools p;
+  p.total = total;
+  p.cut = cut;
+  p.per_shift = a.head_lock == 4 ? 0 : a.head_lock == 2 ? 1 : 2;   // (kWaves = 4 workers in a workgroup)
+  p.half = a.n_workgroups / a.head_lock / 2;
+  return p;
 }
 
 // Exclusive prefix sum of the per-sequence item counts into prefix[0..batch] (LDS).
@@ -252,7 +291,8 @@ __global__ __launch_bounds__(kThreads) void gqa_decode_kernel(GqaArgs a) {
     for (int i = tid; i <= a.batch; i += kThreads) a.ws_prefix[i] = prefix[i];
   }
   if (total == 0) return;
-  const int64_t n_wg = gridDim.x;
+  const int64_t n_wg = used_workers(gridDim.x, total);
+  if (blockIdx.x >= n_wg) return;
   int64_t cur = range_start(blockIdx.x, total, n_wg);
   const int64_t end = range_start(blockIdx.x + 1, total, n_wg);
   bool first_run = true;
@@ -669,7 +709,7 @@ constexpr int kMfmaThreads = 2 * kThreads;   // kWaves loading wavefronts and kW
 
 template <typename QT, bool VL, bool COHERENT = false>
 __device__ __forceinline__ void merge_context(const GqaArgs& a, int dv, int hbk, int b, int tid, int nthreads,
-                                              int p0, int p1, int pt);
+                                              int p0, int p1, int pt, int cut = 0);
 // Words of the partials that workers exchange inside one launch: relaxed atomics at device scope, which go to
 // the level of the memory system that all CUs share (the L2 of an XCD is not coherent with the other seven; a
 // fence that makes it so writes back and invalidates the whole L2, 60 us per launch when 1024 workers do it).
@@ -779,6 +819,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hbl;
   if (blockIdx.x == 0) {
     for (int i = tid; i <= a.batch; i += kMfmaThreads) a.ws_prefix[i] = prefix[i];
+    if (tid == 0 && a.pool_even != 0) a.ws_prefix[a.batch + 1] = static_cast<int>(pool_cut(a, total));
   }
   auto sequence_at = [&](int b, const int32_t*& pages, int& L) {
     if (lens_in_lds) {
@@ -803,8 +844,21 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   const int64_t n_workers = static_cast<int64_t>(gridDim.x) * kWaves / HL;   // groups of HL workers share a range
   const int64_t team = worker / HL;
   const int member = pair % HL;        // head block member + HL * (group of head blocks)
-  const int64_t cur = range_start(team, total, n_workers);
-  const int64_t end = range_start(team + 1, total, n_workers);
+  int64_t cur, end;
+  if (a.pool_even != 0) {   // the list in two parts: one for the teams on even XCDs, one for those on odd XCDs
+    const Pools pools = make_pools(a, total, pool_cut(a, total));
+    int par, q;
+    pools.of_team(static_cast<int>(team), par, q);
+    const int64_t n_use = used_workers(pools.half, pools.size(par));
+    if (q >= n_use) return;
+    cur = pools.base(par) + range_start(q, pools.size(par), n_use);
+    end = pools.base(par) + range_start(q + 1, pools.size(par), n_use);
+  } else {
+    const int64_t n_use = used_workers(n_workers, total);
+    if (team >= n_use) return;
+    cur = range_start(team, total, n_use);
+    end = range_start(team + 1, total, n_use);
+  }
   if (cur >= end) return;
   const int n_stages = static_cast<int>(end - cur);
   lds_vint* landed = sync + 2 * pair;
@@ -1416,13 +1470,9 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         const int n_items = p1 - p0;
         const int64_t first = static_cast<int64_t>(p0) * n_hb + static_cast<int64_t>(hbk) * n_items;
         const int64_t last = first + n_items - 1;
-        const int w_first = workgroup_of(first, total, n_workers), w_last = workgroup_of(last, total, n_workers);
-        int pieces = 0;  // workers of w_first .. w_last whose range is not empty
-        for (int w0 = w_first; w0 <= w_last; w0 += kWave) {
-          const int w = w0 + lane;
-          const bool on = w <= w_last && range_start(w + 1, total, n_workers) > range_start(w, total, n_workers);
-          pieces += __builtin_popcountll(__builtin_amdgcn_ballot_w64(on));
-        }
+        const int64_t n_use = used_workers(n_workers, total);
+        const int w_first = workgroup_of(first, total, n_use), w_last = workgroup_of(last, total, n_use);
+        const int pieces = w_last - w_first + 1;  // (no range in between is empty)
         unsigned old = 0;
         if (lane == 0) old = atomicInc(a.ws_arrivals + w_first, static_cast<unsigned>(pieces - 1));
         old = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(old)));
@@ -1442,11 +1492,12 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
 // group issued together.
 // VL: the columns of a partial are (query token, head) pairs of the sequence's chunk (see gqa_mfma_kernel).
 // The merge of one (head block hbk, sequence b) by `nthreads` threads (this one is `tid`); p0, p1, pt = item
-// prefix of the sequence, of the next one, and the batch total.  COHERENT: the partials were written by
+// prefix of the sequence, of the next one, and the batch total; cut = where the second pool's part of the list
+// begins (GqaArgs::pool_even).  COHERENT: the partials were written by
 // other workers of the same launch (store_shared) and are read the same way.
 template <typename QT, bool VL, bool COHERENT>
 __device__ __forceinline__ void merge_context(const GqaArgs& a, int dv, int hbk, int b, int tid, int nthreads,
-                                              int p0, int p1, int pt) {
+                                              int p0, int p1, int pt, int cut) {
   const int G = a.g_block;
   const int hb_per_kv = VL ? a.chunk_blocks : (a.group + G - 1) / G;
   const int n_hb = a.n_kv_heads * hb_per_kv;
@@ -1498,37 +1549,58 @@ __device__ __forceinline__ void merge_context(const GqaArgs& a, int dv, int hbk,
   const int64_t total = static_cast<int64_t>(pt) * n_hbl;
   const int64_t first = static_cast<int64_t>(p0) * n_hbl + static_cast<int64_t>(hbk / HL) * n_items;
   const int64_t last = first + n_items - 1;
-  const int64_t n = a.n_workgroups / HL;
-  const int w_first = workgroup_of(first, total, n);
-  const int w_last = workgroup_of(last, total, n);
-  if (w_first == w_last) return;  // one worker saw the whole context and wrote the output
-  // range_start(w) = w * q + floor(w * r / n) with total = q * n + r: stepped from w to w + 1
-  // without a division
-  const bool fits32 = total * n < (1LL << 31);
-  const int64_t q = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(total) / static_cast<uint32_t>(n)) : total / n, r = total - q * n;
-  const int64_t acc0 = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(w_first) * static_cast<uint32_t>(r) % static_cast<uint32_t>(n))
-                              : (static_cast<int64_t>(w_first) * r) % n;
-  // the first worker holds this context as its last run (slot 1) unless its range starts
-  // exactly here; every later one holds it as its first run (slot 0)
-  const int slot_first = range_start(w_first, total, n) < first ? 1 : 0;
+  // The pieces of the context lie with consecutive teams of a list: of the whole list, or with the two pools of
+  // GqaArgs::pool_even of one or both of its parts (two segments then).  A segment: teams wf .. wl of a list of `tot`
+  // items dealt to `n` teams.
+  const bool pooled = a.pool_even != 0;
+  Pools pools = {};
+  if (pooled) pools = make_pools(a, total, cut);
+  const bool in0 = !pooled || first < pools.cut;         // pieces in the whole list / in the first pool's part
+  const bool in1 = pooled && last >= pools.cut;          // pieces in the second pool's part
+  const int64_t tot0 = pooled ? pools.cut : total, n0 = used_workers(pooled ? pools.half : a.n_workgroups / HL, tot0);
+  const int64_t tot1 = total - pools.cut, n1 = used_workers(pools.half, tot1);
+  const int64_t lo1 = first >= pools.cut ? first : pools.cut, hi0 = in1 ? pools.cut - 1 : last;
+  // (one copy of the arithmetic for both segments: two trips through a loop that is not unrolled, the second one
+  // for the few contexts that lie across the cut)
+  int wf0 = 0, wl0 = -1, sf0 = 0, wf1 = 0, wl1 = -1, sf1 = 0;
+#pragma nounroll
+  for (int sg = 0; sg < 2; ++sg) {
+    if (!(sg ? in1 : in0)) continue;
+    const int64_t base = sg ? pools.cut : 0, tot = sg ? tot1 : tot0, n = sg ? n1 : n0;
+    const int wf = workgroup_of((sg ? lo1 : first) - base, tot, n);
+    const int wl = workgroup_of((sg ? last : hi0) - base, tot, n);
+    // the first team of a segment holds this context as its last run (slot 1) unless its range starts inside the
+    // context; every later one holds it as its first run (slot 0)
+    const int sf = base + range_start(wf, tot, n) < first ? 1 : 0;
+    if (sg) {
+      wf1 = wf;
+      wl1 = wl;
+      sf1 = sf;
+    } else {
+      wf0 = wf;
+      wl0 = wl;
+      sf0 = sf;
+    }
+  }
+  const int cnt0 = wl0 - wf0 + 1, cnt = cnt0 + (wl1 - wf1 + 1);   // teams of the first segment, of both
+  if (cnt == 1) return;  // one team saw the whole context and wrote the output
   for (int v = tid; v < n_vec; v += nthreads) {
     const int h = v / dv4, d = (v - h * dv4) * 4;
-    int64_t acc = acc0;
     float M = kNegBig, W = 0.0f;
     f32x4 O = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int wb = w_first; wb <= w_last; wb += 4) {
+    for (int j0 = 0; j0 < cnt; j0 += 4) {
       float lse[4];
       f32x4 x[4];
       bool on[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        const int w = wb + k;
-        acc += r;
-        const int64_t step = q + (acc >= n ? 1 : 0);
-        acc -= acc >= n ? n : 0;
-        // with fewer items than workers some ranges in between are empty and own no partial
-        on[k] = w <= w_last && step > 0;
-        const int64_t ps = ((static_cast<int64_t>(w) * HL + member) * 2 + (w == w_first ? slot_first : 0)) * G + h;
+        const int j = min(j0 + k, cnt - 1);
+        const bool second = j >= cnt0;
+        const int w = second ? wf1 + (j - cnt0) : wf0 + j;
+        on[k] = j0 + k < cnt;
+        const int team = pooled ? pools.of_pool(second ? 1 : 0, w) : w;
+        const int slot = j == 0 ? (in0 ? sf0 : sf1) : (j == cnt0 ? sf1 : 0);
+        const int64_t ps = ((static_cast<int64_t>(team) * HL + member) * 2 + slot) * G + h;
         if constexpr (COHERENT) {
           const float* xp = a.ws_out + ps * dv + d;
           lse[k] = on[k] ? load_shared(a.ws_lse + ps) : kNegBig;
@@ -1561,7 +1633,7 @@ template <typename QT, bool VL>
 __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int dv) {
   const int b = blockIdx.y;
   merge_context<QT, VL>(a, dv, blockIdx.x, b, threadIdx.x, kThreads, a.ws_prefix[b], a.ws_prefix[b + 1],
-                        a.ws_prefix[a.batch]);
+                        a.ws_prefix[a.batch], a.pool_even != 0 ? a.ws_prefix[a.batch + 1] : 0);
 }
 
 int device_cu_count() {
@@ -1601,6 +1673,17 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
 }
 
 constexpr int kMfmaStages = 4;
+
+// Tuning knob XLLM_MI355_GQA_XCD_POOLS: the share of the teams on even XCDs in eighths of the share of those on odd
+// XCDs (default 9, see GqaArgs::pool_even; 0 = one list for all teams).
+int xcd_pools_knob() {
+  static const int v = [] {
+    const char* e = getenv("XLLM_MI355_GQA_XCD_POOLS");
+    const int x = e ? atoi(e) : -1;
+    return x >= 0 && x <= 16 ? x : 9;
+  }();
+  return v;
+}
 
 // Tuning knob XLLM_MI355_GQA_HEAD_LOCK (1, 2 or 4; default 4): see GqaArgs::head_lock.
 int head_lock_knob() {
@@ -1668,6 +1751,12 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
         a.head_lock = hl;
         break;
       }
+  }
+  // (the pools need whole groups of eight workgroups, one per XCD; the in-kernel merge walks one list)
+  a.pool_even = a.pool_odd = 0;
+  if (a.fold_merge == 0 && n_wg % 8 == 0 && xcd_pools_knob() != 0) {
+    a.pool_even = xcd_pools_knob();
+    a.pool_odd = 8;
   }
   const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 1) * 4;
   launch_timed(kern, dim3(static_cast<unsigned>(n_wg)), dim3(kMfmaThreads), smem, stream, a);
