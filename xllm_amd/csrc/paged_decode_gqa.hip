@@ -1752,9 +1752,11 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
         break;
       }
   }
-  // (the pools need whole groups of eight workgroups, one per XCD; the in-kernel merge walks one list)
+  // (the pools need whole groups of eight workgroups, one per XCD; the in-kernel merge walks one list; fp8 rows of
+  // 64 bytes keep the computing wavefronts busy enough that the XCDs end together with equal ranges: 134 us against
+  // 139 us with the cut)
   a.pool_even = a.pool_odd = 0;
-  if (a.fold_merge == 0 && n_wg % 8 == 0 && xcd_pools_knob() != 0) {
+  if (a.fold_merge == 0 && n_wg % 8 == 0 && xcd_pools_knob() != 0 && !(FP8 && D == 64)) {
     a.pool_even = xcd_pools_knob();
     a.pool_odd = 8;
   }
