@@ -348,6 +348,42 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     merge_ms = sum(ms[1::2]) / max(len(ms[1::2]), 1)
     ops.decode_status(dev)                 # raises if a wait inside a decode kernel gave up
 
+    # ---- the same step as the layers after the first see it when the step was planned once (not the headline:
+    # `value` above is the self-contained call, which derives its schedule in every launch)
+    planned = None
+    if not cfg.mla:
+        plan = torch.empty(lib.xllm_mi355_paged_decode_plan_bytes(), dtype=torch.uint8, device=dev)
+        plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), None, None, None, cfg.batch,
+                     cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, -1, code[cache_dt], stream)
+        planned_args = (ptr(plan),) + decode_args[:8] + (None, None, None) + decode_args[8:]
+        plain_out = out.clone()
+
+        def planned_step():
+            rc = reshape_fn(*reshape_args)
+            rc2 = lib.xllm_mi355_paged_decode_gqa_planned(*planned_args)
+            if rc or rc2:
+                capi.check(rc or rc2, "bench planned step")
+
+        capi.check(lib.xllm_mi355_profile_enable(1), "profile_enable")
+        capi.check(lib.xllm_mi355_paged_decode_gqa_plan(*plan_args), "xllm_mi355_paged_decode_gqa_plan")
+        torch.cuda.synchronize()
+        plan_ms = collect_ms(lib, 1)
+        for _ in range(args.warmup):
+            planned_step()
+        torch.cuda.synchronize()
+        capi.check(lib.xllm_mi355_profile_enable(2 * args.steps), "profile_enable")
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            planned_step()
+        torch.cuda.synchronize()
+        p_elapsed = time.perf_counter() - t0
+        pms = collect_ms(lib, 2 * args.steps)
+        ops.decode_status(dev)
+        planned = {"kernel_ms": sum(pms[0::2]) / max(len(pms[0::2]), 1),
+                   "merge_kernel_ms": sum(pms[1::2]) / max(len(pms[1::2]), 1),
+                   "ms_per_step": p_elapsed / args.steps * 1e3, "plan_kernel_ms": plan_ms[0] if plan_ms else None,
+                   "bit_identical": bool(torch.equal(plain_out, out))}
+
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = cfg.batch / (ms_per_step * 1e-3)
 
@@ -379,6 +415,8 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
                      "algorithmic_bytes": nbytes})
     if flops is not None:
         roofline["algorithmic_flops"] = flops
+    if planned is not None:
+        roofline["planned"] = planned
     # the same number of bytes through the plain read kernel: the rate this GPU sustains at this size
     roofline["stream_read_gbs_same_bytes"], _ = stream_rate(lib, capi, torch, dev, nbytes)
 

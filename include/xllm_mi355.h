@@ -59,7 +59,8 @@ enum {
   XLLM_MI355_EWORKSPACE = -4,  /* workspace missing or too small                */
   XLLM_MI355_EALIGN = -5,      /* pointer or stride not 16-byte aligned         */
   XLLM_MI355_ESTALLED = -6,    /* xllm_mi355_decode_status: a bounded wait inside a decode kernel gave up */
-  XLLM_MI355_ESCRATCH = -7     /* the problem does not fit the static scratch of the no-allocation entry point */
+  XLLM_MI355_ESCRATCH = -7,    /* the problem does not fit the static scratch of the no-allocation entry point */
+  XLLM_MI355_EPLAN = -8        /* xllm_mi355_decode_status: a decode launch met a plan made for another shape */
 };
 
 /* Human-readable text for a return code of this library (host pointer, static). */
@@ -131,7 +132,8 @@ size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads,
  * xllm_mi355_decode_status is the voice of the kernels: the wavefronts of the matrix-core GQA kernel wait for
  * each other with bounded polls; if a poll ever runs out, the wavefront sets a flag in the header and exits,
  * and the outputs of that launch are invalid.  The call waits for `stream`, reads the flag from the host and
- * clears it: 0 = no launch since the last call gave up, XLLM_MI355_ESTALLED otherwise.  It synchronises, so it
+ * clears it: 0 = no launch since the last call gave up, XLLM_MI355_ESTALLED otherwise (XLLM_MI355_EPLAN when the
+ * flag is that of a planned call whose plan was made for another shape, see xllm_mi355_paged_decode_gqa_plan).  It synchronises, so it
  * is for use outside graph capture (for example once per step, or when a result looks wrong).  The reference
  * has no counterpart (its fast paths are closed libraries that abort on error).
  */
@@ -210,6 +212,48 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                                     int64_t max_seq_len, int64_t window_left, float sm_scale,
                                     void* workspace, size_t workspace_bytes,
                                     int q_dtype, int cache_dtype, void* stream);
+
+/*
+ * The plan of a decode step, made once and used by the decode calls of every layer: the counterpart of the
+ * reference's FlashInfer plan, which update_decode_plan_info computes at layer 0 only and every layer's
+ * batch_decode then takes (xllm/core/layers/cuda/flashinfer_planinfo.cpp:248-264 with the early return of :263-264
+ * for layer_id != 0; plan_info argument of xllm/core/kernels/cuda/cuda_ops_api.h:128-144).
+ * xllm_mi355_paged_decode_gqa_plan is one small launch that writes into `plan` (device memory of
+ * xllm_mi355_paged_decode_plan_bytes() bytes, 256-byte aligned, the caller's): the prefix of the per-sequence work
+ * items, where the work list is cut between the workers, and for every group of workers the page-table entries
+ * its first loads need.  xllm_mi355_paged_decode_gqa_planned is xllm_mi355_paged_decode_gqa (block_table form,
+ * paged_kv_indptr == NULL) or xllm_mi355_paged_decode_gqa_csr (paged_kv_indptr != NULL) that starts from the plan
+ * instead of deriving all that in every launch: same kernels, same order of arithmetic, bit-identical results.
+ * The plan holds for the sequence lengths, tables, head counts, head dim, block size, window and cache dtype it
+ * was made with: make it again when any of them changes (every decode step).  Shapes that the matrix-core kernel
+ * does not serve take no plan and are decoded as by the plain entry points.  A planned call whose shape differs
+ * from the plan's writes no output and raises a flag that xllm_mi355_decode_status reports as XLLM_MI355_EPLAN;
+ * lengths or tables that changed under the same shape are not detected.  Plan and planned calls are plain
+ * launches on `stream` (legal under graph capture; a replay plans again from the current lengths).
+ */
+size_t xllm_mi355_paged_decode_plan_bytes(void);
+int xllm_mi355_paged_decode_gqa_plan(void* plan, size_t plan_bytes,
+                                     const int32_t* block_table, int64_t table_stride,
+                                     const int32_t* seq_lens,
+                                     const int32_t* paged_kv_indptr, const int32_t* paged_kv_indices,
+                                     const int32_t* paged_kv_last_page_len,
+                                     int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
+                                     int64_t head_dim, int64_t block_size, int64_t window_left,
+                                     int cache_dtype, void* stream);
+int xllm_mi355_paged_decode_gqa_planned(const void* plan,
+                                        const void* q, const void* k_cache, const void* v_cache,
+                                        void* out, float* lse,
+                                        const int32_t* block_table, int64_t table_stride,
+                                        const int32_t* seq_lens,
+                                        const int32_t* paged_kv_indptr, const int32_t* paged_kv_indices,
+                                        const int32_t* paged_kv_last_page_len,
+                                        const float* k_scale, const float* v_scale,
+                                        int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
+                                        int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                        int64_t q_token_stride, int64_t out_token_stride,
+                                        int64_t max_seq_len, int64_t window_left, float sm_scale,
+                                        void* workspace, size_t workspace_bytes,
+                                        int q_dtype, int cache_dtype, void* stream);
 
 /*
  * Rows of paged sequences gathered into one packed buffer, sequence after sequence.

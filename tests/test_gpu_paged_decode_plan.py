@@ -1,0 +1,200 @@
+"""GPU tests of the step plan: a decode call that starts from a plan runs the same kernels over the same ranges as one
+that derives its schedule itself, so its outputs must be bit-identical; the plain call is checked against the
+reference's libtorch CPU path elsewhere and once more here."""
+import pytest
+import torch
+
+import oracle
+from helpers import assert_close_to_reference, fill_caches_gpu
+from xllm_amd import capi, ops, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(inp, kg, vg, device, ks=None, vs=None, window_left=-1, lens=None):
+    cfg, lay = inp.cfg, inp.layout
+    q = inp.q.to(device)
+    table = lay.block_table.to(device)
+    lens = (lay.seq_lens if lens is None else lens).to(device)
+    hi = max(1, int(lens.max()))
+    plain, plain_lse = ops.batch_decode(q, kg, torch.empty_like(q), table, lens, v_cache=vg, k_cache_quant_scale=ks,
+                                        v_cache_quant_scale=vs, scale=cfg.scale, return_lse=True, max_seq_len=hi,
+                                        window_left=window_left)
+    plan = ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                       block_table=table, seq_lens=lens, window_left=window_left)
+    outs = []
+    for _ in range(2):  # the layers of a step share the plan
+        o, l = ops.batch_decode(q, kg, torch.full_like(q, 7.0), table, lens, v_cache=vg, k_cache_quant_scale=ks,
+                                v_cache_quant_scale=vs, scale=cfg.scale, return_lse=True, max_seq_len=hi,
+                                window_left=window_left, plan=plan)
+        outs.append((o, l))
+    torch.cuda.synchronize()
+    for o, l in outs:
+        assert torch.equal(o, plain), cfg.name
+        assert torch.equal(l, plain_lse), cfg.name
+    assert ops.decode_status(device) == 0
+    return plain
+
+
+def test_planned_decode_is_bit_identical_on_the_benchmark_shapes(device):
+    for name, batch, seed in (("llama3_8b", 64, 3), ("long_b256", 24, 4)):
+        cfg = workloads.scaled(workloads.CONFIGS[name], batch=batch)
+        inp = workloads.make_inputs(cfg, seed, device=device)
+        kg, vg, _, _ = fill_caches_gpu(inp, device)
+        out = _both(inp, kg, vg, device)
+        lay = inp.layout
+        sample = [0, 1, batch // 2, batch - 1]
+        ref = oracle.aten_paged_decode(inp.q.cpu()[sample].contiguous(), kg.cpu(), vg.cpu(),
+                                       lay.block_table[sample].contiguous(), lay.seq_lens[sample].contiguous(), cfg.scale)
+        assert_close_to_reference(out[sample], ref, cfg.name)
+
+
+def test_planned_decode_over_shapes_windows_and_empty_sequences(device):
+    g = torch.Generator().manual_seed(11)
+    # (Hq, Hkv, D, block size, fp8): the stage sizes and head-block groupings of the matrix-core kernel, and two
+    # shapes that the kernel does not serve (block size 8; fp8 with head dim 256), which take no plan
+    shapes = ((32, 8, 128, 16, False), (32, 8, 128, 16, True), (8, 2, 64, 32, False), (16, 4, 64, 16, True),
+              (6, 1, 256, 128, False), (40, 2, 128, 16, False), (12, 3, 128, 64, False), (8, 2, 128, 8, False),
+              (4, 1, 256, 16, True))
+    for i, (Hq, Hkv, D, bs, fp8) in enumerate(shapes):
+        batch = int(torch.randint(1, 40, (1,), generator=g))
+        cfg = workloads.DecodeConfig(f"plan_{Hq}_{Hkv}_{D}_{bs}_{fp8}", batch, Hq, Hkv, D, bs, 1, 1500,
+                                     cache_dtype="fp8" if fp8 else "bf16")
+        inp = workloads.make_inputs(cfg, 300 + i, device=device)
+        kg, vg, ks, vs = fill_caches_gpu(inp, device, cache_dtype=torch.float8_e4m3fn if fp8 else None)
+        _both(inp, kg, vg, device, ks, vs)
+        _both(inp, kg, vg, device, ks, vs, window_left=200)
+        lens = inp.layout.seq_lens.clone()
+        lens[torch.rand(batch, generator=g) < 0.4] = 0
+        _both(inp, kg, vg, device, ks, vs, lens=lens)
+        _both(inp, kg, vg, device, ks, vs, lens=torch.zeros_like(lens))
+
+
+def test_planned_decode_in_csr_form(device):
+    cfg = workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=37, len_lo=1, len_hi=3000)
+    inp = workloads.make_inputs(cfg, 21, device=device)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    q = inp.q.to(device)
+    indptr, indices, last = lay.indptr.to(device), lay.indices.to(device), lay.last_page_len.to(device)
+    hi = int(lay.seq_lens.max())
+    plain = ops.batch_decode_csr(q, kg, vg, indptr, indices, last, -1, cfg.scale, torch.empty_like(q), max_seq_len=hi)
+    plan = ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                       paged_kv_indptr=indptr, paged_kv_indices=indices, paged_kv_last_page_len=last)
+    planned = ops.batch_decode_csr(q, kg, vg, indptr, indices, last, -1, cfg.scale, torch.full_like(q, 7.0),
+                                   max_seq_len=hi, plan=plan)
+    torch.cuda.synchronize()
+    assert torch.equal(plain, planned)
+    assert ops.decode_status(device) == 0
+
+
+def test_a_plan_for_another_shape_is_reported(device):
+    cfg = workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=9)
+    inp = workloads.make_inputs(cfg, 5, device=device)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    q, table, lens = inp.q.to(device), lay.block_table.to(device), lay.seq_lens.to(device)
+    assert ops.decode_status(device) == 0
+    # made for 8 of the 9 sequences
+    plan = ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                       block_table=table[:8], seq_lens=lens[:8].contiguous())
+    ops.batch_decode(q, kg, torch.empty_like(q), table, lens, v_cache=vg, scale=cfg.scale, plan=plan)
+    with pytest.raises(capi.XllmMi355Error, match="plan"):
+        ops.decode_status(device)
+    assert ops.decode_status(device) == 0   # reported once
+    good = ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                       block_table=table, seq_lens=lens, plan=plan)
+    assert good.data_ptr() == plan.data_ptr()
+    a, _ = ops.batch_decode(q, kg, torch.empty_like(q), table, lens, v_cache=vg, scale=cfg.scale, plan=good)
+    b, _ = ops.batch_decode(q, kg, torch.empty_like(q), table, lens, v_cache=vg, scale=cfg.scale)
+    assert torch.equal(a, b)
+    assert ops.decode_status(device) == 0
+    with pytest.raises(ValueError):   # a plan buffer that is too small
+        ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                    block_table=table, seq_lens=lens, plan=plan[:4096])
+
+
+def test_a_captured_step_plans_again_on_every_replay(device):
+    # plan + two planned layers in one graph; the lengths change between replays (the persistent buffers of a
+    # captured decode step), eager calls run in between
+    cfg = workloads.DecodeConfig("plan_graph", 48, 32, 8, 128, 16, 200, 2500)
+    inp = workloads.make_inputs(cfg, 31, device=device)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    q, table = inp.q.to(device), lay.block_table.to(device)
+    lens = lay.seq_lens.to(device).clone()
+    plan = ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                       block_table=table, seq_lens=lens)
+    o1, o2 = torch.zeros_like(q), torch.zeros_like(q)
+    ops.batch_decode(q, kg, o1, table, lens, v_cache=vg, scale=cfg.scale, max_seq_len=2500, plan=plan)  # warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                    block_table=table, seq_lens=lens, plan=plan)
+        ops.batch_decode(q, kg, o1, table, lens, v_cache=vg, scale=cfg.scale, max_seq_len=2500, plan=plan)
+        ops.batch_decode(q, kg, o2, table, lens, v_cache=vg, scale=cfg.scale, max_seq_len=2500, plan=plan)
+    g = torch.Generator().manual_seed(3)
+    for rep in range(4):
+        cut = torch.randint(0, 200, (cfg.batch,), generator=g, dtype=torch.int32)
+        cut[torch.rand(cfg.batch, generator=g) < 0.2] = 100000   # some sequences leave the batch
+        lens.copy_(torch.clamp(lay.seq_lens - cut, min=0).to(device))
+        o1.zero_()
+        o2.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager, _ = ops.batch_decode(q, kg, torch.empty_like(q), table, lens, v_cache=vg, scale=cfg.scale, max_seq_len=2500)
+        torch.cuda.synchronize()
+        assert torch.equal(o1, eager) and torch.equal(o2, eager), f"replay {rep}"
+    assert ops.decode_status(device) == 0
+
+
+def test_layer_zero_plans_and_the_other_layers_decode_from_its_plan(device):
+    """AttentionMetadata::plan_info of the reference (layers/common/attention_metadata.h:163): every layer's forward
+    calls update_decode_plan_info, which returns at once unless layer_id == 0
+    (layers/cuda/flashinfer_planinfo.cpp:263-264), and hands the plan to batch_decode."""
+    from xllm_amd import torch_ops
+    xops = torch_ops.load()
+    cfg = workloads.DecodeConfig("layer_plan", 21, 32, 8, 128, 16, 60, 2500)
+    inp = workloads.make_inputs(cfg, 78)
+    lay = inp.layout
+    B, Hq, Hkv, D = cfg.batch, cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim
+    caches = []
+    for layer in range(3):   # every layer has its own cache; the tables and lengths are the step's
+        kg = torch.zeros(lay.num_blocks, cfg.block_size, Hkv, D, dtype=torch.bfloat16, device=device)
+        vg = torch.zeros_like(kg)
+        scale = 1.0 + 0.25 * layer
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(
+            key=(inp.k_ctx * scale).to(device), value=(inp.v_ctx * scale).to(device), k_cache=kg, v_cache=vg,
+            slot_mapping=lay.ctx_slots.to(device)))
+        caches.append((kg, vg))
+    query = inp.q.to(device).view(B, Hq * D)
+    key = inp.k_new.to(device).view(B, Hkv * D)
+    value = inp.v_new.to(device).view(B, Hkv * D)
+    table, lens, slots = lay.block_table.to(device), lay.seq_lens.to(device), lay.new_slots.to(device)
+    hi = int(lay.seq_lens.max())
+
+    def layer_forward(layer, plan, layer_id):
+        kg, vg = caches[layer]
+        out, lse = xops.attention_layer_forward(query, key, value, kg, vg, None, None, slots, table, lens, None, hi, 1,
+                                                Hq, D, Hkv, cfg.scale, -1, True, True, plan, layer_id)
+        return out.clone(), lse.clone()
+
+    plain = [layer_forward(layer, None, -1) for layer in range(3)]
+    plan = torch.zeros(capi.lib().xllm_mi355_paged_decode_plan_bytes(), dtype=torch.uint8, device=device)
+    planned = [layer_forward(layer, plan, layer) for layer in range(3)]
+    torch.cuda.synchronize()
+    assert int(plan.view(torch.int32)[0]) != 0, "layer 0 did not plan"
+    for (a, al), (b, bl) in zip(plain, planned):
+        assert torch.equal(a, b) and torch.equal(al, bl)
+    assert not torch.equal(plain[0][0], plain[1][0])
+    assert ops.decode_status(device) == 0
+    # the dispatcher ops on their own
+    p2 = xops.update_decode_plan(table, lens, Hq, Hkv, D, cfg.block_size, -1, False)
+    kg, vg = caches[0]
+    q3 = inp.q.to(device)
+    a, _ = xops.batch_decode(q3, kg, vg, torch.empty_like(q3), table, lens, None, None, hi, cfg.scale, p2)
+    b, _ = xops.batch_decode(q3, kg, vg, torch.empty_like(q3), table, lens, None, None, hi, cfg.scale)
+    assert torch.equal(a, b)
+    w2, w = p2.view(torch.int32), plan.view(torch.int32)   # the same plan: its first word and the item prefix
+    assert int(w2[0]) == int(w[0]) and torch.equal(w2[64 : 64 + B + 2], w[64 : 64 + B + 2])

@@ -57,6 +57,7 @@ const char* xllm_mi355_error_string(int code) {
     case XLLM_MI355_EWORKSPACE: return "split-K workspace missing, misaligned or too small";
     case XLLM_MI355_EALIGN: return "pointer or stride not 16-byte aligned";
     case XLLM_MI355_ESTALLED: return "a bounded wait inside a decode kernel gave up: the outputs of that launch are invalid";
+    case XLLM_MI355_EPLAN: return "a decode launch was given a plan made for another shape: it wrote no output";
     case XLLM_MI355_ESCRATCH: return "the problem needs more scratch than the static scratch of the no-allocation entry point holds";
     default: break;
   }
@@ -111,7 +112,7 @@ int xllm_mi355_decode_status(void* workspace, void* stream) {
   if (rc != 0) return rc;
   e = hipStreamSynchronize(s);
   if (e != hipSuccess) return static_cast<int>(e);
-  return XLLM_MI355_ESTALLED;
+  return (status & kStatusWaitGaveUp) != 0 ? XLLM_MI355_ESTALLED : XLLM_MI355_EPLAN;
 }
 
 int xllm_mi355_debug_set(int what, int value) {
@@ -190,6 +191,59 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
                           n_kv_heads, head_dim, block_size, num_blocks, q_token_stride,
                           out_token_stride, max_seq_len, sm_scale, workspace, workspace_bytes, q_dtype,
                           cache_dtype, static_cast<hipStream_t>(stream));
+}
+
+size_t xllm_mi355_paged_decode_plan_bytes(void) { return gqa_plan_bytes(); }
+
+int xllm_mi355_paged_decode_gqa_plan(void* plan, size_t plan_bytes, const int32_t* block_table,
+                                     int64_t table_stride, const int32_t* seq_lens,
+                                     const int32_t* paged_kv_indptr, const int32_t* paged_kv_indices,
+                                     const int32_t* paged_kv_last_page_len, int64_t batch, int64_t n_q_heads,
+                                     int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
+                                     int64_t window_left, int cache_dtype, void* stream) {
+  PageAddressing addr;
+  addr.window_left = window_left;
+  if (paged_kv_indptr != nullptr) {
+    addr.indptr = paged_kv_indptr;
+    addr.indices = paged_kv_indices;
+    addr.last_page_len = paged_kv_last_page_len;
+  } else {
+    addr.block_table = block_table;
+    addr.table_stride = table_stride;
+    addr.seq_lens = seq_lens;
+  }
+  return paged_decode_gqa_plan(plan, plan_bytes, addr, batch, n_q_heads, n_kv_heads, head_dim, block_size,
+                               cache_dtype, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_paged_decode_gqa_planned(const void* plan, const void* q, const void* k_cache,
+                                        const void* v_cache, void* out, float* lse,
+                                        const int32_t* block_table, int64_t table_stride,
+                                        const int32_t* seq_lens, const int32_t* paged_kv_indptr,
+                                        const int32_t* paged_kv_indices,
+                                        const int32_t* paged_kv_last_page_len, const float* k_scale,
+                                        const float* v_scale, int64_t batch, int64_t n_q_heads,
+                                        int64_t n_kv_heads, int64_t head_dim, int64_t block_size,
+                                        int64_t num_blocks, int64_t q_token_stride, int64_t out_token_stride,
+                                        int64_t max_seq_len, int64_t window_left, float sm_scale,
+                                        void* workspace, size_t workspace_bytes, int q_dtype, int cache_dtype,
+                                        void* stream) {
+  if (plan == nullptr) return XLLM_MI355_EINVAL;
+  PageAddressing addr;
+  addr.window_left = window_left;
+  addr.plan = plan;
+  if (paged_kv_indptr != nullptr) {
+    addr.indptr = paged_kv_indptr;
+    addr.indices = paged_kv_indices;
+    addr.last_page_len = paged_kv_last_page_len;
+  } else {
+    addr.block_table = block_table;
+    addr.table_stride = table_stride;
+    addr.seq_lens = seq_lens;
+  }
+  return paged_decode_gqa(q, k_cache, v_cache, out, lse, addr, k_scale, v_scale, batch, n_q_heads, n_kv_heads,
+                          head_dim, block_size, num_blocks, q_token_stride, out_token_stride, max_seq_len, sm_scale,
+                          workspace, workspace_bytes, q_dtype, cache_dtype, static_cast<hipStream_t>(stream));
 }
 
 int xllm_mi355_gather_paged_rows(const void* cache, const int32_t* block_table, int64_t table_stride,

@@ -38,6 +38,8 @@ struct PageAddressing {
   const int32_t* last_page_len = nullptr;
   // sliding window: the query at position L - 1 attends to positions >= L - 1 - window_left; negative: all
   int64_t window_left = -1;
+  // the step's plan (paged_decode_gqa_plan with the same shape, lengths and tables), or null
+  const void* plan = nullptr;
 };
 
 // Layout of a decode workspace, the same for every decode entry point and independent of the batch, so that
@@ -53,6 +55,7 @@ constexpr size_t kWsHeaderBytes = kWsCountersOff + static_cast<size_t>(kWsMaxWor
 constexpr int kWsMaxBatch = 2048;
 constexpr size_t kWsPartialsOff = kWsHeaderBytes + (static_cast<size_t>(kWsMaxBatch + 1) * 4 + 255) / 256 * 256;
 constexpr int kStatusWaitGaveUp = 1;  // a bounded wait of one wavefront on another ran out: the launch's output is invalid
+constexpr int kStatusPlanMismatch = 2;  // a decode launch was given a plan made for another shape: it wrote no output
 
 // Bound of the polls of one wavefront on another (test hook: xllm_mi355_debug_set_wait_spins).
 int wait_spin_limit();
@@ -72,6 +75,13 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
                      int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
                      int64_t out_token_stride, int64_t max_seq_len, float sm_scale, void* workspace,
                      size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream);
+
+// The plan of a decode step (item prefix, pool cut, first page-table chunk of every group of workers), made
+// once and handed to the decode calls of all layers through PageAddressing::plan.
+size_t gqa_plan_bytes();
+int paged_decode_gqa_plan(void* plan, size_t plan_bytes, const PageAddressing& addr, int64_t batch, int64_t n_q_heads,
+                          int64_t n_kv_heads, int64_t head_dim, int64_t block_size, int cache_dtype,
+                          hipStream_t stream);
 
 int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out, float* lse,
                      const PageAddressing& addr, int64_t batch, int64_t n_heads, int64_t d_latent,

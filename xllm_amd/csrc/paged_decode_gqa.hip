@@ -103,6 +103,12 @@ struct GqaArgs {
   // With equal shares the workgroups on the odd XCDs stream their rows 8-11 % slower and end a launch that much later
   // (every MI355X measured, five of them); 9 : 8 ends the decode kernels 1.7-2.7 % earlier.  0 : 0 = one list.
   int pool_even, pool_odd;
+  // Matrix-core kernel: a plan of the step, made once by gqa_plan_kernel for all layers (see kPlan*), or null: the
+  // item prefix, the cut between the pools and, for every group of workers, the 64 page-table entries its first
+  // stage needs.  With it the kernel's start is one trip to memory (prefix, lengths and pages together), then rows,
+  // instead of three in a row (lengths -> prefix -> pages of the range's first context) before the first row moves.
+  const int* plan;
+  int plan_sig;       // what the plan must have been made for (plan_signature), checked against the plan's own word
   int wait_spins;     // bound of the polls of one wavefront of a pair on the other
   int window_left;    // sliding window: the query (position L - 1) attends to positions >= L - 1 - window_left; < 0: all
   float scale_log2;   // sm_scale * log2(e)
@@ -179,6 +185,34 @@ __device__ __forceinline__ Pools make_pools(const GqaArgs& a, int64_t total, int
   p.per_shift = a.head_lock == 4 ? 0 : a.head_lock == 2 ? 1 : 2;   // (kWaves = 4 workers in a workgroup)
   p.half = a.n_workgroups / a.head_lock / 2;
   return p;
+}
+
+// A plan (ints): word 0 the signature of what it was made for | from kPlanPrefixOff the item prefix [batch + 1] and
+// the cut between the pools | from kPlanChunksOff 64 page-table entries per group of workers (the chunk of the
+// context's table that holds the page of the group's first stage; the tail repeats the context's last page).
+constexpr int kPlanPrefixOff = 64;
+constexpr int kPlanChunksOff = kPlanPrefixOff + (kMaxBatch + 2 + 63) / 64 * 64;
+constexpr int kPlanMaxTeams = 4096;
+constexpr size_t kPlanBytes = (static_cast<size_t>(kPlanChunksOff) + static_cast<size_t>(kPlanMaxTeams) * kWave) * 4;
+
+// The range [cur, end) of the flat list that group of workers `team` of `n_teams` takes; false: none.
+__device__ __forceinline__ bool team_range(const GqaArgs& a, int64_t total, int64_t cut, int64_t team, int64_t n_teams,
+                                           int64_t& cur, int64_t& end) {
+  if (a.pool_even != 0) {   // the list in two parts: one for the teams on even XCDs, one for those on odd XCDs
+    const Pools pools = make_pools(a, total, cut);
+    int par, q;
+    pools.of_team(static_cast<int>(team), par, q);
+    const int64_t n_use = used_workers(pools.half, pools.size(par));
+    if (q >= n_use) return false;
+    cur = pools.base(par) + range_start(q, pools.size(par), n_use);
+    end = pools.base(par) + range_start(q + 1, pools.size(par), n_use);
+  } else {
+    const int64_t n_use = used_workers(n_teams, total);
+    if (team >= n_use) return false;
+    cur = range_start(team, total, n_use);
+    end = range_start(team + 1, total, n_use);
+  }
+  return cur < end;
 }
 
 // Exclusive prefix sum of the per-sequence item counts into prefix[0..batch] (LDS).
@@ -815,11 +849,37 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // then finds a sequence without a trip to memory (one of the four in a row before its first row moves).
   int* lens = reinterpret_cast<int*>(smem + Lay::kLensOff);
   const bool lens_in_lds = a.indptr == nullptr && a.table_rows == nullptr && a.batch <= kThreads;
-  item_prefix<T>(a, prefix, tmp, lens_in_lds ? lens : nullptr);
+  const bool loader = wave < kWaves;   // wavefronts 0 .. kWaves - 1 load, wavefront kWaves + w computes what w loads
+  const int pair = wave & (kWaves - 1);
+  const int64_t worker = static_cast<int64_t>(blockIdx.x) * kWaves + pair;   // owns the partial slots 2 worker, 2 worker + 1
+  const int64_t n_workers = static_cast<int64_t>(gridDim.x) * kWaves / HL;   // groups of HL workers share a range
+  const int64_t team = worker / HL;
+  const int member = pair % HL;        // head block member + HL * (group of head blocks)
+  const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
+  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + pair * 3 * kWave * 4);
+  const bool planned = !VL && a.plan != nullptr;
+  if (planned) {
+    // one trip to memory: the pages of the first stage straight into the worker's chunk buffer, the plan's prefix
+    // and the lengths into LDS (a plan made for another shape says so in its first word: nothing is written then)
+    if (loader) dma4(a.plan + kPlanChunksOff + team * kWave + lane, page_lds);
+    const int sig = a.plan[0];
+    for (int i = tid; i <= a.batch + 1; i += kMfmaThreads) prefix[i] = a.plan[kPlanPrefixOff + i];
+    if (lens_in_lds)
+      for (int i = tid; i < a.batch; i += kMfmaThreads) lens[i] = a.seq_lens[i];
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (sig != a.plan_sig) {
+      if (tid == 0) atomicOr(a.ws_status, kStatusPlanMismatch);
+      return;
+    }
+    __syncthreads();
+  } else {
+    item_prefix<T>(a, prefix, tmp, lens_in_lds ? lens : nullptr);
+  }
   const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hbl;
-  if (blockIdx.x == 0) {
+  const int64_t cut = a.pool_even == 0 ? 0 : planned ? prefix[a.batch + 1] : pool_cut(a, total);
+  if (blockIdx.x == 0 && !planned) {   // (with a plan the merge kernel reads the plan's)
     for (int i = tid; i <= a.batch; i += kMfmaThreads) a.ws_prefix[i] = prefix[i];
-    if (tid == 0 && a.pool_even != 0) a.ws_prefix[a.batch + 1] = static_cast<int>(pool_cut(a, total));
+    if (tid == 0 && a.pool_even != 0) a.ws_prefix[a.batch + 1] = static_cast<int>(cut);
   }
   auto sequence_at = [&](int b, const int32_t*& pages, int& L) {
     if (lens_in_lds) {
@@ -838,36 +898,14 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   }
   if (total == 0) return;
   // ---- from here on the pairs are independent: no workgroup barrier below this line
-  const bool loader = wave < kWaves;   // wavefronts 0 .. kWaves - 1 load, wavefront kWaves + w computes what w loads
-  const int pair = wave & (kWaves - 1);
-  const int64_t worker = static_cast<int64_t>(blockIdx.x) * kWaves + pair;   // owns the partial slots 2 worker, 2 worker + 1
-  const int64_t n_workers = static_cast<int64_t>(gridDim.x) * kWaves / HL;   // groups of HL workers share a range
-  const int64_t team = worker / HL;
-  const int member = pair % HL;        // head block member + HL * (group of head blocks)
   int64_t cur, end;
-  if (a.pool_even != 0) {   // the list in two parts: one for the teams on even XCDs, one for those on odd XCDs
-    const Pools pools = make_pools(a, total, pool_cut(a, total));
-    int par, q;
-    pools.of_team(static_cast<int>(team), par, q);
-    const int64_t n_use = used_workers(pools.half, pools.size(par));
-    if (q >= n_use) return;
-    cur = pools.base(par) + range_start(q, pools.size(par), n_use);
-    end = pools.base(par) + range_start(q + 1, pools.size(par), n_use);
-  } else {
-    const int64_t n_use = used_workers(n_workers, total);
-    if (team >= n_use) return;
-    cur = range_start(team, total, n_use);
-    end = range_start(team + 1, total, n_use);
-  }
-  if (cur >= end) return;
+  if (!team_range(a, total, cut, team, n_workers, cur, end)) return;
   const int n_stages = static_cast<int>(end - cur);
   lds_vint* landed = sync + 2 * pair;
   lds_vint* freed = landed + 1;
 
-  const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
   const u32 ring_lds = __builtin_amdgcn_readfirstlane(lds_base + pair * NS * kStageBytes);
   const char* ring = smem + pair * NS * kStageBytes;
-  const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kPageOff + pair * 3 * kWave * 4);
   const char* pagebuf = smem + Lay::kPageOff + pair * 3 * kWave * 4;
   const u32 q_lds = __builtin_amdgcn_readfirstlane(lds_base + Lay::kQOff + pair * G * Lay::kQRow);
   const char* qbuf = smem + Lay::kQOff + pair * G * Lay::kQRow;
@@ -974,7 +1012,7 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   auto begin_context = [&](bool first) {
     if (first) {
       ck_a = (((pc.st0 + pc.st) * T) >> a.bs_shift) >> 6;
-      issue_chunk(pc, ck_a, off_a);
+      if (!planned) issue_chunk(pc, ck_a, off_a);   // (a plan brought that chunk in with the prefix)
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     } else {
       const u32 t = off_a;
@@ -1629,9 +1667,48 @@ __device__ __forceinline__ void merge_context(const GqaArgs& a, int dv, int hbk,
   }
 }
 
+// The plan of a step for gqa_mfma_kernel (GqaArgs::plan): one wavefront per group of workers finds the start of the
+// group's range as the decode kernel would and copies the 64 page-table entries around the first stage's page.
+// T: tokens per stage of the decode kernel the plan is for.
+template <int T>
+__global__ __launch_bounds__(kThreads) void gqa_plan_kernel(GqaArgs a, int* plan, int n_teams) {
+  extern __shared__ __align__(16) char smem[];
+  int* tmp = reinterpret_cast<int*>(smem);
+  int* prefix = tmp + kThreads;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  item_prefix<T>(a, prefix, tmp);
+  const int hb_per_kv = (a.group + kMfmaHeads - 1) / kMfmaHeads;
+  const int n_hbl = a.n_kv_heads * hb_per_kv / a.head_lock;
+  const int64_t total = static_cast<int64_t>(prefix[a.batch]) * n_hbl;
+  const int64_t cut = a.pool_even == 0 ? 0 : pool_cut(a, total);
+  if (blockIdx.x == 0) {
+    for (int i = tid; i <= a.batch; i += kThreads) plan[kPlanPrefixOff + i] = prefix[i];
+    if (tid == 0) plan[kPlanPrefixOff + a.batch + 1] = static_cast<int>(cut);
+    if (tid == 0) plan[0] = a.plan_sig;
+  }
+  const int team = blockIdx.x * kWaves + wave;
+  int64_t cur, end;
+  if (team >= n_teams || !team_range(a, total, cut, team, n_teams, cur, end)) return;
+  int lo = 0, hi = a.batch;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (static_cast<int64_t>(prefix[mid]) * n_hbl <= cur) lo = mid; else hi = mid;
+  }
+  const int n_st = prefix[lo + 1] - prefix[lo];
+  const int st = static_cast<int>((cur - static_cast<int64_t>(prefix[lo]) * n_hbl) % n_st);
+  const int32_t* pages;
+  int L;
+  sequence_of(a, lo, pages, L);
+  const int st0 = first_token(a, L) / T;
+  const int ck = (((st0 + st) * T) >> a.bs_shift) >> 6;
+  const int n_pages = (L + a.block_size - 1) >> a.bs_shift;
+  plan[kPlanChunksOff + team * kWave + lane] = pages[min(ck * kWave + lane, n_pages - 1)];
+}
+
 template <typename QT, bool VL>
 __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int dv) {
   const int b = blockIdx.y;
+  if (a.plan != nullptr && a.plan[0] != a.plan_sig) return;   // the decode kernel wrote nothing and raised the flag
   merge_context<QT, VL>(a, dv, blockIdx.x, b, threadIdx.x, kThreads, a.ws_prefix[b], a.ws_prefix[b + 1],
                         a.ws_prefix[a.batch], a.pool_even != 0 ? a.ws_prefix[a.batch + 1] : 0);
 }
@@ -1662,6 +1739,7 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
     return n;
   }();
   a.n_workgroups = device_cu_count() * per_cu;
+  a.plan = nullptr;   // (plans are for the matrix-core kernel)
   const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * G * (D + 1);
   *need = kWsPartialsOff + part_floats * 4;
   if (plan_only) return XLLM_MI355_OK;
@@ -1712,38 +1790,28 @@ bool fold_merge_enabled() {
   return v != 0;
 }
 
-template <typename QT, bool FP8, bool VL = false, int D = 128>
-int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
-  // (head dim 256: the Q rows of the four pairs take 32 KB of the LDS, which leaves room for three stages each)
-  constexpr int NS = D == 256 ? kMfmaStages - 1 : kMfmaStages;
-  using Lay = MfmaLayout<NS, D>;
-  static_assert(Lay::kPrefixOff + (kMaxBatch + 1) * 4 <= 160 * 1024, "LDS of a CU");
-  auto kern = gqa_mfma_kernel<QT, FP8, NS, VL, D>;
-  static std::atomic<uint64_t> configured{0};
-  if (first_use_on_current_device(configured)) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             Lay::kPrefixOff + (kMaxBatch + 1) * 4);
-    if (e != hipSuccess) return static_cast<int>(e);
-  }
+// What a plan is made for: everything that the list and its ranges depend on besides the lengths themselves.
+int plan_signature(const GqaArgs& a, int stage_tokens) {
+  uint32_t h = 2166136261u;
+  const int v[] = {a.batch, a.n_kv_heads, a.group, stage_tokens, a.head_lock, a.pool_even, a.pool_odd, a.n_workgroups,
+                   a.window_left, a.bs_shift, a.indptr != nullptr ? 1 : 0};
+  for (int x : v) h = (h ^ static_cast<uint32_t>(x)) * 16777619u;
+  return static_cast<int>(h | 1u);
+}
+
+// The shape of the matrix-core kernel's launch: workers, workers side by side, pools.
+void configure_mfma(GqaArgs& a, bool fp8, int head_dim, bool varlen) {
   a.g_block = kMfmaHeads;
   const int n_wg = device_cu_count();  // the ring fills a CU's LDS: one workgroup each
   a.n_workgroups = n_wg * kWaves;      // independent workers = wavefronts
-  const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * (D + 1);
-  *need = kWsPartialsOff + part_floats * 4;
-  if (plan_only) return XLLM_MI355_OK;
-  if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
-  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_status) + kWsPartialsOff);
-  a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
-  a.ws_arrivals = reinterpret_cast<unsigned*>(reinterpret_cast<char*>(a.ws_status) + kWsCountersOff);
-  a.fold_merge = !VL && a.n_workgroups <= kWsMaxWorkers && fold_merge_enabled() ? 1 : 0;
+  a.fold_merge = !varlen && a.n_workgroups <= kWsMaxWorkers && fold_merge_enabled() ? 1 : 0;
   // Adjacent head blocks side by side: adjacent KV heads when a KV head has one head block; with several (more than
   // 16 query heads per KV head, or packed query chunks of more than 16 / group tokens) the blocks of one KV head, which
   // read the same rows, so that all but the first find them in L2.  (The in-kernel merge keeps its own bookkeeping
   // per worker.)
   a.head_lock = 1;
   if (a.fold_merge == 0) {
-    const int hb_per_kv = VL ? a.chunk_blocks : (a.group + kMfmaHeads - 1) / kMfmaHeads;
+    const int hb_per_kv = varlen ? a.chunk_blocks : (a.group + kMfmaHeads - 1) / kMfmaHeads;
     const int n_hb = a.n_kv_heads * hb_per_kv;
     const int want = head_lock_knob();
     for (int hl = kWaves; hl > 1; hl >>= 1)
@@ -1756,11 +1824,42 @@ int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool
   // 64 bytes keep the computing wavefronts busy enough that the XCDs end together with equal ranges: 134 us against
   // 139 us with the cut)
   a.pool_even = a.pool_odd = 0;
-  if (a.fold_merge == 0 && n_wg % 8 == 0 && xcd_pools_knob() != 0 && !(FP8 && D == 64)) {
+  if (a.fold_merge == 0 && n_wg % 8 == 0 && xcd_pools_knob() != 0 && !(fp8 && head_dim == 64)) {
     a.pool_even = xcd_pools_knob();
     a.pool_odd = 8;
   }
-  const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 1) * 4;
+}
+constexpr int stage_tokens(bool fp8, int head_dim) { return kStageBytes / 2 / (fp8 ? head_dim : 2 * head_dim); }
+
+template <typename QT, bool FP8, bool VL = false, int D = 128>
+int launch_gqa_mfma(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan_only, size_t* need) {
+  // (head dim 256: the Q rows of the four pairs take 32 KB of the LDS, which leaves room for three stages each)
+  constexpr int NS = D == 256 ? kMfmaStages - 1 : kMfmaStages;
+  using Lay = MfmaLayout<NS, D>;
+  static_assert(Lay::kPrefixOff + (kMaxBatch + 2) * 4 <= 160 * 1024, "LDS of a CU");
+  auto kern = gqa_mfma_kernel<QT, FP8, NS, VL, D>;
+  static std::atomic<uint64_t> configured{0};
+  if (first_use_on_current_device(configured)) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             Lay::kPrefixOff + (kMaxBatch + 2) * 4);
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
+  configure_mfma(a, FP8, D, VL);
+  const int n_wg = a.n_workgroups / kWaves;
+  const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * (D + 1);
+  *need = kWsPartialsOff + part_floats * 4;
+  if (plan_only) return XLLM_MI355_OK;
+  if (*need > workspace_bytes) return XLLM_MI355_EWORKSPACE;
+  a.ws_out = reinterpret_cast<float*>(reinterpret_cast<char*>(a.ws_status) + kWsPartialsOff);
+  a.ws_lse = a.ws_out + static_cast<size_t>(a.n_workgroups) * 2 * kMfmaHeads * D;
+  a.ws_arrivals = reinterpret_cast<unsigned*>(reinterpret_cast<char*>(a.ws_status) + kWsCountersOff);
+  if (VL || a.fold_merge != 0 || a.n_workgroups / a.head_lock > kPlanMaxTeams) a.plan = nullptr;
+  if (a.plan != nullptr) {   // the merge kernel reads the plan's prefix and cut
+    a.plan_sig = plan_signature(a, stage_tokens(FP8, D));
+    a.ws_prefix = const_cast<int*>(a.plan) + kPlanPrefixOff;
+  }
+  const size_t smem = Lay::kPrefixOff + (static_cast<size_t>(a.batch) + 2) * 4;
   launch_timed(kern, dim3(static_cast<unsigned>(n_wg)), dim3(kMfmaThreads), smem, stream, a);
   return static_cast<int>(hipGetLastError());
 }
@@ -1829,6 +1928,60 @@ int group_block(int group) {
 
 void set_fold_merge(int on) { g_fold_merge.store(on != 0 ? 1 : 0, std::memory_order_relaxed); }
 
+size_t gqa_plan_bytes() { return kPlanBytes; }
+
+int paged_decode_gqa_plan(void* plan, size_t plan_bytes, const PageAddressing& addr, int64_t batch, int64_t n_q_heads,
+                          int64_t n_kv_heads, int64_t head_dim, int64_t block_size, int cache_dtype,
+                          hipStream_t stream) {
+  if (batch == 0) return XLLM_MI355_OK;
+  if (plan == nullptr || (reinterpret_cast<uintptr_t>(plan) & 255) != 0 || plan_bytes < kPlanBytes)
+    return XLLM_MI355_EWORKSPACE;
+  const bool csr = addr.indptr != nullptr;
+  if (csr ? (addr.indices == nullptr || addr.last_page_len == nullptr)
+          : (addr.block_table == nullptr || addr.seq_lens == nullptr || addr.table_stride <= 0))
+    return XLLM_MI355_EINVAL;
+  if (batch < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || block_size <= 0 || n_q_heads % n_kv_heads != 0 ||
+      n_q_heads > 65535)
+    return XLLM_MI355_EINVAL;
+  if (head_dim != 64 && head_dim != 128 && head_dim != 256) return XLLM_MI355_ESHAPE;
+  const bool fp8 = cache_dtype == XLLM_MI355_FP8_E4M3;
+  GqaArgs a = {};
+  a.block_table = csr ? nullptr : addr.block_table;
+  a.seq_lens = csr ? nullptr : addr.seq_lens;
+  a.indptr = csr ? addr.indptr : nullptr;
+  a.indices = addr.indices;
+  a.last_page_len = csr ? addr.last_page_len : nullptr;
+  a.table_stride = addr.table_stride;
+  a.window_left = addr.window_left < 0 ? -1 : static_cast<int>(addr.window_left < 0x7fffffffLL ? addr.window_left : 0x7fffffffLL);
+  a.batch = static_cast<int>(batch);
+  a.n_q_heads = static_cast<int>(n_q_heads);
+  a.n_kv_heads = static_cast<int>(n_kv_heads);
+  a.group = static_cast<int>(n_q_heads / n_kv_heads);
+  a.block_size = static_cast<int>(block_size);
+  a.bs_shift = -1;
+  for (int s = 0; s < 31; ++s)
+    if ((1LL << s) == block_size) a.bs_shift = s;
+  // Shapes that the matrix-core kernel does not serve, and batches decoded in slices, take no plan: the planned
+  // entry point decodes them like the plain one.
+  if (batch > kMaxBatch || a.bs_shift < 4 || (fp8 && head_dim == 256) || !use_mfma_kernel()) return XLLM_MI355_OK;
+  configure_mfma(a, fp8, static_cast<int>(head_dim), false);
+  const int n_teams = a.n_workgroups / a.head_lock;
+  if (a.fold_merge != 0 || n_teams > kPlanMaxTeams) return XLLM_MI355_OK;
+  const int T = stage_tokens(fp8, static_cast<int>(head_dim));
+  a.plan_sig = plan_signature(a, T);
+  const dim3 grid(static_cast<unsigned>((n_teams + kWaves - 1) / kWaves));
+  const size_t smem = (static_cast<size_t>(kThreads) + a.batch + 1) * 4;
+  int* words = static_cast<int*>(plan);
+  switch (T) {
+    case 8: launch_timed(gqa_plan_kernel<8>, grid, dim3(kThreads), smem, stream, a, words, n_teams); break;
+    case 16: launch_timed(gqa_plan_kernel<16>, grid, dim3(kThreads), smem, stream, a, words, n_teams); break;
+    case 32: launch_timed(gqa_plan_kernel<32>, grid, dim3(kThreads), smem, stream, a, words, n_teams); break;
+    case 64: launch_timed(gqa_plan_kernel<64>, grid, dim3(kThreads), smem, stream, a, words, n_teams); break;
+    default: return XLLM_MI355_ESHAPE;
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
 size_t gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim) {
   // Upper bound over every kernel variant, independent of the batch: at most 8 workgroups per CU, 8 heads
   // per block (the matrix-core kernel: 4 workers per CU, 16 heads).
@@ -1865,6 +2018,7 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (q_token_stride * 2) % 16 != 0)
     return XLLM_MI355_EALIGN;
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0) return XLLM_MI355_EWORKSPACE;
+  if (addr.plan != nullptr && (reinterpret_cast<uintptr_t>(addr.plan) & 255) != 0) return XLLM_MI355_EWORKSPACE;
 
   const int group = static_cast<int>(n_q_heads / n_kv_heads);
   const bool packed = addr.cu_q != nullptr;  // several query tokens per sequence in the MFMA columns
@@ -1902,6 +2056,7 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     a.v_scale = v_scale;
     a.ws_status = static_cast<int*>(workspace);
     a.ws_prefix = reinterpret_cast<int*>(static_cast<char*>(workspace) + kWsHeaderBytes);
+    a.plan = !packed && batch <= kMaxBatch ? static_cast<const int*>(addr.plan) : nullptr;
     a.wait_spins = wait_spin_limit();
     a.window_left = addr.window_left < 0 ? -1 : static_cast<int>(addr.window_left < 0x7fffffffLL ? addr.window_left : 0x7fffffffLL);
     a.table_stride = addr.table_stride;

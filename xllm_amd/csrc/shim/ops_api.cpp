@@ -153,7 +153,7 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
                   const std::optional<torch::Tensor>& v_cache, std::optional<torch::Tensor>& output_lse,
                   const std::optional<torch::Tensor>& k_cache_quant_scale,
                   const std::optional<torch::Tensor>& v_cache_quant_scale, int64_t max_seq_len,
-                  int64_t window_size_left, float scale, bool return_lse) {
+                  int64_t window_size_left, float scale, bool return_lse, const std::optional<torch::Tensor>& plan) {
   TORCH_CHECK(v_cache.has_value() && v_cache->defined(), "GQA decode needs v_cache");
   check_decode_operands(query, output, k_cache, *v_cache, k_cache_quant_scale, v_cache_quant_scale);
   TORCH_CHECK(block_table.scalar_type() == torch::kInt32 && block_table.dim() == 2 && block_table.stride(1) == 1 &&
@@ -174,6 +174,18 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
   if (max_seq_len <= 0) max_seq_len = block_table.size(1) * k_cache.size(1);
   const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len);
   torch::Tensor ws = decode_workspace(query.device(), nbytes);
+  if (plan.has_value() && plan->defined()) {
+    TORCH_CHECK(plan->is_cuda() && plan->is_contiguous(), "plan must be the buffer of update_decode_plan");
+    const int rc = xllm_mi355_paged_decode_gqa_planned(
+        plan->data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache->data_ptr(), output.data_ptr(), lse,
+        block_table.data_ptr<int32_t>(), block_table.stride(0), seq_lens.data_ptr<int32_t>(), nullptr, nullptr, nullptr,
+        static_cast<const float*>(ptr_or_null(k_cache_quant_scale)),
+        static_cast<const float*>(ptr_or_null(v_cache_quant_scale)), B, Hq, k_cache.size(2), D, k_cache.size(1),
+        k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, window_size_left, scale, ws.data_ptr(),
+        static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
+    check_rc(rc, "xllm_mi355_paged_decode_gqa_planned");
+    return;
+  }
   const int rc = xllm_mi355_paged_decode_gqa(
       query.data_ptr(), k_cache.data_ptr(), v_cache->data_ptr(), output.data_ptr(), lse,
       block_table.data_ptr<int32_t>(), block_table.stride(0), seq_lens.data_ptr<int32_t>(),
@@ -187,7 +199,8 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
 void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache,
                       torch::Tensor paged_kv_indptr, torch::Tensor paged_kv_indices,
                       torch::Tensor paged_kv_last_page_len, int64_t window_left, double sm_scale,
-                      torch::Tensor output, std::optional<torch::Tensor>& output_lse, int64_t max_seq_len) {
+                      torch::Tensor output, std::optional<torch::Tensor>& output_lse, int64_t max_seq_len,
+                      const std::optional<torch::Tensor>& plan) {
   check_decode_operands(query, output, k_cache, v_cache, std::nullopt, std::nullopt);
   const int64_t B = query.size(0), Hq = query.size(1), D = query.size(2);
   for (const torch::Tensor* t : {&paged_kv_indptr, &paged_kv_indices, &paged_kv_last_page_len})
@@ -204,6 +217,17 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
   if (max_seq_len <= 0) max_seq_len = std::max<int64_t>(1, paged_kv_indices.numel()) * k_cache.size(1);
   const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len);
   torch::Tensor ws = decode_workspace(query.device(), nbytes);
+  if (plan.has_value() && plan->defined()) {
+    TORCH_CHECK(plan->is_cuda() && plan->is_contiguous(), "plan must be the buffer of update_decode_plan");
+    const int rc = xllm_mi355_paged_decode_gqa_planned(
+        plan->data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), lse, nullptr, 0,
+        nullptr, paged_kv_indptr.data_ptr<int32_t>(), paged_kv_indices.data_ptr<int32_t>(),
+        paged_kv_last_page_len.data_ptr<int32_t>(), nullptr, nullptr, B, Hq, k_cache.size(2), D, k_cache.size(1),
+        k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, window_left, static_cast<float>(sm_scale),
+        ws.data_ptr(), static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
+    check_rc(rc, "xllm_mi355_paged_decode_gqa_planned");
+    return;
+  }
   const int rc = xllm_mi355_paged_decode_gqa_csr(
       query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), lse,
       paged_kv_indptr.data_ptr<int32_t>(), paged_kv_indices.data_ptr<int32_t>(),
@@ -212,6 +236,56 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
       ws.data_ptr(), static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache),
       current_stream(query));
   check_rc(rc, "xllm_mi355_paged_decode_gqa_csr");
+}
+
+torch::Tensor update_decode_plan(const std::optional<torch::Tensor>& plan,
+                                 const std::optional<torch::Tensor>& block_table,
+                                 const std::optional<torch::Tensor>& seq_lens,
+                                 const std::optional<torch::Tensor>& paged_kv_indptr,
+                                 const std::optional<torch::Tensor>& paged_kv_indices,
+                                 const std::optional<torch::Tensor>& paged_kv_last_page_len,
+                                 int64_t num_qo_heads, int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                                 int64_t window_left, torch::ScalarType cache_dtype) {
+  auto defined = [](const std::optional<torch::Tensor>& t) { return t.has_value() && t->defined(); };
+  auto int32_device = [](const torch::Tensor& t) {
+    return t.is_cuda() && t.scalar_type() == torch::kInt32;
+  };
+  const bool csr = defined(paged_kv_indptr);
+  const torch::Tensor& anchor = csr ? *paged_kv_indptr : *seq_lens;
+  const int64_t nbytes = static_cast<int64_t>(xllm_mi355_paged_decode_plan_bytes());
+  torch::Tensor buf = defined(plan) ? *plan : torch::empty({nbytes}, anchor.options().dtype(torch::kUInt8));
+  TORCH_CHECK(buf.is_cuda() && buf.is_contiguous() && static_cast<int64_t>(buf.nbytes()) >= nbytes,
+              "plan must be a contiguous device buffer of xllm_mi355_paged_decode_plan_bytes() bytes");
+  int64_t B = 0;
+  const int32_t *table = nullptr, *lens = nullptr, *indptr = nullptr, *indices = nullptr, *last = nullptr;
+  int64_t stride = 0;
+  if (csr) {
+    TORCH_CHECK(defined(paged_kv_indices) && defined(paged_kv_last_page_len), "the CSR form needs all three arrays");
+    for (const torch::Tensor* t : {&*paged_kv_indptr, &*paged_kv_indices, &*paged_kv_last_page_len})
+      TORCH_CHECK(int32_device(*t) && t->is_contiguous(), "CSR arrays must be contiguous int32 device tensors");
+    B = paged_kv_last_page_len->numel();
+    TORCH_CHECK(paged_kv_indptr->numel() == B + 1, "CSR sizes");
+    indptr = paged_kv_indptr->data_ptr<int32_t>();
+    indices = paged_kv_indices->data_ptr<int32_t>();
+    last = paged_kv_last_page_len->data_ptr<int32_t>();
+  } else {
+    TORCH_CHECK(defined(block_table) && defined(seq_lens), "the block-table form needs the table and the lengths");
+    TORCH_CHECK(int32_device(*block_table) && block_table->dim() == 2 && block_table->stride(1) == 1 &&
+                    int32_device(*seq_lens) && seq_lens->is_contiguous() && block_table->size(0) == seq_lens->numel(),
+                "block_table must be int32 [B, W], seq_lens contiguous int32 [B]");
+    B = seq_lens->numel();
+    table = block_table->data_ptr<int32_t>();
+    stride = block_table->stride(0);
+    lens = seq_lens->data_ptr<int32_t>();
+  }
+  const int code = cache_dtype == torch::kFloat8_e4m3fn ? XLLM_MI355_FP8_E4M3
+                   : cache_dtype == torch::kFloat16     ? XLLM_MI355_FP16
+                                                        : XLLM_MI355_BF16;
+  const int rc = xllm_mi355_paged_decode_gqa_plan(buf.data_ptr(), static_cast<size_t>(buf.nbytes()), table, stride, lens,
+                                                  indptr, indices, last, B, num_qo_heads, num_kv_heads, head_dim,
+                                                  block_size, window_left, code, current_stream(anchor));
+  check_rc(rc, "xllm_mi355_paged_decode_gqa_plan");
+  return buf;
 }
 
 void paged_forward(const torch::Tensor& query, torch::Tensor& output, const torch::Tensor& k_cache,
@@ -602,13 +676,41 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> Mi355AttentionImpl::forw
                                        attn_metadata.is_causal, attn_metadata.max_seq_len,
                                        attn_metadata.max_query_len, window_left, k_scale, v_scale);
   } else {
-    // decode: one query token per sequence, a token attends to its whole context whatever is_causal says
+    // decode: one query token per sequence, a token attends to its whole context whatever is_causal says.
+    // With a PlanInfo in the metadata, layer 0 plans the step and every layer decodes from that plan
+    // (xllm/core/layers/cuda/flashinfer_attention.cpp:305-323 and the plan_info argument of its batch_decode call).
+    std::optional<torch::Tensor> plan = std::nullopt;
+    if (attn_metadata.plan_info != nullptr) {
+      AttentionMetadata planned_meta = attn_metadata;
+      planned_meta.block_table = block_table;
+      planned_meta.kv_seq_lens = kv_seq_lens;
+      flashinfer::update_decode_plan_info(attn_metadata.plan_info, planned_meta, k_cache.scalar_type(),
+                                          static_cast<int32_t>(num_heads_), static_cast<int32_t>(num_kv_heads_),
+                                          static_cast<int32_t>(head_size_), static_cast<int32_t>(k_cache.size(1)),
+                                          static_cast<int32_t>(window_left));
+      TORCH_CHECK(attn_metadata.plan_info->plan_info.defined(), "no layer 0 has planned this step");
+      plan = attn_metadata.plan_info->plan_info;
+    }
     xllm::kernel::mi355::batch_decode(query, k_cache, output, block_table, kv_seq_lens, v_cache, output_lse, k_scale,
-                                      v_scale, attn_metadata.max_seq_len, window_left, scale_, return_lse_);
+                                      v_scale, attn_metadata.max_seq_len, window_left, scale_, return_lse_, plan);
   }
   output = output.view({-1, num_heads_ * head_size_});
   return std::make_tuple(output, output_lse);
 }
+
+namespace flashinfer {
+void update_decode_plan_info(std::shared_ptr<PlanInfo> plan_info, const AttentionMetadata& attn_meta,
+                             c10::ScalarType key_dtype, int32_t num_qo_heads, int32_t num_kv_heads, int32_t head_dim,
+                             int32_t block_size, int32_t window_size_left) {
+  TORCH_CHECK(plan_info != nullptr && plan_info->layer_id != -1, "Need to set layer_id to PlanInfo.");
+  if (plan_info->layer_id != 0) return;
+  std::optional<torch::Tensor> old = std::nullopt;
+  if (plan_info->plan_info.defined()) old = plan_info->plan_info;
+  plan_info->plan_info = xllm::kernel::mi355::update_decode_plan(
+      old, attn_meta.block_table, attn_meta.kv_seq_lens, std::nullopt, std::nullopt, std::nullopt, num_qo_heads,
+      num_kv_heads, head_dim, block_size, window_size_left, key_dtype);
+}
+}  // namespace flashinfer
 
 }  // namespace xllm::layer
 
@@ -648,11 +750,20 @@ std::tuple<torch::Tensor, torch::Tensor> op_batch_decode(torch::Tensor query, to
                                                          torch::Tensor block_table, torch::Tensor seq_lens,
                                                          std::optional<torch::Tensor> k_scale,
                                                          std::optional<torch::Tensor> v_scale, int64_t max_seq_len,
-                                                         double scale) {
+                                                         double scale, std::optional<torch::Tensor> plan) {
   std::optional<torch::Tensor> lse;
   xllm::kernel::mi355::batch_decode(query, k_cache, output, block_table, seq_lens, v_cache, lse, k_scale, v_scale,
-                                    max_seq_len, /*window_size_left=*/-1, static_cast<float>(scale), /*return_lse=*/true);
+                                    max_seq_len, /*window_size_left=*/-1, static_cast<float>(scale), /*return_lse=*/true,
+                                    plan);
   return {output, lse.value()};
+}
+
+torch::Tensor op_update_decode_plan(torch::Tensor block_table, torch::Tensor seq_lens, int64_t num_qo_heads,
+                                    int64_t num_kv_heads, int64_t head_dim, int64_t block_size, int64_t window_left,
+                                    bool fp8_cache, std::optional<torch::Tensor> plan) {
+  return xllm::kernel::mi355::update_decode_plan(plan, block_table, seq_lens, std::nullopt, std::nullopt, std::nullopt,
+                                                 num_qo_heads, num_kv_heads, head_dim, block_size, window_left,
+                                                 fp8_cache ? torch::kFloat8_e4m3fn : torch::kBFloat16);
 }
 
 torch::Tensor op_lse_combine(torch::Tensor output, torch::Tensor shared_o, torch::Tensor shared_lse,
@@ -668,8 +779,14 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> op_attention_layer_forwa
     std::optional<torch::Tensor> k_cache_scale, std::optional<torch::Tensor> v_cache_scale, torch::Tensor slot_mapping,
     torch::Tensor block_table, torch::Tensor kv_seq_lens, std::optional<torch::Tensor> q_cu_seq_lens, int64_t max_seq_len,
     int64_t max_query_len, int64_t num_heads, int64_t head_size, int64_t num_kv_heads, double scale,
-    int64_t sliding_window, bool is_causal, bool return_lse) {
+    int64_t sliding_window, bool is_causal, bool return_lse, std::optional<torch::Tensor> plan, int64_t layer_id) {
   xllm::layer::AttentionMetadata meta;
+  if (layer_id >= 0) {  // the step's PlanInfo as this layer sees it: layer 0 fills `plan`, the others read it
+    TORCH_CHECK(plan.has_value() && plan->defined(), "a layer with a layer_id needs the step's plan buffer");
+    meta.plan_info = std::make_shared<xllm::layer::PlanInfo>();
+    meta.plan_info->layer_id = static_cast<int32_t>(layer_id);
+    meta.plan_info->plan_info = *plan;
+  }
   meta.kv_seq_lens = kv_seq_lens;
   meta.block_table = block_table;
   meta.slot_mapping = slot_mapping;
@@ -803,14 +920,17 @@ TORCH_LIBRARY(xllm_ops, m) {
   m.def("quant_to_paged_cache(Tensor slot_mapping, Tensor keys, Tensor values, Tensor(a!) key_cache, "
         "Tensor(b!) value_cache, Tensor k_scale, Tensor v_scale) -> Tensor");
   m.def("batch_decode(Tensor query, Tensor k_cache, Tensor v_cache, Tensor(a!) output, Tensor block_table, "
-        "Tensor seq_lens, Tensor? k_scale, Tensor? v_scale, int max_seq_len, float scale) -> (Tensor, Tensor)");
+        "Tensor seq_lens, Tensor? k_scale, Tensor? v_scale, int max_seq_len, float scale, Tensor? plan=None) -> (Tensor, Tensor)");
+  m.def("update_decode_plan(Tensor block_table, Tensor seq_lens, int num_qo_heads, int num_kv_heads, int head_dim, "
+        "int block_size, int window_left, bool fp8_cache, Tensor(a!)? plan=None) -> Tensor");
   m.def("mla_dense_decode(Tensor q_nope, Tensor q_pe, Tensor k_cache, Tensor seqlens_k, Tensor block_table, "
         "int head_size_v, float softmax_scale, bool is_causal=False) -> (Tensor, Tensor)");
   m.def("lse_combine(Tensor(a!) output, Tensor shared_o, Tensor shared_lse, Tensor unshared_o, Tensor unshared_lse) -> Tensor");
   m.def("attention_layer_forward(Tensor query, Tensor key, Tensor value, Tensor(a!) k_cache, Tensor(b!) v_cache, "
         "Tensor? k_cache_scale, Tensor? v_cache_scale, Tensor slot_mapping, Tensor block_table, Tensor kv_seq_lens, "
         "Tensor? q_cu_seq_lens, int max_seq_len, int max_query_len, int num_heads, int head_size, int num_kv_heads, "
-        "float scale, int sliding_window, bool is_causal, bool return_lse) -> (Tensor, Tensor?)");
+        "float scale, int sliding_window, bool is_causal, bool return_lse, Tensor(c!)? plan=None, int layer_id=-1) "
+        "-> (Tensor, Tensor?)");
   m.def("merge_dcp_attention_shards(Tensor partial_outputs, Tensor partial_lse) -> (Tensor, Tensor)");
   m.def("paged_forward(Tensor query, Tensor(a!) output, Tensor k_cache, Tensor v_cache, Tensor block_table, "
         "Tensor kv_seq_lens, Tensor q_cu_seq_lens, float scale, bool is_causal, int max_seq_len, int max_query_len) -> Tensor");
@@ -834,6 +954,7 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("reshape_paged_cache", &op_reshape_paged_cache);
   m.impl("quant_to_paged_cache", &op_quant_to_paged_cache);
   m.impl("batch_decode", &op_batch_decode);
+  m.impl("update_decode_plan", &op_update_decode_plan);
   m.impl("mla_dense_decode", &op_mla_dense_decode);
   m.impl("lse_combine", &op_lse_combine);
   m.impl("attention_layer_forward", &op_attention_layer_forward);

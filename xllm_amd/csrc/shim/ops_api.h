@@ -61,7 +61,22 @@ void batch_decode(const torch::Tensor& query,        // [B, Hq, D]
                   std::optional<torch::Tensor>& output_lse,  // [B, Hq, 1] fp32, natural log
                   const std::optional<torch::Tensor>& k_cache_quant_scale,
                   const std::optional<torch::Tensor>& v_cache_quant_scale,
-                  int64_t max_seq_len, int64_t window_size_left, float scale, bool return_lse);
+                  int64_t max_seq_len, int64_t window_size_left, float scale, bool return_lse,
+                  const std::optional<torch::Tensor>& plan = std::nullopt);
+
+// The plan of a decode step, made once and taken by the decode calls of every layer (`plan` above and in
+// batch_decode_csr): the part of update_decode_plan_info (xllm/core/layers/cuda/flashinfer_planinfo.cpp:248-264),
+// whose result the reference hands to cuda::batch_decode as plan_info (cuda_ops_api.h:128-129).  One small launch;
+// `plan` is reused when given (a captured step must reuse it), else allocated.  Either the block table with the
+// lengths or the three CSR arrays; cache_dtype is the dtype of the KV cache.
+torch::Tensor update_decode_plan(const std::optional<torch::Tensor>& plan,
+                                 const std::optional<torch::Tensor>& block_table,
+                                 const std::optional<torch::Tensor>& seq_lens,
+                                 const std::optional<torch::Tensor>& paged_kv_indptr,
+                                 const std::optional<torch::Tensor>& paged_kv_indices,
+                                 const std::optional<torch::Tensor>& paged_kv_last_page_len,
+                                 int64_t num_qo_heads, int64_t num_kv_heads, int64_t head_dim, int64_t block_size,
+                                 int64_t window_left, torch::ScalarType cache_dtype);
 
 // The CSR form, with the arguments of xllm::kernel::cuda::batch_decode (cuda_ops_api.h:128-144) that are not
 // FlashInfer's own (uri, plan_info, the three workspace buffers, use_tensor_core, qo_indptr), in its order;
@@ -69,7 +84,8 @@ void batch_decode(const torch::Tensor& query,        // [B, Hq, D]
 void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor v_cache,
                       torch::Tensor paged_kv_indptr, torch::Tensor paged_kv_indices,
                       torch::Tensor paged_kv_last_page_len, int64_t window_left, double sm_scale,
-                      torch::Tensor output, std::optional<torch::Tensor>& output_lse, int64_t max_seq_len);
+                      torch::Tensor output, std::optional<torch::Tensor>& output_lse, int64_t max_seq_len,
+                      const std::optional<torch::Tensor>& plan = std::nullopt);
 
 // Short query chunks against paged KV: the decode branch of FlashAttentionImpl::paged_forward
 // (xllm/core/layers/dcu/flash_attention.cpp:447-545).  query / output packed [T, Hq, D]; kv_seq_lens [B] are the
@@ -208,6 +224,13 @@ class KVCache final {
 };
 
 namespace layer {
+// xllm::layer::PlanInfo (xllm/core/layers/common/attention_metadata.h:49-53): the layer that holds it and the plan
+// (here the device buffer of update_decode_plan instead of FlashInfer's integer array; no kernel uri).
+struct PlanInfo {
+  int32_t layer_id = -1;
+  torch::Tensor plan_info;
+};
+
 // xllm::layer::AttentionMetadata (xllm/core/layers/common/attention_metadata.h:99-156), decode subset.
 struct AttentionMetadata {
   torch::Tensor q_cu_seq_lens;
@@ -228,7 +251,18 @@ struct AttentionMetadata {
   torch::Tensor paged_kv_indices;
   torch::Tensor paged_kv_last_page_len;
   bool enable_cuda_graph = false;
+  // attention_metadata.h:163; null: every layer's decode call derives its schedule itself
+  std::shared_ptr<PlanInfo> plan_info;
 };
+
+namespace flashinfer {
+// update_decode_plan_info (xllm/core/layers/cuda/flashinfer_planinfo.cpp:248-264): every layer calls it, layer 0
+// plans.  The plan is a launch on the current stream, so a captured step re-plans on every replay and
+// enable_cuda_graph needs no host-side update before a replay.
+void update_decode_plan_info(std::shared_ptr<PlanInfo> plan_info, const AttentionMetadata& attn_meta,
+                             c10::ScalarType key_dtype, int32_t num_qo_heads, int32_t num_kv_heads, int32_t head_dim,
+                             int32_t block_size, int32_t window_size_left);
+}  // namespace flashinfer
 
 // xllm::layer::BaseAttentionImpl (xllm/core/layers/dcu/base_attention_impl.h:30-57), unchanged.
 class BaseAttentionImpl {

@@ -214,19 +214,59 @@ def _decode_common(query, k_cache, output, v_cache=None, k_scale=None, v_scale=N
         raise TypeError("the cache dtype must equal the query dtype (or be fp8)")
 
 
+def update_decode_plan_info(num_qo_heads, num_kv_heads, head_dim, block_size, cache_dtype, block_table=None,
+                            seq_lens=None, paged_kv_indptr=None, paged_kv_indices=None, paged_kv_last_page_len=None,
+                            window_left=-1, plan=None):
+    """The plan of a decode step, made once and handed to the decode calls of all layers (plan=...): the role of
+    update_decode_plan_info, which the reference runs at layer 0 only (layers/cuda/flashinfer_planinfo.cpp:248-264).
+    Takes the step's block table and lengths, or its CSR arrays; cache_dtype is the dtype of the KV cache.
+    Returns the plan (a device buffer; pass one back in to reuse it, as a captured step must)."""
+    csr = paged_kv_indptr is not None
+    dev = _require_cuda(block_table, seq_lens, paged_kv_indptr, paged_kv_indices, paged_kv_last_page_len, plan)
+    lib = capi.lib()
+    nbytes = int(lib.xllm_mi355_paged_decode_plan_bytes())
+    if plan is None:
+        plan = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    if plan.dtype != torch.uint8 or plan.numel() < nbytes or not plan.is_contiguous():
+        raise ValueError(f"plan must be a contiguous uint8 buffer of {nbytes} bytes")
+    if csr:
+        B = paged_kv_indptr.numel() - 1
+        for t, n in ((paged_kv_indptr, B + 1), (paged_kv_last_page_len, B)):
+            if t.dtype != torch.int32 or t.numel() != n or not t.is_contiguous():
+                raise ValueError("CSR arrays must be contiguous int32 of the documented sizes")
+        if paged_kv_indices.dtype != torch.int32 or not paged_kv_indices.is_contiguous():
+            raise ValueError("paged_kv_indices must be contiguous int32")
+        table, stride, lens = None, 0, None
+    else:
+        B = seq_lens.numel()
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1:
+            raise ValueError("block_table must be int32 [B, W] with unit column stride")
+        if seq_lens.dtype != torch.int32 or not seq_lens.is_contiguous() or block_table.shape[0] != B:
+            raise ValueError("seq_lens must be contiguous int32 [B], one per block_table row")
+        table, stride, lens = block_table, block_table.stride(0), seq_lens
+    code = capi.FP8_E4M3 if cache_dtype == torch.float8_e4m3fn else (capi.FP16 if cache_dtype == torch.float16 else capi.BF16)
+    rc = lib.xllm_mi355_paged_decode_gqa_plan(
+        plan.data_ptr(), plan.numel(), _ptr(table), stride, _ptr(lens), _ptr(paged_kv_indptr), _ptr(paged_kv_indices),
+        _ptr(paged_kv_last_page_len), B, num_qo_heads, num_kv_heads, head_dim, block_size, int(window_left), code,
+        _stream(dev))
+    capi.check(rc, "xllm_mi355_paged_decode_gqa_plan")
+    return plan
+
+
 def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, output_lse=None,
                  k_cache_quant_scale=None, v_cache_quant_scale=None, scale=None, return_lse=False,
-                 max_seq_len=0, window_left=-1):
+                 max_seq_len=0, window_left=-1, plan=None):
     """Block-table paged decode.  Argument order and meaning follow mlu::batch_decode
     (mlu_ops_api.h:127) restricted to what npu::batch_decode (npu_ops_api.h:46) also has.
     query/output [B, Hq, D]; caches [P, bs, Hkv, D]; block_table [B, W] int32; seq_lens [B] int32.
     window_left >= 0: sliding window, the query attends to the last window_left + 1 tokens of its context
     (sliding_window_ of layers/dcu/flash_attention.cpp:484).
+    plan: the step's plan from update_decode_plan_info (same tables, lengths, heads and window), or None.
     Returns (output, lse or None) with lse [B, Hq, 1] fp32 natural log."""
     if v_cache is None:
         raise ValueError("GQA decode needs v_cache; the latent-KV variant is dense_decode")
     dev = _require_cuda(query, k_cache, v_cache, output, block_table, seq_lens, output_lse,
-                        k_cache_quant_scale, v_cache_quant_scale)
+                        k_cache_quant_scale, v_cache_quant_scale, plan)
     _decode_common(query, k_cache, output, v_cache, k_cache_quant_scale, v_cache_quant_scale)
     B, Hq, D = query.shape
     P, bs, Hkv, _ = k_cache.shape
@@ -248,6 +288,15 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     lib = capi.lib()
     nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len)
     ws = decode_workspace(dev, nbytes)
+    if plan is not None:
+        rc = lib.xllm_mi355_paged_decode_gqa_planned(
+            plan.data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(lse),
+            block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), None, None, None,
+            _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D, bs, P,
+            query.stride(0), output.stride(0), max_seq_len, int(window_left), float(scale), ws.data_ptr(), ws.numel(),
+            _dtype_code(query), _dtype_code(k_cache), _stream(dev))
+        capi.check(rc, "xllm_mi355_paged_decode_gqa_planned")
+        return output, lse
     rc = lib.xllm_mi355_paged_decode_gqa(
         query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(lse),
         block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(),
@@ -260,12 +309,13 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
 
 def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
                      paged_kv_last_page_len, window_left, sm_scale, output, output_lse=None, max_seq_len=0,
-                     k_cache_quant_scale=None, v_cache_quant_scale=None):
+                     k_cache_quant_scale=None, v_cache_quant_scale=None, plan=None):
     """CSR paged decode: cuda::batch_decode (cuda_ops_api.h:128-144) without the FlashInfer
-    uri / plan_info / workspace arguments; window_left as there (-1 = the whole context).  max_seq_len bounds the longest context; 0 means
+    uri / workspace arguments; plan plays the part of its plan_info (update_decode_plan_info; None = the launch
+    derives its schedule itself); window_left as there (-1 = the whole context).  max_seq_len bounds the longest context; 0 means
     "all pages of the call could belong to one sequence"."""
     dev = _require_cuda(query, k_cache, v_cache, output, paged_kv_indptr, paged_kv_indices,
-                        paged_kv_last_page_len, output_lse, k_cache_quant_scale, v_cache_quant_scale)
+                        paged_kv_last_page_len, output_lse, k_cache_quant_scale, v_cache_quant_scale, plan)
     _decode_common(query, k_cache, output, v_cache, k_cache_quant_scale, v_cache_quant_scale)
     B, Hq, D = query.shape
     P, bs, Hkv, _ = k_cache.shape
@@ -279,6 +329,15 @@ def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
     lib = capi.lib()
     nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len)
     ws = decode_workspace(dev, nbytes)
+    if plan is not None:
+        rc = lib.xllm_mi355_paged_decode_gqa_planned(
+            plan.data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
+            _ptr(output_lse), None, 0, None, paged_kv_indptr.data_ptr(), paged_kv_indices.data_ptr(),
+            paged_kv_last_page_len.data_ptr(), _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D,
+            bs, P, query.stride(0), output.stride(0), max_seq_len, int(window_left), float(sm_scale), ws.data_ptr(),
+            ws.numel(), _dtype_code(query), _dtype_code(k_cache), _stream(dev))
+        capi.check(rc, "xllm_mi355_paged_decode_gqa_planned")
+        return output
     rc = lib.xllm_mi355_paged_decode_gqa_csr(
         query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(output_lse),
         paged_kv_indptr.data_ptr(), paged_kv_indices.data_ptr(), paged_kv_last_page_len.data_ptr(),
