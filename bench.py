@@ -44,6 +44,8 @@ def parse_args():
                          "gqa_d64 | gqa_d64_fp8 | gqa_d256 | mla_tp8 (side workloads)")
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline (and with it the parity check)")
+    ap.add_argument("--no-planned", action="store_true",
+                    help="skip the second timed loop (the GQA step with the plan made once per step)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run only the plain stream_read / stream_copy kernels over 1 GiB (counter calibration)")
@@ -351,7 +353,7 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     # ---- the same step as the layers after the first see it when the step was planned once (not the headline:
     # `value` above is the self-contained call, which derives its schedule in every launch)
     planned = None
-    if not cfg.mla:
+    if not cfg.mla and not args.no_planned:
         plan = torch.empty(lib.xllm_mi355_paged_decode_plan_bytes(), dtype=torch.uint8, device=dev)
         plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), None, None, None, cfg.batch,
                      cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, -1, code[cache_dt], stream)

@@ -71,6 +71,15 @@ def test_whole_batch_full_size_parity(device, name):
         out, lse = ops.batch_decode(inp.q, kg, out, lay.block_table.to(device), lay.seq_lens.to(device), v_cache=vg,
                                     k_cache_quant_scale=ks, v_cache_quant_scale=vs, scale=cfg.scale,
                                     return_lse=True, max_seq_len=max_len)
+        # the same step from a plan made once (as the layers after the first see it): bit-identical
+        plan = ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                           block_table=lay.block_table.to(device), seq_lens=lay.seq_lens.to(device))
+        out_p, lse_p = ops.batch_decode(inp.q, kg, torch.empty_like(inp.q), lay.block_table.to(device),
+                                        lay.seq_lens.to(device), v_cache=vg, k_cache_quant_scale=ks,
+                                        v_cache_quant_scale=vs, scale=cfg.scale, return_lse=True, max_seq_len=max_len,
+                                        plan=plan)
+        assert torch.equal(out_p, out) and torch.equal(lse_p, lse), "planned decode differs from the plain one"
+        assert ops.decode_status(device) == 0
     torch.cuda.synchronize()
     out, lse = out.cpu(), lse.cpu().view(cfg.batch, cfg.n_q_heads)
 

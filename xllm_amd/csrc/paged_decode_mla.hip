@@ -1419,6 +1419,12 @@ constexpr int kW4Threads = 256;
 // At the start of a run the Q rows of the 128 heads pass through the ring and the P^T area on their way into the
 // registers: latent parts at a pitch of 1040 bytes (16 lanes that read 16 bytes of 16 rows hit 64 different banks),
 // then the rope parts.  The small arrays sit behind them.
+// What the schedule of mla_decode_w4_kernel divides: sub-tiles.  The loop runs sub-tile by sub-tile, so a range may
+// end at any of them, and the workgroups' shares differ by one sub-tile at most instead of one 64-token tile.
+#ifndef XLLM_W4_ITEM
+#define XLLM_W4_ITEM 32
+#endif
+constexpr int kW4Item = XLLM_W4_ITEM;
 constexpr int kW4QRow = kDL * 2 + 16;
 constexpr int kW4QRopeOff = kHeadsPerWg16 * kW4QRow;
 constexpr int kW4QEnd = kW4QRopeOff + kHeadsPerWg16 * kDR * 2;
@@ -1482,7 +1488,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     const int per = (a.batch + kW4Threads - 1) / kW4Threads;
     const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
     int local = 0;
-    auto span_of = [&](int len) { return len > 0 ? tiles_of(len) + a.run_cost : 0; };
+    auto span_of = [&](int len) { return len > 0 ? (len + kW4Item - 1) / kW4Item + a.run_cost : 0; };
     for (int b = lo; b < hi; ++b) local += span_of(a.seq_lens[b]);
     tmp[tid] = local;
     __syncthreads();
@@ -1539,8 +1545,8 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     if (run_tiles <= 0) continue;   // (the range ends inside the allowance in front of this context's tiles)
     const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
     const int L = __builtin_amdgcn_readfirstlane(a.seq_lens[b]);
-    const int t_begin = tile0 * kTile;
-    const int t_end = min(L, (tile0 + run_tiles) * kTile);
+    const int t_begin = tile0 * kW4Item;
+    const int t_end = min(L, (tile0 + run_tiles) * kW4Item);
     const int n_sub = (t_end - t_begin + kSubTok - 1) / kSubTok;
     const int n_pages = (L + a.block_size - 1) >> a.bs_shift;
 
@@ -2985,7 +2991,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       const int v = e ? atoi(e) : -1;
       return v >= 0 && v <= 64 ? v : 4;
     }();
-    a.run_cost = w4 ? run_cost : 0;
+    a.run_cost = w4 ? run_cost * (kTile / kW4Item) : 0;
 
     const dim3 grid(static_cast<unsigned>(a.n_teams * a.n_hb));
     if (pairs) {
