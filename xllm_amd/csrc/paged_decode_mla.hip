@@ -2050,19 +2050,24 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     }
     __syncthreads();
     // Output rows of a whole context go out head by head (COMPLETE).  Partial rows go out as the tiles they are in the
-    // registers, [16-head block][wavefront][dim block][lane][4 floats]: every store instruction then writes 1 KB in
-    // one piece.  Head by head it writes sixteen pieces of 64 bytes, and the burst of partial rows that ends a launch
-    // takes twice as long to issue (it is bound by the number of write requests, not by their bytes).
+    // registers, [16-head block][wavefront][pair of dim blocks][lane][2 x 4 values]: every store instruction then
+    // writes 1 KB in one piece.  Head by head it writes sixteen pieces of 64 bytes, and the burst of partial rows that
+    // ends a launch takes twice as long to issue (it is bound by the number of write requests, not by their bytes).
+    // A partial row is normalised (a convex combination of V rows, like the output), so it is stored in the output's
+    // own 16-bit type: half the stores here, half the bytes for the merge kernel, whose time is reading them; the
+    // LSEs stay fp32.
 #define XLLM_W4_OUT(DB, HB, R0, R1, R2, R3)                                                          \
   {                                                                                                  \
     f32x4 t;                                                                                         \
     XLLM_W4_GET(R0, R1, R2, R3, t);                                                                  \
     t *= inv;                                                                                        \
+    const u32x2 w = {QT::pack(t[0], t[1]), QT::pack(t[2], t[3])};                                    \
     if (COMPLETE) {                                                                                  \
-      const u32x2 w = {QT::pack(t[0], t[1]), QT::pack(t[2], t[3])};                                  \
       *reinterpret_cast<u32x2*>(dst + DB * 32) = w;                                                  \
+    } else if ((DB & 1) == 0) {                                                                      \
+      held = w;                                                                                      \
     } else {                                                                                         \
-      *reinterpret_cast<f32x4*>(dst + DB * 1024) = t;                                                \
+      *reinterpret_cast<u32x4*>(dst + (DB >> 1) * 1024) = u32x4{held[0], held[1], w[0], w[1]};       \
     }                                                                                                \
   }
 #define XLLM_W4_OUT_ROW(HB, ROW)                                                                     \
@@ -2070,8 +2075,9 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     const int hd = head0 + HB * 16 + c16e;                                                           \
     if (HB < n16 && hd < H) {                                                                        \
       const float inv = fac[HB * 16 + c16e];                                                         \
+      u32x2 held = {0u, 0u};                                                                         \
       char* dst = COMPLETE ? a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + wave * 128 + 4 * ge) * 2 \
-                           : tiles + (HB * 4 + wave) * 8192;                                         \
+                           : tiles + (HB * 4 + wave) * 4096;                                         \
       ROW(XLLM_W4_OUT)                                                                               \
     }                                                                                                \
   }
@@ -2086,7 +2092,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
   XLLM_W4_OUT_ROW(7, XLLM_W4_ROW7)
     // (16-head blocks of this workgroup's 128 heads: block hb128 * 8 + HB of the slot)
     char* tiles = reinterpret_cast<char*>(a.ws_out) +
-                  ((static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * a.slot_heads + head0) * (kDL * 4) + ln * 16;
+                  ((static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * a.slot_heads + head0) * (kDL * 2) + ln * 16;
     if (complete) {
       constexpr bool COMPLETE = true;
       XLLM_W4_OUT_ROWS
@@ -2801,15 +2807,15 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
                        : (static_cast<int64_t>(t_first) * r) % n;
   // (a range that starts in front of the context holds the last tile of an earlier one)
   const int slot_first = team_start(t_first, total, n) < front ? 1 : 0;
-  const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 4;
-  const char* tiles = reinterpret_cast<const char*>(a.ws_out) + (hb * 4 + w) * 8192 + lane * 16;
+  const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 2;
+  const char* tiles = reinterpret_cast<const char*>(a.ws_out) + (hb * 4 + w) * 4096 + lane * 16;
   float M = kNegBig, W = 0.0f;
   f32x4 O[8];
 #pragma unroll
   for (int db = 0; db < 8; ++db) O[db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   for (int tb = t_first; tb <= t_last; tb += 4) {
     float lse[4];
-    f32x4 x[4][8];
+    u32x4 x[4][4];   // pairs of dim blocks, 16-bit values
     bool on[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -2821,8 +2827,8 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
       const int64_t slot = static_cast<int64_t>(t) * 2 + (t == t_first ? slot_first : 0);
       lse[k] = on[k] ? a.ws_lse[slot * H + hd] : kNegBig;
 #pragma unroll
-      for (int db = 0; db < 8; ++db)
-        x[k][db] = on[k] ? *reinterpret_cast<const f32x4*>(tiles + slot * slot_bytes + db * 1024) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int dp = 0; dp < 4; ++dp)
+        x[k][dp] = on[k] ? *reinterpret_cast<const u32x4*>(tiles + slot * slot_bytes + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
     }
     const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
     const float keep = fast_exp2(M - m_new);
@@ -2834,7 +2840,11 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
       const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
       W += e;
 #pragma unroll
-      for (int db = 0; db < 8; ++db) O[db] += e * x[k][db];
+      for (int dp = 0; dp < 4; ++dp) {
+        const u32x4 v = x[k][dp];
+        O[2 * dp] += e * f32x4{QT::lo(v[0]), QT::hi(v[0]), QT::lo(v[1]), QT::hi(v[1])};
+        O[2 * dp + 1] += e * f32x4{QT::lo(v[2]), QT::hi(v[2]), QT::lo(v[3]), QT::hi(v[3])};
+      }
     }
     M = m_new;
   }
