@@ -70,6 +70,15 @@ def test_planned_decode_over_shapes_windows_and_empty_sequences(device):
         _both(inp, kg, vg, device, ks, vs, lens=torch.zeros_like(lens))
 
 
+def test_batches_decoded_in_slices_and_tiny_batches_with_a_plan(device):
+    # more sequences than one launch takes (the plan is not used then), and fewer work items than workers
+    for batch, hi in ((2100, 40), (1, 5), (3, 70)):
+        cfg = workloads.DecodeConfig(f"plan_b{batch}", batch, 32, 8, 128, 16, 1, hi)
+        inp = workloads.make_inputs(cfg, 500 + batch, device=device)
+        kg, vg, _, _ = fill_caches_gpu(inp, device)
+        _both(inp, kg, vg, device)
+
+
 def test_planned_decode_in_csr_form(device):
     cfg = workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=37, len_lo=1, len_hi=3000)
     inp = workloads.make_inputs(cfg, 21, device=device)
