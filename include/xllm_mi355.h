@@ -228,7 +228,8 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
  * was made with: make it again when any of them changes (every decode step).  Shapes that the matrix-core kernel
  * does not serve take no plan and are decoded as by the plain entry points.  A planned call whose shape differs
  * from the plan's writes no output and raises a flag that xllm_mi355_decode_status reports as XLLM_MI355_EPLAN;
- * lengths or tables that changed under the same shape are not detected.  Plan and planned calls are plain
+ * lengths or tables that changed under the same shape are not detected (the reads of such a call stay inside the
+ * tables and caches; its results are undefined).  Plan and planned calls are plain
  * launches on `stream` (legal under graph capture; a replay plans again from the current lengths).
  */
 size_t xllm_mi355_paged_decode_plan_bytes(void);

@@ -962,7 +962,8 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // into the chunk buffer at byte offset off
   auto issue_chunk = [&](const CtxCursor& cu, int ck, u32 off) {
     const int n_pages = (cu.L + a.block_size - 1) >> a.bs_shift;
-    dma4(cu.pages + min(ck * kWave + lane, n_pages - 1), page_lds + off);
+    // (never in front of the table: with a plan made for other lengths a context may have no pages here)
+    dma4(cu.pages + max(0, min(ck * kWave + lane, n_pages - 1)), page_lds + off);
   };
 
   // byte offset of the lane's 16 bytes from the first row of a stage: row 4i + g, chunk swizzled
@@ -1702,7 +1703,7 @@ __global__ __launch_bounds__(kThreads) void gqa_plan_kernel(GqaArgs a, int* plan
   const int st0 = first_token(a, L) / T;
   const int ck = (((st0 + st) * T) >> a.bs_shift) >> 6;
   const int n_pages = (L + a.block_size - 1) >> a.bs_shift;
-  plan[kPlanChunksOff + team * kWave + lane] = pages[min(ck * kWave + lane, n_pages - 1)];
+  plan[kPlanChunksOff + team * kWave + lane] = pages[max(0, min(ck * kWave + lane, n_pages - 1))];
 }
 
 template <typename QT, bool VL>
