@@ -46,6 +46,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline (and with it the parity check)")
     ap.add_argument("--no-planned", action="store_true",
                     help="skip the second timed loop (the GQA step with the plan made once per step)")
+    ap.add_argument("--graph", action="store_true",
+                    help="add a third timed loop: the step captured in a HIP graph and replayed (graph_replay in the line)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run only the plain stream_read / stream_copy kernels over 1 GiB (counter calibration)")
@@ -386,6 +388,36 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
                    "ms_per_step": p_elapsed / args.steps * 1e3, "plan_kernel_ms": plan_ms[0] if plan_ms else None,
                    "bit_identical": bool(torch.equal(plain_out, out))}
 
+    # ---- the same step captured once in a HIP graph and replayed, as the reference's graph executor runs a decode
+    # step (not the headline either: `value` is the eager loop above)
+    graph_replay = None
+    if args.graph:
+        ref_out = out.clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            cs = torch.cuda.current_stream(dev).cuda_stream
+            rc = reshape_fn(*(reshape_args[:-1] + (cs,)))
+            rc2 = decode_fn(*(decode_args[:-1] + (cs,)))
+        if rc or rc2:
+            capi.check(rc or rc2, "bench captured step")
+        t_settle = time.perf_counter()   # (the capture left the GPU idle: let the clocks settle again)
+        while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+            for _ in range(20):
+                graph.replay()
+            torch.cuda.synchronize()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        g_elapsed = time.perf_counter() - t0
+        graph_replay = {"ms_per_step": g_elapsed / args.steps * 1e3,
+                        "tokens_per_s": cfg.batch / (g_elapsed / args.steps),
+                        "bit_identical": bool(torch.equal(ref_out, out))}
+        del graph
+
     ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = cfg.batch / (ms_per_step * 1e-3)
 
@@ -448,6 +480,8 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
             / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,
     }
+    if graph_replay is not None:
+        result["graph_replay"] = graph_replay
     if not args.no_cpu_baseline:
         result["cpu_baseline"], result["parity"] = cpu_baseline(
             inp, k_cache, v_cache, k_scale, v_scale, out.view(cfg.batch, cfg.n_q_heads, cfg.dv), args.cpu_sample,
