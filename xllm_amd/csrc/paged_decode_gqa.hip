@@ -109,6 +109,14 @@ struct GqaArgs {
   // instead of three in a row (lengths -> prefix -> pages of the range's first context) before the first row moves.
   const int* plan;
   int plan_sig;       // what the plan must have been made for (plan_signature), checked against the plan's own word
+  // Matrix-core kernel: output rows and partial rows leave with non-temporal stores (written through, no line kept in
+  // L2).  With ordinary stores a launch that ends many runs (many sequences, many heads) has workers that are held up
+  // after a run's stores and at their exit: on 256 sequences x 64 heads the last worker leaves at 487-491 us instead
+  // of 502-507 us and the launch takes 2 % less; all stores have to be non-temporal for that (only those in the
+  // middle of a range, or only those at its end, changed nothing).  Launches with few run ends lose 1-1.5 % (64
+  // sequences x 32 heads: 91.1 -> 92.3 us, and the merge kernel, which then finds no partial in L2, 5.2 -> 5.5 us), so
+  // the host turns it on from 8192 output rows (sequences x heads) per launch.
+  int stream_stores;
   int wait_spins;     // bound of the polls of one wavefront of a pair on the other
   int window_left;    // sliding window: the query (position L - 1) attends to positions >= L - 1 - window_left; < 0: all
   float scale_log2;   // sm_scale * log2(e)
@@ -1436,19 +1444,41 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       if (head_on && complete) {
         char* op = VL ? a.out + out_off + 4 * g * 2
                       : a.out + cc.b * a.out_stride_bytes + (static_cast<int64_t>(hq) * D + 4 * g) * 2;
+        if (a.stream_stores != 0) {
+          // (behind an offset the compiler cannot see through, store by store: it otherwise folds the stores of the two
+          // branches into one sequence and drops the hint)
+          int zero = 0;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          const u32x2 w = {QT::pack(o[mb][0] * inv, o[mb][1] * inv), QT::pack(o[mb][2] * inv, o[mb][3] * inv)};
-          *reinterpret_cast<u32x2*>(op + mb * 32) = w;
+          for (int mb = 0; mb < MB; ++mb) {
+            const u32x2 w = {QT::pack(o[mb][0] * inv, o[mb][1] * inv), QT::pack(o[mb][2] * inv, o[mb][3] * inv)};
+            asm volatile("" : "+s"(zero));
+            __builtin_nontemporal_store(w, reinterpret_cast<u32x2*>(op + zero + mb * 32));
+          }
+        } else {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            const u32x2 w = {QT::pack(o[mb][0] * inv, o[mb][1] * inv), QT::pack(o[mb][2] * inv, o[mb][3] * inv)};
+            *reinterpret_cast<u32x2*>(op + mb * 32) = w;
+          }
         }
       }
       const bool shared = !VL && a.fold_merge != 0;  // another worker of this launch reads the partial
       if (head_on && !complete && !shared) {
         float* wp = a.ws_out + pidx * D + 4 * g;
+        if (a.stream_stores != 0) {
+          int zero = 0;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          const f32x4 w = {o[mb][0] * inv, o[mb][1] * inv, o[mb][2] * inv, o[mb][3] * inv};
-          *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
+          for (int mb = 0; mb < MB; ++mb) {
+            const f32x4 w = {o[mb][0] * inv, o[mb][1] * inv, o[mb][2] * inv, o[mb][3] * inv};
+            asm volatile("" : "+s"(zero));
+            __builtin_nontemporal_store(w, reinterpret_cast<f32x4*>(wp + zero + mb * 16));
+          }
+        } else {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            const f32x4 w = {o[mb][0] * inv, o[mb][1] * inv, o[mb][2] * inv, o[mb][3] * inv};
+            *reinterpret_cast<f32x4*>(wp + mb * 16) = w;
+          }
         }
       }
       if (head_on && !complete && shared) {
@@ -1774,6 +1804,16 @@ int head_lock_knob() {
   return v;
 }
 
+// Tuning knob XLLM_MI355_GQA_STREAM_STORES: 0 / 1 force GqaArgs::stream_stores off / on; anything else leaves the
+// choice to the number of output rows of the launch.
+int stream_stores_knob() {
+  static const int v = [] {
+    const char* e = getenv("XLLM_MI355_GQA_STREAM_STORES");
+    return e != nullptr && (e[0] == '0' || e[0] == '1') ? e[0] - '0' : -1;
+  }();
+  return v;
+}
+
 // Whether the matrix-core kernel merges the partials itself: the worker that brings a context's last piece
 // reads the others' partials and writes the output, and no merge kernel is launched.  Off by default: the
 // exchange inside one launch has to go through the memory level that all XCDs share (store_shared /
@@ -1824,6 +1864,8 @@ void configure_mfma(GqaArgs& a, bool fp8, int head_dim, bool varlen) {
   // (the pools need whole groups of eight workgroups, one per XCD; the in-kernel merge walks one list; fp8 rows of
   // 64 bytes keep the computing wavefronts busy enough that the XCDs end together with equal ranges: 134 us against
   // 139 us with the cut)
+  const int64_t out_rows = static_cast<int64_t>(varlen ? a.n_tokens : a.batch) * a.n_q_heads;
+  a.stream_stores = stream_stores_knob() >= 0 ? stream_stores_knob() : (out_rows >= 8192 ? 1 : 0);
   a.pool_even = a.pool_odd = 0;
   if (a.fold_merge == 0 && n_wg % 8 == 0 && xcd_pools_knob() != 0 && !(fp8 && head_dim == 64)) {
     a.pool_even = xcd_pools_knob();
