@@ -240,12 +240,21 @@ __device__ __forceinline__ void item_prefix(const GqaArgs& a, int* prefix, int* 
     local += items_of<ITEM>(a, L);
     last_len = L;
   }
-  if (on) tmp[tid] = local;
+  // scan inside the wavefront, then over the wavefronts' totals (a thread that summed the counts of all threads before
+  // it one by one took 2.5 us at 256 sequences, and every worker waits for the prefix)
+  const int lane = tid & (kWave - 1), wave = tid / kWave;
+  int incl = local;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int t = __shfl_up(incl, d, kWave);
+    if (lane >= d) incl += t;
+  }
+  if (on && lane == kWave - 1) tmp[wave] = incl;
   if (lens != nullptr && per == 1 && lo < hi) lens[lo] = last_len;  // (kept for the workers: saves them a load each)
   __syncthreads();
   if (lo < hi) {  // (threads without a slice have nothing to place: most of them at decode batch sizes)
-    int excl = 0;
-    for (int j = 0; j < tid; ++j) excl += tmp[j];
+    int excl = incl - local;
+    for (int w = 0; w < wave; ++w) excl += tmp[w];
     if (per == 1) {  // the slice is one sequence: its count is still in `local`
       prefix[lo] = excl;
       excl += local;

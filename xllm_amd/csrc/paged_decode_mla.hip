@@ -1490,11 +1490,18 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     int local = 0;
     auto span_of = [&](int len) { return len > 0 ? (len + kW4Item - 1) / kW4Item + a.run_cost : 0; };
     for (int b = lo; b < hi; ++b) local += span_of(a.seq_lens[b]);
-    tmp[tid] = local;
+    // (scan inside the wavefront, then over the wavefronts' totals)
+    int incl = local;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int t = __shfl_up(incl, d, kWave);
+      if (lane >= d) incl += t;
+    }
+    if (lane == kWave - 1) tmp[wave] = incl;
     __syncthreads();
     if (lo < hi) {
-      int excl = 0;
-      for (int j = 0; j < tid; ++j) excl += tmp[j];
+      int excl = incl - local;
+      for (int w = 0; w < wave; ++w) excl += tmp[w];
       if (per == 1) {
         prefix[lo] = excl;
         excl += local;
