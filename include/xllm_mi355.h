@@ -473,8 +473,16 @@ int xllm_mi355_profile_collect(float* ms_out, int max_n);
  * once per process (0 default, 'p' pairs, 's' split, 'h' heads, 'n' narrow).  XLLM_MI355_DEBUG_GQA_FOLD: 1 makes
  * the matrix-core GQA kernel merge the partial results itself instead of leaving them to a second launch (same
  * as XLLM_MI355_GQA_FOLD=1 in the environment; off by default because it measures slower).
+ * XLLM_MI355_DEBUG_GQA_STREAM_STORES: 1 / 0 make the matrix-core GQA kernel write its output and partial rows with /
+ * without non-temporal stores whatever the size of the launch, negative gives the choice back to the library (same
+ * as XLLM_MI355_GQA_STREAM_STORES in the environment; the bytes written are the same either way).
  */
-enum { XLLM_MI355_DEBUG_WAIT_SPINS = 0, XLLM_MI355_DEBUG_MLA_KERNEL = 1, XLLM_MI355_DEBUG_GQA_FOLD = 2 };
+enum {
+  XLLM_MI355_DEBUG_WAIT_SPINS = 0,
+  XLLM_MI355_DEBUG_MLA_KERNEL = 1,
+  XLLM_MI355_DEBUG_GQA_FOLD = 2,
+  XLLM_MI355_DEBUG_GQA_STREAM_STORES = 3
+};
 int xllm_mi355_debug_set(int what, int value);
 
 /*

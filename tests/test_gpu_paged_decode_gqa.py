@@ -726,3 +726,48 @@ def test_a_wait_that_gives_up_is_reported(device):
     assert ops.decode_status(device) == 0   # reported once, then cleared
     again, _ = _decode_gpu(inp, kg, vg, device)
     assert torch.equal(again, good) and ops.decode_status(device) == 0
+
+
+def test_both_kinds_of_stores_write_the_same_bytes(device):
+    # the matrix-core kernel writes output and partial rows with ordinary or with non-temporal stores (the library
+    # chooses by the size of the launch): the same bytes either way, for whole contexts, contexts cut across workers,
+    # fp8 pages, other head dims and packed query chunks; the first case is also checked against the oracle
+    from xllm_amd import capi
+    lib = capi.lib()
+
+    def both(run):
+        outs = []
+        try:
+            for kind in (0, 1):
+                assert lib.xllm_mi355_debug_set(3, kind) == 0
+                outs.append(run())
+                torch.cuda.synchronize()
+        finally:
+            assert lib.xllm_mi355_debug_set(3, -1) == 0
+        for a, b in zip(outs[0], outs[1]):
+            assert torch.equal(a, b)
+        return outs[1]
+
+    shapes = (("st_g4", 40, 32, 8, 128, 16, 1, 3000, False), ("st_g8", 12, 64, 8, 128, 128, 500, 9000, False),
+              ("st_fp8", 9, 32, 8, 128, 16, 100, 5000, True), ("st_d64", 17, 16, 4, 64, 32, 1, 2000, False),
+              ("st_d256", 5, 6, 1, 256, 16, 50, 4000, False), ("st_short", 300, 8, 2, 128, 16, 1, 40, False))
+    for i, (name, batch, Hq, Hkv, D, bs, lo, hi, fp8) in enumerate(shapes):
+        cfg = workloads.DecodeConfig(name, batch, Hq, Hkv, D, bs, lo, hi, cache_dtype="fp8" if fp8 else "bf16")
+        inp = workloads.make_inputs(cfg, 800 + i, device=device)
+        kg, vg, ks, vs = fill_caches_gpu(inp, device, cache_dtype=torch.float8_e4m3fn if fp8 else None)
+        out, lse = both(lambda: _decode_gpu(inp, kg, vg, device, ks, vs))
+        if i == 0:
+            lay = inp.layout
+            ref = oracle.aten_paged_decode(inp.q.cpu(), kg.cpu(), vg.cpu(), lay.block_table, lay.seq_lens, cfg.scale)
+            assert_close_to_reference(out, ref, name)
+    cfg = workloads.DecodeConfig("st_chunks", 11, 32, 8, 128, 16, 30, 2500)
+    inp = workloads.make_inputs(cfg, 820, device=device)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    g = torch.Generator().manual_seed(4)
+    q_lens = torch.randint(1, 9, (cfg.batch,), generator=g)
+    cu = torch.tensor([0] + list(q_lens.cumsum(0)), dtype=torch.int32).to(device)
+    q = (torch.randn(int(cu[-1]), 32, 128, generator=g) * cfg.sigma).to(torch.bfloat16).to(device)
+    both(lambda: (ops.paged_forward(q, torch.empty_like(q), kg, vg, lay.block_table.to(device), lay.seq_lens.to(device),
+                                    cu, scale=cfg.scale, is_causal=True, max_query_len=8),))
+    assert ops.decode_status(device) == 0

@@ -13,6 +13,7 @@ std::atomic<int> g_wait_spins{kDefaultWaitSpins};
 int wait_spin_limit() { return g_wait_spins.load(std::memory_order_relaxed); }
 void set_mla_kernel_knob(int first_letter);  // paged_decode_mla.hip
 void set_fold_merge(int on);                 // paged_decode_gqa.hip
+void set_stream_stores(int v);               // paged_decode_gqa.hip
 }  // namespace xllm_mi355
 
 // Scratch of xllm_mi355_paged_decode_gqa_static: a decode workspace that lives in the code object, one copy
@@ -125,6 +126,9 @@ int xllm_mi355_debug_set(int what, int value) {
       return XLLM_MI355_OK;
     case XLLM_MI355_DEBUG_GQA_FOLD:
       set_fold_merge(value);
+      return XLLM_MI355_OK;
+    case XLLM_MI355_DEBUG_GQA_STREAM_STORES:
+      set_stream_stores(value);
       return XLLM_MI355_OK;
     default: return XLLM_MI355_EINVAL;
   }

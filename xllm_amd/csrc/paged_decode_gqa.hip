@@ -1813,13 +1813,17 @@ int head_lock_knob() {
   return v;
 }
 
-// Tuning knob XLLM_MI355_GQA_STREAM_STORES: 0 / 1 force GqaArgs::stream_stores off / on; anything else leaves the
-// choice to the number of output rows of the launch.
+// Tuning knob XLLM_MI355_GQA_STREAM_STORES, read once per process: 0 / 1 force GqaArgs::stream_stores off / on;
+// anything else leaves the choice to the number of output rows of the launch.  set_stream_stores (test hook)
+// overrides it: 0, 1, or negative for the choice per launch.
+std::atomic<int> g_stream_stores{-2};
 int stream_stores_knob() {
-  static const int v = [] {
+  int v = g_stream_stores.load(std::memory_order_relaxed);
+  if (v == -2) {
     const char* e = getenv("XLLM_MI355_GQA_STREAM_STORES");
-    return e != nullptr && (e[0] == '0' || e[0] == '1') ? e[0] - '0' : -1;
-  }();
+    v = e != nullptr && (e[0] == '0' || e[0] == '1') ? e[0] - '0' : -1;
+    g_stream_stores.store(v, std::memory_order_relaxed);
+  }
   return v;
 }
 
@@ -1979,6 +1983,7 @@ int group_block(int group) {
 }  // namespace
 
 void set_fold_merge(int on) { g_fold_merge.store(on != 0 ? 1 : 0, std::memory_order_relaxed); }
+void set_stream_stores(int v) { g_stream_stores.store(v < 0 ? -1 : (v != 0 ? 1 : 0), std::memory_order_relaxed); }
 
 size_t gqa_plan_bytes() { return kPlanBytes; }
 
