@@ -245,8 +245,9 @@ def neighbours(ops, workloads, torch, dev, steps):
 
 
 # The KV caches of every workload are views of ONE pool, allocated before anything else on the device, as a server
-# allocates its KV pool at start-up: the caches of the second and later workloads of a run then lie where those of a
-# fresh process lie (long_b256 as the second workload: 505.7 -> 500.6 us; alone in a process 494.5-498.5 us).
+# allocates its KV pool at start-up, and nothing is handed back to the driver between workloads.  Device memory that
+# a process frees (torch.cuda.empty_cache) and allocates again is slower to work from: a workload that ran after such
+# a cycle took 386.7 us per decode launch against 373.2-373.7 us without it (fp8_kv; alone in a process 373.6 us).
 _KV_POOL = None
 
 
@@ -524,8 +525,9 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
         result["cpu_baseline"], result["parity"] = cpu_baseline(
             inp, k_cache, v_cache, k_scale, v_scale, out.view(cfg.batch, cfg.n_q_heads, cfg.dv), args.cpu_sample,
             cpu_budget_s)
+    # (no torch.cuda.empty_cache() here: memory handed back to the driver and allocated again makes the kernels of the
+    # next workload 1-3.5 % slower, see kv_pool_caches; a serving process keeps its allocations anyway)
     del k_cache, v_cache, inp, out
-    torch.cuda.empty_cache()
     return result
 
 
