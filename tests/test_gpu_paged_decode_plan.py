@@ -207,3 +207,62 @@ def test_layer_zero_plans_and_the_other_layers_decode_from_its_plan(device):
     assert torch.equal(a, b)
     w2, w = p2.view(torch.int32), plan.view(torch.int32)   # the same plan: its first word and the item prefix
     assert int(w2[0]) == int(w[0]) and torch.equal(w2[64 : 64 + B + 2], w[64 : 64 + B + 2])
+
+
+def test_random_shapes_plain_planned_and_both_kinds_of_stores_agree(device):
+    # head dims, head groupings, block sizes, batch sizes, windows, fp8 pages and empty sequences drawn at random: the
+    # planned call and either kind of stores must reproduce the plain call bit for bit; small cases also go to the oracle
+    lib = capi.lib()
+    g = torch.Generator().manual_seed(5)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    for case in range(16):
+        D = [64, 128, 128, 256][ri(0, 3)]
+        fp8 = ri(0, 3) == 0 and D != 256
+        Hkv = [1, 2, 3, 4, 8][ri(0, 4)]
+        Hq = Hkv * [1, 2, 4, 5, 8, 16, 20][ri(0, 6)]
+        bs = [16, 32, 64, 128][ri(0, 3)]
+        batch = [1, 2, 7, 33, 64, 130, 300][ri(0, 6)]
+        hi = [40, 600, 3000][ri(0, 2)]
+        if batch * hi * Hkv * D > 1e9:
+            hi = 600
+        window = [-1, -1, 100, 1000][ri(0, 3)]
+        cfg = workloads.DecodeConfig(f"rnd{case}_{batch}_{Hq}_{Hkv}_{D}_{bs}", batch, Hq, Hkv, D, bs, 1, hi,
+                                     cache_dtype="fp8" if fp8 else "bf16")
+        inp = workloads.make_inputs(cfg, 1000 + case, device=device)
+        lay = inp.layout
+        kg, vg, ks, vs = fill_caches_gpu(inp, device, cache_dtype=torch.float8_e4m3fn if fp8 else None)
+        lens = lay.seq_lens.clone()
+        if ri(0, 2) == 0:
+            lens[torch.rand(batch, generator=g) < 0.3] = 0
+        q, table, lens_d = inp.q.to(device), lay.block_table.to(device), lens.to(device)
+        longest = max(1, int(lens.max()))
+
+        def run(plan=None):
+            o, l = ops.batch_decode(q, kg, torch.full_like(q, 3.0), table, lens_d, v_cache=vg, k_cache_quant_scale=ks,
+                                    v_cache_quant_scale=vs, scale=cfg.scale, return_lse=True, max_seq_len=longest,
+                                    window_left=window, plan=plan)
+            torch.cuda.synchronize()
+            return o, l
+
+        base = run()
+        plan = ops.update_decode_plan_info(Hq, Hkv, D, bs, kg.dtype, block_table=table, seq_lens=lens_d,
+                                           window_left=window)
+        outs = [run(plan)]
+        try:
+            for kind in (0, 1):
+                assert lib.xllm_mi355_debug_set(3, kind) == 0
+                outs += [run(), run(plan)]
+        finally:
+            assert lib.xllm_mi355_debug_set(3, -1) == 0
+        for o, l in outs:
+            assert torch.equal(o, base[0]) and torch.equal(l, base[1]), cfg.name
+        assert ops.decode_status(device) == 0
+        keep = (lens > 0).nonzero().flatten()
+        if batch * hi <= 40000 and window < 0 and len(keep) > 0:
+            ref = oracle.aten_paged_decode(inp.q.cpu()[keep].contiguous(), kg.cpu(), vg.cpu(),
+                                           lay.block_table[keep].contiguous(), lens[keep].contiguous(), cfg.scale,
+                                           None if ks is None else ks.cpu(), None if vs is None else vs.cpu())
+            assert_close_to_reference(base[0][keep.to(device)], ref, cfg.name)
