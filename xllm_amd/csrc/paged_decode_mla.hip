@@ -79,9 +79,9 @@ struct MlaArgs {
   int batch;
   int n_heads;
   int slot_heads;  // n_heads rounded up to 16
-  // mla_decode_w4_kernel and mla_merge_tiles_kernel: the schedule counts every context that holds tokens as its tiles
-  // plus this many, in front of them (the start of a run costs a workgroup about as much as four tiles; a range that
-  // holds the start of a context receives that many fewer).  0: the schedule counts tiles only
+  // mla_decode_w4_kernel and mla_merge_tiles_kernel: the schedule counts every context that holds tokens as its
+  // sub-tiles plus this many, in front of them (the start of a run costs a workgroup about as much as six sub-tiles; a
+  // range that holds the start of a context receives that many fewer).  0: the schedule counts sub-tiles only
   int run_cost;
   int n_hb;        // head blocks of 64 = workgroups per team
   int n_teams;
@@ -3006,7 +3006,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     static const int run_cost = [] {
       const char* e = getenv("XLLM_MI355_MLA_RUN_COST");  // tuning knob: tiles charged for the start of a run
       const int v = e ? atoi(e) : -1;
-      return v >= 0 && v <= 64 ? v : 4;
+      return v >= 0 && v <= 64 ? v : 3;
     }();
     a.run_cost = w4 ? run_cost * (kTile / kW4Item) : 0;
 
