@@ -60,7 +60,7 @@ enum {
   XLLM_MI355_EALIGN = -5,      /* pointer or stride not 16-byte aligned         */
   XLLM_MI355_ESTALLED = -6,    /* xllm_mi355_decode_status: a bounded wait inside a decode kernel gave up */
   XLLM_MI355_ESCRATCH = -7,    /* the problem does not fit the static scratch of the no-allocation entry point */
-  XLLM_MI355_EPLAN = -8        /* xllm_mi355_decode_status: a decode launch met a plan made for another shape */
+  XLLM_MI355_EPLAN = -8        /* xllm_mi355_decode_status: a decode launch met a plan made for another shape or other lengths */
 };
 
 /* Human-readable text for a return code of this library (host pointer, static). */
@@ -110,6 +110,10 @@ int xllm_mi355_kv_head_scales(const void* x, float* scales,
  * xllm/core/layers/common/attention_metadata.h:99-156).  Counterpart of the
  * FlashInfer float workspace (xllm/core/layers/cuda/flashinfer_workspace.cpp:25-41).
  */
+size_t xllm_mi355_paged_decode_gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim);
+size_t xllm_mi355_paged_decode_mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len);
+/* The first form of the two above, kept for existing callers: it takes v_head_dim == 512 to mean the MLA latent
+ * and every other width to be a GQA head dim.  New code names the variant. */
 size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads,
                                                int64_t v_head_dim, int64_t max_seq_len);
 
@@ -226,10 +230,14 @@ int xllm_mi355_paged_decode_gqa_csr(const void* q, const void* k_cache, const vo
  * instead of deriving all that in every launch: same kernels, same order of arithmetic, bit-identical results.
  * The plan holds for the sequence lengths, tables, head counts, head dim, block size, window and cache dtype it
  * was made with: make it again when any of them changes (every decode step).  Shapes that the matrix-core kernel
- * does not serve take no plan and are decoded as by the plain entry points.  A planned call whose shape differs
- * from the plan's writes no output and raises a flag that xllm_mi355_decode_status reports as XLLM_MI355_EPLAN;
- * lengths or tables that changed under the same shape are not detected (the reads of such a call stay inside the
- * tables and caches; its results are undefined).  Plan and planned calls are plain
+ * does not serve take no plan and are decoded as by the plain entry points.  A stale plan is reported, not
+ * followed silently: a planned call whose shape differs from the plan's writes no output, and one whose sequence
+ * lengths differ from those the plan was made with (the plan keeps them; the same shape one step later, a forgotten
+ * re-plan) writes an output that is invalid; both raise a flag that xllm_mi355_decode_status reports as
+ * XLLM_MI355_EPLAN.  Page ids that changed under unchanged lengths are not detected (page ids are clamped: the reads
+ * of such a call stay inside the caches).  plan_bytes is the size of the caller's buffer: a planned call reads the
+ * plan up to its last word, and a buffer below xllm_mi355_paged_decode_plan_bytes() is refused with
+ * XLLM_MI355_EWORKSPACE before anything is launched.  Plan and planned calls are plain
  * launches on `stream` (legal under graph capture; a replay plans again from the current lengths).
  */
 size_t xllm_mi355_paged_decode_plan_bytes(void);
@@ -241,7 +249,7 @@ int xllm_mi355_paged_decode_gqa_plan(void* plan, size_t plan_bytes,
                                      int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
                                      int64_t head_dim, int64_t block_size, int64_t window_left,
                                      int cache_dtype, void* stream);
-int xllm_mi355_paged_decode_gqa_planned(const void* plan,
+int xllm_mi355_paged_decode_gqa_planned(const void* plan, size_t plan_bytes,
                                         const void* q, const void* k_cache, const void* v_cache,
                                         void* out, float* lse,
                                         const int32_t* block_table, int64_t table_stride,

@@ -66,10 +66,34 @@ def test_host_only_entry_points_without_a_gpu():
     assert lib.xllm_mi355_rope_and_cache(fake, None, None, fake + 4, fake, None, None, None, None, None, 4, 6144, 32, 8,
                                          8, 128, 128, 1e-6, 0, 16, 10, capi.BF16, capi.FP32, capi.BF16, None) == -5
     # workspace sizes are positive and grow with the head dim
-    a = lib.xllm_mi355_paged_decode_workspace_bytes(64, 32, 128, 4096)
-    b = lib.xllm_mi355_paged_decode_workspace_bytes(64, 32, 256, 4096)
-    c = lib.xllm_mi355_paged_decode_workspace_bytes(64, 128, 512, 16384)
+    a = lib.xllm_mi355_paged_decode_gqa_workspace_bytes(64, 32, 128)
+    b = lib.xllm_mi355_paged_decode_gqa_workspace_bytes(64, 32, 256)
+    c = lib.xllm_mi355_paged_decode_mla_workspace_bytes(64, 128, 16384)
     assert 0 < a < b and c > 0
+    # the variant is named, not guessed from a width: a GQA head dim of 512 is not taken for the MLA latent
+    assert lib.xllm_mi355_paged_decode_gqa_workspace_bytes(64, 32, 512) > b
+    # (the first form of the call still answers, for callers written against it)
+    assert lib.xllm_mi355_paged_decode_workspace_bytes(64, 32, 128, 4096) == a
+    assert lib.xllm_mi355_paged_decode_workspace_bytes(64, 128, 512, 16384) == c
+
+
+def test_planned_decode_refuses_a_short_plan_buffer_before_any_launch():
+    """A planned decode reads its plan up to the last word before it looks at the signature: a buffer that is too
+    small must be refused on the host (XLLM_MI355_EWORKSPACE), whatever else the call holds."""
+    lib = capi.lib()
+    fake = 1 << 20
+    need = lib.xllm_mi355_paged_decode_plan_bytes()
+    assert need > 1 << 20
+
+    def planned(plan, plan_bytes):
+        return lib.xllm_mi355_paged_decode_gqa_planned(
+            plan, plan_bytes, fake, fake, fake, fake, None, fake, 8, fake, None, None, None, None, None,
+            4, 32, 8, 128, 16, 10, 4096, 4096, 100, -1, 0.1, fake, 1 << 30, capi.BF16, capi.BF16, None)
+
+    assert planned(None, need) == -1
+    assert planned(fake, 0) == -4
+    assert planned(fake, 4096) == -4
+    assert planned(fake, need - 1) == -4
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

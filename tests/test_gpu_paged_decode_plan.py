@@ -123,6 +123,47 @@ def test_a_plan_for_another_shape_is_reported(device):
                                     block_table=table, seq_lens=lens, plan=plan[:4096])
 
 
+def test_a_plan_that_was_not_made_again_for_new_lengths_is_reported(device):
+    """The serving-loop mistake: the lengths move on, the shape stays, the plan of the step before is passed again.
+    The kernels follow the old ranges (their reads stay inside the tables and the caches, also when contexts shrank
+    or emptied), and the status call says so."""
+    cfg = workloads.scaled(workloads.CONFIGS["llama3_8b"], batch=19, len_lo=40, len_hi=900)
+    inp = workloads.make_inputs(cfg, 6, device=device)
+    lay = inp.layout
+    kg, vg, _, _ = fill_caches_gpu(inp, device)
+    q, table = inp.q.to(device), lay.block_table.to(device)
+    lens = lay.seq_lens.to(device)
+    plan_of = lambda l: ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size,
+                                                    kg.dtype, block_table=table, seq_lens=l)
+    assert ops.decode_status(device) == 0
+    plan = plan_of(lens)
+    shorter = (lens - 1).contiguous()                       # one token fewer each: the same work items, other lengths
+    much_shorter = torch.clamp(lens - 300, min=0).contiguous()   # contexts that shrank by pages, some to nothing
+    one_moved = lens.clone()
+    one_moved[7] -= 1
+    for stale in (shorter, much_shorter, one_moved):
+        ops.batch_decode(q, kg, torch.empty_like(q), table, stale, v_cache=vg, scale=cfg.scale, plan=plan)
+        with pytest.raises(capi.XllmMi355Error, match="plan"):
+            ops.decode_status(device)
+        assert ops.decode_status(device) == 0
+        # planned again for those lengths: bit-identical to the plain call, nothing to report
+        a, _ = ops.batch_decode(q, kg, torch.empty_like(q), table, stale, v_cache=vg, scale=cfg.scale,
+                                plan=plan_of(stale))
+        b, _ = ops.batch_decode(q, kg, torch.empty_like(q), table, stale, v_cache=vg, scale=cfg.scale)
+        assert torch.equal(a, b)
+        assert ops.decode_status(device) == 0
+    # CSR form, the last sequence emptied under the old plan
+    indptr, indices, last = lay.indptr.to(device), lay.indices.to(device), lay.last_page_len.to(device)
+    plan = ops.update_decode_plan_info(cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, kg.dtype,
+                                       paged_kv_indptr=indptr, paged_kv_indices=indices, paged_kv_last_page_len=last)
+    emptied = indptr.clone()
+    emptied[-1] = emptied[-2]
+    ops.batch_decode_csr(q, kg, vg, emptied, indices, last, -1, cfg.scale, torch.empty_like(q), plan=plan)
+    with pytest.raises(capi.XllmMi355Error, match="plan"):
+        ops.decode_status(device)
+    assert ops.decode_status(device) == 0
+
+
 def test_a_captured_step_plans_again_on_every_replay(device):
     # plan + two planned layers in one graph; the lengths change between replays (the persistent buffers of a
     # captured decode step), eager calls run in between

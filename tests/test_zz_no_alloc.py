@@ -26,10 +26,20 @@ def _call(lib, static, inp, kg, vg, ks, vs, device):
             cfg.scale)
     code = capi.FP8_E4M3 if kg.dtype == torch.float8_e4m3fn else capi.BF16
     if static:
+        # once outside the measurement (the first call on a device looks the scratch address up), then with the
+        # device's memory watched: neither the driver's free memory nor torch's allocator may move across the call
+        capi.check(lib.xllm_mi355_paged_decode_gqa_static(*head, capi.BF16, code, stream), "decode")
+        torch.cuda.synchronize()
+        free_before, _ = torch.cuda.mem_get_info(device)
+        torch_before = torch.cuda.memory_allocated(device), torch.cuda.memory_reserved(device)
         rc = lib.xllm_mi355_paged_decode_gqa_static(*head, capi.BF16, code, stream)
+        torch.cuda.synchronize()
+        free_after, _ = torch.cuda.mem_get_info(device)
+        assert free_after == free_before, "the static entry point changed the device's free memory"
+        assert (torch.cuda.memory_allocated(device), torch.cuda.memory_reserved(device)) == torch_before
     else:
-        ws = ops.decode_workspace(device, lib.xllm_mi355_paged_decode_workspace_bytes(
-            cfg.batch, cfg.n_q_heads, cfg.head_dim, 0))
+        ws = ops.decode_workspace(device, lib.xllm_mi355_paged_decode_gqa_workspace_bytes(
+            cfg.batch, cfg.n_q_heads, cfg.head_dim))
         rc = lib.xllm_mi355_paged_decode_gqa(*head, ws.data_ptr(), ws.numel(), capi.BF16, code, stream)
     capi.check(rc, "decode")
     torch.cuda.synchronize()
@@ -39,11 +49,13 @@ def _call(lib, static, inp, kg, vg, ks, vs, device):
 def test_static_scratch_entry_point_matches_the_workspace_entry_point(device):
     lib = capi.lib()
     # contexts that span several workers (partials + merge through the scratch), then a smaller batch on the
-    # same scratch, which still holds the first call's partials; then fp8 pages and the dot-product kernel
+    # same scratch, which still holds the first call's partials; then fp8 pages, head dim 256 (matrix-core kernel
+    # with 8-token stages) and a block size of 8, which the dot-product kernel serves on the same scratch
     cases = [workloads.DecodeConfig("static_a", 48, 32, 8, 128, 16, 500, 3000),
              workloads.DecodeConfig("static_b", 5, 32, 8, 128, 16, 100, 900),
              workloads.DecodeConfig("static_fp8", 6, 32, 8, 128, 16, 300, 2500, cache_dtype="fp8"),
-             workloads.DecodeConfig("static_d256", 4, 8, 2, 256, 32, 200, 1500)]
+             workloads.DecodeConfig("static_d256", 4, 8, 2, 256, 32, 200, 1500),
+             workloads.DecodeConfig("static_rows_bs8", 7, 32, 8, 128, 8, 100, 1200)]
     for i, cfg in enumerate(cases):
         inp = workloads.make_inputs(cfg, 70 + i)
         fp8 = cfg.cache_dtype == "fp8"

@@ -25,6 +25,52 @@ def _stale(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
+# mla_decode_w4_kernel keeps its 256 accumulators under fixed register names (a0 .. a255) that only inline assembly
+# touches; the statements' clobber lists make the compiler count them but do not reserve them between statements.  The
+# kernel is sound as long as the compiler has no reason to put values of its own there: all 256 accumulation registers
+# in use by the kernel, nothing spilled, no scratch memory.  The build checks exactly that from the compiler's own
+# resource report and, if it ever fails (another compiler, other flags, a change that raises register pressure),
+# compiles the file again with the eight-wavefront kernel (XLLM_MI355_MLA_KERNEL=narrow) as the default for more than
+# 64 heads, and says so.
+GUARDED_SOURCE = "paged_decode_mla.hip"
+GUARDED_KERNEL = "mla_decode_w4_kernel"
+GUARD_FLAG = "-Rpass-analysis=kernel-resource-usage"
+FALLBACK_DEFINE = "-DXLLM_MLA_DEFAULT_NARROW=1"
+
+
+def resource_report(text, kernel):
+    """{field: value} per instantiation of `kernel` from the remarks of -Rpass-analysis=kernel-resource-usage."""
+    import re
+    reports, cur = [], None
+    for line in text.splitlines():
+        m = re.search(r"remark:\s+Function Name:\s+(\S+)", line)
+        if m:
+            cur = {} if kernel in m.group(1) else None
+            if cur is not None:
+                reports.append(cur)
+            continue
+        m = re.search(r"remark:\s+([A-Za-z][A-Za-z /\[\]]*?):\s+(\S+)\s+\[-Rpass-analysis", line)
+        if m and cur is not None:
+            cur[m.group(1).strip()] = m.group(2)
+    return reports
+
+
+def accumulators_untouched(reports):
+    """The condition under which the fixed-name accumulators of mla_decode_w4_kernel are safe (see above)."""
+    if not reports:
+        return False, "the compiler reported no instantiation of the kernel"
+    for r in reports:
+        if r.get("AGPRs") != "256":
+            return False, f"AGPRs = {r.get('AGPRs')} (must be 256)"
+        if r.get("VGPRs Spill") != "0":
+            return False, f"VGPRs Spill = {r.get('VGPRs Spill')} (must be 0)"
+        if r.get("ScratchSize [bytes/lane]") != "0":
+            return False, f"ScratchSize = {r.get('ScratchSize [bytes/lane]')} (must be 0)"
+        if r.get("Dynamic Stack") != "False":
+            return False, "dynamic stack"
+    return True, "ok"
+
+
 def build(force=True, verbose=True, extra_flags=()):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     hdrs = [os.path.join(CSRC, h) for h in HEADERS]
@@ -39,7 +85,20 @@ def build(force=True, verbose=True, extra_flags=()):
     def run(cmd):
         if verbose:
             print("+", " ".join(cmd), flush=True)
-        subprocess.run(cmd, check=True)
+        if os.path.basename(cmd[-3]) != GUARDED_SOURCE:
+            subprocess.run(cmd, check=True)
+            return
+        res = subprocess.run([*cmd, GUARD_FLAG], check=True, stderr=subprocess.PIPE, text=True)
+        ok, why = accumulators_untouched(resource_report(res.stderr, GUARDED_KERNEL))
+        if verbose:
+            sys.stderr.write("".join(l + "\n" for l in res.stderr.splitlines() if "remark:" not in l
+                                     and not l.lstrip().startswith(("|", "^")) and "__launch_bounds__" not in l))
+        if ok:
+            print(f"build: {GUARDED_KERNEL}: 256 accumulation registers, no spill, no scratch", flush=True)
+            return
+        print(f"build: WARNING: {GUARDED_KERNEL} fails its register check ({why}); compiling {GUARDED_SOURCE} again with "
+              f"the eight-wavefront MLA kernel as the default", file=sys.stderr, flush=True)
+        subprocess.run([*cmd, FALLBACK_DEFINE], check=True)
 
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         list(ex.map(run, jobs))

@@ -26,6 +26,8 @@ SIGNATURES = {
                                             _i64, _i64, _i32, _i32, _p]),
     "xllm_mi355_kv_head_scales": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "xllm_mi355_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
+    "xllm_mi355_paged_decode_gqa_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "xllm_mi355_paged_decode_mla_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "xllm_mi355_paged_decode_gqa": (_i32, [_p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _i64, _i64, _i64,
                                            _i64, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _p, _sz, _i32,
                                            _i32, _p]),
@@ -41,7 +43,7 @@ SIGNATURES = {
     "xllm_mi355_paged_decode_plan_bytes": (_sz, []),
     "xllm_mi355_paged_decode_gqa_plan": (_i32, [_p, _sz, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64,
                                                 _i64, _i32, _p]),
-    "xllm_mi355_paged_decode_gqa_planned": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _p, _p, _p,
+    "xllm_mi355_paged_decode_gqa_planned": (_i32, [_p, _sz, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _p, _p, _p,
                                                    _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                                    _f32, _p, _sz, _i32, _i32, _p]),
     "xllm_mi355_gather_paged_rows": (_i32, [_p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),

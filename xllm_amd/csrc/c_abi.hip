@@ -58,7 +58,7 @@ const char* xllm_mi355_error_string(int code) {
     case XLLM_MI355_EWORKSPACE: return "split-K workspace missing, misaligned or too small";
     case XLLM_MI355_EALIGN: return "pointer or stride not 16-byte aligned";
     case XLLM_MI355_ESTALLED: return "a bounded wait inside a decode kernel gave up: the outputs of that launch are invalid";
-    case XLLM_MI355_EPLAN: return "a decode launch was given a plan made for another shape: it wrote no output";
+    case XLLM_MI355_EPLAN: return "a decode launch was given a plan made for another shape or for other sequence lengths: its output is invalid";
     case XLLM_MI355_ESCRATCH: return "the problem needs more scratch than the static scratch of the no-allocation entry point holds";
     default: break;
   }
@@ -86,9 +86,20 @@ int xllm_mi355_kv_head_scales(const void* x, float* scales, int64_t n_tokens, in
 size_t xllm_mi355_paged_decode_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t v_head_dim,
                                                int64_t max_seq_len) {
   if (batch <= 0 || n_q_heads <= 0 || v_head_dim <= 0) return 0;
-  // 512 is the latent width of the MLA kernel; every other width is a GQA head dim
+  // (kept for callers written against the first version of this header, which asked for both variants here: a width
+  // of 512 meant the MLA latent; new code asks xllm_mi355_paged_decode_mla_workspace_bytes for that)
   if (v_head_dim == 512) return mla_workspace_bytes(batch, n_q_heads, max_seq_len);
   return gqa_workspace_bytes(batch, n_q_heads, v_head_dim);
+}
+
+size_t xllm_mi355_paged_decode_gqa_workspace_bytes(int64_t batch, int64_t n_q_heads, int64_t head_dim) {
+  if (batch <= 0 || n_q_heads <= 0 || head_dim <= 0) return 0;
+  return gqa_workspace_bytes(batch, n_q_heads, head_dim);
+}
+
+size_t xllm_mi355_paged_decode_mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) {
+  if (batch <= 0 || n_heads <= 0) return 0;
+  return mla_workspace_bytes(batch, n_heads, max_seq_len);
 }
 
 size_t xllm_mi355_decode_workspace_bound(void) { return decode_workspace_bound(); }
@@ -220,7 +231,7 @@ int xllm_mi355_paged_decode_gqa_plan(void* plan, size_t plan_bytes, const int32_
                                cache_dtype, static_cast<hipStream_t>(stream));
 }
 
-int xllm_mi355_paged_decode_gqa_planned(const void* plan, const void* q, const void* k_cache,
+int xllm_mi355_paged_decode_gqa_planned(const void* plan, size_t plan_bytes, const void* q, const void* k_cache,
                                         const void* v_cache, void* out, float* lse,
                                         const int32_t* block_table, int64_t table_stride,
                                         const int32_t* seq_lens, const int32_t* paged_kv_indptr,
@@ -233,6 +244,8 @@ int xllm_mi355_paged_decode_gqa_planned(const void* plan, const void* q, const v
                                         void* workspace, size_t workspace_bytes, int q_dtype, int cache_dtype,
                                         void* stream) {
   if (plan == nullptr) return XLLM_MI355_EINVAL;
+  // (the kernels read the plan up to its last word before they look at its signature)
+  if (plan_bytes < gqa_plan_bytes()) return XLLM_MI355_EWORKSPACE;
   PageAddressing addr;
   addr.window_left = window_left;
   addr.plan = plan;

@@ -55,7 +55,7 @@ constexpr size_t kWsHeaderBytes = kWsCountersOff + static_cast<size_t>(kWsMaxWor
 constexpr int kWsMaxBatch = 2048;
 constexpr size_t kWsPartialsOff = kWsHeaderBytes + (static_cast<size_t>(kWsMaxBatch + 1) * 4 + 255) / 256 * 256;
 constexpr int kStatusWaitGaveUp = 1;  // a bounded wait of one wavefront on another ran out: the launch's output is invalid
-constexpr int kStatusPlanMismatch = 2;  // a decode launch was given a plan made for another shape: it wrote no output
+constexpr int kStatusPlanMismatch = 2;  // a decode launch was given a plan made for another shape (it wrote no output) or for other lengths
 
 // Bound of the polls of one wavefront on another (test hook: xllm_mi355_debug_set_wait_spins).
 int wait_spin_limit();
@@ -152,6 +152,23 @@ inline bool first_use_on_current_device(std::atomic<uint64_t>& seen) {
   if ((seen.load(std::memory_order_acquire) & bit) != 0) return false;
   seen.fetch_or(bit, std::memory_order_acq_rel);
   return true;
+}
+
+// Compute units of the current device, looked up once per device (a process may drive several GPUs, and they need
+// not be alike).  256 if the runtime cannot say.
+inline int device_cu_count() {
+  static std::atomic<int> cached[64];  // zero-initialised; 0 = not looked up yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  const bool slot = dev >= 0 && dev < 64;
+  if (slot) {
+    const int n = cached[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+  }
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+  if (slot) cached[dev].store(n, std::memory_order_relaxed);
+  return n;
 }
 
 // Opt-in timing of the dominant kernel (profile.hip).  While it is enabled, launch_timed hands the launch

@@ -99,9 +99,11 @@ struct GqaArgs {
   // i - 1, or i - 3, or i - 9) they were 1-2 % slower than free, which is 2-5 % faster than apart.
   int head_lock;
   // Matrix-core kernel: the flat list is cut in two, in the ratio pool_even : pool_odd, and the first part dealt to
-  // the groups of workers on XCDs 0, 2, 4, 6, the second to those on XCDs 1, 3, 5, 7 (workgroup i runs on XCD i % 8).
-  // With equal shares the workgroups on the odd XCDs stream their rows 8-11 % slower and end a launch that much later
-  // (every MI355X measured, five of them); 9 : 8 ends the decode kernels 1.7-2.7 % earlier.  0 : 0 = one list.
+  // the workgroups whose index is even modulo 8, the second to the others.  A tuned default, not a fact the results
+  // rest on: on the full MI355X (256 CUs, workgroup i dispatched to XCD i % 8) the workgroups on the odd XCDs were
+  // seen to stream their rows 8-11 % slower with equal shares, and 9 : 8 ends the decode kernels 1.7-2.7 % earlier; a
+  // device that dispatches otherwise only loses that gain (the merge walks whatever cut the decode kernel used).  The
+  // host sets it only for a device of 256 CUs; 0 : 0 = one list.
   int pool_even, pool_odd;
   // Matrix-core kernel: a plan of the step, made once by gqa_plan_kernel for all layers (see kPlan*), or null: the
   // item prefix, the cut between the pools and, for every group of workers, the 64 page-table entries its first
@@ -197,11 +199,15 @@ __device__ __forceinline__ Pools make_pools(const GqaArgs& a, int64_t total, int
 
 // A plan (ints): word 0 the signature of what it was made for | from kPlanPrefixOff the item prefix [batch + 1] and
 // the cut between the pools | from kPlanChunksOff 64 page-table entries per group of workers (the chunk of the
-// context's table that holds the page of the group's first stage; the tail repeats the context's last page).
+// context's table that holds the page of the group's first stage; the tail repeats the context's last page) | from
+// kPlanLensOff the context lengths [batch] the plan was made with: the merge kernel of a planned call compares them
+// with the lengths of the call, so that a plan that was not made again for a new step is reported
+// (kStatusPlanMismatch) instead of followed silently.
 constexpr int kPlanPrefixOff = 64;
 constexpr int kPlanChunksOff = kPlanPrefixOff + (kMaxBatch + 2 + 63) / 64 * 64;
 constexpr int kPlanMaxTeams = 4096;
-constexpr size_t kPlanBytes = (static_cast<size_t>(kPlanChunksOff) + static_cast<size_t>(kPlanMaxTeams) * kWave) * 4;
+constexpr int kPlanLensOff = kPlanChunksOff + kPlanMaxTeams * kWave;
+constexpr size_t kPlanBytes = (static_cast<size_t>(kPlanLensOff) + static_cast<size_t>(kMaxBatch)) * 4;
 
 // The range [cur, end) of the flat list that group of workers `team` of `n_teams` takes; false: none.
 __device__ __forceinline__ bool team_range(const GqaArgs& a, int64_t total, int64_t cut, int64_t team, int64_t n_teams,
@@ -979,8 +985,12 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // into the chunk buffer at byte offset off
   auto issue_chunk = [&](const CtxCursor& cu, int ck, u32 off) {
     const int n_pages = (cu.L + a.block_size - 1) >> a.bs_shift;
-    // (never in front of the table: with a plan made for other lengths a context may have no pages here)
-    dma4(cu.pages + max(0, min(ck * kWave + lane, n_pages - 1)), page_lds + off);
+    // (never in front of the table, and never entry 0 of a context that has no pages, which in the CSR form may lie
+    // past the end of the index array: with a plan made for other lengths a context may have no pages here; any
+    // readable word will do then, page ids are clamped)
+    const int32_t* src = cu.pages + max(0, min(ck * kWave + lane, n_pages - 1));
+    if (n_pages <= 0 && a.indptr != nullptr) src = a.indptr;
+    dma4(src, page_lds + off);
   };
 
   // byte offset of the lane's 16 bytes from the first row of a stage: row 4i + g, chunk swizzled
@@ -1089,7 +1099,9 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       begin_context(false);
     }
     const int tok0 = (pc.st0 + pc.st) * T;
-    const int lim = pc.L - tok0 - 1;  // last valid row of the stage
+    // last valid row of the stage (never negative: under a plan made for longer contexts a stage may lie past the end
+    // of its context, and its rows then repeat the stage's first row, which is inside the page)
+    const int lim = max(0, pc.L - tok0 - 1);
     // block size >= 16: a sub-block of 16 tokens lies in one page
     constexpr int NSUB = T >= 16 ? T / 16 : 1;
     uint64_t kb[NSUB], vb[NSUB];
@@ -1723,6 +1735,12 @@ __global__ __launch_bounds__(kThreads) void gqa_plan_kernel(GqaArgs a, int* plan
   const int64_t cut = a.pool_even == 0 ? 0 : pool_cut(a, total);
   if (blockIdx.x == 0) {
     for (int i = tid; i <= a.batch; i += kThreads) plan[kPlanPrefixOff + i] = prefix[i];
+    for (int i = tid; i < a.batch; i += kThreads) {
+      const int32_t* pages;
+      int L;
+      sequence_of(a, i, pages, L);
+      plan[kPlanLensOff + i] = L;
+    }
     if (tid == 0) plan[kPlanPrefixOff + a.batch + 1] = static_cast<int>(cut);
     if (tid == 0) plan[0] = a.plan_sig;
   }
@@ -1749,18 +1767,16 @@ template <typename QT, bool VL>
 __global__ __launch_bounds__(kThreads) void merge_partials_kernel(GqaArgs a, int dv) {
   const int b = blockIdx.y;
   if (a.plan != nullptr && a.plan[0] != a.plan_sig) return;   // the decode kernel wrote nothing and raised the flag
+  if (!VL && a.plan != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+    // a plan made with other lengths (the step before, say): the decode kernel followed its ranges, the output is
+    // invalid, and the caller hears of it through the status word
+    const int32_t* pages;
+    int L;
+    sequence_of(a, b, pages, L);
+    if (L != a.plan[kPlanLensOff + b]) atomicOr(a.ws_status, kStatusPlanMismatch);
+  }
   merge_context<QT, VL>(a, dv, blockIdx.x, b, threadIdx.x, kThreads, a.ws_prefix[b], a.ws_prefix[b + 1],
                         a.ws_prefix[a.batch], a.pool_even != 0 ? a.ws_prefix[a.batch + 1] : 0);
-}
-
-int device_cu_count() {
-  static const int n = [] {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 256;
-    return p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
-  }();
-  return n;
 }
 
 template <typename QT, bool FP8, int D, int LPT, int G, int U>
@@ -1769,15 +1785,22 @@ int launch_gqa(GqaArgs& a, size_t workspace_bytes, hipStream_t stream, bool plan
   auto kern = gqa_decode_kernel<QT, FP8, D, LPT, G, U>;
   const size_t smem = kSub * 4 + static_cast<size_t>(NP) * (D + 2) * 4 + kThreads * 4 +
                       (static_cast<size_t>(a.batch) + 1) * 4;
-  static const int per_cu = [&] {
+  // workgroups of this kernel that a CU of the current device holds, asked once per device
+  static std::atomic<int> per_cu_of[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) dev = 0;
+  int per_cu = per_cu_of[dev].load(std::memory_order_relaxed);
+  if (per_cu <= 0) {
     const char* e = getenv("XLLM_MI355_GQA_WGS_PER_CU");  // tuning knob
-    if (e != nullptr && atoi(e) > 0) return atoi(e);
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(kern), kThreads,
-                                                     kSub * 4 + NP * (D + 2) * 4 + kThreads * 4 + 1028) != hipSuccess || n < 1)
-      n = 2;
-    return n;
-  }();
+    if (e != nullptr && atoi(e) > 0) {
+      per_cu = atoi(e);
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), kThreads,
+                                                            kSub * 4 + NP * (D + 2) * 4 + kThreads * 4 + 1028) != hipSuccess ||
+               per_cu < 1) {
+      per_cu = 2;
+    }
+    per_cu_of[dev].store(per_cu, std::memory_order_relaxed);
+  }
   a.n_workgroups = device_cu_count() * per_cu;
   a.plan = nullptr;   // (plans are for the matrix-core kernel)
   const size_t part_floats = static_cast<size_t>(a.n_workgroups) * 2 * G * (D + 1);
@@ -1880,7 +1903,9 @@ void configure_mfma(GqaArgs& a, bool fp8, int head_dim, bool varlen) {
   const int64_t out_rows = static_cast<int64_t>(varlen ? a.n_tokens : a.batch) * a.n_q_heads;
   a.stream_stores = stream_stores_knob() >= 0 ? stream_stores_knob() : (out_rows >= 8192 ? 1 : 0);
   a.pool_even = a.pool_odd = 0;
-  if (a.fold_merge == 0 && n_wg % 8 == 0 && xcd_pools_knob() != 0 && !(fp8 && head_dim == 64)) {
+  // The cut is a tuned default for the full MI355X (256 CUs in 8 XCDs, workgroups dealt to the XCDs round robin), not
+  // a property of the algorithm: any other CU count (a partitioned or CU-masked device) gets one list.
+  if (a.fold_merge == 0 && n_wg == 256 && xcd_pools_knob() != 0 && !(fp8 && head_dim == 64)) {
     a.pool_even = xcd_pools_knob();
     a.pool_odd = 8;
   }

@@ -2863,23 +2863,14 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
   if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * H + hd] = (M + fast_log2(W)) * kLn2;
 }
 
-int mla_cu_count() {
-  static const int n = [] {
-    int dev = 0;
-    hipDeviceProp_t p;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return 256;
-    return p.multiProcessorCount > 0 ? p.multiProcessorCount : 256;
-  }();
-  return n;
-}
-
 // Teams: as many as there are CUs for the team size, a multiple of 8 (one per XCD slot).
 int mla_teams(int n_hb) {
-  static const int wgs = [] {
+  static const int knob = [] {
     const char* e = getenv("XLLM_MI355_MLA_WGS");  // tuning knob: workgroups in flight
     const int v = e ? atoi(e) : 0;
-    return v > 0 ? v : mla_cu_count();
+    return v > 0 ? v : 0;
   }();
+  const int wgs = knob > 0 ? knob : device_cu_count();
   int teams = wgs / n_hb / 8 * 8;
   return teams < 8 ? 8 : teams;
 }
@@ -3002,7 +2993,13 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.ws_out = reinterpret_cast<float*>(static_cast<char*>(workspace) + kWsPartialsOff);
     a.slot_heads = static_cast<int>((n_heads + 15) / 16 * 16);
     a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * a.slot_heads * kDL;
+    // (XLLM_MLA_DEFAULT_NARROW: the build found that the compiler did not leave the fixed-name accumulators of
+    // mla_decode_w4_kernel alone and made the eight-wavefront kernel the default; 'w' still asks for the other)
+#ifdef XLLM_MLA_DEFAULT_NARROW
+    const bool w4 = !pairs && !use_p && by_dims && knob == 'w';
+#else
     const bool w4 = !pairs && !use_p && by_dims && knob != 'n';
+#endif
     static const int run_cost = [] {
       const char* e = getenv("XLLM_MI355_MLA_RUN_COST");  // tuning knob: tiles charged for the start of a run
       const int v = e ? atoi(e) : -1;

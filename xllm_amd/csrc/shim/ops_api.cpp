@@ -172,12 +172,14 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
     lse = output_lse->data_ptr<float>();
   }
   if (max_seq_len <= 0) max_seq_len = block_table.size(1) * k_cache.size(1);
-  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len);
+  const size_t nbytes = xllm_mi355_paged_decode_gqa_workspace_bytes(B, Hq, D);
   torch::Tensor ws = decode_workspace(query.device(), nbytes);
   if (plan.has_value() && plan->defined()) {
-    TORCH_CHECK(plan->is_cuda() && plan->is_contiguous(), "plan must be the buffer of update_decode_plan");
+    TORCH_CHECK(plan->is_cuda() && plan->is_contiguous() && plan->scalar_type() == torch::kUInt8 &&
+                    static_cast<size_t>(plan->numel()) >= xllm_mi355_paged_decode_plan_bytes(),
+                "plan must be the buffer of update_decode_plan (uint8, xllm_mi355_paged_decode_plan_bytes() bytes)");
     const int rc = xllm_mi355_paged_decode_gqa_planned(
-        plan->data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache->data_ptr(), output.data_ptr(), lse,
+        plan->data_ptr(), static_cast<size_t>(plan->numel()), query.data_ptr(), k_cache.data_ptr(), v_cache->data_ptr(), output.data_ptr(), lse,
         block_table.data_ptr<int32_t>(), block_table.stride(0), seq_lens.data_ptr<int32_t>(), nullptr, nullptr, nullptr,
         static_cast<const float*>(ptr_or_null(k_cache_quant_scale)),
         static_cast<const float*>(ptr_or_null(v_cache_quant_scale)), B, Hq, k_cache.size(2), D, k_cache.size(1),
@@ -215,12 +217,14 @@ void batch_decode_csr(torch::Tensor query, torch::Tensor k_cache, torch::Tensor 
     lse = output_lse->data_ptr<float>();
   }
   if (max_seq_len <= 0) max_seq_len = std::max<int64_t>(1, paged_kv_indices.numel()) * k_cache.size(1);
-  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len);
+  const size_t nbytes = xllm_mi355_paged_decode_gqa_workspace_bytes(B, Hq, D);
   torch::Tensor ws = decode_workspace(query.device(), nbytes);
   if (plan.has_value() && plan->defined()) {
-    TORCH_CHECK(plan->is_cuda() && plan->is_contiguous(), "plan must be the buffer of update_decode_plan");
+    TORCH_CHECK(plan->is_cuda() && plan->is_contiguous() && plan->scalar_type() == torch::kUInt8 &&
+                    static_cast<size_t>(plan->numel()) >= xllm_mi355_paged_decode_plan_bytes(),
+                "plan must be the buffer of update_decode_plan (uint8, xllm_mi355_paged_decode_plan_bytes() bytes)");
     const int rc = xllm_mi355_paged_decode_gqa_planned(
-        plan->data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), lse, nullptr, 0,
+        plan->data_ptr(), static_cast<size_t>(plan->numel()), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), lse, nullptr, 0,
         nullptr, paged_kv_indptr.data_ptr<int32_t>(), paged_kv_indices.data_ptr<int32_t>(),
         paged_kv_last_page_len.data_ptr<int32_t>(), nullptr, nullptr, B, Hq, k_cache.size(2), D, k_cache.size(1),
         k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, window_left, static_cast<float>(sm_scale),
@@ -577,7 +581,7 @@ torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {
     lse = lse_rows.data_ptr<float>();
   }
   const int64_t max_seq_len = table.size(1) * p.k_cache.size(1);
-  const size_t nbytes = xllm_mi355_paged_decode_workspace_bytes(rows, heads, p.head_size_v, max_seq_len);
+  const size_t nbytes = xllm_mi355_paged_decode_mla_workspace_bytes(rows, heads, max_seq_len);
   torch::Tensor ws = mi355::decode_workspace(q_nope.device(), nbytes);
   const int rc = xllm_mi355_paged_decode_mla(
       q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), lse, table.data_ptr<int32_t>(),

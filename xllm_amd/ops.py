@@ -46,6 +46,13 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def _check_plan(plan):
+    """The planned decode reads the plan up to its last word: refuse anything but the whole buffer."""
+    need = capi.lib().xllm_mi355_paged_decode_plan_bytes()
+    if plan.dtype != torch.uint8 or not plan.is_contiguous() or plan.numel() < need:
+        raise ValueError(f"plan must be the contiguous uint8 buffer of update_decode_plan ({need} bytes)")
+
+
 def _require_cuda(*tensors):
     dev = None
     for t in tensors:
@@ -286,11 +293,12 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     if max_seq_len <= 0:
         max_seq_len = block_table.shape[1] * bs
     lib = capi.lib()
-    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len)
+    nbytes = lib.xllm_mi355_paged_decode_gqa_workspace_bytes(B, Hq, D)
     ws = decode_workspace(dev, nbytes)
     if plan is not None:
+        _check_plan(plan)
         rc = lib.xllm_mi355_paged_decode_gqa_planned(
-            plan.data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(lse),
+            plan.data_ptr(), plan.numel(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(lse),
             block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), None, None, None,
             _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D, bs, P,
             query.stride(0), output.stride(0), max_seq_len, int(window_left), float(scale), ws.data_ptr(), ws.numel(),
@@ -327,11 +335,12 @@ def batch_decode_csr(query, k_cache, v_cache, paged_kv_indptr, paged_kv_indices,
     if max_seq_len <= 0:
         max_seq_len = max(1, paged_kv_indices.numel()) * bs
     lib = capi.lib()
-    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(B, Hq, D, max_seq_len)
+    nbytes = lib.xllm_mi355_paged_decode_gqa_workspace_bytes(B, Hq, D)
     ws = decode_workspace(dev, nbytes)
     if plan is not None:
+        _check_plan(plan)
         rc = lib.xllm_mi355_paged_decode_gqa_planned(
-            plan.data_ptr(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
+            plan.data_ptr(), plan.numel(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(),
             _ptr(output_lse), None, 0, None, paged_kv_indptr.data_ptr(), paged_kv_indices.data_ptr(),
             paged_kv_last_page_len.data_ptr(), _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D,
             bs, P, query.stride(0), output.stride(0), max_seq_len, int(window_left), float(sm_scale), ws.data_ptr(),
@@ -462,7 +471,7 @@ def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0):
     if max_seq_len <= 0:
         max_seq_len = table.shape[1] * bs
     lib = capi.lib()
-    nbytes = lib.xllm_mi355_paged_decode_workspace_bytes(rows, heads, d_latent, max_seq_len)
+    nbytes = lib.xllm_mi355_paged_decode_mla_workspace_bytes(rows, heads, max_seq_len)
     ws = decode_workspace(dev, nbytes)
     rc = lib.xllm_mi355_paged_decode_mla(
         q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), _ptr(lse),
