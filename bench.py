@@ -29,6 +29,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 METRIC = "paged-decode tokens/s + achieved HBM GB/s (% of 8 TB/s) on 1 MI355X"
 ALL = ("llama3_8b", "long_b256", "fp8_kv", "mla_dsv3")
 HEADLINE = "long_b256"
+# The timed steps go round this many copies of the KV cache at different addresses, so that no step finds a page of
+# the step before in a cache: two copies of the smallest timed cache (577 MB) put 1.15 GB between two reads of a page,
+# against 256 MB of last-level cache.  (`same_cache` in the line is the loop over one copy.)
+ROTATE = 2
 MAX_ABS_TOL, MEAN_ABS_TOL = 2e-2, 2e-3   # attention output against the reference's libtorch CPU path, bf16
 
 
@@ -260,6 +264,7 @@ def kv_pool_reserve(torch, dev, nbytes):
 
 
 def kv_pool_caches(torch, dev, shape, dtype, n):
+    """n zeroed caches of `shape` as views of the pool."""
     one = 1
     for x in shape:
         one *= x
@@ -271,7 +276,7 @@ def kv_pool_caches(torch, dev, shape, dtype, n):
         v = pool[i * stride : i * stride + one].view(dtype).view(shape)
         v.zero_()
         views.append(v)
-    return views[0], (views[1] if n > 1 else None)
+    return views
 
 
 def kv_pool_bytes(workloads, names, seed):
@@ -280,7 +285,7 @@ def kv_pool_bytes(workloads, names, seed):
         cfg = workloads.CONFIGS[name]
         lay = workloads.make_layout(cfg, seed)
         one = lay.num_blocks * cfg.block_size * cfg.n_kv_heads * cfg.head_dim * (1 if cfg.cache_dtype == "fp8" else 2)
-        need = max(need, ((one + 4095) // 4096 * 4096) * (1 if cfg.mla else 2))
+        need = max(need, ((one + 4095) // 4096 * 4096) * (1 if cfg.mla else 2) * ROTATE)
     return need
 
 
@@ -304,7 +309,10 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     lay = inp.layout
     cache_dt = torch.float8_e4m3fn if fp8 else torch.bfloat16
     shape = (lay.num_blocks, cfg.block_size, cfg.n_kv_heads, cfg.head_dim)
-    k_cache, v_cache = kv_pool_caches(torch, dev, shape, cache_dt, 1 if cfg.mla else 2)
+    views = kv_pool_caches(torch, dev, shape, cache_dt, (1 if cfg.mla else 2) * ROTATE)
+    k_caches = views[:ROTATE]
+    v_caches = [None] * ROTATE if cfg.mla else views[ROTATE:]
+    k_cache, v_cache = k_caches[0], v_caches[0]
     k_scale = v_scale = None
     if fp8:
         k_scale = ops.kv_head_scales(torch.cat([inp.k_ctx, inp.k_new]))
@@ -315,6 +323,10 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     store(ops.ReshapePagedCacheParams(key=inp.k_ctx, value=inp.v_ctx, k_cache=k_cache, v_cache=v_cache,
                                       slot_mapping=ctx_slots, k_cache_scale=k_scale, v_cache_scale=v_scale))
     inp.k_ctx = inp.v_ctx = None   # (the context now lives in the cache)
+    for i in range(1, ROTATE):     # the other copies: the same bytes at other addresses
+        k_caches[i].view(torch.uint8).copy_(k_cache.view(torch.uint8))
+        if v_cache is not None:
+            v_caches[i].view(torch.uint8).copy_(v_cache.view(torch.uint8))
     table = lay.block_table.to(dev)
     seq_lens = lay.seq_lens.to(dev)
     max_len = int(lay.seq_lens.max())
@@ -342,54 +354,90 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     ptr = lambda t: None if t is None else t.data_ptr()
     code = {torch.bfloat16: capi.BF16, torch.float8_e4m3fn: capi.FP8_E4M3}
     row = cfg.n_kv_heads * cfg.head_dim
-    reshape_args = (ptr(inp.k_new), ptr(inp.v_new), ptr(k_cache), ptr(v_cache), ptr(new_slots),
-                    ptr(k_scale), ptr(v_scale), cfg.batch, cfg.n_kv_heads, cfg.head_dim, cfg.block_size,
-                    lay.num_blocks, row, row, capi.BF16, code[cache_dt], stream)
-    ws_bytes = lib.xllm_mi355_paged_decode_workspace_bytes(cfg.batch, cfg.n_q_heads, cfg.dv, max_len)
+    reshape_fn = lib.xllm_mi355_reshape_and_cache
+    if cfg.mla:
+        ws_bytes = lib.xllm_mi355_paged_decode_mla_workspace_bytes(cfg.batch, cfg.n_q_heads, max_len)
+    else:
+        ws_bytes = lib.xllm_mi355_paged_decode_gqa_workspace_bytes(cfg.batch, cfg.n_q_heads, cfg.head_dim)
     ws = ops.decode_workspace(dev, ws_bytes)
     if cfg.mla:
         out = torch.empty(cfg.batch, 1, cfg.n_q_heads, cfg.v_dim, dtype=torch.bfloat16, device=dev)
         decode_fn = lib.xllm_mi355_paged_decode_mla
-        decode_args = (ptr(mla.q_nope), ptr(mla.q_pe), ptr(k_cache), ptr(out), None, ptr(table),
-                       table.stride(0), ptr(seq_lens), cfg.batch, cfg.n_q_heads, cfg.v_dim,
-                       cfg.head_dim - cfg.v_dim, cfg.block_size, lay.num_blocks, max_len, cfg.scale,
-                       ptr(ws), ws.numel(), capi.BF16, stream)
     else:
         decode_fn = lib.xllm_mi355_paged_decode_gqa
-        decode_args = (ptr(inp.q), ptr(k_cache), ptr(v_cache), ptr(out), None, ptr(table),
-                       table.stride(0), ptr(seq_lens), ptr(k_scale), ptr(v_scale), cfg.batch,
-                       cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, lay.num_blocks,
-                       inp.q.stride(0), out.stride(0), max_len, -1, cfg.scale, ptr(ws), ws.numel(),
-                       capi.BF16, code[cache_dt], stream)
-    reshape_fn = lib.xllm_mi355_reshape_and_cache
 
-    def step():
-        rc = reshape_fn(*reshape_args)
-        rc2 = decode_fn(*decode_args)
-        if rc or rc2:
-            capi.check(rc or rc2, "bench step")
+    def bound_args(kc, vc):
+        reshape_args = (ptr(inp.k_new), ptr(inp.v_new), ptr(kc), ptr(vc), ptr(new_slots),
+                        ptr(k_scale), ptr(v_scale), cfg.batch, cfg.n_kv_heads, cfg.head_dim, cfg.block_size,
+                        lay.num_blocks, row, row, capi.BF16, code[cache_dt], stream)
+        if cfg.mla:
+            decode_args = (ptr(mla.q_nope), ptr(mla.q_pe), ptr(kc), ptr(out), None, ptr(table),
+                           table.stride(0), ptr(seq_lens), cfg.batch, cfg.n_q_heads, cfg.v_dim,
+                           cfg.head_dim - cfg.v_dim, cfg.block_size, lay.num_blocks, max_len, cfg.scale,
+                           ptr(ws), ws.numel(), capi.BF16, stream)
+        else:
+            decode_args = (ptr(inp.q), ptr(kc), ptr(vc), ptr(out), None, ptr(table),
+                           table.stride(0), ptr(seq_lens), ptr(k_scale), ptr(v_scale), cfg.batch,
+                           cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, lay.num_blocks,
+                           inp.q.stride(0), out.stride(0), max_len, -1, cfg.scale, ptr(ws), ws.numel(),
+                           capi.BF16, code[cache_dt], stream)
+        return reshape_args, decode_args
+
+    bound = [bound_args(k_caches[i], v_caches[i]) for i in range(ROTATE)]
+    reshape_args, decode_args = bound[0]
+
+    def make_step(copies):
+        state = [0]
+
+        def step():
+            r_args, d_args = bound[state[0] % copies]
+            state[0] += 1
+            rc = reshape_fn(*r_args)
+            rc2 = decode_fn(*d_args)
+            if rc or rc2:
+                capi.check(rc or rc2, "bench step")
+        return step
+
+    def timed_loop(step, events):
+        """W warm-up steps, then K steps between two synchronisations.  With `events` every decode and merge launch of
+        the K steps carries an event pair (their kernel times come back; the wall clock of such a loop is not used:
+        the instrumented launch path is not the one a caller takes)."""
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        if events:
+            capi.check(lib.xllm_mi355_profile_enable(2 * args.steps), "profile_enable")
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        if not events:
+            return elapsed / args.steps * 1e3, None, None
+        ms = collect_ms(lib, 2 * args.steps)   # per step: the decode kernel, then the merge kernel
+        return elapsed / args.steps * 1e3, sum(ms[0::2]) / max(len(ms[0::2]), 1), sum(ms[1::2]) / max(len(ms[1::2]), 1)
 
     # The first tens of milliseconds of work after an idle period run at other clocks than the steady state a
     # serving loop sees (kernel times swing by 20-30 % over the first ~100 launches): run the step untimed until
     # --settle-ms have passed, then the W warm-up steps, then the K timed ones.
+    step = make_step(ROTATE)
     t_settle = time.perf_counter()
     while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
         for _ in range(20):
             step()
         torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    capi.check(lib.xllm_mi355_profile_enable(2 * args.steps), "profile_enable")
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms = collect_ms(lib, 2 * args.steps)   # per step: the decode kernel, then the merge kernel
-    kernel_ms = sum(ms[0::2]) / max(len(ms[0::2]), 1)
-    merge_ms = sum(ms[1::2]) / max(len(ms[1::2]), 1)
+    # the headline: plain launches (no event pairs), the caches taken in turn
+    ms_per_step, _, _ = timed_loop(step, events=False)
+    # the kernels' own times: the same loop with an event pair on every decode and merge launch
+    instrumented_ms_per_step, kernel_ms, merge_ms = timed_loop(step, events=True)
     ops.decode_status(dev)                 # raises if a wait inside a decode kernel gave up
+    # the same two loops over ONE copy of the cache (every step reads the pages the step before read)
+    same_step = make_step(1)
+    same_ms_per_step, _, _ = timed_loop(same_step, events=False)
+    _, same_kernel_ms, same_merge_ms = timed_loop(same_step, events=True)
+    same_cache = {"ms_per_step": same_ms_per_step, "kernel_ms": same_kernel_ms, "merge_kernel_ms": same_merge_ms,
+                  "tokens_per_s": cfg.batch / (same_ms_per_step * 1e-3)}
+    elapsed = ms_per_step * 1e-3 * args.steps
 
     # ---- the same step as the layers after the first see it when the step was planned once (not the headline:
     # `value` above is the self-contained call, which derives its schedule in every launch)
@@ -398,12 +446,15 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
         plan = torch.empty(lib.xllm_mi355_paged_decode_plan_bytes(), dtype=torch.uint8, device=dev)
         plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), None, None, None, cfg.batch,
                      cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, -1, code[cache_dt], stream)
-        planned_args = (ptr(plan),) + decode_args[:8] + (None, None, None) + decode_args[8:]
+        planned_bound = [(r, (ptr(plan), plan.numel()) + d[:8] + (None, None, None) + d[8:]) for r, d in bound]
         plain_out = out.clone()
+        p_state = [0]
 
         def planned_step():
-            rc = reshape_fn(*reshape_args)
-            rc2 = lib.xllm_mi355_paged_decode_gqa_planned(*planned_args)
+            r_args, d_args = planned_bound[p_state[0] % ROTATE]
+            p_state[0] += 1
+            rc = reshape_fn(*r_args)
+            rc2 = lib.xllm_mi355_paged_decode_gqa_planned(*d_args)
             if rc or rc2:
                 capi.check(rc or rc2, "bench planned step")
 
@@ -411,20 +462,11 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
         capi.check(lib.xllm_mi355_paged_decode_gqa_plan(*plan_args), "xllm_mi355_paged_decode_gqa_plan")
         torch.cuda.synchronize()
         plan_ms = collect_ms(lib, 1)
-        for _ in range(args.warmup):
-            planned_step()
-        torch.cuda.synchronize()
-        capi.check(lib.xllm_mi355_profile_enable(2 * args.steps), "profile_enable")
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            planned_step()
-        torch.cuda.synchronize()
-        p_elapsed = time.perf_counter() - t0
-        pms = collect_ms(lib, 2 * args.steps)
+        p_ms_per_step, _, _ = timed_loop(planned_step, events=False)
+        _, p_kernel_ms, p_merge_ms = timed_loop(planned_step, events=True)
         ops.decode_status(dev)
-        planned = {"kernel_ms": sum(pms[0::2]) / max(len(pms[0::2]), 1),
-                   "merge_kernel_ms": sum(pms[1::2]) / max(len(pms[1::2]), 1),
-                   "ms_per_step": p_elapsed / args.steps * 1e3, "plan_kernel_ms": plan_ms[0] if plan_ms else None,
+        planned = {"kernel_ms": p_kernel_ms, "merge_kernel_ms": p_merge_ms,
+                   "ms_per_step": p_ms_per_step, "plan_kernel_ms": plan_ms[0] if plan_ms else None,
                    "bit_identical": bool(torch.equal(plain_out, out))}
 
     # ---- the same step captured once in a HIP graph and replayed, as the reference's graph executor runs a decode
@@ -457,7 +499,6 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
                         "bit_identical": bool(torch.equal(ref_out, out))}
         del graph
 
-    ms_per_step = elapsed / args.steps * 1e3
     tokens_per_s = cfg.batch / (ms_per_step * 1e-3)
 
     # ---- roofline of the dominant kernel (the decode kernel), from algorithmic work
@@ -485,7 +526,12 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                     "op_frac": nbytes / (op_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     roofline.update({"kernel": decode_kernel_name(cfg), "kernel_ms": kernel_ms, "merge_kernel_ms": merge_ms,
-                     "algorithmic_bytes": nbytes})
+                     "algorithmic_bytes": nbytes,
+                     "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
+                                       "workload, scaled by a plain copy of known size; a constant of the build, not "
+                                       "measured in this run",
+                     "kernel_ms_source": "HIP event pairs on the decode and merge dispatches of a second loop of "
+                                         "the same steps; ms_per_step and value come from the loop without them"})
     if flops is not None:
         roofline["algorithmic_flops"] = flops
     if planned is not None:
@@ -514,6 +560,9 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
             "context_tokens": int(lay.seq_lens.sum()), "max_context": max_len,
             "step": "reshape_and_cache(new K/V rows) + paged decode attention, inputs resident in HBM",
         },
+        "instrumented_ms_per_step": instrumented_ms_per_step,
+        "kv_cache_copies_in_rotation": ROTATE,
+        "same_cache": same_cache,
         "hbm_gbs_whole_step": (nbytes + workloads.reshape_bytes(
             cfg.batch, cfg.n_kv_heads * cfg.head_dim, 2, 1 if fp8 else 2, 1 if cfg.mla else 2))
             / (ms_per_step * 1e-3) / 1e9,
@@ -527,7 +576,7 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
             cpu_budget_s)
     # (no torch.cuda.empty_cache() here: memory handed back to the driver and allocated again makes the kernels of the
     # next workload 1-3.5 % slower, see kv_pool_caches; a serving process keeps its allocations anyway)
-    del k_cache, v_cache, inp, out
+    del k_cache, v_cache, k_caches, v_caches, views, inp, out
     return result
 
 
@@ -572,7 +621,7 @@ def main():
         result = dict(per[HEADLINE])
         result["gate"] = {"workload": "tiny", "parity": gate.get("parity")}
         keep = ("value", "unit", "ms_per_step", "dtype", "config", "hbm_gbs_whole_step", "roofline", "cpu_baseline",
-                "parity")
+                "parity", "same_cache", "instrumented_ms_per_step", "kv_cache_copies_in_rotation")
         result["per_config"] = [{k: per[name][k] for k in keep if k in per[name]} for name in ALL]
         if not args.no_cpu_baseline:
             result["parity_all_ok"] = all(per[name]["parity"]["ok"] for name in ALL) and gate["parity"]["ok"]
