@@ -478,7 +478,7 @@ int xllm_mi355_profile_collect(float* ms_out, int max_n);
  * at xllm_mi355_decode_status (negative = default, 2^22; 0 makes the first wait of a launch give up, which is
  * how the status path is tested: every wavefront still exits normally).  XLLM_MI355_DEBUG_MLA_KERNEL: the MLA
  * kernel choice, as the first letter of the environment variable XLLM_MI355_MLA_KERNEL, which the library reads
- * once per process (0 default, 'p' pairs, 's' split, 'h' heads, 'n' narrow).  XLLM_MI355_DEBUG_GQA_FOLD: 1 makes
+ * once per process (0 default, 'p' pairs, 'h' heads, 'n' narrow, 'w' the four-wavefront kernel).  XLLM_MI355_DEBUG_GQA_FOLD: 1 makes
  * the matrix-core GQA kernel merge the partial results itself instead of leaving them to a second launch (same
  * as XLLM_MI355_GQA_FOLD=1 in the environment; off by default because it measures slower).
  * XLLM_MI355_DEBUG_GQA_STREAM_STORES: 1 / 0 make the matrix-core GQA kernel write its output and partial rows with /

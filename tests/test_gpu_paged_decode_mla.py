@@ -66,8 +66,8 @@ def _select_kernel(name):
 
 def test_batches_larger_than_a_workgroup_and_than_a_launch(device):
     # more sequences than threads in a workgroup (several per thread in the tile prefix) and more than one launch
-    # holds (1024), in all three kernels
-    for knob in ("", "pairs", "split"):
+    # holds (1024), in the default kernel and in the one for other block sizes
+    for knob in ("", "pairs"):
         _select_kernel(knob)
         try:
             _check(_mla_cfg(f"mla_b600_{knob}", 600, 16, 1, 150), 90, device)
@@ -217,25 +217,15 @@ def test_many_short_sequences_with_128_heads(device):
     _check(_mla_cfg("mla128_b1100", 1100, 128, 1, 40), 19, device)
 
 
-def test_producer_consumer_kernel(device):
-    # the kernel with the two products on different wavefronts, selected by the tuning knob
-    _select_kernel("split")
-    try:
-        _producer_consumer_cases(device)
-    finally:
-        _select_kernel("")
-
-
-def _producer_consumer_cases(device):
-    _check(_mla_cfg("split128", 3, 128, 100, 1500), 5, device)
+def test_head_counts_page_table_chunk_boundaries_and_long_contexts(device):
+    _check(_mla_cfg("d128", 3, 128, 100, 1500), 5, device)
     for heads in (2, 16, 80):
-        _check(_mla_cfg(f"split{heads}", 2, heads, 1, 400), 60 + heads, device)
-    _check(_mla_cfg("split_bs16", 2, 16, 50, 700, bs=16), 3, device)
+        _check(_mla_cfg(f"d{heads}", 2, heads, 1, 400), 60 + heads, device)
     for i, L in enumerate((1023, 1025, 2049, 3100)):  # page-table chunk boundaries (block 16: 1024 tokens per chunk)
-        _check(_mla_cfg(f"split_chunks{L}", 1, 16, L, L, bs=16), 70 + i, device)
-    _check(_mla_cfg("split_short", 96, 16, 1, 200, bs=16), 13, device)
-    _check(_mla_cfg("split_long", 1, 128, 6000, 9000), 6, device)
-    test_scores_that_rise_along_the_context(device)
+        _check(_mla_cfg(f"chunks{L}", 1, 16, L, L, bs=16), 70 + i, device)
+        _check(_mla_cfg(f"chunks128_{L}", 1, 128, L, L, bs=16), 80 + i, device)
+    _check(_mla_cfg("short", 96, 16, 1, 200, bs=16), 13, device)
+    _check(_mla_cfg("long", 1, 128, 6000, 9000), 6, device)
 
 
 def test_shard_merge_equals_full_decode(device):

@@ -89,6 +89,13 @@ struct MlaArgs {
   int bs_shift;
   int num_blocks;
   float scale_log2;
+  // mla_decode_w4_kernel merges the pieces of a context itself and no merge kernel follows (see the fold at the end of
+  // that kernel): ws_written holds one counter per (team, head block of 128), zero between launches, that counts the
+  // pieces of the context that starts in that team's range as they reach memory
+  int fold;
+  unsigned* ws_written;
+  int* ws_status;   // status flags of the workspace (kStatus*), only ever OR-ed into
+  int wait_spins;   // bound of the folding workgroup's polls on ws_written
 };
 
 __device__ __forceinline__ int tiles_of(int L) { return L > 0 ? (L + kTile - 1) / kTile : 0; }
@@ -1416,6 +1423,141 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
 #define XLLM_W4_ROW7(F) F(0, 7, 224, 225, 226, 227) F(1, 7, 228, 229, 230, 231) F(2, 7, 232, 233, 234, 235) F(3, 7, 236, 237, 238, 239) F(4, 7, 240, 241, 242, 243) F(5, 7, 244, 245, 246, 247) F(6, 7, 248, 249, 250, 251) F(7, 7, 252, 253, 254, 255)
 #define XLLM_W4_ALL(F) XLLM_W4_ROW0(F) XLLM_W4_ROW1(F) XLLM_W4_ROW2(F) XLLM_W4_ROW3(F) XLLM_W4_ROW4(F) XLLM_W4_ROW5(F) XLLM_W4_ROW6(F) XLLM_W4_ROW7(F)
 constexpr int kW4Threads = 256;
+
+// ---- pieces of a context that spans several teams, and their merge (tiles of mla_decode_w4_kernel) ----------------
+// Where the pieces of a context lie: teams t_first .. t_last of the launch, whose ranges are stepped without a
+// division (team_start(t) = t * q + floor(t * r / n) with total = q * n + r).
+struct MlaPieces {
+  int t_first, t_last;
+  int slot_first;   // slot of the first team's piece (1 when its range starts in front of the context, with an earlier run)
+  int count;        // pieces: teams of t_first .. t_last whose range is not empty
+  int64_t q, r, acc, n;
+};
+// front, stop: the context's share of what the schedule divides, [prefix[b], prefix[b + 1]): run_cost, then its tiles.
+// False: the context has no tiles.
+__device__ __forceinline__ bool mla_locate_pieces(const MlaArgs& a, int64_t front, int64_t stop, int64_t total, MlaPieces& p) {
+  const int64_t first = front + a.run_cost, last = stop - 1;
+  if (last < first) return false;
+  const int64_t n = a.n_teams;
+  p.n = n;
+  p.t_first = team_of(first, total, n);
+  p.t_last = team_of(last, total, n);
+  const bool fits32 = total * n < (1LL << 31);
+  p.q = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(total) / static_cast<uint32_t>(n)) : total / n;
+  p.r = total - p.q * n;
+  p.acc = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(p.t_first) * static_cast<uint32_t>(p.r) % static_cast<uint32_t>(n))
+                 : (static_cast<int64_t>(p.t_first) * p.r) % n;
+  // (a range that starts in front of the context holds the last tile of an earlier one)
+  p.slot_first = team_start(p.t_first, total, n) < front ? 1 : 0;
+  // with fewer items than teams a range holds one item or none, and the teams that hold first .. last are one per tile
+  p.count = total >= n ? p.t_last - p.t_first + 1 : static_cast<int>(last - first + 1);
+  return true;
+}
+
+typedef __attribute__((address_space(3))) const u32x4 lds_cu32x4;
+// A 16-byte load / store that other workgroups of the same launch are the counterpart of: at the scope of the whole
+// GPU (the L2 of an XCD is not coherent with the other seven inside a launch; these go to the level that all share).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t coherent_window(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
+}
+constexpr int kAuxDeviceScope = 16;   // the cache-policy bit that the compiler sets for device-scope atomics (sc1)
+__device__ __forceinline__ u32x4 coherent_load16(__amdgpu_buffer_rsrc_t w, u32 byte_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(w, byte_off, 0, kAuxDeviceScope);
+}
+__device__ __forceinline__ void coherent_store16(__amdgpu_buffer_rsrc_t w, u32 byte_off, u32x4 v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, w, byte_off, 0, kAuxDeviceScope);
+}
+
+// The merge of one (block of 16 heads hb, context b) by 256 threads laid out like the four wavefronts that wrote the
+// tiles: wavefront w, lane (head c16, k-group g) owns dims 128 w + 16 db + 4 g .. + 3 of head 16 hb + c16 for the
+// eight dim blocks db, and every load instruction reads 1 KB in one piece.  Four teams at a time, their 32 loads per
+// lane issued together.  FOLD: called by the workgroup of mla_decode_w4_kernel that holds the context's first piece:
+// that piece (team p.t_first) is read from the workgroup's LDS (tiles at own_tiles, LSEs at own_lse[head of the 128]),
+// the others, which other workgroups of the same launch wrote, with coherent loads.  Same arithmetic in the same
+// order either way: the result does not depend on who merges.
+template <typename QT, bool FOLD>
+__device__ __forceinline__ void mla_merge_tiles(const MlaArgs& a, const MlaPieces& p, int hb, int b, int w, int lane,
+                                                const char* own_tiles, const float* own_lse) {
+  const int H = a.n_heads;
+  const int c16 = lane & 15, g = lane >> 4;
+  const int hd = hb * 16 + c16;
+  const bool head_ok = hd < H;
+  char* out = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + w * 128 + 4 * g) * 2;
+  const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 2;
+  const u32 tile_off = static_cast<u32>((hb * 4 + w) * 4096 + lane * 16);
+  const char* tiles = reinterpret_cast<const char*>(a.ws_out) + tile_off;
+  const __amdgpu_buffer_rsrc_t window = coherent_window(a.ws_out);
+  int64_t acc = p.acc;
+  float M = kNegBig, W = 0.0f;
+  f32x4 O[8];
+#pragma unroll
+  for (int db = 0; db < 8; ++db) O[db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int tb = p.t_first; tb <= p.t_last; tb += 4) {
+    float lse[4];
+    u32x4 x[4][4];   // pairs of dim blocks, 16-bit values
+    bool on[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = tb + k;
+      acc += p.r;
+      const int64_t step = p.q + (acc >= p.n ? 1 : 0);
+      acc -= acc >= p.n ? p.n : 0;
+      // with fewer tiles than teams some ranges in between are empty and own no partial
+      on[k] = t <= p.t_last && step > 0 && head_ok;
+      const int64_t slot = static_cast<int64_t>(t) * 2 + (t == p.t_first ? p.slot_first : 0);
+      if (FOLD && t == p.t_first) {
+        lse[k] = on[k] ? own_lse[hd & (kHeadsPerWg16 - 1)] : kNegBig;
+#pragma unroll
+        for (int dp = 0; dp < 4; ++dp)
+          x[k][dp] = on[k] ? *(lds_cu32x4*)(own_tiles + ((hb & 7) * 4 + w) * 4096 + lane * 16 + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
+      } else if (FOLD) {
+        lse[k] = on[k] ? __hip_atomic_load(a.ws_lse + slot * H + hd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : kNegBig;
+#pragma unroll
+        for (int dp = 0; dp < 4; ++dp)
+          x[k][dp] = on[k] ? coherent_load16(window, tile_off + static_cast<u32>(slot * slot_bytes) + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
+      } else {
+        lse[k] = on[k] ? a.ws_lse[slot * H + hd] : kNegBig;
+#pragma unroll
+        for (int dp = 0; dp < 4; ++dp)
+          x[k][dp] = on[k] ? *reinterpret_cast<const u32x4*>(tiles + slot * slot_bytes + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+    const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
+    const float keep = fast_exp2(M - m_new);
+    W *= keep;
+#pragma unroll
+    for (int db = 0; db < 8; ++db) O[db] *= keep;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
+      W += e;
+#pragma unroll
+      for (int dp = 0; dp < 4; ++dp) {
+        const u32x4 v = x[k][dp];
+        O[2 * dp] += e * f32x4{QT::lo(v[0]), QT::hi(v[0]), QT::lo(v[1]), QT::hi(v[1])};
+        O[2 * dp + 1] += e * f32x4{QT::lo(v[2]), QT::hi(v[2]), QT::lo(v[3]), QT::hi(v[3])};
+      }
+    }
+    M = m_new;
+  }
+  if (!head_ok) return;
+  const float inv = 1.0f / W;
+#pragma unroll
+  for (int db = 0; db < 8; ++db)
+    *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{QT::pack(O[db][0] * inv, O[db][1] * inv), QT::pack(O[db][2] * inv, O[db][3] * inv)};
+  if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * H + hd] = (M + fast_log2(W)) * kLn2;
+}
+// Output rows of a context without tokens: zeros, LSE -inf (same layout of the 256 threads).
+template <typename QT>
+__device__ __forceinline__ void mla_write_empty(const MlaArgs& a, int hb, int b, int w, int lane) {
+  const int c16 = lane & 15, g = lane >> 4;
+  const int hd = hb * 16 + c16;
+  if (hd >= a.n_heads) return;
+  char* out = a.out + ((static_cast<int64_t>(b) * a.n_heads + hd) * kDL + w * 128 + 4 * g) * 2;
+#pragma unroll
+  for (int db = 0; db < 8; ++db) *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{0u, 0u};
+  if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * a.n_heads + hd] = -INFINITY;
+}
 // At the start of a run the Q rows of the 128 heads pass through the ring and the P^T area on their way into the
 // registers: latent parts at a pitch of 1040 bytes (16 lanes that read 16 bytes of 16 rows hit 64 different banks),
 // then the rope parts.  The small arrays sit behind them.
@@ -2129,577 +2271,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
 #undef W4_PTICK
 }
 
-// ---------------------------------------------------------------------------------------------
-// Producer / consumer kernel (selected with XLLM_MI355_MLA_KERNEL=split): 32 heads per wavefront, the
-// two products on different wavefronts.
-//
-// Workgroup = 512 threads = 8 wavefronts = 64 heads; a SIMD holds one producer and one consumer.
-//   producers 0-3, wavefront (hb, th): S^T[tok, head] = K[tok, 576] . Q^T[576, head] for the 16 tokens
-//       16th..16th+15 of a 32-token sub-tile and the heads 32hb..32hb+31: 18 k-steps x 2 head halves of
-//       v_mfma_f32_16x16x32_bf16, A = K rows from LDS (one 16-byte read feeds both halves), B = Q^T in
-//       144 VGPRs; then the softmax of those scores and the bf16 P^T block (1 KB) to LDS
-//   consumers 4-7, wavefront (hb, th): O^T[dim, head] += V^T[dim, tok] . P^T[tok, head] for all 32 tokens,
-//       the dims 256th..256th+255 and the same heads: 16 v_mfma_f32_32x32x16_bf16, A = V^T through the
-//       transposing LDS read, B = the two P^T blocks of the head block from LDS.  They also move the tile
-//       rows from global memory into LDS and write the output.
-// No MFMA is repeated (1088 matrix-pipe cycles per SIMD and sub-tile) and every K / V byte is read from
-// LDS once per 32 heads: 148 KB per sub-tile and 64 heads, against 272 KB with 16 heads per wavefront
-// (which runs at the LDS limit).  In iteration t the producers work on sub-tile t + 1 while the consumers
-// multiply sub-tile t, so a SIMD has the softmax arithmetic of one wavefront and the MFMAs of the other
-// to interleave.  One barrier per iteration: P(t) visible, sub-tile t + 1 landed, slot of sub-tile t - 1
-// released.  Two sub-tiles are live in LDS, two more are in flight (ring of four).
-//
-// Softmax without a second exchange: every producer keeps its own reference maximum per head, an
-// INTEGER (log2 units) that only follows the scores when they exceed it by more than kPSlack, and
-// publishes it with its P block.  A consumer keeps the reference R of its accumulators (also an
-// integer) and scales a block by 2^-(R - m): for bf16 that is a saturating subtraction of
-// (R - m) << 7 from the 16-bit patterns, one packed instruction per two values.  Normaliser
-// shares are kept per producer and joined at the end of a run.
-//
-// Measured on the configuration with 128 heads it is as fast as the kernel with 16 heads per wavefront,
-// not faster: an iteration takes about 2400 cycles, set by the producers' serial chain (first operands,
-// 36 MFMAs, softmax, LDS write, barrier), with the matrix pipe busy for 1088 of them.
-//
-// LDS layout of a sub-tile: the 1024 latent bytes of the 32 rows, 1056 bytes apart, 16-byte chunks
-// XOR-ed with bit 2 of the row; then the 128 rope bytes of the rows, 128 bytes apart, chunks XOR-ed
-// with the low 3 bits of the row (one 64-lane load moves the rope parts of 8 rows).  The ring and the
-// exchange blocks fill the 160 KB, which leaves room for the tile prefix of kPMaxBatch sequences.
-constexpr int kPRowL = kDL * 2 + 32;               // 1056
-constexpr int kPSubTok = 32;                       // tokens per sub-tile
-constexpr int kPRing = 4;                          // ring slots
-constexpr int kPRopeOff = kPSubTok * kPRowL;       // 33792
-constexpr int kPSubBytes = kPRopeOff + kPSubTok * kDR * 2;  // 37888
-// LDS: ring | exchange [2 buffers][2 head blocks][2 token blocks] x (1024 B of P^T + 32 references) |
-//      page-table chunks [2][64] | prefix
-constexpr int kPXchBlk = 1024 + 128;
-constexpr int kPXchOff = kPRing * kPSubBytes;
-constexpr int kPPageOff = kPXchOff + 2 * 2 * 2 * kPXchBlk;
-constexpr int kPPrefixOff = kPPageOff + 2 * kWave * 4;
-constexpr int kPLdsBytes = 160 * 1024;
-constexpr int kPMaxBatch = (kPLdsBytes - kPPrefixOff) / 4 - 1;  // sequences per launch of this kernel
-constexpr int kWThreads = 512;
-constexpr float kPSlack = 24.0f;                  // a reference follows scores that exceed it by more than this (log2 units)
-constexpr float kPRefInit = -1048576.0f;           // reference before any score was seen (integer valued)
-
-#define XLLM_DMA_ROWP(lds, gbase, lane_off, lds_off)                                                      \
-  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds), "v"(lane_off), \
-               "s"(gbase), "n"(lds_off)                                                                   \
-               : "memory", "scc")
-
-// The same under an execution mask (all ones or zero, wave-uniform): with the mask at zero the load moves
-// nothing, which lets a caller place it in straight-line code between MFMAs instead of under a branch.
-#define XLLM_DMA_ROWP_MASKED(lds, gbase, lane_off, lds_off, mask)                                          \
-  do {                                                                                                     \
-    uint64_t saved_;                                                                                       \
-    asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, exec, %5\n\ts_add_u32 m0, %1, %4\n\ts_nop 0\n\t"  \
-                 "global_load_lds_dwordx4 %2, %3 nt\n\ts_mov_b64 exec, %0"                                   \
-                 : "=&s"(saved_)                                                                           \
-                 : "s"(lds), "v"(lane_off), "s"(gbase), "n"(lds_off), "s"(mask)                            \
-                 : "memory", "scc");                                                                       \
-  } while (0)
-__device__ __forceinline__ void dma16_masked(const void* gptr, u32 lds_addr, uint64_t mask) {
-  const u32 base = __builtin_amdgcn_readfirstlane(lds_addr);
-  uint64_t saved;
-  asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, exec, %3\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-               "global_load_lds_dwordx4 %2, off nt\n\ts_mov_b64 exec, %0"
-               : "=&s"(saved)
-               : "s"(base), "v"(gptr), "s"(mask)
-               : "memory", "scc");
-}
-
-typedef __attribute__((ext_vector_type(2))) unsigned short u16x2;
-// bf16 pair times 2^-k (k >= 0 in `dec` = k << 7 in both halves): exponent fields decremented, flushed to +0
-__device__ __forceinline__ u32 bf16x2_scale_down(u32 w, u32 dec) {
-  return __builtin_bit_cast(u32, __builtin_elementwise_sub_sat(__builtin_bit_cast(u16x2, w), __builtin_bit_cast(u16x2, dec)));
-}
-
-__global__ __launch_bounds__(kWThreads) void mla_decode32w_kernel(MlaArgs a) {
-  extern __shared__ __align__(16) char smem[];
-  int* prefix = reinterpret_cast<int*>(smem + kPPrefixOff);
-  const int* pagebuf = reinterpret_cast<const int*>(smem + kPPageOff);
-  int* tmp = reinterpret_cast<int*>(smem);  // prologue only
-
-  const int tid = threadIdx.x;
-  const int lane = tid & (kWave - 1);
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const bool consumer = wave >= 4;  // wavefronts 0-3 produce probabilities, 4-7 consume them
-  const int w4 = wave & 3;
-  const int H = a.n_heads;
-
-  // block id -> (team, head block): members of a team are 8 ids apart (same XCD)
-  const int xcd = blockIdx.x & 7;
-  const int y = blockIdx.x >> 3;
-  const int hb64 = y % a.n_hb;
-  const int team = (y / a.n_hb) * 8 + xcd;
-  const int hb32 = w4 >> 1;   // 32-head block of the wavefront
-  const int th = w4 & 1;      // producer: its 16 tokens of a sub-tile; consumer: its half of the output dims
-  const int head0 = hb64 * kHeadsPerWg + hb32 * 32;
-  const bool wave_ok = head0 < H;
-
-  // ---- tile prefix over the batch (every workgroup computes it; no extra launch)
-  {
-    const int per = (a.batch + kWThreads - 1) / kWThreads;
-    const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
-    int local = 0;
-    for (int b = lo; b < hi; ++b) local += tiles_of(a.seq_lens[b]);
-    tmp[tid] = local;
-    __syncthreads();
-    if (lo < hi) {  // (threads without a slice have nothing to place: most of them at decode batch sizes)
-      int excl = 0;
-      for (int j = 0; j < tid; ++j) excl += tmp[j];
-      if (per == 1) {  // the slice is one sequence: its count is still in `local`
-        prefix[lo] = excl;
-        excl += local;
-      } else {
-        for (int b = lo; b < hi; ++b) {
-          prefix[b] = excl;
-          excl += tiles_of(a.seq_lens[b]);
-        }
-      }
-      if (hi == a.batch) prefix[a.batch] = excl;
-    }
-    __syncthreads();
-  }
-  const int64_t total = prefix[a.batch];
-  if (blockIdx.x == 0)
-    for (int i = tid; i <= a.batch; i += kWThreads) a.ws_prefix[i] = prefix[i];
-  if (total == 0) return;
-  int64_t cur = team_start(team, total, a.n_teams);
-  const int64_t end = team_start(team + 1, total, a.n_teams);
-  bool first_run = true;
-
-  const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
-  // exchange blocks of this head block: buffer parity p at + p * 4 * kPXchBlk, token block tb at + tb * kPXchBlk
-  const u32 xch_hb = lds_base + kPXchOff + hb32 * 2 * kPXchBlk;
-
-  while (cur < end) {
-    int lo = 0, hi = a.batch;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (prefix[mid] <= cur) lo = mid; else hi = mid;
-    }
-    const int b = __builtin_amdgcn_readfirstlane(lo);
-    const int n_tiles_seq = prefix[b + 1] - prefix[b];
-    const int tile0 = static_cast<int>(cur - prefix[b]);
-    const int run_tiles = static_cast<int>(min<int64_t>(n_tiles_seq - tile0, end - cur));
-    const bool complete = tile0 == 0 && run_tiles == n_tiles_seq;
-    cur += run_tiles;
-    const int L = __builtin_amdgcn_readfirstlane(a.seq_lens[b]);
-    const int t_begin = tile0 * kTile;
-    const int t_end = min(L, (tile0 + run_tiles) * kTile);
-    const int n_sub = (t_end - t_begin + kPSubTok - 1) / kPSubTok;
-
-    if (!consumer) {
-      // =================================== producer: S^T = K . Q^T, softmax, P^T and references to LDS
-      const int c16 = lane & 15;    // head column (of each head half) / token row supplied by the lane
-      const int g4 = lane >> 4;     // k-group of the lane; its score rows are tokens 4 g4 .. 4 g4 + 3
-      // Q^T operands: lane (c16, g4) keeps dims 32 kk + 8 g4 .. + 8 of every k-step for the heads c16 and
-      // 16 + c16 of the block; k-steps 16, 17 hold the rope dims
-      bf16x8 q[kKSteps32][2];
-      {
-        const int64_t row = static_cast<int64_t>(b) * H + head0 + c16;
-        const char* qn = a.q_nope + row * kDL * 2 + g4 * 16;
-        const char* qp = a.q_pe + row * kDR * 2 + g4 * 16;
-        asm volatile("" : "+v"(qn), "+v"(qp));  // two address registers; the rest goes into instruction offsets
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const bool ok = head0 + 16 * h + c16 < H;
-#pragma unroll
-          for (int kk = 0; kk < kKSteps32; ++kk) {
-            u32x4 x = {0u, 0u, 0u, 0u};
-            if (ok) x = ldg16(kk < kDL / 32 ? qn + h * 16 * kDL * 2 + kk * 64 : qp + h * 16 * kDR * 2 + (kk - kDL / 32) * 64);
-            q[kk][h] = __builtin_bit_cast(bf16x8, x);
-          }
-        }
-      }
-      // K operand addresses inside ring slot 0: row th*16 + c16, 16-byte chunk 4 kk + g4 XOR-ed with bit 2 of
-      // the row (latent part) / with the low 3 bits of the row (rope part, 128 bytes per row)
-      const int krow = th * 16 + c16;
-      const u32 ka0 = lds_base + krow * kPRowL + (((g4 ^ (krow >> 2)) & 1) * 16) + ((g4 >> 1) * 32);
-      const u32 kr0 = lds_base + kPRopeOff + krow * (kDR * 2) + ((g4 ^ (krow & 7)) * 16);
-      // reference and normaliser share of heads c16 (index 0) and 16 + c16 (index 1) over the wavefront's tokens
-      float m0 = kPRefInit, m1 = kPRefInit, l0 = 0.0f, l1 = 0.0f;
-      // make the compiler wait for the Q loads here, not inside the loop
-#pragma unroll
-      for (int kk = 0; kk < kKSteps32; ++kk)
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          u32x4 x = __builtin_bit_cast(u32x4, q[kk][h]);
-          asm volatile("" : "+v"(x));
-          q[kk][h] = __builtin_bit_cast(bf16x8, x);
-        }
-      __syncthreads();  // the previous run no longer reads the ring, the chunks or the exchange blocks
-      __syncthreads();  // (the consumers fetch the first page-table chunks between these two)
-
-      for (int t = -1; t < n_sub; ++t) {
-        __syncthreads();  // sub-tile t + 1 has landed; the consumers are past P(t - 1)
-        if (!wave_ok || t + 1 >= n_sub) continue;
-        // ---- S^T of the wavefront's 16 tokens of sub-tile t + 1: lane (head c16 / 16 + c16, tokens 4 g4 + r).
-        // One K read feeds both head halves; the reads run 6 k-steps ahead of the MFMAs.
-        const u32 slot_off = ((t + 1) & (kPRing - 1)) * kPSubBytes;
-        u32 ka = ka0 + slot_off, kr = kr0 + slot_off;
-        asm volatile("" : "+v"(ka), "+v"(kr));  // one register each; the k-step goes into the instruction offset
-        auto k_operand = [&](int kk) {  // k-steps 16, 17 are the rope dims: chunk 4 j + g4 is at the address of chunk g4, XOR 64 j
-          return kk < kDL / 32 ? *(lds_u32x4*)(ka + kk * 64) : *(lds_u32x4*)(kr ^ ((kk - kDL / 32) * 64));
-        };
-        constexpr int kAheadK = 6;
-        f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
-        __builtin_amdgcn_sched_barrier(0);  // the pipeline below covers the K reads and the score MFMAs only
-#pragma unroll
-        for (int kk = 0; kk < kKSteps32; ++kk) {
-          const bf16x8 x = __builtin_bit_cast(bf16x8, k_operand(kk));
-          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, q[kk][0], s0, 0, 0, 0);
-          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, q[kk][1], s1, 0, 0, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x100, kAheadK, 0);
-#pragma unroll
-        for (int i = 0; i < kKSteps32 - kAheadK; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2 * kAheadK, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- softmax: scores in log2 units, tokens past the end of the run masked
-        const int tok_base = t_begin + (t + 1) * kPSubTok + th * 16 + 4 * g4;
-        float sv0[4], sv1[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const bool in = tok_base + r < t_end;
-          sv0[r] = in ? s0[r] * a.scale_log2 : -INFINITY;
-          sv1[r] = in ? s1[r] * a.scale_log2 : -INFINITY;
-        }
-        bool over = false;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) over |= (sv0[r] > m0 + kPSlack) | (sv1[r] > m1 + kPSlack);
-        if (__builtin_amdgcn_ballot_w64(over) != 0) {  // rare: the references only follow maxima that exceed them by more than kPSlack
-          const float mx0 = quad_rows_max(fmaxf(fmaxf(sv0[0], sv0[1]), fmaxf(sv0[2], sv0[3])));
-          const float mx1 = quad_rows_max(fmaxf(fmaxf(sv1[0], sv1[1]), fmaxf(sv1[2], sv1[3])));
-          const float n0 = mx0 > m0 + kPSlack ? __builtin_ceilf(mx0) : m0;
-          const float n1 = mx1 > m1 + kPSlack ? __builtin_ceilf(mx1) : m1;
-          l0 *= fast_exp2(m0 - n0);
-          l1 *= fast_exp2(m1 - n1);
-          m0 = n0;
-          m1 = n1;
-        }
-        float p0[4], p1[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          p0[r] = fast_exp2(sv0[r] - m0);
-          p1[r] = fast_exp2(sv1[r] - m1);
-          l0 += p0[r];
-          l1 += p1[r];
-        }
-        // P^T block of this wavefront in the B-operand layout of the P.V MFMA: k-slot (g2, j) of head n holds
-        // token 4 g2 + j (j < 4) / 8 + 4 g2 + j - 4 (j >= 4) at (g2 * 32 + n) * 16 + 2 j
-        const u32 xw = xch_hb + ((t + 1) & 1) * 4 * kPXchBlk + th * kPXchBlk;
-        const u32 wa = xw + ((g4 & 1) * 32 + c16) * 16 + (g4 >> 1) * 8;
-        *(lds_u32x2*)(wa) = u32x2{BF16::pack(p0[0], p0[1]), BF16::pack(p0[2], p0[3])};
-        *(lds_u32x2*)(wa + 16 * 16) = u32x2{BF16::pack(p1[0], p1[1]), BF16::pack(p1[2], p1[3])};
-        // (the four lanes that own a head all write its reference: same value, no branch)
-        *(lds_f32*)(xw + 1024 + c16 * 4) = m0;
-        *(lds_f32*)(xw + 1024 + (16 + c16) * 4) = m1;
-      }
-
-      // ---- end of the run: the normaliser shares and final references go to the consumers
-      __syncthreads();  // the consumers are past their last P.V: the exchange blocks are free
-      {
-        const u32 xe = xch_hb + th * kPXchBlk;
-        const float ls0 = quad_rows_sum(l0), ls1 = quad_rows_sum(l1);
-        *(lds_f32*)(xe + c16 * 4) = ls0;
-        *(lds_f32*)(xe + (16 + c16) * 4) = ls1;
-        *(lds_f32*)(xe + 128 + c16 * 4) = m0;
-        *(lds_f32*)(xe + 128 + (16 + c16) * 4) = m1;
-      }
-      __syncthreads();
-    } else {
-      // =================================== consumer: tile loads, O^T += V^T . P^T, output
-      const int c32 = lane & 31;    // head column of the lane
-      const int g2 = lane >> 5;     // k-group of the lane
-      const int head = head0 + c32;
-      const bool head_ok = head < H;
-      const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
-      const int n_pages = (L + a.block_size - 1) >> a.bs_shift;
-      const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + kPPageOff);
-      // tile loads: consumer w4 moves rows w4*8 .. +7 of a sub-tile; bit 2 is clear in the first four.
-      // In the rope load lane (rr, pc) = (lane / 8, lane % 8) moves chunk pc ^ rr of row w4*8 + rr.
-      const u32 lane_off0 = lane * 16, lane_off1 = (lane ^ 1) * 16;
-      const int rr = lane >> 3;
-      const u32 rope_goff = (rr & 3) * kRowBytes + kDL * 2 + (((lane & 7) ^ rr) * 16);
-
-      f32x16 o[8];  // O^T blocks: dims th*256 + mb*32 + (8*(r/4) + 4 g2 + r%4), head c32
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[i][r] = 0.0f;
-      float R = kPRefInit;  // reference of the accumulators (head c32)
-
-      // 64 entries of the page table from page 64 ck on (the tail repeats the last page) -> chunk buffer ck & 1
-      auto issue_chunk = [&](int ck) {
-        dma4(pages + min(ck * kWave + lane, n_pages - 1), page_lds + (ck & 1) * kWave * 4);
-      };
-      int ck_cur = (t_begin >> a.bs_shift) >> 6;  // chunk of the sub-tile being issued
-      int chunk_pages = 0;                        // its 64 page ids, one per lane: a lookup is one v_readlane
-      // ---- issue state of the sub-tile being loaded: LDS targets and the bases of its two groups of 4 rows
-      uint64_t base0 = 0, base1 = 0;
-      u32 dst = 0, dst_rope = 0;
-      int tok0 = 0;
-      const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
-      auto page_of = [&](int tok) {  // wave-uniform token of the current chunk -> page id (clamped: a corrupt table must not fault the GPU)
-        const int page = __builtin_amdgcn_readlane(chunk_pages, (tok >> a.bs_shift) & 63);
-        return max(0, min(page, a.num_blocks - 1));
-      };
-      auto row_base = [&](int tok) {
-        const uint64_t row = cache + static_cast<uint64_t>(page_of(tok) * a.block_size + (tok & (a.block_size - 1))) * kRowBytes;
-        const u32 lo32 = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row)));
-        const u32 hi32 = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row >> 32)));
-        return (static_cast<uint64_t>(hi32) << 32) | lo32;
-      };
-      // returns true when all 8 rows of the wavefront are inside the context (block_size >= 16: each
-      // group of 4 rows then lies in one page and is loaded from one base)
-      auto prepare = [&](int sub) {
-        tok0 = t_begin + sub * kPSubTok + w4 * 8;
-        const u32 slot = lds_base + (sub & (kPRing - 1)) * kPSubBytes;
-        dst = __builtin_amdgcn_readfirstlane(slot + w4 * 8 * kPRowL);
-        dst_rope = __builtin_amdgcn_readfirstlane(slot + kPRopeOff + w4 * 8 * kDR * 2);
-        const int ck = (min(tok0, L - 1) >> a.bs_shift) >> 6;
-        if (ck != ck_cur) {  // first sub-tile of a chunk: consumer 0 fetches the one after it
-          ck_cur = ck;
-          if (w4 == 0 && (ck + 1) * kWave < n_pages) issue_chunk(ck + 1);
-          chunk_pages = pagebuf[(ck & 1) * kWave + lane];  // landed at least 32 sub-tiles (and as many barriers) ago
-        }
-        const bool inside = tok0 + 7 < L;
-        if (inside) {
-          base0 = row_base(tok0);
-          base1 = row_base(tok0 + 4);
-        }
-        return inside;
-      };
-      // load j of the 9 loads of a prepared sub-tile: latent rows 0..7, then the rope parts of all 8 rows
-      auto issue_part = [&](int j) {
-        switch (j) {  // (the row offset goes into the base: an instruction offset would also move the LDS address)
-          case 0: XLLM_DMA_ROWP(dst, base0, lane_off0, 0 * kPRowL); break;
-          case 1: XLLM_DMA_ROWP(dst, base0 + 1 * kRowBytes, lane_off0, 1 * kPRowL); break;
-          case 2: XLLM_DMA_ROWP(dst, base0 + 2 * kRowBytes, lane_off0, 2 * kPRowL); break;
-          case 3: XLLM_DMA_ROWP(dst, base0 + 3 * kRowBytes, lane_off0, 3 * kPRowL); break;
-          case 4: XLLM_DMA_ROWP(dst, base1, lane_off1, 4 * kPRowL); break;
-          case 5: XLLM_DMA_ROWP(dst, base1 + 1 * kRowBytes, lane_off1, 5 * kPRowL); break;
-          case 6: XLLM_DMA_ROWP(dst, base1 + 2 * kRowBytes, lane_off1, 6 * kPRowL); break;
-          case 7: XLLM_DMA_ROWP(dst, base1 + 3 * kRowBytes, lane_off1, 7 * kPRowL); break;
-          default: dma16(reinterpret_cast<const char*>(rr < 4 ? base0 : base1) + rope_goff, dst_rope); break;
-        }
-      };
-      // load j under an execution mask (all ones, or zero: nothing moves), for straight-line code
-      auto issue_part_masked = [&](int j, uint64_t mask) {
-        switch (j) {
-          case 0: XLLM_DMA_ROWP_MASKED(dst, base0, lane_off0, 0 * kPRowL, mask); break;
-          case 1: XLLM_DMA_ROWP_MASKED(dst, base0 + 1 * kRowBytes, lane_off0, 1 * kPRowL, mask); break;
-          case 2: XLLM_DMA_ROWP_MASKED(dst, base0 + 2 * kRowBytes, lane_off0, 2 * kPRowL, mask); break;
-          case 3: XLLM_DMA_ROWP_MASKED(dst, base0 + 3 * kRowBytes, lane_off0, 3 * kPRowL, mask); break;
-          case 4: XLLM_DMA_ROWP_MASKED(dst, base1, lane_off1, 4 * kPRowL, mask); break;
-          case 5: XLLM_DMA_ROWP_MASKED(dst, base1 + 1 * kRowBytes, lane_off1, 5 * kPRowL, mask); break;
-          case 6: XLLM_DMA_ROWP_MASKED(dst, base1 + 2 * kRowBytes, lane_off1, 6 * kPRowL, mask); break;
-          case 7: XLLM_DMA_ROWP_MASKED(dst, base1 + 3 * kRowBytes, lane_off1, 7 * kPRowL, mask); break;
-          default: dma16_masked(reinterpret_cast<const char*>(rr < 4 ? base0 : base1) + rope_goff, dst_rope, mask); break;
-        }
-      };
-      // the same 9 loads for a sub-tile that holds the ragged end of the context: rows past it repeat
-      // the last valid row, every row has its own base
-      auto issue_ragged = [&]() {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          dma16_row(row_base(min(tok0 + i, L - 1)), i < 4 ? lane_off0 : lane_off1, dst + i * kPRowL);
-        const int tok = min(tok0 + rr, L - 1);
-        int page = pagebuf[(((tok >> a.bs_shift) >> 6) & 1) * kWave + ((tok >> a.bs_shift) & 63)];
-        page = max(0, min(page, a.num_blocks - 1));
-        const char* row = a.k_cache + static_cast<int64_t>(page * a.block_size + (tok & (a.block_size - 1))) * kRowBytes;
-        dma16(row + kDL * 2 + (((lane & 7) ^ rr) * 16), dst_rope);
-      };
-
-      __syncthreads();  // the previous run no longer reads the ring, the chunks or the exchange blocks
-      if (w4 == 0) {
-        issue_chunk(ck_cur);
-        if ((ck_cur + 1) * kWave < n_pages) issue_chunk(ck_cur + 1);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
-      __syncthreads();
-      chunk_pages = pagebuf[(ck_cur & 1) * kWave + lane];
-      for (int sub = 0; sub < 2 && sub < n_sub; ++sub) {
-        if (prepare(sub)) {
-#pragma unroll
-          for (int j = 0; j < 9; ++j) issue_part(j);
-        } else {
-          issue_ragged();
-        }
-      }
-
-      // The loop exists twice.  In the first copy nothing but MFMAs touches the accumulators and the tile
-      // loads sit between the MFMAs; it is left when a head's reference has to rise after values were
-      // accumulated for it (a score more than kPSlack log2 units above every score seen before).  The
-      // second copy finishes the run: it rescales the accumulators whenever that happens again and issues
-      // its tile loads in one burst (with both in one loop body the compiler spills the accumulators).
-      auto iteration_begin = [&](int t) __attribute__((always_inline)) {
-        if (t + 2 < n_sub) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");  // the 9 loads of sub-tile t + 2 may be in flight
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();  // P(t) is visible, sub-tile t + 1 has landed, every wavefront is past sub-tile t - 1
-      };
-      // returns true (first copy only, before anything was issued or written) when the accumulators need rescaling
-      auto iteration_body = [&](int t, auto rescaling) __attribute__((always_inline)) -> bool {
-        constexpr bool kRescaling = decltype(rescaling)::value;
-        if (!wave_ok || t < 0) {  // nothing to multiply: the rows are still moved
-          if (t + 3 < n_sub) {
-            if (prepare(t + 3)) {
-#pragma unroll
-              for (int j = 0; j < 9; ++j) issue_part(j);
-            } else {
-              issue_ragged();
-            }
-          }
-          return false;
-        }
-        // ---- P^T(t) of both token blocks with their references, and the first V operands.  The transposing
-        // LDS read works on groups of 16 lanes (lane p supplies the address of 4 dims of token row p/4 and
-        // receives the 4 tokens of dim column p); the reads run kAheadV MFMAs ahead.
-        const u32 xr = xch_hb + (t & 1) * 4 * kPXchBlk;
-        const u32x4 pw0 = *(lds_u32x4*)(xr + (g2 * 32 + c32) * 16);
-        const u32x4 pw1 = *(lds_u32x4*)(xr + kPXchBlk + (g2 * 32 + c32) * 16);
-        const float ref0 = *(lds_f32*)(xr + 1024 + c32 * 4);
-        const float ref1 = *(lds_f32*)(xr + kPXchBlk + 1024 + c32 * 4);
-        u32 va;
-        {
-          int lv = lane;
-          asm volatile("" : "+v"(lv));
-          const int p16 = lv & 15, gg = lv >> 5;
-          va = lds_base + (t & (kPRing - 1)) * kPSubBytes + (4 * gg + (p16 >> 2)) * kPRowL + th * 512 +
-               (((((lv >> 4) & 1) * 2 + ((p16 & 3) >> 1)) ^ gg) * 16) + (p16 & 1) * 8;
-          asm volatile("" : "+v"(va));
-        }
-        constexpr int kAheadV = 4;
-        s16x4 vlo[kAheadV], vhi[kAheadV];
-        auto v_read = [&](int i) {  // operands of MFMA i: k-step i / 8 (tokens 16 kk ..), dim block i % 8
-          const u32 rows = va + (16 * (i >> 3)) * kPRowL + (i & 7) * 64;
-          vlo[i % kAheadV] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows));
-          vhi[i % kAheadV] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(rows + 8 * kPRowL));
-        };
-#pragma unroll
-        for (int i = 0; i < kAheadV; ++i) v_read(i);
-        asm volatile("" ::: "memory");
-        // ---- reference of the accumulators (a head whose reference is still the initial one has accumulated nothing)
-        const float Rn = fmaxf(R, fmaxf(ref0, ref1));
-        const bool rising = __builtin_amdgcn_ballot_w64(Rn != R && R != kPRefInit) != 0;
-        if constexpr (kRescaling) {
-          if (rising) {
-            const float alpha = fast_exp2(R - Rn);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] *= alpha;
-          }
-        } else {
-          if (rising) return true;
-        }
-        R = Rn;
-        bool spread = false;
-        if (t + 3 < n_sub) {  // sub-tile t + 3 goes into the slot of sub-tile t - 1
-          spread = prepare(t + 3);
-          if (!spread) issue_ragged();
-        }
-        if constexpr (kRescaling) {
-          if (spread) {
-#pragma unroll
-            for (int j = 0; j < 9; ++j) issue_part(j);
-          }
-        }
-        const uint64_t dma_mask = spread ? ~0ull : 0ull;
-        // ---- P^T(t) as B operands, scaled to the reference of the accumulators
-        const u32 dec0 = static_cast<u32>(fminf(R - ref0, 255.0f)) * 0x00800080u;
-        const u32 dec1 = static_cast<u32>(fminf(R - ref1, 255.0f)) * 0x00800080u;
-        bf16x8 pb[2];
-        {
-          const u32x4 w0 = {bf16x2_scale_down(pw0[0], dec0), bf16x2_scale_down(pw0[1], dec0),
-                            bf16x2_scale_down(pw0[2], dec0), bf16x2_scale_down(pw0[3], dec0)};
-          const u32x4 w1 = {bf16x2_scale_down(pw1[0], dec1), bf16x2_scale_down(pw1[1], dec1),
-                            bf16x2_scale_down(pw1[2], dec1), bf16x2_scale_down(pw1[3], dec1)};
-          pb[0] = __builtin_bit_cast(bf16x8, w0);
-          pb[1] = __builtin_bit_cast(bf16x8, w1);
-        }
-        // ---- O^T += V^T . P^T over the 32 tokens.  Step i: MFMA i, the V reads of MFMA i + kAheadV and, in
-        // the first copy of the loop, one tile load for i < 9 (under an execution mask that is zero when
-        // there is nothing to load).  The statements between the steps also keep the compiler from sinking
-        // the reads, so they stay kAheadV steps ahead of their use.  A wavefront that issues its 9 tile
-        // loads in one burst is held for 800 cycles: all four consumers queue at the one address unit of
-        // the CU.
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const s16x8 v = {vlo[i % kAheadV][0], vlo[i % kAheadV][1], vlo[i % kAheadV][2], vlo[i % kAheadV][3],
-                           vhi[i % kAheadV][0], vhi[i % kAheadV][1], vhi[i % kAheadV][2], vhi[i % kAheadV][3]};
-          o[i & 7] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, v), pb[i >> 3], o[i & 7], 0, 0, 0);
-          if (i + kAheadV < 16) v_read(i + kAheadV);
-          if constexpr (!kRescaling) {
-            if (i < 9) issue_part_masked(i, dma_mask);
-          }
-          asm volatile("" ::: "memory");
-        }
-        return false;
-      };
-      {
-        int t = -1;
-        bool rescale = false;
-        for (; t < n_sub; ++t) {
-          iteration_begin(t);
-          if (iteration_body(t, std::false_type{})) {
-            rescale = true;
-            break;
-          }
-        }
-        if (rescale) {
-          for (;;) {
-            iteration_body(t, std::true_type{});
-            if (++t >= n_sub) break;
-            iteration_begin(t);
-          }
-        }
-      }
-
-      // ---- end of the run: join the normaliser shares of the two producers of the head block
-      __syncthreads();
-      __syncthreads();  // (the producers write their shares between these two)
-      float lsum = 0.0f;
-#pragma unroll
-      for (int tb = 0; tb < 2; ++tb) {
-        const u32 xo = xch_hb + tb * kPXchBlk;
-        const float ls = *(lds_f32*)(xo + c32 * 4);
-        const float mr = *(lds_f32*)(xo + 128 + c32 * 4);
-        lsum += ls * fast_exp2(mr - R);  // R >= both references: every published reference was consumed
-      }
-      const float inv = 1.0f / lsum;
-      const float lse2 = R + fast_log2(lsum);
-      const int64_t ps = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H + head;
-      if (head_ok && complete) {
-        char* op = a.out + ((static_cast<int64_t>(b) * H + head) * kDL + th * 256) * 2;
-#pragma unroll
-        for (int mb = 0; mb < 8; ++mb)
-#pragma unroll
-          for (int qd = 0; qd < 4; ++qd) {
-            const u32x2 w = {BF16::pack(o[mb][4 * qd] * inv, o[mb][4 * qd + 1] * inv),
-                             BF16::pack(o[mb][4 * qd + 2] * inv, o[mb][4 * qd + 3] * inv)};
-            *reinterpret_cast<u32x2*>(op + (mb * 32 + 8 * qd + 4 * g2) * 2) = w;
-          }
-      }
-      if (head_ok && !complete) {
-        float* wp = a.ws_out + ps * kDL + th * 256;
-#pragma unroll
-        for (int mb = 0; mb < 8; ++mb)
-#pragma unroll
-          for (int qd = 0; qd < 4; ++qd) {
-            const f32x4 w = {o[mb][4 * qd] * inv, o[mb][4 * qd + 1] * inv, o[mb][4 * qd + 2] * inv, o[mb][4 * qd + 3] * inv};
-            *reinterpret_cast<f32x4*>(wp + mb * 32 + 8 * qd + 4 * g2) = w;
-          }
-      }
-      if (head_ok && g2 == 0 && th == 0 && complete && a.lse != nullptr) a.lse[b * H + head] = lse2 * kLn2;
-      if (head_ok && g2 == 0 && th == 0 && !complete) a.ws_lse[ps] = lse2;
-    }
-    first_run = false;
-  }
-}
-
 // Merge of the partials of contexts that span several teams; also writes the output of
 // empty sequences.  One workgroup per (head, sequence).
 template <typename QT>
@@ -2771,96 +2342,25 @@ __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
   if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * H + h] = (M + fast_log2(W)) * kLn2;
 }
 
-// The same merge for partial rows kept as tiles (mla_decode_w4_kernel).  One workgroup per (block of 16 heads,
-// sequence), laid out like the four wavefronts that wrote the tiles: wavefront w, lane (head c16, k-group g) owns
-// dims 128 w + 16 db + 4 g .. + 3 of head 16 hb + c16 for the eight dim blocks db, and every load instruction reads
-// 1 KB in one piece.  Four teams at a time, their 32 loads per lane issued together.
+// The merge of mla_decode_w4_kernel's partial rows as a launch of its own (when the decode kernel does not fold them
+// itself): one workgroup per (block of 16 heads, sequence); also writes the output of empty sequences.
 template <typename QT>
 __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
   const int hb = blockIdx.x;
   const int b = blockIdx.y;
-  const int H = a.n_heads;
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
-  const int c16 = lane & 15, g = lane >> 4;
-  const int hd = hb * 16 + c16;
-  const bool head_ok = hd < H;
 #ifdef XLLM_DS_TIMING
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)   // (measurement build only) when the merge kernel starts
-    reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H)[2048 * 10] = wall_clock64();
+    reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * a.n_heads)[2048 * 10] = wall_clock64();
 #endif
-  // (a context's share of what the schedule divides: run_cost, then its tiles)
-  const int64_t front = a.ws_prefix[b];
-  const int64_t first = front + a.run_cost;
-  const int64_t last = static_cast<int64_t>(a.ws_prefix[b + 1]) - 1;
-  const int64_t total = a.ws_prefix[a.batch];
-  char* out = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + w * 128 + 4 * g) * 2;
-  if (last < first) {  // empty sequence
-    if (head_ok) {
-#pragma unroll
-      for (int db = 0; db < 8; ++db) *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{0u, 0u};
-      if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * H + hd] = -INFINITY;
-    }
+  MlaPieces p;
+  if (!mla_locate_pieces(a, a.ws_prefix[b], a.ws_prefix[b + 1], a.ws_prefix[a.batch], p)) {  // empty sequence
+    mla_write_empty<QT>(a, hb, b, w, lane);
     return;
   }
-  const int64_t n = a.n_teams;
-  const int t_first = team_of(first, total, n);
-  const int t_last = team_of(last, total, n);
-  if (t_first == t_last) return;  // one team saw the whole context and wrote the output
-  // (team ranges stepped as in mla_merge_kernel)
-  const bool fits32 = total * n < (1LL << 31);
-  const int64_t q = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(total) / static_cast<uint32_t>(n)) : total / n, r = total - q * n;
-  int64_t acc = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(t_first) * static_cast<uint32_t>(r) % static_cast<uint32_t>(n))
-                       : (static_cast<int64_t>(t_first) * r) % n;
-  // (a range that starts in front of the context holds the last tile of an earlier one)
-  const int slot_first = team_start(t_first, total, n) < front ? 1 : 0;
-  const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 2;
-  const char* tiles = reinterpret_cast<const char*>(a.ws_out) + (hb * 4 + w) * 4096 + lane * 16;
-  float M = kNegBig, W = 0.0f;
-  f32x4 O[8];
-#pragma unroll
-  for (int db = 0; db < 8; ++db) O[db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  for (int tb = t_first; tb <= t_last; tb += 4) {
-    float lse[4];
-    u32x4 x[4][4];   // pairs of dim blocks, 16-bit values
-    bool on[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int t = tb + k;
-      acc += r;
-      const int64_t step = q + (acc >= n ? 1 : 0);
-      acc -= acc >= n ? n : 0;
-      on[k] = t <= t_last && step > 0 && head_ok;
-      const int64_t slot = static_cast<int64_t>(t) * 2 + (t == t_first ? slot_first : 0);
-      lse[k] = on[k] ? a.ws_lse[slot * H + hd] : kNegBig;
-#pragma unroll
-      for (int dp = 0; dp < 4; ++dp)
-        x[k][dp] = on[k] ? *reinterpret_cast<const u32x4*>(tiles + slot * slot_bytes + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
-    }
-    const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
-    const float keep = fast_exp2(M - m_new);
-    W *= keep;
-#pragma unroll
-    for (int db = 0; db < 8; ++db) O[db] *= keep;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
-      W += e;
-#pragma unroll
-      for (int dp = 0; dp < 4; ++dp) {
-        const u32x4 v = x[k][dp];
-        O[2 * dp] += e * f32x4{QT::lo(v[0]), QT::hi(v[0]), QT::lo(v[1]), QT::hi(v[1])};
-        O[2 * dp + 1] += e * f32x4{QT::lo(v[2]), QT::hi(v[2]), QT::lo(v[3]), QT::hi(v[3])};
-      }
-    }
-    M = m_new;
-  }
-  if (!head_ok) return;
-  const float inv = 1.0f / W;
-#pragma unroll
-  for (int db = 0; db < 8; ++db)
-    *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{QT::pack(O[db][0] * inv, O[db][1] * inv), QT::pack(O[db][2] * inv, O[db][3] * inv)};
-  if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * H + hd] = (M + fast_log2(W)) * kLn2;
+  if (p.t_first == p.t_last) return;  // one team saw the whole context and wrote the output
+  mla_merge_tiles<QT, false>(a, p, hb, b, w, lane, nullptr, nullptr);
 }
 
 // Teams: as many as there are CUs for the team size, a multiple of 8 (one per XCD slot).
@@ -2875,7 +2375,7 @@ int mla_teams(int n_hb) {
   return teams < 8 ? 8 : teams;
 }
 
-// Tuning knob XLLM_MI355_MLA_KERNEL, read once per process (first letter: 'p' pairs, 's' split); a test may
+// Tuning knob XLLM_MI355_MLA_KERNEL, read once per process (first letter: 'p' pairs, 'h' heads, 'n' narrow); a test may
 // override it through set_mla_kernel_knob.
 std::atomic<int> g_mla_knob{-1};
 int mla_kernel_knob() {
@@ -2927,17 +2427,14 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     return XLLM_MI355_EWORKSPACE;
 
   // "pairs" selects the kernel with the per-tile exchange (also taken for block sizes below 16 or not a power
-  // of two: the other kernels look pages up per group of 4 tokens inside chunks of 64 pages), "split" the
-  // producer / consumer kernel
+  // of two: the other kernels look pages up per group of 4 tokens inside chunks of 64 pages)
   const int knob = mla_kernel_knob();
   const bool pairs = knob == 'p' || block_size < 16 || (block_size & (block_size - 1)) != 0;
-  const bool split = knob == 's' && !pairs && !f16;  // (the producer / consumer kernel is written for bf16)
   // more than 64 heads: scores by head block, P.V by dim block ("heads" keeps P.V by head block, for comparison)
-  const bool by_dims = !pairs && !split && knob != 'h' && n_heads > 64;
+  const bool by_dims = !pairs && knob != 'h' && n_heads > 64;
   const int64_t max_batch = by_dims ? (kDsMaxBatch < kMaxBatchMla ? kDsMaxBatch : kMaxBatchMla) : kMaxBatchMla;
   const int n_hb = static_cast<int>(pairs ? (n_heads + kHeadsPerWg - 1) / kHeadsPerWg
                                           : (n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
-  const int n_hb_p = static_cast<int>((n_heads + kHeadsPerWg - 1) / kHeadsPerWg);
   static std::atomic<uint64_t> configured{0};
   const size_t smem = pairs ? kPrefixOff + (kMaxBatchMla + 1) * 4 : kPrefix16Off + (kMaxBatchMla + 1) * 4;
   if (first_use_on_current_device(configured)) {
@@ -2962,9 +2459,6 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
                                 reinterpret_cast<const void*>(mla_decode_w4_kernel<FP16>)};
     for (const void* k : kernels_w4)
       if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kW4LdsBytes);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(mla_decode32w_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
     if (e != hipSuccess) return static_cast<int>(e);
   }
   for (int64_t b0 = 0; b0 < batch; b0 += max_batch) {
@@ -2980,8 +2474,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.table_stride = addr.table_stride;
     a.batch = static_cast<int>(nb);
     a.n_heads = static_cast<int>(n_heads);
-    const bool use_p = split && nb <= kPMaxBatch;  // (its LDS has room for the tile prefix of kPMaxBatch sequences)
-    a.n_hb = use_p ? n_hb_p : n_hb;
+    a.n_hb = n_hb;
     a.n_teams = mla_teams(a.n_hb);
     a.block_size = static_cast<int>(block_size);
     a.bs_shift = -1;
@@ -2996,9 +2489,9 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     // (XLLM_MLA_DEFAULT_NARROW: the build found that the compiler did not leave the fixed-name accumulators of
     // mla_decode_w4_kernel alone and made the eight-wavefront kernel the default; 'w' still asks for the other)
 #ifdef XLLM_MLA_DEFAULT_NARROW
-    const bool w4 = !pairs && !use_p && by_dims && knob == 'w';
+    const bool w4 = !pairs && by_dims && knob == 'w';
 #else
-    const bool w4 = !pairs && !use_p && by_dims && knob != 'n';
+    const bool w4 = !pairs && by_dims && knob != 'n';
 #endif
     static const int run_cost = [] {
       const char* e = getenv("XLLM_MI355_MLA_RUN_COST");  // tuning knob: tiles charged for the start of a run
@@ -3011,8 +2504,6 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     if (pairs) {
       if (f16) launch_timed(mla_decode_kernel<FP16>, grid, dim3(kMlaThreads), smem, stream, a);
       else launch_timed(mla_decode_kernel<BF16>, grid, dim3(kMlaThreads), smem, stream, a);
-    } else if (use_p) {
-      launch_timed(mla_decode32w_kernel, grid, dim3(kWThreads), kPLdsBytes, stream, a);
     } else if (w4) {  // ('n'arrow: the kernel with 16 heads per scoring wavefront, 3 % slower on 128 heads)
       if (f16) launch_timed(mla_decode_w4_kernel<FP16>, grid, dim3(kW4Threads), kW4LdsBytes, stream, a);
       else launch_timed(mla_decode_w4_kernel<BF16>, grid, dim3(kW4Threads), kW4LdsBytes, stream, a);
