@@ -296,7 +296,7 @@ def decode_kernel_name(cfg):
             return "mla_decode16_kernel"
         return "mla_decode_ds_kernel" if knob == "n" else "mla_decode_w4_kernel"
     mfma = (cfg.head_dim in (64, 128) or (cfg.head_dim == 256 and cfg.cache_dtype != "fp8")) and cfg.block_size >= 16 \
-        and cfg.block_size & (cfg.block_size - 1) == 0
+        and cfg.block_size & (cfg.block_size - 1) == 0 and os.environ.get("XLLM_MI355_GQA_KERNEL", "")[:1] != "r"
     return "gqa_mfma_kernel" if mfma else "gqa_decode_kernel"
 
 
