@@ -442,11 +442,18 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     # ---- the same step as the layers after the first see it when the step was planned once (not the headline:
     # `value` above is the self-contained call, which derives its schedule in every launch)
     planned = None
-    if not cfg.mla and not args.no_planned:
+    if not args.no_planned and (not cfg.mla or cfg.n_q_heads > 64):
         plan = torch.empty(lib.xllm_mi355_paged_decode_plan_bytes(), dtype=torch.uint8, device=dev)
-        plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), None, None, None, cfg.batch,
-                     cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, -1, code[cache_dt], stream)
-        planned_bound = [(r, (ptr(plan), plan.numel()) + d[:8] + (None, None, None) + d[8:]) for r, d in bound]
+        if cfg.mla:
+            plan_fn, planned_fn = lib.xllm_mi355_paged_decode_mla_plan, lib.xllm_mi355_paged_decode_mla_planned
+            plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), cfg.batch, cfg.n_q_heads,
+                         cfg.block_size, stream)
+            planned_bound = [(r, (ptr(plan), plan.numel()) + d) for r, d in bound]
+        else:
+            plan_fn, planned_fn = lib.xllm_mi355_paged_decode_gqa_plan, lib.xllm_mi355_paged_decode_gqa_planned
+            plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), None, None, None, cfg.batch,
+                         cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, -1, code[cache_dt], stream)
+            planned_bound = [(r, (ptr(plan), plan.numel()) + d[:8] + (None, None, None) + d[8:]) for r, d in bound]
         plain_out = out.clone()
         p_state = [0]
 
@@ -454,12 +461,12 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
             r_args, d_args = planned_bound[p_state[0] % ROTATE]
             p_state[0] += 1
             rc = reshape_fn(*r_args)
-            rc2 = lib.xllm_mi355_paged_decode_gqa_planned(*d_args)
+            rc2 = planned_fn(*d_args)
             if rc or rc2:
                 capi.check(rc or rc2, "bench planned step")
 
         capi.check(lib.xllm_mi355_profile_enable(1), "profile_enable")
-        capi.check(lib.xllm_mi355_paged_decode_gqa_plan(*plan_args), "xllm_mi355_paged_decode_gqa_plan")
+        capi.check(plan_fn(*plan_args), "the plan of the step")
         torch.cuda.synchronize()
         plan_ms = collect_ms(lib, 1)
         p_ms_per_step, _, _ = timed_loop(planned_step, events=False)
@@ -535,6 +542,9 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     if flops is not None:
         roofline["algorithmic_flops"] = flops
     if planned is not None:
+        p_op = (planned["kernel_ms"] + planned["merge_kernel_ms"]) * 1e-3
+        planned["op_frac"] = (flops / p_op / 1e12 / MFMA_BF16_PEAK_TFLOPS) if roofline["bound"] == "mfma" \
+            else (nbytes / p_op / 1e9 / HBM_PEAK_GBS)
         roofline["planned"] = planned
     # the same number of bytes through the plain read kernel: the rate this GPU sustains at this size
     roofline["stream_read_gbs_same_bytes"], _ = stream_rate(lib, capi, torch, dev, nbytes)

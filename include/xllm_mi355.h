@@ -355,6 +355,36 @@ int xllm_mi355_paged_decode_mla(const void* q_nope, const void* q_pe, const void
                                 int dtype, void* stream);
 
 /*
+ * The plan of an MLA decode step, made once and used by the decode calls of every layer: the counterpart of the
+ * tile-scheduler metadata that the reference computes apart from the decode call
+ * (get_mla_decoding_metadata_dense_fp8, xllm/core/kernels/dcu/flash_mla_adapter.cpp:125-130) and of the plan that its
+ * FlashInfer path makes at layer 0 only (xllm/core/layers/cuda/flashinfer_planinfo.cpp:248-264).  Same buffer as the
+ * GQA plan (xllm_mi355_paged_decode_plan_bytes() bytes, 256-byte aligned, the caller's), same rules: one small launch
+ * writes the schedule's prefix, the lengths and every workgroup team's first page-table entries;
+ * xllm_mi355_paged_decode_mla_planned is xllm_mi355_paged_decode_mla that starts from them: same kernel, same order of
+ * arithmetic, bit-identical results.  A plan serves the kernel for more than 64 heads with a block size that is a
+ * power of two >= 16 and batches of at most 1024 sequences; other calls take no plan and are decoded as by the plain
+ * entry point.  A planned call whose shape differs from the plan's writes no output, one whose lengths differ from
+ * those the plan was made with writes an invalid one; both raise the flag that xllm_mi355_decode_status reports as
+ * XLLM_MI355_EPLAN.  A plan buffer below xllm_mi355_paged_decode_plan_bytes() is refused with XLLM_MI355_EWORKSPACE.
+ */
+int xllm_mi355_paged_decode_mla_plan(void* plan, size_t plan_bytes,
+                                     const int32_t* block_table, int64_t table_stride,
+                                     const int32_t* seq_lens,
+                                     int64_t batch, int64_t n_heads, int64_t block_size, void* stream);
+int xllm_mi355_paged_decode_mla_planned(const void* plan, size_t plan_bytes,
+                                        const void* q_nope, const void* q_pe, const void* k_cache,
+                                        void* out, float* lse,
+                                        const int32_t* block_table, int64_t table_stride,
+                                        const int32_t* seq_lens,
+                                        int64_t batch, int64_t n_heads,
+                                        int64_t d_latent, int64_t d_rope,
+                                        int64_t block_size, int64_t num_blocks,
+                                        int64_t max_seq_len, float sm_scale,
+                                        void* workspace, size_t workspace_bytes,
+                                        int dtype, void* stream);
+
+/*
  * Log-sum-exp merge of S partial attention results.
  * Replaces xllm::layer::merge_dcp_attention_shards
  * (xllm/core/layers/mlu/dcp_attention_merge.cpp:26-65):
@@ -484,12 +514,17 @@ int xllm_mi355_profile_collect(float* ms_out, int max_n);
  * XLLM_MI355_DEBUG_GQA_STREAM_STORES: 1 / 0 make the matrix-core GQA kernel write its output and partial rows with /
  * without non-temporal stores whatever the size of the launch, negative gives the choice back to the library (same
  * as XLLM_MI355_GQA_STREAM_STORES in the environment; the bytes written are the same either way).
+ * XLLM_MI355_DEBUG_MLA_FOLD: 1 makes the MLA decode kernel for more than 64 heads merge the contexts that span several
+ * workgroups itself, 0 leaves them to a second launch (the default: it measures the same, and the one launch needs every
+ * workgroup resident at once), negative gives the choice back to the environment (XLLM_MI355_MLA_FOLD = 1 turns it on);
+ * the outputs are the same bits either way.
  */
 enum {
   XLLM_MI355_DEBUG_WAIT_SPINS = 0,
   XLLM_MI355_DEBUG_MLA_KERNEL = 1,
   XLLM_MI355_DEBUG_GQA_FOLD = 2,
-  XLLM_MI355_DEBUG_GQA_STREAM_STORES = 3
+  XLLM_MI355_DEBUG_GQA_STREAM_STORES = 3,
+  XLLM_MI355_DEBUG_MLA_FOLD = 4
 };
 int xllm_mi355_debug_set(int what, int value);
 

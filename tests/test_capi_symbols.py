@@ -95,6 +95,17 @@ def test_planned_decode_refuses_a_short_plan_buffer_before_any_launch():
     assert planned(fake, 4096) == -4
     assert planned(fake, need - 1) == -4
 
+    def mla_planned(plan, plan_bytes):
+        return lib.xllm_mi355_paged_decode_mla_planned(
+            plan, plan_bytes, fake, fake, fake, fake, None, fake, 8, fake, 4, 128, 512, 64, 64, 10, 100, 0.1, fake,
+            1 << 30, capi.BF16, None)
+
+    assert mla_planned(None, need) == -1
+    assert mla_planned(fake, 4096) == -4
+    assert mla_planned(fake, need - 1) == -4
+    assert lib.xllm_mi355_paged_decode_mla_plan(fake, need - 1, fake, 8, fake, 4, 128, 64, None) == -4
+    assert lib.xllm_mi355_paged_decode_mla_plan(fake, need, None, 8, fake, 4, 128, 64, None) == -1
+
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(capi, "_lib", None)

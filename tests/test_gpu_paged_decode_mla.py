@@ -228,6 +228,73 @@ def test_head_counts_page_table_chunk_boundaries_and_long_contexts(device):
     _check(_mla_cfg("long", 1, 128, 6000, 9000), 6, device)
 
 
+def _set_fold(on):
+    """Whether the default kernel for more than 64 heads merges split contexts itself (1) or leaves them to a second
+    launch (0); -1 gives the choice back to the environment."""
+    from xllm_amd import capi
+    assert capi.lib().xllm_mi355_debug_set(4, on) == 0
+
+
+def test_merge_inside_the_decode_kernel_is_the_same_bits_as_the_merge_launch(device):
+    # contexts cut across many workgroups, across two, whole ones, empty ones; head counts that fill one workgroup per
+    # team, leave its last head block ragged, or need two workgroups per team; fewer tiles than workgroups
+    g = torch.Generator().manual_seed(5)
+    cases = [_mla_cfg("fold_b3", 3, 128, 100, 1500), _mla_cfg("fold_b9_long", 9, 128, 3000, 9000),
+             _mla_cfg("fold_b40", 40, 128, 1, 700), _mla_cfg("fold_h80", 5, 80, 200, 4000),
+             _mla_cfg("fold_h200", 4, 200, 500, 5000), _mla_cfg("fold_one", 1, 128, 12000, 12000),
+             _mla_cfg("fold_tiny", 2, 128, 1, 90), _mla_cfg("fold_bs16", 6, 128, 300, 2500, bs=16)]
+    for n, cfg in enumerate(cases):
+        inp = workloads.make_inputs(cfg, 700 + n)
+        kg, _, _, _ = fill_caches_gpu(inp, device)
+        lens = inp.layout.seq_lens.clone()
+        if cfg.batch > 4:
+            lens[torch.rand(cfg.batch, generator=g) < 0.3] = 0
+        results = []
+        try:
+            for on in (0, 1, 1):   # (twice with the merge inside: the counters it leaves behind must be back at zero)
+                _set_fold(on)
+                results.append(_decode_gpu(inp, kg, device, seq_lens=lens))
+        finally:
+            _set_fold(-1)
+        assert ops.decode_status(device) == 0
+        for out, lse in results[1:]:
+            assert torch.equal(out.view(torch.int16), results[0][0].view(torch.int16)), cfg.name
+            assert torch.equal(lse, results[0][1]), cfg.name
+        if n in (0, 3, 6):
+            live = torch.nonzero(lens > 0).flatten().tolist()
+            ref = oracle.aten_paged_decode(inp.q[live].contiguous(), kg.cpu(), None, inp.layout.block_table[live].contiguous(),
+                                           lens[live].contiguous(), cfg.scale, dv=cfg.v_dim)
+            assert_close_to_reference(results[1][0][live], ref, cfg.name)
+            dead = torch.nonzero(lens == 0).flatten().tolist()
+            assert not results[1][0][dead].float().abs().any() and torch.isneginf(results[1][1][dead]).all()
+
+
+def test_a_merging_workgroup_that_gives_up_is_reported(device):
+    """The workgroups that merge a context wait for its pieces with a bounded poll.  With the bound at zero they give
+    up at once (every wavefront still ends normally): the status call reports it, clears the counters the launch left
+    behind, and the next launch is right again."""
+    from xllm_amd import capi
+    lib = capi.lib()
+    cfg = _mla_cfg("fold_stall", 3, 128, 2500, 6000)
+    inp = workloads.make_inputs(cfg, 77)
+    kg, _, _, _ = fill_caches_gpu(inp, device)
+    good, good_lse = _decode_gpu(inp, kg, device)
+    assert ops.decode_status(device) == 0
+    try:
+        _set_fold(1)
+        assert lib.xllm_mi355_debug_set(0, 0) == 0
+        _decode_gpu(inp, kg, device)
+        assert lib.xllm_mi355_debug_set(0, -1) == 0
+        with pytest.raises(capi.XllmMi355Error, match="gave up"):
+            ops.decode_status(device)
+        assert ops.decode_status(device) == 0   # reported once, then cleared
+        again, again_lse = _decode_gpu(inp, kg, device)
+        assert torch.equal(again, good) and torch.equal(again_lse, good_lse) and ops.decode_status(device) == 0
+    finally:
+        assert lib.xllm_mi355_debug_set(0, -1) == 0
+        _set_fold(-1)
+
+
 def test_shard_merge_equals_full_decode(device):
     # ArtificialShardMergeMatchesFullCacheDecode (dcp_attention_merge_test.cpp:146-224): rtol/atol 1e-2, 1e-3
     cfg = _mla_cfg("merge", 4, 128, 256, 2000)

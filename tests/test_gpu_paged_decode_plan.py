@@ -307,3 +307,143 @@ def test_random_shapes_plain_planned_and_both_kinds_of_stores_agree(device):
                                            lay.block_table[keep].contiguous(), lens[keep].contiguous(), cfg.scale,
                                            None if ks is None else ks.cpu(), None if vs is None else vs.cpu())
             assert_close_to_reference(base[0][keep.to(device)], ref, cfg.name)
+
+
+# ---- the MLA decode from a plan -------------------------------------------------------------------------------------
+
+def _mla_cfg(name, batch, heads, lo, hi, bs=64):
+    import math
+    return workloads.DecodeConfig(name, batch, heads, 1, 576, bs, lo, hi, mla=True, v_dim=512, sigma=0.5,
+                                  sm_scale=1.0 / math.sqrt(192.0))
+
+
+def _mla_params(inp, kg, device, lens=None):
+    cfg, lay = inp.cfg, inp.layout
+    q = inp.q.to(device)
+    B, H = cfg.batch, cfg.n_q_heads
+    return ops.DenseDecodeParams(
+        q_nope=q[:, :, :512].contiguous().view(B, 1, H, 512), q_pe=q[:, :, 512:].contiguous().view(B, 1, H, 64),
+        k_cache=kg, seqlens_k=(lay.seq_lens if lens is None else lens).to(device), block_table=lay.block_table.to(device),
+        head_size_v=512, softmax_scale=cfg.scale)
+
+
+def test_mla_planned_decode_is_bit_identical(device):
+    g = torch.Generator().manual_seed(3)
+    # 128 heads (one workgroup per team), a ragged last head block, two workgroups per team, a block size of 16, many
+    # short sequences, fewer tiles than workgroups; and head counts / block sizes that take no plan (other kernels)
+    cases = [_mla_cfg("p128", 7, 128, 200, 5000), _mla_cfg("p80", 4, 80, 100, 3000), _mla_cfg("p200", 3, 200, 500, 4000),
+             _mla_cfg("p_bs16", 5, 128, 100, 2500, bs=16), _mla_cfg("p_short", 300, 128, 1, 150),
+             _mla_cfg("p_tiny", 2, 128, 1, 70), _mla_cfg("p16", 6, 16, 100, 2000), _mla_cfg("p_bs8", 3, 128, 50, 600, bs=8)]
+    for n, cfg in enumerate(cases):
+        inp = workloads.make_inputs(cfg, 900 + n)
+        kg, _, _, _ = fill_caches_gpu(inp, device)
+        lens = inp.layout.seq_lens.clone()
+        if cfg.batch > 4:
+            lens[torch.rand(cfg.batch, generator=g) < 0.25] = 0
+        p = _mla_params(inp, kg, device, lens)
+        plain, plain_lse = ops.dense_decode(p, return_lse=True)
+        plan = ops.get_mla_decoding_metadata(p.seqlens_k, p.block_table, cfg.n_q_heads, cfg.block_size)
+        for _ in range(2):   # the layers of a step share the plan
+            out, lse = ops.dense_decode(p, return_lse=True, metadata=plan)
+            assert torch.equal(out.view(torch.int16), plain.view(torch.int16)), cfg.name
+            assert torch.equal(lse, plain_lse), cfg.name
+        assert ops.decode_status(device) == 0
+    lib = capi.lib()
+    cfg = cases[0]
+    inp = workloads.make_inputs(cfg, 900)
+    kg, _, _, _ = fill_caches_gpu(inp, device)
+    p = _mla_params(inp, kg, device)
+    plain = ops.dense_decode(p)
+    plan = ops.get_mla_decoding_metadata(p.seqlens_k, p.block_table, cfg.n_q_heads, cfg.block_size)
+    try:   # the merge inside the decode kernel, from a plan
+        assert lib.xllm_mi355_debug_set(4, 1) == 0
+        assert torch.equal(ops.dense_decode(p, metadata=plan), plain)
+    finally:
+        assert lib.xllm_mi355_debug_set(4, -1) == 0
+    assert ops.decode_status(device) == 0
+
+
+def test_a_stale_mla_plan_is_reported(device):
+    cfg = _mla_cfg("stale", 9, 128, 300, 4000)
+    inp = workloads.make_inputs(cfg, 31)
+    kg, _, _, _ = fill_caches_gpu(inp, device)
+    p = _mla_params(inp, kg, device)
+    assert ops.decode_status(device) == 0
+    plan = ops.get_mla_decoding_metadata(p.seqlens_k, p.block_table, cfg.n_q_heads, cfg.block_size)
+    good = ops.dense_decode(p, metadata=plan)
+    assert ops.decode_status(device) == 0
+    # the lengths moved on, the plan did not
+    for lens in ((inp.layout.seq_lens - 1), torch.clamp(inp.layout.seq_lens - 900, min=0)):
+        q = _mla_params(inp, kg, device, lens.to(torch.int32).contiguous())
+        ops.dense_decode(q, metadata=plan)
+        with pytest.raises(capi.XllmMi355Error, match="plan"):
+            ops.decode_status(device)
+        assert ops.decode_status(device) == 0
+        fresh = ops.get_mla_decoding_metadata(q.seqlens_k, q.block_table, cfg.n_q_heads, cfg.block_size, plan=plan)
+        assert fresh.data_ptr() == plan.data_ptr()
+        assert torch.equal(ops.dense_decode(q, metadata=fresh), ops.dense_decode(q))
+        assert ops.decode_status(device) == 0
+    # a plan made for another batch: nothing is written
+    other = ops.get_mla_decoding_metadata(p.seqlens_k[:8].contiguous(), p.block_table[:8], cfg.n_q_heads, cfg.block_size)
+    ops.dense_decode(p, metadata=other)
+    with pytest.raises(capi.XllmMi355Error, match="plan"):
+        ops.decode_status(device)
+    assert ops.decode_status(device) == 0
+    again = ops.get_mla_decoding_metadata(p.seqlens_k, p.block_table, cfg.n_q_heads, cfg.block_size)
+    assert torch.equal(ops.dense_decode(p, metadata=again), good) and ops.decode_status(device) == 0
+
+
+def test_a_captured_mla_step_plans_again_on_every_replay(device):
+    # plan + decode captured once; the replays see new lengths and tables in the same buffers and plan from them
+    cfg = _mla_cfg("pgraph", 6, 128, 100, 2500)
+    inputs = [workloads.make_inputs(cfg, 440 + i) for i in range(3)]
+    width = max(inp.layout.block_table.shape[1] for inp in inputs)
+    blocks = max(inp.layout.num_blocks for inp in inputs)
+    k_cache = torch.zeros(blocks, cfg.block_size, 1, 576, dtype=torch.bfloat16, device=device)
+    table = torch.zeros(cfg.batch, width, dtype=torch.int32, device=device)
+    lens = torch.zeros(cfg.batch, dtype=torch.int32, device=device)
+    q_nope = torch.zeros(cfg.batch, 1, cfg.n_q_heads, 512, dtype=torch.bfloat16, device=device)
+    q_pe = torch.zeros(cfg.batch, 1, cfg.n_q_heads, 64, dtype=torch.bfloat16, device=device)
+    plan = torch.zeros(capi.lib().xllm_mi355_paged_decode_plan_bytes(), dtype=torch.uint8, device=device)
+    result = {}
+
+    def load(inp):
+        lay = inp.layout
+        k_cache.zero_()
+        for k, slots in ((inp.k_ctx, lay.ctx_slots), (inp.k_new, lay.new_slots)):
+            ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=k.to(device), value=None, k_cache=k_cache,
+                                                                v_cache=None, slot_mapping=slots.to(device)))
+        table.zero_()
+        table[:, : lay.block_table.shape[1]] = lay.block_table.to(device)
+        lens.copy_(lay.seq_lens.to(device))
+        q = inp.q.to(device)
+        q_nope.copy_(q[:, :, :512].reshape(cfg.batch, 1, cfg.n_q_heads, 512))
+        q_pe.copy_(q[:, :, 512:].reshape(cfg.batch, 1, cfg.n_q_heads, 64))
+
+    def params():
+        return ops.DenseDecodeParams(q_nope=q_nope, q_pe=q_pe, k_cache=k_cache, seqlens_k=lens, block_table=table,
+                                     head_size_v=512, softmax_scale=cfg.scale)
+
+    def step():
+        ops.get_mla_decoding_metadata(lens, table, cfg.n_q_heads, cfg.block_size, plan=plan)
+        result["a"] = ops.dense_decode(params(), max_seq_len=width * cfg.block_size, metadata=plan)
+        result["b"] = ops.dense_decode(params(), max_seq_len=width * cfg.block_size, metadata=plan)   # a second layer
+
+    load(inputs[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up outside the capture: workspace allocation, kernel attributes
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for inp in inputs[1:] + inputs[:1]:
+        load(inp)
+        eager = ops.dense_decode(params(), max_seq_len=width * cfg.block_size)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(result["a"], eager) and torch.equal(result["b"], eager)
+        assert ops.decode_status(device) == 0

@@ -14,6 +14,7 @@ int wait_spin_limit() { return g_wait_spins.load(std::memory_order_relaxed); }
 void set_mla_kernel_knob(int first_letter);  // paged_decode_mla.hip
 void set_fold_merge(int on);                 // paged_decode_gqa.hip
 void set_stream_stores(int v);               // paged_decode_gqa.hip
+void set_mla_fold(int on);                   // paged_decode_mla.hip
 }  // namespace xllm_mi355
 
 // Scratch of xllm_mi355_paged_decode_gqa_static: a decode workspace that lives in the code object, one copy
@@ -140,6 +141,9 @@ int xllm_mi355_debug_set(int what, int value) {
       return XLLM_MI355_OK;
     case XLLM_MI355_DEBUG_GQA_STREAM_STORES:
       set_stream_stores(value);
+      return XLLM_MI355_OK;
+    case XLLM_MI355_DEBUG_MLA_FOLD:
+      set_mla_fold(value);
       return XLLM_MI355_OK;
     default: return XLLM_MI355_EINVAL;
   }
@@ -319,6 +323,35 @@ int xllm_mi355_paged_decode_mla(const void* q_nope, const void* q_pe, const void
   return paged_decode_mla(q_nope, q_pe, k_cache, out, lse, addr, batch, n_heads, d_latent, d_rope,
                           block_size, num_blocks, max_seq_len, sm_scale, workspace, workspace_bytes,
                           dtype, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_paged_decode_mla_plan(void* plan, size_t plan_bytes, const int32_t* block_table, int64_t table_stride,
+                                     const int32_t* seq_lens, int64_t batch, int64_t n_heads, int64_t block_size,
+                                     void* stream) {
+  PageAddressing addr;
+  addr.block_table = block_table;
+  addr.table_stride = table_stride;
+  addr.seq_lens = seq_lens;
+  return paged_decode_mla_plan(plan, plan_bytes, addr, batch, n_heads, block_size, static_cast<hipStream_t>(stream));
+}
+
+int xllm_mi355_paged_decode_mla_planned(const void* plan, size_t plan_bytes, const void* q_nope, const void* q_pe,
+                                        const void* k_cache, void* out, float* lse, const int32_t* block_table,
+                                        int64_t table_stride, const int32_t* seq_lens, int64_t batch, int64_t n_heads,
+                                        int64_t d_latent, int64_t d_rope, int64_t block_size, int64_t num_blocks,
+                                        int64_t max_seq_len, float sm_scale, void* workspace, size_t workspace_bytes,
+                                        int dtype, void* stream) {
+  if (plan == nullptr) return XLLM_MI355_EINVAL;
+  // (the kernel reads the plan up to its last word before it looks at its signature)
+  if (plan_bytes < gqa_plan_bytes()) return XLLM_MI355_EWORKSPACE;
+  PageAddressing addr;
+  addr.block_table = block_table;
+  addr.table_stride = table_stride;
+  addr.seq_lens = seq_lens;
+  addr.plan = plan;
+  return paged_decode_mla(q_nope, q_pe, k_cache, out, lse, addr, batch, n_heads, d_latent, d_rope, block_size,
+                          num_blocks, max_seq_len, sm_scale, workspace, workspace_bytes, dtype,
+                          static_cast<hipStream_t>(stream));
 }
 
 int xllm_mi355_lse_merge(const void* partial_out, const float* partial_lse, void* out, float* lse,

@@ -57,6 +57,19 @@ constexpr size_t kWsPartialsOff = kWsHeaderBytes + (static_cast<size_t>(kWsMaxBa
 constexpr int kStatusWaitGaveUp = 1;  // a bounded wait of one wavefront on another ran out: the launch's output is invalid
 constexpr int kStatusPlanMismatch = 2;  // a decode launch was given a plan made for another shape (it wrote no output) or for other lengths
 
+// A plan of a decode step (ints), made once per step and read by the decode launches of every layer.  Word 0: the
+// signature of what it was made for | from kPlanPrefixOff the item prefix [batch + 1] of the schedule and, for the GQA
+// kernel, the cut between its pools | from kPlanChunksOff 64 page-table entries per team (group of workers of the GQA
+// kernel, workgroup team of the MLA kernel): the chunk of the context's table that holds the page of the team's first
+// tokens; the tail repeats the context's last page | from kPlanLensOff the context lengths [batch] the plan was made
+// with: a planned call compares them with its own, so that a plan that was not made again for a new step is reported
+// (kStatusPlanMismatch) instead of followed silently.
+constexpr int kPlanPrefixOff = 64;
+constexpr int kPlanChunksOff = kPlanPrefixOff + (kWsMaxBatch + 2 + 63) / 64 * 64;
+constexpr int kPlanMaxTeams = 4096;
+constexpr int kPlanLensOff = kPlanChunksOff + kPlanMaxTeams * 64;
+constexpr size_t kPlanBytes = (static_cast<size_t>(kPlanLensOff) + static_cast<size_t>(kWsMaxBatch)) * 4;
+
 // Bound of the polls of one wavefront on another (test hook: xllm_mi355_debug_set_wait_spins).
 int wait_spin_limit();
 
@@ -82,6 +95,10 @@ size_t gqa_plan_bytes();
 int paged_decode_gqa_plan(void* plan, size_t plan_bytes, const PageAddressing& addr, int64_t batch, int64_t n_q_heads,
                           int64_t n_kv_heads, int64_t head_dim, int64_t block_size, int cache_dtype,
                           hipStream_t stream);
+
+// The plan of an MLA decode step (the same buffer as the GQA plan, for the kernel that serves more than 64 heads).
+int paged_decode_mla_plan(void* plan, size_t plan_bytes, const PageAddressing& addr, int64_t batch, int64_t n_heads,
+                          int64_t block_size, hipStream_t stream);
 
 int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out, float* lse,
                      const PageAddressing& addr, int64_t batch, int64_t n_heads, int64_t d_latent,

@@ -175,13 +175,23 @@ __global__ __launch_bounds__(256) void expand_varlen_kernel(const int32_t* cu_se
 // (16 when the row length allows it), consecutive threads taking consecutive pieces of a row.  Rows whose
 // page id is negative or beyond the cache are left untouched, as in the reference kernel (which skips
 // negative ids; an id beyond the cache would be an out-of-bounds read there).
+// The search is a chain of dependent reads, so the row offsets go to LDS first when they fit (one trip to memory for
+// all of them instead of log2(batch) in a row), and a thread asks for four pieces before it stores the first: the
+// launch is a stream of rows that are read once, fetched with non-temporal loads.
+constexpr int kGatherCuLds = 2048;   // row offsets kept in LDS
 template <int VB>
 __global__ __launch_bounds__(256) void gather_paged_rows_kernel(const char* cache, const int32_t* block_table,
                                                                 int64_t table_stride, const int32_t* cu_seq_lens,
                                                                 char* out, int batch, int64_t total_rows,
                                                                 int block_size, int num_blocks, int row_bytes) {
   __shared__ int64_t src_row[32];
+  __shared__ int cu_l[kGatherCuLds + 1];
   const int64_t row0 = static_cast<int64_t>(blockIdx.x) * 32;
+  const bool in_lds = batch <= kGatherCuLds;
+  if (in_lds) {
+    for (int i = threadIdx.x; i <= batch; i += 256) cu_l[i] = cu_seq_lens[i];
+    __syncthreads();
+  }
   if (threadIdx.x < 32) {
     const int64_t row = row0 + threadIdx.x;
     int64_t src = -1;
@@ -189,10 +199,11 @@ __global__ __launch_bounds__(256) void gather_paged_rows_kernel(const char* cach
       int lo = 0, hi = batch;  // largest b in [0, batch) with cu[b] <= row
       while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (cu_seq_lens[mid] <= row) lo = mid; else hi = mid;
+        if ((in_lds ? cu_l[mid] : cu_seq_lens[mid]) <= row) lo = mid; else hi = mid;
       }
-      const int64_t tok = row - cu_seq_lens[lo];
-      if (tok >= 0 && row < cu_seq_lens[lo + 1] && tok / block_size < table_stride) {
+      const int64_t first = in_lds ? cu_l[lo] : cu_seq_lens[lo], next = in_lds ? cu_l[lo + 1] : cu_seq_lens[lo + 1];
+      const int64_t tok = row - first;
+      if (tok >= 0 && row < next && tok / block_size < table_stride) {
         const int page = block_table[lo * table_stride + tok / block_size];
         if (page >= 0 && page < num_blocks) src = static_cast<int64_t>(page) * block_size + tok % block_size;
       }
@@ -201,15 +212,38 @@ __global__ __launch_bounds__(256) void gather_paged_rows_kernel(const char* cach
   }
   __syncthreads();
   const int pieces = row_bytes / VB;
-  for (int i = threadIdx.x; i < 32 * pieces; i += 256) {
-    const int r = i / pieces, c = i - r * pieces;
-    const int64_t src = src_row[r];
-    if (src < 0) continue;
-    const char* from = cache + src * row_bytes + static_cast<int64_t>(c) * VB;
-    char* to = out + (row0 + r) * row_bytes + static_cast<int64_t>(c) * VB;
-    if constexpr (VB == 16) *reinterpret_cast<u32x4*>(to) = *reinterpret_cast<const u32x4*>(from);
-    else if constexpr (VB == 4) *reinterpret_cast<uint32_t*>(to) = *reinterpret_cast<const uint32_t*>(from);
-    else *to = *from;
+  const int n = 32 * pieces;
+  if constexpr (VB == 16) {
+    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * 256) {
+      u32x4 v[4];
+      char* to[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * 256;
+        to[u] = nullptr;
+        if (i < n) {
+          const int r = i / pieces, c = i - r * pieces;
+          const int64_t src = src_row[r];
+          if (src >= 0) {
+            v[u] = ldg16_stream(cache + src * row_bytes + static_cast<int64_t>(c) * 16);
+            to[u] = out + (row0 + r) * row_bytes + static_cast<int64_t>(c) * 16;
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (to[u] != nullptr) *reinterpret_cast<u32x4*>(to[u]) = v[u];
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += 256) {
+      const int r = i / pieces, c = i - r * pieces;
+      const int64_t src = src_row[r];
+      if (src < 0) continue;
+      const char* from = cache + src * row_bytes + static_cast<int64_t>(c) * VB;
+      char* to = out + (row0 + r) * row_bytes + static_cast<int64_t>(c) * VB;
+      if constexpr (VB == 4) *reinterpret_cast<uint32_t*>(to) = *reinterpret_cast<const uint32_t*>(from);
+      else *to = *from;
+    }
   }
 }
 

@@ -197,18 +197,6 @@ __device__ __forceinline__ Pools make_pools(const GqaArgs& a, int64_t total, int
   return p;
 }
 
-// A plan (ints): word 0 the signature of what it was made for | from kPlanPrefixOff the item prefix [batch + 1] and
-// the cut between the pools | from kPlanChunksOff 64 page-table entries per group of workers (the chunk of the
-// context's table that holds the page of the group's first stage; the tail repeats the context's last page) | from
-// kPlanLensOff the context lengths [batch] the plan was made with: the merge kernel of a planned call compares them
-// with the lengths of the call, so that a plan that was not made again for a new step is reported
-// (kStatusPlanMismatch) instead of followed silently.
-constexpr int kPlanPrefixOff = 64;
-constexpr int kPlanChunksOff = kPlanPrefixOff + (kMaxBatch + 2 + 63) / 64 * 64;
-constexpr int kPlanMaxTeams = 4096;
-constexpr int kPlanLensOff = kPlanChunksOff + kPlanMaxTeams * kWave;
-constexpr size_t kPlanBytes = (static_cast<size_t>(kPlanLensOff) + static_cast<size_t>(kMaxBatch)) * 4;
-
 // The range [cur, end) of the flat list that group of workers `team` of `n_teams` takes; false: none.
 __device__ __forceinline__ bool team_range(const GqaArgs& a, int64_t total, int64_t cut, int64_t team, int64_t n_teams,
                                            int64_t& cur, int64_t& end) {

@@ -92,6 +92,9 @@ struct MlaArgs {
   // mla_decode_w4_kernel merges the pieces of a context itself and no merge kernel follows (see the fold at the end of
   // that kernel): ws_written holds one counter per (team, head block of 128), zero between launches, that counts the
   // pieces of the context that starts in that team's range as they reach memory
+  // mla_decode_w4_kernel: the plan of the step (mla_plan_kernel: kPlan*), or null
+  const int* plan;
+  int plan_sig;     // what the plan must have been made for, checked against the plan's own first word
   int fold;
   unsigned* ws_written;
   int* ws_status;   // status flags of the workspace (kStatus*), only ever OR-ed into
@@ -1425,32 +1428,27 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
 constexpr int kW4Threads = 256;
 
 // ---- pieces of a context that spans several teams, and their merge (tiles of mla_decode_w4_kernel) ----------------
-// Where the pieces of a context lie: teams t_first .. t_last of the launch, whose ranges are stepped without a
-// division (team_start(t) = t * q + floor(t * r / n) with total = q * n + r).
+// mla_decode_w4_kernel deals the list to min(teams, items) teams, so that no range in the middle of the list is empty:
+// the pieces of a context lie with consecutive teams, one piece each.
+__device__ __forceinline__ int64_t w4_teams_in_use(const MlaArgs& a, int64_t total) {
+  return total < a.n_teams ? total : static_cast<int64_t>(a.n_teams);
+}
 struct MlaPieces {
-  int t_first, t_last;
-  int slot_first;   // slot of the first team's piece (1 when its range starts in front of the context, with an earlier run)
-  int count;        // pieces: teams of t_first .. t_last whose range is not empty
-  int64_t q, r, acc, n;
+  int t_first, t_last;   // teams t_first .. t_last hold the context's pieces
+  int slot_first;        // slot of the first team's piece (1 when its range starts in front of the context, with an earlier run)
+  int count;             // t_last - t_first + 1
 };
 // front, stop: the context's share of what the schedule divides, [prefix[b], prefix[b + 1]): run_cost, then its tiles.
 // False: the context has no tiles.
 __device__ __forceinline__ bool mla_locate_pieces(const MlaArgs& a, int64_t front, int64_t stop, int64_t total, MlaPieces& p) {
   const int64_t first = front + a.run_cost, last = stop - 1;
   if (last < first) return false;
-  const int64_t n = a.n_teams;
-  p.n = n;
+  const int64_t n = w4_teams_in_use(a, total);
   p.t_first = team_of(first, total, n);
   p.t_last = team_of(last, total, n);
-  const bool fits32 = total * n < (1LL << 31);
-  p.q = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(total) / static_cast<uint32_t>(n)) : total / n;
-  p.r = total - p.q * n;
-  p.acc = fits32 ? static_cast<int64_t>(static_cast<uint32_t>(p.t_first) * static_cast<uint32_t>(p.r) % static_cast<uint32_t>(n))
-                 : (static_cast<int64_t>(p.t_first) * p.r) % n;
   // (a range that starts in front of the context holds the last tile of an earlier one)
   p.slot_first = team_start(p.t_first, total, n) < front ? 1 : 0;
-  // with fewer items than teams a range holds one item or none, and the teams that hold first .. last are one per tile
-  p.count = total >= n ? p.t_last - p.t_first + 1 : static_cast<int>(last - first + 1);
+  p.count = p.t_last - p.t_first + 1;
   return true;
 }
 
@@ -1461,33 +1459,57 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t coherent_window(const void* ba
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
 }
 constexpr int kAuxDeviceScope = 16;   // the cache-policy bit that the compiler sets for device-scope atomics (sc1)
-__device__ __forceinline__ u32x4 coherent_load16(__amdgpu_buffer_rsrc_t w, u32 byte_off) {
-  return __builtin_amdgcn_raw_buffer_load_b128(w, byte_off, 0, kAuxDeviceScope);
-}
 __device__ __forceinline__ void coherent_store16(__amdgpu_buffer_rsrc_t w, u32 byte_off, u32x4 v) {
   __builtin_amdgcn_raw_buffer_store_b128(v, w, byte_off, 0, kAuxDeviceScope);
+}
+
+// One piece joins the running merge of a head's rows: maximum M, weight sum W, O[db] = the lane's four values of dim block
+// db.  Piece by piece in the order of the teams, with every product and sum spelled out, so that the result is the same
+// bits whoever merges and however the loads are grouped.  x: the lane's 16-bit values of the piece, pairs of dim blocks.
+template <typename QT>
+__device__ __forceinline__ void mla_merge_piece(float lse, bool on, const u32x4 (&x)[4], float& M, float& W, f32x4 (&O)[8]) {
+  const float l = on ? lse : kNegBig;
+  const float m_new = fmaxf(M, l);
+  const float keep = fast_exp2(M - m_new);
+  const float e = on ? fast_exp2(l - m_new) : 0.0f;
+  W = __builtin_fmaf(W, keep, e);
+#pragma unroll
+  for (int dp = 0; dp < 4; ++dp) {
+    const u32x4 v = x[dp];
+    const float lo[4] = {QT::lo(v[0]), QT::hi(v[0]), QT::lo(v[1]), QT::hi(v[1])};
+    const float hi[4] = {QT::lo(v[2]), QT::hi(v[2]), QT::lo(v[3]), QT::hi(v[3])};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      O[2 * dp][r] = __builtin_fmaf(e, lo[r], O[2 * dp][r] * keep);
+      O[2 * dp + 1][r] = __builtin_fmaf(e, hi[r], O[2 * dp + 1][r] * keep);
+    }
+  }
+  M = m_new;
+}
+// The rows of head hd of context b from a finished merge: dims 128 w + 16 db + 4 g .. + 3 (out points at the first).
+template <typename QT>
+__device__ __forceinline__ void mla_merge_store(const MlaArgs& a, char* out, int b, int hd, bool lse_lane, float M, float W,
+                                                const f32x4 (&O)[8]) {
+  const float inv = 1.0f / W;
+#pragma unroll
+  for (int db = 0; db < 8; ++db)
+    *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{QT::pack(O[db][0] * inv, O[db][1] * inv), QT::pack(O[db][2] * inv, O[db][3] * inv)};
+  if (a.lse != nullptr && lse_lane) a.lse[b * a.n_heads + hd] = (M + fast_log2(W)) * kLn2;
 }
 
 // The merge of one (block of 16 heads hb, context b) by 256 threads laid out like the four wavefronts that wrote the
 // tiles: wavefront w, lane (head c16, k-group g) owns dims 128 w + 16 db + 4 g .. + 3 of head 16 hb + c16 for the
 // eight dim blocks db, and every load instruction reads 1 KB in one piece.  Four teams at a time, their 32 loads per
-// lane issued together.  FOLD: called by the workgroup of mla_decode_w4_kernel that holds the context's first piece:
-// that piece (team p.t_first) is read from the workgroup's LDS (tiles at own_tiles, LSEs at own_lse[head of the 128]),
-// the others, which other workgroups of the same launch wrote, with coherent loads.  Same arithmetic in the same
-// order either way: the result does not depend on who merges.
-template <typename QT, bool FOLD>
-__device__ __forceinline__ void mla_merge_tiles(const MlaArgs& a, const MlaPieces& p, int hb, int b, int w, int lane,
-                                                const char* own_tiles, const float* own_lse) {
+// lane issued together.
+template <typename QT>
+__device__ __forceinline__ void mla_merge_tiles(const MlaArgs& a, const MlaPieces& p, int hb, int b, int w, int lane) {
   const int H = a.n_heads;
   const int c16 = lane & 15, g = lane >> 4;
   const int hd = hb * 16 + c16;
   const bool head_ok = hd < H;
   char* out = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + w * 128 + 4 * g) * 2;
   const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 2;
-  const u32 tile_off = static_cast<u32>((hb * 4 + w) * 4096 + lane * 16);
-  const char* tiles = reinterpret_cast<const char*>(a.ws_out) + tile_off;
-  const __amdgpu_buffer_rsrc_t window = coherent_window(a.ws_out);
-  int64_t acc = p.acc;
+  const char* tiles = reinterpret_cast<const char*>(a.ws_out) + (hb * 4 + w) * 4096 + lane * 16;
   float M = kNegBig, W = 0.0f;
   f32x4 O[8];
 #pragma unroll
@@ -1499,54 +1521,120 @@ __device__ __forceinline__ void mla_merge_tiles(const MlaArgs& a, const MlaPiece
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int t = tb + k;
-      acc += p.r;
-      const int64_t step = p.q + (acc >= p.n ? 1 : 0);
-      acc -= acc >= p.n ? p.n : 0;
-      // with fewer tiles than teams some ranges in between are empty and own no partial
-      on[k] = t <= p.t_last && step > 0 && head_ok;
+      on[k] = t <= p.t_last && head_ok;
       const int64_t slot = static_cast<int64_t>(t) * 2 + (t == p.t_first ? p.slot_first : 0);
-      if (FOLD && t == p.t_first) {
-        lse[k] = on[k] ? own_lse[hd & (kHeadsPerWg16 - 1)] : kNegBig;
+      lse[k] = on[k] ? a.ws_lse[slot * H + hd] : kNegBig;
 #pragma unroll
-        for (int dp = 0; dp < 4; ++dp)
-          x[k][dp] = on[k] ? *(lds_cu32x4*)(own_tiles + ((hb & 7) * 4 + w) * 4096 + lane * 16 + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
-      } else if (FOLD) {
-        lse[k] = on[k] ? __hip_atomic_load(a.ws_lse + slot * H + hd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : kNegBig;
-#pragma unroll
-        for (int dp = 0; dp < 4; ++dp)
-          x[k][dp] = on[k] ? coherent_load16(window, tile_off + static_cast<u32>(slot * slot_bytes) + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
-      } else {
-        lse[k] = on[k] ? a.ws_lse[slot * H + hd] : kNegBig;
-#pragma unroll
-        for (int dp = 0; dp < 4; ++dp)
-          x[k][dp] = on[k] ? *reinterpret_cast<const u32x4*>(tiles + slot * slot_bytes + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
-      }
+      for (int dp = 0; dp < 4; ++dp)
+        x[k][dp] = on[k] ? *reinterpret_cast<const u32x4*>(tiles + slot * slot_bytes + dp * 1024) : u32x4{0u, 0u, 0u, 0u};
     }
-    const float m_new = fmaxf(fmaxf(M, fmaxf(lse[0], lse[1])), fmaxf(lse[2], lse[3]));
-    const float keep = fast_exp2(M - m_new);
-    W *= keep;
 #pragma unroll
-    for (int db = 0; db < 8; ++db) O[db] *= keep;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const float e = on[k] ? fast_exp2(lse[k] - m_new) : 0.0f;
-      W += e;
-#pragma unroll
-      for (int dp = 0; dp < 4; ++dp) {
-        const u32x4 v = x[k][dp];
-        O[2 * dp] += e * f32x4{QT::lo(v[0]), QT::hi(v[0]), QT::lo(v[1]), QT::hi(v[1])};
-        O[2 * dp + 1] += e * f32x4{QT::lo(v[2]), QT::hi(v[2]), QT::lo(v[3]), QT::hi(v[3])};
-      }
-    }
-    M = m_new;
+    for (int k = 0; k < 4; ++k)
+      if (on[k]) mla_merge_piece<QT>(lse[k], true, x[k], M, W, O);   // (on[k] is uniform over the head's lanes)
   }
   if (!head_ok) return;
-  const float inv = 1.0f / W;
-#pragma unroll
-  for (int db = 0; db < 8; ++db)
-    *reinterpret_cast<u32x2*>(out + db * 32) = u32x2{QT::pack(O[db][0] * inv, O[db][1] * inv), QT::pack(O[db][2] * inv, O[db][3] * inv)};
-  if (a.lse != nullptr && w == 0 && g == 0) a.lse[b * H + hd] = (M + fast_log2(W)) * kLn2;
+  mla_merge_store<QT>(a, out, b, hd, w == 0 && g == 0, M, W, O);
 }
+
+// The same merge inside mla_decode_w4_kernel, by one wavefront (w of the workgroup's four, each on its own: no barrier in
+// here) for the head blocks hb_first, hb_first + hb_step, ... < n16 of the workgroup's 128 heads (block 0 = heads
+// 16 hb_base ..).  The pieces were written by other workgroups of the same launch, so they are fetched at the scope of
+// the whole GPU, and straight into LDS (no register is in flight): a stream of (head block, piece) units of 4 KB per
+// wavefront, four units to a step, the next step's 20 loads in flight while the current one is merged.  region: this
+// wavefront's 2 x 17 KB of LDS (4 units + their LSEs, twice).
+template <typename QT>
+__device__ __forceinline__ void mla_fold_stream(const MlaArgs& a, const MlaPieces& p, int b,
+                                                int hb_base, int hb_first, int hb_step, int n16, int w, int lane,
+                                                const char* region, u32 region_lds) {
+  const int P = p.count;
+  const int m = hb_first < n16 ? (n16 - hb_first + hb_step - 1) / hb_step : 0;
+  if (m <= 0 || P <= 0) return;
+  const int H = a.n_heads;
+  const int U = m * P, S = (U + 3) >> 2;
+  constexpr int kBuf = 4 * 4096 + 1024;
+  const int64_t slot_bytes = static_cast<int64_t>(a.slot_heads) * kDL * 2;
+  const int c16 = lane & 15, g = lane >> 4;
+  // (the lane's offsets, opaque to the compiler: it would otherwise carry them from the top of the kernel)
+  u32 lane16 = static_cast<u32>(lane) * 16u;
+  asm volatile("" : "+v"(lane16));
+  auto slot_of = [&](int i) -> int64_t { return static_cast<int64_t>(p.t_first + i) * 2 + (i == 0 ? p.slot_first : 0); };
+  auto uniform64 = [](uint64_t x) -> uint64_t {
+    const u32 lo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(x)));
+    const u32 hi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(x >> 32)));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+  };
+  int iu = 0, ihh = 0, ii = 0;   // the unit the next load belongs to: index, head block of the share, piece
+  auto issue = [&](int s) {
+    const u32 buf = region_lds + static_cast<u32>(s & 1) * kBuf;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      // (past the last unit: that one's again, so that every step is 20 loads and the waits below can count)
+      const int hb = hb_base + hb_first + ihh * hb_step;
+      const int64_t slot = slot_of(ii);
+      const uint64_t src = uniform64(reinterpret_cast<uint64_t>(a.ws_out) + static_cast<uint64_t>(slot * slot_bytes) +
+                                     static_cast<uint64_t>((hb * 4 + w) * 4096));
+      const u32 dst = __builtin_amdgcn_readfirstlane(buf + k * 4096);
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                   "global_load_lds_dwordx4 %1, %2 sc1\n\t"
+                   "global_load_lds_dwordx4 %1, %2 offset:1024 sc1\n\t"
+                   "global_load_lds_dwordx4 %1, %2 offset:2048 sc1\n\t"
+                   "global_load_lds_dwordx4 %1, %2 offset:3072 sc1" ::"s"(dst), "v"(lane16), "s"(src) : "memory");
+      const int hd = min(hb * 16 + c16, H - 1);
+      const uint64_t lsrc = uniform64(reinterpret_cast<uint64_t>(a.ws_lse) + static_cast<uint64_t>(slot * H) * 4);
+      const u32 ldst = __builtin_amdgcn_readfirstlane(buf + 4 * 4096 + k * 256);
+      const u32 loff = static_cast<u32>(hd) * 4u;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2 sc1" ::"s"(ldst), "v"(loff), "s"(lsrc) : "memory");
+      if (iu + 1 < U) {
+        ++iu;
+        if (++ii == P) {
+          ii = 0;
+          ++ihh;
+        }
+      }
+    }
+  };
+  float M = kNegBig, W = 0.0f;
+  f32x4 O[8];
+  int hh = 0, i = 0;
+  issue(0);
+  for (int s = 0; s < S; ++s) {
+    if (s + 1 < S) {
+      issue(s + 1);
+      asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    const char* buf = region + (s & 1) * kBuf;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (4 * s + k < U) {
+        if (i == 0) {
+          M = kNegBig;
+          W = 0.0f;
+#pragma unroll
+          for (int db = 0; db < 8; ++db) O[db] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        const int hb = hb_base + hb_first + hh * hb_step;
+        const int hd = hb * 16 + c16;
+        const float lse = *(const lds_f32*)(buf + 4 * 4096 + k * 256 + lane * 4);
+        u32x4 x[4];
+#pragma unroll
+        for (int dp = 0; dp < 4; ++dp) x[dp] = *(lds_cu32x4*)(buf + k * 4096 + dp * 1024 + lane * 16);
+        mla_merge_piece<QT>(lse, true, x, M, W, O);
+        if (++i == P) {
+          i = 0;
+          ++hh;
+          if (hd < H) {
+            char* out = a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + w * 128 + 4 * g) * 2;
+            mla_merge_store<QT>(a, out, b, hd, w == 0 && g == 0, M, W, O);
+          }
+        }
+      }
+    }
+    asm volatile("" ::: "memory");   // (the reads of this step's buffer stay in front of the loads that refill it)
+  }
+}
+
 // Output rows of a context without tokens: zeros, LSE -inf (same layout of the 256 threads).
 template <typename QT>
 __device__ __forceinline__ void mla_write_empty(const MlaArgs& a, int hb, int b, int w, int lane) {
@@ -1574,12 +1662,85 @@ constexpr int kW4FacOff = kW4QEnd > kDsPOff + 2 * 8 * 1024 ? kW4QEnd : kDsPOff +
 constexpr int kW4FlagOff = kW4FacOff + 2 * kHeadsPerWg16 * 4;
 constexpr int kW4PageOff = kW4FlagOff + 16;
 constexpr int kW4PrefixOff = kW4PageOff + 2 * kWave * 4;
-constexpr int kW4LdsBytes = kW4PrefixOff + (kMaxBatchMla + 1) * 4;
+constexpr int kW4LdsBytes = kW4PrefixOff + (kMaxBatchMla + 1) * 4 + kMaxBatchMla * 4;   // prefix, then (with a plan) the lengths
 constexpr int kW4Loads = 9;   // loads a wavefront sends for a sub-tile: 8 rows and their rope parts
+// The fold at the end of a run (mla_fold_stream): every wavefront streams pieces through 2 x 17 KB of the LDS that the
+// ring and the Q rows no longer need; the second counter of a context (how many merging workgroups have seen the first
+// one full) lies kFoldSeenOff words behind the first.
+constexpr int kFoldRegion = 2 * (4 * 4096 + 1024);
+constexpr int kFoldSeenOff = kWsMaxWorkers / 2;
+static_assert(4 * kFoldRegion <= kW4FacOff, "the fold's LDS lies in front of the factors, flags and the prefix");
 static_assert(kW4LdsBytes <= 160 * 1024, "LDS of a CU");
 #ifndef XLLM_W4_AHEAD
 #define XLLM_W4_AHEAD 3
 #endif
+
+// The prefix over the batch of what mla_decode_w4_kernel's schedule divides (sub-tiles, and run_cost more at the front of
+// every context that holds tokens) into prefix[0 .. batch] (LDS), by 256 threads; tmp: 4 words of LDS.
+__device__ __forceinline__ void w4_item_prefix(const MlaArgs& a, int* prefix, int* tmp) {
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  const int per = (a.batch + kW4Threads - 1) / kW4Threads;
+  const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
+  int local = 0;
+  auto span_of = [&](int len) { return len > 0 ? (len + kW4Item - 1) / kW4Item + a.run_cost : 0; };
+  for (int b = lo; b < hi; ++b) local += span_of(a.seq_lens[b]);
+  // (scan inside the wavefront, then over the wavefronts' totals)
+  int incl = local;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int t = __shfl_up(incl, d, kWave);
+    if (lane >= d) incl += t;
+  }
+  if (lane == kWave - 1) tmp[wave] = incl;
+  __syncthreads();
+  if (lo < hi) {
+    int excl = incl - local;
+    for (int w = 0; w < wave; ++w) excl += tmp[w];
+    if (per == 1) {
+      prefix[lo] = excl;
+      excl += local;
+    } else {
+      for (int b = lo; b < hi; ++b) {
+        prefix[b] = excl;
+        excl += span_of(a.seq_lens[b]);
+      }
+    }
+    if (hi == a.batch) prefix[a.batch] = excl;
+  }
+  __syncthreads();
+}
+
+// The plan of a step for mla_decode_w4_kernel (MlaArgs::plan): the prefix, the lengths it was made with, and for every
+// team the 64 page-table entries around the page of its range's first tokens, found as the decode kernel finds them.
+// One wavefront per team.
+__global__ __launch_bounds__(kW4Threads) void mla_plan_kernel(MlaArgs a, int* plan) {
+  extern __shared__ __align__(16) char smem[];
+  int* tmp = reinterpret_cast<int*>(smem);
+  int* prefix = tmp + 8;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid >> 6;
+  w4_item_prefix(a, prefix, tmp);
+  if (blockIdx.x == 0) {
+    for (int i = tid; i <= a.batch; i += kW4Threads) plan[kPlanPrefixOff + i] = prefix[i];
+    for (int i = tid; i < a.batch; i += kW4Threads) plan[kPlanLensOff + i] = a.seq_lens[i];
+    if (tid == 0) plan[0] = a.plan_sig;
+  }
+  const int64_t total = prefix[a.batch];
+  const int64_t n_use = w4_teams_in_use(a, total);
+  const int team = blockIdx.x * (kW4Threads / kWave) + wave;
+  if (team >= n_use) return;
+  const int64_t cur = team_start(team, total, n_use);
+  int lo = 0, hi = a.batch;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (prefix[mid] <= cur) lo = mid; else hi = mid;
+  }
+  const int L = a.seq_lens[lo];
+  const int tile0 = max(0, static_cast<int>(cur - prefix[lo]) - a.run_cost);
+  const int ck = ((tile0 * kW4Item) >> a.bs_shift) >> 6;
+  const int n_pages = max(1, (L + a.block_size - 1) >> a.bs_shift);
+  const int32_t* pages = a.block_table + static_cast<int64_t>(lo) * a.table_stride;
+  plan[kPlanChunksOff + team * kWave + lane] = pages[max(0, min(ck * kWave + lane, n_pages - 1))];
+}
 
 template <typename QT>
 __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
@@ -1624,49 +1785,61 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
   const int head0 = hb128 * kHeadsPerWg16;
   const int n16 = min(8, (H - head0 + 15) >> 4);       // 16-head blocks of this workgroup that hold heads
 
-  // ---- prefix over the batch of what the schedule divides: tiles, and run_cost more at the front of every context
-  // (every workgroup computes it; no extra launch)
-  {
-    const int per = (a.batch + kW4Threads - 1) / kW4Threads;
-    const int lo = min(a.batch, tid * per), hi = min(a.batch, lo + per);
-    int local = 0;
-    auto span_of = [&](int len) { return len > 0 ? (len + kW4Item - 1) / kW4Item + a.run_cost : 0; };
-    for (int b = lo; b < hi; ++b) local += span_of(a.seq_lens[b]);
-    // (scan inside the wavefront, then over the wavefronts' totals)
-    int incl = local;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const int t = __shfl_up(incl, d, kWave);
-      if (lane >= d) incl += t;
-    }
-    if (lane == kWave - 1) tmp[wave] = incl;
-    __syncthreads();
-    if (lo < hi) {
-      int excl = incl - local;
-      for (int w = 0; w < wave; ++w) excl += tmp[w];
-      if (per == 1) {
-        prefix[lo] = excl;
-        excl += local;
-      } else {
-        for (int b = lo; b < hi; ++b) {
-          prefix[b] = excl;
-          excl += span_of(a.seq_lens[b]);
-        }
-      }
-      if (hi == a.batch) prefix[a.batch] = excl;
-    }
-    __syncthreads();
-  }
-  const int64_t total = prefix[a.batch];
-  if (blockIdx.x == 0)
-    for (int i = tid; i <= a.batch; i += kW4Threads) a.ws_prefix[i] = prefix[i];
-  if (total == 0) return;
-  int64_t cur = team_start(team, total, a.n_teams);
-  const int64_t end = team_start(team + 1, total, a.n_teams);
-  bool first_run = true;
-
   const u32 lds_base = static_cast<u32>(reinterpret_cast<uintptr_t>(smem));
   const u32 page_lds = __builtin_amdgcn_readfirstlane(lds_base + kW4PageOff);
+  // ---- prefix over the batch of what the schedule divides: tiles, and run_cost more at the front of every context.
+  // Every workgroup computes it (no extra launch), or takes it from the step's plan: then one trip to memory brings
+  // the prefix, the lengths and the page-table entries of the team's first tokens together, where a launch on its own
+  // makes three in a row (lengths -> prefix -> the length and the pages of the context its range starts in).
+  const bool planned = a.plan != nullptr;
+  int* lens_l = prefix + kMaxBatchMla + 1;   // (with a plan) the context lengths
+  if (planned) {
+    if (wave == 0) {   // (into both chunk buffers: which one the first run reads depends on where it starts)
+      dma4(a.plan + kPlanChunksOff + team * kWave + lane, page_lds);
+      dma4(a.plan + kPlanChunksOff + team * kWave + lane, page_lds + kWave * 4);
+    }
+    const int sig = a.plan[0];
+    for (int i = tid; i <= a.batch; i += kW4Threads) prefix[i] = a.plan[kPlanPrefixOff + i];
+    bool stale = false;
+    for (int i = tid; i < a.batch; i += kW4Threads) {
+      const int len = a.plan[kPlanLensOff + i];
+      lens_l[i] = len;
+      if (blockIdx.x == 0) stale |= len != a.seq_lens[i];   // (one workgroup checks for all)
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (sig != a.plan_sig) {   // a plan for another shape: nothing is written
+      if (tid == 0) atomicOr(a.ws_status, kStatusPlanMismatch);
+      return;
+    }
+    // a plan made with other lengths (the step before, say): the launch follows it, and its output is invalid
+    if (stale) atomicOr(a.ws_status, kStatusPlanMismatch);
+    __syncthreads();
+  } else {
+    w4_item_prefix(a, prefix, tmp);
+  }
+  const int64_t total = prefix[a.batch];
+  if (blockIdx.x == 0 && !planned)   // (the merge kernel of a planned call reads the plan's)
+    for (int i = tid; i <= a.batch; i += kW4Threads) a.ws_prefix[i] = prefix[i];
+  if (a.fold != 0) {   // no merge kernel follows: the rows of sequences without tokens, which no run ever meets
+    for (int b = team; b < a.batch; b += a.n_teams)
+      if (prefix[b + 1] == prefix[b])
+        for (int hb = 0; hb < n16; ++hb) mla_write_empty<QT>(a, hb128 * 8 + hb, b, wave, lane);
+  }
+  if (total == 0) return;
+  // (min(teams, items) teams take part: no range in the middle of the list is empty)
+  const int64_t n_use = w4_teams_in_use(a, total);
+  if (team >= n_use) return;
+  int64_t cur = team_start(team, total, n_use);
+  const int64_t end = team_start(team + 1, total, n_use);
+  bool first_run = true;
+  bool plan_chunk = planned;   // the chunk buffers hold the plan's entries for the range's first tokens
+  // fold: the counter of a piece this workgroup has stored and not yet announced (its stores are known to have landed
+  // after the next run's wait for its Q rows, or at the end of the kernel), or -1
+  int pending = -1;
+  auto announce = [&](int counter) {
+    __hip_atomic_fetch_add(a.ws_written + counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+
   // per-lane constants of the operand reads (byte offsets inside a sub-tile), as in mla_decode16_kernel
   const int k_row0 = c16 * kRow16 + ((g ^ ((c16 >> 2) & 1)) * 16);
   const int v_row0 = (4 * g + (c16 >> 2)) * kRow16 + ((((c16 & 3) >> 1) ^ (g & 1)) * 16) + (c16 & 1) * 8 + wave * (8 * 32);
@@ -1691,9 +1864,12 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     const int run_tiles = max(0, static_cast<int>(piece_end - prefix[b]) - a.run_cost) - tile0;
     const bool complete = tile0 == 0 && run_tiles == n_tiles_seq;
     cur = piece_end;
-    if (run_tiles <= 0) continue;   // (the range ends inside the allowance in front of this context's tiles)
+    if (run_tiles <= 0) {   // (the range ends inside the allowance in front of this context's tiles)
+      plan_chunk = false;
+      continue;
+    }
     const int32_t* pages = a.block_table + static_cast<int64_t>(b) * a.table_stride;
-    const int L = __builtin_amdgcn_readfirstlane(a.seq_lens[b]);
+    const int L = __builtin_amdgcn_readfirstlane(planned ? lens_l[b] : a.seq_lens[b]);
     const int t_begin = tile0 * kW4Item;
     const int t_end = min(L, (tile0 + run_tiles) * kW4Item);
     const int n_sub = (t_end - t_begin + kSubTok - 1) / kSubTok;
@@ -1706,9 +1882,10 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     __syncthreads();  // the previous run no longer reads the ring, the chunks, the factors or the flags
     // the page-table chunks of the run's first sub-tiles travel while the Q rows do
     if (wave == 0) {
-      issue_chunk(ck_cur);
+      if (!plan_chunk) issue_chunk(ck_cur);   // (the plan brought the first run's chunk in with the prefix)
       if ((ck_cur + 1) * kWave < n_pages) issue_chunk(ck_cur + 1);
     }
+    plan_chunk = false;
     // (the lane's coordinates, opaque to the compiler: what it can compute from them before the first run it keeps in
     // scratch memory through the loop, and a reload here waits for the chunk loads just issued)
     const int lane_p = lane_again();
@@ -2089,6 +2266,10 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
                                  : *reinterpret_cast<const u32x4*>(qrope + (kk - kDL / 32) * 64);
     }
     __syncthreads();   // (the ring is free for the first sub-tiles)
+    if (pending >= 0) {   // every wavefront's stores of the piece before have landed (the wait above), and all are past it
+      if (tid == 0) announce(pending);
+      pending = -1;
+    }
     W4_PTICK(4)   // Q and chunks landed, barrier
     for (int sub = 0; sub < kDsRing && sub < n_sub; ++sub) issue_sub(sub);
     W4_PTICK(5)   // three sub-tiles issued
@@ -2175,8 +2356,17 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     }
 
     // ---- end of the run: the owners publish 1 / sum per head, every wavefront writes its dims of every head
+#ifdef XLLM_DS_TIMING
+    unsigned long long fold_t[5] = {static_cast<unsigned long long>(wall_clock64()), 0, 0, 0, 0};
+#define W4_FOLD_MARK(i) fold_t[i] = static_cast<unsigned long long>(wall_clock64());
+#else
+#define W4_FOLD_MARK(i)
+#endif
     const float lsum0 = quad_rows_sum(l[0]), lsum1 = quad_rows_sum(l[1]);
-    const int64_t ps_base = (static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * H;
+    const int64_t slot_id = static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1);
+    const int64_t ps_base = slot_id * H;
+    // fold: a piece goes to memory at the scope of the whole GPU, for the workgroups of this launch that merge it
+    const bool shared = a.fold != 0 && !complete;
     // The lane's coordinates once more, opaque to the compiler.  Address arithmetic of the epilogue that can be done
     // before the loop is done there otherwise, and carried through the loop in scratch memory: every reload then waits
     // for all the stores issued before it (one counter covers loads and stores), a round trip to memory per row.
@@ -2193,30 +2383,34 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
         if (hd < H) {
           const float lse2 = m[j] + fast_log2(j == 0 ? lsum0 : lsum1);
           if (complete && a.lse != nullptr) a.lse[b * H + hd] = lse2 * kLn2;
-          if (!complete) a.ws_lse[ps_base + hd] = lse2;
+          if (!complete && !shared) a.ws_lse[ps_base + hd] = lse2;
+          if (shared) __hip_atomic_store(a.ws_lse + ps_base + hd, lse2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
     }
     __syncthreads();
-    // Output rows of a whole context go out head by head (COMPLETE).  Partial rows go out as the tiles they are in the
+    // Output rows of a whole context go out head by head (MODE 0).  Partial rows go out as the tiles they are in the
     // registers, [16-head block][wavefront][pair of dim blocks][lane][2 x 4 values]: every store instruction then
-    // writes 1 KB in one piece.  Head by head it writes sixteen pieces of 64 bytes, and the burst of partial rows that
-    // ends a launch takes twice as long to issue (it is bound by the number of write requests, not by their bytes).
-    // A partial row is normalised (a convex combination of V rows, like the output), so it is stored in the output's
-    // own 16-bit type: half the stores here, half the bytes for the merge kernel, whose time is reading them; the
-    // LSEs stay fp32.
+    // writes 1 KB in one piece (MODE 1; MODE 2: the same at the scope of the whole GPU).  Head by head it writes sixteen
+    // pieces of 64 bytes, and the burst of partial rows that ends a launch takes twice as long to issue (it is bound by
+    // the number of write requests, not by their bytes).  A partial row is normalised (a convex combination of V rows,
+    // like the output), so it is stored in the output's own 16-bit type: half the stores here, half the bytes for the
+    // merge, whose time is reading them; the LSEs stay fp32.
 #define XLLM_W4_OUT(DB, HB, R0, R1, R2, R3)                                                          \
   {                                                                                                  \
     f32x4 t;                                                                                         \
     XLLM_W4_GET(R0, R1, R2, R3, t);                                                                  \
     t *= inv;                                                                                        \
     const u32x2 w = {QT::pack(t[0], t[1]), QT::pack(t[2], t[3])};                                    \
-    if (COMPLETE) {                                                                                  \
+    if (MODE == 0) {                                                                                 \
       *reinterpret_cast<u32x2*>(dst + DB * 32) = w;                                                  \
     } else if ((DB & 1) == 0) {                                                                      \
       held = w;                                                                                      \
-    } else {                                                                                         \
+    } else if (MODE == 1) {                                                                          \
       *reinterpret_cast<u32x4*>(dst + (DB >> 1) * 1024) = u32x4{held[0], held[1], w[0], w[1]};       \
+    } else {                                                                                         \
+      coherent_store16(window, voff + (HB * 4 + wave) * 4096 + (DB >> 1) * 1024,                     \
+                       u32x4{held[0], held[1], w[0], w[1]});                                         \
     }                                                                                                \
   }
 #define XLLM_W4_OUT_ROW(HB, ROW)                                                                     \
@@ -2225,8 +2419,8 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     if (HB < n16 && hd < H) {                                                                        \
       const float inv = fac[HB * 16 + c16e];                                                         \
       u32x2 held = {0u, 0u};                                                                         \
-      char* dst = COMPLETE ? a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + wave * 128 + 4 * ge) * 2 \
-                           : tiles + (HB * 4 + wave) * 4096;                                         \
+      char* dst = MODE == 0 ? a.out + ((static_cast<int64_t>(b) * H + hd) * kDL + wave * 128 + 4 * ge) * 2 \
+                            : tiles + (HB * 4 + wave) * 4096;                                        \
       ROW(XLLM_W4_OUT)                                                                               \
     }                                                                                                \
   }
@@ -2240,20 +2434,86 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
   XLLM_W4_OUT_ROW(6, XLLM_W4_ROW6)                                                                   \
   XLLM_W4_OUT_ROW(7, XLLM_W4_ROW7)
     // (16-head blocks of this workgroup's 128 heads: block hb128 * 8 + HB of the slot)
-    char* tiles = reinterpret_cast<char*>(a.ws_out) +
-                  ((static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1)) * a.slot_heads + head0) * (kDL * 2) + ln * 16;
+    const int64_t tile_base = (slot_id * a.slot_heads + head0) * (kDL * 2) + ln * 16;
+    char* tiles = reinterpret_cast<char*>(a.ws_out) + tile_base;
+    const u32 voff = static_cast<u32>(tile_base);
+    const __amdgpu_buffer_rsrc_t window = coherent_window(a.ws_out);
     if (complete) {
-      constexpr bool COMPLETE = true;
+      constexpr int MODE = 0;
+      XLLM_W4_OUT_ROWS
+    } else if (!shared) {
+      constexpr int MODE = 1;
       XLLM_W4_OUT_ROWS
     } else {
-      constexpr bool COMPLETE = false;
+      constexpr int MODE = 2;
       XLLM_W4_OUT_ROWS
     }
 #undef XLLM_W4_OUT_ROWS
 #undef XLLM_W4_OUT_ROW
 #undef XLLM_W4_OUT
+    if (shared) {
+      // The pieces of the context lie with teams t_first .. t_last; one counter per context (kept with its first team)
+      // counts them as they reach memory.  The workgroups whose piece ends their range (all but the one that holds the
+      // context's end, which has another run to go) wait for the count and merge the head blocks between them, team j
+      // of the nf taking blocks j, j + nf, ...: nobody waits before it has announced everything it wrote itself, so
+      // every wait ends.  The last of the nf to have seen the full count clears it for the next launch.
+      MlaPieces pc;
+      mla_locate_pieces(a, prefix[b], prefix[b + 1], total, pc);
+      const int counter = pc.t_first * a.n_hb + hb128;
+      const int nf = pc.t_last - pc.t_first;
+      const int jf = team - pc.t_first;
+      if (team == pc.t_last) {
+        pending = counter;   // announced once its stores have landed: after the next run's wait, or at the kernel's end
+      } else {
+        W4_FOLD_MARK(1)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();   // every wavefront's stores have landed
+        W4_FOLD_MARK(2)
+        if (tid == 0) {
+          if (pending >= 0) announce(pending);
+          announce(counter);
+          const unsigned need = static_cast<unsigned>(pc.count);
+          bool ok = a.wait_spins > 0;
+          for (int spins = a.wait_spins; ok; --spins) {
+            if (__hip_atomic_load(a.ws_written + counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= need) break;
+            if (spins <= 1) ok = false;
+            __builtin_amdgcn_s_sleep(16);
+          }
+          if (!ok) atomicOr(a.ws_status, kStatusWaitGaveUp);
+          flags[3] = ok ? 1 : 0;
+        }
+        pending = -1;
+        __syncthreads();
+        W4_FOLD_MARK(3)
+        if (flags[3] != 0) {
+          mla_fold_stream<QT>(a, pc, b, hb128 * 8, jf, nf, n16, wave, lane_again(),
+                              smem + wave * kFoldRegion, lds_base + wave * kFoldRegion);
+          __syncthreads();   // every wavefront has read what it needs of the pieces
+          if (tid == 0) {
+            const unsigned seen = atomicInc(a.ws_written + kFoldSeenOff + counter, static_cast<unsigned>(nf - 1));
+            if (seen == static_cast<unsigned>(nf - 1))
+              __hip_atomic_store(a.ws_written + counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+        W4_FOLD_MARK(4)
+#ifdef XLLM_DS_TIMING
+        if (lane == 0) {   // (measurement build only) the fold's time stamps, behind the phase sums
+          unsigned long long* ft = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H) +
+                                   4096 * 12 + (blockIdx.x * 4 + wave) * 8;
+          for (int i = 0; i < 5; ++i) ft[i] = fold_t[i];
+          ft[5] = static_cast<unsigned long long>(pc.count);
+        }
+#endif
+      }
+    }
+#undef W4_FOLD_MARK
     first_run = false;
     W4_TICK(7)   // run epilogue
+  }
+  if (pending >= 0) {   // a piece stored by this workgroup's last run that it does not merge itself
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) announce(pending);
   }
 #ifdef XLLM_DS_TIMING
   // (measurement build only) per-phase cycle sums of every wavefront of every workgroup, behind the partials
@@ -2262,7 +2522,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
                               (blockIdx.x * 4 + wave) * 12;
     for (int i = 0; i < 8; ++i) dst[i] = tm[i];
     dst[8] = __builtin_readcyclecounter() - t_entry;
-    dst[9] = static_cast<unsigned long long>(end - team_start(team, total, a.n_teams));
+    dst[9] = static_cast<unsigned long long>(end - team_start(team, total, n_use));
     dst[10] = w_entry;
     dst[11] = wall_clock64();
   }
@@ -2354,13 +2614,14 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)   // (measurement build only) when the merge kernel starts
     reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * a.n_heads)[2048 * 10] = wall_clock64();
 #endif
+  if (a.plan != nullptr && a.plan[0] != a.plan_sig) return;   // the decode kernel wrote nothing and raised the flag
   MlaPieces p;
   if (!mla_locate_pieces(a, a.ws_prefix[b], a.ws_prefix[b + 1], a.ws_prefix[a.batch], p)) {  // empty sequence
     mla_write_empty<QT>(a, hb, b, w, lane);
     return;
   }
   if (p.t_first == p.t_last) return;  // one team saw the whole context and wrote the output
-  mla_merge_tiles<QT, false>(a, p, hb, b, w, lane, nullptr, nullptr);
+  mla_merge_tiles<QT>(a, p, hb, b, w, lane);
 }
 
 // Teams: as many as there are CUs for the team size, a multiple of 8 (one per XCD slot).
@@ -2388,9 +2649,94 @@ int mla_kernel_knob() {
   return v;
 }
 
+// Whether mla_decode_w4_kernel merges the pieces of a context itself instead of leaving them to mla_merge_tiles_kernel.
+// Off by default.  The merge moves the same bytes either way (every piece, 128 KB of 16-bit rows per workgroup and run,
+// written once and read once: 41 MB on 64 contexts over 256 workgroups), and that is what it costs: the merging
+// workgroups of one launch read them at 4.8 TB/s between them (6.3 us per workgroup after 2.3 us of waiting for the
+// count), whether they ask for them at the scope of the GPU or of the workgroup, where the second launch takes 11.5 us:
+// decode + merge 182.6 us as two launches, 183.5 us as one, a step 189 us against 191 us.  What the one launch adds is
+// a wait of workgroups on each other, which needs all of them resident at once; a device that runs fewer at a time
+// reports XLLM_MI355_ESTALLED instead of an output.  "1" in XLLM_MI355_MLA_FOLD, read once per process, or set_mla_fold
+// (test hook) turn it on.  Same bits either way.
+std::atomic<int> g_mla_fold{-1};
+bool mla_fold_enabled() {
+  int v = g_mla_fold.load(std::memory_order_relaxed);
+  if (v < 0) {
+    const char* e = getenv("XLLM_MI355_MLA_FOLD");  // tuning knob
+    v = e != nullptr && e[0] == '1' ? 1 : 0;
+    g_mla_fold.store(v, std::memory_order_relaxed);
+  }
+  return v != 0;
+}
+
 }  // namespace
 
+void set_mla_fold(int on) { g_mla_fold.store(on < 0 ? -1 : (on != 0 ? 1 : 0), std::memory_order_relaxed); }
 void set_mla_kernel_knob(int first_letter) { g_mla_knob.store(first_letter < 0 ? 0 : first_letter, std::memory_order_relaxed); }
+
+namespace {
+// Tiles that the schedule of mla_decode_w4_kernel charges for the start of a run (tuning knob XLLM_MI355_MLA_RUN_COST).
+int w4_run_cost() {
+  static const int run_cost = [] {
+    const char* e = getenv("XLLM_MI355_MLA_RUN_COST");
+    const int v = e ? atoi(e) : -1;
+    return v >= 0 && v <= 64 ? v : 3;
+  }();
+  return run_cost * (kTile / kW4Item);
+}
+// Whether mla_decode_w4_kernel serves a call (more than 64 heads, block size a power of two >= 16, no knob that asks
+// for another kernel); a plan is made for it and for no other.
+bool w4_serves(int64_t n_heads, int64_t block_size) {
+  const int knob = mla_kernel_knob();
+  const bool pairs = knob == 'p' || block_size < 16 || (block_size & (block_size - 1)) != 0;
+  const bool by_dims = !pairs && knob != 'h' && n_heads > 64;
+#ifdef XLLM_MLA_DEFAULT_NARROW
+  return by_dims && knob == 'w';
+#else
+  return by_dims && knob != 'n';
+#endif
+}
+// What a plan is made for: everything that the schedule depends on besides the lengths themselves.
+int mla_plan_signature(const MlaArgs& a) {
+  uint32_t h = 2166136261u;
+  const int v[] = {a.batch, a.n_heads, a.n_teams, a.n_hb, a.run_cost, a.bs_shift, 0x6d6c61};
+  for (int x : v) h = (h ^ static_cast<uint32_t>(x)) * 16777619u;
+  return static_cast<int>(h | 1u);
+}
+}  // namespace
+
+int paged_decode_mla_plan(void* plan, size_t plan_bytes, const PageAddressing& addr, int64_t batch, int64_t n_heads,
+                          int64_t block_size, hipStream_t stream) {
+  if (batch == 0) return XLLM_MI355_OK;
+  if (plan == nullptr || (reinterpret_cast<uintptr_t>(plan) & 255) != 0 || plan_bytes < kPlanBytes)
+    return XLLM_MI355_EWORKSPACE;
+  if (addr.block_table == nullptr || addr.seq_lens == nullptr || addr.table_stride <= 0) return XLLM_MI355_EINVAL;
+  if (batch < 0 || n_heads <= 0 || n_heads > 65535 || block_size <= 0) return XLLM_MI355_EINVAL;
+  // Shapes that mla_decode_w4_kernel does not serve, and batches decoded in slices, take no plan: the planned entry
+  // point decodes them like the plain one.
+  const int64_t max_batch = kDsMaxBatch < kMaxBatchMla ? kDsMaxBatch : kMaxBatchMla;
+  if (!w4_serves(n_heads, block_size) || batch > max_batch) return XLLM_MI355_OK;
+  MlaArgs a = {};
+  a.block_table = addr.block_table;
+  a.seq_lens = addr.seq_lens;
+  a.table_stride = addr.table_stride;
+  a.batch = static_cast<int>(batch);
+  a.n_heads = static_cast<int>(n_heads);
+  a.n_hb = static_cast<int>((n_heads + kHeadsPerWg16 - 1) / kHeadsPerWg16);
+  a.n_teams = mla_teams(a.n_hb);
+  if (a.n_teams > kPlanMaxTeams) return XLLM_MI355_OK;
+  a.block_size = static_cast<int>(block_size);
+  a.bs_shift = -1;
+  for (int s = 0; s < 31; ++s)
+    if ((1LL << s) == block_size) a.bs_shift = s;
+  a.run_cost = w4_run_cost();
+  a.plan_sig = mla_plan_signature(a);
+  const int per_wg = kW4Threads / kWave;
+  const dim3 grid(static_cast<unsigned>((a.n_teams + per_wg - 1) / per_wg));
+  const size_t smem = (static_cast<size_t>(a.batch) + 1 + 8) * 4;
+  launch_timed(mla_plan_kernel, grid, dim3(kW4Threads), smem, stream, a, static_cast<int*>(plan));
+  return static_cast<int>(hipGetLastError());
+}
 
 size_t mla_workspace_bytes(int64_t batch, int64_t n_heads, int64_t max_seq_len) {
   (void)batch;  // (the layout does not depend on it)
@@ -2425,6 +2771,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
   if (workspace == nullptr || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
       workspace_bytes < mla_workspace_bytes(batch, n_heads, 0))
     return XLLM_MI355_EWORKSPACE;
+  if (addr.plan != nullptr && (reinterpret_cast<uintptr_t>(addr.plan) & 255) != 0) return XLLM_MI355_EWORKSPACE;
 
   // "pairs" selects the kernel with the per-tile exchange (also taken for block sizes below 16 or not a power
   // of two: the other kernels look pages up per group of 4 tokens inside chunks of 64 pages)
@@ -2493,12 +2840,18 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
 #else
     const bool w4 = !pairs && by_dims && knob != 'n';
 #endif
-    static const int run_cost = [] {
-      const char* e = getenv("XLLM_MI355_MLA_RUN_COST");  // tuning knob: tiles charged for the start of a run
-      const int v = e ? atoi(e) : -1;
-      return v >= 0 && v <= 64 ? v : 3;
-    }();
-    a.run_cost = w4 ? run_cost * (kTile / kW4Item) : 0;
+    a.run_cost = w4 ? w4_run_cost() : 0;
+    // the step's plan: for the kernel it was made for, and not for a batch decoded in slices
+    a.plan = w4 && batch <= max_batch && a.n_teams <= kPlanMaxTeams ? static_cast<const int*>(addr.plan) : nullptr;
+    if (a.plan != nullptr) {
+      a.plan_sig = mla_plan_signature(a);
+      a.ws_prefix = const_cast<int*>(a.plan) + kPlanPrefixOff;   // (what the merge kernel reads)
+    }
+    // (two counters per context, kept with its first team, in the header of the workspace)
+    a.fold = w4 && a.n_teams * a.n_hb <= kFoldSeenOff && mla_fold_enabled() ? 1 : 0;
+    a.ws_status = static_cast<int*>(workspace);
+    a.ws_written = reinterpret_cast<unsigned*>(static_cast<char*>(workspace) + kWsCountersOff);
+    a.wait_spins = wait_spin_limit();
 
     const dim3 grid(static_cast<unsigned>(a.n_teams * a.n_hb));
     if (pairs) {
@@ -2520,7 +2873,9 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     int rc = static_cast<int>(hipGetLastError());
     if (rc != 0) return rc;
     const dim3 mgrid(static_cast<unsigned>(n_heads), static_cast<unsigned>(nb));
-    if (w4) {   // (its partial rows are tiles)
+    if (a.fold != 0) {   // the decode kernel merged
+      profile_skip();
+    } else if (w4) {   // (its partial rows are tiles)
       const dim3 tgrid(static_cast<unsigned>(a.slot_heads / 16), static_cast<unsigned>(nb));
       if (f16) launch_timed(mla_merge_tiles_kernel<FP16>, tgrid, dim3(256), 0, stream, a);
       else launch_timed(mla_merge_tiles_kernel<BF16>, tgrid, dim3(256), 0, stream, a);

@@ -27,17 +27,20 @@ struct ReshapeArgs {
   int64_t k_stride_bytes;
   int64_t v_stride_bytes;
   int64_t n_slots;     // num_blocks * block_size
+  int64_t n_tokens;
   int row_elems;       // Hkv * D
   int head_dim;
   int n_vec;           // 16-byte input vectors per row
 };
 
-// IN: 0 bf16, 1 fp16, 2 fp32.  FP8: quantise, else byte copy.
-template <int IN, bool FP8>
+// IN: 0 bf16, 1 fp16, 2 fp32.  FP8: quantise, else byte copy.  TPW: tokens per workgroup row.  With one token a
+// thread has 16 bytes in flight, which is right for the few tokens of a decode step (the launch is then a chain of two
+// trips to memory, slot id then row) and leaves a prefill chunk bound by latency: from kStreamTokens tokens on a
+// thread takes the same vector of TPW = 4 consecutive tokens, asks for all four before it stores the first, and the
+// rows come and go with non-temporal accesses (a row is read once and written once).
+constexpr int kStreamTokens = 2048;
+template <int IN, bool FP8, int TPW>
 __global__ __launch_bounds__(256) void reshape_vec_kernel(ReshapeArgs a) {
-  const int64_t t = blockIdx.x;
-  const int64_t slot = a.slots[t];
-  if (slot < 0 || slot >= a.n_slots) return;
   int w = blockIdx.y * 256 + threadIdx.x;
   const bool is_v = w >= a.n_vec;
   if (is_v) w -= a.n_vec;
@@ -46,32 +49,50 @@ __global__ __launch_bounds__(256) void reshape_vec_kernel(ReshapeArgs a) {
   char* cache = is_v ? a.v_cache : a.k_cache;
   if (src == nullptr || cache == nullptr) return;
   const int64_t stride = is_v ? a.v_stride_bytes : a.k_stride_bytes;
-  const u32x4 x = ldg16(src + t * stride + static_cast<int64_t>(w) * 16);
-  if constexpr (!FP8) {
-    constexpr int ES = IN == 2 ? 4 : 2;
-    stg16(cache + slot * (static_cast<int64_t>(a.row_elems) * ES) + static_cast<int64_t>(w) * 16, x);
-  } else {
-    constexpr int EPV = IN == 2 ? 4 : 8;  // elements per 16-byte input vector
-    const int e0 = w * EPV;
-    const float scale = (is_v ? a.v_scale : a.k_scale)[e0 / a.head_dim];
-    const float inv_scale = 1.0f / scale;
-    char* dst = cache + slot * static_cast<int64_t>(a.row_elems) + e0;
-    if constexpr (IN == 2) {
-      u32 c = 0;
+  int64_t slot[TPW];
+  u32x4 x[TPW];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) c |= fp8_quantize(as_f32(x[i]), inv_scale) << (8 * i);
-      *reinterpret_cast<u32*>(dst) = c;
+  for (int u = 0; u < TPW; ++u) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * TPW + u;
+    slot[u] = t < a.n_tokens ? a.slots[t] : -1;
+    if (slot[u] >= a.n_slots) slot[u] = -1;
+  }
+#pragma unroll
+  for (int u = 0; u < TPW; ++u) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * TPW + u;
+    const char* p = src + t * stride + static_cast<int64_t>(w) * 16;
+    if (slot[u] >= 0) x[u] = TPW > 1 ? ldg16_stream(p) : ldg16(p);
+  }
+  constexpr int EPV = IN == 2 ? 4 : 8;  // elements per 16-byte input vector
+  float inv_scale = 0.0f;
+  if constexpr (FP8) inv_scale = 1.0f / (is_v ? a.v_scale : a.k_scale)[w * EPV / a.head_dim];
+#pragma unroll
+  for (int u = 0; u < TPW; ++u) {
+    if (slot[u] < 0) continue;
+    if constexpr (!FP8) {
+      constexpr int ES = IN == 2 ? 4 : 2;
+      char* dst = cache + slot[u] * (static_cast<int64_t>(a.row_elems) * ES) + static_cast<int64_t>(w) * 16;
+      if constexpr (TPW > 1) __builtin_nontemporal_store(x[u], reinterpret_cast<u32x4*>(dst));
+      else stg16(dst, x[u]);
     } else {
-      u32x2 c = {0u, 0u};
+      char* dst = cache + slot[u] * static_cast<int64_t>(a.row_elems) + w * EPV;
+      if constexpr (IN == 2) {
+        u32 c = 0;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float lo, hi;
-        if constexpr (IN == 0) { lo = BF16::lo(x[i]); hi = BF16::hi(x[i]); }
-        else { lo = FP16::lo(x[i]); hi = FP16::hi(x[i]); }
-        const u32 two = fp8_quantize(lo, inv_scale) | (fp8_quantize(hi, inv_scale) << 8);
-        c[i >> 1] |= two << (16 * (i & 1));
+        for (int i = 0; i < 4; ++i) c |= fp8_quantize(as_f32(x[u][i]), inv_scale) << (8 * i);
+        *reinterpret_cast<u32*>(dst) = c;
+      } else {
+        u32x2 c = {0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float lo, hi;
+          if constexpr (IN == 0) { lo = BF16::lo(x[u][i]); hi = BF16::hi(x[u][i]); }
+          else { lo = FP16::lo(x[u][i]); hi = FP16::hi(x[u][i]); }
+          const u32 two = fp8_quantize(lo, inv_scale) | (fp8_quantize(hi, inv_scale) << 8);
+          c[i >> 1] |= two << (16 * (i & 1));
+        }
+        *reinterpret_cast<u32x2*>(dst) = c;
       }
-      *reinterpret_cast<u32x2*>(dst) = c;
     }
   }
 }
@@ -181,9 +202,16 @@ template <int IN>
 int launch_reshape(const ReshapeArgs& a, int64_t n_tokens, bool fp8, bool vec_ok, hipStream_t stream) {
   if (vec_ok) {
     const int n_work = a.n_vec * (a.value != nullptr ? 2 : 1);
-    dim3 grid(static_cast<unsigned>(n_tokens), static_cast<unsigned>((n_work + 255) / 256));
-    if (fp8) reshape_vec_kernel<IN, true><<<grid, 256, 0, stream>>>(a);
-    else reshape_vec_kernel<IN, false><<<grid, 256, 0, stream>>>(a);
+    const unsigned gy = static_cast<unsigned>((n_work + 255) / 256);
+    if (n_tokens >= kStreamTokens) {
+      dim3 grid(static_cast<unsigned>((n_tokens + 3) / 4), gy);
+      if (fp8) reshape_vec_kernel<IN, true, 4><<<grid, 256, 0, stream>>>(a);
+      else reshape_vec_kernel<IN, false, 4><<<grid, 256, 0, stream>>>(a);
+    } else {
+      dim3 grid(static_cast<unsigned>(n_tokens), gy);
+      if (fp8) reshape_vec_kernel<IN, true, 1><<<grid, 256, 0, stream>>>(a);
+      else reshape_vec_kernel<IN, false, 1><<<grid, 256, 0, stream>>>(a);
+    }
   } else {
     dim3 grid(static_cast<unsigned>(n_tokens));
     if (fp8) reshape_elem_kernel<IN, true><<<grid, 256, 0, stream>>>(a);
@@ -226,6 +254,7 @@ int reshape_and_cache(const void* key, const void* value, void* k_cache, void* v
   a.k_stride_bytes = k_token_stride * es;
   a.v_stride_bytes = v_token_stride * es;
   a.n_slots = num_blocks * block_size;
+  a.n_tokens = n_tokens;
   a.row_elems = static_cast<int>(row);
   a.head_dim = static_cast<int>(head_dim);
   a.n_vec = static_cast<int>(row * es / 16);

@@ -549,7 +549,45 @@ void check_dense_decode_inputs(const DenseDecodeParams& p) {
 }
 }  // namespace
 
-torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {
+namespace {
+torch::Tensor dense_decode_impl(DenseDecodeParams& p, const torch::Tensor* plan, torch::Tensor* lse_out);
+}
+torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) { return dense_decode_impl(p, nullptr, lse_out); }
+torch::Tensor dense_decode(DenseDecodeParams& p, const torch::Tensor& tile_scheduler_metadata, torch::Tensor* lse_out) {
+  TORCH_CHECK(tile_scheduler_metadata.defined() && tile_scheduler_metadata.is_cuda() &&
+                  tile_scheduler_metadata.is_contiguous() && tile_scheduler_metadata.scalar_type() == torch::kUInt8 &&
+                  static_cast<size_t>(tile_scheduler_metadata.numel()) >= xllm_mi355_paged_decode_plan_bytes(),
+              "flash_mla: tile_scheduler_metadata must be the buffer of get_mla_decoding_metadata");
+  return dense_decode_impl(p, &tile_scheduler_metadata, lse_out);
+}
+
+std::vector<torch::Tensor> get_mla_decoding_metadata(const torch::Tensor& seqlens_k, const torch::Tensor& block_table,
+                                                     int64_t num_heads_per_head_k, int64_t num_heads_k,
+                                                     int64_t block_size, const std::optional<torch::Tensor>& reuse) {
+  TORCH_CHECK(num_heads_k == 1, "flash_mla: the latent cache has one KV head");
+  TORCH_CHECK(seqlens_k.is_cuda() && seqlens_k.dim() == 1 && seqlens_k.scalar_type() == torch::kInt32 &&
+                  seqlens_k.is_contiguous(),
+              "flash_mla: seqlens_k must be contiguous int32 [B] on the device");
+  TORCH_CHECK(block_table.is_cuda() && block_table.dim() == 2 && block_table.scalar_type() == torch::kInt32 &&
+                  block_table.stride(1) == 1 && block_table.size(0) == seqlens_k.numel(),
+              "flash_mla: block_table must be int32 [B, max_blocks] with unit column stride");
+  const int64_t nbytes = static_cast<int64_t>(xllm_mi355_paged_decode_plan_bytes());
+  torch::Tensor buf = reuse.has_value() && reuse->defined()
+                          ? *reuse
+                          : torch::empty({nbytes}, seqlens_k.options().dtype(torch::kUInt8));
+  TORCH_CHECK(buf.is_cuda() && buf.is_contiguous() && buf.scalar_type() == torch::kUInt8 && buf.numel() >= nbytes,
+              "flash_mla: the plan must be a contiguous uint8 device buffer of xllm_mi355_paged_decode_plan_bytes() bytes");
+  const int rc = xllm_mi355_paged_decode_mla_plan(buf.data_ptr(), static_cast<size_t>(buf.numel()),
+                                                  block_table.data_ptr<int32_t>(), block_table.stride(0),
+                                                  seqlens_k.data_ptr<int32_t>(), seqlens_k.numel(), num_heads_per_head_k,
+                                                  block_size, current_stream(seqlens_k));
+  check_rc(rc, "xllm_mi355_paged_decode_mla_plan");
+  // (the reference returns {tile_scheduler_metadata, num_splits}; the splits live in the same buffer here)
+  return {buf, torch::empty({0}, seqlens_k.options())};
+}
+
+namespace {
+torch::Tensor dense_decode_impl(DenseDecodeParams& p, const torch::Tensor* plan, torch::Tensor* lse_out) {
   TORCH_CHECK(p.kind == DenseDecodeKind::kQNopePe,
               "flash_mla: only DenseDecodeKind::kQNopePe (BF16/FP16 split-q) is supported");
   check_dense_decode_inputs(p);
@@ -583,15 +621,25 @@ torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) {
   const int64_t max_seq_len = table.size(1) * p.k_cache.size(1);
   const size_t nbytes = xllm_mi355_paged_decode_mla_workspace_bytes(rows, heads, max_seq_len);
   torch::Tensor ws = mi355::decode_workspace(q_nope.device(), nbytes);
-  const int rc = xllm_mi355_paged_decode_mla(
-      q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), lse, table.data_ptr<int32_t>(),
-      table.stride(0), seqlens.data_ptr<int32_t>(), rows, heads, q_nope.size(3), q_pe.size(3), p.k_cache.size(1),
-      p.k_cache.size(0), max_seq_len, p.softmax_scale, ws.data_ptr(), static_cast<size_t>(ws.numel()),
-      dtype_code(q_nope), current_stream(q_nope));
-  check_rc(rc, "xllm_mi355_paged_decode_mla");
+  if (plan != nullptr && !per_token) {   // (a causal multi-token step rewrites lengths and table per token: no plan)
+    const int rc = xllm_mi355_paged_decode_mla_planned(
+        plan->data_ptr(), static_cast<size_t>(plan->numel()), q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(),
+        out.data_ptr(), lse, table.data_ptr<int32_t>(), table.stride(0), seqlens.data_ptr<int32_t>(), rows, heads,
+        q_nope.size(3), q_pe.size(3), p.k_cache.size(1), p.k_cache.size(0), max_seq_len, p.softmax_scale, ws.data_ptr(),
+        static_cast<size_t>(ws.numel()), dtype_code(q_nope), current_stream(q_nope));
+    check_rc(rc, "xllm_mi355_paged_decode_mla_planned");
+  } else {
+    const int rc = xllm_mi355_paged_decode_mla(
+        q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), lse, table.data_ptr<int32_t>(),
+        table.stride(0), seqlens.data_ptr<int32_t>(), rows, heads, q_nope.size(3), q_pe.size(3), p.k_cache.size(1),
+        p.k_cache.size(0), max_seq_len, p.softmax_scale, ws.data_ptr(), static_cast<size_t>(ws.numel()),
+        dtype_code(q_nope), current_stream(q_nope));
+    check_rc(rc, "xllm_mi355_paged_decode_mla");
+  }
   if (lse_out != nullptr) *lse_out = lse_rows.view({B, Sq, H}).transpose(1, 2).contiguous();  // [B, H, S_q]
   return out;
 }
+}  // namespace
 
 torch::Tensor dense_decode(DenseDecodeParams& params) { return dense_decode(params, nullptr); }
 
@@ -810,7 +858,8 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> op_attention_layer_forwa
 std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nope, torch::Tensor q_pe,
                                                              torch::Tensor k_cache, torch::Tensor seqlens_k,
                                                              torch::Tensor block_table, int64_t head_size_v,
-                                                             double softmax_scale, bool is_causal) {
+                                                             double softmax_scale, bool is_causal,
+                                                             std::optional<torch::Tensor> plan) {
   xllm::kernel::dcu::flash_mla::DenseDecodeParams p;
   p.q_nope = q_nope;
   p.q_pe = q_pe;
@@ -822,8 +871,15 @@ std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nop
   p.is_causal = is_causal;
   p.kind = xllm::kernel::dcu::flash_mla::DenseDecodeKind::kQNopePe;
   torch::Tensor lse;
-  torch::Tensor out = xllm::kernel::dcu::flash_mla::dense_decode(p, &lse);
+  torch::Tensor out = plan.has_value() && plan->defined() ? xllm::kernel::dcu::flash_mla::dense_decode(p, *plan, &lse)
+                                                          : xllm::kernel::dcu::flash_mla::dense_decode(p, &lse);
   return {out, lse};
+}
+
+torch::Tensor op_mla_decoding_metadata(torch::Tensor seqlens_k, torch::Tensor block_table, int64_t num_heads_per_head_k,
+                                       int64_t block_size, std::optional<torch::Tensor> plan) {
+  return xllm::kernel::dcu::flash_mla::get_mla_decoding_metadata(seqlens_k, block_table, num_heads_per_head_k, 1,
+                                                                 block_size, plan)[0];
 }
 
 torch::Tensor op_paged_forward(torch::Tensor query, torch::Tensor output, torch::Tensor k_cache, torch::Tensor v_cache,
@@ -928,7 +984,9 @@ TORCH_LIBRARY(xllm_ops, m) {
   m.def("update_decode_plan(Tensor block_table, Tensor seq_lens, int num_qo_heads, int num_kv_heads, int head_dim, "
         "int block_size, int window_left, bool fp8_cache, Tensor(a!)? plan=None) -> Tensor");
   m.def("mla_dense_decode(Tensor q_nope, Tensor q_pe, Tensor k_cache, Tensor seqlens_k, Tensor block_table, "
-        "int head_size_v, float softmax_scale, bool is_causal=False) -> (Tensor, Tensor)");
+        "int head_size_v, float softmax_scale, bool is_causal=False, Tensor? plan=None) -> (Tensor, Tensor)");
+  m.def("mla_decoding_metadata(Tensor seqlens_k, Tensor block_table, int num_heads_per_head_k, int block_size, "
+        "Tensor(a!)? plan=None) -> Tensor");
   m.def("lse_combine(Tensor(a!) output, Tensor shared_o, Tensor shared_lse, Tensor unshared_o, Tensor unshared_lse) -> Tensor");
   m.def("attention_layer_forward(Tensor query, Tensor key, Tensor value, Tensor(a!) k_cache, Tensor(b!) v_cache, "
         "Tensor? k_cache_scale, Tensor? v_cache_scale, Tensor slot_mapping, Tensor block_table, Tensor kv_seq_lens, "
@@ -960,6 +1018,7 @@ TORCH_LIBRARY_IMPL(xllm_ops, CUDA, m) {
   m.impl("batch_decode", &op_batch_decode);
   m.impl("update_decode_plan", &op_update_decode_plan);
   m.impl("mla_dense_decode", &op_mla_dense_decode);
+  m.impl("mla_decoding_metadata", &op_mla_decoding_metadata);
   m.impl("lse_combine", &op_lse_combine);
   m.impl("attention_layer_forward", &op_attention_layer_forward);
   m.impl("merge_dcp_attention_shards", &op_merge);

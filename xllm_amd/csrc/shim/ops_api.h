@@ -22,6 +22,7 @@
 
 #include <memory>
 #include <optional>
+#include <vector>
 #include <string>
 #include <tuple>
 
@@ -193,6 +194,18 @@ torch::Tensor dense_decode(DenseDecodeParams& params);
 // The same with the natural-log LSE, [B, H_q, S_q] fp32 (the layout of MluMlaDecodeLseTest,
 // tests/core/layers/mlu/dcp_attention_merge_test.cpp:127-143, for S_q = 1: [B, H, 1]).
 torch::Tensor dense_decode(DenseDecodeParams& params, torch::Tensor* lse);
+// The plan of an MLA decode step, made once per step for the dense_decode calls of all layers: the role of
+// get_mla_decoding_metadata_dense_fp8, which the reference's adapter calls apart from the decode
+// (flash_mla_adapter.cpp:125-130: seqlens_k, num_heads_per_head_k = S_q * H_q, num_heads_k = 1; it returns
+// {tile_scheduler_metadata, num_splits}), and of the FlashInfer plan made at layer 0
+// (xllm/core/layers/cuda/flashinfer_planinfo.cpp:248-264).  Here the one buffer holds both; `reuse` is a buffer of an
+// earlier step (a captured step must keep its address).
+std::vector<torch::Tensor> get_mla_decoding_metadata(const torch::Tensor& seqlens_k, const torch::Tensor& block_table,
+                                                     int64_t num_heads_per_head_k, int64_t num_heads_k,
+                                                     int64_t block_size,
+                                                     const std::optional<torch::Tensor>& reuse = std::nullopt);
+// dense_decode from that plan (same lengths and table): bit-identical to the call without it.
+torch::Tensor dense_decode(DenseDecodeParams& params, const torch::Tensor& tile_scheduler_metadata, torch::Tensor* lse);
 
 }  // namespace flash_mla
 }  // namespace dcu

@@ -420,11 +420,37 @@ class DenseDecodeParams:
     kind: int = DenseDecodeKind.kQNopePe
 
 
-def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0):
+def get_mla_decoding_metadata(seqlens_k, block_table, num_heads_per_head_k, block_size, plan=None):
+    """The plan of an MLA decode step, made once per step for the dense_decode calls of all layers (metadata=...): the
+    role of get_mla_decoding_metadata_dense_fp8, which the reference's adapter calls apart from the decode
+    (flash_mla_adapter.cpp:125-130), and of the FlashInfer plan made at layer 0 (flashinfer_planinfo.cpp:248-264).
+    num_heads_per_head_k = S_q * H_q as there; takes the step's lengths and block table; returns the plan (a device
+    buffer; pass one back in to reuse it, as a captured step must)."""
+    dev = _require_cuda(seqlens_k, block_table, plan)
+    lib = capi.lib()
+    nbytes = int(lib.xllm_mi355_paged_decode_plan_bytes())
+    if plan is None:
+        plan = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    _check_plan(plan)
+    if seqlens_k.dtype != torch.int32 or not seqlens_k.is_contiguous() or seqlens_k.dim() != 1:
+        raise ValueError("seqlens_k must be contiguous int32 [B]")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.stride(1) != 1 or \
+            block_table.shape[0] != seqlens_k.numel():
+        raise ValueError("block_table must be int32 [B, W] with unit column stride, one row per sequence")
+    rc = lib.xllm_mi355_paged_decode_mla_plan(plan.data_ptr(), plan.numel(), block_table.data_ptr(),
+                                              block_table.stride(0), seqlens_k.data_ptr(), seqlens_k.numel(),
+                                              int(num_heads_per_head_k), int(block_size), _stream(dev))
+    capi.check(rc, "xllm_mi355_paged_decode_mla_plan")
+    return plan
+
+
+def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0, metadata=None):
     """flash_mla::dense_decode (flash_mla_adapter.cpp:104-153): returns [B, S_q, H, head_size_v] (and the natural-log
     lse [B, H, S_q] fp32 when asked).  The same argument checks.  BF16 and FP16.  The S_q query tokens of a sequence
     are folded into the head count as the reference folds them (:119-123); with is_causal and S_q > 1 token j attends
-    to the first seqlens_k - (S_q - 1 - j) tokens and every (sequence, token) becomes a row of its own."""
+    to the first seqlens_k - (S_q - 1 - j) tokens and every (sequence, token) becomes a row of its own.
+    metadata: the step's plan from get_mla_decoding_metadata (same lengths and table), or None: the launch derives its
+    schedule itself.  (A causal multi-token step rewrites lengths and table per token and takes no plan.)"""
     p = params
     if p.kind != DenseDecodeKind.kQNopePe:
         raise ValueError("flash_mla: only DenseDecodeKind::kQNopePe (BF16/FP16 split-q) is supported")
@@ -473,12 +499,21 @@ def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0):
     lib = capi.lib()
     nbytes = lib.xllm_mi355_paged_decode_mla_workspace_bytes(rows, heads, max_seq_len)
     ws = decode_workspace(dev, nbytes)
-    rc = lib.xllm_mi355_paged_decode_mla(
-        q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), _ptr(lse),
-        table.data_ptr(), table.stride(0), seqlens.data_ptr(), rows, heads, d_latent, d_rope, bs, P,
-        max_seq_len, float(p.softmax_scale), ws.data_ptr(), ws.numel(), _dtype_code(q_nope),
-        _stream(dev))
-    capi.check(rc, "xllm_mi355_paged_decode_mla")
+    if metadata is not None and not (p.is_causal and Sq > 1):
+        _check_plan(metadata)
+        rc = lib.xllm_mi355_paged_decode_mla_planned(
+            metadata.data_ptr(), metadata.numel(), q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(),
+            out.data_ptr(), _ptr(lse), table.data_ptr(), table.stride(0), seqlens.data_ptr(), rows, heads, d_latent,
+            d_rope, bs, P, max_seq_len, float(p.softmax_scale), ws.data_ptr(), ws.numel(), _dtype_code(q_nope),
+            _stream(dev))
+        capi.check(rc, "xllm_mi355_paged_decode_mla_planned")
+    else:
+        rc = lib.xllm_mi355_paged_decode_mla(
+            q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), _ptr(lse),
+            table.data_ptr(), table.stride(0), seqlens.data_ptr(), rows, heads, d_latent, d_rope, bs, P,
+            max_seq_len, float(p.softmax_scale), ws.data_ptr(), ws.numel(), _dtype_code(q_nope),
+            _stream(dev))
+        capi.check(rc, "xllm_mi355_paged_decode_mla")
     if return_lse:
         return out, lse.view(B, Sq, H).transpose(1, 2).contiguous()
     return out
