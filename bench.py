@@ -180,7 +180,7 @@ def calibrate(lib, capi, torch, dev):
             "stream_copy_gbs_read_plus_write": copy_gbs, "stream_copy_ms": copy_ms}
 
 
-def neighbours(ops, workloads, torch, dev, steps):
+def neighbours(ops, workloads, torch, dev, steps, lib=None, capi=None):
     """The ops that feed the decode and take its result, at the shapes of the benchmark configurations: every one is
     HBM-bound integer / byte movement or a skinny batched matmul, so each is priced by its algorithmic bytes."""
     import math
@@ -201,8 +201,14 @@ def neighbours(ops, workloads, torch, dev, steps):
     rows = []
 
     def row(op, kernel, shape, us, nbytes):
+        # the yardstick: the library's plain copy kernel moving the same number of bytes (half read, half written),
+        # timed by its own event pair
+        copy_gbs = None
+        if lib is not None:
+            copy_gbs, _ = stream_rate(lib, capi, torch, dev, nbytes // 2, copy=True, reps=20)
         rows.append({"op": op, "kernel": kernel, "shape": shape, "us": us, "algorithmic_bytes": nbytes,
-                     "gbs": nbytes / us / 1e3, "frac_of_hbm_peak": nbytes / us / 1e3 / HBM_PEAK_GBS})
+                     "gbs": nbytes / us / 1e3, "frac_of_hbm_peak": nbytes / us / 1e3 / HBM_PEAK_GBS,
+                     "plain_copy_gbs_same_bytes": copy_gbs})
 
     # reshape_and_cache: a prefill chunk of 8192 tokens into bf16 pages (configuration 2's heads), read + write
     T, nk, D = 8192, 8, 128
@@ -611,7 +617,7 @@ def main():
         print(json.dumps(calibrate(lib, capi, torch, dev)))
         return
     if args.neighbours:
-        print(json.dumps(neighbours(ops, workloads, torch, dev, max(args.steps, 1))))
+        print(json.dumps(neighbours(ops, workloads, torch, dev, max(args.steps, 1), lib, capi)))
         return
     run = lambda name, budget: run_workload(name, args, lib, capi, ops, workloads, torch, dev, budget)
     if args.workload != "all":

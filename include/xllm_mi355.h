@@ -454,7 +454,7 @@ int xllm_mi355_mask_block_table_padding(const int32_t* block_table, int64_t tabl
  *   position_ids   [T] int64
  *   interleave     nonzero: pairs (2i, 2i + 1); zero: pairs (i, i + rotary_dim / 2)
  * head_dim 64, 128 or 256; rotary_dim a multiple of head_dim / 16.  k_cache null: no cache write.
- * qkv, cos_sin_cache and the caches 16-byte aligned.
+ * qkv, the norm weights, cos_sin_cache and the caches 16-byte aligned.
  */
 int xllm_mi355_rope_and_cache(void* qkv, const void* q_weight, const void* k_weight,
                               const void* cos_sin_cache, const int64_t* position_ids,

@@ -399,6 +399,16 @@ def test_step_captured_in_a_graph_follows_new_metadata(device):
         assert_close_to_reference(replayed.view(cfg.batch, cfg.n_q_heads, 512), ref, f"mla graph replay {rep}")
 
 
+def test_step_captured_in_a_graph_with_the_merge_inside_the_decode_kernel(device):
+    # the same capture with the decode kernel merging split contexts itself: the counters it keeps in the workspace
+    # must be back at zero after every replay
+    try:
+        _set_fold(1)
+        test_step_captured_in_a_graph_follows_new_metadata(device)
+    finally:
+        _set_fold(-1)
+
+
 def test_absorbed_attention_layer_captured_in_a_graph(device):
     # The decode branch of the reference's absorbed MLA attention (layers/dcu/deepseek_v2_attention.cpp:221-263,
     # 428-432) as one captured step: q_nope . w_kc, latent store, dense decode, output . w_vc -- replayed over

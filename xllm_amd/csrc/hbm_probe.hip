@@ -55,16 +55,18 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const char* __restrict
 
 __global__ __launch_bounds__(256) void stream_copy_kernel(u32x4* __restrict__ dst,
                                                           const u32x4* __restrict__ src, size_t n_vec) {
+  // every workgroup a contiguous share; a thread asks for eight vectors before it stores the first; bytes that are
+  // read once and written once: non-temporal both ways
   const size_t per = (n_vec + gridDim.x - 1) / gridDim.x;
   const size_t lo = per * blockIdx.x;
   const size_t hi = lo + per < n_vec ? lo + per : n_vec;
   size_t i = lo + threadIdx.x;
-  for (; i + 3 * 256 < hi; i += 4 * 256) {
-    u32x4 v[4];
+  for (; i + 7 * 256 < hi; i += 8 * 256) {
+    u32x4 v[8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = src[i + u * 256];
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * 256);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) dst[i + u * 256] = v[u];
+    for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], dst + i + u * 256);
   }
   for (; i < hi; i += 256) dst[i] = src[i];
 }

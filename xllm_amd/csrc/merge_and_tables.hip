@@ -170,29 +170,31 @@ __global__ __launch_bounds__(256) void expand_varlen_kernel(const int32_t* cu_se
   tok_rows[t] = b;
 }
 
-// One workgroup per 32 output rows.  The first 32 threads find the sequence of their row (cu[b] <= row <
+// One workgroup per kGatherRows output rows.  Their first threads find the sequence of their row (cu[b] <= row <
 // cu[b + 1]) and its source row in the paged cache; then the 256 threads copy the rows in pieces of VB bytes
 // (16 when the row length allows it), consecutive threads taking consecutive pieces of a row.  Rows whose
 // page id is negative or beyond the cache are left untouched, as in the reference kernel (which skips
 // negative ids; an id beyond the cache would be an out-of-bounds read there).
 // The search is a chain of dependent reads, so the row offsets go to LDS first when they fit (one trip to memory for
-// all of them instead of log2(batch) in a row), and a thread asks for four pieces before it stores the first: the
-// launch is a stream of rows that are read once, fetched with non-temporal loads.
+// all of them instead of log2(batch) in a row), and a thread asks for kGatherDepth pieces before it stores the first: the
+// launch is a stream of rows that are read once and written once, with non-temporal loads and stores.
 constexpr int kGatherCuLds = 2048;   // row offsets kept in LDS
+constexpr int kGatherRows = 64;      // output rows per workgroup
+constexpr int kGatherDepth = 8;      // pieces a thread asks for before it stores the first
 template <int VB>
 __global__ __launch_bounds__(256) void gather_paged_rows_kernel(const char* cache, const int32_t* block_table,
                                                                 int64_t table_stride, const int32_t* cu_seq_lens,
                                                                 char* out, int batch, int64_t total_rows,
                                                                 int block_size, int num_blocks, int row_bytes) {
-  __shared__ int64_t src_row[32];
-  __shared__ int cu_l[kGatherCuLds + 1];
-  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * 32;
+  __shared__ int64_t src_row[kGatherRows];
+  extern __shared__ int cu_l[];   // [batch + 1] when batch <= kGatherCuLds
+  const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kGatherRows;
   const bool in_lds = batch <= kGatherCuLds;
   if (in_lds) {
     for (int i = threadIdx.x; i <= batch; i += 256) cu_l[i] = cu_seq_lens[i];
     __syncthreads();
   }
-  if (threadIdx.x < 32) {
+  if (threadIdx.x < kGatherRows) {
     const int64_t row = row0 + threadIdx.x;
     int64_t src = -1;
     if (row < total_rows) {
@@ -212,13 +214,13 @@ __global__ __launch_bounds__(256) void gather_paged_rows_kernel(const char* cach
   }
   __syncthreads();
   const int pieces = row_bytes / VB;
-  const int n = 32 * pieces;
+  const int n = kGatherRows * pieces;
   if constexpr (VB == 16) {
-    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * 256) {
-      u32x4 v[4];
-      char* to[4];
+    for (int i0 = threadIdx.x; i0 < n; i0 += kGatherDepth * 256) {
+      u32x4 v[kGatherDepth];
+      char* to[kGatherDepth];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < kGatherDepth; ++u) {
         const int i = i0 + u * 256;
         to[u] = nullptr;
         if (i < n) {
@@ -231,8 +233,8 @@ __global__ __launch_bounds__(256) void gather_paged_rows_kernel(const char* cach
         }
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (to[u] != nullptr) *reinterpret_cast<u32x4*>(to[u]) = v[u];
+      for (int u = 0; u < kGatherDepth; ++u)
+        if (to[u] != nullptr) __builtin_nontemporal_store(v[u], reinterpret_cast<u32x4*>(to[u]));
     }
   } else {
     for (int i = threadIdx.x; i < n; i += 256) {
@@ -256,9 +258,9 @@ int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t tab
   if (cache == nullptr || block_table == nullptr || cu_seq_lens == nullptr || out == nullptr) return XLLM_MI355_EINVAL;
   if (batch < 0 || total_rows < 0 || batch > 0x7fffffffLL || table_stride <= 0 || block_size <= 0 ||
       block_size > 0x7fffffffLL || num_blocks <= 0 || num_blocks > 0x7fffffffLL || row_bytes <= 0 ||
-      row_bytes > 0x7fffffffLL / 32)
+      row_bytes > 0x7fffffffLL / kGatherRows)
     return XLLM_MI355_EINVAL;
-  const int64_t n_groups = (total_rows + 31) / 32;
+  const int64_t n_groups = (total_rows + kGatherRows - 1) / kGatherRows;
   if (n_groups > 0x7fffffffLL) return XLLM_MI355_ESHAPE;
   const dim3 grid(static_cast<unsigned>(n_groups));
   const char* c = static_cast<const char*>(cache);
@@ -267,12 +269,13 @@ int gather_paged_rows(const void* cache, const int32_t* block_table, int64_t tab
   const bool a4 = ((reinterpret_cast<uintptr_t>(cache) | reinterpret_cast<uintptr_t>(out)) & 3) == 0;
   const int b = static_cast<int>(batch), bs = static_cast<int>(block_size), nb = static_cast<int>(num_blocks),
             rb = static_cast<int>(row_bytes);
+  const size_t lds = batch <= kGatherCuLds ? (static_cast<size_t>(batch) + 1) * 4 : 0;
   if (row_bytes % 16 == 0 && a16)
-    gather_paged_rows_kernel<16><<<grid, 256, 0, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
+    gather_paged_rows_kernel<16><<<grid, 256, lds, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
   else if (row_bytes % 4 == 0 && a4)
-    gather_paged_rows_kernel<4><<<grid, 256, 0, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
+    gather_paged_rows_kernel<4><<<grid, 256, lds, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
   else
-    gather_paged_rows_kernel<1><<<grid, 256, 0, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
+    gather_paged_rows_kernel<1><<<grid, 256, lds, stream>>>(c, block_table, table_stride, cu_seq_lens, o, b, total_rows, bs, nb, rb);
   return static_cast<int>(hipGetLastError());
 }
 
