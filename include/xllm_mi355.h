@@ -153,7 +153,9 @@ int xllm_mi355_decode_status(void* workspace, void* stream);
  *     out[b, h, :] = softmax(sm_scale * q[b, h, :] . K_b[:, h / group, :]^T) . V_b[:, h / group, :]
  * q/out: [B, Hq, D] with token strides in elements; lse: [B, Hq] fp32 natural log or null.
  * k_scale / v_scale: [Hkv] fp32, required iff cache_dtype is fp8 (dequantised value
- * = float(code) * scale[h]).  q_dtype also is the dtype of `out`.
+ * = float(code) * scale[h]).  q_dtype also is the dtype of `out`: XLLM_MI355_BF16 or XLLM_MI355_FP16 over pages of the
+ * same type or fp8 pages, or XLLM_MI355_FP32 over fp32 pages (what reshape_and_cache stores for an fp32 model: a
+ * compatibility path, one workgroup per query head and sequence, no workspace needed).
  * max_seq_len <= 0 means "table_stride * block_size".
  * window_left: sliding window (window_left of xllm/core/kernels/cuda/cuda_ops_api.h:139; sliding_window_ of
  * xllm/core/layers/dcu/flash_attention.cpp:484): the query, at position L - 1, attends to positions
@@ -263,6 +265,39 @@ int xllm_mi355_paged_decode_gqa_planned(const void* plan, size_t plan_bytes,
                                         int64_t max_seq_len, int64_t window_left, float sm_scale,
                                         void* workspace, size_t workspace_bytes,
                                         int q_dtype, int cache_dtype, void* stream);
+
+/*
+ * One decode step of an attention layer in one call: store the step's K / V rows, then attend.  Replaces the pair
+ * that the reference's attention layer issues per layer and step, reshape_paged_cache followed by batch_decode
+ * (xllm/core/layers/dcu/torch_attention.cpp:138-144 then :285-347; xllm/core/layers/cuda/flashinfer_attention.cpp
+ * :136-142 then :329), with the arguments of xllm_mi355_reshape_and_cache (key, value [batch, Hkv, D]
+ * of q's dtype, token strides in elements, slot_mapping [batch]) in front of those of
+ * xllm_mi355_paged_decode_gqa_planned.  plan may be NULL (then plan_bytes is ignored and the call derives its
+ * schedule itself).  Sequence b's slot must be the place of its token seq_lens[b] - 1 in its block table (what the
+ * reference's slot mapping holds on a decode step); negative slots and slots beyond the cache are skipped, and such a
+ * sequence attends to whatever its table holds.  The caches and `out` afterwards hold the same bytes as after
+ * xllm_mi355_reshape_and_cache followed by the decode call.  Where the matrix-core kernel serves the shape (16-bit or
+ * fp8 pages of a power-of-two block size >= 16, head dim 64 / 128, or 256 with 16-bit pages; key / value 16-byte
+ * aligned with strides that are multiples of 8 elements) the rows are written inside the decode launch, by the
+ * worker that attends to the context's last tokens, and the step saves a launch; otherwise the library issues the
+ * two launches itself.  The caches are written: a sequence with seq_lens[b] == 0 has no token to store and stores
+ * none in the one-launch form.
+ */
+int xllm_mi355_write_and_decode_gqa(const void* key, const void* value, const int32_t* slot_mapping,
+                                    int64_t k_token_stride, int64_t v_token_stride,
+                                    const void* plan, size_t plan_bytes,
+                                    const void* q, void* k_cache, void* v_cache, void* out, float* lse,
+                                    const int32_t* block_table, int64_t table_stride,
+                                    const int32_t* seq_lens,
+                                    const int32_t* paged_kv_indptr, const int32_t* paged_kv_indices,
+                                    const int32_t* paged_kv_last_page_len,
+                                    const float* k_scale, const float* v_scale,
+                                    int64_t batch, int64_t n_q_heads, int64_t n_kv_heads,
+                                    int64_t head_dim, int64_t block_size, int64_t num_blocks,
+                                    int64_t q_token_stride, int64_t out_token_stride,
+                                    int64_t max_seq_len, int64_t window_left, float sm_scale,
+                                    void* workspace, size_t workspace_bytes,
+                                    int q_dtype, int cache_dtype, void* stream);
 
 /*
  * Rows of paged sequences gathered into one packed buffer, sequence after sequence.

@@ -59,6 +59,52 @@ def test_fp16_and_other_head_dims(device):
         _check_config(cfg, 100 + D + Hq, device, dtype=dt)
 
 
+def test_fp32_query_over_fp32_pages(device):
+    """What reshape_and_cache stores for an fp32 model can be attended: fp32 query, fp32 pages, fp32 output and LSE,
+    against the libtorch decode in fp32 (no 16-bit rounding on either side: a tight tolerance).  The shapes of the
+    reference's own fp32 cache cases (tests/core/kernels/dcu/reshape_paged_cache_test.cpp:135-158) and the three
+    head dims; contexts shorter than a workgroup's four wavefronts, empty ones, a sliding window, the CSR form."""
+    cases = [workloads.DecodeConfig("f32_ref_a", 4, 1, 1, 64, 16, 1, 40), workloads.DecodeConfig("f32_ref_b", 3, 4, 4, 128, 16, 1, 60),
+             workloads.DecodeConfig("f32_gqa", 5, 8, 2, 128, 32, 100, 900), workloads.DecodeConfig("f32_d256", 2, 6, 3, 256, 16, 50, 300)]
+    for n, cfg in enumerate(cases):
+        inp = workloads.make_inputs(cfg, 50 + n, dtype=torch.float32)
+        lay = inp.layout
+        kg, vg, _, _ = fill_caches_gpu(inp, device)
+        kc, vc = fill_caches_cpu(inp)
+        assert kg.dtype == torch.float32 and torch.equal(kg.cpu(), kc) and torch.equal(vg.cpu(), vc)
+        q = inp.q.to(device)
+        table = lay.block_table.to(device)
+        lens = lay.seq_lens.clone()
+        if cfg.batch > 3:
+            lens[1] = 0
+        out, lse = ops.batch_decode(q, kg, torch.empty_like(q), table, lens.to(device), v_cache=vg, scale=cfg.scale,
+                                    return_lse=True)
+        live = torch.nonzero(lens > 0).flatten().tolist()
+        ref = oracle.aten_paged_decode(inp.q[live].contiguous(), kc, vc, lay.block_table[live].contiguous(),
+                                       lens[live].contiguous(), cfg.scale)
+        assert out.dtype == torch.float32
+        assert torch.allclose(out.cpu()[live], ref, rtol=2e-4, atol=2e-5), cfg.name
+        ref_lse = oracle.aten_paged_decode_lse(inp.q[live].contiguous(), kc, lay.block_table[live].contiguous(),
+                                               lens[live].contiguous(), cfg.scale)
+        assert torch.allclose(lse.cpu().view(cfg.batch, -1)[live], ref_lse.view(len(live), -1), rtol=1e-4, atol=1e-4)
+        dead = torch.nonzero(lens == 0).flatten().tolist()
+        assert not out.cpu()[dead].abs().any() and torch.isneginf(lse.cpu().view(cfg.batch, -1)[dead]).all()
+        if n == 2:
+            # the window through the oracle on the trimmed context; the CSR form through the table form
+            from helpers import trimmed_context
+            win = 64
+            first = torch.clamp(lay.seq_lens - 1 - win, min=0)
+            wout, _ = ops.batch_decode(q, kg, torch.empty_like(q), table, lay.seq_lens.to(device), v_cache=vg,
+                                       scale=cfg.scale, window_left=win)
+            tk, tv, ttable, tlens = trimmed_context(kc, vc, lay.block_table, lay.seq_lens, first)
+            wref = oracle.aten_paged_decode(inp.q, tk, tv, ttable, tlens, cfg.scale)
+            assert torch.allclose(wout.cpu(), wref, rtol=2e-4, atol=2e-5)
+            full, _ = ops.batch_decode(q, kg, torch.empty_like(q), table, lay.seq_lens.to(device), v_cache=vg, scale=cfg.scale)
+            csr = ops.batch_decode_csr(q, kg, vg, lay.indptr.to(device), lay.indices.to(device),
+                                       lay.last_page_len.to(device), -1, cfg.scale, torch.empty_like(q))
+            assert torch.equal(csr, full)
+
+
 def test_head_dim_64_with_fp8_pages_on_the_matrix_core_kernel(device):
     # fp8 pages with head dim 64: rows of 64 bytes, 64 tokens per stage multiplied as two halves of 32.  Group sizes
     # 1, 4, 16 and one that needs two head blocks; block sizes 16 / 64 / 128; lengths around the 16-, 32- and

@@ -46,6 +46,9 @@ SIGNATURES = {
     "xllm_mi355_paged_decode_gqa_planned": (_i32, [_p, _sz, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _p, _p, _p, _p,
                                                    _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
                                                    _f32, _p, _sz, _i32, _i32, _p]),
+    "xllm_mi355_write_and_decode_gqa": (_i32, [_p, _p, _p, _i64, _i64, _p, _sz, _p, _p, _p, _p, _p, _p, _i64, _p, _p,
+                                               _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+                                               _i64, _f32, _p, _sz, _i32, _i32, _p]),
     "xllm_mi355_gather_paged_rows": (_i32, [_p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64, _i64, _p]),
     "xllm_mi355_paged_decode_varlen_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "xllm_mi355_paged_decode_gqa_varlen": (_i32, [_p, _p, _p, _p, _p, _p, _p, _i64, _p, _p, _i64, _i64, _i64, _i64,

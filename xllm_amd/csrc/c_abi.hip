@@ -235,6 +235,43 @@ int xllm_mi355_paged_decode_gqa_plan(void* plan, size_t plan_bytes, const int32_
                                cache_dtype, static_cast<hipStream_t>(stream));
 }
 
+int xllm_mi355_write_and_decode_gqa(const void* key, const void* value, const int32_t* slot_mapping,
+                                    int64_t k_token_stride, int64_t v_token_stride, const void* plan, size_t plan_bytes,
+                                    const void* q, void* k_cache, void* v_cache, void* out, float* lse,
+                                    const int32_t* block_table, int64_t table_stride, const int32_t* seq_lens,
+                                    const int32_t* paged_kv_indptr, const int32_t* paged_kv_indices,
+                                    const int32_t* paged_kv_last_page_len, const float* k_scale, const float* v_scale,
+                                    int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim,
+                                    int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
+                                    int64_t out_token_stride, int64_t max_seq_len, int64_t window_left, float sm_scale,
+                                    void* workspace, size_t workspace_bytes, int q_dtype, int cache_dtype,
+                                    void* stream) {
+  if (key == nullptr || value == nullptr || slot_mapping == nullptr) return XLLM_MI355_EINVAL;
+  if (k_token_stride < n_kv_heads * head_dim || v_token_stride < n_kv_heads * head_dim) return XLLM_MI355_EINVAL;
+  if (plan != nullptr && plan_bytes < gqa_plan_bytes()) return XLLM_MI355_EWORKSPACE;
+  PageAddressing addr;
+  addr.window_left = window_left;
+  addr.plan = plan;
+  if (paged_kv_indptr != nullptr) {
+    addr.indptr = paged_kv_indptr;
+    addr.indices = paged_kv_indices;
+    addr.last_page_len = paged_kv_last_page_len;
+  } else {
+    addr.block_table = block_table;
+    addr.table_stride = table_stride;
+    addr.seq_lens = seq_lens;
+  }
+  NewKvRows fresh;
+  fresh.key = key;
+  fresh.value = value;
+  fresh.slots = slot_mapping;
+  fresh.k_token_stride = k_token_stride;
+  fresh.v_token_stride = v_token_stride;
+  return paged_decode_gqa(q, k_cache, v_cache, out, lse, addr, k_scale, v_scale, batch, n_q_heads, n_kv_heads,
+                          head_dim, block_size, num_blocks, q_token_stride, out_token_stride, max_seq_len, sm_scale,
+                          workspace, workspace_bytes, q_dtype, cache_dtype, static_cast<hipStream_t>(stream), &fresh);
+}
+
 int xllm_mi355_paged_decode_gqa_planned(const void* plan, size_t plan_bytes, const void* q, const void* k_cache,
                                         const void* v_cache, void* out, float* lse,
                                         const int32_t* block_table, int64_t table_stride,

@@ -82,12 +82,24 @@ size_t decode_workspace_bound();
 // Clears the header of a workspace (a fill kernel: legal under graph capture).
 int decode_workspace_init(void* workspace, size_t workspace_bytes, hipStream_t stream);
 
+// The K / V rows of the step's new tokens, [batch, Hkv, D] of the query's dtype with token strides in elements, and
+// their slots [batch]: the decode call writes them to the caches before it attends, as reshape_and_cache would
+// (slots outside [0, num_blocks * block_size) are skipped; with fp8 pages the rows are quantised with the call's
+// scales).  Sequence b's slot must be the place of its token seq_len - 1 in its table.
+struct NewKvRows {
+  const void* key = nullptr;
+  const void* value = nullptr;
+  const int32_t* slots = nullptr;
+  int64_t k_token_stride = 0, v_token_stride = 0;
+};
+
 int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, void* out, float* lse,
                      const PageAddressing& addr, const float* k_scale, const float* v_scale,
                      int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim,
                      int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
                      int64_t out_token_stride, int64_t max_seq_len, float sm_scale, void* workspace,
-                     size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream);
+                     size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream,
+                     const NewKvRows* fresh = nullptr);
 
 // The plan of a decode step (item prefix, pool cut, first page-table chunk of every group of workers), made
 // once and handed to the decode calls of all layers through PageAddressing::plan.

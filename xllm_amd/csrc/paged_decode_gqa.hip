@@ -56,6 +56,8 @@ struct GqaArgs {
   const char* q;
   const char* k_cache;
   const char* v_cache;
+  char* k_cache_w;   // the same caches, writable (write-then-attend only)
+  char* v_cache_w;
   char* out;
   float* lse;
   const int32_t* block_table;
@@ -119,6 +121,16 @@ struct GqaArgs {
   // sequences x 32 heads: 91.1 -> 92.3 us, and the merge kernel, which then finds no partial in L2, 5.2 -> 5.5 us), so
   // the host turns it on from 8192 output rows (sequences x heads) per launch.
   int stream_stores;
+  // Write-then-attend in one launch: the step's new K / V rows [batch, Hkv, D] of the query's 16-bit type (token strides
+  // in bytes) and their slots, or null.  The worker that reaches the last stage of (sequence, KV head) puts the new
+  // row where the stage expects it in LDS (quantised for fp8 pages, over whatever the loader fetched from the slot
+  // that is not written yet) and writes the same bytes to the cache: what reshape_and_cache would have written before
+  // the launch.  Slots outside [0, n_slots) are skipped, as there.
+  const char* new_k;
+  const char* new_v;
+  const int32_t* new_slots;
+  int64_t new_k_stride_bytes, new_v_stride_bytes;
+  int64_t n_slots;
   int wait_spins;     // bound of the polls of one wavefront of a pair on the other
   int window_left;    // sliding window: the query (position L - 1) attends to positions >= L - 1 - window_left; < 0: all
   float scale_log2;   // sm_scale * log2(e)
@@ -650,6 +662,8 @@ typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((ext_vector_type(2))) int i32x2;
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
 typedef __attribute__((address_space(3))) volatile int lds_vint;  // a word of LDS that other wavefronts write
+typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 
 // 16 (4) bytes per lane from global memory straight into LDS at lds_addr + lane * 16 (4);
 // lds_addr is wave-uniform and travels in M0.
@@ -1203,6 +1217,11 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   f32x4 o[MB];
   float m = kNegBig, l = 0.0f;
   float score_scale = a.scale_log2, out_scale = 1.0f;
+  // write-then-attend: the lane's 16 bytes of the new K and V rows as the cache holds them (chunk dc of the row; with
+  // fp8 pages the codes of 16 values), fetched when a run begins that reaches its context's end; the slot, or -1
+  const bool fused = !VL && a.new_k != nullptr;
+  u32x4 new_k = {0u, 0u, 0u, 0u}, new_v = {0u, 0u, 0u, 0u};
+  int64_t new_slot = -1;
 
   int arrived = 0;
   for (int s = 0; s < n_stages; ++s) {
@@ -1264,13 +1283,64 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       m = kNegBig;
       l = 0.0f;
       c_ctx_first = s;
+      float k_scale_h = 1.0f;
       if constexpr (FP8) {  // per-KV-head scales, through the scalar cache like the lengths
-        score_scale = a.scale_log2 * as_f32(sload32(reinterpret_cast<const int32_t*>(a.k_scale) + kvh));
+        k_scale_h = as_f32(sload32(reinterpret_cast<const int32_t*>(a.k_scale) + kvh));
+        score_scale = a.scale_log2 * k_scale_h;
         out_scale = as_f32(sload32(reinterpret_cast<const int32_t*>(a.v_scale) + kvh));
+      }
+      if constexpr (!VL) {
+        new_slot = -1;
+        if (fused && cc.n_st - cc.st <= n_stages - s) {   // this run holds the context's last stage: the new token's
+          const int64_t slot = sload32(a.new_slots + cc.b);
+          if (slot >= 0 && slot < a.n_slots) {
+            new_slot = slot;
+            const char* kp = a.new_k + cc.b * a.new_k_stride_bytes + static_cast<int64_t>(kvh) * D * 2;
+            const char* vp = a.new_v + cc.b * a.new_v_stride_bytes + static_cast<int64_t>(kvh) * D * 2;
+            if constexpr (!FP8) {
+              new_k = ldg16(kp + dc * 16);
+              new_v = ldg16(vp + dc * 16);
+            } else {
+              // 16 codes from 32 bytes of input, with the arithmetic of reshape_and_cache
+              const u32x4 k0 = ldg16(kp + dc * 32), k1 = ldg16(kp + dc * 32 + 16);
+              const u32x4 v0 = ldg16(vp + dc * 32), v1 = ldg16(vp + dc * 32 + 16);
+              const float ik = 1.0f / k_scale_h, iv = 1.0f / out_scale;
+              auto codes = [](u32 w, float inv) {
+                return fp8_quantize(QT::lo(w), inv) | (fp8_quantize(QT::hi(w), inv) << 8);
+              };
+#pragma unroll
+              for (int i = 0; i < 2; ++i) {
+                new_k[i] = codes(k0[2 * i], ik) | (codes(k0[2 * i + 1], ik) << 16);
+                new_k[2 + i] = codes(k1[2 * i], ik) | (codes(k1[2 * i + 1], ik) << 16);
+                new_v[i] = codes(v0[2 * i], iv) | (codes(v0[2 * i + 1], iv) << 16);
+                new_v[2 + i] = codes(v1[2 * i], iv) | (codes(v1[2 * i + 1], iv) << 16);
+              }
+            }
+          }
+        }
       }
     }
 
     const char* st = ring + (s % NS) * kStageBytes;
+    if constexpr (!VL) {
+      if (new_slot >= 0 && cc.st == cc.n_st - 1) {
+        // The context's last stage: the new token is row r of it, and the rows behind it repeat it (the loader fetched
+        // them from the slot, which holds whatever it held before).  Every row from r on gets the new row, chunk by chunk
+        // where the operand reads expect it; row r also goes to the cache.
+        const int r = cc.L - 1 - (cc.st0 + cc.st) * T;
+        char* stw = const_cast<char*>(st);
+        for (int row = r + dr; row < T; row += RPI) {
+          *(lds_u32x4*)(stw + row * RB + ((dc ^ swz_k(row)) * 16)) = new_k;
+          *(lds_u32x4*)(stw + T * RB + row * RB + ((dc ^ swz_v(row)) * 16)) = new_v;
+        }
+        if (dr == 0) {
+          const int64_t off = new_slot * a.row_bytes + static_cast<int64_t>(cc.kvh) * RB + dc * 16;
+          stg16(a.k_cache_w + off, new_k);
+          stg16(a.v_cache_w + off, new_v);
+        }
+        new_slot = -1;
+      }
+    }
     if constexpr (!FP8 && T <= 16) {
       // ---- all operand reads of the stage first: the latency of the V^T reads passes behind the score
       // MFMAs and the softmax (the scheduler would otherwise place them next to their use)
@@ -1953,15 +2023,21 @@ int dispatch_group(GqaArgs& a, size_t wsb, hipStream_t s, bool plan_only, size_t
   }
 }
 
+// Whether the matrix-core kernel serves a one-query-token call (its epilogue stores 8 output bytes at a time; its
+// stages are whole parts of a page of a power-of-two size from 16 tokens on; fp8 rows of 256 bytes have no loop there).
+bool mfma_serves(const GqaArgs& a, bool fp8, int head_dim) {
+  const bool out_aligned = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
+  const bool dim_ok = head_dim == 64 || head_dim == 128 || (head_dim == 256 && !fp8);
+  return dim_ok && a.bs_shift >= 4 && out_aligned && use_mfma_kernel();
+}
+
 template <typename QT, bool FP8>
 int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_only, size_t* need) {
   // lanes per token row: one 16-byte load per lane and row
+  const bool mfma = mfma_serves(a, FP8, head_dim);
   if constexpr (FP8) {
-    const bool out_aligned8 = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
-    if (head_dim == 128 && a.bs_shift >= 4 && out_aligned8 && use_mfma_kernel())
-      return launch_gqa_mfma<QT, true>(a, wsb, s, plan_only, need);
-    if (head_dim == 64 && a.bs_shift >= 4 && out_aligned8 && use_mfma_kernel())
-      return launch_gqa_mfma<QT, true, false, 64>(a, wsb, s, plan_only, need);
+    if (head_dim == 128 && mfma) return launch_gqa_mfma<QT, true>(a, wsb, s, plan_only, need);
+    if (head_dim == 64 && mfma) return launch_gqa_mfma<QT, true, false, 64>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, true, 64, 4, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, true, 128, 8, 2>(a, wsb, s, plan_only, need);
@@ -1969,14 +2045,9 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
       default: return XLLM_MI355_ESHAPE;
     }
   } else {
-    // (its epilogue stores 8 output bytes at a time)
-    const bool out_aligned = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
-    if (head_dim == 128 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
-      return launch_gqa_mfma<QT, false>(a, wsb, s, plan_only, need);
-    if (head_dim == 64 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
-      return launch_gqa_mfma<QT, false, false, 64>(a, wsb, s, plan_only, need);
-    if (head_dim == 256 && a.bs_shift >= 4 && out_aligned && use_mfma_kernel())
-      return launch_gqa_mfma<QT, false, false, 256>(a, wsb, s, plan_only, need);
+    if (head_dim == 128 && mfma) return launch_gqa_mfma<QT, false>(a, wsb, s, plan_only, need);
+    if (head_dim == 64 && mfma) return launch_gqa_mfma<QT, false, false, 64>(a, wsb, s, plan_only, need);
+    if (head_dim == 256 && mfma) return launch_gqa_mfma<QT, false, false, 256>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, false, 64, 8, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, false, 128, 16, 4>(a, wsb, s, plan_only, need);
@@ -1984,6 +2055,84 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
       default: return XLLM_MI355_ESHAPE;
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 query, fp32 pages, fp32 output: the caches that reshape_and_cache stores for fp32 models (the reference's
+// own cases {4,1,16,1,64,f32} and {1,4,16,4,128,f32}, tests/core/kernels/dcu/reshape_paged_cache_test.cpp:135-158)
+// can be attended too, as the reference's libtorch decode attends any dtype (kernels/npu/attention.cpp:26-78).  A
+// compatibility path, not a tuned one: one workgroup per (query head, sequence), no split over workgroups, no
+// workspace; a wavefront takes every fourth token, a lane D / 64 dims of it; a score is a sum over the wavefront's
+// lanes; the four wavefronts' states meet in LDS at the end.
+template <int D>
+__global__ __launch_bounds__(256) void gqa_decode_f32_kernel(GqaArgs a) {
+  constexpr int E = D / 64;   // dims per lane
+  __shared__ float part[4][D + 2];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kvh = h / a.group;
+  const int32_t* pages;
+  int L;
+  sequence_of(a, b, pages, L);
+  float* out = reinterpret_cast<float*>(a.out + b * a.out_stride_bytes) + static_cast<int64_t>(h) * D;
+  if (L <= 0) {
+    for (int d = threadIdx.x; d < D; d += 256) out[d] = 0.0f;
+    if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * a.n_q_heads + h] = -INFINITY;
+    return;
+  }
+  const float* q = reinterpret_cast<const float*>(a.q + b * a.q_stride_bytes) + static_cast<int64_t>(h) * D + lane * E;
+  float qv[E], o[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) {
+    qv[i] = q[i] * a.scale_log2;
+    o[i] = 0.0f;
+  }
+  float m = kNegBig, l = 0.0f;
+  const int64_t head_off = static_cast<int64_t>(kvh) * D + lane * E;
+  for (int t = first_token(a, L) + wave; t < L; t += 4) {
+    int page = pages[t / a.block_size];
+    page = max(0, min(page, a.num_blocks - 1));   // a corrupt table must not fault the GPU
+    const int64_t row = (static_cast<int64_t>(page) * a.block_size + t % a.block_size) * (a.row_bytes / 4) + head_off;
+    const float* k = reinterpret_cast<const float*>(a.k_cache) + row;
+    const float* v = reinterpret_cast<const float*>(a.v_cache) + row;
+    float kv[E], vv[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      kv[i] = k[i];
+      vv[i] = v[i];
+    }
+    float sc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < E; ++i) sc += qv[i] * kv[i];
+    sc = group_sum<32>(sc);
+    sc += __shfl_xor(sc, 32, kWave);
+    const float m_new = fmaxf(m, sc);
+    const float keep = fast_exp2(m - m_new), p = fast_exp2(sc - m_new);
+    l = l * keep + p;
+#pragma unroll
+    for (int i = 0; i < E; ++i) o[i] = o[i] * keep + p * vv[i];
+    m = m_new;
+  }
+#pragma unroll
+  for (int i = 0; i < E; ++i) part[wave][lane * E + i] = o[i];
+  if (lane == 0) {
+    part[wave][D] = m;
+    part[wave][D + 1] = l;
+  }
+  __syncthreads();
+  float M = kNegBig;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) M = fmaxf(M, part[w][D]);
+  float W = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) W += part[w][D + 1] * fast_exp2(part[w][D] - M);   // (a wavefront without tokens: 0 * 1)
+  for (int d = threadIdx.x; d < D; d += 256) {
+    float x = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) x += part[w][d] * fast_exp2(part[w][D] - M);
+    out[d] = x / W;
+  }
+  if (a.lse != nullptr && threadIdx.x == 0) a.lse[b * a.n_q_heads + h] = (M + fast_log2(W)) * kLn2;
 }
 
 int group_block(int group) {
@@ -2065,10 +2214,13 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
                      int64_t batch, int64_t n_q_heads, int64_t n_kv_heads, int64_t head_dim,
                      int64_t block_size, int64_t num_blocks, int64_t q_token_stride,
                      int64_t out_token_stride, int64_t max_seq_len, float sm_scale, void* workspace,
-                     size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream) {
+                     size_t workspace_bytes, int q_dtype, int cache_dtype, hipStream_t stream, const NewKvRows* fresh) {
   (void)max_seq_len;  // the schedule is computed on the device from the actual lengths
   if (batch == 0) return XLLM_MI355_OK;
   if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr) return XLLM_MI355_EINVAL;
+  if (fresh != nullptr && (fresh->key == nullptr || fresh->value == nullptr || fresh->slots == nullptr ||
+                           addr.cu_q != nullptr))
+    return XLLM_MI355_EINVAL;
   const bool csr = addr.indptr != nullptr;
   if (csr ? (addr.indices == nullptr || addr.last_page_len == nullptr)
           : (addr.block_table == nullptr || addr.seq_lens == nullptr || addr.table_stride <= 0))
@@ -2077,13 +2229,58 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
       n_q_heads % n_kv_heads != 0 || n_q_heads > 65535 || !(sm_scale > 0.0f))
     return XLLM_MI355_EINVAL;
   if (num_blocks * block_size > 0x7fffffffLL) return XLLM_MI355_ESHAPE;
-  if (q_dtype != XLLM_MI355_BF16 && q_dtype != XLLM_MI355_FP16) return XLLM_MI355_EDTYPE;
+  if (q_dtype != XLLM_MI355_BF16 && q_dtype != XLLM_MI355_FP16 && q_dtype != XLLM_MI355_FP32) return XLLM_MI355_EDTYPE;
   const bool fp8 = cache_dtype == XLLM_MI355_FP8_E4M3;
   if (!fp8 && cache_dtype != q_dtype) return XLLM_MI355_EDTYPE;
+  if (fp8 && q_dtype == XLLM_MI355_FP32) return XLLM_MI355_EDTYPE;
   if (fp8 && (k_scale == nullptr || v_scale == nullptr)) return XLLM_MI355_EINVAL;
   if (head_dim != 64 && head_dim != 128 && head_dim != 256) return XLLM_MI355_ESHAPE;
   if (q_token_stride < n_q_heads * head_dim || out_token_stride < n_q_heads * head_dim)
     return XLLM_MI355_EINVAL;
+  if (q_dtype == XLLM_MI355_FP32) {   // fp32 query over fp32 pages: the compatibility kernel, no workspace
+    if (addr.cu_q != nullptr || addr.table_rows != nullptr) return XLLM_MI355_EDTYPE;
+    if (((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(k_cache) |
+          reinterpret_cast<uintptr_t>(v_cache)) & 15) != 0 || (q_token_stride * 4) % 16 != 0 || (out_token_stride * 4) % 16 != 0)
+      return XLLM_MI355_EALIGN;
+    if (batch > 65535) return XLLM_MI355_ESHAPE;
+    if (fresh != nullptr) {
+      const int rc = reshape_and_cache(fresh->key, fresh->value, const_cast<void*>(k_cache), const_cast<void*>(v_cache),
+                                       fresh->slots, k_scale, v_scale, batch, n_kv_heads, head_dim, block_size, num_blocks,
+                                       fresh->k_token_stride, fresh->v_token_stride, q_dtype, cache_dtype, stream);
+      if (rc != 0) return rc;
+    }
+    GqaArgs a = {};
+    a.q = static_cast<const char*>(q);
+    a.k_cache = static_cast<const char*>(k_cache);
+    a.v_cache = static_cast<const char*>(v_cache);
+    a.out = static_cast<char*>(out);
+    a.lse = lse;
+    a.block_table = csr ? nullptr : addr.block_table;
+    a.seq_lens = csr ? nullptr : addr.seq_lens;
+    a.indptr = csr ? addr.indptr : nullptr;
+    a.indices = addr.indices;
+    a.last_page_len = csr ? addr.last_page_len : nullptr;
+    a.table_stride = addr.table_stride;
+    a.window_left = addr.window_left < 0 ? -1 : static_cast<int>(addr.window_left < 0x7fffffffLL ? addr.window_left : 0x7fffffffLL);
+    a.q_stride_bytes = q_token_stride * 4;
+    a.out_stride_bytes = out_token_stride * 4;
+    a.row_bytes = n_kv_heads * head_dim * 4;
+    a.batch = static_cast<int>(batch);
+    a.n_q_heads = static_cast<int>(n_q_heads);
+    a.n_kv_heads = static_cast<int>(n_kv_heads);
+    a.group = static_cast<int>(n_q_heads / n_kv_heads);
+    a.block_size = static_cast<int>(block_size);
+    a.num_blocks = static_cast<int>(num_blocks);
+    a.scale_log2 = sm_scale * kLog2e;
+    const dim3 grid(static_cast<unsigned>(n_q_heads), static_cast<unsigned>(batch));
+    switch (head_dim) {
+      case 64: launch_timed(gqa_decode_f32_kernel<64>, grid, dim3(256), 0, stream, a); break;
+      case 128: launch_timed(gqa_decode_f32_kernel<128>, grid, dim3(256), 0, stream, a); break;
+      default: launch_timed(gqa_decode_f32_kernel<256>, grid, dim3(256), 0, stream, a); break;
+    }
+    profile_skip();   // (no merge launch)
+    return static_cast<int>(hipGetLastError());
+  }
   auto aligned16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (q_token_stride * 2) % 16 != 0)
     return XLLM_MI355_EALIGN;
@@ -2100,6 +2297,26 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
         addr.n_tokens <= 0 || addr.n_tokens > 0x7fffffffLL || addr.chunk_blocks <= 0 || addr.chunk_blocks > kMfmaHeads ||
         addr.window_left >= 0)
       return XLLM_MI355_EINVAL;
+  }
+  // The step's new rows: inside the matrix-core kernel when it serves the call and a lane can take 16 bytes of a row
+  // at a time; otherwise the write is a launch of its own before the decode, with the same result.
+  bool fused = false;
+  if (fresh != nullptr) {
+    GqaArgs probe = {};
+    probe.out = static_cast<char*>(out);
+    probe.out_stride_bytes = out_token_stride * 2;
+    probe.bs_shift = -1;
+    for (int s = 0; s < 31; ++s)
+      if ((1LL << s) == block_size) probe.bs_shift = s;
+    fused = mfma_serves(probe, fp8, static_cast<int>(head_dim)) && aligned16(fresh->key) && aligned16(fresh->value) &&
+            (fresh->k_token_stride * 2) % 16 == 0 && (fresh->v_token_stride * 2) % 16 == 0 &&
+            fresh->k_token_stride >= n_kv_heads * head_dim && fresh->v_token_stride >= n_kv_heads * head_dim;
+    if (!fused) {
+      const int rc = reshape_and_cache(fresh->key, fresh->value, const_cast<void*>(k_cache), const_cast<void*>(v_cache),
+                                       fresh->slots, k_scale, v_scale, batch, n_kv_heads, head_dim, block_size, num_blocks,
+                                       fresh->k_token_stride, fresh->v_token_stride, q_dtype, cache_dtype, stream);
+      if (rc != 0) return rc;
+    }
   }
   // Batches beyond the LDS prefix capacity are decoded in slices; each slice is an
   // independent launch pair on the same stream and workspace.
@@ -2124,6 +2341,16 @@ int paged_decode_gqa(const void* q, const void* k_cache, const void* v_cache, vo
     a.last_page_len = csr ? addr.last_page_len + b0 : nullptr;
     a.k_scale = k_scale;
     a.v_scale = v_scale;
+    if (fused) {
+      a.k_cache_w = const_cast<char*>(a.k_cache);
+      a.v_cache_w = const_cast<char*>(a.v_cache);
+      a.new_k = static_cast<const char*>(fresh->key) + b0 * fresh->k_token_stride * 2;
+      a.new_v = static_cast<const char*>(fresh->value) + b0 * fresh->v_token_stride * 2;
+      a.new_slots = fresh->slots + b0;
+      a.new_k_stride_bytes = fresh->k_token_stride * 2;
+      a.new_v_stride_bytes = fresh->v_token_stride * 2;
+      a.n_slots = num_blocks * block_size;
+    }
     a.ws_status = static_cast<int*>(workspace);
     a.ws_prefix = reinterpret_cast<int*>(static_cast<char*>(workspace) + kWsHeaderBytes);
     a.plan = !packed && batch <= kMaxBatch ? static_cast<const int*>(addr.plan) : nullptr;

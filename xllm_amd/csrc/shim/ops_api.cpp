@@ -153,7 +153,8 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
                   const std::optional<torch::Tensor>& v_cache, std::optional<torch::Tensor>& output_lse,
                   const std::optional<torch::Tensor>& k_cache_quant_scale,
                   const std::optional<torch::Tensor>& v_cache_quant_scale, int64_t max_seq_len,
-                  int64_t window_size_left, float scale, bool return_lse, const std::optional<torch::Tensor>& plan) {
+                  int64_t window_size_left, float scale, bool return_lse, const std::optional<torch::Tensor>& plan,
+                  const NewKvRows* fresh) {
   TORCH_CHECK(v_cache.has_value() && v_cache->defined(), "GQA decode needs v_cache");
   check_decode_operands(query, output, k_cache, *v_cache, k_cache_quant_scale, v_cache_quant_scale);
   TORCH_CHECK(block_table.scalar_type() == torch::kInt32 && block_table.dim() == 2 && block_table.stride(1) == 1 &&
@@ -174,10 +175,32 @@ void batch_decode(const torch::Tensor& query, const torch::Tensor& k_cache, torc
   if (max_seq_len <= 0) max_seq_len = block_table.size(1) * k_cache.size(1);
   const size_t nbytes = xllm_mi355_paged_decode_gqa_workspace_bytes(B, Hq, D);
   torch::Tensor ws = decode_workspace(query.device(), nbytes);
-  if (plan.has_value() && plan->defined()) {
+  const bool planned = plan.has_value() && plan->defined();
+  if (planned)
     TORCH_CHECK(plan->is_cuda() && plan->is_contiguous() && plan->scalar_type() == torch::kUInt8 &&
                     static_cast<size_t>(plan->numel()) >= xllm_mi355_paged_decode_plan_bytes(),
                 "plan must be the buffer of update_decode_plan (uint8, xllm_mi355_paged_decode_plan_bytes() bytes)");
+  if (fresh != nullptr) {
+    for (const torch::Tensor* t : {&fresh->key, &fresh->value})
+      TORCH_CHECK(t->is_cuda() && t->dim() == 3 && t->size(0) == B && t->size(1) == k_cache.size(2) && t->size(2) == D &&
+                      t->stride(2) == 1 && t->stride(1) == D && t->scalar_type() == query.scalar_type(),
+                  "the step's key / value must be device tensors [B, Hkv, D] of the query's dtype, tokens contiguous");
+    TORCH_CHECK(fresh->slot_mapping.is_cuda() && fresh->slot_mapping.scalar_type() == torch::kInt32 &&
+                    fresh->slot_mapping.is_contiguous() && fresh->slot_mapping.numel() == B,
+                "slot_mapping must be contiguous int32 [B]");
+    const int rc = xllm_mi355_write_and_decode_gqa(
+        fresh->key.data_ptr(), fresh->value.data_ptr(), fresh->slot_mapping.data_ptr<int32_t>(), fresh->key.stride(0),
+        fresh->value.stride(0), planned ? plan->data_ptr() : nullptr, planned ? static_cast<size_t>(plan->numel()) : 0,
+        query.data_ptr(), k_cache.data_ptr(), v_cache->data_ptr(), output.data_ptr(), lse,
+        block_table.data_ptr<int32_t>(), block_table.stride(0), seq_lens.data_ptr<int32_t>(), nullptr, nullptr, nullptr,
+        static_cast<const float*>(ptr_or_null(k_cache_quant_scale)),
+        static_cast<const float*>(ptr_or_null(v_cache_quant_scale)), B, Hq, k_cache.size(2), D, k_cache.size(1),
+        k_cache.size(0), query.stride(0), output.stride(0), max_seq_len, window_size_left, scale, ws.data_ptr(),
+        static_cast<size_t>(ws.numel()), dtype_code(query), dtype_code(k_cache), current_stream(query));
+    check_rc(rc, "xllm_mi355_write_and_decode_gqa");
+    return;
+  }
+  if (planned) {
     const int rc = xllm_mi355_paged_decode_gqa_planned(
         plan->data_ptr(), static_cast<size_t>(plan->numel()), query.data_ptr(), k_cache.data_ptr(), v_cache->data_ptr(), output.data_ptr(), lse,
         block_table.data_ptr<int32_t>(), block_table.stride(0), seq_lens.data_ptr<int32_t>(), nullptr, nullptr, nullptr,
@@ -691,8 +714,14 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> Mi355AttentionImpl::forw
   const bool quantized = k_scale.has_value() && k_scale->defined();
 
   // store the step's K / V rows; the quantising store where the cache carries scales
-  // (xllm/core/layers/mlu/attention.cpp:109-117)
-  if (k_cache.defined() && k_cache.dim() >= 2) {
+  // (xllm/core/layers/mlu/attention.cpp:109-117).  A plain decode step stores them inside its decode call below.
+  const bool has_cache = k_cache.defined() && k_cache.dim() >= 2;
+  const bool decode_step = !attn_metadata.is_chunked_prefill && !attn_metadata.is_prefill;
+  const bool one_call = has_cache && decode_step && key.size(0) == query.size(0) && key.stride(1) == head_size_ &&
+                        value.stride(1) == head_size_ && attn_metadata.slot_mapping.scalar_type() == torch::kInt32 &&
+                        attn_metadata.slot_mapping.is_contiguous() &&
+                        (quantized || k_cache.scalar_type() == key.scalar_type());
+  if (has_cache && !one_call) {
     xllm::kernel::ReshapePagedCacheParams params;
     params.key = key;
     params.value = value;
@@ -743,8 +772,10 @@ std::tuple<torch::Tensor, std::optional<torch::Tensor>> Mi355AttentionImpl::forw
       TORCH_CHECK(attn_metadata.plan_info->plan_info.defined(), "no layer 0 has planned this step");
       plan = attn_metadata.plan_info->plan_info;
     }
+    const xllm::kernel::mi355::NewKvRows fresh{key, value, attn_metadata.slot_mapping};
     xllm::kernel::mi355::batch_decode(query, k_cache, output, block_table, kv_seq_lens, v_cache, output_lse, k_scale,
-                                      v_scale, attn_metadata.max_seq_len, window_left, scale_, return_lse_, plan);
+                                      v_scale, attn_metadata.max_seq_len, window_left, scale_, return_lse_, plan,
+                                      one_call ? &fresh : nullptr);
   }
   output = output.view({-1, num_heads_ * head_size_});
   return std::make_tuple(output, output_lse);

@@ -53,6 +53,13 @@ torch::Tensor decode_workspace(const torch::Device& device, size_t nbytes);
 // invalid).  Synchronises the current stream: not for use under graph capture.
 void decode_status(const torch::Device& device);
 
+// The K / V rows of a decode step's new tokens [B, Hkv, D] and their slots [B] int32: handed to batch_decode, they
+// are stored into the caches by the decode call itself (the reshape_paged_cache + batch_decode pair of
+// xllm/core/layers/dcu/torch_attention.cpp:138-144 and :285-347 in one call, with the pair's cache bytes and output).
+struct NewKvRows {
+  torch::Tensor key, value, slot_mapping;
+};
+
 void batch_decode(const torch::Tensor& query,        // [B, Hq, D]
                   const torch::Tensor& k_cache,      // [P, bs, Hkv, D]
                   torch::Tensor& output,             // [B, Hq, D]
@@ -63,7 +70,7 @@ void batch_decode(const torch::Tensor& query,        // [B, Hq, D]
                   const std::optional<torch::Tensor>& k_cache_quant_scale,
                   const std::optional<torch::Tensor>& v_cache_quant_scale,
                   int64_t max_seq_len, int64_t window_size_left, float scale, bool return_lse,
-                  const std::optional<torch::Tensor>& plan = std::nullopt);
+                  const std::optional<torch::Tensor>& plan = std::nullopt, const NewKvRows* fresh = nullptr);
 
 // The plan of a decode step, made once and taken by the decode calls of every layer (`plan` above and in
 // batch_decode_csr): the part of update_decode_plan_info (xllm/core/layers/cuda/flashinfer_planinfo.cpp:248-264),

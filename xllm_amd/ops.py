@@ -262,18 +262,21 @@ def update_decode_plan_info(num_qo_heads, num_kv_heads, head_dim, block_size, ca
 
 def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, output_lse=None,
                  k_cache_quant_scale=None, v_cache_quant_scale=None, scale=None, return_lse=False,
-                 max_seq_len=0, window_left=-1, plan=None):
+                 max_seq_len=0, window_left=-1, plan=None, new_key=None, new_value=None, slot_mapping=None):
     """Block-table paged decode.  Argument order and meaning follow mlu::batch_decode
     (mlu_ops_api.h:127) restricted to what npu::batch_decode (npu_ops_api.h:46) also has.
     query/output [B, Hq, D]; caches [P, bs, Hkv, D]; block_table [B, W] int32; seq_lens [B] int32.
     window_left >= 0: sliding window, the query attends to the last window_left + 1 tokens of its context
     (sliding_window_ of layers/dcu/flash_attention.cpp:484).
     plan: the step's plan from update_decode_plan_info (same tables, lengths, heads and window), or None.
+    new_key / new_value [B, Hkv, D] with slot_mapping [B] int32: the step's K / V rows, stored into the caches by the
+    same call before it attends (the reshape_paged_cache + batch_decode pair of an attention layer's decode step,
+    layers/dcu/torch_attention.cpp:138-144 and :285-347, in one call; same cache bytes and output as the pair).
     Returns (output, lse or None) with lse [B, Hq, 1] fp32 natural log."""
     if v_cache is None:
         raise ValueError("GQA decode needs v_cache; the latent-KV variant is dense_decode")
     dev = _require_cuda(query, k_cache, v_cache, output, block_table, seq_lens, output_lse,
-                        k_cache_quant_scale, v_cache_quant_scale, plan)
+                        k_cache_quant_scale, v_cache_quant_scale, plan, new_key, new_value, slot_mapping)
     _decode_common(query, k_cache, output, v_cache, k_cache_quant_scale, v_cache_quant_scale)
     B, Hq, D = query.shape
     P, bs, Hkv, _ = k_cache.shape
@@ -297,6 +300,25 @@ def batch_decode(query, k_cache, output, block_table, seq_lens, v_cache=None, ou
     ws = decode_workspace(dev, nbytes)
     if plan is not None:
         _check_plan(plan)
+    if new_key is not None or new_value is not None or slot_mapping is not None:
+        if new_key is None or new_value is None or slot_mapping is None:
+            raise ValueError("new_key, new_value and slot_mapping come together")
+        for t in (new_key, new_value):
+            if t.dtype != query.dtype or t.dim() != 3 or tuple(t.shape) != (B, Hkv, D) or t.stride(2) != 1 or \
+                    t.stride(1) != D:
+                raise ValueError("new_key / new_value must be [B, Hkv, D] of the query's dtype with contiguous tokens")
+        if slot_mapping.dtype != torch.int32 or slot_mapping.numel() != B or not slot_mapping.is_contiguous():
+            raise ValueError("slot_mapping must be contiguous int32 [B]")
+        rc = lib.xllm_mi355_write_and_decode_gqa(
+            new_key.data_ptr(), new_value.data_ptr(), slot_mapping.data_ptr(), new_key.stride(0), new_value.stride(0),
+            _ptr(plan), 0 if plan is None else plan.numel(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            output.data_ptr(), _ptr(lse), block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), None,
+            None, None, _ptr(k_cache_quant_scale), _ptr(v_cache_quant_scale), B, Hq, Hkv, D, bs, P,
+            query.stride(0), output.stride(0), max_seq_len, int(window_left), float(scale), ws.data_ptr(), ws.numel(),
+            _dtype_code(query), _dtype_code(k_cache), _stream(dev))
+        capi.check(rc, "xllm_mi355_write_and_decode_gqa")
+        return output, lse
+    if plan is not None:
         rc = lib.xllm_mi355_paged_decode_gqa_planned(
             plan.data_ptr(), plan.numel(), query.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), output.data_ptr(), _ptr(lse),
             block_table.data_ptr(), block_table.stride(0), seq_lens.data_ptr(), None, None, None,
