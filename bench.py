@@ -50,6 +50,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline (and with it the parity check)")
     ap.add_argument("--no-planned", action="store_true",
                     help="skip the second timed loop (the GQA step with the plan made once per step)")
+    ap.add_argument("--two-calls", action="store_true",
+                    help="GQA: time the pair reshape_and_cache + paged_decode_gqa as the step instead of the one call "
+                         "write_and_decode_gqa (the default line reports the pair beside the one call anyway)")
     ap.add_argument("--graph", action="store_true",
                     help="add a third timed loop: the step captured in a HIP graph and replayed (graph_replay in the line)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
@@ -391,17 +394,38 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
 
     bound = [bound_args(k_caches[i], v_caches[i]) for i in range(ROTATE)]
     reshape_args, decode_args = bound[0]
+    # GQA: the step as the attention layer issues it, one call that stores the new rows and attends
+    # (xllm_mi355_write_and_decode_gqa); the pair of calls it replaces is timed beside it.  MLA: the pair.
+    one_call = not cfg.mla and not args.two_calls
+    one_fn = lib.xllm_mi355_write_and_decode_gqa
 
-    def make_step(copies):
+    def one_call_args(d_args, plan=None):
+        return (ptr(inp.k_new), ptr(inp.v_new), ptr(new_slots), row, row, ptr(plan), 0 if plan is None else plan.numel()) \
+            + d_args[:8] + (None, None, None) + d_args[8:]
+
+    def step_calls(i, one, plan=None):
+        """The calls of one step on cache copy i: [(fn, args), ...]."""
+        r_args, d_args = bound[i]
+        if one:
+            return [(one_fn, one_call_args(d_args, plan))]
+        if plan is None:
+            return [(reshape_fn, r_args), (decode_fn, d_args)]
+        if cfg.mla:
+            return [(reshape_fn, r_args), (lib.xllm_mi355_paged_decode_mla_planned, (ptr(plan), plan.numel()) + d_args)]
+        return [(reshape_fn, r_args), (lib.xllm_mi355_paged_decode_gqa_planned,
+                                       (ptr(plan), plan.numel()) + d_args[:8] + (None, None, None) + d_args[8:])]
+
+    def make_step(copies, one=one_call, plan=None):
         state = [0]
+        calls = [step_calls(i, one, plan) for i in range(copies)]
 
         def step():
-            r_args, d_args = bound[state[0] % copies]
+            todo = calls[state[0] % copies]
             state[0] += 1
-            rc = reshape_fn(*r_args)
-            rc2 = decode_fn(*d_args)
-            if rc or rc2:
-                capi.check(rc or rc2, "bench step")
+            for fn, fn_args in todo:
+                rc = fn(*fn_args)
+                if rc:
+                    capi.check(rc, "bench step")
         return step
 
     def timed_loop(step, events):
@@ -443,6 +467,18 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     _, same_kernel_ms, same_merge_ms = timed_loop(same_step, events=True)
     same_cache = {"ms_per_step": same_ms_per_step, "kernel_ms": same_kernel_ms, "merge_kernel_ms": same_merge_ms,
                   "tokens_per_s": cfg.batch / (same_ms_per_step * 1e-3)}
+    # the pair of calls (store, then decode) that the one call replaces
+    two_calls = None
+    if one_call:
+        pair_step = make_step(ROTATE, one=False)
+        pair_ms_per_step, _, _ = timed_loop(pair_step, events=False)
+        _, pair_kernel_ms, pair_merge_ms = timed_loop(pair_step, events=True)
+        pair_out = out.clone()
+        step()
+        torch.cuda.synchronize()
+        two_calls = {"ms_per_step": pair_ms_per_step, "kernel_ms": pair_kernel_ms, "merge_kernel_ms": pair_merge_ms,
+                     "tokens_per_s": cfg.batch / (pair_ms_per_step * 1e-3),
+                     "bit_identical": bool(torch.equal(pair_out, out))}
     elapsed = ms_per_step * 1e-3 * args.steps
 
     # ---- the same step as the layers after the first see it when the step was planned once (not the headline:
@@ -451,25 +487,15 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     if not args.no_planned and (not cfg.mla or cfg.n_q_heads > 64):
         plan = torch.empty(lib.xllm_mi355_paged_decode_plan_bytes(), dtype=torch.uint8, device=dev)
         if cfg.mla:
-            plan_fn, planned_fn = lib.xllm_mi355_paged_decode_mla_plan, lib.xllm_mi355_paged_decode_mla_planned
+            plan_fn = lib.xllm_mi355_paged_decode_mla_plan
             plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), cfg.batch, cfg.n_q_heads,
                          cfg.block_size, stream)
-            planned_bound = [(r, (ptr(plan), plan.numel()) + d) for r, d in bound]
         else:
-            plan_fn, planned_fn = lib.xllm_mi355_paged_decode_gqa_plan, lib.xllm_mi355_paged_decode_gqa_planned
+            plan_fn = lib.xllm_mi355_paged_decode_gqa_plan
             plan_args = (ptr(plan), plan.numel(), ptr(table), table.stride(0), ptr(seq_lens), None, None, None, cfg.batch,
                          cfg.n_q_heads, cfg.n_kv_heads, cfg.head_dim, cfg.block_size, -1, code[cache_dt], stream)
-            planned_bound = [(r, (ptr(plan), plan.numel()) + d[:8] + (None, None, None) + d[8:]) for r, d in bound]
         plain_out = out.clone()
-        p_state = [0]
-
-        def planned_step():
-            r_args, d_args = planned_bound[p_state[0] % ROTATE]
-            p_state[0] += 1
-            rc = reshape_fn(*r_args)
-            rc2 = planned_fn(*d_args)
-            if rc or rc2:
-                capi.check(rc or rc2, "bench planned step")
+        planned_step = make_step(ROTATE, plan=plan)
 
         capi.check(lib.xllm_mi355_profile_enable(1), "profile_enable")
         capi.check(plan_fn(*plan_args), "the plan of the step")
@@ -490,10 +516,8 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             cs = torch.cuda.current_stream(dev).cuda_stream
-            rc = reshape_fn(*(reshape_args[:-1] + (cs,)))
-            rc2 = decode_fn(*(decode_args[:-1] + (cs,)))
-        if rc or rc2:
-            capi.check(rc or rc2, "bench captured step")
+            for fn, fn_args in step_calls(0, one_call):
+                capi.check(fn(*(fn_args[:-1] + (cs,))), "bench captured step")
         t_settle = time.perf_counter()   # (the capture left the GPU idle: let the clocks settle again)
         while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
             for _ in range(20):
@@ -574,11 +598,14 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
             "batch": cfg.batch, "n_q_heads": cfg.n_q_heads, "n_kv_heads": cfg.n_kv_heads,
             "head_dim": cfg.head_dim, "block_size": cfg.block_size,
             "context_tokens": int(lay.seq_lens.sum()), "max_context": max_len,
-            "step": "reshape_and_cache(new K/V rows) + paged decode attention, inputs resident in HBM",
+            "step": ("write_and_decode_gqa: the new K/V rows stored and attended to in one call, inputs resident in HBM"
+                     if one_call else
+                     "reshape_and_cache(new K/V rows) + paged decode attention, inputs resident in HBM"),
         },
         "instrumented_ms_per_step": instrumented_ms_per_step,
         "kv_cache_copies_in_rotation": ROTATE,
         "same_cache": same_cache,
+        "two_calls": two_calls,
         "hbm_gbs_whole_step": (nbytes + workloads.reshape_bytes(
             cfg.batch, cfg.n_kv_heads * cfg.head_dim, 2, 1 if fp8 else 2, 1 if cfg.mla else 2))
             / (ms_per_step * 1e-3) / 1e9,
@@ -637,7 +664,7 @@ def main():
         result = dict(per[HEADLINE])
         result["gate"] = {"workload": "tiny", "parity": gate.get("parity")}
         keep = ("value", "unit", "ms_per_step", "dtype", "config", "hbm_gbs_whole_step", "roofline", "cpu_baseline",
-                "parity", "same_cache", "instrumented_ms_per_step", "kv_cache_copies_in_rotation")
+                "parity", "same_cache", "two_calls", "instrumented_ms_per_step", "kv_cache_copies_in_rotation")
         result["per_config"] = [{k: per[name][k] for k in keep if k in per[name]} for name in ALL]
         if not args.no_cpu_baseline:
             result["parity_all_ok"] = all(per[name]["parity"]["ok"] for name in ALL) and gate["parity"]["ok"]

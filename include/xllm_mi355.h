@@ -277,7 +277,7 @@ int xllm_mi355_paged_decode_gqa_planned(const void* plan, size_t plan_bytes,
  * reference's slot mapping holds on a decode step); negative slots and slots beyond the cache are skipped, and such a
  * sequence attends to whatever its table holds.  The caches and `out` afterwards hold the same bytes as after
  * xllm_mi355_reshape_and_cache followed by the decode call.  Where the matrix-core kernel serves the shape (16-bit or
- * fp8 pages of a power-of-two block size >= 16, head dim 64 / 128, or 256 with 16-bit pages; key / value 16-byte
+ * fp8 pages of a power-of-two block size >= 16, head dim 64 / 128 / 256; key / value 16-byte
  * aligned with strides that are multiples of 8 elements) the rows are written inside the decode launch, by the
  * worker that attends to the context's last tokens, and the step saves a launch; otherwise the library issues the
  * two launches itself.  The caches are written: a sequence with seq_lens[b] == 0 has no token to store and stores

@@ -293,6 +293,19 @@ def test_fp8_kv_cache_decode(device):
     _check_fp8(cfg, 4242, device)
 
 
+def test_head_dim_256_with_fp8_pages_on_the_matrix_core_kernel(device):
+    # rows of 256 bytes: 16 tokens per stage, one score block, the second half of the 32-token P.V masked.  Group
+    # sizes 1, 4, 16 and one with two head blocks; block sizes 16 / 64; contexts from one token to many workers'
+    # worth; lengths around the 16-token boundaries; the dot-product kernel on the same inputs agrees closely.
+    for name, batch, Hq, Hkv, bs, lo, hi in (("g1", 4, 4, 4, 32, 1, 700), ("g4", 5, 16, 4, 16, 1, 3000),
+                                             ("g16", 3, 16, 1, 64, 100, 2500), ("g20", 3, 40, 2, 64, 50, 1200),
+                                             ("long", 3, 8, 2, 16, 10000, 20000)):
+        _check_fp8(workloads.DecodeConfig(f"d256_fp8_{name}", batch, Hq, Hkv, 256, bs, lo, hi, cache_dtype="fp8"),
+                   800 + Hq, device)
+    for L in (1, 15, 16, 17, 31, 32, 33, 48, 65):
+        _check_fp8(workloads.DecodeConfig(f"d256_fp8_L{L}", 2, 8, 2, 256, 16, L, L, cache_dtype="fp8"), 900 + L, device)
+
+
 def test_kv_head_counts_and_the_heads_read_side_by_side(device):
     # The four workers of a workgroup read four adjacent KV heads side by side when the KV heads come in fours
     # (12 = three groups), two when they come in pairs (6, 2), one otherwise (3, 1); contexts long enough to be cut

@@ -21,12 +21,13 @@ CASES = [
     (C("w_d64", 7, 16, 4, 64, 32, 1, 1500), torch.bfloat16),
     (C("w_d64_fp8", 7, 16, 4, 64, 32, 1, 1500, cache_dtype="fp8"), torch.bfloat16),
     (C("w_d256", 6, 8, 2, 256, 32, 1, 1200), torch.bfloat16),
+    (C("w_d256_fp8", 4, 8, 2, 256, 32, 1, 900, cache_dtype="fp8"), torch.bfloat16),
     (C("w_group32", 5, 64, 2, 128, 16, 1, 2000), torch.bfloat16),     # two head blocks per KV head store the same row
     (C("w_bs128", 10, 64, 8, 128, 128, 1, 4000), torch.bfloat16),
     (C("w_long", 3, 32, 8, 128, 16, 20000, 40000), torch.bfloat16),   # contexts cut over many workers
     # served by the other kernels: the library issues the two launches itself
     (C("w_bs8", 6, 32, 8, 128, 8, 1, 700), torch.bfloat16),
-    (C("w_d256_fp8", 4, 8, 2, 256, 32, 1, 900, cache_dtype="fp8"), torch.bfloat16),
+    (C("w_bs24_fp8", 4, 8, 2, 128, 24, 1, 900, cache_dtype="fp8"), torch.bfloat16),
 ]
 
 

@@ -808,7 +808,7 @@ struct MfmaLayout {
 template <typename QT, bool FP8, int NS, bool VL, int D>
 __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   static_assert(NS >= 2 && NS <= 4, "wait_younger_stages covers up to three stages in flight");
-  static_assert(D == 128 || D == 64 || (D == 256 && !FP8), "head dims of the matrix-core loop");
+  static_assert(D == 128 || D == 64 || D == 256, "head dims of the matrix-core loop");
   using Lay = MfmaLayout<NS, D>;
   constexpr int G = kMfmaHeads;
   constexpr int KS = D / 32;               // k-steps of a score block
@@ -820,9 +820,6 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   constexpr int LPR = RB / 16;             // lanes (16-byte chunks) per row in a load instruction
   constexpr int RPI = kWave / LPR;         // rows per load instruction
 
-#ifdef XLLM_GQA_TIMING
-  const unsigned long long t_entry = wall_clock64();
-#endif
   extern __shared__ __align__(16) char smem[];
   int* tmp = reinterpret_cast<int*>(smem + Lay::kTmpOff);
   int* prefix = reinterpret_cast<int*>(smem + Lay::kPrefixOff);
@@ -1016,7 +1013,9 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   // fp8 pages.  K: rows c16 and 16 + c16, 8 bytes of chunk kk*2 + g/2.  V: lane c16 of a 16-lane group
   // addresses 8 dims (8 bytes) of the token in k-slot c16/2 of the group: tokens 4g .. 4g+3, then
   // 16 + 4g .. 16 + 4g+3 -- the order in which the two score blocks leave the P^T registers
-  const int v8_row = ((c16 >> 1) < 4 ? 0 : 12) + 4 * g + (c16 >> 1);
+  // (a 16-token stage, rows of 256 bytes, has one score block: the k-slots of the second repeat the first's tokens
+  // and meet zeros in P^T)
+  const int v8_row = T >= 32 ? ((c16 >> 1) < 4 ? 0 : 12) + 4 * g + (c16 >> 1) : 4 * g + ((c16 >> 1) & 3);
   const int v8_read = T * RB + v8_row * RB + (c16 & 1) * 8;
   const int v8_y = (v8_row & SW8) << 4;
 
@@ -1198,10 +1197,6 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
   }  // loader
 
   // ---- the computing wavefront
-#ifdef XLLM_GQA_TIMING   // (measurement build only) wall-clock stamps of every worker, behind the partials
-  const unsigned long long t_compute = wall_clock64();
-  unsigned long long t_first = 0;
-#endif
   CtxCursor cc;
   locate(cur, cc);
   bool run_start = true;
@@ -1235,9 +1230,6 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
       __builtin_amdgcn_s_sleep(1);
     }
     asm volatile("" ::: "memory");  // no read of the stage moves above the poll
-#ifdef XLLM_GQA_TIMING
-    if (s == 0) t_first = wall_clock64();
-#endif
 
     if (run_start) {  // first stage of a run: the (sequence, head block) changes
       run_start = false;
@@ -1450,21 +1442,28 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
         o[mb] = Mfma<QT>::k32(u32x4{lo[0], lo[1], hi[0], hi[1]}, pb, o[mb]);
       }
     } else {
-      // ---- fp8 pages: the stage's tokens in halves of 32 (one half at head dim 128, two at head dim 64)
+      // ---- fp8 pages: the stage's tokens in halves of 32 (one half at head dim 128, two at head dim 64; the 16 tokens
+      // of a stage at head dim 256 are the first score block of one half whose second block is masked)
+      constexpr int NTB = T >= 32 ? 2 : 1;
 #pragma unroll
-      for (int hf = 0; hf < T / 32; ++hf) {
+      for (int hf = 0; hf < (T >= 32 ? T / 32 : 1); ++hf) {
       const char* sth = st + hf * 32 * RB;
       // scores of the half's 32 tokens, two blocks of 16: lane (head c16, tokens 16 tb + 4g ..)
       float sv[8];
       bool over = false;
 #pragma unroll
       for (int tb = 0; tb < 2; ++tb) {
+        if (tb >= NTB) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sv[tb * 4 + r] = -INFINITY;
+          continue;
+        }
         f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
         const int tok = tb * 16 + c16;
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) {
           const u32x2 k8 = *reinterpret_cast<const u32x2*>(
-              sth + tok * RB + (((kk * 2 + (g >> 1)) ^ (tok & SW8)) * 16) + (g & 1) * 8);
+              sth + tok * RB + (((kk * 2 + (g >> 1)) ^ (tok & (LPR - 1))) * 16) + (g & 1) * 8);
           const u32x4 kr = {QT::template from_fp8x2<false>(k8[0]), QT::template from_fp8x2<true>(k8[0]),
                             QT::template from_fp8x2<false>(k8[1]), QT::template from_fp8x2<true>(k8[1])};
           sc = Mfma<QT>::k32(kr, q[kk], sc);
@@ -1596,15 +1595,6 @@ __global__ __launch_bounds__(kMfmaThreads) void gqa_mfma_kernel(GqaArgs a) {
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#ifdef XLLM_GQA_TIMING
-  if (lane == 0) {
-    unsigned long long* dst = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_workgroups) * 2 * G) + worker * 4;
-    dst[0] = t_entry;
-    dst[1] = t_compute;
-    dst[2] = t_first;
-    dst[3] = wall_clock64();
-  }
-#endif
   // ---- the pieces this worker wrote as partials: the worker that brings a context's last piece merges them.
   // One counter per context that spans workers, kept with the worker in whose range it starts (at most one
   // such context per worker); atomicInc wraps it back to zero with the last arrival.  The partials were
@@ -2024,10 +2014,11 @@ int dispatch_group(GqaArgs& a, size_t wsb, hipStream_t s, bool plan_only, size_t
 }
 
 // Whether the matrix-core kernel serves a one-query-token call (its epilogue stores 8 output bytes at a time; its
-// stages are whole parts of a page of a power-of-two size from 16 tokens on; fp8 rows of 256 bytes have no loop there).
+// stages are whole parts of a page of a power-of-two size from 16 tokens on).
 bool mfma_serves(const GqaArgs& a, bool fp8, int head_dim) {
+  (void)fp8;
   const bool out_aligned = (reinterpret_cast<uintptr_t>(a.out) & 7) == 0 && (a.out_stride_bytes & 7) == 0;
-  const bool dim_ok = head_dim == 64 || head_dim == 128 || (head_dim == 256 && !fp8);
+  const bool dim_ok = head_dim == 64 || head_dim == 128 || head_dim == 256;
   return dim_ok && a.bs_shift >= 4 && out_aligned && use_mfma_kernel();
 }
 
@@ -2038,6 +2029,7 @@ int dispatch_dim(GqaArgs& a, int head_dim, size_t wsb, hipStream_t s, bool plan_
   if constexpr (FP8) {
     if (head_dim == 128 && mfma) return launch_gqa_mfma<QT, true>(a, wsb, s, plan_only, need);
     if (head_dim == 64 && mfma) return launch_gqa_mfma<QT, true, false, 64>(a, wsb, s, plan_only, need);
+    if (head_dim == 256 && mfma) return launch_gqa_mfma<QT, true, false, 256>(a, wsb, s, plan_only, need);
     switch (head_dim) {
       case 64: return dispatch_group<QT, true, 64, 4, 2>(a, wsb, s, plan_only, need);
       case 128: return dispatch_group<QT, true, 128, 8, 2>(a, wsb, s, plan_only, need);
@@ -2182,7 +2174,7 @@ int paged_decode_gqa_plan(void* plan, size_t plan_bytes, const PageAddressing& a
     if ((1LL << s) == block_size) a.bs_shift = s;
   // Shapes that the matrix-core kernel does not serve, and batches decoded in slices, take no plan: the planned
   // entry point decodes them like the plain one.
-  if (batch > kMaxBatch || a.bs_shift < 4 || (fp8 && head_dim == 256) || !use_mfma_kernel()) return XLLM_MI355_OK;
+  if (batch > kMaxBatch || a.bs_shift < 4 || !use_mfma_kernel()) return XLLM_MI355_OK;
   configure_mfma(a, fp8, static_cast<int>(head_dim), false);
   const int n_teams = a.n_workgroups / a.head_lock;
   if (a.fold_merge != 0 || n_teams > kPlanMaxTeams) return XLLM_MI355_OK;

@@ -1,5 +1,18 @@
 // Paged decode attention, MLA latent-KV variant, for gfx950.
 //
+// Four decode kernels live here, each with shapes that no other serves (paged_decode_mla at the end of the file picks):
+//   mla_decode_w4_kernel   more than 64 heads, block size a power of two >= 16: the full-model shape (128 heads).  One
+//                          workgroup holds O^T of 128 heads in its accumulation registers.  The default there.
+//   mla_decode_ds_kernel   the same shapes with 16 heads per MFMA block and O^T by dim block in ordinary registers:
+//                          what the build switches those shapes to when the compiler's resource report shows that the
+//                          fixed accumulation registers of mla_decode_w4_kernel are not left alone (build.py), and
+//                          XLLM_MI355_MLA_KERNEL=narrow by hand.
+//   mla_decode16_kernel    up to 64 heads (the heads of a tensor-parallel shard: 16 per MFMA block), same block sizes.
+//                          (With more heads only under XLLM_MI355_MLA_KERNEL=heads, for comparison.)
+//   mla_decode_kernel      every other block size (below 16, or not a power of two): whole 64-token tiles gathered row
+//                          by row.  Described first, below; the others say where they differ.
+// mla_merge_tiles_kernel folds the partial pieces of mla_decode_w4_kernel, mla_merge_kernel those of the others.
+//
 // All query heads share ONE latent KV head of 576 dims (512 latent + 64 rope); V is the
 // first 512 dims of the same rows.  With up to 128 heads per sequence the two products are
 // dense contractions, so they run on MFMA (v_mfma_f32_32x32x16_bf16):
@@ -526,10 +539,6 @@ __device__ __forceinline__ void wait_younger_subs(int subs) {
 // theirs to their partners through the (then idle) ring, merged like two partials.
 template <typename QT, bool SPLIT>
 __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
-#ifdef XLLM_DS_TIMING
-  const unsigned long long w_entry16 = wall_clock64();
-  const unsigned long long t_entry16 = __builtin_readcyclecounter();
-#endif
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kPrefix16Off);
   const int* pagebuf = reinterpret_cast<const int*>(smem + kPage16Off);
@@ -895,16 +904,6 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
     if (writer && g == 0 && !complete) a.ws_lse[ps] = lse2;
     first_run = false;
   }
-#ifdef XLLM_DS_TIMING
-  if ((threadIdx.x & 63) == 0) {
-    unsigned long long* dst = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * a.n_heads) +
-                              (blockIdx.x * 8 + (threadIdx.x >> 6)) * 10;
-    dst[0] = w_entry16;
-    dst[1] = wall_clock64();
-    dst[8] = __builtin_readcyclecounter() - t_entry16;
-    dst[9] = (dst[1] - dst[0]) << 32;
-  }
-#endif
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -934,9 +933,6 @@ __global__ __launch_bounds__(kThreads16) void mla_decode16_kernel(MlaArgs a) {
 // wavefront rescales that head block's accumulators before it adds the sub-tile.  At the end of a run the
 // owners publish 1 / sum and every wavefront writes its dims.
 // LDS: ring [3 sub-tiles] | P^T [2][8 blocks] | factors [2][128] | flags [3] | page chunks [2][64] | prefix.
-#ifndef XLLM_DS_AHEAD
-#define XLLM_DS_AHEAD 2
-#endif
 constexpr int kDsRing = 3;
 constexpr int kDsPOff = kDsRing * kSubBytes;               // P^T blocks: [2][8][64 lanes][16 bytes]
 constexpr int kDsFacOff = kDsPOff + 2 * 8 * 1024;          // [2][128] rescale factors of a sub-tile; [128] 1 / sum at the end
@@ -950,10 +946,6 @@ static_assert(kDsLdsBytes <= 160 * 1024, "LDS of a CU");
 
 template <typename QT>
 __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
-#ifdef XLLM_DS_TIMING
-  const unsigned long long t_entry = __builtin_readcyclecounter();
-  const unsigned long long w_entry = wall_clock64();
-#endif
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kDsPrefixOff);
   const int* pagebuf = reinterpret_cast<const int*>(smem + kDsPageOff);
@@ -967,11 +959,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
   const int c16 = lane & 15;    // MFMA row / column index owned by the lane
   const int g = lane >> 4;      // MFMA k-group of the lane
   const int H = a.n_heads;
-#ifdef XLLM_DS_SAME_ORDER
-  constexpr bool pv_first = true;
-#else
   const bool pv_first = wave < 4;  // order of the two jobs between barriers (the SIMD's other wavefront has the other)
-#endif
 
   // block id -> (team, head block of 128): members of a team are 8 ids apart (same XCD)
   const int xcd = blockIdx.x & 7;
@@ -1032,16 +1020,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
     return static_cast<int>(x >> 4) ^ (wave & 1);
   };
 
-#ifdef XLLM_DS_TIMING
-  unsigned long long tm[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  unsigned long long tk = __builtin_readcyclecounter();
-  const unsigned long long t_start = t_entry;
-  const unsigned long long w_start = w_entry;
-  tm[7] += tk - t_entry;   // (the time before the first run is booked as epilogue)
-#define DS_TICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; }
-#else
 #define DS_TICK(i)
-#endif
   while (cur < end) {
     int lo = 0, hi = a.batch;
     while (hi - lo > 1) {
@@ -1133,7 +1112,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
       // K operands kDsAhead k-steps ahead of the MFMAs that take them, in an order the scheduler may not change:
       // left to itself it puts every read right in front of its MFMA, and a k-step then costs a whole LDS round
       // trip (about 120 cycles against the 32 of its two MFMAs).
-      constexpr int kDsAhead = XLLM_DS_AHEAD;
+      constexpr int kDsAhead = 2;
       auto k_addr = [&](int kk) -> const char* {
         return kk < kDL / 32 ? ka + kk * 64 : kr + (kk == kDL / 32 ? kr_x : kr_x ^ 4) * 16;
       };
@@ -1147,18 +1126,9 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps32; ++kk) {
         __builtin_amdgcn_sched_barrier(0);
-#ifdef XLLM_DS_WHATIF_NO_QK_MFMA   // (measurement only: wrong results)
-        s0[0] += as_f32(xa[kk % kDsAhead][0]);
-        s1[0] += as_f32(xb[kk % kDsAhead][0]);
-#else
         s0 = Mfma<QT>::k32(xa[kk % kDsAhead], q[kk], s0);
         s1 = Mfma<QT>::k32(xb[kk % kDsAhead], q[kk], s1);
-#endif
-#ifdef XLLM_DS_WHATIF_NO_K_READS   // (measurement only: wrong results)
-        if (false) {
-#else
         if (kk + kDsAhead < kKSteps32) {
-#endif
           const int kn = kk + kDsAhead;
           xa[kk % kDsAhead] = *reinterpret_cast<const u32x4*>(k_addr(kn));
           xb[kk % kDsAhead] = *reinterpret_cast<const u32x4*>(k_addr(kn) + 16 * (kn < kDL / 32 ? kRow16 : kDR * 2));
@@ -1367,19 +1337,6 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
     first_run = false;
     DS_TICK(7)   // run epilogue
   }
-#ifdef XLLM_DS_TIMING
-  // (measurement build only) per-phase cycle sums of every wavefront of every workgroup, behind the partials
-  if (lane == 0) {
-    unsigned long long* dst = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H) +
-                              (blockIdx.x * 8 + wave) * 10;
-    for (int i = 0; i < 8; ++i) dst[i] = tm[i];
-    dst[0] = w_entry;            // (absolute 100 MHz time stamps of entry and exit instead of two of the sums)
-    dst[1] = wall_clock64();
-    dst[8] = __builtin_readcyclecounter() - t_start;
-    dst[9] = static_cast<unsigned long long>(end - team_start(team, total, a.n_teams)) |
-             ((wall_clock64() - w_start) << 32);   // high half: the same span on the constant 100 MHz clock
-  }
-#endif
 #undef DS_TICK
 }
 
@@ -1651,10 +1608,7 @@ __device__ __forceinline__ void mla_write_empty(const MlaArgs& a, int hb, int b,
 // then the rope parts.  The small arrays sit behind them.
 // What the schedule of mla_decode_w4_kernel divides: sub-tiles.  The loop runs sub-tile by sub-tile, so a range may
 // end at any of them, and the workgroups' shares differ by one sub-tile at most instead of one 64-token tile.
-#ifndef XLLM_W4_ITEM
-#define XLLM_W4_ITEM 32
-#endif
-constexpr int kW4Item = XLLM_W4_ITEM;
+constexpr int kW4Item = 32;
 constexpr int kW4QRow = kDL * 2 + 16;
 constexpr int kW4QRopeOff = kHeadsPerWg16 * kW4QRow;
 constexpr int kW4QEnd = kW4QRopeOff + kHeadsPerWg16 * kDR * 2;
@@ -1671,9 +1625,6 @@ constexpr int kFoldRegion = 2 * (4 * 4096 + 1024);
 constexpr int kFoldSeenOff = kWsMaxWorkers / 2;
 static_assert(4 * kFoldRegion <= kW4FacOff, "the fold's LDS lies in front of the factors, flags and the prefix");
 static_assert(kW4LdsBytes <= 160 * 1024, "LDS of a CU");
-#ifndef XLLM_W4_AHEAD
-#define XLLM_W4_AHEAD 3
-#endif
 
 // The prefix over the batch of what mla_decode_w4_kernel's schedule divides (sub-tiles, and run_cost more at the front of
 // every context that holds tokens) into prefix[0 .. batch] (LDS), by 256 threads; tmp: 4 words of LDS.
@@ -1744,22 +1695,8 @@ __global__ __launch_bounds__(kW4Threads) void mla_plan_kernel(MlaArgs a, int* pl
 
 template <typename QT>
 __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
-#ifdef XLLM_DS_TIMING
-  const unsigned long long t_entry = __builtin_readcyclecounter();
-  const unsigned long long w_entry = wall_clock64();
-  unsigned long long tm[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  unsigned long long tk = t_entry;
-#ifdef XLLM_W4_PROLOGUE_TIMING   // (slots 2-6 hold parts of the run prologue instead of the loop's phases)
-#define W4_PTICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; }
-#define W4_TICK(i) { if (i < 2 || i > 6) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; } }
-#else
-#define W4_PTICK(i)
-#define W4_TICK(i) { const unsigned long long now_ = __builtin_readcyclecounter(); tm[i] += now_ - tk; tk = now_; }
-#endif
-#else
 #define W4_TICK(i)
 #define W4_PTICK(i)
-#endif
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kW4PrefixOff);
   const int* pagebuf = reinterpret_cast<const int*>(smem + kW4PageOff);
@@ -1955,9 +1892,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       const uint64_t cache = reinterpret_cast<uint64_t>(a.k_cache);
       int page = __builtin_amdgcn_readfirstlane(page_read);
       page = max(0, min(page, a.num_blocks - 1));
-#ifdef XLLM_W4_WHATIF_ONE_PAGE   // (measurement only: wrong results) every tile from the same pages: the loads hit in L2
-      page = page & 7;
-#endif
       const uint64_t row = cache + static_cast<uint64_t>(page * a.block_size + (tb & (a.block_size - 1))) * kRowBytes;
       const u32 rlo = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row)));
       const u32 rhi = static_cast<u32>(__builtin_amdgcn_readfirstlane(static_cast<u32>(row >> 32)));
@@ -1986,16 +1920,13 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     // all but the youngest `subs` sub-tiles this wavefront has sent are in LDS
     auto wait_sent = [&](int subs) {
       static_assert(kW4Loads == 9, "the immediates below are multiples of the loads per sub-tile");
-#ifdef XLLM_W4_WHATIF_NO_WAIT   // (measurement only: wrong results)
-      return;
-#endif
       if (subs <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       else if (subs == 1) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
     };
 
     // ---- S^T of sub-tile `sub` for the wavefront's 32 heads: s[j][tb] = tokens 16 tb + 4g + r, head 16 j + c16
-    constexpr int kAheadW = XLLM_W4_AHEAD;
+    constexpr int kAheadW = 3;
     // the K operands of the first kAheadW k-steps of sub-tile `sub` (its rows have landed): sent for before the first
     // half of P.V, so that the scores start on operands that are there
     auto scores_begin = [&](int sub, u32x4 (&xa)[kAheadW], u32x4 (&xb)[kAheadW]) {
@@ -2026,20 +1957,11 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps32; ++kk) {
         __builtin_amdgcn_sched_barrier(0);
-#ifdef XLLM_W4_WHATIF_NO_QK_MFMA   // (measurement only: wrong results)
-        s[0][0][0] += as_f32(xa[kk % kAheadW][0]);
-        s[0][1][0] += as_f32(xb[kk % kAheadW][0]);
-#else
         Mfma<QT>::k32_v(xa[kk % kAheadW], q[0][kk], s[0][0]);
         Mfma<QT>::k32_v(xa[kk % kAheadW], q[1][kk], s[1][0]);
         Mfma<QT>::k32_v(xb[kk % kAheadW], q[0][kk], s[0][1]);
         Mfma<QT>::k32_v(xb[kk % kAheadW], q[1][kk], s[1][1]);
-#endif
-#ifdef XLLM_W4_WHATIF_NO_K_READS   // (measurement only: wrong results)
-        if (false) {
-#else
         if (kk + kAheadW < kKSteps32) {
-#endif
           const int kn = kk + kAheadW;
           xa[kk % kAheadW] = *reinterpret_cast<const u32x4*>(k_addr(kn));
           xb[kk % kAheadW] = *reinterpret_cast<const u32x4*>(k_addr(kn) + 16 * (kn < kDL / 32 ? kRow16 : kDR * 2));
@@ -2356,12 +2278,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     }
 
     // ---- end of the run: the owners publish 1 / sum per head, every wavefront writes its dims of every head
-#ifdef XLLM_DS_TIMING
-    unsigned long long fold_t[5] = {static_cast<unsigned long long>(wall_clock64()), 0, 0, 0, 0};
-#define W4_FOLD_MARK(i) fold_t[i] = static_cast<unsigned long long>(wall_clock64());
-#else
-#define W4_FOLD_MARK(i)
-#endif
     const float lsum0 = quad_rows_sum(l[0]), lsum1 = quad_rows_sum(l[1]);
     const int64_t slot_id = static_cast<int64_t>(team) * 2 + (first_run ? 0 : 1);
     const int64_t ps_base = slot_id * H;
@@ -2465,10 +2381,8 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       if (team == pc.t_last) {
         pending = counter;   // announced once its stores have landed: after the next run's wait, or at the kernel's end
       } else {
-        W4_FOLD_MARK(1)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();   // every wavefront's stores have landed
-        W4_FOLD_MARK(2)
         if (tid == 0) {
           if (pending >= 0) announce(pending);
           announce(counter);
@@ -2484,7 +2398,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
         }
         pending = -1;
         __syncthreads();
-        W4_FOLD_MARK(3)
         if (flags[3] != 0) {
           mla_fold_stream<QT>(a, pc, b, hb128 * 8, jf, nf, n16, wave, lane_again(),
                               smem + wave * kFoldRegion, lds_base + wave * kFoldRegion);
@@ -2495,18 +2408,8 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
               __hip_atomic_store(a.ws_written + counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
         }
-        W4_FOLD_MARK(4)
-#ifdef XLLM_DS_TIMING
-        if (lane == 0) {   // (measurement build only) the fold's time stamps, behind the phase sums
-          unsigned long long* ft = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H) +
-                                   4096 * 12 + (blockIdx.x * 4 + wave) * 8;
-          for (int i = 0; i < 5; ++i) ft[i] = fold_t[i];
-          ft[5] = static_cast<unsigned long long>(pc.count);
-        }
-#endif
       }
     }
-#undef W4_FOLD_MARK
     first_run = false;
     W4_TICK(7)   // run epilogue
   }
@@ -2515,18 +2418,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     __syncthreads();
     if (tid == 0) announce(pending);
   }
-#ifdef XLLM_DS_TIMING
-  // (measurement build only) per-phase cycle sums of every wavefront of every workgroup, behind the partials
-  if (lane == 0) {
-    unsigned long long* dst = reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H) +
-                              (blockIdx.x * 4 + wave) * 12;
-    for (int i = 0; i < 8; ++i) dst[i] = tm[i];
-    dst[8] = __builtin_readcyclecounter() - t_entry;
-    dst[9] = static_cast<unsigned long long>(end - team_start(team, total, n_use));
-    dst[10] = w_entry;
-    dst[11] = wall_clock64();
-  }
-#endif
 #undef W4_TICK
 #undef W4_PTICK
 }
@@ -2542,10 +2433,6 @@ __global__ __launch_bounds__(128) void mla_merge_kernel(MlaArgs a) {
   const int b = blockIdx.y;
   const int H = a.n_heads;
   const int d = threadIdx.x * 4;
-#ifdef XLLM_DS_TIMING
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)   // (measurement build only) when the merge kernel starts
-    reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * H)[2048 * 10] = wall_clock64();
-#endif
   const int64_t first = a.ws_prefix[b];
   const int64_t last = static_cast<int64_t>(a.ws_prefix[b + 1]) - 1;
   const int64_t total = a.ws_prefix[a.batch];
@@ -2610,10 +2497,6 @@ __global__ __launch_bounds__(256) void mla_merge_tiles_kernel(MlaArgs a) {
   const int b = blockIdx.y;
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
-#ifdef XLLM_DS_TIMING
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)   // (measurement build only) when the merge kernel starts
-    reinterpret_cast<unsigned long long*>(a.ws_lse + static_cast<size_t>(a.n_teams) * 2 * a.n_heads)[2048 * 10] = wall_clock64();
-#endif
   if (a.plan != nullptr && a.plan[0] != a.plan_sig) return;   // the decode kernel wrote nothing and raised the flag
   MlaPieces p;
   if (!mla_locate_pieces(a, a.ws_prefix[b], a.ws_prefix[b + 1], a.ws_prefix[a.batch], p)) {  // empty sequence
