@@ -45,7 +45,7 @@ def parse_args():
                     help="untimed run of the step before the warm-up steps, until the clocks have settled")
     ap.add_argument("--workload", default="all",
                     help="all (default) | tiny | llama3_8b | long_b256 | fp8_kv | mla_dsv3 (the five configurations); "
-                         "gqa_d64 | gqa_d64_fp8 | gqa_d256 | mla_tp8 (side workloads)")
+                         "gqa_d64 | gqa_d64_fp8 | gqa_d256 | gqa_d256_fp8 | mla_tp8 (side workloads)")
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU baseline (and with it the parity check)")
     ap.add_argument("--no-planned", action="store_true",
@@ -304,7 +304,7 @@ def decode_kernel_name(cfg):
         if knob == "h" or cfg.n_q_heads <= 64:
             return "mla_decode16_kernel"
         return "mla_decode_ds_kernel" if knob == "n" else "mla_decode_w4_kernel"
-    mfma = (cfg.head_dim in (64, 128) or (cfg.head_dim == 256 and cfg.cache_dtype != "fp8")) and cfg.block_size >= 16 \
+    mfma = cfg.head_dim in (64, 128, 256) and cfg.block_size >= 16 \
         and cfg.block_size & (cfg.block_size - 1) == 0 and os.environ.get("XLLM_MI355_GQA_KERNEL", "")[:1] != "r"
     return "gqa_mfma_kernel" if mfma else "gqa_decode_kernel"
 

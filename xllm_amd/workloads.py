@@ -49,6 +49,7 @@ CONFIGS = {
     "gqa_d64": DecodeConfig("gqa_d64", 64, 32, 8, 64, 16, 1024, 8192),
     "gqa_d256": DecodeConfig("gqa_d256", 64, 16, 4, 256, 16, 512, 4096),
     "gqa_d64_fp8": DecodeConfig("gqa_d64_fp8", 64, 32, 8, 64, 16, 2048, 16384, cache_dtype="fp8"),
+    "gqa_d256_fp8": DecodeConfig("gqa_d256_fp8", 64, 16, 4, 256, 16, 1024, 8192, cache_dtype="fp8"),
     "mla_tp8": DecodeConfig("mla_tp8", 64, 16, 1, 576, 64, 2048, 16384, mla=True, v_dim=512,
                             sigma=0.5, sm_scale=1.0 / math.sqrt(192.0)),
 }
