@@ -1020,7 +1020,6 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
     return static_cast<int>(x >> 4) ^ (wave & 1);
   };
 
-#define DS_TICK(i)
   while (cur < end) {
     int lo = 0, hi = a.batch;
     while (hi - lo > 1) {
@@ -1249,23 +1248,17 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
       // ---- wavefronts 0-3: P.V of `sub`, then the scores of sub + 1; the V^T operands wait in registers
       u32x4 vt[4];  // V^T operands of the sub-tile whose P.V comes next: dims 64 wave + 16 db .., its 32 tokens
       read_vt(0, vt);
-      DS_TICK(0)   // run prologue
       for (int sub = 0; sub < n_sub; ++sub) {
         // the wavefront's rows of sub-tile sub + 1 have landed (sub + 2 may still be in flight)
         wait_younger_subs(min(kDsRing - 2, n_sub - 2 - sub));
-        DS_TICK(1)
         __syncthreads();  // P^T of `sub` is complete; sub + 1 has landed; nobody reads sub-tile `sub` in LDS any more
-        DS_TICK(2)
         if (tid == 0) flags[(sub + 2) % 3] = 0;   // (last read before this barrier, next raised after the next one)
         if (sub + kDsRing < n_sub) issue_sub(sub + kDsRing);
-        DS_TICK(3)
         pv(sub, vt);
-        DS_TICK(6)
         if (sub + 1 < n_sub) {
           scores(sub + 1);
           read_vt(sub + 1, vt);
         }
-        DS_TICK(4)
       }
     } else {
       // ---- wavefronts 4-7: the scores of sub + 1, then P.V of `sub`.  They park the V^T operands (read while the
@@ -1277,17 +1270,12 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
 #pragma unroll
         for (int db = 0; db < 4; ++db) *reinterpret_cast<u32x4*>(stash + db * 1024) = vt[db];
       }
-      DS_TICK(0)
       for (int sub = 0; sub < n_sub; ++sub) {
         wait_younger_subs(min(kDsRing - 2, n_sub - 2 - sub));
-        DS_TICK(1)
         __syncthreads();
-        DS_TICK(2)
         const bool more = sub + 1 < n_sub;
         if (more) scores(sub + 1);
-        DS_TICK(4)
         if (sub + kDsRing < n_sub) issue_sub(sub + kDsRing);
-        DS_TICK(3)
         u32x4 vt[4];
 #pragma unroll
         for (int db = 0; db < 4; ++db) vt[db] = *reinterpret_cast<const u32x4*>(stash + db * 1024);
@@ -1297,7 +1285,6 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
 #pragma unroll
           for (int db = 0; db < 4; ++db) *reinterpret_cast<u32x4*>(stash + db * 1024) = vt[db];
         }
-        DS_TICK(6)
       }
     }
 
@@ -1335,9 +1322,7 @@ __global__ __launch_bounds__(kThreads16) void mla_decode_ds_kernel(MlaArgs a) {
       }
     }
     first_run = false;
-    DS_TICK(7)   // run epilogue
   }
-#undef DS_TICK
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1695,8 +1680,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_plan_kernel(MlaArgs a, int* pl
 
 template <typename QT>
 __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
-#define W4_TICK(i)
-#define W4_PTICK(i)
   extern __shared__ __align__(16) char smem[];
   int* prefix = reinterpret_cast<int*>(smem + kW4PrefixOff);
   const int* pagebuf = reinterpret_cast<const int*>(smem + kW4PageOff);
@@ -1787,7 +1770,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     return static_cast<int>(x >> 4);
   };
 
-  W4_TICK(0)   // kernel prologue (tile prefix)
   while (cur < end) {
     int lo = 0, hi = a.batch;
     while (hi - lo > 1) {
@@ -1828,7 +1810,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     const int lane_p = lane_again();
     const int c16p = lane_p & 15, gp = lane_p >> 4;
     if (wave == 0 && lane_p < 3) flags[lane_p] = 0;
-    W4_PTICK(2)   // search, barrier, chunk loads issued
 
     // Q^T operands of the two 16-head blocks: lane (head c16, k-group g) keeps dims kk*32 + g*8 .. +8 of every k-step.
     // The rows of the wavefront's 32 heads travel through LDS, 36 loads of 1 KB (whole rows) and then 72 LDS reads per
@@ -2175,7 +2156,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       pb[1] = *reinterpret_cast<const u32x4*>(pbase + 1024);
     };
 
-    W4_PTICK(3)   // Q loads issued, accumulators cleared
     // the chunk loads and the Q rows have landed (one wait for both latencies); the wavefront reads the rows it sent
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
@@ -2192,12 +2172,9 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       if (tid == 0) announce(pending);
       pending = -1;
     }
-    W4_PTICK(4)   // Q and chunks landed, barrier
     for (int sub = 0; sub < kDsRing && sub < n_sub; ++sub) issue_sub(sub);
-    W4_PTICK(5)   // three sub-tiles issued
     wait_sent(min(kDsRing - 1, n_sub - 1));
     __syncthreads();
-    W4_PTICK(6)   // first sub-tile landed, barrier
     u32x4 vt[8];  // V^T operands of the sub-tile whose P.V comes next: dims 128 wave + 16 db .., its 32 tokens
     {
       f32x4 s[2][2];
@@ -2215,15 +2192,12 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     sd.last = 0;
     sd.dst = sd.dst_rope = 0;
     if (sends) issue_prepare(kDsRing, sd);
-    W4_TICK(1)   // run prologue
     for (int sub = 0; sub < n_sub; ++sub) {
       const bool more = sub + 1 < n_sub;
       // the wavefront's rows of sub-tile sub + 1 have landed (sub + 2 may still be in flight)
       wait_sent(min(kDsRing - 2, n_sub - 2 - sub));
       __syncthreads();  // P^T of `sub` is complete; sub + 1 has landed; nobody reads sub-tile `sub` in LDS any more
-      W4_TICK(2)
       if (tid == 0) flags[(sub + 2) % 3] = 0;   // (last read before this barrier, next raised after the next one)
-      W4_TICK(3)
       using I0 = std::integral_constant<int, 0>;
       using I1 = std::integral_constant<int, 1>;
       using I2 = std::integral_constant<int, 2>;
@@ -2247,12 +2221,10 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       // ---- first half of P.V of `sub` (dim blocks 0-3), with the loads of sub + 3
       if (sends) pv_rows(I0{}, I0{}, I0{}, I8{}, std::true_type{}, sub, vt, sd, pb, sc, sv, top, sends_next, page_read, &sd_next);
       else pv_rows(I0{}, I0{}, I0{}, I8{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top, sends_next, page_read, &sd_next);
-      W4_TICK(4)
       if (more) {
         u32x4 xa[kAheadW], xb[kAheadW];
         scores_begin(sub + 1, xa, xb);
         scores(sub + 1, sc, xa, xb);
-        W4_TICK(5)
         // ---- second half of P.V of `sub` (dim blocks 4-7) with the softmax of sub + 1 in the shadow of its MFMAs
         pv_again(sub, pb);
         pv_rows(I1{}, I1{}, I0{}, I3{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top);
@@ -2265,7 +2237,6 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
           probabilities(sub + 1, sv);
         }
         read_vt(sub + 1, vt);
-        W4_TICK(6)
       } else {   // (the last sub-tile of a run sends nothing: sub + 3 is past its end)
         pv_again(sub, pb);
         pv_rows(I1{}, I0{}, I0{}, I8{}, std::false_type{}, sub, vt, sd, pb, sc, sv, top);
@@ -2411,15 +2382,12 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
       }
     }
     first_run = false;
-    W4_TICK(7)   // run epilogue
   }
   if (pending >= 0) {   // a piece stored by this workgroup's last run that it does not merge itself
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) announce(pending);
   }
-#undef W4_TICK
-#undef W4_PTICK
 }
 
 // Merge of the partials of contexts that span several teams; also writes the output of
