@@ -149,6 +149,64 @@ def test_one_call_with_csr_addressing_and_strided_rows(device):
     assert torch.isfinite(out_b.float()).all()
 
 
+def _pair_and_one_call(inp, device, dtype, fp8, slots, **kw):
+    cfg, lay = inp.cfg, inp.layout
+    kc0, vc0, ks, vs, store = _caches_before_the_step(inp, device, fp8, dtype)
+    q = inp.q.to(device)
+    k_new, v_new = inp.k_new.to(device), inp.v_new.to(device)
+    table, lens = lay.block_table.to(device), lay.seq_lens.to(device)
+    kc_a, vc_a = kc0.clone(), vc0.clone()
+    store(ops.ReshapePagedCacheParams(key=k_new, value=v_new, k_cache=kc_a, v_cache=vc_a, slot_mapping=slots,
+                                      k_cache_scale=ks, v_cache_scale=vs))
+    out_a, lse_a = ops.batch_decode(q, kc_a, torch.full_like(q, float("nan")), table, lens, v_cache=vc_a,
+                                    k_cache_quant_scale=ks, v_cache_quant_scale=vs, scale=cfg.scale, return_lse=True, **kw)
+    kc_b, vc_b = kc0.clone(), vc0.clone()
+    out_b, lse_b = ops.batch_decode(q, kc_b, torch.full_like(q, float("nan")), table, lens, v_cache=vc_b,
+                                    k_cache_quant_scale=ks, v_cache_quant_scale=vs, scale=cfg.scale, return_lse=True,
+                                    new_key=k_new, new_value=v_new, slot_mapping=slots, **kw)
+    torch.cuda.synchronize()
+    ops.decode_status(device)
+    assert torch.equal(_bits(kc_a), _bits(kc_b)) and torch.equal(_bits(vc_a), _bits(vc_b)), cfg.name
+    return out_a, lse_a, out_b, lse_b
+
+
+def test_one_call_with_a_sliding_window_fp16_over_fp8_and_slots_beyond_the_cache(device):
+    # a window (the first scheduled stage of a context is not its first)
+    cfg = C("w_window", 9, 32, 8, 128, 16, 1, 2500)
+    inp = workloads.make_inputs(cfg, 31)
+    slots = inp.layout.new_slots.to(device)
+    out_a, lse_a, out_b, lse_b = _pair_and_one_call(inp, device, torch.bfloat16, False, slots, window_left=300)
+    assert torch.equal(_bits(out_a), _bits(out_b)) and torch.equal(lse_a, lse_b)
+    assert torch.isfinite(out_b.float()).all()
+    # an fp16 query over fp8 pages: the rows are quantised from fp16 inside the decode launch
+    cfg = C("w_fp16_fp8", 7, 16, 4, 128, 32, 1, 1800, cache_dtype="fp8")
+    inp = workloads.make_inputs(cfg, 32, dtype=torch.float16)
+    slots = inp.layout.new_slots.to(device)
+    out_a, lse_a, out_b, lse_b = _pair_and_one_call(inp, device, torch.float16, True, slots)
+    assert torch.equal(_bits(out_a), _bits(out_b)) and torch.equal(lse_a, lse_b)
+    assert torch.isfinite(out_b.float()).all()
+    # a slot beyond the cache is skipped like a negative one (the caches stay equal; that sequence attends to the NaN row)
+    cfg = C("w_beyond", 6, 32, 8, 128, 16, 20, 900)
+    inp = workloads.make_inputs(cfg, 33)
+    slots = inp.layout.new_slots.to(device).clone()
+    slots[4] = inp.layout.num_blocks * cfg.block_size + 5
+    out_a, lse_a, out_b, lse_b = _pair_and_one_call(inp, device, torch.bfloat16, False, slots)
+    live = torch.ones(cfg.batch, dtype=torch.bool, device=device)
+    live[4] = False
+    assert torch.equal(_bits(out_a[live]), _bits(out_b[live])) and torch.equal(lse_a[live], lse_b[live])
+    assert torch.isfinite(out_b[live].float()).all()
+
+
+def test_one_call_on_a_batch_decoded_in_slices(device):
+    # more sequences than one launch takes: every slice stores the rows of its own sequences
+    cfg = C("w_slices", 2100, 4, 1, 128, 16, 1, 40)
+    inp = workloads.make_inputs(cfg, 34)
+    slots = inp.layout.new_slots.to(device)
+    out_a, lse_a, out_b, lse_b = _pair_and_one_call(inp, device, torch.bfloat16, False, slots)
+    assert torch.equal(_bits(out_a), _bits(out_b)) and torch.equal(lse_a, lse_b)
+    assert torch.isfinite(out_b.float()).all()
+
+
 def test_one_call_rejects_missing_rows(device):
     lib = capi.lib()
     fake = 1 << 20
