@@ -241,7 +241,12 @@ def test_fused_qk_norm_rope_and_its_cache_write(device):
              # prefill sizes, where a lane group takes four (token, head) units: unit counts that are not multiples of
              # four, head counts that let a group straddle two tokens
              (4999, 11, 3, 3, 128, 128, torch.bfloat16, torch.float32, False),
-             (4501, 13, 2, 2, 64, 64, torch.float16, torch.float32, True))
+             (4501, 13, 2, 2, 64, 64, torch.float16, torch.float32, True),
+             # ... with 128-dim heads a unit is 16 lanes of 16 bytes there: groups of one token (48 heads), a partial
+             # rotary dim in both pair layouts, and one whose halves are not whole 16-byte pieces (32 lanes again)
+             (1400, 32, 8, 8, 128, 64, torch.bfloat16, torch.float32, True),
+             (1400, 32, 8, 8, 128, 32, torch.float16, torch.float16, False),
+             (1400, 32, 8, 8, 128, 8, torch.bfloat16, torch.float32, False))
     for T, n_q, n_k, n_v, D, rd, dt, cdt, inter in cases:
         qkv = (torch.randn(T, (n_q + n_k + n_v) * D, generator=g) * 0.3).to(dt)
         qw, kw = (1 + 0.2 * torch.randn(D, generator=g)).to(dt), (1 + 0.2 * torch.randn(D, generator=g)).to(dt)
