@@ -293,8 +293,8 @@ int launch_rope(const RopeArgs& a, bool interleave, bool fp8, hipStream_t stream
   // one unit per group while that still gives every CU several workgroups (decode), four beyond (eight, with the
   // registers they take, measured slower: 57.7 us against 50.3 us on 8192 tokens of 48 heads; sixteen lanes of 16 bytes
   // per unit instead of 32 of 8 at head dim 128: the same 47.3 us)
-  return a.n_units * 32 / 256 < 8192 ? launch_rope_units<QT, D, CT, 1>(a, interleave, fp8, stream)
-                                      : launch_rope_units<QT, D, CT, 4>(a, interleave, fp8, stream);
+  if (a.n_units * 32 / 256 < 8192) return launch_rope_units<QT, D, CT, 1>(a, interleave, fp8, stream);
+  return launch_rope_units<QT, D, CT, 4>(a, interleave, fp8, stream);
 }
 
 template <typename QT, int D>
