@@ -420,6 +420,31 @@ int xllm_mi355_paged_decode_mla_planned(const void* plan, size_t plan_bytes,
                                         int dtype, void* stream);
 
 /*
+ * One decode step of an MLA attention layer in one call: store the step's latent rows, then attend.  Replaces the
+ * pair that the reference's MLA layer issues per layer and step, the latent store (store_latent_cache: the rows of
+ * compressed KV and rope key copied into the cache by slot, xllm/core/layers/dcu/deepseek_v2_attention.cpp:221-229)
+ * followed by dense_decode (decode_flash_mla, :242-263), with new_latent [batch] rows of 576 values of `dtype` (row stride in elements) and
+ * slot_mapping [batch] in front of the arguments of xllm_mi355_paged_decode_mla_planned.  plan may be NULL.
+ * Sequence b's slot must be the place of its token seq_lens[b] - 1 in its block table; negative slots and slots
+ * beyond the cache are skipped.  The cache and `out` afterwards hold the same bytes as after
+ * xllm_mi355_reshape_and_cache followed by the decode call.  Where the kernel for more than 64 heads serves the call
+ * (block size a power of two >= 16; new_latent 16-byte aligned with a stride that is a multiple of 8 elements) the
+ * rows are stored inside the decode launch, by the workgroup that attends to the context's last tokens; otherwise
+ * the library issues the two launches itself.  A sequence with seq_lens[b] == 0 stores nothing in the one-launch form.
+ */
+int xllm_mi355_write_and_decode_mla(const void* new_latent, const int32_t* slot_mapping,
+                                    int64_t latent_row_stride,
+                                    const void* plan, size_t plan_bytes,
+                                    const void* q_nope, const void* q_pe, void* k_cache,
+                                    void* out, float* lse,
+                                    const int32_t* block_table, int64_t table_stride,
+                                    const int32_t* seq_lens,
+                                    int64_t batch, int64_t n_heads, int64_t d_latent, int64_t d_rope,
+                                    int64_t block_size, int64_t num_blocks, int64_t max_seq_len,
+                                    float sm_scale, void* workspace, size_t workspace_bytes,
+                                    int dtype, void* stream);
+
+/*
  * Log-sum-exp merge of S partial attention results.
  * Replaces xllm::layer::merge_dcp_attention_shards
  * (xllm/core/layers/mlu/dcp_attention_merge.cpp:26-65):

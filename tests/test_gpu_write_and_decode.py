@@ -224,3 +224,85 @@ def test_one_call_rejects_missing_rows(device):
         fake, fake, fake, 1024, 1024, fake, 4096, fake, fake, fake, fake, None, fake, 8, fake, None, None, None, None,
         None, 4, 32, 8, 128, 16, 100, 4096, 4096, 100, -1, 0.1, fake, 1 << 30, capi.BF16, capi.BF16, None)
     assert rc == -4
+
+
+# ---- the MLA layer's step: store_latent_cache + decode_flash_mla (layers/dcu/deepseek_v2_attention.cpp:221-229,
+# :242-263) in one call, against the two calls
+
+def _mla_cfg(name, batch, heads, lo, hi, bs=64):
+    import math
+    return C(name, batch, heads, 1, 576, bs, lo, hi, mla=True, v_dim=512, sigma=0.5, sm_scale=1.0 / math.sqrt(192.0))
+
+
+MLA_CASES = [
+    # mla_decode_w4_kernel stores the rows itself
+    (_mla_cfg("m_128", 6, 128, 1, 3000), torch.bfloat16),
+    (_mla_cfg("m_128_fp16", 4, 128, 1, 2000), torch.float16),
+    (_mla_cfg("m_80_bs16", 5, 80, 1, 1500, bs=16), torch.bfloat16),
+    (_mla_cfg("m_256", 3, 256, 1, 2500), torch.bfloat16),          # two workgroups per team store the same row
+    (_mla_cfg("m_long", 2, 128, 30000, 50000), torch.bfloat16),    # contexts cut over many workgroups
+    (_mla_cfg("m_many", 300, 128, 1, 90), torch.bfloat16),         # several whole contexts per workgroup
+    # the other kernels: the library issues the two launches itself
+    (_mla_cfg("m_16", 6, 16, 1, 1200), torch.bfloat16),
+    (_mla_cfg("m_bs24", 4, 128, 1, 900, bs=24), torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("cfg,dtype", MLA_CASES, ids=[c.name for c, _ in MLA_CASES])
+@pytest.mark.parametrize("planned", [False, True], ids=["unplanned", "planned"])
+def test_mla_one_call_equals_store_then_decode(device, cfg, dtype, planned):
+    inp = workloads.make_inputs(cfg, 700 + len(cfg.name), dtype=dtype)
+    lay = inp.layout
+    B, H = cfg.batch, cfg.n_q_heads
+    shape = (lay.num_blocks, cfg.block_size, 1, cfg.head_dim)
+    kc0 = torch.full(shape, float("nan"), dtype=dtype, device=device)
+    if inp.k_ctx.shape[0] > 0:
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=inp.k_ctx.to(device), value=None, k_cache=kc0, v_cache=None,
+                                                            slot_mapping=lay.ctx_slots.to(device)))
+    # the step's rows as a slice of a wider buffer (the layer's kv_a projection output), 16-byte aligned rows
+    wide = torch.zeros(B, cfg.head_dim + 64, dtype=dtype, device=device)
+    wide[:, : cfg.head_dim] = inp.k_new.to(device).view(B, cfg.head_dim)
+    latent = wide[:, : cfg.head_dim]
+    slots = lay.new_slots.to(device).clone()
+    skipped = -1
+    if B >= 5:
+        skipped = 1
+        slots[skipped] = -1
+    q = inp.q.to(device)
+    table, lens = lay.block_table.to(device), lay.seq_lens.to(device)
+
+    def params(kc):
+        return ops.DenseDecodeParams(q_nope=q[:, :, : cfg.v_dim].contiguous().view(B, 1, H, cfg.v_dim),
+                                     q_pe=q[:, :, cfg.v_dim:].contiguous().view(B, 1, H, cfg.head_dim - cfg.v_dim),
+                                     k_cache=kc, seqlens_k=lens, block_table=table, head_size_v=cfg.v_dim,
+                                     softmax_scale=cfg.scale)
+    plan = ops.get_mla_decoding_metadata(lens, table, H, cfg.block_size) if planned else None
+    kc_a = kc0.clone()
+    ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=latent.unsqueeze(1), value=None, k_cache=kc_a, v_cache=None,
+                                                        slot_mapping=slots))
+    out_a, lse_a = ops.dense_decode(params(kc_a), return_lse=True, metadata=plan)
+    kc_b = kc0.clone()
+    out_b, lse_b = ops.dense_decode(params(kc_b), return_lse=True, metadata=plan, new_latent=latent, slot_mapping=slots)
+    torch.cuda.synchronize()
+    ops.decode_status(device)
+    assert torch.equal(_bits(kc_a), _bits(kc_b)), "latent cache bytes differ"
+    live = torch.ones(B, dtype=torch.bool, device=device)
+    if skipped >= 0:
+        live[skipped] = False
+    assert torch.equal(_bits(out_a[live]), _bits(out_b[live]))
+    assert torch.equal(lse_a[live], lse_b[live])
+    assert torch.isfinite(out_b[live].float()).all()
+    if cfg.name != "m_long":   # (the CPU checker on 80 000 tokens of 128 heads takes minutes; the pair is checked elsewhere)
+        lc = live.cpu()
+        ref = oracle.aten_paged_decode(inp.q[lc], kc_a.cpu(), None, lay.block_table[lc], lay.seq_lens[lc], cfg.scale,
+                                       dv=cfg.v_dim)
+        assert_close_to_reference(out_b[live].view(-1, H, cfg.v_dim), ref, cfg.name)
+
+
+def test_mla_one_call_rejects_missing_rows(device):
+    lib = capi.lib()
+    fake = 1 << 20
+    tail = (fake, fake, fake, fake, None, fake, 8, fake, 4, 128, 512, 64, 64, 100, 4096, 0.1, fake, 1 << 30, capi.BF16, None)
+    assert lib.xllm_mi355_write_and_decode_mla(None, fake, 576, None, 0, *tail) == -1
+    assert lib.xllm_mi355_write_and_decode_mla(fake, fake, 512, None, 0, *tail) == -1      # rows narrower than 576
+    assert lib.xllm_mi355_write_and_decode_mla(fake, fake, 576, fake, 4096, *tail) == -4   # an undersized plan

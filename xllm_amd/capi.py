@@ -59,6 +59,8 @@ SIGNATURES = {
     "xllm_mi355_paged_decode_mla_plan": (_i32, [_p, _sz, _p, _i64, _p, _i64, _i64, _i64, _p]),
     "xllm_mi355_paged_decode_mla_planned": (_i32, [_p, _sz, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i64, _i64,
                                                    _i64, _i64, _i64, _f32, _p, _sz, _i32, _p]),
+    "xllm_mi355_write_and_decode_mla": (_i32, [_p, _p, _i64, _p, _sz, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i64,
+                                               _i64, _i64, _i64, _i64, _f32, _p, _sz, _i32, _p]),
     "xllm_mi355_lse_merge": (_i32, [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i32, _p]),
     "xllm_mi355_lse_combine": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _i32, _p]),
     "xllm_mi355_build_block_table": (_i32, [_p, _p, _p, _p, _i64, _p, _i64, _i64, _p]),

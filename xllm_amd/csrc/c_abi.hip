@@ -372,6 +372,29 @@ int xllm_mi355_paged_decode_mla_plan(void* plan, size_t plan_bytes, const int32_
   return paged_decode_mla_plan(plan, plan_bytes, addr, batch, n_heads, block_size, static_cast<hipStream_t>(stream));
 }
 
+int xllm_mi355_write_and_decode_mla(const void* new_latent, const int32_t* slot_mapping, int64_t latent_row_stride,
+                                    const void* plan, size_t plan_bytes, const void* q_nope, const void* q_pe,
+                                    void* k_cache, void* out, float* lse, const int32_t* block_table,
+                                    int64_t table_stride, const int32_t* seq_lens, int64_t batch, int64_t n_heads,
+                                    int64_t d_latent, int64_t d_rope, int64_t block_size, int64_t num_blocks,
+                                    int64_t max_seq_len, float sm_scale, void* workspace, size_t workspace_bytes,
+                                    int dtype, void* stream) {
+  if (new_latent == nullptr || slot_mapping == nullptr || latent_row_stride < d_latent + d_rope) return XLLM_MI355_EINVAL;
+  if (plan != nullptr && plan_bytes < gqa_plan_bytes()) return XLLM_MI355_EWORKSPACE;
+  PageAddressing addr;
+  addr.block_table = block_table;
+  addr.table_stride = table_stride;
+  addr.seq_lens = seq_lens;
+  addr.plan = plan;
+  NewLatentRows fresh;
+  fresh.rows = new_latent;
+  fresh.slots = slot_mapping;
+  fresh.row_stride = latent_row_stride;
+  return paged_decode_mla(q_nope, q_pe, k_cache, out, lse, addr, batch, n_heads, d_latent, d_rope, block_size,
+                          num_blocks, max_seq_len, sm_scale, workspace, workspace_bytes, dtype,
+                          static_cast<hipStream_t>(stream), &fresh);
+}
+
 int xllm_mi355_paged_decode_mla_planned(const void* plan, size_t plan_bytes, const void* q_nope, const void* q_pe,
                                         const void* k_cache, void* out, float* lse, const int32_t* block_table,
                                         int64_t table_stride, const int32_t* seq_lens, int64_t batch, int64_t n_heads,

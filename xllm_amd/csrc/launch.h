@@ -112,11 +112,20 @@ int paged_decode_gqa_plan(void* plan, size_t plan_bytes, const PageAddressing& a
 int paged_decode_mla_plan(void* plan, size_t plan_bytes, const PageAddressing& addr, int64_t batch, int64_t n_heads,
                           int64_t block_size, hipStream_t stream);
 
+// The latent rows of the step's new tokens, [batch] rows of 576 values of the query's dtype (row stride in elements),
+// and their slots [batch]: the MLA decode call stores them into the cache before it attends, as reshape_and_cache
+// without a value tensor would.  Sequence b's slot must be the place of its token seq_len - 1 in its table.
+struct NewLatentRows {
+  const void* rows = nullptr;
+  const int32_t* slots = nullptr;
+  int64_t row_stride = 0;
+};
+
 int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, void* out, float* lse,
                      const PageAddressing& addr, int64_t batch, int64_t n_heads, int64_t d_latent,
                      int64_t d_rope, int64_t block_size, int64_t num_blocks, int64_t max_seq_len,
                      float sm_scale, void* workspace, size_t workspace_bytes, int dtype,
-                     hipStream_t stream);
+                     hipStream_t stream, const NewLatentRows* fresh = nullptr);
 
 // Several query tokens per sequence (packed q, cu_seqlens_q) through the decode kernels: token j of a
 // sequence with q_len tokens attends to the first kv_len - q_len + j + 1 tokens (causal) or to all kv_len.

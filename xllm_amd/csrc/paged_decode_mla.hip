@@ -112,6 +112,15 @@ struct MlaArgs {
   unsigned* ws_written;
   int* ws_status;   // status flags of the workspace (kStatus*), only ever OR-ed into
   int wait_spins;   // bound of the folding workgroup's polls on ws_written
+  // mla_decode_w4_kernel, store-then-attend in one launch: the step's new latent rows [batch] of 576 values (row stride
+  // in bytes) and their slots, or null.  The workgroup whose run holds a context's last token writes that row to the
+  // cache at the start of the run, before it fetches the first tile: what reshape_and_cache would have written before
+  // the launch.  Slots outside [0, n_slots) are skipped, as there.
+  const char* new_rows;
+  const int32_t* new_slots;
+  int64_t new_row_stride_bytes;
+  int64_t n_slots;
+  char* k_cache_w;
 };
 
 __device__ __forceinline__ int tiles_of(int L) { return L > 0 ? (L + kTile - 1) / kTile : 0; }
@@ -1799,6 +1808,20 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     };
     int ck_cur = (t_begin >> a.bs_shift) >> 6;
     __syncthreads();  // the previous run no longer reads the ring, the chunks, the factors or the flags
+    // Store-then-attend: this run holds the context's last token, whose row the step has not stored yet.  Wavefront 0
+    // stores it now; the barrier in front of the run's first tile loads comes after the store has completed, so the
+    // loads of the last sub-tile find the row in the cache like any other.  (Every workgroup of a team does so for
+    // itself, with the same bytes: what it reads later is what it wrote.)
+    if (a.new_rows != nullptr && t_end == L && wave == 0) {
+      const int64_t slot = a.new_slots[b];
+      if (slot >= 0 && slot < a.n_slots) {
+        const int ln = lane_again();
+        const char* nrow = a.new_rows + static_cast<int64_t>(b) * a.new_row_stride_bytes;
+        char* dst = a.k_cache_w + slot * kRowBytes;
+        stg16(dst + ln * 16, ldg16(nrow + ln * 16));
+        if (ln < kDR * 2 / 16) stg16(dst + kDL * 2 + ln * 16, ldg16(nrow + kDL * 2 + ln * 16));
+      }
+    }
     // the page-table chunks of the run's first sub-tiles travel while the Q rows do
     if (wave == 0) {
       if (!plan_chunk) issue_chunk(ck_cur);   // (the plan brought the first run's chunk in with the prefix)
@@ -2603,11 +2626,13 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
                      const PageAddressing& addr, int64_t batch, int64_t n_heads, int64_t d_latent,
                      int64_t d_rope, int64_t block_size, int64_t num_blocks, int64_t max_seq_len,
                      float sm_scale, void* workspace, size_t workspace_bytes, int dtype,
-                     hipStream_t stream) {
+                     hipStream_t stream, const NewLatentRows* fresh) {
   (void)max_seq_len;  // the schedule is computed on the device from the actual lengths
   if (batch == 0) return XLLM_MI355_OK;
   if (q_nope == nullptr || q_pe == nullptr || k_cache == nullptr || out == nullptr ||
       addr.block_table == nullptr || addr.seq_lens == nullptr || addr.table_stride <= 0)
+    return XLLM_MI355_EINVAL;
+  if (fresh != nullptr && (fresh->rows == nullptr || fresh->slots == nullptr || fresh->row_stride < kDK))
     return XLLM_MI355_EINVAL;
   if (batch < 0 || n_heads <= 0 || n_heads > 65535 || block_size <= 0 || num_blocks <= 0 ||
       !(sm_scale > 0.0f))
@@ -2659,9 +2684,26 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
       if (e == hipSuccess) e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kW4LdsBytes);
     if (e != hipSuccess) return static_cast<int>(e);
   }
+  // The step's new rows: inside mla_decode_w4_kernel where it serves the call and the rows can be fetched 16 bytes at
+  // a time; otherwise the store is a launch of its own before the decode, with the same result.
+  const bool w4_call = w4_serves(n_heads, block_size);
+  const bool fused = fresh != nullptr && w4_call && aligned16(fresh->rows) && (fresh->row_stride * 2) % 16 == 0;
+  if (fresh != nullptr && !fused) {
+    const int rc = reshape_and_cache(fresh->rows, nullptr, const_cast<void*>(k_cache), nullptr, fresh->slots, nullptr,
+                                     nullptr, batch, 1, kDK, block_size, num_blocks, fresh->row_stride, 0, dtype, dtype,
+                                     stream);
+    if (rc != 0) return rc;
+  }
   for (int64_t b0 = 0; b0 < batch; b0 += max_batch) {
     const int64_t nb = batch - b0 < max_batch ? batch - b0 : max_batch;
     MlaArgs a = {};
+    if (fused) {
+      a.new_rows = static_cast<const char*>(fresh->rows) + b0 * fresh->row_stride * 2;
+      a.new_slots = fresh->slots + b0;
+      a.new_row_stride_bytes = fresh->row_stride * 2;
+      a.n_slots = num_blocks * block_size;
+      a.k_cache_w = static_cast<char*>(const_cast<void*>(k_cache));
+    }
     a.q_nope = static_cast<const char*>(q_nope) + b0 * n_heads * kDL * 2;
     a.q_pe = static_cast<const char*>(q_pe) + b0 * n_heads * kDR * 2;
     a.k_cache = static_cast<const char*>(k_cache);
@@ -2686,11 +2728,7 @@ int paged_decode_mla(const void* q_nope, const void* q_pe, const void* k_cache, 
     a.ws_lse = a.ws_out + static_cast<size_t>(a.n_teams) * 2 * a.slot_heads * kDL;
     // (XLLM_MLA_DEFAULT_NARROW: the build found that the compiler did not leave the fixed-name accumulators of
     // mla_decode_w4_kernel alone and made the eight-wavefront kernel the default; 'w' still asks for the other)
-#ifdef XLLM_MLA_DEFAULT_NARROW
-    const bool w4 = !pairs && by_dims && knob == 'w';
-#else
-    const bool w4 = !pairs && by_dims && knob != 'n';
-#endif
+    const bool w4 = w4_call;
     a.run_cost = w4 ? w4_run_cost() : 0;
     // the step's plan: for the kernel it was made for, and not for a batch decoded in slices
     a.plan = w4 && batch <= max_batch && a.n_teams <= kPlanMaxTeams ? static_cast<const int*>(addr.plan) : nullptr;

@@ -573,7 +573,25 @@ void check_dense_decode_inputs(const DenseDecodeParams& p) {
 }  // namespace
 
 namespace {
-torch::Tensor dense_decode_impl(DenseDecodeParams& p, const torch::Tensor* plan, torch::Tensor* lse_out);
+struct NewLatent {
+  torch::Tensor rows, slots;
+};
+torch::Tensor dense_decode_impl(DenseDecodeParams& p, const torch::Tensor* plan, torch::Tensor* lse_out,
+                                const NewLatent* fresh = nullptr);
+}
+torch::Tensor store_and_dense_decode(DenseDecodeParams& p, const torch::Tensor& latent_cache,
+                                     const torch::Tensor& slot_mapping,
+                                     const std::optional<torch::Tensor>& tile_scheduler_metadata, torch::Tensor* lse_out) {
+  const bool planned = tile_scheduler_metadata.has_value() && tile_scheduler_metadata->defined();
+  if (planned)
+    TORCH_CHECK(tile_scheduler_metadata->is_cuda() && tile_scheduler_metadata->is_contiguous() &&
+                    tile_scheduler_metadata->scalar_type() == torch::kUInt8 &&
+                    static_cast<size_t>(tile_scheduler_metadata->numel()) >= xllm_mi355_paged_decode_plan_bytes(),
+                "flash_mla: tile_scheduler_metadata must be the buffer of get_mla_decoding_metadata");
+  TORCH_CHECK(latent_cache.defined() && latent_cache.is_cuda() && (latent_cache.dim() == 2 || latent_cache.dim() == 3),
+              "flash_mla: latent_cache must be a device tensor [B, D] or [B, 1, D]");
+  const NewLatent fresh{latent_cache.dim() == 3 ? latent_cache.view({latent_cache.size(0), -1}) : latent_cache, slot_mapping};
+  return dense_decode_impl(p, planned ? &*tile_scheduler_metadata : nullptr, lse_out, &fresh);
 }
 torch::Tensor dense_decode(DenseDecodeParams& p, torch::Tensor* lse_out) { return dense_decode_impl(p, nullptr, lse_out); }
 torch::Tensor dense_decode(DenseDecodeParams& p, const torch::Tensor& tile_scheduler_metadata, torch::Tensor* lse_out) {
@@ -610,7 +628,8 @@ std::vector<torch::Tensor> get_mla_decoding_metadata(const torch::Tensor& seqlen
 }
 
 namespace {
-torch::Tensor dense_decode_impl(DenseDecodeParams& p, const torch::Tensor* plan, torch::Tensor* lse_out) {
+torch::Tensor dense_decode_impl(DenseDecodeParams& p, const torch::Tensor* plan, torch::Tensor* lse_out,
+                                const NewLatent* fresh) {
   TORCH_CHECK(p.kind == DenseDecodeKind::kQNopePe,
               "flash_mla: only DenseDecodeKind::kQNopePe (BF16/FP16 split-q) is supported");
   check_dense_decode_inputs(p);
@@ -644,7 +663,23 @@ torch::Tensor dense_decode_impl(DenseDecodeParams& p, const torch::Tensor* plan,
   const int64_t max_seq_len = table.size(1) * p.k_cache.size(1);
   const size_t nbytes = xllm_mi355_paged_decode_mla_workspace_bytes(rows, heads, max_seq_len);
   torch::Tensor ws = mi355::decode_workspace(q_nope.device(), nbytes);
-  if (plan != nullptr && !per_token) {   // (a causal multi-token step rewrites lengths and table per token: no plan)
+  if (fresh != nullptr) {
+    TORCH_CHECK(Sq == 1, "flash_mla: the one-call step stores one new row per sequence (S_q == 1)");
+    TORCH_CHECK(fresh->rows.size(0) == B && fresh->rows.size(1) == p.k_cache.size(3) && fresh->rows.stride(1) == 1 &&
+                    fresh->rows.scalar_type() == q_nope.scalar_type(),
+                "flash_mla: latent_cache must hold one row of the cache's width per sequence, in the query's dtype");
+    TORCH_CHECK(fresh->slots.is_cuda() && fresh->slots.scalar_type() == torch::kInt32 && fresh->slots.is_contiguous() &&
+                    fresh->slots.numel() == B,
+                "flash_mla: slot_mapping must be contiguous int32 [B]");
+    const int rc = xllm_mi355_write_and_decode_mla(
+        fresh->rows.data_ptr(), fresh->slots.data_ptr<int32_t>(), fresh->rows.stride(0),
+        plan != nullptr ? plan->data_ptr() : nullptr, plan != nullptr ? static_cast<size_t>(plan->numel()) : 0,
+        q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(), out.data_ptr(), lse, table.data_ptr<int32_t>(),
+        table.stride(0), seqlens.data_ptr<int32_t>(), rows, heads, q_nope.size(3), q_pe.size(3), p.k_cache.size(1),
+        p.k_cache.size(0), max_seq_len, p.softmax_scale, ws.data_ptr(), static_cast<size_t>(ws.numel()),
+        dtype_code(q_nope), current_stream(q_nope));
+    check_rc(rc, "xllm_mi355_write_and_decode_mla");
+  } else if (plan != nullptr && !per_token) {   // (a causal multi-token step rewrites lengths and table per token: no plan)
     const int rc = xllm_mi355_paged_decode_mla_planned(
         plan->data_ptr(), static_cast<size_t>(plan->numel()), q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(),
         out.data_ptr(), lse, table.data_ptr<int32_t>(), table.stride(0), seqlens.data_ptr<int32_t>(), rows, heads,
@@ -890,7 +925,9 @@ std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nop
                                                              torch::Tensor k_cache, torch::Tensor seqlens_k,
                                                              torch::Tensor block_table, int64_t head_size_v,
                                                              double softmax_scale, bool is_causal,
-                                                             std::optional<torch::Tensor> plan) {
+                                                             std::optional<torch::Tensor> plan,
+                                                             std::optional<torch::Tensor> latent_cache,
+                                                             std::optional<torch::Tensor> slot_mapping) {
   xllm::kernel::dcu::flash_mla::DenseDecodeParams p;
   p.q_nope = q_nope;
   p.q_pe = q_pe;
@@ -902,6 +939,11 @@ std::tuple<torch::Tensor, torch::Tensor> op_mla_dense_decode(torch::Tensor q_nop
   p.is_causal = is_causal;
   p.kind = xllm::kernel::dcu::flash_mla::DenseDecodeKind::kQNopePe;
   torch::Tensor lse;
+  if (latent_cache.has_value() && latent_cache->defined()) {   // the layer's store + decode in one call
+    TORCH_CHECK(slot_mapping.has_value() && slot_mapping->defined(), "latent_cache and slot_mapping come together");
+    torch::Tensor out = xllm::kernel::dcu::flash_mla::store_and_dense_decode(p, *latent_cache, *slot_mapping, plan, &lse);
+    return {out, lse};
+  }
   torch::Tensor out = plan.has_value() && plan->defined() ? xllm::kernel::dcu::flash_mla::dense_decode(p, *plan, &lse)
                                                           : xllm::kernel::dcu::flash_mla::dense_decode(p, &lse);
   return {out, lse};
@@ -1014,8 +1056,9 @@ TORCH_LIBRARY(xllm_ops, m) {
         "Tensor seq_lens, Tensor? k_scale, Tensor? v_scale, int max_seq_len, float scale, Tensor? plan=None) -> (Tensor, Tensor)");
   m.def("update_decode_plan(Tensor block_table, Tensor seq_lens, int num_qo_heads, int num_kv_heads, int head_dim, "
         "int block_size, int window_left, bool fp8_cache, Tensor(a!)? plan=None) -> Tensor");
-  m.def("mla_dense_decode(Tensor q_nope, Tensor q_pe, Tensor k_cache, Tensor seqlens_k, Tensor block_table, "
-        "int head_size_v, float softmax_scale, bool is_causal=False, Tensor? plan=None) -> (Tensor, Tensor)");
+  m.def("mla_dense_decode(Tensor q_nope, Tensor q_pe, Tensor(a!) k_cache, Tensor seqlens_k, Tensor block_table, "
+        "int head_size_v, float softmax_scale, bool is_causal=False, Tensor? plan=None, Tensor? latent_cache=None, "
+        "Tensor? slot_mapping=None) -> (Tensor, Tensor)");
   m.def("mla_decoding_metadata(Tensor seqlens_k, Tensor block_table, int num_heads_per_head_k, int block_size, "
         "Tensor(a!)? plan=None) -> Tensor");
   m.def("lse_combine(Tensor(a!) output, Tensor shared_o, Tensor shared_lse, Tensor unshared_o, Tensor unshared_lse) -> Tensor");

@@ -213,6 +213,13 @@ std::vector<torch::Tensor> get_mla_decoding_metadata(const torch::Tensor& seqlen
                                                      const std::optional<torch::Tensor>& reuse = std::nullopt);
 // dense_decode from that plan (same lengths and table): bit-identical to the call without it.
 torch::Tensor dense_decode(DenseDecodeParams& params, const torch::Tensor& tile_scheduler_metadata, torch::Tensor* lse);
+// The decode step of the MLA layer in one call: store_latent_cache(latent_cache, slot_mapping, k_cache) followed by
+// decode_flash_mla (xllm/core/layers/dcu/deepseek_v2_attention.cpp:221-229 and :242-263).  latent_cache [B, 576] (or
+// [B, 1, 576]) of the query's dtype, slot_mapping [B] int32; one query token per sequence; the plan may be undefined.
+// Same cache bytes and output as the two calls.
+torch::Tensor store_and_dense_decode(DenseDecodeParams& params, const torch::Tensor& latent_cache,
+                                     const torch::Tensor& slot_mapping,
+                                     const std::optional<torch::Tensor>& tile_scheduler_metadata, torch::Tensor* lse);
 
 }  // namespace flash_mla
 }  // namespace dcu

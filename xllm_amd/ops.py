@@ -466,13 +466,17 @@ def get_mla_decoding_metadata(seqlens_k, block_table, num_heads_per_head_k, bloc
     return plan
 
 
-def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0, metadata=None):
+def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0, metadata=None, new_latent=None,
+                 slot_mapping=None):
     """flash_mla::dense_decode (flash_mla_adapter.cpp:104-153): returns [B, S_q, H, head_size_v] (and the natural-log
     lse [B, H, S_q] fp32 when asked).  The same argument checks.  BF16 and FP16.  The S_q query tokens of a sequence
     are folded into the head count as the reference folds them (:119-123); with is_causal and S_q > 1 token j attends
     to the first seqlens_k - (S_q - 1 - j) tokens and every (sequence, token) becomes a row of its own.
     metadata: the step's plan from get_mla_decoding_metadata (same lengths and table), or None: the launch derives its
-    schedule itself.  (A causal multi-token step rewrites lengths and table per token and takes no plan.)"""
+    schedule itself.  (A causal multi-token step rewrites lengths and table per token and takes no plan.)
+    new_latent [B, 576] (or [B, 1, 576]) with slot_mapping [B] int32: the step's latent rows, stored into the cache by
+    the same call before it attends (store_latent_cache + decode_flash_mla of the MLA layer,
+    layers/dcu/deepseek_v2_attention.cpp:221-229 and :242-263, in one call; one query token per sequence)."""
     p = params
     if p.kind != DenseDecodeKind.kQNopePe:
         raise ValueError("flash_mla: only DenseDecodeKind::kQNopePe (BF16/FP16 split-q) is supported")
@@ -521,8 +525,28 @@ def dense_decode(params: DenseDecodeParams, return_lse=False, max_seq_len=0, met
     lib = capi.lib()
     nbytes = lib.xllm_mi355_paged_decode_mla_workspace_bytes(rows, heads, max_seq_len)
     ws = decode_workspace(dev, nbytes)
-    if metadata is not None and not (p.is_causal and Sq > 1):
+    planned = metadata is not None and not (p.is_causal and Sq > 1)
+    if planned:
         _check_plan(metadata)
+    if new_latent is not None or slot_mapping is not None:
+        if new_latent is None or slot_mapping is None:
+            raise ValueError("new_latent and slot_mapping come together")
+        if Sq != 1:
+            raise ValueError("the one-call step stores one new row per sequence: S_q must be 1")
+        _require_cuda(new_latent, slot_mapping)
+        rows_new = new_latent.view(B, d_latent + d_rope) if new_latent.dim() == 3 else new_latent
+        if rows_new.dtype != q_nope.dtype or tuple(rows_new.shape) != (B, d_latent + d_rope) or rows_new.stride(1) != 1:
+            raise ValueError("new_latent must be [B, kv_lora_rank + rope dim] of the query's dtype with contiguous rows")
+        if slot_mapping.dtype != torch.int32 or slot_mapping.numel() != B or not slot_mapping.is_contiguous():
+            raise ValueError("slot_mapping must be contiguous int32 [B]")
+        rc = lib.xllm_mi355_write_and_decode_mla(
+            rows_new.data_ptr(), slot_mapping.data_ptr(), rows_new.stride(0), _ptr(metadata) if planned else None,
+            metadata.numel() if planned else 0, q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(),
+            out.data_ptr(), _ptr(lse), table.data_ptr(), table.stride(0), seqlens.data_ptr(), rows, heads, d_latent,
+            d_rope, bs, P, max_seq_len, float(p.softmax_scale), ws.data_ptr(), ws.numel(), _dtype_code(q_nope),
+            _stream(dev))
+        capi.check(rc, "xllm_mi355_write_and_decode_mla")
+    elif planned:
         rc = lib.xllm_mi355_paged_decode_mla_planned(
             metadata.data_ptr(), metadata.numel(), q_nope.data_ptr(), q_pe.data_ptr(), p.k_cache.data_ptr(),
             out.data_ptr(), _ptr(lse), table.data_ptr(), table.stride(0), seqlens.data_ptr(), rows, heads, d_latent,
