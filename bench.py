@@ -51,8 +51,8 @@ def parse_args():
     ap.add_argument("--no-planned", action="store_true",
                     help="skip the second timed loop (the GQA step with the plan made once per step)")
     ap.add_argument("--two-calls", action="store_true",
-                    help="GQA: time the pair reshape_and_cache + paged_decode_gqa as the step instead of the one call "
-                         "write_and_decode_gqa (the default line reports the pair beside the one call anyway)")
+                    help="time the pair reshape_and_cache + paged decode as the step instead of the one call "
+                         "write_and_decode_gqa / _mla (the default line reports the pair beside the one call anyway)")
     ap.add_argument("--graph", action="store_true",
                     help="add a third timed loop: the step captured in a HIP graph and replayed (graph_replay in the line)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
@@ -394,13 +394,16 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
 
     bound = [bound_args(k_caches[i], v_caches[i]) for i in range(ROTATE)]
     reshape_args, decode_args = bound[0]
-    # GQA: the step as the attention layer issues it, one call that stores the new rows and attends
-    # (xllm_mi355_write_and_decode_gqa); the pair of calls it replaces is timed beside it.  MLA: the pair.
-    one_call = not cfg.mla and not args.two_calls
-    one_fn = lib.xllm_mi355_write_and_decode_gqa
+    # The step as the attention layer issues it: one call that stores the new rows and attends
+    # (xllm_mi355_write_and_decode_gqa / _mla); the pair of calls it replaces is timed beside it.
+    one_call = not args.two_calls
+    one_fn = lib.xllm_mi355_write_and_decode_mla if cfg.mla else lib.xllm_mi355_write_and_decode_gqa
 
     def one_call_args(d_args, plan=None):
-        return (ptr(inp.k_new), ptr(inp.v_new), ptr(new_slots), row, row, ptr(plan), 0 if plan is None else plan.numel()) \
+        plan_args = (ptr(plan), 0 if plan is None else plan.numel())
+        if cfg.mla:
+            return (ptr(inp.k_new), ptr(new_slots), row) + plan_args + d_args
+        return (ptr(inp.k_new), ptr(inp.v_new), ptr(new_slots), row, row) + plan_args \
             + d_args[:8] + (None, None, None) + d_args[8:]
 
     def step_calls(i, one, plan=None):
@@ -598,7 +601,8 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
             "batch": cfg.batch, "n_q_heads": cfg.n_q_heads, "n_kv_heads": cfg.n_kv_heads,
             "head_dim": cfg.head_dim, "block_size": cfg.block_size,
             "context_tokens": int(lay.seq_lens.sum()), "max_context": max_len,
-            "step": ("write_and_decode_gqa: the new K/V rows stored and attended to in one call, inputs resident in HBM"
+            "step": (("write_and_decode_mla: the new latent rows" if cfg.mla else "write_and_decode_gqa: the new K/V rows")
+                     + " stored and attended to in one call, inputs resident in HBM"
                      if one_call else
                      "reshape_and_cache(new K/V rows) + paged decode attention, inputs resident in HBM"),
         },
