@@ -1809,18 +1809,19 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
     int ck_cur = (t_begin >> a.bs_shift) >> 6;
     __syncthreads();  // the previous run no longer reads the ring, the chunks, the factors or the flags
     // Store-then-attend: this run holds the context's last token, whose row the step has not stored yet.  Wavefront 0
-    // stores it now; the barrier in front of the run's first tile loads comes after the store has completed, so the
-    // loads of the last sub-tile find the row in the cache like any other.  (Every workgroup of a team does so for
-    // itself, with the same bytes: what it reads later is what it wrote.)
-    if (a.new_rows != nullptr && t_end == L && wave == 0) {
-      const int64_t slot = a.new_slots[b];
-      if (slot >= 0 && slot < a.n_slots) {
-        const int ln = lane_again();
-        const char* nrow = a.new_rows + static_cast<int64_t>(b) * a.new_row_stride_bytes;
-        char* dst = a.k_cache_w + slot * kRowBytes;
-        stg16(dst + ln * 16, ldg16(nrow + ln * 16));
-        if (ln < kDR * 2 / 16) stg16(dst + kDL * 2 + ln * 16, ldg16(nrow + kDL * 2 + ln * 16));
-      }
+    // fetches it now, with the loads of the run's prologue, and stores it behind their common wait; the barrier in
+    // front of the run's first tile loads comes after the store has completed, so the loads of the last sub-tile find
+    // the row in the cache like any other.  (Every workgroup of a team does so for itself, with the same bytes: what it
+    // reads later is what it wrote.)
+    u32x4 new_latent = {0u, 0u, 0u, 0u}, new_rope = {0u, 0u, 0u, 0u};
+    int64_t new_slot = -1;
+    const bool stores_row = a.new_rows != nullptr && t_end == L && wave == 0;
+    if (stores_row) {   // (slot and row travel together: the slot is looked at when the row is stored)
+      new_slot = a.new_slots[b];
+      const int ln = lane_again();
+      const char* nrow = a.new_rows + static_cast<int64_t>(b) * a.new_row_stride_bytes;
+      new_latent = ldg16(nrow + ln * 16);
+      if (ln < kDR * 2 / 16) new_rope = ldg16(nrow + kDL * 2 + ln * 16);
     }
     // the page-table chunks of the run's first sub-tiles travel while the Q rows do
     if (wave == 0) {
@@ -2181,6 +2182,12 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
 
     // the chunk loads and the Q rows have landed (one wait for both latencies); the wavefront reads the rows it sent
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (stores_row && new_slot >= 0 && new_slot < a.n_slots) {   // (wavefront 0 of a run that ends its context)
+      const int ln = lane_again();
+      char* dst = a.k_cache_w + new_slot * kRowBytes;
+      stg16(dst + ln * 16, new_latent);
+      if (ln < kDR * 2 / 16) stg16(dst + kDL * 2 + ln * 16, new_rope);
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const char* qrow = smem + (wave * 32 + j * 16 + c16p) * kW4QRow + gp * 16;
@@ -2190,6 +2197,7 @@ __global__ __launch_bounds__(kW4Threads) void mla_decode_w4_kernel(MlaArgs a) {
         q[j][kk] = kk < kDL / 32 ? *reinterpret_cast<const u32x4*>(qrow + kk * 64)
                                  : *reinterpret_cast<const u32x4*>(qrope + (kk - kDL / 32) * 64);
     }
+    if (stores_row) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the step's row is in the cache
     __syncthreads();   // (the ring is free for the first sub-tiles)
     if (pending >= 0) {   // every wavefront's stores of the piece before have landed (the wait above), and all are past it
       if (tid == 0) announce(pending);
