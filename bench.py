@@ -51,8 +51,9 @@ def parse_args():
     ap.add_argument("--no-planned", action="store_true",
                     help="skip the second timed loop (the GQA step with the plan made once per step)")
     ap.add_argument("--two-calls", action="store_true",
-                    help="time the pair reshape_and_cache + paged decode as the step instead of the one call "
-                         "write_and_decode_gqa / _mla (the default line reports the pair beside the one call anyway)")
+                    help="GQA: time the pair reshape_and_cache + paged_decode_gqa as the step instead of the one call "
+                         "write_and_decode_gqa, and do not time the other form beside the step (two_calls / one_call "
+                         "in the default line)")
     ap.add_argument("--graph", action="store_true",
                     help="add a third timed loop: the step captured in a HIP graph and replayed (graph_replay in the line)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="sequences timed on the CPU (0 = auto)")
@@ -394,9 +395,11 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
 
     bound = [bound_args(k_caches[i], v_caches[i]) for i in range(ROTATE)]
     reshape_args, decode_args = bound[0]
-    # The step as the attention layer issues it: one call that stores the new rows and attends
-    # (xllm_mi355_write_and_decode_gqa / _mla); the pair of calls it replaces is timed beside it.
-    one_call = not args.two_calls
+    # GQA: the step as the attention layer issues it, one call that stores the new rows and attends
+    # (xllm_mi355_write_and_decode_gqa); the pair of calls it replaces is timed beside it.  MLA: the pair is the step
+    # (xllm_mi355_write_and_decode_mla takes as long, with a decode kernel that is longer by the store it holds), and
+    # the one call is timed beside it.
+    one_call = not args.two_calls and not cfg.mla
     one_fn = lib.xllm_mi355_write_and_decode_mla if cfg.mla else lib.xllm_mi355_write_and_decode_gqa
 
     def one_call_args(d_args, plan=None):
@@ -470,18 +473,21 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
     _, same_kernel_ms, same_merge_ms = timed_loop(same_step, events=True)
     same_cache = {"ms_per_step": same_ms_per_step, "kernel_ms": same_kernel_ms, "merge_kernel_ms": same_merge_ms,
                   "tokens_per_s": cfg.batch / (same_ms_per_step * 1e-3)}
-    # the pair of calls (store, then decode) that the one call replaces
-    two_calls = None
-    if one_call:
-        pair_step = make_step(ROTATE, one=False)
-        pair_ms_per_step, _, _ = timed_loop(pair_step, events=False)
-        _, pair_kernel_ms, pair_merge_ms = timed_loop(pair_step, events=True)
-        pair_out = out.clone()
+    # the other form of the step: the pair of calls (store, then decode) beside the one call, or the one call beside
+    # the pair
+    two_calls = other_form = None
+    if not args.two_calls:
+        other_step = make_step(ROTATE, one=not one_call)
+        other_ms_per_step, _, _ = timed_loop(other_step, events=False)
+        _, other_kernel_ms, other_merge_ms = timed_loop(other_step, events=True)
+        other_out = out.clone()
         step()
         torch.cuda.synchronize()
-        two_calls = {"ms_per_step": pair_ms_per_step, "kernel_ms": pair_kernel_ms, "merge_kernel_ms": pair_merge_ms,
-                     "tokens_per_s": cfg.batch / (pair_ms_per_step * 1e-3),
-                     "bit_identical": bool(torch.equal(pair_out, out))}
+        other_form = {"ms_per_step": other_ms_per_step, "kernel_ms": other_kernel_ms, "merge_kernel_ms": other_merge_ms,
+                      "tokens_per_s": cfg.batch / (other_ms_per_step * 1e-3),
+                      "bit_identical": bool(torch.equal(other_out, out))}
+        if one_call:
+            two_calls = other_form
     elapsed = ms_per_step * 1e-3 * args.steps
 
     # ---- the same step as the layers after the first see it when the step was planned once (not the headline:
@@ -610,6 +616,7 @@ def run_workload(name, args, lib, capi, ops, workloads, torch, dev, cpu_budget_s
         "kv_cache_copies_in_rotation": ROTATE,
         "same_cache": same_cache,
         "two_calls": two_calls,
+        "one_call": None if one_call else other_form,
         "hbm_gbs_whole_step": (nbytes + workloads.reshape_bytes(
             cfg.batch, cfg.n_kv_heads * cfg.head_dim, 2, 1 if fp8 else 2, 1 if cfg.mla else 2))
             / (ms_per_step * 1e-3) / 1e9,
@@ -668,7 +675,8 @@ def main():
         result = dict(per[HEADLINE])
         result["gate"] = {"workload": "tiny", "parity": gate.get("parity")}
         keep = ("value", "unit", "ms_per_step", "dtype", "config", "hbm_gbs_whole_step", "roofline", "cpu_baseline",
-                "parity", "same_cache", "two_calls", "instrumented_ms_per_step", "kv_cache_copies_in_rotation")
+                "parity", "same_cache", "two_calls", "one_call", "instrumented_ms_per_step",
+                "kv_cache_copies_in_rotation")
         result["per_config"] = [{k: per[name][k] for k in keep if k in per[name]} for name in ALL]
         if not args.no_cpu_baseline:
             result["parity_all_ok"] = all(per[name]["parity"]["ok"] for name in ALL) and gate["parity"]["ok"]
