@@ -306,3 +306,39 @@ def test_mla_one_call_rejects_missing_rows(device):
     assert lib.xllm_mi355_write_and_decode_mla(None, fake, 576, None, 0, *tail) == -1
     assert lib.xllm_mi355_write_and_decode_mla(fake, fake, 512, None, 0, *tail) == -1      # rows narrower than 576
     assert lib.xllm_mi355_write_and_decode_mla(fake, fake, 576, fake, 4096, *tail) == -4   # an undersized plan
+
+
+def test_one_call_on_random_shapes(device):
+    """Random head counts, head dims, block sizes, page types, batch sizes and lengths (lengths around the stage
+    boundaries included): the one call and the pair leave the same bytes everywhere."""
+    g = torch.Generator().manual_seed(2024)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=g))
+
+    for case in range(14):
+        D = [64, 128, 128, 256][ri(0, 3)]
+        fp8 = ri(0, 2) == 0
+        Hkv = [1, 2, 3, 4, 8][ri(0, 4)]
+        Hq = Hkv * [1, 2, 4, 5, 8, 16, 20][ri(0, 6)]
+        bs = [8, 16, 32, 64, 128][ri(0, 4)]
+        batch = [1, 2, 7, 33, 64, 130][ri(0, 5)]
+        hi = [17, 70, 600, 3000][ri(0, 3)]
+        if batch * hi * Hkv * D > 4e8:
+            batch = max(1, batch // 8)
+        dtype = torch.float16 if ri(0, 3) == 0 else torch.bfloat16
+        cfg = C(f"w_rand{case}", batch, Hq, Hkv, D, bs, 1, hi, cache_dtype="fp8" if fp8 else "bf16")
+        inp = workloads.make_inputs(cfg, 5000 + case, dtype=dtype)
+        slots = inp.layout.new_slots.to(device).clone()
+        dead = None
+        if batch > 2 and ri(0, 1) == 0:
+            dead = ri(0, batch - 1)
+            slots[dead] = -1
+        out_a, lse_a, out_b, lse_b = _pair_and_one_call(inp, device, dtype, fp8, slots)
+        live = torch.ones(batch, dtype=torch.bool, device=device)
+        if dead is not None:
+            live[dead] = False
+        what = f"{cfg.name}: Hq {Hq} Hkv {Hkv} D {D} bs {bs} fp8 {fp8} batch {batch} hi {hi} {dtype}"
+        assert torch.equal(_bits(out_a[live]), _bits(out_b[live])), what
+        assert torch.equal(lse_a[live], lse_b[live]), what
+        assert torch.isfinite(out_b[live].float()).all(), what
