@@ -210,9 +210,15 @@ def neighbours(ops, workloads, torch, dev, steps, lib=None, capi=None):
         copy_gbs = None
         if lib is not None:
             copy_gbs, _ = stream_rate(lib, capi, torch, dev, nbytes // 2, copy=True, reps=20)
+        # ... and the runtime's own device-to-device copy of the same bytes (Tensor.copy_), timed like the op
+        src = torch.empty(nbytes // 2, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        torch_us = timed(lambda: dst.copy_(src))
+        del src, dst
         rows.append({"op": op, "kernel": kernel, "shape": shape, "us": us, "algorithmic_bytes": nbytes,
                      "gbs": nbytes / us / 1e3, "frac_of_hbm_peak": nbytes / us / 1e3 / HBM_PEAK_GBS,
-                     "plain_copy_gbs_same_bytes": copy_gbs})
+                     "plain_copy_gbs_same_bytes": copy_gbs,
+                     "torch_copy_gbs_same_bytes": nbytes // 2 * 2 / torch_us / 1e3})
 
     # reshape_and_cache: a prefill chunk of 8192 tokens into bf16 pages (configuration 2's heads), read + write
     T, nk, D = 8192, 8, 128

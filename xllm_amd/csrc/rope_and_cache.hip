@@ -138,36 +138,23 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeArgs a) {
   }
   // cos | sin of the lane's dims: c[u][i], sn[u][i] belong to pair i of the interleaved form, to dim i of the split form
   constexpr int NC = INTERLEAVE ? E / 2 : E;
-  float c[U][NC], sn[U][NC];
+  constexpr int UC = SAME ? 1 : U;   // (one set for the group when its units share a token: a set per unit costs the
+                                     // registers that decide how many wavefronts a SIMD holds)
+  float c[UC][NC], sn[UC][NC];
   // the lane's dims lie on one side of the split form (rotary_dim / 2 is a multiple of E)
   const int j0 = INTERLEAVE ? (sub * E) / 2 : (sub * E < half ? sub * E : sub * E - half);
-  if constexpr (SAME) {   // (the row of the token's position exists whatever the unit's kind)
-    if (rotated) {
-      cache_vec<CT, NC>(a.cos_sin, cs[0] + j0, c[0]);
-      cache_vec<CT, NC>(a.cos_sin, cs[0] + half + j0, sn[0]);
+  // (lanes and units that are not rotated never look at their entries: the rotation below is under the same conditions)
+#pragma unroll
+  for (int u = 0; u < UC; ++u) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      c[u][i] = 1.0f;
+      sn[u][i] = 0.0f;
     }
-  }
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    if (rotated && !is_v[u]) {
-      if constexpr (SAME) {
-        if (u > 0) {
-#pragma unroll
-          for (int i = 0; i < NC; ++i) {
-            c[u][i] = c[0][i];
-            sn[u][i] = sn[0][i];
-          }
-        }
-      } else {
-        cache_vec<CT, NC>(a.cos_sin, cs[u] + j0, c[u]);
-        cache_vec<CT, NC>(a.cos_sin, cs[u] + half + j0, sn[u]);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < NC; ++i) {
-        c[u][i] = 1.0f;
-        sn[u][i] = 0.0f;
-      }
+    // (SAME: the row of the token's position exists whatever the units' kinds)
+    if (rotated && (SAME || !is_v[u])) {
+      cache_vec<CT, NC>(a.cos_sin, cs[u] + j0, c[u]);
+      cache_vec<CT, NC>(a.cos_sin, cs[u] + half + j0, sn[u]);
     }
   }
 
@@ -209,6 +196,7 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeArgs a) {
       for (int i = 0; i < E; ++i) x[i] *= r * (is_q[u] ? wq[i] : wk[i]);
     }
     // rotary embedding of the leading rotary_dim dims
+    const int uc = SAME ? 0 : u;
     if constexpr (INTERLEAVE) {
       if (!is_v[u] && rotated) {
 #pragma unroll
@@ -216,8 +204,8 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeArgs a) {
           // (the fused multiply-adds spelled out: left to the compiler, the instantiations for decode and prefill sizes
           // rounded differently in the last bit)
           const float e = x[2 * i], o = x[2 * i + 1];
-          x[2 * i] = __builtin_fmaf(e, c[u][i], -(o * sn[u][i]));
-          x[2 * i + 1] = __builtin_fmaf(e, sn[u][i], o * c[u][i]);
+          x[2 * i] = __builtin_fmaf(e, c[uc][i], -(o * sn[uc][i]));
+          x[2 * i + 1] = __builtin_fmaf(e, sn[uc][i], o * c[uc][i]);
         }
       }
     } else {
@@ -229,7 +217,7 @@ __global__ __launch_bounds__(256) void rope_and_cache_kernel(RopeArgs a) {
 #pragma unroll
         for (int i = 0; i < E; ++i) {
           const int d = sub * E + i;
-          x[i] = __builtin_fmaf(x[i], c[u][i], (d < half ? -other[i] : other[i]) * sn[u][i]);
+          x[i] = __builtin_fmaf(x[i], c[uc][i], (d < half ? -other[i] : other[i]) * sn[uc][i]);
         }
       }
     }
