@@ -54,21 +54,23 @@ __global__ __launch_bounds__(256) void reshape_vec_kernel(ReshapeArgs a) {
 #pragma unroll
   for (int u = 0; u < TPW; ++u) {
     const int64_t t = static_cast<int64_t>(blockIdx.x) * TPW + u;
-    slot[u] = t < a.n_tokens ? a.slots[t] : -1;
-    if (slot[u] >= a.n_slots) slot[u] = -1;
+    slot[u] = t < a.n_tokens ? a.slots[t] : -1;   // (looked at below, behind the row loads)
   }
+  // (a row is asked for whether or not its slot turns out to be one to write: the two loads then travel together
+  // instead of one after the other)
 #pragma unroll
   for (int u = 0; u < TPW; ++u) {
     const int64_t t = static_cast<int64_t>(blockIdx.x) * TPW + u;
     const char* p = src + t * stride + static_cast<int64_t>(w) * 16;
-    if (slot[u] >= 0) x[u] = TPW > 1 ? ldg16_stream(p) : ldg16(p);
+    x[u] = u32x4{0u, 0u, 0u, 0u};
+    if (t < a.n_tokens) x[u] = TPW > 1 ? ldg16_stream(p) : ldg16(p);
   }
   constexpr int EPV = IN == 2 ? 4 : 8;  // elements per 16-byte input vector
   float inv_scale = 0.0f;
   if constexpr (FP8) inv_scale = 1.0f / (is_v ? a.v_scale : a.k_scale)[w * EPV / a.head_dim];
 #pragma unroll
   for (int u = 0; u < TPW; ++u) {
-    if (slot[u] < 0) continue;
+    if (slot[u] < 0 || slot[u] >= a.n_slots) continue;
     if constexpr (!FP8) {
       constexpr int ES = IN == 2 ? 4 : 2;
       char* dst = cache + slot[u] * (static_cast<int64_t>(a.row_elems) * ES) + static_cast<int64_t>(w) * 16;
