@@ -87,6 +87,38 @@ def test_fp8_mla_and_merge_through_the_dispatcher(device, xops):
     assert torch.equal(mo.cpu(), torch.zeros(1, 1, 2, 3)) and torch.isneginf(ml).all()
 
 
+def test_mla_store_and_decode_in_one_call_through_the_dispatcher(device, xops):
+    """mla_dense_decode with latent_cache and slot_mapping (flash_mla::store_and_dense_decode) against the store
+    followed by the decode, both through the dispatcher: 128 heads (the rows are stored inside the decode launch) and
+    16 heads (the host side's library call issues two launches), with and without the step's plan."""
+    for heads in (128, 16):
+        cfg = workloads.DecodeConfig(f"mla{heads}", 4, heads, 1, 576, 64, 1, 900, mla=True, v_dim=512, sigma=0.5,
+                                     sm_scale=1 / math.sqrt(192.0))
+        inp = workloads.make_inputs(cfg, 50 + heads)
+        lay = inp.layout
+        cache0 = torch.full((lay.num_blocks, 64, 1, 576), float("nan"), dtype=torch.bfloat16, device=device)
+        ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=inp.k_ctx.to(device), k_cache=cache0,
+                                                            slot_mapping=lay.ctx_slots.to(device)))
+        q = inp.q.to(device)
+        qn = q[:, :, :512].contiguous().view(4, 1, heads, 512)
+        qp = q[:, :, 512:].contiguous().view(4, 1, heads, 64)
+        lens, table = lay.seq_lens.to(device), lay.block_table.to(device)
+        latent, slots = inp.k_new.to(device), lay.new_slots.to(device)
+        for planned in (False, True):
+            plan = xops.mla_decoding_metadata(lens, table, heads, 64) if planned else None
+            ca = cache0.clone()
+            ops.reshape_paged_cache(ops.ReshapePagedCacheParams(key=latent, k_cache=ca, slot_mapping=slots))
+            out_a, lse_a = xops.mla_dense_decode(qn, qp, ca, lens, table, 512, cfg.scale, False, plan)
+            cb = cache0.clone()
+            out_b, lse_b = xops.mla_dense_decode(qn, qp, cb, lens, table, 512, cfg.scale, False, plan, latent, slots)
+            torch.cuda.synchronize()
+            assert torch.equal(ca.view(torch.int16), cb.view(torch.int16))
+            assert torch.equal(out_a.view(torch.int16), out_b.view(torch.int16)) and torch.equal(lse_a, lse_b)
+            assert torch.isfinite(out_b.float()).all()
+        ref = oracle.aten_paged_decode(inp.q, cb.cpu(), None, lay.block_table, lay.seq_lens, cfg.scale, dv=512)
+        assert_close_to_reference(out_b.view(4, heads, 512), ref, cfg.name)
+
+
 def test_query_chunks_and_latent_gather_through_the_dispatcher(device, xops):
     cfg = workloads.DecodeConfig("shim_chunks", 5, 32, 8, 128, 16, 10, 600)
     inp = workloads.make_inputs(cfg, 23)
